@@ -1,0 +1,65 @@
+/*
+ * ggml-mi355x.h — public entry points of the MI355X (gfx950) ggml compute backend.
+ *
+ * The backend is a plugin for ggml's backend interface (ggml/src/ggml-backend-impl.h:17-207 of the
+ * whisper.cpp tree): it implements the buffer-type, buffer, backend(stream), device and reg vtables
+ * and is found by a ggml host in either of two ways:
+ *
+ *   - dynamically: ggml_backend_load("libggml-mi355x.so") (ggml/include/ggml-backend.h:228) resolves
+ *     ggml_backend_score() and ggml_backend_init() (ggml/src/ggml-backend-impl.h:215-218,
+ *     ggml/src/ggml-backend-reg.cpp:227-271) and registers the returned reg;
+ *   - statically: the host calls ggml_backend_register(ggml_backend_mi355x_reg())
+ *     (ggml/src/ggml-backend-impl.h:210), the same pattern as ggml_backend_cuda_reg()
+ *     (ggml/include/ggml-cuda.h:45).
+ *
+ * This header is compiled against the host tree's ggml.h / ggml-backend.h, like every other backend's
+ * public header (ggml/include/ggml-cuda.h:3-4).
+ */
+#pragma once
+
+#include "ggml.h"
+#include "ggml-backend.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define GGML_MI355X_NAME "MI355X"
+
+/* counterpart of ggml_backend_cuda_reg (ggml/include/ggml-cuda.h:45) */
+GGML_BACKEND_API ggml_backend_reg_t         ggml_backend_mi355x_reg(void);
+/* counterpart of ggml_backend_cuda_init (ggml/include/ggml-cuda.h:23); NULL if `device` is not a gfx950 GPU */
+GGML_BACKEND_API ggml_backend_t             ggml_backend_mi355x_init(int device);
+/* counterpart of ggml_backend_is_cuda (ggml/include/ggml-cuda.h:25) */
+GGML_BACKEND_API bool                       ggml_backend_is_mi355x(ggml_backend_t backend);
+/* counterpart of ggml_backend_cuda_buffer_type (ggml/include/ggml-cuda.h:28) */
+GGML_BACKEND_API ggml_backend_buffer_type_t ggml_backend_mi355x_buffer_type(int device);
+/* counterpart of ggml_backend_cuda_get_device_count (ggml/include/ggml-cuda.h:36): number of gfx950 devices */
+GGML_BACKEND_API int                        ggml_backend_mi355x_get_device_count(void);
+
+/* dynamic-loading entry points (ggml/src/ggml-backend-impl.h:215-218) */
+GGML_BACKEND_API ggml_backend_reg_t ggml_backend_init(void);
+GGML_BACKEND_API int                ggml_backend_score(void);
+
+/*
+ * Extras reachable through ggml_backend_reg_get_proc_address(reg, name) (ggml/include/ggml-backend.h:185-200):
+ *
+ *   "ggml_backend_get_features"        ggml_backend_get_features_t
+ *   "ggml_backend_mi355x_set_option"   ggml_backend_mi355x_set_option_t
+ *   "ggml_backend_mi355x_get_stats"    ggml_backend_mi355x_get_stats_t
+ */
+
+/* Options: "fuse" (0/1: fold bias/activation/residual/LayerNorm-affine neighbours into one kernel, default 1),
+ * "profile" (0/1: bracket every kernel with HIP events on the backend's stream, default 0).
+ * The environment variables GGML_MI355X_FUSE and GGML_MI355X_PROFILE give the initial values. */
+typedef int (*ggml_backend_mi355x_set_option_t)(ggml_backend_t backend, const char * name, int value);
+
+/* Per-kernel statistics gathered while "profile" is on: writes a JSON array
+ * [{"kernel": name, "calls": n, "ms": total, "bytes": algorithmic bytes, "flops": algorithmic flops}, ...]
+ * into buf (at most size bytes, NUL-terminated), resets the counters when `reset` is non-zero and returns the
+ * length needed. */
+typedef size_t (*ggml_backend_mi355x_get_stats_t)(ggml_backend_t backend, char * buf, size_t size, int reset);
+
+#ifdef __cplusplus
+}
+#endif

@@ -1,0 +1,164 @@
+/*
+ * mi355x_kernels.h — C ABI of the hand-written gfx950 (MI355X) kernels behind the ggml-mi355x backend.
+ *
+ * Every entry point takes plain device pointers, element counts and byte strides (the same
+ * ne[]/nb[] convention as ggml: ne[0] is the contiguous dimension, nb[i] is the byte stride of
+ * dimension i), launches asynchronously on the HIP stream handed in as `stream` (a hipStream_t passed
+ * as void*, NULL = default stream) and returns MI355X_OK or a negative error code.  Nothing here
+ * allocates device memory; ops that need scratch take a caller-provided workspace.
+ *
+ * Each declaration cites the function of the reference's CPU backend whose results it reproduces
+ * (paths relative to the whisper.cpp tree).
+ */
+#ifndef MI355X_KERNELS_H
+#define MI355X_KERNELS_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MI355X_API __attribute__((visibility("default")))
+
+/* element types; numeric values equal the reference's enum ggml_type (ggml/include/ggml.h:351-392) */
+enum mi355x_type {
+    MI355X_TYPE_F32  = 0,
+    MI355X_TYPE_F16  = 1,
+    MI355X_TYPE_Q5_0 = 6,  /* block_q5_0, 22 bytes per 32 weights (ggml/src/ggml-common.h:187-193) */
+    MI355X_TYPE_Q8_0 = 8,  /* block_q8_0, 34 bytes per 32 weights (ggml/src/ggml-common.h:209-214) */
+    MI355X_TYPE_I32  = 26,
+};
+
+enum mi355x_status {
+    MI355X_OK               =  0,
+    MI355X_ERR_UNSUPPORTED  = -1,  /* type / layout combination has no kernel */
+    MI355X_ERR_INVALID      = -2,  /* inconsistent shapes, NULL pointer, misaligned operand */
+    MI355X_ERR_WORKSPACE    = -3,  /* workspace missing or too small */
+    MI355X_ERR_HIP          = -4,  /* the HIP runtime reported an error at launch */
+};
+
+/* A strided view of device memory.  For block-quantized types ne[0] counts weights (a multiple of 32)
+ * and nb[0] is the block size in bytes. */
+typedef struct mi355x_tensor {
+    void *  data;
+    int32_t type;       /* enum mi355x_type */
+    int32_t _pad;
+    int64_t ne[4];
+    size_t  nb[4];
+} mi355x_tensor;
+
+/* epilogue fused into MUL_MAT: dst = act((src0^T src1) + bias) * scale + residual, each part optional */
+enum mi355x_epilogue_flags {
+    MI355X_EPI_NONE     = 0,
+    MI355X_EPI_BIAS     = 1,   /* + bias[m]      (f32, ne0 = dst ne0)            : ggml ADD with a row vector  */
+    MI355X_EPI_GELU     = 2,   /* tanh-GELU       (ggml/src/ggml-cpu/vec.h:432-457)                            */
+    MI355X_EPI_SCALE    = 4,   /* * scale         (ggml/src/ggml-cpu/ops.cpp:3840-3878)                        */
+    MI355X_EPI_RESIDUAL = 8,   /* + residual[m,n] (f32, same shape and strides as dst)                         */
+    MI355X_EPI_BIAS_COL = 16,  /* + bias[n]       (f32, one value per dst row n: conv bias [1,d], broadcast along ne0) */
+    MI355X_EPI_OUT_F16  = 32,  /* dst is f16 instead of f32 (ggml CPY f32->f16 folded in)                      */
+};
+
+typedef struct mi355x_epilogue {
+    int32_t      flags;
+    float        scale;
+    const void * bias;
+    const void * residual;
+} mi355x_epilogue;
+
+/* library / device ---------------------------------------------------------------------------------- */
+
+/* Version of this ABI (bumped on any incompatible change). */
+MI355X_API int          mi355x_abi_version(void);
+/* 1 if HIP device `device` is a gfx950 part, 0 otherwise, negative on HIP error. */
+MI355X_API int          mi355x_device_is_gfx950(int device);
+MI355X_API const char * mi355x_status_string(int status);
+
+/* quantization formats -------------------------------------------------------------------------------
+ * dequantize_row_q5_0 / dequantize_row_q8_0 (ggml/src/ggml-quants.c:296-319, 349-363): y[i] = d * q,
+ * bit-exact.  `k` weights (multiple of 32) from `src` (device) to f32 `dst` (device). */
+MI355X_API int mi355x_dequantize_row(int type, const void * src, float * dst, int64_t k, void * stream);
+
+/* quantize_row_q8_0 of the CPU backend's AVX2 build (ggml/src/ggml-cpu/ggml-cpu-quants.c:738,808-865):
+ * per 32 values d = amax/127 stored as f16, q = round-to-nearest-even(x * (127/amax)).  `k` multiple of 32. */
+MI355X_API int mi355x_quantize_row_q8_0(const float * src, void * dst, int64_t k, void * stream);
+
+/* MUL_MAT ---------------------------------------------------------------------------------------------
+ * ggml_compute_forward_mul_mat (ggml/src/ggml-cpu/ggml-cpu.c:1266-1458):
+ *   dst[m, n, b2, b3] = sum_k src0[k, m, b2/r2, b3/r3] * src1[k, n, b2, b3]
+ * src0: Q5_0 | Q8_0 | F16 | F32, ne0 = K contiguous.  src1: F32 | F16, ne0 = K contiguous.  dst: F32
+ * (F16 with MI355X_EPI_OUT_F16), ne0 = M contiguous.  `epi` may be NULL.
+ * Columns n <= MI355X_GEMV_MAX_COLS with a quantized src0 take the HBM-streaming GEMV path, which
+ * quantizes src1 to Q8_0 in `workspace` exactly like the CPU backend does (ggml-cpu.c:1328-1363) and
+ * accumulates integer block dot products like ggml_vec_dot_q5_0_q8_0 / ggml_vec_dot_q8_0_q8_0
+ * (ggml-cpu-quants.c:2930, 3597).  Everything else runs the MFMA GEMM (weights dequantized to f16 on the
+ * way into LDS, f32 accumulation). */
+#define MI355X_GEMV_MAX_COLS 8
+/* name of the kernel mi355x_mul_mat would launch for these operands ("mul_mat.gemm_q5_0", "mul_mat.gemv_q8_0", ...);
+ * a static string, used to label profiles */
+MI355X_API const char * mi355x_mul_mat_kernel_name(const mi355x_tensor * src0, const mi355x_tensor * src1);
+MI355X_API size_t mi355x_mul_mat_workspace_size(const mi355x_tensor * src0, const mi355x_tensor * src1);
+MI355X_API int    mi355x_mul_mat(const mi355x_tensor * src0, const mi355x_tensor * src1, const mi355x_tensor * dst,
+                                 const mi355x_epilogue * epi, void * workspace, size_t workspace_size, void * stream);
+
+/* FLASH_ATTN_EXT --------------------------------------------------------------------------------------
+ * ggml_compute_forward_flash_attn_ext_f16 (ggml/src/ggml-cpu/ops.cpp:6638-6851), max_bias = 0 and
+ * logit_softcap = 0 (the only values whisper uses):
+ *   dst[:, h, n] = softmax_over_keys(scale * q[:, n, h] . k[:, key, h] + mask[key, n]) @ v[:, key, h]
+ * q: F32 [D, N, H], k/v: F16 [D, KV, H] (D = 64), mask: F16 [KV, >=N] or NULL (-inf entries skip the
+ * key), dst: F32 [D, H, N] contiguous.  `workspace` is used when the key range is split across
+ * workgroups (small N); size from mi355x_flash_attn_ext_workspace_size. */
+MI355X_API const char * mi355x_flash_attn_ext_kernel_name(const mi355x_tensor * q, const mi355x_tensor * k);
+MI355X_API size_t mi355x_flash_attn_ext_workspace_size(const mi355x_tensor * q, const mi355x_tensor * k);
+MI355X_API int    mi355x_flash_attn_ext(const mi355x_tensor * q, const mi355x_tensor * k, const mi355x_tensor * v,
+                                        const mi355x_tensor * mask, const mi355x_tensor * dst, float scale,
+                                        void * workspace, size_t workspace_size, void * stream);
+
+/* elementwise / row ops ------------------------------------------------------------------------------ */
+
+/* ADD / MUL with src1 repeated over any dimension, including ne0 (ggml/src/ggml-cpu/binary-ops.cpp:49-142).
+ * All F32; dst may alias src0 or src1.  op: 0 = add, 1 = mul. */
+MI355X_API int mi355x_binary(int op, const mi355x_tensor * src0, const mi355x_tensor * src1, const mi355x_tensor * dst, void * stream);
+
+/* SCALE: dst = src * s (ggml/src/ggml-cpu/ops.cpp:3840-3878).  F32, may run in place. */
+MI355X_API int mi355x_scale(const mi355x_tensor * src, const mi355x_tensor * dst, float s, void * stream);
+
+/* UNARY GELU (ggml/src/ggml-cpu/ops.cpp:2606-2643, vec.h:432-457): 0.5x(1+tanh(sqrt(2/pi) x (1+0.044715x^2))),
+ * evaluated in f32 (the CPU backend looks the value up in an f16 table; the difference is below 1e-6 NMSE). */
+MI355X_API int mi355x_gelu(const mi355x_tensor * src, const mi355x_tensor * dst, void * stream);
+
+/* NORM (ggml/src/ggml-cpu/ops.cpp:3109-3158): y = (x - mean) / sqrt(var + eps) over ne0.  With w and/or b
+ * non-NULL also applies the following MUL by w[ne0] and ADD of b[ne0] (whisper's LayerNorm affine,
+ * src/whisper.cpp:2116-2121).  All F32. */
+MI355X_API int mi355x_norm(const mi355x_tensor * src, const mi355x_tensor * dst, float eps,
+                           const float * w, const float * b, void * stream);
+
+/* SOFT_MAX (ggml/src/ggml-cpu/ops.cpp:4641-4737), max_bias = 0: softmax(scale * x + mask) over ne0.
+ * mask F32 or F16 [ne0, >= ne1], broadcast over ne2/ne3, or NULL. */
+MI355X_API int mi355x_soft_max(const mi355x_tensor * src, const mi355x_tensor * mask, const mi355x_tensor * dst,
+                               float scale, void * stream);
+
+/* CPY / CONT / DUP (ggml/src/ggml-cpu/ops.cpp:670-1183): strided element copy with conversion between
+ * F32 and F16 (round-to-nearest-even).  src and dst hold the same number of elements; either may be
+ * a strided / permuted view. */
+MI355X_API int mi355x_cpy(const mi355x_tensor * src, const mi355x_tensor * dst, void * stream);
+
+/* GET_ROWS (ggml/src/ggml-cpu/ops.cpp:4146-4188, 4313): dst[:, i] = dequant(src0[:, ids[i]]).
+ * src0: Q5_0 | Q8_0 | F16 | F32, ids: I32, dst: F32. */
+MI355X_API int mi355x_get_rows(const mi355x_tensor * src0, const mi355x_tensor * ids, const mi355x_tensor * dst, void * stream);
+
+/* IM2COL, 1-D, F16 output (ggml/src/ggml-cpu/ops.cpp:5784-5855; ggml/src/ggml.c:3818-3858):
+ * dst[ic*KW + kw, ow, n] = f16(src[ow*s0 + kw*d0 - p0, ic, n]) or 0 outside.  src F32 [IW, IC, N]. */
+MI355X_API int mi355x_im2col_1d(const mi355x_tensor * src, const mi355x_tensor * dst, int kw, int s0, int p0, int d0, void * stream);
+
+/* CONCAT along `dim` (ggml/src/ggml-cpu/ops.cpp:2575).  F32. */
+MI355X_API int mi355x_concat(const mi355x_tensor * src0, const mi355x_tensor * src1, const mi355x_tensor * dst, int dim, void * stream);
+
+/* Fill `n` bytes at `dst` with `value` through a kernel (safe inside HIP graph capture). */
+MI355X_API int mi355x_fill_bytes(void * dst, uint8_t value, size_t n, void * stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MI355X_KERNELS_H */

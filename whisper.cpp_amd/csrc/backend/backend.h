@@ -1,0 +1,74 @@
+// Internal declarations shared by the ggml-mi355x backend sources.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <map>
+#include <mutex>
+#include <string>
+#include <vector>
+
+#include "ggml.h"
+#include "ggml-backend.h"
+#include "ggml-backend-impl.h"
+#include "ggml-impl.h"
+
+#include "ggml-mi355x.h"
+#include "mi355x_kernels.h"
+
+#define MI355X_BUFFER_ALIGN 256
+
+#define HIP_TRY(expr, on_fail)                                                                            \
+    do {                                                                                                  \
+        hipError_t err_ = (expr);                                                                         \
+        if (err_ != hipSuccess) {                                                                         \
+            GGML_LOG_ERROR("ggml-mi355x: %s failed: %s (%s:%d)\n", #expr, hipGetErrorString(err_), __FILE__, __LINE__); \
+            (void) hipGetLastError();                                                                     \
+            on_fail;                                                                                      \
+        }                                                                                                 \
+    } while (0)
+
+struct mi355x_device_ctx {
+    int         device;        // HIP ordinal
+    std::string name;          // "MI355X0"
+    std::string description;   // marketing name from the driver
+};
+
+struct mi355x_buffer_ctx {
+    int    device;
+    void * base;
+    size_t size;
+};
+
+struct mi355x_kernel_stat {
+    int64_t calls = 0;
+    double  ms    = 0.0;
+    double  bytes = 0.0;
+    double  flops = 0.0;
+};
+
+struct mi355x_pending_event {
+    hipEvent_t  start, stop;
+    const char *name;
+    double      bytes, flops;
+};
+
+struct mi355x_backend_ctx {
+    int         device;
+    std::string name;
+    hipStream_t stream = nullptr;
+    bool        fuse    = true;
+    bool        profile = false;
+
+    // profiling
+    std::vector<mi355x_pending_event>         pending;
+    std::vector<hipEvent_t>                   event_pool;
+    std::map<std::string, mi355x_kernel_stat> stats;
+
+    hipEvent_t take_event();
+    void       drain_events();           // call after the stream has been synchronized
+};
+
+// graph.cpp
+enum ggml_status mi355x_graph_compute(mi355x_backend_ctx * ctx, struct ggml_cgraph * cgraph);
+bool             mi355x_supports_op(const struct ggml_tensor * op);

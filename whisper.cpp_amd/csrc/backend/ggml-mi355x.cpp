@@ -1,0 +1,419 @@
+// The five ggml-backend vtables for MI355X (ggml/src/ggml-backend-impl.h:17-207 of the whisper.cpp tree)
+// and the two dynamic-loading entry points (ggml-backend-impl.h:215-218).  Host-side only: device memory
+// comes from hipMalloc, transfers are hipMemcpy on the backend's stream, all arithmetic goes through the
+// kernel C ABI declared in mi355x_kernels.h.
+#include "backend.h"
+
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+
+// ------------------------------------------------------------------------------------------------------
+// device discovery
+// ------------------------------------------------------------------------------------------------------
+
+static std::vector<int> & gfx950_devices() {
+    static std::vector<int> devs = [] {
+        std::vector<int> v;
+        int n = 0;
+        if (hipGetDeviceCount(&n) != hipSuccess) { (void) hipGetLastError(); return v; }
+        for (int i = 0; i < n; ++i) if (mi355x_device_is_gfx950(i) == 1) v.push_back(i);
+        return v;
+    }();
+    return devs;
+}
+
+static bool env_flag(const char * name, bool dflt) {
+    const char * v = getenv(name);
+    if (!v || !*v) return dflt;
+    return atoi(v) != 0;
+}
+
+// ------------------------------------------------------------------------------------------------------
+// buffer  (ggml_backend_buffer_i, ggml-backend-impl.h:41-58)
+// ------------------------------------------------------------------------------------------------------
+
+static void buffer_free(ggml_backend_buffer_t buffer) {
+    mi355x_buffer_ctx * ctx = (mi355x_buffer_ctx *) buffer->context;
+    HIP_TRY(hipSetDevice(ctx->device), (void) 0);
+    HIP_TRY(hipDeviceSynchronize(), (void) 0);
+    HIP_TRY(hipFree(ctx->base), (void) 0);
+    delete ctx;
+}
+
+static void * buffer_get_base(ggml_backend_buffer_t buffer) {
+    return ((mi355x_buffer_ctx *) buffer->context)->base;
+}
+
+static enum ggml_status buffer_init_tensor(ggml_backend_buffer_t, struct ggml_tensor *) {
+    return GGML_STATUS_SUCCESS;   // tensors need no per-tensor state
+}
+
+// Buffer-level transfers are synchronous (the scheduler synchronizes the backend before it calls them,
+// ggml/src/ggml-backend.cpp:1371-1375); they run on the null stream, which orders itself against the
+// backend's (blocking) stream.
+static void buffer_memset_tensor(ggml_backend_buffer_t buffer, struct ggml_tensor * tensor, uint8_t value, size_t offset, size_t size) {
+    mi355x_buffer_ctx * ctx = (mi355x_buffer_ctx *) buffer->context;
+    HIP_TRY(hipSetDevice(ctx->device), return);
+    HIP_TRY(hipMemset((char *) tensor->data + offset, value, size), return);
+    HIP_TRY(hipStreamSynchronize(nullptr), return);
+}
+
+static void buffer_set_tensor(ggml_backend_buffer_t buffer, struct ggml_tensor * tensor, const void * data, size_t offset, size_t size) {
+    mi355x_buffer_ctx * ctx = (mi355x_buffer_ctx *) buffer->context;
+    HIP_TRY(hipSetDevice(ctx->device), return);
+    HIP_TRY(hipMemcpy((char *) tensor->data + offset, data, size, hipMemcpyHostToDevice), return);
+}
+
+static void buffer_get_tensor(ggml_backend_buffer_t buffer, const struct ggml_tensor * tensor, void * data, size_t offset, size_t size) {
+    mi355x_buffer_ctx * ctx = (mi355x_buffer_ctx *) buffer->context;
+    HIP_TRY(hipSetDevice(ctx->device), return);
+    HIP_TRY(hipMemcpy(data, (const char *) tensor->data + offset, size, hipMemcpyDeviceToHost), return);
+}
+
+static bool buffer_is_mi355x(ggml_backend_buffer_t buffer) { return buffer && buffer->iface.get_base == buffer_get_base; }
+
+static bool buffer_cpy_tensor(ggml_backend_buffer_t buffer, const struct ggml_tensor * src, struct ggml_tensor * dst) {
+    mi355x_buffer_ctx * ctx = (mi355x_buffer_ctx *) buffer->context;
+    ggml_backend_buffer_t sbuf = src->view_src ? src->view_src->buffer : src->buffer;
+    if (!ggml_is_contiguous(src) || !ggml_is_contiguous(dst) || ggml_nbytes(src) != ggml_nbytes(dst)) return false;
+    HIP_TRY(hipSetDevice(ctx->device), return false);
+    if (buffer_is_mi355x(sbuf)) {
+        HIP_TRY(hipMemcpy(dst->data, src->data, ggml_nbytes(src), hipMemcpyDeviceToDevice), return false);
+        HIP_TRY(hipStreamSynchronize(nullptr), return false);
+        return true;
+    }
+    if (sbuf && ggml_backend_buffer_is_host(sbuf)) {
+        HIP_TRY(hipMemcpy(dst->data, src->data, ggml_nbytes(src), hipMemcpyHostToDevice), return false);
+        return true;
+    }
+    return false;
+}
+
+static void buffer_clear(ggml_backend_buffer_t buffer, uint8_t value) {
+    mi355x_buffer_ctx * ctx = (mi355x_buffer_ctx *) buffer->context;
+    HIP_TRY(hipSetDevice(ctx->device), return);
+    HIP_TRY(hipMemset(ctx->base, value, ctx->size), return);
+    HIP_TRY(hipDeviceSynchronize(), return);
+}
+
+static const struct ggml_backend_buffer_i mi355x_buffer_iface = {
+    /* .free_buffer   = */ buffer_free,
+    /* .get_base      = */ buffer_get_base,
+    /* .init_tensor   = */ buffer_init_tensor,
+    /* .memset_tensor = */ buffer_memset_tensor,
+    /* .set_tensor    = */ buffer_set_tensor,
+    /* .get_tensor    = */ buffer_get_tensor,
+    /* .cpy_tensor    = */ buffer_cpy_tensor,
+    /* .clear         = */ buffer_clear,
+    /* .reset         = */ NULL,
+};
+
+// ------------------------------------------------------------------------------------------------------
+// buffer type  (ggml_backend_buffer_type_i, ggml-backend-impl.h:17-29)
+// ------------------------------------------------------------------------------------------------------
+
+static const char * buft_get_name(ggml_backend_buffer_type_t buft) {
+    return ((mi355x_device_ctx *) buft->device->context)->name.c_str();
+}
+
+static ggml_backend_buffer_t buft_alloc_buffer(ggml_backend_buffer_type_t buft, size_t size) {
+    mi355x_device_ctx * dev = (mi355x_device_ctx *) buft->device->context;
+    HIP_TRY(hipSetDevice(dev->device), return NULL);
+    void * base = nullptr;
+    const size_t alloc = size ? size : 1;
+    hipError_t err = hipMalloc(&base, alloc);
+    if (err != hipSuccess || !base) {
+        (void) hipGetLastError();
+        GGML_LOG_ERROR("ggml-mi355x: allocating %.2f MiB on device %d failed: %s\n", alloc / 1048576.0, dev->device, hipGetErrorString(err));
+        return NULL;
+    }
+    mi355x_buffer_ctx * ctx = new mi355x_buffer_ctx{ dev->device, base, size };
+    return ggml_backend_buffer_init(buft, mi355x_buffer_iface, ctx, size);
+}
+
+static size_t buft_get_alignment(ggml_backend_buffer_type_t) { return MI355X_BUFFER_ALIGN; }
+
+static size_t buft_get_max_size(ggml_backend_buffer_type_t buft) {
+    mi355x_device_ctx * dev = (mi355x_device_ctx *) buft->device->context;
+    hipDeviceProp_t prop;
+    if (hipGetDeviceProperties(&prop, dev->device) != hipSuccess) { (void) hipGetLastError(); return SIZE_MAX; }
+    return prop.totalGlobalMem;
+}
+
+// No kernel reads past the last block of a row or the last row of a tensor, so tensors need no padding.
+static size_t buft_get_alloc_size(ggml_backend_buffer_type_t, const struct ggml_tensor * tensor) {
+    return ggml_nbytes(tensor);
+}
+
+static bool buft_is_host(ggml_backend_buffer_type_t) { return false; }
+
+static const struct ggml_backend_buffer_type_i mi355x_buft_iface = {
+    /* .get_name       = */ buft_get_name,
+    /* .alloc_buffer   = */ buft_alloc_buffer,
+    /* .get_alignment  = */ buft_get_alignment,
+    /* .get_max_size   = */ buft_get_max_size,
+    /* .get_alloc_size = */ buft_get_alloc_size,
+    /* .is_host        = */ buft_is_host,
+};
+
+// ------------------------------------------------------------------------------------------------------
+// backend / stream  (ggml_backend_i, ggml-backend-impl.h:87-117)
+// ------------------------------------------------------------------------------------------------------
+
+static ggml_guid_t backend_guid() {
+    static ggml_guid guid = { 0x4d, 0x49, 0x33, 0x35, 0x35, 0x58, 0x2d, 0x67, 0x66, 0x78, 0x39, 0x35, 0x30, 0x2d, 0x76, 0x31 };
+    return &guid;
+}
+
+static const char * backend_get_name(ggml_backend_t backend) {
+    return ((mi355x_backend_ctx *) backend->context)->name.c_str();
+}
+
+static void backend_synchronize(ggml_backend_t backend) {
+    mi355x_backend_ctx * ctx = (mi355x_backend_ctx *) backend->context;
+    HIP_TRY(hipSetDevice(ctx->device), return);
+    HIP_TRY(hipStreamSynchronize(ctx->stream), return);
+    if (!ctx->pending.empty()) ctx->drain_events();
+}
+
+static void backend_free(ggml_backend_t backend) {
+    mi355x_backend_ctx * ctx = (mi355x_backend_ctx *) backend->context;
+    backend_synchronize(backend);
+    for (hipEvent_t e : ctx->event_pool) (void) hipEventDestroy(e);
+    if (ctx->stream) (void) hipStreamDestroy(ctx->stream);
+    delete ctx;
+    delete backend;
+}
+
+static void backend_set_tensor_async(ggml_backend_t backend, struct ggml_tensor * tensor, const void * data, size_t offset, size_t size) {
+    mi355x_backend_ctx * ctx = (mi355x_backend_ctx *) backend->context;
+    HIP_TRY(hipSetDevice(ctx->device), return);
+    HIP_TRY(hipMemcpyAsync((char *) tensor->data + offset, data, size, hipMemcpyHostToDevice, ctx->stream), return);
+}
+
+static void backend_get_tensor_async(ggml_backend_t backend, const struct ggml_tensor * tensor, void * data, size_t offset, size_t size) {
+    mi355x_backend_ctx * ctx = (mi355x_backend_ctx *) backend->context;
+    HIP_TRY(hipSetDevice(ctx->device), return);
+    HIP_TRY(hipMemcpyAsync(data, (const char *) tensor->data + offset, size, hipMemcpyDeviceToHost, ctx->stream), return);
+}
+
+static enum ggml_status backend_graph_compute(ggml_backend_t backend, struct ggml_cgraph * cgraph) {
+    return mi355x_graph_compute((mi355x_backend_ctx *) backend->context, cgraph);
+}
+
+static const struct ggml_backend_i mi355x_backend_iface = {
+    /* .get_name           = */ backend_get_name,
+    /* .free               = */ backend_free,
+    /* .set_tensor_async   = */ backend_set_tensor_async,
+    /* .get_tensor_async   = */ backend_get_tensor_async,
+    /* .cpy_tensor_async   = */ NULL,
+    /* .synchronize        = */ backend_synchronize,
+    /* .graph_plan_create  = */ NULL,
+    /* .graph_plan_free    = */ NULL,
+    /* .graph_plan_update  = */ NULL,
+    /* .graph_plan_compute = */ NULL,
+    /* .graph_compute      = */ backend_graph_compute,
+    /* .event_record       = */ NULL,
+    /* .event_wait         = */ NULL,
+};
+
+// ------------------------------------------------------------------------------------------------------
+// device  (ggml_backend_device_i, ggml-backend-impl.h:137-179)
+// ------------------------------------------------------------------------------------------------------
+
+static const char * device_get_name(ggml_backend_dev_t dev)        { return ((mi355x_device_ctx *) dev->context)->name.c_str(); }
+static const char * device_get_description(ggml_backend_dev_t dev) { return ((mi355x_device_ctx *) dev->context)->description.c_str(); }
+
+static void device_get_memory(ggml_backend_dev_t dev, size_t * free, size_t * total) {
+    mi355x_device_ctx * ctx = (mi355x_device_ctx *) dev->context;
+    *free = 0; *total = 0;
+    HIP_TRY(hipSetDevice(ctx->device), return);
+    HIP_TRY(hipMemGetInfo(free, total), return);
+}
+
+static enum ggml_backend_dev_type device_get_type(ggml_backend_dev_t) { return GGML_BACKEND_DEVICE_TYPE_GPU; }
+
+static void device_get_props(ggml_backend_dev_t dev, struct ggml_backend_dev_props * props) {
+    props->name        = device_get_name(dev);
+    props->description = device_get_description(dev);
+    props->type        = device_get_type(dev);
+    device_get_memory(dev, &props->memory_free, &props->memory_total);
+    props->caps = { /* async */ false, /* host_buffer */ false, /* buffer_from_host_ptr */ false, /* events */ false };
+}
+
+static ggml_backend_t device_init_backend(ggml_backend_dev_t dev, const char *) {
+    mi355x_device_ctx * dctx = (mi355x_device_ctx *) dev->context;
+    HIP_TRY(hipSetDevice(dctx->device), return NULL);
+    mi355x_backend_ctx * ctx = new mi355x_backend_ctx;
+    ctx->device  = dctx->device;
+    ctx->name    = dctx->name;
+    ctx->fuse    = env_flag("GGML_MI355X_FUSE", true);
+    ctx->profile = env_flag("GGML_MI355X_PROFILE", false);
+    // default priority, blocking with respect to the null stream used by the buffer-level copies
+    HIP_TRY(hipStreamCreate(&ctx->stream), { delete ctx; return NULL; });
+    ggml_backend_t backend = new ggml_backend{
+        /* .guid    = */ backend_guid(),
+        /* .iface   = */ mi355x_backend_iface,
+        /* .device  = */ dev,
+        /* .context = */ ctx,
+    };
+    return backend;
+}
+
+static ggml_backend_buffer_type_t device_get_buffer_type(ggml_backend_dev_t dev);
+
+static bool device_supports_op(ggml_backend_dev_t, const struct ggml_tensor * op) { return mi355x_supports_op(op); }
+
+static bool device_supports_buft(ggml_backend_dev_t dev, ggml_backend_buffer_type_t buft) {
+    return buft->iface.get_name == buft_get_name && buft->device == dev;
+}
+
+static bool device_offload_op(ggml_backend_dev_t, const struct ggml_tensor *) { return false; }
+
+static const struct ggml_backend_device_i mi355x_device_iface = {
+    /* .get_name             = */ device_get_name,
+    /* .get_description      = */ device_get_description,
+    /* .get_memory           = */ device_get_memory,
+    /* .get_type             = */ device_get_type,
+    /* .get_props            = */ device_get_props,
+    /* .init_backend         = */ device_init_backend,
+    /* .get_buffer_type      = */ device_get_buffer_type,
+    /* .get_host_buffer_type = */ NULL,
+    /* .buffer_from_host_ptr = */ NULL,
+    /* .supports_op          = */ device_supports_op,
+    /* .supports_buft        = */ device_supports_buft,
+    /* .offload_op           = */ device_offload_op,
+    /* .event_new            = */ NULL,
+    /* .event_free           = */ NULL,
+    /* .event_synchronize    = */ NULL,
+};
+
+// ------------------------------------------------------------------------------------------------------
+// reg  (ggml_backend_reg_i, ggml-backend-impl.h:191-207)
+// ------------------------------------------------------------------------------------------------------
+
+struct mi355x_reg_ctx {
+    std::vector<ggml_backend_device>      devices;
+    std::vector<ggml_backend_buffer_type> bufts;
+};
+
+static const char * reg_get_name(ggml_backend_reg_t) { return GGML_MI355X_NAME; }
+
+static size_t reg_get_device_count(ggml_backend_reg_t reg) { return ((mi355x_reg_ctx *) reg->context)->devices.size(); }
+
+static ggml_backend_dev_t reg_get_device(ggml_backend_reg_t reg, size_t index) {
+    mi355x_reg_ctx * ctx = (mi355x_reg_ctx *) reg->context;
+    return index < ctx->devices.size() ? &ctx->devices[index] : NULL;
+}
+
+static struct ggml_backend_feature * get_features(ggml_backend_reg_t) {
+    static struct ggml_backend_feature features[] = {
+        { "GFX950",   "1" },
+        { "MFMA_F16", "1" },
+        { "DOT4_I8",  "1" },
+        { NULL, NULL },
+    };
+    return features;
+}
+
+static int set_option(ggml_backend_t backend, const char * name, int value) {
+    if (!ggml_backend_is_mi355x(backend) || !name) return -1;
+    mi355x_backend_ctx * ctx = (mi355x_backend_ctx *) backend->context;
+    if (strcmp(name, "fuse") == 0)    { ctx->fuse = value != 0; return 0; }
+    if (strcmp(name, "profile") == 0) { backend_synchronize(backend); ctx->profile = value != 0; return 0; }
+    return -1;
+}
+
+static size_t get_stats(ggml_backend_t backend, char * buf, size_t size, int reset) {
+    if (!ggml_backend_is_mi355x(backend)) return 0;
+    mi355x_backend_ctx * ctx = (mi355x_backend_ctx *) backend->context;
+    backend_synchronize(backend);
+    std::string s = "[";
+    bool first = true;
+    for (auto & kv : ctx->stats) {
+        char line[512];
+        snprintf(line, sizeof(line), "%s{\"kernel\": \"%s\", \"calls\": %lld, \"ms\": %.6f, \"bytes\": %.0f, \"flops\": %.0f}",
+                 first ? "" : ", ", kv.first.c_str(), (long long) kv.second.calls, kv.second.ms, kv.second.bytes, kv.second.flops);
+        s += line; first = false;
+    }
+    s += "]";
+    if (buf && size) { const size_t n = s.size() < size - 1 ? s.size() : size - 1; memcpy(buf, s.data(), n); buf[n] = 0; }
+    if (reset) ctx->stats.clear();
+    return s.size() + 1;
+}
+
+static void * reg_get_proc_address(ggml_backend_reg_t, const char * name) {
+    if (!name) return NULL;
+    if (strcmp(name, "ggml_backend_get_features") == 0)      return (void *) get_features;
+    if (strcmp(name, "ggml_backend_mi355x_set_option") == 0) return (void *) set_option;
+    if (strcmp(name, "ggml_backend_mi355x_get_stats") == 0)  return (void *) get_stats;
+    return NULL;
+}
+
+static const struct ggml_backend_reg_i mi355x_reg_iface = {
+    /* .get_name         = */ reg_get_name,
+    /* .get_device_count = */ reg_get_device_count,
+    /* .get_device       = */ reg_get_device,
+    /* .get_proc_address = */ reg_get_proc_address,
+};
+
+static ggml_backend_buffer_type_t device_get_buffer_type(ggml_backend_dev_t dev) {
+    mi355x_reg_ctx * rctx = (mi355x_reg_ctx *) dev->reg->context;
+    for (size_t i = 0; i < rctx->devices.size(); ++i) if (&rctx->devices[i] == dev) return &rctx->bufts[i];
+    return NULL;
+}
+
+// ------------------------------------------------------------------------------------------------------
+// public entry points
+// ------------------------------------------------------------------------------------------------------
+
+extern "C" {
+
+ggml_backend_reg_t ggml_backend_mi355x_reg(void) {
+    static struct ggml_backend_reg reg;
+    static std::once_flag once;
+    std::call_once(once, [] {
+        mi355x_reg_ctx * ctx = new mi355x_reg_ctx;   // lives as long as the process, like the registry itself
+        const std::vector<int> & devs = gfx950_devices();
+        ctx->devices.reserve(devs.size());
+        ctx->bufts.reserve(devs.size());
+        reg = { GGML_BACKEND_API_VERSION, mi355x_reg_iface, ctx };
+        for (size_t i = 0; i < devs.size(); ++i) {
+            mi355x_device_ctx * d = new mi355x_device_ctx;
+            d->device = devs[i];
+            d->name   = std::string(GGML_MI355X_NAME) + std::to_string(i);
+            hipDeviceProp_t prop;
+            if (hipGetDeviceProperties(&prop, devs[i]) == hipSuccess) d->description = std::string(prop.name) + " (" + prop.gcnArchName + ")";
+            else { (void) hipGetLastError(); d->description = "AMD Instinct MI355X"; }
+            ctx->devices.push_back({ mi355x_device_iface, &reg, d });
+            ctx->bufts.push_back({ mi355x_buft_iface, &ctx->devices.back(), NULL });
+        }
+    });
+    return &reg;
+}
+
+int ggml_backend_mi355x_get_device_count(void) { return (int) gfx950_devices().size(); }
+
+ggml_backend_t ggml_backend_mi355x_init(int device) {
+    ggml_backend_reg_t reg = ggml_backend_mi355x_reg();
+    ggml_backend_dev_t dev = reg_get_device(reg, (size_t) device);
+    return dev ? device_init_backend(dev, NULL) : NULL;
+}
+
+bool ggml_backend_is_mi355x(ggml_backend_t backend) {
+    return backend != NULL && backend->iface.graph_compute == backend_graph_compute;
+}
+
+ggml_backend_buffer_type_t ggml_backend_mi355x_buffer_type(int device) {
+    ggml_backend_reg_t reg = ggml_backend_mi355x_reg();
+    ggml_backend_dev_t dev = reg_get_device(reg, (size_t) device);
+    return dev ? device_get_buffer_type(dev) : NULL;
+}
+
+// ggml_backend_registry::load_backend (ggml/src/ggml-backend-reg.cpp:227-271) rejects a library whose score is 0
+int ggml_backend_score(void) { return gfx950_devices().empty() ? 0 : 100; }
+
+ggml_backend_reg_t ggml_backend_init(void) { return ggml_backend_mi355x_reg(); }
+
+} // extern "C"

@@ -1,0 +1,371 @@
+// graph_compute for the MI355X backend: walks the nodes of a ggml graph in order on one HIP stream and
+// launches the hand-written kernels through their C ABI.  Takes the place of
+// ggml_backend_cpu_graph_compute -> ggml_graph_compute -> ggml_compute_forward
+// (ggml/src/ggml-cpu/ggml-cpu.cpp:149-169, ggml/src/ggml-cpu/ggml-cpu.c:3111, 1722).
+//
+// Neighbouring nodes that whisper always emits together are folded into one launch when the
+// intermediate result has no other reader in the graph:
+//     NORM -> MUL(w) -> ADD(b)                                    (src/whisper.cpp:2116-2121)
+//     MUL_MAT [-> ADD(bias)] [-> GELU | -> SCALE | -> ADD(resid)]  (src/whisper.cpp:2126-2249)
+//     MUL_MAT [-> ADD | -> SCALE] -> CPY(f32 -> f16, dense)        (src/whisper.cpp:2316-2351, 2564-2601)
+#include "backend.h"
+
+#include <string.h>
+#include <unordered_map>
+
+static mi355x_tensor to_view(const ggml_tensor * t) {
+    mi355x_tensor v;
+    v.data = t->data;
+    v.type = (int32_t) t->type;   // numeric values are shared with enum mi355x_type
+    v._pad = 0;
+    for (int i = 0; i < 4; ++i) { v.ne[i] = t->ne[i]; v.nb[i] = t->nb[i]; }
+    return v;
+}
+
+static bool type_in(enum ggml_type t, std::initializer_list<enum ggml_type> set) {
+    for (auto s : set) if (s == t) return true;
+    return false;
+}
+
+static bool is_view_op(enum ggml_op op) {
+    return op == GGML_OP_NONE || op == GGML_OP_RESHAPE || op == GGML_OP_VIEW || op == GGML_OP_PERMUTE || op == GGML_OP_TRANSPOSE;
+}
+
+// ------------------------------------------------------------------------------------------------------
+// supports_op: true only for (op, types, layout) tuples that have a kernel; everything else is left to the
+// scheduler's CPU fallback (ggml/src/ggml-backend.cpp:1013-1034).
+// ------------------------------------------------------------------------------------------------------
+
+bool mi355x_supports_op(const struct ggml_tensor * op) {
+    const ggml_tensor * s0 = op->src[0];
+    const ggml_tensor * s1 = op->src[1];
+    switch (op->op) {
+        case GGML_OP_NONE: case GGML_OP_RESHAPE: case GGML_OP_VIEW: case GGML_OP_PERMUTE: case GGML_OP_TRANSPOSE:
+            return true;
+        case GGML_OP_MUL_MAT:
+            if (!type_in(s0->type, {GGML_TYPE_Q5_0, GGML_TYPE_Q8_0, GGML_TYPE_F16, GGML_TYPE_F32})) return false;
+            if (!(s1->type == GGML_TYPE_F32 || (s1->type == GGML_TYPE_F16 && s0->type == GGML_TYPE_F16))) return false;
+            if (op->type != GGML_TYPE_F32) return false;
+            return s0->nb[0] == ggml_type_size(s0->type) && s1->nb[0] == ggml_type_size(s1->type) && op->nb[0] == sizeof(float);
+        case GGML_OP_ADD: case GGML_OP_MUL:
+            return s0->type == GGML_TYPE_F32 && s1->type == GGML_TYPE_F32 && op->type == GGML_TYPE_F32;
+        case GGML_OP_SCALE:
+            return s0->type == GGML_TYPE_F32 && op->type == GGML_TYPE_F32;
+        case GGML_OP_UNARY:
+            return ggml_get_unary_op(op) == GGML_UNARY_OP_GELU && s0->type == GGML_TYPE_F32 && op->type == GGML_TYPE_F32;
+        case GGML_OP_NORM:
+            return s0->type == GGML_TYPE_F32 && op->type == GGML_TYPE_F32 && s0->nb[0] == sizeof(float) && op->nb[0] == sizeof(float);
+        case GGML_OP_SOFT_MAX: {
+            float max_bias; memcpy(&max_bias, (const float *) op->op_params + 1, sizeof(float));
+            if (max_bias != 0.0f) return false;
+            if (s1 && !type_in(s1->type, {GGML_TYPE_F32, GGML_TYPE_F16})) return false;
+            return s0->type == GGML_TYPE_F32 && op->type == GGML_TYPE_F32 && s0->nb[0] == sizeof(float) && op->nb[0] == sizeof(float);
+        }
+        case GGML_OP_CPY: case GGML_OP_CONT: case GGML_OP_DUP: {
+            const ggml_tensor * d = op->op == GGML_OP_CPY ? s1 : op;
+            if (type_in(s0->type, {GGML_TYPE_F32, GGML_TYPE_F16}) && type_in(d->type, {GGML_TYPE_F32, GGML_TYPE_F16})) return true;
+            return s0->type == d->type && ggml_is_contiguous(s0) && ggml_is_contiguous(d) &&
+                   type_in(s0->type, {GGML_TYPE_I32, GGML_TYPE_Q5_0, GGML_TYPE_Q8_0});
+        }
+        case GGML_OP_GET_ROWS:
+            return type_in(s0->type, {GGML_TYPE_Q5_0, GGML_TYPE_Q8_0, GGML_TYPE_F16, GGML_TYPE_F32}) &&
+                   s1->type == GGML_TYPE_I32 && op->type == GGML_TYPE_F32 && s1->ne[0] * s1->ne[1] * s1->ne[2] <= 65535;
+        case GGML_OP_IM2COL: {
+            const int32_t is_2d = op->op_params[6];
+            return is_2d == 0 && op->type == GGML_TYPE_F16 && s1->type == GGML_TYPE_F32 && s1->nb[0] == sizeof(float) && s1->ne[3] == 1;
+        }
+        case GGML_OP_FLASH_ATTN_EXT: {
+            const ggml_tensor * k = op->src[1], * v = op->src[2], * m = op->src[3];
+            float max_bias, softcap;
+            memcpy(&max_bias, (const float *) op->op_params + 1, sizeof(float));
+            memcpy(&softcap,  (const float *) op->op_params + 2, sizeof(float));
+            if (max_bias != 0.0f || softcap != 0.0f) return false;
+            if (s0->type != GGML_TYPE_F32 || k->type != GGML_TYPE_F16 || v->type != GGML_TYPE_F16) return false;
+            if (m && m->type != GGML_TYPE_F16) return false;
+            return s0->ne[0] == 64 && k->ne[0] == 64 && v->ne[0] == 64;
+        }
+        case GGML_OP_CONCAT:
+            return s0->type == GGML_TYPE_F32 && s1->type == GGML_TYPE_F32 && op->type == GGML_TYPE_F32;
+        default:
+            return false;
+    }
+}
+
+// ------------------------------------------------------------------------------------------------------
+// profiling helpers
+// ------------------------------------------------------------------------------------------------------
+
+hipEvent_t mi355x_backend_ctx::take_event() {
+    if (!event_pool.empty()) { hipEvent_t e = event_pool.back(); event_pool.pop_back(); return e; }
+    hipEvent_t e = nullptr;
+    if (hipEventCreate(&e) != hipSuccess) { (void) hipGetLastError(); return nullptr; }
+    return e;
+}
+
+void mi355x_backend_ctx::drain_events() {
+    for (auto & p : pending) {
+        float ms = 0.0f;
+        if (p.start && p.stop && hipEventElapsedTime(&ms, p.start, p.stop) == hipSuccess) {
+            auto & s = stats[p.name];
+            s.calls += 1; s.ms += ms; s.bytes += p.bytes; s.flops += p.flops;
+        } else {
+            (void) hipGetLastError();
+        }
+        if (p.start) event_pool.push_back(p.start);
+        if (p.stop)  event_pool.push_back(p.stop);
+    }
+    pending.clear();
+}
+
+namespace {
+
+struct launch_scope {   // brackets one kernel launch with events when profiling
+    mi355x_backend_ctx * ctx;
+    mi355x_pending_event ev;
+    bool on;
+    launch_scope(mi355x_backend_ctx * c, const char * name, double bytes, double flops) : ctx(c), on(c->profile) {
+        if (!on) return;
+        ev.name = name; ev.bytes = bytes; ev.flops = flops;
+        ev.start = ctx->take_event(); ev.stop = ctx->take_event();
+        if (ev.start) (void) hipEventRecord(ev.start, ctx->stream);
+    }
+    ~launch_scope() {
+        if (!on) return;
+        if (ev.stop) (void) hipEventRecord(ev.stop, ctx->stream);
+        ctx->pending.push_back(ev);
+    }
+};
+
+double nbytes_of(const ggml_tensor * t) { return t ? (double) ggml_nbytes(t) : 0.0; }
+
+bool ranges_overlap(const ggml_tensor * a, const ggml_tensor * b) {
+    const char * a0 = (const char *) a->data, * b0 = (const char *) b->data;
+    return a0 < b0 + ggml_nbytes(b) && b0 < a0 + ggml_nbytes(a);
+}
+
+// row vector [ne0] that repeats over the rows of `like`
+bool is_row_vector_of(const ggml_tensor * v, const ggml_tensor * like) {
+    return v->type == GGML_TYPE_F32 && v->ne[0] == like->ne[0] && v->ne[1] == 1 && v->ne[2] == 1 && v->ne[3] == 1 && v->nb[0] == sizeof(float);
+}
+
+struct graph_runner {
+    mi355x_backend_ctx * ctx;
+    ggml_cgraph *        g;
+    std::unordered_map<const ggml_tensor *, int> readers;   // how many nodes of this graph read a tensor
+
+    graph_runner(mi355x_backend_ctx * c, ggml_cgraph * cg) : ctx(c), g(cg) {
+        if (!ctx->fuse) return;
+        readers.reserve((size_t) g->n_nodes * 2);
+        for (int i = 0; i < g->n_nodes; ++i) {
+            const ggml_tensor * n = g->nodes[i];
+            // each distinct tensor a node touches (sources and the tensor it is a view of) counts once
+            const ggml_tensor * seen[GGML_MAX_SRC + 1]; int ns = 0;
+            for (int s = 0; s <= GGML_MAX_SRC; ++s) {
+                const ggml_tensor * t = s < GGML_MAX_SRC ? n->src[s] : n->view_src;
+                if (!t) continue;
+                bool dup = false;
+                for (int k = 0; k < ns; ++k) dup = dup || seen[k] == t;
+                if (!dup) { seen[ns++] = t; readers[t] += 1; }
+            }
+        }
+    }
+
+    // `t` is read by exactly one node of the graph and is not a graph output
+    bool only_feeds_next(const ggml_tensor * t) const {
+        if (t->flags & GGML_TENSOR_FLAG_OUTPUT) return false;
+        auto it = readers.find(t);
+        return it != readers.end() && it->second == 1;
+    }
+
+    ggml_tensor * node_at(int i) const { return i < g->n_nodes ? g->nodes[i] : nullptr; }
+
+    // ---- MUL_MAT and what can be folded behind it; returns the number of nodes consumed --------------
+    int run_mul_mat(int i, int & status) {
+        ggml_tensor * mm = g->nodes[i];
+        const ggml_tensor * w = mm->src[0], * x = mm->src[1];
+        mi355x_epilogue epi = { 0, 1.0f, nullptr, nullptr };
+        ggml_tensor * last = mm;       // node whose value the fused kernel produces
+        ggml_tensor * out  = mm;       // tensor that receives it
+        int used = 1;
+
+        if (ctx->fuse && mm->ne[2] == 1 && mm->ne[3] == 1 && ggml_is_contiguous(mm)) {
+            auto same_layout = [&](const ggml_tensor * t) {
+                return t->type == GGML_TYPE_F32 && ggml_are_same_shape(t, mm) && ggml_is_contiguous(t);
+            };
+            // a dense RESHAPE of the running result (ggml_conv_1d reshapes its MUL_MAT, ggml/src/ggml.c:3899) is the same memory
+            auto hop_views = [&]() {
+                ggml_tensor * t = node_at(i + used);
+                while (t && t->op == GGML_OP_RESHAPE && t->src[0] == last && only_feeds_next(last) && ggml_is_contiguous(t)) {
+                    last = t; ++used; t = node_at(i + used);
+                }
+                return t;
+            };
+            ggml_tensor * n = hop_views();
+            // + bias
+            if (n && n->op == GGML_OP_ADD && n->src[0] == last && only_feeds_next(last) && same_layout(n) && n->src[1]->type == GGML_TYPE_F32) {
+                const ggml_tensor * b = n->src[1];
+                if (is_row_vector_of(b, mm)) {
+                    epi.flags |= MI355X_EPI_BIAS; epi.bias = b->data; last = n; ++used;
+                } else if (b->ne[0] == 1 && b->ne[1] == mm->ne[1] && b->ne[2] == 1 && b->ne[3] == 1 && ggml_is_contiguous(b)) {
+                    epi.flags |= MI355X_EPI_BIAS_COL; epi.bias = b->data; last = n; ++used;   // conv bias [1, d]
+                }
+                n = hop_views();
+            }
+            // + activation / scale / residual (at most one of them)
+            if (n && n->src[0] == last && only_feeds_next(last) && same_layout(n)) {
+                if (n->op == GGML_OP_UNARY && ggml_get_unary_op(n) == GGML_UNARY_OP_GELU) {
+                    epi.flags |= MI355X_EPI_GELU; last = n; ++used;
+                } else if (n->op == GGML_OP_SCALE) {
+                    epi.flags |= MI355X_EPI_SCALE; memcpy(&epi.scale, n->op_params, sizeof(float)); last = n; ++used;
+                } else if (n->op == GGML_OP_ADD && same_layout(n->src[1]) && n->src[1] != last) {
+                    epi.flags |= MI355X_EPI_RESIDUAL; epi.residual = n->src[1]->data; last = n; ++used;
+                }
+                n = node_at(i + used);
+            }
+            out = last;
+            // + store as f16 (K/V cache writes)
+            if (n && n->op == GGML_OP_CPY && n->src[0] == last && only_feeds_next(last) && !(epi.flags & MI355X_EPI_RESIDUAL) &&
+                n->src[1]->type == GGML_TYPE_F16 && ggml_is_contiguous(n->src[1]) && ggml_nelements(n->src[1]) == ggml_nelements(mm)) {
+                epi.flags |= MI355X_EPI_OUT_F16; out = n; ++used;
+            }
+            // the folded result must not land on memory the kernel is still reading
+            if (used > 1 && (ranges_overlap(out, x) || ranges_overlap(out, w))) {
+                epi = { 0, 1.0f, nullptr, nullptr }; out = mm; used = 1;
+            }
+        }
+
+        mi355x_tensor vw = to_view(w), vx = to_view(x), vd = to_view(mm);
+        vd.data = out->data;
+        if (epi.flags & MI355X_EPI_OUT_F16) {
+            vd.type = MI355X_TYPE_F16;
+            vd.nb[0] = 2; vd.nb[1] = 2 * (size_t) mm->ne[0]; vd.nb[2] = vd.nb[1] * mm->ne[1]; vd.nb[3] = vd.nb[2];
+        }
+        const double batch = (double) mm->ne[2] * mm->ne[3];
+        const double flops = 2.0 * mm->ne[0] * mm->ne[1] * w->ne[0] * batch;
+        const double bytes = nbytes_of(w) + nbytes_of(x) + (double) ggml_nelements(mm) * ((epi.flags & MI355X_EPI_OUT_F16) ? 2 : 4) +
+                             ((epi.flags & MI355X_EPI_RESIDUAL) ? nbytes_of(mm) : 0.0);
+        launch_scope ls(ctx, mi355x_mul_mat_kernel_name(&vw, &vx), bytes, flops);
+        status = mi355x_mul_mat(&vw, &vx, &vd, epi.flags ? &epi : nullptr, nullptr, 0, ctx->stream);
+        return used;
+    }
+
+    // ---- NORM [-> MUL(w) -> ADD(b)] ---------------------------------------------------------------------
+    int run_norm(int i, int & status) {
+        ggml_tensor * nm = g->nodes[i];
+        float eps; memcpy(&eps, nm->op_params, sizeof(float));
+        const float * w = nullptr, * b = nullptr;
+        ggml_tensor * out = nm;
+        int used = 1;
+        if (ctx->fuse) {
+            ggml_tensor * mul = node_at(i + 1), * add = node_at(i + 2);
+            if (mul && add && mul->op == GGML_OP_MUL && add->op == GGML_OP_ADD &&
+                mul->src[0] == nm && add->src[0] == mul && only_feeds_next(nm) && only_feeds_next(mul) &&
+                is_row_vector_of(mul->src[1], nm) && is_row_vector_of(add->src[1], nm) &&
+                ggml_are_same_shape(add, nm) && add->type == GGML_TYPE_F32 && add->nb[0] == sizeof(float)) {
+                w = (const float *) mul->src[1]->data; b = (const float *) add->src[1]->data;
+                out = add; used = 3;
+            }
+        }
+        mi355x_tensor vs = to_view(nm->src[0]), vd = to_view(out);
+        launch_scope ls(ctx, used == 3 ? "norm_affine" : "norm", nbytes_of(nm->src[0]) + nbytes_of(out), 0.0);
+        status = mi355x_norm(&vs, &vd, eps, w, b, ctx->stream);
+        return used;
+    }
+
+    int run_node(int i, int & status) {
+        ggml_tensor * n = g->nodes[i];
+        status = MI355X_OK;
+        if (ggml_is_empty(n) || is_view_op(n->op)) return 1;
+        const ggml_tensor * s0 = n->src[0], * s1 = n->src[1];
+        switch (n->op) {
+            case GGML_OP_MUL_MAT: return run_mul_mat(i, status);
+            case GGML_OP_NORM:    return run_norm(i, status);
+            case GGML_OP_ADD: case GGML_OP_MUL: {
+                mi355x_tensor a = to_view(s0), b = to_view(s1), d = to_view(n);
+                launch_scope ls(ctx, n->op == GGML_OP_ADD ? "add" : "mul", nbytes_of(s0) + nbytes_of(s1) + nbytes_of(n), 0.0);
+                status = mi355x_binary(n->op == GGML_OP_ADD ? 0 : 1, &a, &b, &d, ctx->stream);
+                return 1;
+            }
+            case GGML_OP_SCALE: {
+                float s; memcpy(&s, n->op_params, sizeof(float));
+                mi355x_tensor a = to_view(s0), d = to_view(n);
+                launch_scope ls(ctx, "scale", nbytes_of(s0) + nbytes_of(n), 0.0);
+                status = mi355x_scale(&a, &d, s, ctx->stream);
+                return 1;
+            }
+            case GGML_OP_UNARY: {
+                if (ggml_get_unary_op(n) != GGML_UNARY_OP_GELU) { status = MI355X_ERR_UNSUPPORTED; return 1; }
+                mi355x_tensor a = to_view(s0), d = to_view(n);
+                launch_scope ls(ctx, "gelu", nbytes_of(s0) + nbytes_of(n), 0.0);
+                status = mi355x_gelu(&a, &d, ctx->stream);
+                return 1;
+            }
+            case GGML_OP_SOFT_MAX: {
+                float scale; memcpy(&scale, n->op_params, sizeof(float));
+                mi355x_tensor a = to_view(s0), d = to_view(n), m;
+                if (s1) m = to_view(s1);
+                launch_scope ls(ctx, "soft_max", nbytes_of(s0) + nbytes_of(s1) + nbytes_of(n), 0.0);
+                status = mi355x_soft_max(&a, s1 ? &m : nullptr, &d, scale, ctx->stream);
+                return 1;
+            }
+            case GGML_OP_CPY: case GGML_OP_CONT: case GGML_OP_DUP: {
+                const ggml_tensor * dt = n->op == GGML_OP_CPY ? s1 : n;
+                mi355x_tensor a = to_view(s0), d = to_view(dt);
+                launch_scope ls(ctx, "cpy", nbytes_of(s0) + nbytes_of(dt), 0.0);
+                status = mi355x_cpy(&a, &d, ctx->stream);
+                return 1;
+            }
+            case GGML_OP_GET_ROWS: {
+                mi355x_tensor a = to_view(s0), b = to_view(s1), d = to_view(n);
+                launch_scope ls(ctx, "get_rows", 2.0 * nbytes_of(n), 0.0);
+                status = mi355x_get_rows(&a, &b, &d, ctx->stream);
+                return 1;
+            }
+            case GGML_OP_IM2COL: {
+                const int32_t * p = n->op_params;   // s0, s1, p0, p1, d0, d1, is_2D (ggml/src/ggml.c:3849)
+                mi355x_tensor a = to_view(s1), d = to_view(n);
+                launch_scope ls(ctx, "im2col", nbytes_of(s1) + nbytes_of(n), 0.0);
+                status = mi355x_im2col_1d(&a, &d, (int) s0->ne[0], p[0], p[2], p[4], ctx->stream);
+                return 1;
+            }
+            case GGML_OP_FLASH_ATTN_EXT: {
+                const ggml_tensor * k = n->src[1], * v = n->src[2], * m = n->src[3];
+                float scale; memcpy(&scale, n->op_params, sizeof(float));
+                mi355x_tensor vq = to_view(s0), vk = to_view(k), vv = to_view(v), vm, vd = to_view(n);
+                if (m) vm = to_view(m);
+                const double flops = 4.0 * s0->ne[1] * k->ne[1] * 64.0 * s0->ne[2] * s0->ne[3];
+                const double bytes = (double) ggml_nelements(s0) * 4 + 2.0 * (double) k->ne[0] * k->ne[1] * k->ne[2] * k->ne[3] * 2 + nbytes_of(n);
+                launch_scope ls(ctx, mi355x_flash_attn_ext_kernel_name(&vq, &vk), bytes, flops);
+                status = mi355x_flash_attn_ext(&vq, &vk, &vv, m ? &vm : nullptr, &vd, scale, nullptr, 0, ctx->stream);
+                return 1;
+            }
+            case GGML_OP_CONCAT: {
+                mi355x_tensor a = to_view(s0), b = to_view(s1), d = to_view(n);
+                launch_scope ls(ctx, "concat", 2.0 * nbytes_of(n), 0.0);
+                status = mi355x_concat(&a, &b, &d, n->op_params[0], ctx->stream);
+                return 1;
+            }
+            default:
+                status = MI355X_ERR_UNSUPPORTED;
+                return 1;
+        }
+    }
+};
+
+} // namespace
+
+enum ggml_status mi355x_graph_compute(mi355x_backend_ctx * ctx, struct ggml_cgraph * cgraph) {
+    HIP_TRY(hipSetDevice(ctx->device), return GGML_STATUS_FAILED);
+    graph_runner run(ctx, cgraph);
+    for (int i = 0; i < cgraph->n_nodes;) {
+        int status = MI355X_OK;
+        const int used = run.run_node(i, status);
+        if (status != MI355X_OK) {
+            const ggml_tensor * n = cgraph->nodes[i];
+            GGML_LOG_ERROR("ggml-mi355x: %s (%s) failed: %s\n", ggml_op_desc(n), n->name, mi355x_status_string(status));
+            return GGML_STATUS_FAILED;
+        }
+        i += used;
+    }
+    return GGML_STATUS_SUCCESS;
+}

@@ -1,0 +1,116 @@
+// Shared device/host helpers for the gfx950 kernels.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stddef.h>
+
+#include "mi355x_kernels.h"
+
+#define WAVE 64
+
+typedef _Float16 half_t;
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef float    float4_t  __attribute__((ext_vector_type(4)));
+typedef float    float16_t __attribute__((ext_vector_type(16)));
+
+// block formats (ggml/src/ggml-common.h:187-193, 209-214)
+#define QK 32
+struct __attribute__((packed)) blk_q5_0 { uint16_t d; uint8_t qh[4]; uint8_t qs[16]; };
+struct __attribute__((packed)) blk_q8_0 { uint16_t d; int8_t  qs[32]; };
+static_assert(sizeof(blk_q5_0) == 22, "q5_0 block is 22 bytes");
+static_assert(sizeof(blk_q8_0) == 34, "q8_0 block is 34 bytes");
+
+// 4-d tensor view passed to kernels by value
+struct tview {
+    char *  p;
+    int64_t ne0, ne1, ne2, ne3;
+    int64_t nb0, nb1, nb2, nb3;
+};
+
+static inline tview make_view(const mi355x_tensor * t) {
+    tview v;
+    v.p = (char *) t->data;
+    v.ne0 = t->ne[0]; v.ne1 = t->ne[1]; v.ne2 = t->ne[2]; v.ne3 = t->ne[3];
+    v.nb0 = (int64_t) t->nb[0]; v.nb1 = (int64_t) t->nb[1]; v.nb2 = (int64_t) t->nb[2]; v.nb3 = (int64_t) t->nb[3];
+    return v;
+}
+
+static inline int64_t nelements(const mi355x_tensor * t) { return t->ne[0]*t->ne[1]*t->ne[2]*t->ne[3]; }
+
+static inline size_t type_size(int type) {
+    switch (type) {
+        case MI355X_TYPE_F32:  return 4;
+        case MI355X_TYPE_F16:  return 2;
+        case MI355X_TYPE_I32:  return 4;
+        case MI355X_TYPE_Q5_0: return 22;
+        case MI355X_TYPE_Q8_0: return 34;
+        default: return 0;
+    }
+}
+static inline int blck_size(int type) { return (type == MI355X_TYPE_Q5_0 || type == MI355X_TYPE_Q8_0) ? QK : 1; }
+
+// dims 1..3 of `t` are laid out densely after dim 0 (rows may still be padded: nb1 is free)
+static inline bool is_contiguous(const mi355x_tensor * t) {
+    size_t ts = type_size(t->type);
+    int    bs = blck_size(t->type);
+    if (t->nb[0] != ts) return false;
+    size_t nb1 = ts * (size_t)(t->ne[0] / bs);
+    if (t->ne[1] > 1 && t->nb[1] != nb1) return false;
+    if (t->ne[2] > 1 && t->nb[2] != nb1 * (size_t) t->ne[1]) return false;
+    if (t->ne[3] > 1 && t->nb[3] != nb1 * (size_t) t->ne[1] * (size_t) t->ne[2]) return false;
+    return true;
+}
+
+static inline bool same_shape(const mi355x_tensor * a, const mi355x_tensor * b) {
+    return a->ne[0] == b->ne[0] && a->ne[1] == b->ne[1] && a->ne[2] == b->ne[2] && a->ne[3] == b->ne[3];
+}
+
+static inline int launch_status() {
+    hipError_t e = hipGetLastError();
+    return e == hipSuccess ? MI355X_OK : MI355X_ERR_HIP;
+}
+
+#ifdef __HIPCC__
+
+__device__ __forceinline__ float h2f(uint16_t h) {
+    half_t x;
+    __builtin_memcpy(&x, &h, 2);
+    return (float) x;
+}
+__device__ __forceinline__ uint16_t f2h_bits(float f) {
+    half_t x = (half_t) f;   // v_cvt_f16_f32: round-to-nearest-even, like the F16C conversion the CPU backend uses
+    uint16_t h;
+    __builtin_memcpy(&h, &x, 2);
+    return h;
+}
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, WAVE);
+    return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, WAVE));
+    return v;
+}
+
+// tanh-GELU in f32 (ggml/src/ggml-cpu/vec.h:432-434), with the clamps of ggml_vec_gelu_f32 (vec.h:443-457)
+__device__ __forceinline__ float gelu_f32(float x) {
+    if (x <= -10.0f) return 0.0f;
+    if (x >=  10.0f) return x;
+    const float u = 0.79788456080286535587989211986876f * x * (1.0f + 0.044715f * x * x);
+    // 0.5x(1+tanh(u)) = x / (1 + exp(-2u))
+    return x / (1.0f + __expf(-2.0f * u));
+}
+
+// unaligned little-endian loads from byte-addressed block data
+__device__ __forceinline__ uint32_t ld_u16(const uint8_t * p) { return *(const uint16_t *) p; }
+__device__ __forceinline__ uint32_t ld_u32_2(const uint8_t * p) {   // 2-byte aligned 32-bit load
+    return (uint32_t) *(const uint16_t *) p | ((uint32_t) *(const uint16_t *)(p + 2) << 16);
+}
+
+#endif // __HIPCC__

@@ -1,0 +1,141 @@
+// Row reductions: NORM (+ fused LayerNorm affine) and SOFT_MAX.  One 64-lane wavefront owns one row, so
+// the reductions are pure cross-lane shuffles with no LDS traffic and no block barrier; four rows share
+// a 256-thread block.  Both are HBM-bound: one read and one write of the row.
+#include "common.h"
+
+#define ROWS_PER_BLOCK 4
+#define NORM_MAX_V4    8      // rows up to 64*4*8 = 2048 floats are held in registers between the passes
+
+// ------------------------------------------------------------------------------------------------------
+// NORM (ggml/src/ggml-cpu/ops.cpp:3109-3158): mean, then variance of the centred values, then scale.
+// ------------------------------------------------------------------------------------------------------
+
+template <bool IN_REGS>
+__global__ void k_norm(tview s, tview d, int64_t nrows, float eps, const float * __restrict__ w, const float * __restrict__ b) {
+    const int     lane = threadIdx.x % WAVE;
+    const int64_t row  = (int64_t) blockIdx.x * ROWS_PER_BLOCK + threadIdx.x / WAVE;
+    if (row >= nrows) return;
+    const int64_t i1 = row % s.ne1, i2 = (row / s.ne1) % s.ne2, i3 = row / (s.ne1 * s.ne2);
+    const float * x = (const float *)(s.p + i1*s.nb1 + i2*s.nb2 + i3*s.nb3);
+    float *       y = (float *)(d.p + i1*d.nb1 + i2*d.nb2 + i3*d.nb3);
+    const int64_t ne0 = s.ne0;
+
+    if (IN_REGS) {
+        const int n4 = (int)(ne0 / 4);
+        float4 v[NORM_MAX_V4];
+        float sum = 0.0f;
+#pragma unroll
+        for (int j = 0; j < NORM_MAX_V4; ++j) {
+            const int c = lane + j * WAVE;
+            if (c < n4) { v[j] = ((const float4 *) x)[c]; sum += (v[j].x + v[j].y) + (v[j].z + v[j].w); }
+        }
+        const float mean = wave_sum(sum) / (float) ne0;
+        float sum2 = 0.0f;
+#pragma unroll
+        for (int j = 0; j < NORM_MAX_V4; ++j) {
+            const int c = lane + j * WAVE;
+            if (c < n4) {
+                v[j].x -= mean; v[j].y -= mean; v[j].z -= mean; v[j].w -= mean;
+                sum2 += (v[j].x*v[j].x + v[j].y*v[j].y) + (v[j].z*v[j].z + v[j].w*v[j].w);
+            }
+        }
+        const float scale = 1.0f / sqrtf(wave_sum(sum2) / (float) ne0 + eps);
+#pragma unroll
+        for (int j = 0; j < NORM_MAX_V4; ++j) {
+            const int c = lane + j * WAVE;
+            if (c < n4) {
+                float4 r = { v[j].x * scale, v[j].y * scale, v[j].z * scale, v[j].w * scale };
+                if (w) { const float4 ww = ((const float4 *) w)[c]; r.x *= ww.x; r.y *= ww.y; r.z *= ww.z; r.w *= ww.w; }
+                if (b) { const float4 bb = ((const float4 *) b)[c]; r.x += bb.x; r.y += bb.y; r.z += bb.z; r.w += bb.w; }
+                ((float4 *) y)[c] = r;
+            }
+        }
+    } else {
+        float sum = 0.0f;
+        for (int64_t c = lane; c < ne0; c += WAVE) sum += x[c];
+        const float mean = wave_sum(sum) / (float) ne0;
+        float sum2 = 0.0f;
+        for (int64_t c = lane; c < ne0; c += WAVE) { const float t = x[c] - mean; sum2 += t * t; }
+        const float scale = 1.0f / sqrtf(wave_sum(sum2) / (float) ne0 + eps);
+        for (int64_t c = lane; c < ne0; c += WAVE) {
+            float r = (x[c] - mean) * scale;
+            if (w) r *= w[c];
+            if (b) r += b[c];
+            y[c] = r;
+        }
+    }
+}
+
+extern "C" int mi355x_norm(const mi355x_tensor * src, const mi355x_tensor * dst, float eps, const float * w, const float * b, void * stream) {
+    if (!src || !dst || !(eps >= 0.0f)) return MI355X_ERR_INVALID;
+    if (src->type != MI355X_TYPE_F32 || dst->type != MI355X_TYPE_F32) return MI355X_ERR_UNSUPPORTED;
+    if (!same_shape(src, dst) || src->nb[0] != 4 || dst->nb[0] != 4) return MI355X_ERR_INVALID;
+    const int64_t nrows = src->ne[1] * src->ne[2] * src->ne[3];
+    if (nrows == 0 || src->ne[0] == 0) return MI355X_OK;
+    const int64_t grid = (nrows + ROWS_PER_BLOCK - 1) / ROWS_PER_BLOCK;
+    if (grid > 0x7fffffff) return MI355X_ERR_UNSUPPORTED;
+    hipStream_t st = (hipStream_t) stream;
+    auto al16 = [](const void * p, const size_t * nb) {
+        return (uintptr_t) p % 16 == 0 && nb[1] % 16 == 0 && nb[2] % 16 == 0 && nb[3] % 16 == 0;
+    };
+    const bool in_regs = src->ne[0] % 4 == 0 && src->ne[0] <= 4 * WAVE * NORM_MAX_V4 &&
+                         al16(src->data, src->nb) && al16(dst->data, dst->nb) &&
+                         (uintptr_t) w % 16 == 0 && (uintptr_t) b % 16 == 0;
+    if (in_regs) k_norm<true ><<<(unsigned) grid, ROWS_PER_BLOCK * WAVE, 0, st>>>(make_view(src), make_view(dst), nrows, eps, w, b);
+    else         k_norm<false><<<(unsigned) grid, ROWS_PER_BLOCK * WAVE, 0, st>>>(make_view(src), make_view(dst), nrows, eps, w, b);
+    return launch_status();
+}
+
+// ------------------------------------------------------------------------------------------------------
+// SOFT_MAX (ggml/src/ggml-cpu/ops.cpp:4641-4737), max_bias = 0
+// ------------------------------------------------------------------------------------------------------
+
+template <typename TM>
+__global__ void k_soft_max(tview s, tview d, const char * __restrict__ mask, int64_t mask_nb1, int64_t nrows, float scale) {
+    const int     lane = threadIdx.x % WAVE;
+    const int64_t row  = (int64_t) blockIdx.x * ROWS_PER_BLOCK + threadIdx.x / WAVE;
+    if (row >= nrows) return;
+    const int64_t i1 = row % s.ne1, i2 = (row / s.ne1) % s.ne2, i3 = row / (s.ne1 * s.ne2);
+    const float * x = (const float *)(s.p + i1*s.nb1 + i2*s.nb2 + i3*s.nb3);
+    float *       y = (float *)(d.p + i1*d.nb1 + i2*d.nb2 + i3*d.nb3);
+    const TM *    m = mask ? (const TM *)(mask + i1 * mask_nb1) : nullptr;   // the mask is shared by all heads
+    const int64_t ne0 = s.ne0;
+
+    float mx = -INFINITY;
+    for (int64_t c = lane; c < ne0; c += WAVE) {
+        const float v = x[c] * scale + (m ? (float) m[c] : 0.0f);
+        mx = fmaxf(mx, v);
+    }
+    mx = wave_max(mx);
+    float sum = 0.0f;
+    for (int64_t c = lane; c < ne0; c += WAVE) {
+        const float v = x[c] * scale + (m ? (float) m[c] : 0.0f);
+        const float e = (v == -INFINITY) ? 0.0f : __expf(v - mx);
+        y[c] = e;                                  // in-place safe: each lane rereads only what it wrote
+        sum += e;
+    }
+    const float inv = 1.0f / wave_sum(sum);
+    for (int64_t c = lane; c < ne0; c += WAVE) y[c] *= inv;
+}
+
+extern "C" int mi355x_soft_max(const mi355x_tensor * src, const mi355x_tensor * mask, const mi355x_tensor * dst, float scale, void * stream) {
+    if (!src || !dst) return MI355X_ERR_INVALID;
+    if (src->type != MI355X_TYPE_F32 || dst->type != MI355X_TYPE_F32) return MI355X_ERR_UNSUPPORTED;
+    if (!same_shape(src, dst) || src->nb[0] != 4 || dst->nb[0] != 4) return MI355X_ERR_INVALID;
+    if (mask) {
+        if (mask->type != MI355X_TYPE_F32 && mask->type != MI355X_TYPE_F16) return MI355X_ERR_UNSUPPORTED;
+        if (mask->ne[0] != src->ne[0] || mask->ne[1] < src->ne[1] || mask->nb[0] != type_size(mask->type)) return MI355X_ERR_INVALID;
+    }
+    const int64_t nrows = src->ne[1] * src->ne[2] * src->ne[3];
+    if (nrows == 0 || src->ne[0] == 0) return MI355X_OK;
+    const int64_t grid = (nrows + ROWS_PER_BLOCK - 1) / ROWS_PER_BLOCK;
+    if (grid > 0x7fffffff) return MI355X_ERR_UNSUPPORTED;
+    hipStream_t st = (hipStream_t) stream;
+    // when src aliases dst the first pass must not be overwritten before the second reads it: the kernel
+    // recomputes v from x in pass 2 and only then stores, lane-locally, so aliasing is safe.
+    if (mask && mask->type == MI355X_TYPE_F16)
+        k_soft_max<half_t><<<(unsigned) grid, ROWS_PER_BLOCK * WAVE, 0, st>>>(make_view(src), make_view(dst), (const char *) mask->data, (int64_t) mask->nb[1], nrows, scale);
+    else
+        k_soft_max<float ><<<(unsigned) grid, ROWS_PER_BLOCK * WAVE, 0, st>>>(make_view(src), make_view(dst), mask ? (const char *) mask->data : nullptr, mask ? (int64_t) mask->nb[1] : 0, nrows, scale);
+    return launch_status();
+}
