@@ -50,8 +50,13 @@ GGML_BACKEND_API int                ggml_backend_score(void);
  */
 
 /* Options: "fuse" (0/1: fold bias/activation/residual/LayerNorm-affine neighbours into one kernel, default 1),
- * "profile" (0/1: bracket every kernel with HIP events on the backend's stream, default 0).
- * The environment variables GGML_MI355X_FUSE and GGML_MI355X_PROFILE give the initial values. */
+ * "profile" (0/1: bracket every kernel with HIP events on the backend's stream, default 0),
+ * "exact" (0/1, default 0: 0 reproduces the two roundings that the reference's CPU backend applies — Q8_0-rounded
+ * activations in front of quantized MUL_MAT, f16 key-by-key V accumulation in FLASH_ATTN_EXT; 1 keeps f16 activations
+ * and f32 accumulators, which is closer to exact arithmetic and further from the reference).
+ * The environment variables GGML_MI355X_FUSE, GGML_MI355X_PROFILE and GGML_MI355X_EXACT give the initial values.
+ * backend == NULL addresses every live MI355X backend of the process (a host such as whisper.cpp keeps its
+ * backends private). */
 typedef int (*ggml_backend_mi355x_set_option_t)(ggml_backend_t backend, const char * name, int value);
 
 /* Per-kernel statistics gathered while "profile" is on: writes a JSON array

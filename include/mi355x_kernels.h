@@ -58,6 +58,10 @@ enum mi355x_epilogue_flags {
     MI355X_EPI_RESIDUAL = 8,   /* + residual[m,n] (f32, same shape and strides as dst)                         */
     MI355X_EPI_BIAS_COL = 16,  /* + bias[n]       (f32, one value per dst row n: conv bias [1,d], broadcast along ne0) */
     MI355X_EPI_OUT_F16  = 32,  /* dst is f16 instead of f32 (ggml CPY f32->f16 folded in)                      */
+    /* not epilogue parts, but options of the same call: */
+    MI355X_MM_EXACT_ACT = 64,  /* GEMM path: keep src1 at f16 precision instead of rounding it to Q8_0 first   */
+    MI355X_MM_WS_READY  = 128, /* GEMM path: `workspace` already holds the Q8_0-rounded src1 of this call
+                                  (left there by the previous call with the same src1): skip the rounding pass */
 };
 
 typedef struct mi355x_epilogue {
@@ -90,10 +94,12 @@ MI355X_API int mi355x_quantize_row_q8_0(const float * src, void * dst, int64_t k
  * src0: Q5_0 | Q8_0 | F16 | F32, ne0 = K contiguous.  src1: F32 | F16, ne0 = K contiguous.  dst: F32
  * (F16 with MI355X_EPI_OUT_F16), ne0 = M contiguous.  `epi` may be NULL.
  * Columns n <= MI355X_GEMV_MAX_COLS with a quantized src0 take the HBM-streaming GEMV path, which
- * quantizes src1 to Q8_0 in `workspace` exactly like the CPU backend does (ggml-cpu.c:1328-1363) and
+ * quantizes src1 to Q8_0 (in LDS) exactly like the CPU backend does (ggml-cpu.c:1328-1363) and
  * accumulates integer block dot products like ggml_vec_dot_q5_0_q8_0 / ggml_vec_dot_q8_0_q8_0
  * (ggml-cpu-quants.c:2930, 3597).  Everything else runs the MFMA GEMM (weights dequantized to f16 on the
- * way into LDS, f32 accumulation). */
+ * way into LDS, f32 accumulation).  With quantized weights the GEMM, too, first rounds src1 to Q8_0 — one
+ * pass that writes d*q as f16 into `workspace` (size from mi355x_mul_mat_workspace_size) — because that
+ * rounding is part of what the reference computes; MI355X_MM_EXACT_ACT turns it off. */
 #define MI355X_GEMV_MAX_COLS 8
 /* name of the kernel mi355x_mul_mat would launch for these operands ("mul_mat.gemm_q5_0", "mul_mat.gemv_q8_0", ...);
  * a static string, used to label profiles */
@@ -107,12 +113,15 @@ MI355X_API int    mi355x_mul_mat(const mi355x_tensor * src0, const mi355x_tensor
  * logit_softcap = 0 (the only values whisper uses):
  *   dst[:, h, n] = softmax_over_keys(scale * q[:, n, h] . k[:, key, h] + mask[key, n]) @ v[:, key, h]
  * q: F32 [D, N, H], k/v: F16 [D, KV, H] (D = 64), mask: F16 [KV, >=N] or NULL (-inf entries skip the
- * key), dst: F32 [D, H, N] contiguous.  `workspace` is used when the key range is split across
- * workgroups (small N); size from mi355x_flash_attn_ext_workspace_size. */
-MI355X_API const char * mi355x_flash_attn_ext_kernel_name(const mi355x_tensor * q, const mi355x_tensor * k);
+ * key), dst: F32 [D, H, N] contiguous.
+ * mode: MI355X_FA_F16_SEQ accumulates V in f16, key by key in order, as the reference does (ops.cpp:6793-6807) —
+ * with near-uniform attention over ~1500 keys that rounding sequence dominates the low bits of the result;
+ * MI355X_FA_F32 accumulates in f32 (closer to exact arithmetic, further from the reference). */
+enum mi355x_fa_mode { MI355X_FA_F16_SEQ = 0, MI355X_FA_F32 = 1 };
+MI355X_API const char * mi355x_flash_attn_ext_kernel_name(const mi355x_tensor * q, const mi355x_tensor * k, int mode);
 MI355X_API size_t mi355x_flash_attn_ext_workspace_size(const mi355x_tensor * q, const mi355x_tensor * k);
 MI355X_API int    mi355x_flash_attn_ext(const mi355x_tensor * q, const mi355x_tensor * k, const mi355x_tensor * v,
-                                        const mi355x_tensor * mask, const mi355x_tensor * dst, float scale,
+                                        const mi355x_tensor * mask, const mi355x_tensor * dst, float scale, int mode,
                                         void * workspace, size_t workspace_size, void * stream);
 
 /* elementwise / row ops ------------------------------------------------------------------------------ */
@@ -125,7 +134,8 @@ MI355X_API int mi355x_binary(int op, const mi355x_tensor * src0, const mi355x_te
 MI355X_API int mi355x_scale(const mi355x_tensor * src, const mi355x_tensor * dst, float s, void * stream);
 
 /* UNARY GELU (ggml/src/ggml-cpu/ops.cpp:2606-2643, vec.h:432-457): 0.5x(1+tanh(sqrt(2/pi) x (1+0.044715x^2))),
- * evaluated in f32 (the CPU backend looks the value up in an f16 table; the difference is below 1e-6 NMSE). */
+ * with the argument and the result rounded to f16 for |x| < 10, which is what the CPU backend's f16 lookup table
+ * amounts to (table built at ggml/src/ggml-cpu/ggml-cpu.c:3415-3423). */
 MI355X_API int mi355x_gelu(const mi355x_tensor * src, const mi355x_tensor * dst, void * stream);
 
 /* NORM (ggml/src/ggml-cpu/ops.cpp:3109-3158): y = (x - mean) / sqrt(var + eps) over ne0.  With w and/or b

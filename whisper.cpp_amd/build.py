@@ -34,7 +34,7 @@ COMMON = ["-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden", "-Wall", "-Wno-un
 
 KERNEL_SOURCES = ["misc.hip", "elementwise.hip", "rowwise.hip", "mul_mat.hip", "flash_attn.hip"]
 BACKEND_SOURCES = ["ggml-mi355x.cpp", "graph.cpp"]
-HARNESS_SOURCES = ["main.cpp", "synth_model.cpp", "op_cases.cpp"]
+HARNESS_SOURCES = ["main.cpp", "synth_model.cpp", "op_cases.cpp", "verify.cpp"]
 
 
 def _run(cmd, **kw):

@@ -59,6 +59,16 @@ struct mi355x_backend_ctx {
     hipStream_t stream = nullptr;
     bool        fuse    = true;
     bool        profile = false;
+    bool        exact   = false;   // true: f32 attention accumulators and un-rounded GEMM activations instead of the
+                                   // reference's f16-sequential / Q8_0-rounded arithmetic
+
+    // scratch for the kernels (grow-only), and which activations its Q8_0-rounded copy currently mirrors
+    void *       ws       = nullptr;
+    size_t       ws_size  = 0;
+    const void * ws_x     = nullptr;
+    int64_t      ws_x_ne[4] = {0, 0, 0, 0};
+    size_t       ws_x_nb[4] = {0, 0, 0, 0};
+    bool         reserve_workspace(size_t size);
 
     // profiling
     std::vector<mi355x_pending_event>         pending;

@@ -8,6 +8,8 @@
 #include <stdlib.h>
 #include <string.h>
 
+#include <algorithm>
+
 // ------------------------------------------------------------------------------------------------------
 // device discovery
 // ------------------------------------------------------------------------------------------------------
@@ -161,6 +163,11 @@ static const struct ggml_backend_buffer_type_i mi355x_buft_iface = {
 // backend / stream  (ggml_backend_i, ggml-backend-impl.h:87-117)
 // ------------------------------------------------------------------------------------------------------
 
+// live backend contexts, so that options and statistics can address all of them at once (backend == NULL)
+static std::mutex                        g_live_mutex;
+static std::vector<mi355x_backend_ctx *> g_live;
+static std::map<std::string, mi355x_kernel_stat> g_retired_stats;   // statistics of backends that were freed
+
 static ggml_guid_t backend_guid() {
     static ggml_guid guid = { 0x4d, 0x49, 0x33, 0x35, 0x35, 0x58, 0x2d, 0x67, 0x66, 0x78, 0x39, 0x35, 0x30, 0x2d, 0x76, 0x31 };
     return &guid;
@@ -180,7 +187,16 @@ static void backend_synchronize(ggml_backend_t backend) {
 static void backend_free(ggml_backend_t backend) {
     mi355x_backend_ctx * ctx = (mi355x_backend_ctx *) backend->context;
     backend_synchronize(backend);
+    {
+        std::lock_guard<std::mutex> lock(g_live_mutex);
+        g_live.erase(std::remove(g_live.begin(), g_live.end(), ctx), g_live.end());
+        for (auto & kv : ctx->stats) {
+            auto & s = g_retired_stats[kv.first];
+            s.calls += kv.second.calls; s.ms += kv.second.ms; s.bytes += kv.second.bytes; s.flops += kv.second.flops;
+        }
+    }
     for (hipEvent_t e : ctx->event_pool) (void) hipEventDestroy(e);
+    if (ctx->ws) (void) hipFree(ctx->ws);
     if (ctx->stream) (void) hipStreamDestroy(ctx->stream);
     delete ctx;
     delete backend;
@@ -250,6 +266,7 @@ static ggml_backend_t device_init_backend(ggml_backend_dev_t dev, const char *) 
     ctx->name    = dctx->name;
     ctx->fuse    = env_flag("GGML_MI355X_FUSE", true);
     ctx->profile = env_flag("GGML_MI355X_PROFILE", false);
+    ctx->exact   = env_flag("GGML_MI355X_EXACT", false);
     // default priority, blocking with respect to the null stream used by the buffer-level copies
     HIP_TRY(hipStreamCreate(&ctx->stream), { delete ctx; return NULL; });
     ggml_backend_t backend = new ggml_backend{
@@ -258,6 +275,10 @@ static ggml_backend_t device_init_backend(ggml_backend_dev_t dev, const char *) 
         /* .device  = */ dev,
         /* .context = */ ctx,
     };
+    {
+        std::lock_guard<std::mutex> lock(g_live_mutex);
+        g_live.push_back(ctx);
+    }
     return backend;
 }
 
@@ -317,21 +338,48 @@ static struct ggml_backend_feature * get_features(ggml_backend_reg_t) {
     return features;
 }
 
+static void ctx_synchronize(mi355x_backend_ctx * ctx) {
+    if (hipSetDevice(ctx->device) != hipSuccess || hipStreamSynchronize(ctx->stream) != hipSuccess) { (void) hipGetLastError(); return; }
+    if (!ctx->pending.empty()) ctx->drain_events();
+}
+
+// backend == NULL addresses every live MI355X backend of the process
 static int set_option(ggml_backend_t backend, const char * name, int value) {
-    if (!ggml_backend_is_mi355x(backend) || !name) return -1;
-    mi355x_backend_ctx * ctx = (mi355x_backend_ctx *) backend->context;
-    if (strcmp(name, "fuse") == 0)    { ctx->fuse = value != 0; return 0; }
-    if (strcmp(name, "profile") == 0) { backend_synchronize(backend); ctx->profile = value != 0; return 0; }
-    return -1;
+    if (!name || (backend && !ggml_backend_is_mi355x(backend))) return -1;
+    const bool is_fuse = strcmp(name, "fuse") == 0, is_profile = strcmp(name, "profile") == 0, is_exact = strcmp(name, "exact") == 0;
+    if (!is_fuse && !is_profile && !is_exact) return -1;
+    std::lock_guard<std::mutex> lock(g_live_mutex);
+    for (mi355x_backend_ctx * ctx : g_live) {
+        if (backend && ctx != (mi355x_backend_ctx *) backend->context) continue;
+        if (is_fuse) ctx->fuse = value != 0;
+        else if (is_exact) ctx->exact = value != 0;
+        else { ctx_synchronize(ctx); ctx->profile = value != 0; }
+    }
+    return 0;
 }
 
 static size_t get_stats(ggml_backend_t backend, char * buf, size_t size, int reset) {
-    if (!ggml_backend_is_mi355x(backend)) return 0;
-    mi355x_backend_ctx * ctx = (mi355x_backend_ctx *) backend->context;
-    backend_synchronize(backend);
+    if (backend && !ggml_backend_is_mi355x(backend)) return 0;
+    std::map<std::string, mi355x_kernel_stat> total;
+    {
+        std::lock_guard<std::mutex> lock(g_live_mutex);
+        auto add = [&](const std::map<std::string, mi355x_kernel_stat> & m) {
+            for (auto & kv : m) {
+                auto & s = total[kv.first];
+                s.calls += kv.second.calls; s.ms += kv.second.ms; s.bytes += kv.second.bytes; s.flops += kv.second.flops;
+            }
+        };
+        for (mi355x_backend_ctx * ctx : g_live) {
+            if (backend && ctx != (mi355x_backend_ctx *) backend->context) continue;
+            ctx_synchronize(ctx);
+            add(ctx->stats);
+            if (reset) ctx->stats.clear();
+        }
+        if (!backend) { add(g_retired_stats); if (reset) g_retired_stats.clear(); }
+    }
     std::string s = "[";
     bool first = true;
-    for (auto & kv : ctx->stats) {
+    for (auto & kv : total) {
         char line[512];
         snprintf(line, sizeof(line), "%s{\"kernel\": \"%s\", \"calls\": %lld, \"ms\": %.6f, \"bytes\": %.0f, \"flops\": %.0f}",
                  first ? "" : ", ", kv.first.c_str(), (long long) kv.second.calls, kv.second.ms, kv.second.bytes, kv.second.flops);
@@ -339,7 +387,6 @@ static size_t get_stats(ggml_backend_t backend, char * buf, size_t size, int res
     }
     s += "]";
     if (buf && size) { const size_t n = s.size() < size - 1 ? s.size() : size - 1; memcpy(buf, s.data(), n); buf[n] = 0; }
-    if (reset) ctx->stats.clear();
     return s.size() + 1;
 }
 

@@ -117,6 +117,18 @@ void mi355x_backend_ctx::drain_events() {
     pending.clear();
 }
 
+bool mi355x_backend_ctx::reserve_workspace(size_t size) {
+    if (size <= ws_size) return true;
+    // the stream may still be reading the old block
+    if (hipStreamSynchronize(stream) != hipSuccess) { (void) hipGetLastError(); return false; }
+    if (ws) (void) hipFree(ws);
+    ws = nullptr; ws_size = 0; ws_x = nullptr;
+    const size_t want = size + size / 2;
+    if (hipMalloc(&ws, want) != hipSuccess) { (void) hipGetLastError(); ws = nullptr; return false; }
+    ws_size = want;
+    return true;
+}
+
 namespace {
 
 struct launch_scope {   // brackets one kernel launch with events when profiling
@@ -244,8 +256,22 @@ struct graph_runner {
         const double flops = 2.0 * mm->ne[0] * mm->ne[1] * w->ne[0] * batch;
         const double bytes = nbytes_of(w) + nbytes_of(x) + (double) ggml_nelements(mm) * ((epi.flags & MI355X_EPI_OUT_F16) ? 2 : 4) +
                              ((epi.flags & MI355X_EPI_RESIDUAL) ? nbytes_of(mm) : 0.0);
-        launch_scope ls(ctx, mi355x_mul_mat_kernel_name(&vw, &vx), bytes, flops);
-        status = mi355x_mul_mat(&vw, &vx, &vd, epi.flags ? &epi : nullptr, nullptr, 0, ctx->stream);
+        // the GEMM rounds src1 to Q8_0 into the workspace first; consecutive MUL_MATs over the same activations
+        // (Q, K, V projections) share that copy
+        if (ctx->exact) epi.flags |= MI355X_MM_EXACT_ACT;
+        const size_t need = ctx->exact ? 0 : mi355x_mul_mat_workspace_size(&vw, &vx);
+        if (need) {
+            if (!ctx->reserve_workspace(need)) { status = MI355X_ERR_WORKSPACE; return used; }
+            const bool hit = ctx->ws_x == x->data && memcmp(ctx->ws_x_ne, x->ne, sizeof(x->ne)) == 0 && memcmp(ctx->ws_x_nb, x->nb, sizeof(x->nb)) == 0;
+            if (hit) epi.flags |= MI355X_MM_WS_READY;
+            ctx->ws_x = x->data; memcpy(ctx->ws_x_ne, x->ne, sizeof(x->ne)); memcpy(ctx->ws_x_nb, x->nb, sizeof(x->nb));
+            cached_x = x;
+        }
+        {
+            launch_scope ls(ctx, mi355x_mul_mat_kernel_name(&vw, &vx), bytes, flops);
+            status = mi355x_mul_mat(&vw, &vx, &vd, epi.flags ? &epi : nullptr, ctx->ws, ctx->ws_size, ctx->stream);
+        }
+        note_write(out);
         return used;
     }
 
@@ -269,7 +295,14 @@ struct graph_runner {
         mi355x_tensor vs = to_view(nm->src[0]), vd = to_view(out);
         launch_scope ls(ctx, used == 3 ? "norm_affine" : "norm", nbytes_of(nm->src[0]) + nbytes_of(out), 0.0);
         status = mi355x_norm(&vs, &vd, eps, w, b, ctx->stream);
+        note_write(out);
         return used;
+    }
+
+    // the workspace copy of the activations goes stale when something overwrites them
+    const ggml_tensor * cached_x = nullptr;
+    void note_write(const ggml_tensor * out) {
+        if (cached_x && ctx->ws_x && ranges_overlap(out, cached_x)) { ctx->ws_x = nullptr; cached_x = nullptr; }
     }
 
     int run_node(int i, int & status) {
@@ -277,6 +310,7 @@ struct graph_runner {
         status = MI355X_OK;
         if (ggml_is_empty(n) || is_view_op(n->op)) return 1;
         const ggml_tensor * s0 = n->src[0], * s1 = n->src[1];
+        if (n->op != GGML_OP_MUL_MAT && n->op != GGML_OP_NORM) note_write(n->op == GGML_OP_CPY ? s1 : n);
         switch (n->op) {
             case GGML_OP_MUL_MAT: return run_mul_mat(i, status);
             case GGML_OP_NORM:    return run_norm(i, status);
@@ -335,8 +369,9 @@ struct graph_runner {
                 if (m) vm = to_view(m);
                 const double flops = 4.0 * s0->ne[1] * k->ne[1] * 64.0 * s0->ne[2] * s0->ne[3];
                 const double bytes = (double) ggml_nelements(s0) * 4 + 2.0 * (double) k->ne[0] * k->ne[1] * k->ne[2] * k->ne[3] * 2 + nbytes_of(n);
-                launch_scope ls(ctx, mi355x_flash_attn_ext_kernel_name(&vq, &vk), bytes, flops);
-                status = mi355x_flash_attn_ext(&vq, &vk, &vv, m ? &vm : nullptr, &vd, scale, nullptr, 0, ctx->stream);
+                const int mode = ctx->exact ? MI355X_FA_F32 : MI355X_FA_F16_SEQ;
+                launch_scope ls(ctx, mi355x_flash_attn_ext_kernel_name(&vq, &vk, mode), bytes, flops);
+                status = mi355x_flash_attn_ext(&vq, &vk, &vv, m ? &vm : nullptr, &vd, scale, mode, nullptr, 0, ctx->stream);
                 return 1;
             }
             case GGML_OP_CONCAT: {
@@ -356,6 +391,7 @@ struct graph_runner {
 
 enum ggml_status mi355x_graph_compute(mi355x_backend_ctx * ctx, struct ggml_cgraph * cgraph) {
     HIP_TRY(hipSetDevice(ctx->device), return GGML_STATUS_FAILED);
+    ctx->ws_x = nullptr;   // tensors may have been rewritten between graphs
     graph_runner run(ctx, cgraph);
     for (int i = 0; i < cgraph->n_nodes;) {
         int status = MI355X_OK;

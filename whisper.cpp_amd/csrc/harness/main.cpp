@@ -1,0 +1,533 @@
+// mi355x-harness: drives the unmodified whisper.cpp host libraries with the MI355X backend plugged in
+// through ggml_backend_load(), next to ggml's own CPU backend on the same inputs.  Every subcommand prints
+// one JSON object per line on stdout; diagnostics go to stderr.
+//
+//   info                                      devices, features, supports_op table
+//   gen    --arch A --ftype T --out F         write a synthetic model file
+//   ops    [--filter S] [--quick] [--threads N] [--reps R] [--cpu-only]
+//                                             per-op parity (NMSE / bit-exactness) and timing, CPU vs MI355X
+//   model  --model F [--steps 32] [--threads N]
+//                                             whole-model parity: logits NMSE and greedy ids, teacher-forced
+//   verify --model F [--steps 3] [--threads N]
+//                                             per-node parity inside the real whisper graphs (unfused), CPU vs MI355X
+//   bench  --model F --what encoder|decoder|whisper-bench --backend gpu|cpu [--threads N] [--reps R] [--profile]
+//                                             timings with the whisper-bench protocol (examples/bench/bench.cpp:108-138)
+#include <math.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+#include <unistd.h>
+
+#include <algorithm>
+#include <chrono>
+#include <map>
+#include <string>
+#include <thread>
+#include <vector>
+
+#include "ggml.h"
+#include "ggml-alloc.h"
+#include "ggml-backend.h"
+#include "ggml-cpu.h"
+#include "whisper.h"
+
+#include "ggml-mi355x.h"
+#include "op_cases.h"
+#include "synth_model.h"
+#include "verify.h"
+
+// ---------------------------------------------------------------------------------------------------------------
+// small utilities
+// ---------------------------------------------------------------------------------------------------------------
+
+static double now_ms() {
+    return std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now().time_since_epoch()).count();
+}
+
+struct args {
+    std::map<std::string, std::string> kv;
+    bool has(const std::string & k) const { return kv.count(k) != 0; }
+    std::string str(const std::string & k, const std::string & d = "") const { auto it = kv.find(k); return it == kv.end() ? d : it->second; }
+    int num(const std::string & k, int d) const { auto it = kv.find(k); return it == kv.end() ? d : atoi(it->second.c_str()); }
+};
+
+static args parse_args(int argc, char ** argv, int first) {
+    args a;
+    for (int i = first; i < argc; ++i) {
+        std::string k = argv[i];
+        if (k.rfind("--", 0) != 0) continue;
+        k = k.substr(2);
+        if (i + 1 < argc && strncmp(argv[i + 1], "--", 2) != 0) a.kv[k] = argv[++i];
+        else a.kv[k] = "1";
+    }
+    return a;
+}
+
+static void quiet_log(enum ggml_log_level level, const char * text, void *) {
+    if (level == GGML_LOG_LEVEL_ERROR || level == GGML_LOG_LEVEL_WARN) fputs(text, stderr);
+}
+
+static std::string self_dir() {
+    char buf[4096];
+    ssize_t n = readlink("/proc/self/exe", buf, sizeof(buf) - 1);
+    if (n <= 0) return ".";
+    buf[n] = 0;
+    std::string s(buf);
+    return s.substr(0, s.find_last_of('/'));
+}
+
+// the plugin sits next to this binary
+static ggml_backend_reg_t load_plugin(bool required) {
+    const char * env = getenv("GGML_MI355X_PLUGIN");
+    const std::string path = env ? env : self_dir() + "/libggml-mi355x.so";
+    ggml_backend_reg_t reg = ggml_backend_load(path.c_str());
+    if (!reg && required) fprintf(stderr, "harness: could not load %s (no gfx950 device, or the library is missing)\n", path.c_str());
+    return reg;
+}
+
+static ggml_backend_t init_gpu_backend(ggml_backend_reg_t reg) {
+    if (!reg || ggml_backend_reg_dev_count(reg) == 0) return nullptr;
+    return ggml_backend_dev_init(ggml_backend_reg_dev_get(reg, 0), nullptr);
+}
+
+static int default_threads() {
+    const char * e = getenv("OMP_NUM_THREADS");
+    if (e && atoi(e) > 0) return atoi(e);
+    int n = (int) std::thread::hardware_concurrency();
+    return n > 0 ? std::min(n, 16) : 4;
+}
+
+static std::string json_escape(const std::string & s) {
+    std::string o;
+    for (char c : s) { if (c == '"' || c == '\\') o += '\\'; o += c; }
+    return o;
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// comparing two result buffers
+// ---------------------------------------------------------------------------------------------------------------
+
+struct cmp_result { double nmse, max_abs; bool bit_exact; int64_t n, n_nonfinite_mismatch; };
+
+static std::vector<float> to_f32(const std::vector<uint8_t> & raw, ggml_type type, int64_t n) {
+    std::vector<float> out((size_t) n);
+    if (type == GGML_TYPE_F32) memcpy(out.data(), raw.data(), (size_t) n * 4);
+    else if (type == GGML_TYPE_F16) {
+        const uint16_t * h = (const uint16_t *) raw.data();
+        for (int64_t i = 0; i < n; ++i) out[(size_t) i] = synth::f16_to_f32(h[i]);
+    } else out.assign((size_t) n, 0.0f);
+    return out;
+}
+
+static cmp_result compare(const std::vector<uint8_t> & a, const std::vector<uint8_t> & b, ggml_type type, int64_t n) {
+    cmp_result r{};
+    r.n = n;
+    r.bit_exact = a.size() == b.size() && memcmp(a.data(), b.data(), a.size()) == 0;
+    const std::vector<float> fa = to_f32(a, type, n), fb = to_f32(b, type, n);
+    double num = 0, den = 0, mx = 0;
+    for (int64_t i = 0; i < n; ++i) {
+        const float x = fa[(size_t) i], y = fb[(size_t) i];    // x: candidate, y: reference
+        if (!std::isfinite(x) || !std::isfinite(y)) {
+            if (!((std::isnan(x) && std::isnan(y)) || x == y)) r.n_nonfinite_mismatch++;
+            continue;
+        }
+        const double d = (double) x - y;
+        num += d * d; den += (double) y * y; mx = std::max(mx, fabs(d));
+    }
+    r.nmse = den > 0 ? num / den : (num > 0 ? INFINITY : 0.0);
+    r.max_abs = mx;
+    return r;
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// ops: one case on one backend
+// ---------------------------------------------------------------------------------------------------------------
+
+static uint64_t name_seed(const std::string & s) {
+    uint64_t h = 1469598103934665603ull;
+    for (char c : s) { h ^= (uint8_t) c; h *= 1099511628211ull; }
+    return h;
+}
+
+static void fill_input(const ops::input & in, const std::string & case_name) {
+    ggml_tensor * t = in.t;
+    const int64_t n = ggml_nelements(t);
+    const uint64_t seed = name_seed(case_name + "/" + t->name);
+    std::vector<uint8_t> data;
+    switch (in.kind) {
+        case ops::FILL_NORMAL:
+            data = synth::random_tensor((int) t->type, n, seed, in.scale, in.offset);
+            break;
+        case ops::FILL_ZERO_TAIL: {
+            data = synth::random_tensor((int) t->type, n, seed, in.scale, in.offset);
+            const size_t keep = (size_t)(in.range * in.rows) * ggml_type_size(t->type);
+            if (keep < data.size()) memset(data.data() + keep, 0, data.size() - keep);
+        } break;
+        case ops::FILL_IDS: {
+            data.resize((size_t) n * 4);
+            int32_t * ids = (int32_t *) data.data();
+            const bool all = n == in.range;     // "every row once", in a shuffled-looking but fixed order
+            for (int64_t i = 0; i < n; ++i) ids[i] = all ? (int32_t)((i * 2654435761ull + 17) % (uint64_t) in.range)
+                                                         : (int32_t)((seed + (uint64_t) i * 7919ull) % (uint64_t) in.range);
+        } break;
+        case ops::FILL_MASK: {
+            const int64_t kv = t->ne[0], nrow = t->ne[1];
+            std::vector<float> m((size_t) n, -INFINITY);
+            for (int64_t r = 0; r < std::min(nrow, in.rows); ++r)
+                for (int64_t k = 0; k < kv; ++k) {
+                    bool ok;
+                    if (in.range == 2) ok = k <= kv - in.rows + r;                         // causal
+                    else               ok = k < (kv + 1) / 2 || (k % in.rows) == r;        // beam-style cell ownership
+                    if (ok) m[(size_t)(r * kv + k)] = 0.0f;
+                }
+            if (t->type == GGML_TYPE_F32) { data.resize((size_t) n * 4); memcpy(data.data(), m.data(), data.size()); }
+            else { data.resize((size_t) n * 2); uint16_t * h = (uint16_t *) data.data(); for (int64_t i = 0; i < n; ++i) h[i] = synth::f32_to_f16(m[(size_t) i]); }
+        } break;
+    }
+    ggml_backend_tensor_set(t, data.data(), 0, ggml_nbytes(t));
+}
+
+struct run_out { std::vector<uint8_t> data; ggml_type type; int64_t n; double ms; bool ok; };
+
+static run_out run_case(const ops::op_case & c, ggml_backend_t backend, int reps) {
+    run_out out{};
+    ggml_init_params ip = { ggml_tensor_overhead() * 256 + ggml_graph_overhead(), nullptr, true };
+    ggml_context * ctx = ggml_init(ip);
+    ops::built b = c.build(ctx);
+    ggml_cgraph * gf = ggml_new_graph(ctx);
+    for (ggml_tensor * r : b.roots) ggml_build_forward_expand(gf, r);
+    ggml_backend_buffer_t buf = ggml_backend_alloc_ctx_tensors(ctx, backend);
+    if (!buf) { fprintf(stderr, "harness: allocation failed for %s\n", c.name.c_str()); ggml_free(ctx); return out; }
+    for (const ops::input & in : b.inputs) fill_input(in, c.name);
+    bool ok = ggml_backend_graph_compute(backend, gf) == GGML_STATUS_SUCCESS;      // first run doubles as warm-up
+    out.type = b.result->type; out.n = ggml_nelements(b.result);
+    out.data.resize(ggml_nbytes(b.result));
+    if (ok) ggml_backend_tensor_get(b.result, out.data.data(), 0, out.data.size());
+    double best = 1e30;
+    const bool rerunnable = b.result->op != GGML_OP_NONE || true;   // inputs are never overwritten by these graphs' roots
+    for (int r = 0; ok && rerunnable && r < reps; ++r) {
+        const double t0 = now_ms();
+        ok = ggml_backend_graph_compute(backend, gf) == GGML_STATUS_SUCCESS;
+        best = std::min(best, now_ms() - t0);
+    }
+    out.ms = reps > 0 ? best : 0.0;
+    out.ok = ok;
+    ggml_backend_buffer_free(buf);
+    ggml_free(ctx);
+    return out;
+}
+
+static int cmd_ops(const args & a) {
+    const bool cpu_only = a.has("cpu-only");
+    ggml_backend_reg_t reg = cpu_only ? nullptr : load_plugin(true);
+    ggml_backend_t gpu = init_gpu_backend(reg);
+    if (!cpu_only && !gpu) { printf("{\"error\": \"no MI355X backend\"}\n"); return 2; }
+    ggml_backend_t cpu = ggml_backend_cpu_init();
+    const int threads = a.num("threads", default_threads());
+    ggml_backend_cpu_set_n_threads(cpu, threads);
+    const int reps = a.num("reps", 3);
+    const std::string filter = a.str("filter");
+    const bool quick = a.has("quick");
+    int n_fail = 0, n_run = 0;
+    for (const ops::op_case & c : ops::all_cases()) {
+        if (!filter.empty() && c.name.find(filter) == std::string::npos) continue;
+        if (quick && c.heavy) continue;
+        fprintf(stderr, "case %s\n", c.name.c_str()); fflush(stderr);
+        run_out rc = run_case(c, cpu, a.has("time-cpu") ? reps : 0);
+        if (cpu_only) {
+            printf("{\"case\": \"%s\", \"op\": \"%s\", \"cpu_ok\": %s, \"n\": %lld}\n", c.name.c_str(), c.op.c_str(), rc.ok ? "true" : "false", (long long) rc.n);
+            ++n_run; continue;
+        }
+        run_out rg = run_case(c, gpu, reps);
+        cmp_result r = compare(rg.data, rc.data, rc.type, rc.n);
+        const bool pass = rg.ok && rc.ok && r.n_nonfinite_mismatch == 0 && (c.bit_exact ? r.bit_exact : r.nmse <= c.nmse_tol);
+        if (!pass) ++n_fail;
+        ++n_run;
+        printf("{\"case\": \"%s\", \"op\": \"%s\", \"pass\": %s, \"nmse\": %.3e, \"max_abs\": %.3e, \"bit_exact\": %s, \"want_bit_exact\": %s, "
+               "\"nmse_tol\": %.1e, \"nonfinite_mismatch\": %lld, \"n\": %lld, \"gpu_ms\": %.4f, \"cpu_ms\": %.4f, \"cpu_threads\": %d, "
+               "\"flops\": %.0f, \"bytes\": %.0f}\n",
+               c.name.c_str(), c.op.c_str(), pass ? "true" : "false", r.nmse, r.max_abs, r.bit_exact ? "true" : "false",
+               c.bit_exact ? "true" : "false", c.nmse_tol, (long long) r.n_nonfinite_mismatch, (long long) r.n, rg.ms, rc.ms, threads, c.flops, c.bytes);
+        fflush(stdout);
+    }
+    printf("{\"summary\": \"ops\", \"run\": %d, \"failed\": %d}\n", n_run, n_fail);
+    if (gpu) ggml_backend_free(gpu);
+    ggml_backend_free(cpu);
+    return n_fail ? 1 : 0;
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// info
+// ---------------------------------------------------------------------------------------------------------------
+
+static int cmd_info(const args &) {
+    ggml_backend_reg_t reg = load_plugin(false);
+    printf("{\"plugin_loaded\": %s, \"n_registered_devices\": %zu", reg ? "true" : "false", ggml_backend_dev_count());
+    if (reg) {
+        printf(", \"reg\": \"%s\", \"devices\": [", ggml_backend_reg_name(reg));
+        for (size_t i = 0; i < ggml_backend_reg_dev_count(reg); ++i) {
+            ggml_backend_dev_t dev = ggml_backend_reg_dev_get(reg, i);
+            size_t fr = 0, tot = 0; ggml_backend_dev_memory(dev, &fr, &tot);
+            printf("%s{\"name\": \"%s\", \"description\": \"%s\", \"type\": %d, \"free\": %zu, \"total\": %zu}", i ? ", " : "",
+                   ggml_backend_dev_name(dev), json_escape(ggml_backend_dev_description(dev)).c_str(), (int) ggml_backend_dev_type(dev), fr, tot);
+        }
+        printf("]");
+        auto feat = (ggml_backend_get_features_t) ggml_backend_reg_get_proc_address(reg, "ggml_backend_get_features");
+        if (feat) {
+            printf(", \"features\": {");
+            bool first = true;
+            for (ggml_backend_feature * f = feat(reg); f->name; ++f) { printf("%s\"%s\": \"%s\"", first ? "" : ", ", f->name, f->value); first = false; }
+            printf("}");
+        }
+    }
+    printf("}\n");
+    return 0;
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// gen
+// ---------------------------------------------------------------------------------------------------------------
+
+static int cmd_gen(const args & a) {
+    const synth::arch * arch = synth::find_arch(a.str("arch", "base"));
+    const int ftype = synth::ftype_from_name(a.str("ftype", "q5_0"));
+    const std::string out = a.str("out");
+    if (!arch || ftype < 0 || out.empty()) { fprintf(stderr, "usage: gen --arch micro|tiny|base|large-v3|large-v3-turbo --ftype f16|q8_0|q5_0 --out FILE [--seed N]\n"); return 2; }
+    const double t0 = now_ms();
+    const bool ok = synth::write_model(out, *arch, ftype, (uint64_t) a.num("seed", 1234));
+    printf("{\"gen\": \"%s\", \"arch\": \"%s\", \"ftype\": \"%s\", \"ok\": %s, \"ms\": %.1f}\n", out.c_str(), arch->name, a.str("ftype", "q5_0").c_str(), ok ? "true" : "false", now_ms() - t0);
+    return ok ? 0 : 1;
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// whisper contexts
+// ---------------------------------------------------------------------------------------------------------------
+
+static whisper_context * open_model(const std::string & path, bool use_gpu) {
+    whisper_context_params cp = whisper_context_default_params();
+    cp.use_gpu    = use_gpu;
+    cp.flash_attn = true;      // the FLASH_ATTN_EXT graphs are the ones under test (default is off, src/whisper.cpp:3620)
+    return whisper_init_from_file_with_params(path.c_str(), cp);
+}
+
+static int argmax(const float * v, int n, float * margin) {
+    int best = 0; float b1 = -INFINITY, b2 = -INFINITY;
+    for (int i = 0; i < n; ++i) {
+        if (v[i] > b1) { b2 = b1; b1 = v[i]; best = i; } else if (v[i] > b2) b2 = v[i];
+    }
+    if (margin) *margin = b1 - b2;
+    return best;
+}
+
+// whole-model parity: both contexts encode the same synthetic mel, then decode the same token history step by step
+// (teacher-forced with the CPU's greedy choice so that one flipped argmax cannot cascade); per step compares the
+// logits of the newest token.
+static int cmd_model(const args & a) {
+    const std::string path = a.str("model");
+    const int steps = a.num("steps", 32), threads = a.num("threads", default_threads());
+    if (path.empty()) { fprintf(stderr, "usage: model --model FILE [--steps N]\n"); return 2; }
+    if (!load_plugin(true)) { printf("{\"error\": \"no MI355X backend\"}\n"); return 2; }
+    whisper_context * gpu = open_model(path, true);
+    whisper_context * cpu = open_model(path, false);
+    if (!gpu || !cpu) { printf("{\"error\": \"model load failed\"}\n"); return 2; }
+    const int n_mels = whisper_model_n_mels(cpu), n_vocab = whisper_n_vocab(cpu);
+    const std::vector<float> mel = synth::synthetic_mel(n_mels, 3000, (uint64_t) a.num("seed", 7));
+    whisper_set_mel(gpu, mel.data(), 3000, n_mels);
+    whisper_set_mel(cpu, mel.data(), 3000, n_mels);
+    double t0 = now_ms();
+    const int eg = whisper_encode(gpu, 0, threads);
+    const double enc_gpu_ms = now_ms() - t0; t0 = now_ms();
+    const int ec = whisper_encode(cpu, 0, threads);
+    const double enc_cpu_ms = now_ms() - t0;
+    if (eg != 0 || ec != 0) { printf("{\"error\": \"encode failed\", \"gpu\": %d, \"cpu\": %d}\n", eg, ec); return 1; }
+
+    // prompt: <|sot|> <|en|> <|transcribe|> <|notimestamps|>  (4-token batch: exercises the n_tokens > 1 path)
+    std::vector<whisper_token> hist = { whisper_token_sot(cpu), whisper_token_lang(cpu, whisper_lang_id("en")),
+                                        whisper_token_transcribe(cpu), whisper_token_not(cpu) };
+    int n_past = 0, n_same = 0, n_total = 0;
+    double worst_nmse = 0, min_margin = 1e30, sum_nmse = 0;
+    std::vector<whisper_token> feed = hist;
+    bool all_ok = true;
+    for (int s = 0; s < steps; ++s) {
+        const int rg = whisper_decode(gpu, feed.data(), (int) feed.size(), n_past, threads);
+        const int rc = whisper_decode(cpu, feed.data(), (int) feed.size(), n_past, threads);
+        if (rg != 0 || rc != 0) { printf("{\"error\": \"decode failed\", \"step\": %d, \"gpu\": %d, \"cpu\": %d}\n", s, rg, rc); return 1; }
+        // logits of every fed token are returned; compare all rows, sample from the last
+        const int rows = (int) feed.size();
+        const float * lg = whisper_get_logits(gpu), * lc = whisper_get_logits(cpu);
+        double num = 0, den = 0;
+        for (int64_t i = 0; i < (int64_t) rows * n_vocab; ++i) { const double d = (double) lg[i] - lc[i]; num += d * d; den += (double) lc[i] * lc[i]; }
+        const double nmse = den > 0 ? num / den : 0;
+        float margin = 0;
+        const int tok_c = argmax(lc + (size_t)(rows - 1) * n_vocab, n_vocab, &margin);
+        const int tok_g = argmax(lg + (size_t)(rows - 1) * n_vocab, n_vocab, nullptr);
+        worst_nmse = std::max(worst_nmse, nmse); sum_nmse += nmse; min_margin = std::min(min_margin, (double) margin);
+        n_same += tok_c == tok_g; ++n_total;
+        printf("{\"step\": %d, \"n_tokens\": %d, \"n_past\": %d, \"logits_nmse\": %.3e, \"cpu_token\": %d, \"gpu_token\": %d, \"top1_top2_margin\": %.4e}\n",
+               s, rows, n_past, nmse, tok_c, tok_g, margin);
+        if (!(nmse <= 1e-3)) all_ok = false;
+        n_past += rows;
+        feed.assign(1, tok_c);
+    }
+    const bool pass = all_ok && n_same == n_total;
+    printf("{\"summary\": \"model\", \"model\": \"%s\", \"steps\": %d, \"ids_identical\": %d, \"worst_logits_nmse\": %.3e, \"mean_logits_nmse\": %.3e, "
+           "\"min_top1_top2_margin\": %.4e, \"encode_gpu_ms_first_call\": %.2f, \"encode_cpu_ms\": %.2f, \"cpu_threads\": %d, \"pass\": %s}\n",
+           json_escape(path).c_str(), n_total, n_same, worst_nmse, sum_nmse / std::max(1, n_total), min_margin, enc_gpu_ms, enc_cpu_ms, threads, pass ? "true" : "false");
+    whisper_free(gpu); whisper_free(cpu);
+    return pass ? 0 : 1;
+}
+
+// per-node parity on the graphs whisper builds: conv + encoder + cross, one prompt batch, a few single-token steps,
+// one 5-token batch (the shape of a beam-search step)
+static int cmd_verify(const args & a) {
+    const std::string path = a.str("model");
+    const int steps = a.num("steps", 3), threads = a.num("threads", default_threads());
+    if (path.empty()) { fprintf(stderr, "usage: verify --model FILE [--steps N]\n"); return 2; }
+    const char * env = getenv("GGML_MI355X_PLUGIN");
+    if (!verify::load_plugin_hooked(env ? env : self_dir() + "/libggml-mi355x.so")) { printf("{\"error\": \"no MI355X backend\"}\n"); return 2; }
+    verify::set_threads(threads);
+    verify::set_enabled(false);                       // worst-case reserve graphs run on uninitialised data
+    whisper_context * gpu = open_model(path, true);
+    if (!gpu) { printf("{\"error\": \"model load failed\"}\n"); return 2; }
+    verify::set_enabled(true);
+    const int n_mels = whisper_model_n_mels(gpu);
+    const std::vector<float> mel = synth::synthetic_mel(n_mels, 3000, (uint64_t) a.num("seed", 7));
+    whisper_set_mel(gpu, mel.data(), 3000, n_mels);
+    int bad = 0;
+    if (whisper_encode(gpu, 0, threads) != 0) return 1;
+    bad += verify::report("encode");
+    std::vector<whisper_token> prompt = { whisper_token_sot(gpu), whisper_token_lang(gpu, whisper_lang_id("en")), whisper_token_transcribe(gpu), whisper_token_not(gpu) };
+    if (whisper_decode(gpu, prompt.data(), (int) prompt.size(), 0, threads) != 0) return 1;
+    bad += verify::report("decode_prompt4");
+    int n_past = (int) prompt.size();
+    for (int s = 0; s < steps; ++s) {
+        float m; whisper_token t = argmax(whisper_get_logits(gpu), whisper_n_vocab(gpu), &m);
+        if (whisper_decode(gpu, &t, 1, n_past++, threads) != 0) return 1;
+    }
+    bad += verify::report("decode_single");
+    std::vector<whisper_token> five = { 11, 22, 33, 44, 55 };
+    if (whisper_decode(gpu, five.data(), 5, n_past, threads) != 0) return 1;
+    bad += verify::report("decode_batch5");
+    printf("{\"summary\": \"verify\", \"model\": \"%s\", \"nodes_over_tol\": %d, \"pass\": %s}\n", json_escape(path).c_str(), bad, bad == 0 ? "true" : "false");
+    whisper_free(gpu);
+    return bad == 0 ? 0 : 1;
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// bench
+// ---------------------------------------------------------------------------------------------------------------
+
+// whisper.h does not expose the backends of a state, so the options and statistics calls address every live MI355X
+// backend of the process (backend == NULL).
+static void plugin_set_option(ggml_backend_reg_t reg, const char * name, int value) {
+    if (!reg) return;
+    auto set = (ggml_backend_mi355x_set_option_t) ggml_backend_reg_get_proc_address(reg, "ggml_backend_mi355x_set_option");
+    if (set) set(nullptr, name, value);
+}
+
+static std::string plugin_stats(ggml_backend_reg_t reg, bool reset) {
+    if (!reg) return "[]";
+    auto get = (ggml_backend_mi355x_get_stats_t) ggml_backend_reg_get_proc_address(reg, "ggml_backend_mi355x_get_stats");
+    if (!get) return "[]";
+    const size_t need = get(nullptr, nullptr, 0, 0);
+    std::string s(need + 1, '\0');
+    get(nullptr, &s[0], s.size(), reset ? 1 : 0);
+    s.resize(strlen(s.c_str()));
+    return s;
+}
+
+static double median(std::vector<double> v) {
+    if (v.empty()) return 0;
+    std::sort(v.begin(), v.end());
+    return v[v.size() / 2];
+}
+
+static int cmd_bench(const args & a) {
+    const std::string path = a.str("model"), what = a.str("what", "encoder"), be = a.str("backend", "gpu");
+    const int threads = a.num("threads", default_threads()), reps = a.num("reps", 5), warmup = a.num("warmup", 2);
+    if (path.empty()) { fprintf(stderr, "usage: bench --model FILE --what encoder|decoder|whisper-bench --backend gpu|cpu\n"); return 2; }
+    const bool use_gpu = be == "gpu";
+    ggml_backend_reg_t reg = use_gpu ? load_plugin(true) : nullptr;
+    if (use_gpu && !reg) { printf("{\"error\": \"no MI355X backend\"}\n"); return 2; }
+    const bool profile = use_gpu && a.has("profile");
+    if (use_gpu && a.has("no-fuse")) setenv("GGML_MI355X_FUSE", "0", 1);
+    whisper_context * ctx = open_model(path, use_gpu);
+    if (!ctx) { printf("{\"error\": \"model load failed\"}\n"); return 2; }
+    const int n_mels = whisper_model_n_mels(ctx);
+    const std::vector<float> mel = synth::synthetic_mel(n_mels, 3000, 7);
+    whisper_set_mel(ctx, mel.data(), 3000, n_mels);
+
+    if (what == "encoder") {
+        for (int i = 0; i < warmup; ++i) if (whisper_encode(ctx, 0, threads) != 0) return 1;
+        if (profile) { plugin_set_option(reg, "profile", 1); plugin_stats(reg, true); }
+        std::vector<double> wall, enc;
+        for (int i = 0; i < reps; ++i) {
+            whisper_reset_timings(ctx);
+            const double t0 = now_ms();
+            if (whisper_encode(ctx, 0, threads) != 0) return 1;
+            wall.push_back(now_ms() - t0);
+            whisper_timings * t = whisper_get_timings(ctx);
+            enc.push_back(t ? t->encode_ms : 0.0);
+            delete t;
+        }
+        printf("{\"bench\": \"encoder\", \"backend\": \"%s\", \"threads\": %d, \"reps\": %d, \"encode_ms_median\": %.4f, \"encode_ms_min\": %.4f, "
+               "\"wall_ms_median\": %.4f, \"profiled\": %s, \"kernels\": %s, \"model\": \"%s\"}\n",
+               be.c_str(), threads, reps, median(enc), *std::min_element(enc.begin(), enc.end()), median(wall), profile ? "true" : "false",
+               profile ? plugin_stats(reg, true).c_str() : "[]", json_escape(path).c_str());
+    } else if (what == "decoder") {
+        // 5-token batches with a growing self-attention cache: the per-step work of a 5-beam search
+        // (src/whisper.cpp:6089-6117), driven through whisper_decode like the batch-5 leg of whisper-bench.
+        const int n_steps = a.num("steps", 224), batch = a.num("batch", 5);
+        if (whisper_encode(ctx, 0, threads) != 0) return 1;
+        std::vector<whisper_token> tok((size_t) batch, 0);
+        for (int i = 0; i < warmup; ++i) if (whisper_decode(ctx, tok.data(), batch, i, threads) != 0) return 1;
+        if (profile) { plugin_set_option(reg, "profile", 1); plugin_stats(reg, true); }
+        std::vector<double> per_rep;
+        for (int r = 0; r < reps; ++r) {
+            const double t0 = now_ms();
+            for (int i = 0; i < n_steps; ++i) {
+                for (int j = 0; j < batch; ++j) tok[(size_t) j] = (whisper_token)((i * 131 + j * 17) % 50000);
+                if (whisper_decode(ctx, tok.data(), batch, i, threads) != 0) return 1;
+            }
+            per_rep.push_back(now_ms() - t0);
+        }
+        const double ms = median(per_rep);
+        printf("{\"bench\": \"decoder\", \"backend\": \"%s\", \"threads\": %d, \"reps\": %d, \"steps\": %d, \"batch\": %d, \"total_ms_median\": %.3f, "
+               "\"ms_per_step\": %.5f, \"steps_per_s\": %.2f, \"batch_tokens_per_s\": %.2f, \"profiled\": %s, \"kernels\": %s, \"model\": \"%s\"}\n",
+               be.c_str(), threads, reps, n_steps, batch, ms, ms / n_steps, 1000.0 * n_steps / ms, 1000.0 * n_steps * batch / ms,
+               profile ? "true" : "false", profile ? plugin_stats(reg, true).c_str() : "[]", json_escape(path).c_str());
+    } else {   // whisper-bench protocol, verbatim counts (examples/bench/bench.cpp:86-138)
+        whisper_token tokens[512]; memset(tokens, 0, sizeof(tokens));
+        if (whisper_encode(ctx, 0, threads) != 0) return 1;
+        if (whisper_decode(ctx, tokens, 256, 0, threads) != 0) return 1;
+        if (whisper_decode(ctx, tokens, 1, 256, threads) != 0) return 1;
+        whisper_reset_timings(ctx);
+        if (whisper_encode(ctx, 0, threads) != 0) return 1;
+        for (int i = 0; i < 256; i++) if (whisper_decode(ctx, tokens, 1, i, threads) != 0) return 1;
+        for (int i = 0; i < 64; i++)  if (whisper_decode(ctx, tokens, 5, 0, threads) != 0) return 1;
+        for (int i = 0; i < 16; i++)  if (whisper_decode(ctx, tokens, 256, 0, threads) != 0) return 1;
+        whisper_timings * t = whisper_get_timings(ctx);
+        printf("{\"bench\": \"whisper-bench\", \"backend\": \"%s\", \"threads\": %d, \"encode_ms\": %.3f, \"decode_ms_per_token\": %.4f, "
+               "\"batchd_ms_per_token\": %.4f, \"prompt_ms_per_token\": %.4f, \"model\": \"%s\"}\n",
+               be.c_str(), threads, t->encode_ms, t->decode_ms, t->batchd_ms, t->prompt_ms, json_escape(path).c_str());   // already per token (src/whisper.cpp:4256-4260)
+        delete t;
+    }
+    whisper_free(ctx);
+    return 0;
+}
+
+int main(int argc, char ** argv) {
+    if (argc < 2) { fprintf(stderr, "usage: %s info|gen|ops|model|verify|bench [options]\n", argv[0]); return 2; }
+    ggml_log_set(quiet_log, nullptr);
+    whisper_log_set(quiet_log, nullptr);
+    const std::string cmd = argv[1];
+    const args a = parse_args(argc, argv, 2);
+    if (cmd == "info")  return cmd_info(a);
+    if (cmd == "gen")   return cmd_gen(a);
+    if (cmd == "ops")   return cmd_ops(a);
+    if (cmd == "model") return cmd_model(a);
+    if (cmd == "verify") return cmd_verify(a);
+    if (cmd == "bench") return cmd_bench(a);
+    fprintf(stderr, "unknown command %s\n", cmd.c_str());
+    return 2;
+}

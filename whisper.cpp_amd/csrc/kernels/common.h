@@ -98,13 +98,15 @@ __device__ __forceinline__ float wave_max(float v) {
     return v;
 }
 
-// tanh-GELU in f32 (ggml/src/ggml-cpu/vec.h:432-434), with the clamps of ggml_vec_gelu_f32 (vec.h:443-457)
+// tanh-GELU as ggml_vec_gelu_f32 evaluates it (ggml/src/ggml-cpu/vec.h:432-457): outside (-10, 10) the clamps, inside
+// a lookup in a table indexed by f16(x) that holds f16(gelu(f32(f16(x)))) — i.e. argument and result rounded to f16.
 __device__ __forceinline__ float gelu_f32(float x) {
     if (x <= -10.0f) return 0.0f;
     if (x >=  10.0f) return x;
-    const float u = 0.79788456080286535587989211986876f * x * (1.0f + 0.044715f * x * x);
+    const float xh = (float)(half_t) x;
+    const float u  = 0.79788456080286535587989211986876f * xh * (1.0f + 0.044715f * xh * xh);
     // 0.5x(1+tanh(u)) = x / (1 + exp(-2u))
-    return x / (1.0f + __expf(-2.0f * u));
+    return (float)(half_t)(xh / (1.0f + __expf(-2.0f * u)));
 }
 
 // unaligned little-endian loads from byte-addressed block data

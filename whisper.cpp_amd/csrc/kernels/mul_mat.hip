@@ -304,6 +304,32 @@ __global__ void __launch_bounds__(256, 2) k_gemm_mfma(mm_args a) {
 }
 
 // ------------------------------------------------------------------------------------------------------
+// src1 -> Q8_0 -> f16: what the CPU backend's MUL_MAT actually multiplies with (ggml-cpu.c:1328-1363 converts src1
+// to the weights' vec_dot_type with quantize_row_q8_0, ggml-cpu-quants.c:808-865).  One pass per src1, shared by
+// every MUL_MAT that reads the same activations; the GEMM then streams f16 instead of f32.
+// ------------------------------------------------------------------------------------------------------
+
+__global__ void k_round_act_q8_0(const char * __restrict__ x, half_t * __restrict__ out, int64_t K, int64_t N,
+                                 int64_t x_nb1, int64_t x_nb2, int64_t nbatch2, int64_t x_nb3) {
+    // 8 lanes per 32-value block, 4 values each
+    const int64_t t   = (int64_t) blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t k4  = K / 4;
+    const int64_t b   = blockIdx.y;                    // batch index (ne2*ne3 flattened)
+    if (t >= k4 * N) return;                           // K is a multiple of 32: whole 8-lane groups leave together
+    const int64_t n = t / k4, c = t % k4;
+    const char * xr = x + n * x_nb1 + (b % nbatch2) * x_nb2 + (b / nbatch2) * x_nb3;
+    const float4 v = *(const float4 *)(xr + c * 16);
+    float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
+    amax = fmaxf(amax, __shfl_xor(amax, 1, 8));
+    amax = fmaxf(amax, __shfl_xor(amax, 2, 8));
+    amax = fmaxf(amax, __shfl_xor(amax, 4, 8));
+    const float d  = h2f(f2h_bits(amax / 127.0f));     // the block scale is stored as f16
+    const float id = amax != 0.0f ? 127.0f / amax : 0.0f;
+    half4_t o = { (half_t)(d * rintf(v.x * id)), (half_t)(d * rintf(v.y * id)), (half_t)(d * rintf(v.z * id)), (half_t)(d * rintf(v.w * id)) };
+    *(half4_t *)(out + (b * N + n) * K + c * 4) = o;
+}
+
+// ------------------------------------------------------------------------------------------------------
 // quantized GEMV (N <= 8)
 // ------------------------------------------------------------------------------------------------------
 
@@ -546,14 +572,16 @@ extern "C" const char * mi355x_mul_mat_kernel_name(const mi355x_tensor * src0, c
     }
 }
 
+// the GEMM with quantized weights rounds src1 to Q8_0 into `workspace` as f16 [ne13*ne12][N][K]; the GEMV does it in LDS
 extern "C" size_t mi355x_mul_mat_workspace_size(const mi355x_tensor * src0, const mi355x_tensor * src1) {
-    (void) src0; (void) src1;
-    return 0;   // activations are quantized into LDS; no device scratch is needed
+    if (!src0 || !src1) return 0;
+    if (blck_size(src0->type) == 1 || src1->type != MI355X_TYPE_F32 || mm_path(src0, src1) != MM_GEMM) return 0;
+    const size_t n = (size_t) src1->ne[0] * src1->ne[1] * src1->ne[2] * src1->ne[3] * 2;
+    return (n + 255) / 256 * 256;
 }
 
 extern "C" int mi355x_mul_mat(const mi355x_tensor * src0, const mi355x_tensor * src1, const mi355x_tensor * dst,
                               const mi355x_epilogue * epi, void * workspace, size_t workspace_size, void * stream) {
-    (void) workspace; (void) workspace_size;
     if (!src0 || !src1 || !dst) return MI355X_ERR_INVALID;
     const int t0 = src0->type, t1 = src1->type;
     if (t0 != MI355X_TYPE_Q5_0 && t0 != MI355X_TYPE_Q8_0 && t0 != MI355X_TYPE_F16 && t0 != MI355X_TYPE_F32) return MI355X_ERR_UNSUPPORTED;
@@ -589,12 +617,27 @@ extern "C" int mi355x_mul_mat(const mi355x_tensor * src0, const mi355x_tensor * 
     if (nbatch > 65535) return MI355X_ERR_UNSUPPORTED;
 
     const int path = mm_path(src0, src1);
+    const bool quant = blck_size(t0) > 1;
     if (path == MM_GEMV) {
         return t0 == MI355X_TYPE_Q8_0 ? launch_gemv_n<MI355X_TYPE_Q8_0>(a, st) : launch_gemv_n<MI355X_TYPE_Q5_0>(a, st);
     }
     if (path == MM_GEMM) {
         dim3 grid((unsigned)((a.M + GB_M - 1) / GB_M), (unsigned)((a.N + GB_N - 1) / GB_N), (unsigned) nbatch);
         if (grid.y > 65535) return MI355X_ERR_UNSUPPORTED;
+        if (quant && t1 == MI355X_TYPE_F32 && !(flags & MI355X_MM_EXACT_ACT)) {
+            const size_t need = mi355x_mul_mat_workspace_size(src0, src1);
+            if (!workspace || workspace_size < need || (uintptr_t) workspace % 16 != 0) return MI355X_ERR_WORKSPACE;
+            if (!(flags & MI355X_MM_WS_READY)) {
+                const int64_t threads = a.K / 4 * a.N;
+                dim3 qgrid((unsigned)((threads + 255) / 256), (unsigned) nbatch);
+                k_round_act_q8_0<<<qgrid, 256, 0, st>>>(a.x, (half_t *) workspace, a.K, a.N, a.x_nb1, a.x_nb2, a.ne12, a.x_nb3);
+            }
+            a.x = (const char *) workspace;
+            a.x_nb1 = a.K * 2; a.x_nb2 = a.N * a.K * 2; a.x_nb3 = a.ne12 * a.N * a.K * 2;
+            if (t0 == MI355X_TYPE_Q5_0) k_gemm_mfma<MI355X_TYPE_Q5_0, MI355X_TYPE_F16><<<grid, 256, 0, st>>>(a);
+            else                        k_gemm_mfma<MI355X_TYPE_Q8_0, MI355X_TYPE_F16><<<grid, 256, 0, st>>>(a);
+            return launch_status();
+        }
         if (t1 == MI355X_TYPE_F16) {
             k_gemm_mfma<MI355X_TYPE_F16, MI355X_TYPE_F16><<<grid, 256, 0, st>>>(a);
         } else switch (t0) {
