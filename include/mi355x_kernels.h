@@ -5,7 +5,9 @@
  * ne[]/nb[] convention as ggml: ne[0] is the contiguous dimension, nb[i] is the byte stride of
  * dimension i), launches asynchronously on the HIP stream handed in as `stream` (a hipStream_t passed
  * as void*, NULL = default stream) and returns MI355X_OK or a negative error code.  Nothing here
- * allocates device memory; ops that need scratch take a caller-provided workspace.
+ * allocates device memory; ops that need scratch take a caller-provided workspace.  (The one piece of
+ * library-owned device state is the 128 KiB GELU table in a __device__ array, filled by a synchronous
+ * copy the first time GELU is used on a device.)
  *
  * Each declaration cites the function of the reference's CPU backend whose results it reproduces
  * (paths relative to the whisper.cpp tree).
@@ -134,8 +136,9 @@ MI355X_API int mi355x_binary(int op, const mi355x_tensor * src0, const mi355x_te
 MI355X_API int mi355x_scale(const mi355x_tensor * src, const mi355x_tensor * dst, float s, void * stream);
 
 /* UNARY GELU (ggml/src/ggml-cpu/ops.cpp:2606-2643, vec.h:432-457): 0.5x(1+tanh(sqrt(2/pi) x (1+0.044715x^2))),
- * with the argument and the result rounded to f16 for |x| < 10, which is what the CPU backend's f16 lookup table
- * amounts to (table built at ggml/src/ggml-cpu/ggml-cpu.c:3415-3423). */
+ * read for |x| < 10 from a 65536-entry table indexed by f16(x), exactly like the CPU backend (table built at
+ * ggml/src/ggml-cpu/ggml-cpu.c:3415-3423).  The library builds the same table on the host on first use (same
+ * formula, same libm) and keeps a copy in a __device__ array. */
 MI355X_API int mi355x_gelu(const mi355x_tensor * src, const mi355x_tensor * dst, void * stream);
 
 /* NORM (ggml/src/ggml-cpu/ops.cpp:3109-3158): y = (x - mean) / sqrt(var + eps) over ne0.  With w and/or b

@@ -290,8 +290,11 @@ void oracle_norm(const float * x, float * y, int64_t ne0, int64_t nrows, float e
  * GELU (ggml_vec_gelu_f32 with GGML_GELU_FP16, ggml/src/ggml-cpu/vec.h:428-457; table built at
  * ggml/src/ggml-cpu/ggml-cpu.c:3415-3423): x -> f16 -> table[f16] where table = f16(gelu_f32(f32(f16)))
  * ------------------------------------------------------------------------------------------------------- */
+/* The reference's x86 objects are built with FMA contraction: of this expression only 1 + (0.044715 x) x fuses.  Written
+ * out like this (the file is compiled with -ffp-contract=off) all finite table entries match the reference bit for bit. */
 static float gelu_f32(float x) {
-    return 0.5f * x * (1.0f + tanhf(0.79788456080286535587989211986876f * x * (1.0f + 0.044715f * x * x)));
+    const float inner = fmaf(0.044715f * x, x, 1.0f);
+    return 0.5f * x * (1.0f + tanhf(0.79788456080286535587989211986876f * x * inner));
 }
 void oracle_gelu(const float * x, float * y, int64_t n) {
     for (int64_t i = 0; i < n; ++i) {

@@ -77,6 +77,8 @@ def libs():
         cpu.ggml_backend_cpu_init.restype = P
         cpu.ggml_backend_cpu_set_n_threads.argtypes = [P, C.c_int]
         cpu.quantize_row_q8_0.argtypes = [P, P, C.c_int64]
+        # the first ggml_init fills the f16 -> f32 lookup table that GGML_FP16_TO_FP32 reads in the non-F16C objects
+        base.ggml_free(base.ggml_init(_InitParams(1024, None, False)))
         _libs = (base, cpu)
     return _libs
 

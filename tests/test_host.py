@@ -1,0 +1,83 @@
+"""CPU-only checks of the host side: the ABI surface of the two libraries, the synthetic-model writer against the
+reference's loader and quantizers, the op-case graphs on the reference's CPU backend, and the failure modes."""
+from __future__ import annotations
+
+import re
+import subprocess
+import sys
+from pathlib import Path
+
+import pytest
+
+from conftest import ROOT, run_harness
+
+
+def exported(lib: Path) -> set[str]:
+    out = subprocess.run(["nm", "-D", "--defined-only", str(lib)], stdout=subprocess.PIPE, text=True, check=True).stdout
+    return {line.split()[-1] for line in out.splitlines() if line.strip()}
+
+
+def test_kernel_library_exports_every_declared_symbol(pkg):
+    header = (ROOT / "include" / "mi355x_kernels.h").read_text()
+    declared = set(re.findall(r"MI355X_API\s+[\w\s\*]+?\b(mi355x_\w+)\s*\(", header))
+    assert len(declared) >= 20
+    if not pkg.KERNELS_LIB.exists():
+        pytest.skip("kernel library not built")
+    assert declared <= exported(pkg.KERNELS_LIB), declared - exported(pkg.KERNELS_LIB)
+    lib = pkg.kernels()                                # loads without a GPU; every ctypes signature binds
+    assert lib.mi355x_abi_version() == 1
+    assert lib.mi355x_status_string(-1).decode().startswith("unsupported")
+
+
+def test_plugin_exports_the_ggml_entry_points_and_does_not_link_the_checker(pkg):
+    if not pkg.PLUGIN_LIB.exists():
+        pytest.skip("plugin not built")
+    header = (ROOT / "include" / "ggml-mi355x.h").read_text()
+    declared = set(re.findall(r"GGML_BACKEND_API\s+[\w\s\*]+?\b(ggml_backend_\w+)\s*\(", header))
+    assert {"ggml_backend_init", "ggml_backend_score", "ggml_backend_mi355x_reg"} <= declared
+    assert declared <= exported(pkg.PLUGIN_LIB), declared - exported(pkg.PLUGIN_LIB)
+    needed = subprocess.run(["readelf", "-d", str(pkg.PLUGIN_LIB)], stdout=subprocess.PIPE, text=True, check=True).stdout
+    libs = set(re.findall(r"NEEDED.*\[(.+?)\]", needed))
+    assert "libmi355x_kernels.so" in libs
+    # the product never links the CPU backend or the restatement: ggml-base symbols are resolved by the host process
+    assert not any("ggml-cpu" in l or "oracle" in l or "whisper" in l for l in libs), libs
+
+
+def test_missing_extension_fails_loudly(pkg, monkeypatch, tmp_path):
+    monkeypatch.setattr(pkg, "_lib", None)
+    monkeypatch.setattr(pkg, "KERNELS_LIB", tmp_path / "libmi355x_kernels.so")
+    with pytest.raises(pkg.MissingExtension):
+        pkg.kernels()
+
+
+def test_writer_quantizers_and_f16_match_the_reference(harness):
+    rc, rows = run_harness(harness, ["selftest"])
+    assert rc == 0 and rows[-1] == {"summary": "selftest", "failed": 0}, rows
+
+
+def test_synthetic_model_is_accepted_by_the_unmodified_loader(harness, tmp_path):
+    model = tmp_path / "micro-q5_0.bin"
+    rc, rows = run_harness(harness, ["gen", "--arch", "micro", "--ftype", "q5_0", "--out", str(model)])
+    assert rc == 0 and rows[-1]["ok"]
+    # whisper_init_from_file_with_params + whisper_encode + whisper_decode on the reference's CPU backend
+    rc, rows = run_harness(harness, ["bench", "--model", str(model), "--what", "encoder", "--backend", "cpu", "--reps", "1", "--warmup", "0", "--threads", "4"])
+    assert rc == 0 and rows[-1]["encode_ms_median"] > 0
+    rc, rows = run_harness(harness, ["bench", "--model", str(model), "--what", "decoder", "--backend", "cpu", "--reps", "1", "--warmup", "1", "--steps", "6", "--threads", "4"])
+    assert rc == 0 and rows[-1]["steps"] == 6
+    for ftype in ("q8_0", "f16"):
+        m2 = tmp_path / f"micro-{ftype}.bin"
+        run_harness(harness, ["gen", "--arch", "micro", "--ftype", ftype, "--out", str(m2)])
+        rc, rows = run_harness(harness, ["bench", "--model", str(m2), "--what", "encoder", "--backend", "cpu", "--reps", "1", "--warmup", "0", "--threads", "4"])
+        assert rc == 0
+
+
+def test_every_op_case_builds_and_runs_on_the_cpu_backend(harness):
+    rc, rows = run_harness(harness, ["ops", "--cpu-only", "--quick", "--threads", "8"], timeout=600)
+    assert rc == 0
+    cases = [r for r in rows if "case" in r]
+    assert len(cases) >= 80 and all(r["cpu_ok"] for r in cases)
+
+
+def test_bench_refuses_more_than_one_gpu():
+    res = subprocess.run([sys.executable, str(ROOT / "bench.py"), "--gpus", "2"], stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True)
+    assert res.returncode == 2 and "one GPU" in res.stderr

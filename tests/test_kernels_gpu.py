@@ -1,0 +1,341 @@
+"""GPU parity of the HIP kernels, called through the C ABI of include/mi355x_kernels.h with device memory owned by
+torch, against the CPU restatement in oracle/ on the same seeded inputs.
+
+Bars: bit-exact for dequantization, gathers, copies/conversions, IM2COL and the f32 elementwise ops; for the
+floating-point kernels the tolerance is written next to each check (the north-star per-op bound is NMSE <= 5e-4 against
+the CPU backend; the reference-faithful paths are held to <= 1e-6)."""
+from __future__ import annotations
+
+import ctypes as C
+
+import numpy as np
+import pytest
+
+torch = pytest.importorskip("torch")
+pytestmark = pytest.mark.gpu
+
+RNG = np.random.default_rng(7)
+
+
+def rnd(shape, scale=1.0, offset=0.0):
+    return (RNG.normal(size=shape) * scale + offset).astype(np.float32)
+
+
+@pytest.fixture(scope="module")
+def gpu(pkg):
+    if not torch.cuda.is_available():
+        pytest.fail("no GPU visible: the gpu-marked tests must run on the MI355X box")
+    lib = pkg.kernels()
+    assert lib.mi355x_device_is_gfx950(0) == 1
+
+    class G:
+        dev = torch.device("cuda:0")
+        stream = C.c_void_p(0)
+
+        @staticmethod
+        def up(a: np.ndarray):
+            a = np.ascontiguousarray(a)
+            if a.dtype == np.uint16:
+                a = a.view(np.int16)
+            return torch.from_numpy(a).to(G.dev)
+
+        @staticmethod
+        def down(t, dtype=None):
+            torch.cuda.synchronize()
+            a = t.cpu().numpy()
+            return a.view(dtype) if dtype is not None else a
+
+    return G
+
+
+def run_mul_mat(pkg, gpu, wtype, wdata, x, k, m, flags=0, bias=None, resid=None, scale=1.0, out_f16=False):
+    lib = pkg.kernels()
+    d_w, d_x = gpu.up(wdata), gpu.up(x)
+    n = x.shape[0]
+    d_y = torch.empty((n, m), dtype=torch.float16 if out_f16 else torch.float32, device=gpu.dev)
+    tw = pkg.tensor(d_w, wtype, ne=[k, m])
+    tx = pkg.tensor(d_x, pkg.F32)
+    ty = pkg.tensor(d_y, pkg.F16 if out_f16 else pkg.F32)
+    ws_size = lib.mi355x_mul_mat_workspace_size(tw, tx)
+    ws = torch.empty(max(ws_size, 16), dtype=torch.uint8, device=gpu.dev)
+    epi = pkg.Epilogue()
+    epi.flags, epi.scale = flags | (pkg.EPI_OUT_F16 if out_f16 else 0), scale
+    keep = []
+    if bias is not None:
+        keep.append(gpu.up(bias)); epi.bias = keep[-1].data_ptr()
+    if resid is not None:
+        keep.append(gpu.up(resid)); epi.residual = keep[-1].data_ptr()
+    pkg.check(lib.mi355x_mul_mat(tw, tx, ty, C.byref(epi) if epi.flags else None, ws.data_ptr(), ws_size, gpu.stream), "mul_mat")
+    name = lib.mi355x_mul_mat_kernel_name(tw, tx).decode()
+    return gpu.down(d_y).astype(np.float32), name
+
+
+# ------------------------------------------------------------------------------------------------------------------
+
+@pytest.mark.parametrize("wtype", ["Q5_0", "Q8_0"])
+def test_dequantize_row_bit_exact(pkg, oracle, gpu, wtype):
+    t = getattr(pkg, wtype)
+    k = 32 * 4099                                        # odd number of blocks
+    blocks = RNG.integers(0, 256, size=(k // 32, pkg.BLOCK_BYTES[t]), dtype=np.uint8)      # arbitrary bytes: every scale pattern incl. inf / nan / subnormal
+    d_b = gpu.up(blocks)
+    d_y = torch.empty(k, dtype=torch.float32, device=gpu.dev)
+    pkg.check(pkg.kernels().mi355x_dequantize_row(t, d_b.data_ptr(), d_y.data_ptr(), k, gpu.stream))
+    got, want = gpu.down(d_y).view(np.uint32), oracle.dequantize(t, blocks, 32).reshape(-1).view(np.uint32)
+    nan = np.isnan(want.view(np.float32))
+    assert np.array_equal(got[~nan], want[~nan]) and np.array_equal(np.isnan(got.view(np.float32)), nan)
+    # empty input is a no-op
+    assert pkg.kernels().mi355x_dequantize_row(t, d_b.data_ptr(), d_y.data_ptr(), 0, gpu.stream) == 0
+    assert pkg.kernels().mi355x_dequantize_row(t, d_b.data_ptr(), d_y.data_ptr(), 33, gpu.stream) == -2
+
+
+def test_quantize_row_q8_0_matches_activation_quantizer(pkg, oracle, gpu):
+    x = rnd((64, 256), 2.0)
+    x[0, :32] = 0.0
+    x[1, :32] = np.arange(32) - 15.5
+    d_x = gpu.up(x)
+    d_q = torch.empty(x.size // 32 * 34, dtype=torch.uint8, device=gpu.dev)
+    pkg.check(pkg.kernels().mi355x_quantize_row_q8_0(d_x.data_ptr(), d_q.data_ptr(), x.size, gpu.stream))
+    assert np.array_equal(gpu.down(d_q).reshape(64, -1), oracle.quantize(oracle.Q8_0, x, act=True))
+
+
+@pytest.mark.parametrize("wtype", ["Q5_0", "Q8_0"])
+@pytest.mark.parametrize("shape", [(512, 2048, 1500), (1280, 1280, 129), (512, 130, 9), (32, 64, 200), (5120, 1280, 5), (1280, 5120, 1), (512, 1001, 3), (1280, 51866, 5), (256, 96, 8)])
+def test_mul_mat_quantized(pkg, oracle, gpu, wtype, shape):
+    k, m, n = shape
+    if m > 20000 and wtype == "Q5_0":
+        pytest.skip("one logits-sized case is enough")
+    t = getattr(pkg, wtype)
+    blocks = oracle.quantize(t, rnd((m, k), 0.02))
+    x = rnd((n, k))
+    got, name = run_mul_mat(pkg, gpu, t, blocks, x, k, m)
+    assert ("gemv" in name) == (n <= 8)
+    if n * m * k <= 2e9:
+        want = oracle.mul_mat(t, blocks, x)
+    else:                                                   # keep the scalar oracle to seconds: check a slab of rows
+        sel = np.r_[0:64, m - 64:m]
+        want = oracle.mul_mat(t, blocks[sel], x)
+        got = got[:, sel]
+    # both paths reproduce the reference's Q8_0 rounding of the activations: NMSE <= 1e-6 (GEMV: integer dot products, <= 1e-10)
+    assert oracle.nmse(got, want) <= (1e-10 if n <= 8 else 1e-6)
+
+
+@pytest.mark.parametrize("wtype", ["F16", "F32"])
+@pytest.mark.parametrize("shape", [(1280, 1280, 300), (240, 512, 200), (37, 50, 11), (1280, 640, 1)])
+def test_mul_mat_float_weights(pkg, oracle, gpu, wtype, shape):
+    k, m, n = shape
+    t = getattr(pkg, wtype)
+    w = rnd((m, k), 0.02)
+    wdata = oracle.f32_to_f16_bits(w) if t == pkg.F16 else w
+    x = rnd((n, k))
+    got, _ = run_mul_mat(pkg, gpu, t, wdata, x, k, m)
+    assert oracle.nmse(got, oracle.mul_mat(t, wdata, x)) <= 1e-6        # f16 operands, f32 accumulation
+
+
+def test_mul_mat_exact_activation_mode_is_closer_to_float64(pkg, oracle, gpu):
+    k, m, n = 1280, 256, 100
+    blocks = oracle.quantize(pkg.Q5_0, rnd((m, k), 0.02))
+    x = rnd((n, k))
+    exact = x.astype(np.float64) @ oracle.dequantize(pkg.Q5_0, blocks, k).astype(np.float64).T
+    faithful, _ = run_mul_mat(pkg, gpu, pkg.Q5_0, blocks, x, k, m)
+    precise, _ = run_mul_mat(pkg, gpu, pkg.Q5_0, blocks, x, k, m, flags=pkg.MM_EXACT_ACT)
+    assert oracle.nmse(precise, exact) < 1e-6 < oracle.nmse(faithful, exact) < 5e-4
+
+
+def test_mul_mat_epilogues(pkg, oracle, gpu):
+    k, m, n = 512, 384, 150
+    blocks = oracle.quantize(pkg.Q8_0, rnd((m, k), 0.02))
+    for nn in (n, 5):
+        x, bias, resid = rnd((nn, k)), rnd((m,), 0.5), rnd((nn, m))
+        base = oracle.mul_mat(pkg.Q8_0, blocks, x)
+        got, _ = run_mul_mat(pkg, gpu, pkg.Q8_0, blocks, x, k, m, flags=pkg.EPI_BIAS | pkg.EPI_GELU, bias=bias)
+        assert oracle.nmse(got, oracle.gelu(base + bias)) <= 1e-5
+        got, _ = run_mul_mat(pkg, gpu, pkg.Q8_0, blocks, x, k, m, flags=pkg.EPI_BIAS | pkg.EPI_RESIDUAL, bias=bias, resid=resid)
+        assert oracle.nmse(got, base + bias + resid) <= 1e-6
+        got, _ = run_mul_mat(pkg, gpu, pkg.Q8_0, blocks, x, k, m, flags=pkg.EPI_BIAS | pkg.EPI_SCALE, bias=bias, scale=0.35355339)
+        assert oracle.nmse(got, (base + bias) * np.float32(0.35355339)) <= 1e-6
+        got, _ = run_mul_mat(pkg, gpu, pkg.Q8_0, blocks, x, k, m, flags=pkg.EPI_SCALE, scale=0.35355339, out_f16=True)
+        want16 = oracle.f16_bits_to_f32(oracle.f32_to_f16_bits(base * np.float32(0.35355339)))
+        assert oracle.nmse(got, want16) <= 1e-6
+        colbias = rnd((nn,), 0.5)
+        got, _ = run_mul_mat(pkg, gpu, pkg.Q8_0, blocks, x, k, m, flags=pkg.EPI_BIAS_COL, bias=colbias)
+        assert oracle.nmse(got, base + colbias[:, None]) <= 1e-6
+
+
+def test_mul_mat_rejects_bad_arguments(pkg, gpu):
+    lib = pkg.kernels()
+    d_w = torch.zeros(22 * 4, dtype=torch.uint8, device=gpu.dev)
+    d_x = torch.zeros((3, 64), dtype=torch.float32, device=gpu.dev)
+    d_y = torch.zeros((3, 2), dtype=torch.float32, device=gpu.dev)
+    tw, tx, ty = pkg.tensor(d_w, pkg.Q5_0, ne=[64, 2]), pkg.tensor(d_x, pkg.F32), pkg.tensor(d_y, pkg.F32)
+    assert lib.mi355x_mul_mat(None, tx, ty, None, None, 0, gpu.stream) == -2
+    bad = pkg.tensor(d_y, pkg.F32, ne=[3, 3])
+    assert lib.mi355x_mul_mat(tw, tx, bad, None, None, 0, gpu.stream) == -2           # dst shape does not match
+    empty = pkg.tensor(d_x, pkg.F32, ne=[64, 0])
+    empty_y = pkg.tensor(d_y, pkg.F32, ne=[2, 0])
+    assert lib.mi355x_mul_mat(tw, empty, empty_y, None, None, 0, gpu.stream) == 0     # zero columns: nothing to do
+    d_x2 = torch.zeros((40, 64), dtype=torch.float32, device=gpu.dev)
+    d_y2 = torch.zeros((40, 2), dtype=torch.float32, device=gpu.dev)
+    assert lib.mi355x_mul_mat(tw, pkg.tensor(d_x2, pkg.F32), pkg.tensor(d_y2, pkg.F32), None, None, 0, gpu.stream) == -3   # GEMM needs its workspace
+
+
+# ------------------------------------------------------------------------------------------------------------------
+
+def _attention_inputs(oracle, H, N, KV, flat=False, pad_from=None):
+    q = rnd((H, N, 64), 0.05 if flat else 1.0)
+    k, v = rnd((H, KV, 64)), rnd((H, KV, 64), 0.3, 1.0 if flat else 0.0)
+    if pad_from is not None:
+        k[:, pad_from:] = 0.0
+        v[:, pad_from:] = 0.0
+    return q, oracle.f32_to_f16_bits(k), oracle.f32_to_f16_bits(v)
+
+
+def run_fa(pkg, gpu, q, kb, vb, mask, scale, mode):
+    H, N, D = q.shape
+    d_q, d_k, d_v = gpu.up(q), gpu.up(kb), gpu.up(vb)
+    d_m = gpu.up(mask) if mask is not None else None
+    d_o = torch.empty((N, H, D), dtype=torch.float32, device=gpu.dev)
+    tq, tk = pkg.tensor(d_q, pkg.F32), pkg.tensor(d_k, pkg.F16)
+    pkg.check(pkg.kernels().mi355x_flash_attn_ext(tq, tk, pkg.tensor(d_v, pkg.F16), pkg.tensor(d_m, pkg.F16) if d_m is not None else None,
+                                                   pkg.tensor(d_o, pkg.F32), scale, mode, None, 0, gpu.stream), "flash_attn_ext")
+    return gpu.down(d_o), pkg.kernels().mi355x_flash_attn_ext_kernel_name(tq, tk, mode).decode()
+
+
+@pytest.mark.parametrize("case", [
+    dict(H=2, N=70, KV=100), dict(H=3, N=200, KV=1536, flat=True, pad_from=1500), dict(H=20, N=5, KV=1536, flat=True, pad_from=1500),
+    dict(H=4, N=1, KV=1), dict(H=4, N=5, KV=37, mask="beam"), dict(H=2, N=3, KV=200, mask="causal"), dict(H=2, N=100, KV=100, mask="causal"),
+    dict(H=2, N=8, KV=448, mask="beam"), dict(H=2, N=9, KV=63)])
+def test_flash_attn_reference_faithful(pkg, oracle, gpu, case):
+    H, N, KV = case["H"], case["N"], case["KV"]
+    q, kb, vb = _attention_inputs(oracle, H, N, KV, case.get("flat", False), case.get("pad_from"))
+    mask = None
+    if "mask" in case:
+        m = np.full((-(-N // 64) * 64, KV), -np.inf, dtype=np.float32)
+        for r in range(N):
+            if case["mask"] == "causal":
+                m[r, : KV - N + r + 1] = 0.0
+            else:
+                m[r, : (KV + 1) // 2] = 0.0
+                m[r, [c for c in range(KV) if c % N == r]] = 0.0
+        mask = oracle.f32_to_f16_bits(m)
+    got, name = run_fa(pkg, gpu, q, kb, vb, mask, 0.125, pkg.FA_F16_SEQ)
+    assert name == ("flash_attn.seq_row" if N <= 8 else "flash_attn.seq_tile")
+    want = oracle.flash_attn_ext(q, kb, vb, None if mask is None else mask[:N], 0.125)
+    assert oracle.nmse(got, want) <= 1e-6      # same key order, same f16 accumulator: only exp() and dot-product ulps differ
+
+
+def test_flash_attn_f32_mode_matches_float64(pkg, oracle, gpu):
+    q, kb, vb = _attention_inputs(oracle, 2, 30, 300, flat=True, pad_from=280)
+    got, name = run_fa(pkg, gpu, q, kb, vb, None, 0.125, pkg.FA_F32)
+    assert name == "flash_attn.vec_f32"
+    qf = oracle.f16_bits_to_f32(oracle.f32_to_f16_bits(q)).astype(np.float64)
+    s = np.einsum("hnd,hkd->hnk", qf, oracle.f16_bits_to_f32(kb).astype(np.float64)) * 0.125
+    p = np.exp(s - s.max(-1, keepdims=True)); p /= p.sum(-1, keepdims=True)
+    exact = np.einsum("hnk,hkd->nhd", p, oracle.f16_bits_to_f32(vb).astype(np.float64))
+    assert oracle.nmse(got, exact) <= 1e-9
+
+
+def test_flash_attn_strided_views_like_whisper(pkg, oracle, gpu):
+    # Q is the permuted view of a [d, N] projection; K / V are slices of a 1-d cache with row pitch d (src/whisper.cpp:2149-2172)
+    H, N, KV, D = 4, 20, 96, 64
+    d = H * D
+    qcur, kc, vc = rnd((N, d)), rnd((KV, d)), rnd((KV, d))
+    d_q, d_k, d_v = gpu.up(qcur), gpu.up(oracle.f32_to_f16_bits(kc)), gpu.up(oracle.f32_to_f16_bits(vc))
+    d_o = torch.empty((N, H, D), dtype=torch.float32, device=gpu.dev)
+    tq = pkg.tensor(d_q, pkg.F32, ne=[D, N, H], nb=[4, d * 4, D * 4, d * 4 * N])
+    tk = pkg.tensor(d_k, pkg.F16, ne=[D, KV, H], nb=[2, d * 2, D * 2, d * 2 * KV])
+    tv = pkg.tensor(d_v, pkg.F16, ne=[D, KV, H], nb=[2, d * 2, D * 2, d * 2 * KV])
+    pkg.check(pkg.kernels().mi355x_flash_attn_ext(tq, tk, tv, None, pkg.tensor(d_o, pkg.F32), 0.125, pkg.FA_F16_SEQ, None, 0, gpu.stream))
+    q = qcur.reshape(N, H, D).transpose(1, 0, 2)
+    kb = oracle.f32_to_f16_bits(kc).reshape(KV, H, D).transpose(1, 0, 2)
+    vb = oracle.f32_to_f16_bits(vc).reshape(KV, H, D).transpose(1, 0, 2)
+    assert oracle.nmse(gpu.down(d_o), oracle.flash_attn_ext(q, kb, vb, None, 0.125)) <= 1e-6
+
+
+# ------------------------------------------------------------------------------------------------------------------
+
+def test_norm_and_affine(pkg, oracle, gpu):
+    lib = pkg.kernels()
+    for shape in [(1500, 1280), (7, 100), (3, 5000), (5, 512)]:
+        x = rnd(shape, 2.0, 0.3)
+        d_x = gpu.up(x)
+        d_y = torch.empty_like(d_x)
+        pkg.check(lib.mi355x_norm(pkg.tensor(d_x, pkg.F32), pkg.tensor(d_y, pkg.F32), 1e-5, None, None, gpu.stream))
+        want = oracle.norm(x, 1e-5)
+        assert oracle.nmse(gpu.down(d_y), want) <= 1e-10
+        w, b = rnd((shape[1],), 0.02, 1.0), rnd((shape[1],), 0.02)
+        d_w, d_b = gpu.up(w), gpu.up(b)
+        pkg.check(lib.mi355x_norm(pkg.tensor(d_x, pkg.F32), pkg.tensor(d_y, pkg.F32), 1e-5, d_w.data_ptr(), d_b.data_ptr(), gpu.stream))
+        assert oracle.nmse(gpu.down(d_y), want * w + b) <= 1e-10
+
+
+def test_gelu_scale_binary(pkg, oracle, gpu):
+    lib = pkg.kernels()
+    x = rnd((1500, 640), 3.0)
+    d_x = gpu.up(x)
+    d_y = torch.empty_like(d_x)
+    pkg.check(lib.mi355x_gelu(pkg.tensor(d_x, pkg.F32), pkg.tensor(d_y, pkg.F32), gpu.stream))
+    got, want = gpu.down(d_y), oracle.gelu(x)
+    assert oracle.nmse(got, want) <= 1e-7 and np.mean(got != want) < 0.02       # same f16-table semantics; exp() ulps flip a few f16 roundings
+    pkg.check(lib.mi355x_scale(pkg.tensor(d_x, pkg.F32), pkg.tensor(d_y, pkg.F32), 0.35355339, gpu.stream))
+    assert np.array_equal(gpu.down(d_y), oracle.scale(x, 0.35355339))
+    a = rnd((6, 5, 7))
+    for op in (0, 1):
+        for bshape in [(6, 5, 7), (7,), (1, 5, 1), (6, 1, 7), (3, 1, 7)]:
+            b = rnd(bshape)
+            d_a, d_b = gpu.up(a), gpu.up(b)
+            d_o = torch.empty_like(d_a)
+            pkg.check(lib.mi355x_binary(op, pkg.tensor(d_a, pkg.F32), pkg.tensor(d_b, pkg.F32), pkg.tensor(d_o, pkg.F32), gpu.stream))
+            assert np.array_equal(gpu.down(d_o), oracle.binary(op, a, b))
+    # in place, big, row vector (bias add of whisper)
+    big, bias = rnd((1500, 1280)), rnd((1280,))
+    d_a, d_b = gpu.up(big), gpu.up(bias)
+    pkg.check(lib.mi355x_binary(0, pkg.tensor(d_a, pkg.F32), pkg.tensor(d_b, pkg.F32), pkg.tensor(d_a, pkg.F32), gpu.stream))
+    assert np.array_equal(gpu.down(d_a), big + bias)
+
+
+def test_cpy_get_rows_im2col_softmax_concat(pkg, oracle, gpu):
+    lib = pkg.kernels()
+    # f32 -> f16 dense and transposed
+    x = rnd((1500, 320))
+    d_x = gpu.up(x)
+    d_h = torch.empty(x.shape, dtype=torch.float16, device=gpu.dev)
+    pkg.check(lib.mi355x_cpy(pkg.tensor(d_x, pkg.F32), pkg.tensor(d_h, pkg.F16), gpu.stream))
+    assert np.array_equal(gpu.down(d_h).view(np.uint16), oracle.f32_to_f16_bits(x))
+    d_t = torch.empty((320, 1500), dtype=torch.float32, device=gpu.dev)
+    pkg.check(lib.mi355x_cpy(pkg.tensor(d_x.t(), pkg.F32), pkg.tensor(d_t, pkg.F32), gpu.stream))     # CONT of a transposed view
+    assert np.array_equal(gpu.down(d_t), x.T)
+    # get_rows
+    w = rnd((300, 128), 0.02)
+    ids = np.array([5, 299, 0, 5, 17], dtype=np.int32)
+    for t in (pkg.Q5_0, pkg.Q8_0):
+        blocks = oracle.quantize(t, w)
+        d_w, d_i = gpu.up(blocks), gpu.up(ids)
+        d_o = torch.empty((5, 128), dtype=torch.float32, device=gpu.dev)
+        pkg.check(lib.mi355x_get_rows(pkg.tensor(d_w, t, ne=[128, 300]), pkg.tensor(d_i, pkg.I32), pkg.tensor(d_o, pkg.F32), gpu.stream))
+        assert np.array_equal(gpu.down(d_o), oracle.get_rows(t, blocks, ids, 128))
+    # im2col, the two strides of the conv stem, odd sizes
+    src = rnd((33, 77))
+    for s0 in (1, 2):
+        want = oracle.im2col_1d(src, 3, s0, 1, 1)
+        d_s = gpu.up(src)
+        d_o = torch.empty(want.shape, dtype=torch.float16, device=gpu.dev)
+        pkg.check(lib.mi355x_im2col_1d(pkg.tensor(d_s, pkg.F32), pkg.tensor(d_o, pkg.F16), 3, s0, 1, 1, gpu.stream))
+        assert np.array_equal(gpu.down(d_o).view(np.uint16), want)
+    # soft_max with an f32 mask shared by all heads
+    kq = rnd((4, 5, 37), 3.0)
+    mask = np.zeros((64, 37), dtype=np.float32); mask[:, 30:] = -np.inf
+    d_k, d_m = gpu.up(kq), gpu.up(mask)
+    d_o = torch.empty_like(d_k)
+    pkg.check(lib.mi355x_soft_max(pkg.tensor(d_k, pkg.F32), pkg.tensor(d_m, pkg.F32), pkg.tensor(d_o, pkg.F32), 0.125, gpu.stream))
+    assert oracle.nmse(gpu.down(d_o), oracle.soft_max(kq, mask[:5], 0.125)) <= 1e-10
+    # concat along ggml dim 2
+    a, b = rnd((2, 5, 30)), rnd((3, 5, 30))
+    d_a, d_b = gpu.up(a), gpu.up(b)
+    d_o = torch.empty((5, 5, 30), dtype=torch.float32, device=gpu.dev)
+    pkg.check(lib.mi355x_concat(pkg.tensor(d_a, pkg.F32), pkg.tensor(d_b, pkg.F32), pkg.tensor(d_o, pkg.F32), 2, gpu.stream))
+    assert np.array_equal(gpu.down(d_o), np.concatenate([a, b], axis=0))
+
+
+def test_smoke_entry_point():
+    import __graft_entry__ as entry
+    entry.smoke()

@@ -59,6 +59,7 @@ struct mi355x_backend_ctx {
     hipStream_t stream = nullptr;
     bool        fuse    = true;
     bool        profile = false;
+    bool        debug   = false;   // log what every MUL_MAT launch folds in (GGML_MI355X_DEBUG=1)
     bool        exact   = false;   // true: f32 attention accumulators and un-rounded GEMM activations instead of the
                                    // reference's f16-sequential / Q8_0-rounded arithmetic
 

@@ -267,6 +267,7 @@ static ggml_backend_t device_init_backend(ggml_backend_dev_t dev, const char *) 
     ctx->fuse    = env_flag("GGML_MI355X_FUSE", true);
     ctx->profile = env_flag("GGML_MI355X_PROFILE", false);
     ctx->exact   = env_flag("GGML_MI355X_EXACT", false);
+    ctx->debug   = env_flag("GGML_MI355X_DEBUG", false);
     // default priority, blocking with respect to the null stream used by the buffer-level copies
     HIP_TRY(hipStreamCreate(&ctx->stream), { delete ctx; return NULL; });
     ggml_backend_t backend = new ggml_backend{

@@ -204,11 +204,18 @@ struct graph_runner {
             auto same_layout = [&](const ggml_tensor * t) {
                 return t->type == GGML_TYPE_F32 && ggml_are_same_shape(t, mm) && ggml_is_contiguous(t);
             };
-            // a dense RESHAPE of the running result (ggml_conv_1d reshapes its MUL_MAT, ggml/src/ggml.c:3899) is the same memory
+            // Views are no-ops for the device, so they can be stepped over while looking for the next link: a dense
+            // RESHAPE of the running result becomes the running result (ggml_conv_1d reshapes its MUL_MAT,
+            // ggml/src/ggml.c:3899); a view of anything else (the cache slice a CPY is about to write, src/whisper.cpp:2155)
+            // is simply skipped.  A view of the running result that is not such a reshape ends the chain.
             auto hop_views = [&]() {
                 ggml_tensor * t = node_at(i + used);
-                while (t && t->op == GGML_OP_RESHAPE && t->src[0] == last && only_feeds_next(last) && ggml_is_contiguous(t)) {
-                    last = t; ++used; t = node_at(i + used);
+                while (t && is_view_op(t->op)) {
+                    const bool of_last = t->src[0] == last || t->view_src == last;
+                    if (of_last) {
+                        if (t->op == GGML_OP_RESHAPE && only_feeds_next(last) && ggml_is_contiguous(t)) last = t; else return (ggml_tensor *) nullptr;
+                    }
+                    ++used; t = node_at(i + used);
                 }
                 return t;
             };
@@ -232,8 +239,9 @@ struct graph_runner {
                 } else if (n->op == GGML_OP_ADD && same_layout(n->src[1]) && n->src[1] != last) {
                     epi.flags |= MI355X_EPI_RESIDUAL; epi.residual = n->src[1]->data; last = n; ++used;
                 }
-                n = node_at(i + used);
+                n = hop_views();
             }
+            // views stepped over after the last folded link stay in the graph walk (they are no-ops there, too)
             out = last;
             // + store as f16 (K/V cache writes)
             if (n && n->op == GGML_OP_CPY && n->src[0] == last && only_feeds_next(last) && !(epi.flags & MI355X_EPI_RESIDUAL) &&
@@ -266,6 +274,10 @@ struct graph_runner {
             if (hit) epi.flags |= MI355X_MM_WS_READY;
             ctx->ws_x = x->data; memcpy(ctx->ws_x_ne, x->ne, sizeof(x->ne)); memcpy(ctx->ws_x_nb, x->nb, sizeof(x->nb));
             cached_x = x;
+        }
+        if (ctx->debug) {
+            GGML_LOG_INFO("ggml-mi355x: %s %s [%lld x %lld x %lld] folds %d nodes, flags 0x%x\n", mi355x_mul_mat_kernel_name(&vw, &vx), mm->name,
+                          (long long) mm->ne[0], (long long) mm->ne[1], (long long) w->ne[0], used, epi.flags);
         }
         {
             launch_scope ls(ctx, mi355x_mul_mat_kernel_name(&vw, &vx), bytes, flops);

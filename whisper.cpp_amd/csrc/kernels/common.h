@@ -73,6 +73,11 @@ static inline int launch_status() {
     return e == hipSuccess ? MI355X_OK : MI355X_ERR_HIP;
 }
 
+// Device address of the GELU table for the current device; built on the host on first use with the reference's own
+// formula and libm (ggml/src/ggml-cpu/ggml-cpu.c:3415-3423, vec.h:432-434) and copied into a __device__ array.
+// NULL on failure.
+const uint16_t * gelu_table_device();
+
 #ifdef __HIPCC__
 
 __device__ __forceinline__ float h2f(uint16_t h) {
@@ -98,15 +103,13 @@ __device__ __forceinline__ float wave_max(float v) {
     return v;
 }
 
-// tanh-GELU as ggml_vec_gelu_f32 evaluates it (ggml/src/ggml-cpu/vec.h:432-457): outside (-10, 10) the clamps, inside
-// a lookup in a table indexed by f16(x) that holds f16(gelu(f32(f16(x)))) — i.e. argument and result rounded to f16.
-__device__ __forceinline__ float gelu_f32(float x) {
+// GELU as ggml_vec_gelu_f32 evaluates it (ggml/src/ggml-cpu/vec.h:443-457): outside (-10, 10) the clamps, inside a
+// lookup in a 65536-entry table indexed by the f16 bits of x that holds f16(gelu(f32(f16 x))).  `table` is the device
+// copy of that table (gelu_table_device below).
+__device__ __forceinline__ float gelu_f32(float x, const uint16_t * __restrict__ table) {
     if (x <= -10.0f) return 0.0f;
     if (x >=  10.0f) return x;
-    const float xh = (float)(half_t) x;
-    const float u  = 0.79788456080286535587989211986876f * xh * (1.0f + 0.044715f * xh * xh);
-    // 0.5x(1+tanh(u)) = x / (1 + exp(-2u))
-    return (float)(half_t)(xh / (1.0f + __expf(-2.0f * u)));
+    return h2f(table[f2h_bits(x)]);
 }
 
 // unaligned little-endian loads from byte-addressed block data

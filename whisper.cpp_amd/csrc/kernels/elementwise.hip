@@ -78,26 +78,26 @@ extern "C" int mi355x_binary(int op, const mi355x_tensor * src0, const mi355x_te
 // SCALE, GELU  (ggml/src/ggml-cpu/ops.cpp:3840-3878, 2606-2643)
 // ------------------------------------------------------------------------------------------------------
 
-template <int OP> __device__ __forceinline__ float un_op(float x, float s) { return OP == 0 ? x * s : gelu_f32(x); }
+template <int OP> __device__ __forceinline__ float un_op(float x, float s, const uint16_t * tab) { return OP == 0 ? x * s : gelu_f32(x, tab); }
 
 template <int OP>
-__global__ void k_unary_contig4(const float4 * __restrict__ a, float4 * __restrict__ d, int64_t n4, float s) {
+__global__ void k_unary_contig4(const float4 * __restrict__ a, float4 * __restrict__ d, int64_t n4, float s, const uint16_t * __restrict__ tab) {
     int64_t i = (int64_t) blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= n4) return;
     float4 x = a[i];
-    x.x = un_op<OP>(x.x, s); x.y = un_op<OP>(x.y, s); x.z = un_op<OP>(x.z, s); x.w = un_op<OP>(x.w, s);
+    x.x = un_op<OP>(x.x, s, tab); x.y = un_op<OP>(x.y, s, tab); x.z = un_op<OP>(x.z, s, tab); x.w = un_op<OP>(x.w, s, tab);
     d[i] = x;
 }
 
 template <int OP>
-__global__ void k_unary_generic(tview a, tview d, int64_t n, float s) {
+__global__ void k_unary_generic(tview a, tview d, int64_t n, float s, const uint16_t * __restrict__ tab) {
     int64_t i = (int64_t) blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= n) return;
     int64_t i0 = i % d.ne0; int64_t t = i / d.ne0;
     int64_t i1 = t % d.ne1; t /= d.ne1;
     int64_t i2 = t % d.ne2; int64_t i3 = t / d.ne2;
     const float x = *(const float *)(a.p + i0*a.nb0 + i1*a.nb1 + i2*a.nb2 + i3*a.nb3);
-    *(float *)(d.p + i0*d.nb0 + i1*d.nb1 + i2*d.nb2 + i3*d.nb3) = un_op<OP>(x, s);
+    *(float *)(d.p + i0*d.nb0 + i1*d.nb1 + i2*d.nb2 + i3*d.nb3) = un_op<OP>(x, s, tab);
 }
 
 template <int OP>
@@ -108,11 +108,13 @@ static int unary_launch(const mi355x_tensor * src, const mi355x_tensor * dst, fl
     const int64_t n = nelements(dst);
     if (n == 0) return MI355X_OK;
     hipStream_t st = (hipStream_t) stream;
+    const uint16_t * tab = nullptr;
+    if (OP == 1 && !(tab = gelu_table_device())) return MI355X_ERR_HIP;
     if (is_contiguous(src) && is_contiguous(dst) && n % 4 == 0 &&
         ((uintptr_t) src->data % 16 == 0) && ((uintptr_t) dst->data % 16 == 0)) {
-        k_unary_contig4<OP><<<ew_grid(n / 4), EW_BLOCK, 0, st>>>((const float4 *) src->data, (float4 *) dst->data, n / 4, s);
+        k_unary_contig4<OP><<<ew_grid(n / 4), EW_BLOCK, 0, st>>>((const float4 *) src->data, (float4 *) dst->data, n / 4, s, tab);
     } else {
-        k_unary_generic<OP><<<ew_grid(n), EW_BLOCK, 0, st>>>(make_view(src), make_view(dst), n, s);
+        k_unary_generic<OP><<<ew_grid(n), EW_BLOCK, 0, st>>>(make_view(src), make_view(dst), n, s, tab);
     }
     return launch_status();
 }

@@ -115,8 +115,9 @@ __device__ __forceinline__ half_t seq_mad(half_t acc, half_t v, float vs) { retu
 __device__ __forceinline__ void seq_factors(float s, float & M, float & vs, float & ms, float & P, float & A) {
     if (s == -INFINITY) { vs = 0.0f; ms = 1.0f; return; }       // masked key: the reference skips it
     const float Mn = fmaxf(M, s);
-    ms = expf(M - Mn);                                           // 1 when the maximum stands, 0 for the first key
-    vs = expf(s - Mn);                                           // 1 when s is the new maximum
+    ms = M == Mn ? 1.0f : expf(M - Mn);                          // 1 when the maximum stands, 0 for the first key
+    vs = expf(s - Mn);                                           // 1 when s is the new maximum (libm-grade exp: the factors
+                                                                 // feed f16 roundings that amplify last-bit differences)
     M = Mn;
     P *= ms;
     A = A * ms + vs;
@@ -126,7 +127,7 @@ __device__ __forceinline__ void seq_factors(float s, float & M, float & vs, floa
 // k_fattn_seq_row: one block per (query, head)
 // ------------------------------------------------------------------------------------------------------
 
-#define ROW_UNROLL 8
+#define ROW_CHUNK 64
 
 __global__ void __launch_bounds__(256) k_fattn_seq_row(fa_args a, int kv_pad) {
     extern __shared__ __attribute__((aligned(16))) float sm[];
@@ -208,21 +209,38 @@ __global__ void __launch_bounds__(256) k_fattn_seq_row(fa_args a, int kv_pad) {
     __syncthreads();
     if (wave != 0) return;
 
-    // ---- the sequential f16 chain: lane = d --------------------------------------------------------------------------------
+    // ---- the sequential f16 chain: lane = d -----------------------------------------------------------------------------------
+    // 64 keys at a time: their V values sit in registers (the next 64 are in flight while these are consumed), their
+    // factors are read once, one per lane, and handed to the chain through v_readlane, so that the dependent part of
+    // every step is a single v_fma_mixlo_f16.
     half_t acc = (half_t) 0.0f;
-    const half_t * vcol = (const half_t *) vb + lane;
-    for (int key0 = 0; key0 < kv_pad; key0 += ROW_UNROLL) {
-        half_t v[ROW_UNROLL];
+    const char * vcol = vb + lane * 2;
+    half_t va[ROW_CHUNK], vn[ROW_CHUNK];
+    auto load_chunk = [&](half_t * dst, int key0) {
 #pragma unroll
-        for (int j = 0; j < ROW_UNROLL; ++j) {
+        for (int j = 0; j < ROW_CHUNK; ++j) {
             const int key = key0 + j;
-            v[j] = key < KV ? *(const half_t *)((const char *) vcol + (int64_t) key * a.v_nb1) : (half_t) 0.0f;
+            dst[j] = key < KV ? *(const half_t *)(vcol + (int64_t) key * a.v_nb1) : (half_t) 0.0f;
         }
+    };
+    auto run_chunk = [&](const half_t * v, int key0) {
+        const int vs_l = __float_as_int(vs_s[key0 + lane]), ms_l = __float_as_int(ms_s[key0 + lane]);
 #pragma unroll
-        for (int j = 0; j < ROW_UNROLL; ++j) {
-            const float vs = vs_s[key0 + j], ms = ms_s[key0 + j];
-            if (ms != 1.0f) acc = seq_scale(acc, ms);      // uniform across the wavefront
+        for (int j = 0; j < ROW_CHUNK; ++j) {
+            const float vs = __int_as_float(__builtin_amdgcn_readlane(vs_l, j));
+            const float ms = __int_as_float(__builtin_amdgcn_readlane(ms_l, j));
+            if (ms != 1.0f) acc = seq_scale(acc, ms);      // scalar condition: uniform across the wavefront
             if (vs != 0.0f) acc = seq_mad(acc, v[j], vs);
+        }
+    };
+    load_chunk(va, 0);
+    for (int key0 = 0; key0 < kv_pad; key0 += 2 * ROW_CHUNK) {
+        const bool more = key0 + ROW_CHUNK < kv_pad;
+        if (more) load_chunk(vn, key0 + ROW_CHUNK);
+        run_chunk(va, key0);
+        if (more) {
+            if (key0 + 2 * ROW_CHUNK < kv_pad) load_chunk(va, key0 + 2 * ROW_CHUNK);
+            run_chunk(vn, key0 + ROW_CHUNK);
         }
     }
     float * dp = (float *) a.d + ((i3 * a.N + n) * a.H + h) * FA_D;
@@ -453,7 +471,7 @@ extern "C" int mi355x_flash_attn_ext(const mi355x_tensor * q, const mi355x_tenso
 
     switch (fa_kernel(q, k, mode)) {
         case FA_K_SEQ_ROW: {
-            const int kv_pad = (int)((KV + ROW_UNROLL - 1) / ROW_UNROLL * ROW_UNROLL);
+            const int kv_pad = (int)((KV + ROW_CHUNK - 1) / ROW_CHUNK * ROW_CHUNK);
             dim3 grid((unsigned) N, (unsigned) H, (unsigned) q->ne[3]);
             k_fattn_seq_row<<<grid, 256, (size_t) kv_pad * 8, st>>>(a, kv_pad);
         } break;

@@ -28,12 +28,13 @@ struct epi_args {
     float        scale;
     const float *bias;
     const char * residual;   // same strides as dst, f32
+    const uint16_t * gelu;   // GELU table (device), set when MI355X_EPI_GELU is
 };
 
 __device__ __forceinline__ float apply_epilogue(float v, const epi_args & e, int64_t m, int64_t n, int64_t res_off) {
     if (e.flags & MI355X_EPI_BIAS)     v += e.bias[m];
     if (e.flags & MI355X_EPI_BIAS_COL) v += e.bias[n];
-    if (e.flags & MI355X_EPI_GELU)     v  = gelu_f32(v);
+    if (e.flags & MI355X_EPI_GELU)     v  = gelu_f32(v, e.gelu);
     if (e.flags & MI355X_EPI_SCALE)    v *= e.scale;
     if (e.flags & MI355X_EPI_RESIDUAL) v += *(const float *)(e.residual + res_off);
     return v;
@@ -304,29 +305,237 @@ __global__ void __launch_bounds__(256, 2) k_gemm_mfma(mm_args a) {
 }
 
 // ------------------------------------------------------------------------------------------------------
-// src1 -> Q8_0 -> f16: what the CPU backend's MUL_MAT actually multiplies with (ggml-cpu.c:1328-1363 converts src1
-// to the weights' vec_dot_type with quantize_row_q8_0, ggml-cpu-quants.c:808-865).  One pass per src1, shared by
-// every MUL_MAT that reads the same activations; the GEMM then streams f16 instead of f32.
+// Quantized-weight GEMM on the int8 matrix cores.
+//
+// ggml's MUL_MAT with Q5_0 / Q8_0 weights is, by definition of the CPU backend, an integer computation
+// (ggml-cpu.c:1328-1363 converts src1 to Q8_0 with quantize_row_q8_0; ggml_vec_dot_q5_0_q8_0 / ggml_vec_dot_q8_0_q8_0,
+// ggml-cpu-quants.c:2930, 3597, then form per 32-value block the exact integer dot product of the quants and add
+// it, times d_w * d_x, to an f32 sum).  The kernel does exactly that: one pass quantizes src1 (k_quantize_act), then
+// each 32x32 accumulator patch takes one v_mfma_i32_32x32x32_i8 per block — K = 32 is one quant block — and the
+// exact i32 block sums are folded into f32 accumulators with the outer product of the block scales.
+//
+// Tile 128 (src1 rows) x 128 (weight rows) x 64 (two blocks), 4 wavefronts as 2 x 2, LDS double-buffered: the
+// global loads of step s+2 and the nibble unpacking / LDS stores of step s+1 are issued in the same basic block as
+// the MFMAs and scale FMAs of step s.
 // ------------------------------------------------------------------------------------------------------
 
-__global__ void k_round_act_q8_0(const char * __restrict__ x, half_t * __restrict__ out, int64_t K, int64_t N,
-                                 int64_t x_nb1, int64_t x_nb2, int64_t nbatch2, int64_t x_nb3) {
-    // 8 lanes per 32-value block, 4 values each
-    const int64_t t   = (int64_t) blockIdx.x * blockDim.x + threadIdx.x;
-    const int64_t k4  = K / 4;
-    const int64_t b   = blockIdx.y;                    // batch index (ne2*ne3 flattened)
-    if (t >= k4 * N) return;                           // K is a multiple of 32: whole 8-lane groups leave together
+typedef int v4i_t  __attribute__((ext_vector_type(4)));
+typedef int v16i_t __attribute__((ext_vector_type(16)));
+
+static inline size_t round256(size_t n) { return (n + 255) / 256 * 256; }
+
+// workspace of one batch slice: int8 quants [N][K], then f32 block scales [K/32][N]
+__global__ void k_quantize_act(const char * __restrict__ x, char * __restrict__ ws, int64_t K, int64_t N,
+                               int64_t x_nb1, int64_t x_nb2, int64_t ne12, int64_t x_nb3, int64_t slice_bytes, int64_t xd_off) {
+    const int64_t t  = (int64_t) blockIdx.x * blockDim.x + threadIdx.x;     // 8 lanes per block of 32 values, 4 values each
+    const int64_t k4 = K / 4;
+    const int64_t b  = blockIdx.y;
+    if (t >= k4 * N) return;                                                // whole 8-lane groups leave together
     const int64_t n = t / k4, c = t % k4;
-    const char * xr = x + n * x_nb1 + (b % nbatch2) * x_nb2 + (b / nbatch2) * x_nb3;
-    const float4 v = *(const float4 *)(xr + c * 16);
+    const float4 v = *(const float4 *)(x + n * x_nb1 + (b % ne12) * x_nb2 + (b / ne12) * x_nb3 + c * 16);
     float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
     amax = fmaxf(amax, __shfl_xor(amax, 1, 8));
     amax = fmaxf(amax, __shfl_xor(amax, 2, 8));
     amax = fmaxf(amax, __shfl_xor(amax, 4, 8));
-    const float d  = h2f(f2h_bits(amax / 127.0f));     // the block scale is stored as f16
     const float id = amax != 0.0f ? 127.0f / amax : 0.0f;
-    half4_t o = { (half_t)(d * rintf(v.x * id)), (half_t)(d * rintf(v.y * id)), (half_t)(d * rintf(v.z * id)), (half_t)(d * rintf(v.w * id)) };
-    *(half4_t *)(out + (b * N + n) * K + c * 4) = o;
+    const int q0 = (int) rintf(v.x * id), q1 = (int) rintf(v.y * id), q2 = (int) rintf(v.z * id), q3 = (int) rintf(v.w * id);
+    char * slice = ws + b * slice_bytes;
+    *(int32_t *)(slice + n * K + c * 4) = (q0 & 0xFF) | ((q1 & 0xFF) << 8) | ((q2 & 0xFF) << 16) | ((q3 & 0xFF) << 24);
+    if ((c & 7) == 0) ((float *)(slice + xd_off))[(c / 8) * N + n] = h2f(f2h_bits(amax / 127.0f));   // the scale goes through f16, like block_q8_0.d
+}
+
+#define I8_N   128
+#define I8_M   128
+#define I8_K   64            // two quant blocks per step
+#define I8_LD  80            // byte pitch of the quant tiles: 64 + 16, so that 8 consecutive rows start 4 banks apart
+
+struct i8_args {
+    mm_args m;               // x = workspace quants of this launch, x_nb* describe them; w / d as usual
+    const char * xd;         // block scales [K/32][N] of batch slice 0
+    int64_t xd_slice;        // bytes between batch slices
+};
+
+template <int T0> struct wq_frag;
+template <> struct wq_frag<MI355X_TYPE_Q5_0> { uint32_t d, qh, qs[4]; };
+template <> struct wq_frag<MI355X_TYPE_Q8_0> { uint32_t d, qs[8]; };
+
+template <int T0>
+__device__ __forceinline__ void i8_load_w(wq_frag<T0> & f, const char * wrow, bool row_ok, int64_t k0, int64_t K) {
+    const int64_t k = k0 + (threadIdx.x & 1) * 32;
+    if constexpr (T0 == MI355X_TYPE_Q5_0) {
+        if (row_ok && k < K) {
+            const uint8_t * b = (const uint8_t *) wrow + (k / QK) * 22;
+            f.d  = *(const uint16_t *) b;
+            f.qh = *(const u32a2 *)(b + 2);
+            const u128a2 q = *(const u128a2 *)(b + 6);
+            f.qs[0] = q.x; f.qs[1] = q.y; f.qs[2] = q.z; f.qs[3] = q.w;
+        } else { f.d = 0; f.qh = 0; f.qs[0] = f.qs[1] = f.qs[2] = f.qs[3] = 0; }
+    } else {
+        if (row_ok && k < K) {
+            const uint8_t * b = (const uint8_t *) wrow + (k / QK) * 34;
+            f.d = *(const uint16_t *) b;
+            const u128a2 q0 = *(const u128a2 *)(b + 2), q1 = *(const u128a2 *)(b + 18);
+            f.qs[0] = q0.x; f.qs[1] = q0.y; f.qs[2] = q0.z; f.qs[3] = q0.w;
+            f.qs[4] = q1.x; f.qs[5] = q1.y; f.qs[6] = q1.z; f.qs[7] = q1.w;
+        } else {
+            f.d = 0;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) f.qs[i] = 0;
+        }
+    }
+}
+
+// block -> 32 signed bytes in weight order, plus the f32 scale
+template <int T0>
+__device__ __forceinline__ void i8_store_w(const wq_frag<T0> & f, char * wq_s, float * wd_s) {
+    const int row = threadIdx.x >> 1, blk = threadIdx.x & 1;
+    uint32_t o[8];
+    if constexpr (T0 == MI355X_TYPE_Q5_0) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            // q - 16 as a signed byte: the nibble, with 0xF0 on top where the fifth bit is clear
+            const uint32_t lo_h = ((~(f.qh >> (4*i))      & 0xFu) * 0x00204081u) & 0x01010101u;
+            const uint32_t hi_h = ((~(f.qh >> (16 + 4*i)) & 0xFu) * 0x00204081u) & 0x01010101u;
+            o[i]     = (f.qs[i] & 0x0F0F0F0Fu)        | (lo_h * 0xF0u);
+            o[4 + i] = ((f.qs[i] >> 4) & 0x0F0F0F0Fu) | (hi_h * 0xF0u);
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) o[i] = f.qs[i];
+    }
+    uint4 * p = (uint4 *)(wq_s + row * I8_LD + blk * 32);
+    p[0] = make_uint4(o[0], o[1], o[2], o[3]);
+    p[1] = make_uint4(o[4], o[5], o[6], o[7]);
+    wd_s[blk * I8_M + row] = h2f((uint16_t) f.d);
+}
+
+struct xq_frag { uint32_t q[8]; float d; };
+
+__device__ __forceinline__ void i8_load_x(xq_frag & f, const char * xq, const float * xd, int64_t n0, int64_t N, int64_t k0, int64_t K) {
+    const int row = threadIdx.x >> 1, half = threadIdx.x & 1;
+    const int64_t n = n0 + row, k = k0 + half * 32;
+    if (n < N && k < K) {
+        const uint4 * p = (const uint4 *)(xq + n * K + k);
+        const uint4 v0 = p[0], v1 = p[1];
+        f.q[0] = v0.x; f.q[1] = v0.y; f.q[2] = v0.z; f.q[3] = v0.w; f.q[4] = v1.x; f.q[5] = v1.y; f.q[6] = v1.z; f.q[7] = v1.w;
+    } else {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) f.q[i] = 0;
+    }
+    // scales: thread t -> block t / 128 of this step, row t % 128
+    const int64_t sn = n0 + (threadIdx.x & 127), sk = k0 + (threadIdx.x >> 7) * 32;
+    f.d = (sn < N && sk < K) ? xd[(sk / QK) * N + sn] : 0.0f;
+}
+__device__ __forceinline__ void i8_store_x(const xq_frag & f, char * xq_s, float * xd_s) {
+    uint4 * p = (uint4 *)(xq_s + (threadIdx.x >> 1) * I8_LD + (threadIdx.x & 1) * 32);
+    p[0] = make_uint4(f.q[0], f.q[1], f.q[2], f.q[3]);
+    p[1] = make_uint4(f.q[4], f.q[5], f.q[6], f.q[7]);
+    xd_s[threadIdx.x] = f.d;               // [blk][row]
+}
+
+template <int T0>
+__global__ void __launch_bounds__(256, 2) k_gemm_i8(i8_args ia) {
+    const mm_args & a = ia.m;
+    __shared__ __attribute__((aligned(16))) char  xq_s[2][I8_N * I8_LD];
+    __shared__ __attribute__((aligned(16))) char  wq_s[2][I8_M * I8_LD];
+    __shared__ __attribute__((aligned(16))) float xd_s[2][2 * I8_N];
+    __shared__ __attribute__((aligned(16))) float wd_s[2][2 * I8_M];
+
+    const int64_t m0 = (int64_t) blockIdx.x * I8_M, n0 = (int64_t) blockIdx.y * I8_N;
+    const int64_t bz = blockIdx.z, b2 = bz % a.ne12, b3 = bz / a.ne12;
+    const char *  wb = a.w + (b2 / a.r2) * a.w_nb2 + (b3 / a.r3) * a.w_nb3;
+    const char *  xq = a.x + bz * a.x_nb2;
+    const float * xd = (const float *)(ia.xd + bz * ia.xd_slice);
+    char *        db = a.d + b2 * a.d_nb2 + b3 * a.d_nb3;
+
+    const int64_t wm   = m0 + (threadIdx.x >> 1);
+    const bool    w_ok = wm < a.M;
+    const char *  wrow = wb + (w_ok ? wm : 0) * a.w_nb1;
+
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int wn = (wave >> 1) * 64, wmo = (wave & 1) * 64, l32 = lane & 31, g = lane >> 5;
+
+    float16_t acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+    wq_frag<T0> wf;
+    xq_frag     xf;
+    i8_load_w<T0>(wf, wrow, w_ok, 0, a.K);
+    i8_load_x(xf, xq, xd, n0, a.N, 0, a.K);
+    i8_store_w<T0>(wf, wq_s[0], wd_s[0]);
+    i8_store_x(xf, xq_s[0], xd_s[0]);
+    if (I8_K < a.K) { i8_load_w<T0>(wf, wrow, w_ok, I8_K, a.K); i8_load_x(xf, xq, xd, n0, a.N, I8_K, a.K); }
+    __syncthreads();
+
+    int buf = 0;
+    for (int64_t k0 = 0; k0 < a.K; k0 += I8_K, buf ^= 1) {
+        if (k0 + I8_K < a.K) {                      // stage s+1 goes to the other buffer (its last readers passed the barrier)
+            i8_store_w<T0>(wf, wq_s[buf ^ 1], wd_s[buf ^ 1]);
+            i8_store_x(xf, xq_s[buf ^ 1], xd_s[buf ^ 1]);
+        }
+        if (k0 + 2 * I8_K < a.K) { i8_load_w<T0>(wf, wrow, w_ok, k0 + 2 * I8_K, a.K); i8_load_x(xf, xq, xd, n0, a.N, k0 + 2 * I8_K, a.K); }
+
+        const char *  xs = xq_s[buf]; const char * ws = wq_s[buf];
+        const float * xds = xd_s[buf]; const float * wds = wd_s[buf];
+#pragma unroll
+        for (int blk = 0; blk < 2; ++blk) {
+            v4i_t av[2], bv[2];
+            float dw[2];
+            float4 dx[2][4];
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                av[i] = *(const v4i_t *)(xs + (wn + 32 * i + l32) * I8_LD + blk * 32 + 16 * g);
+#pragma unroll
+                for (int q = 0; q < 4; ++q) dx[i][q] = *(const float4 *)(xds + blk * I8_N + wn + 32 * i + 8 * q + 4 * g);
+            }
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                bv[j] = *(const v4i_t *)(ws + (wmo + 32 * j + l32) * I8_LD + blk * 32 + 16 * g);
+                dw[j] = wds[blk * I8_M + wmo + 32 * j + l32];
+            }
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {
+                    v16i_t c;
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) c[r] = 0;
+                    c = __builtin_amdgcn_mfma_i32_32x32x32_i8(av[i], bv[j], c, 0, 0, 0);
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        acc[i][j][4*q + 0] += (float) c[4*q + 0] * (dx[i][q].x * dw[j]);
+                        acc[i][j][4*q + 1] += (float) c[4*q + 1] * (dx[i][q].y * dw[j]);
+                        acc[i][j][4*q + 2] += (float) c[4*q + 2] * (dx[i][q].z * dw[j]);
+                        acc[i][j][4*q + 3] += (float) c[4*q + 3] * (dx[i][q].w * dw[j]);
+                    }
+                }
+        }
+        __syncthreads();
+    }
+
+    const bool out_f16 = a.e.flags & MI355X_EPI_OUT_F16;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int64_t m = m0 + wmo + 32 * j + l32;
+            if (m >= a.M) continue;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int64_t n = n0 + wn + 32 * i + 8 * (r >> 2) + 4 * g + (r & 3);
+                if (n >= a.N) continue;
+                const int64_t res_off = (b2 * a.d_nb2 + b3 * a.d_nb3) + n * a.d_nb1 + m * 4;
+                const float v = apply_epilogue(acc[i][j][r], a.e, m, n, res_off);
+                if (out_f16) *(half_t *)(db + n * a.d_nb1 + m * 2) = (half_t) v;
+                else         *(float  *)(db + n * a.d_nb1 + m * 4) = v;
+            }
+        }
+    }
 }
 
 // ------------------------------------------------------------------------------------------------------
@@ -343,27 +552,41 @@ __global__ void __launch_bounds__(256) k_gemv_q(mm_args a) {
     float *   xd   = (float *)(smem + (size_t) NC * K);
     int32_t * xsum = (int32_t *)(smem + (size_t) NC * K + (size_t) NC * nbk * 4);
 
-    // --- quantize X: 8 lanes per 32-value block, round-to-nearest-even like _mm256_round_ps(_MM_ROUND_NEAREST)
+    // --- quantize X: 8 lanes per 32-value block, round-to-nearest-even like _mm256_round_ps(_MM_ROUND_NEAREST).
+    // Eight independent loads per thread are in flight before the first is consumed.
     {
-        const int sub = threadIdx.x & 7;
-        for (int b = threadIdx.x >> 3; b < NC * nbk; b += 32) {
-            const int n = b / nbk, kb = b % nbk;
-            const float4 v = *(const float4 *)(a.x + (int64_t) n * a.x_nb1 + ((int64_t) kb * QK + sub * 4) * 4);
-            float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
-            amax = fmaxf(amax, __shfl_xor(amax, 1, 8));
-            amax = fmaxf(amax, __shfl_xor(amax, 2, 8));
-            amax = fmaxf(amax, __shfl_xor(amax, 4, 8));
-            const float d  = amax / 127.0f;
-            const float id = amax != 0.0f ? 127.0f / amax : 0.0f;
-            const int q0 = (int) rintf(v.x * id), q1 = (int) rintf(v.y * id), q2 = (int) rintf(v.z * id), q3 = (int) rintf(v.w * id);
-            xq[(int64_t) n * (K / 4) + kb * 8 + sub] = (q0 & 0xFF) | ((q1 & 0xFF) << 8) | ((q2 & 0xFF) << 16) | ((q3 & 0xFF) << 24);
-            int s = q0 + q1 + q2 + q3;
-            s += __shfl_xor(s, 1, 8);
-            s += __shfl_xor(s, 2, 8);
-            s += __shfl_xor(s, 4, 8);
-            if (sub == 0) {
-                xd[n * nbk + kb]   = h2f(f2h_bits(d));     // the CPU backend stores d as f16 and reads it back
-                xsum[n * nbk + kb] = s;
+        const int total = NC * nbk * 8;                         // float4 pieces
+        const int k8 = nbk * 8;
+        for (int base = 0; base < total; base += 256 * 8) {
+            float4 v[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const int idx = base + u * 256 + (int) threadIdx.x;
+                v[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (idx < total) v[u] = *(const float4 *)(a.x + (int64_t)(idx / k8) * a.x_nb1 + (int64_t)(idx % k8) * 16);
+            }
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const int idx = base + u * 256 + (int) threadIdx.x;      // lanes 8i .. 8i+7 share a block
+                float amax = fmaxf(fmaxf(fabsf(v[u].x), fabsf(v[u].y)), fmaxf(fabsf(v[u].z), fabsf(v[u].w)));
+                amax = fmaxf(amax, __shfl_xor(amax, 1, 8));
+                amax = fmaxf(amax, __shfl_xor(amax, 2, 8));
+                amax = fmaxf(amax, __shfl_xor(amax, 4, 8));
+                const float d  = amax / 127.0f;
+                const float id = amax != 0.0f ? 127.0f / amax : 0.0f;
+                const int q0 = (int) rintf(v[u].x * id), q1 = (int) rintf(v[u].y * id), q2 = (int) rintf(v[u].z * id), q3 = (int) rintf(v[u].w * id);
+                int sum = q0 + q1 + q2 + q3;
+                sum += __shfl_xor(sum, 1, 8);
+                sum += __shfl_xor(sum, 2, 8);
+                sum += __shfl_xor(sum, 4, 8);
+                if (idx < total) {
+                    const int n = idx / k8, c = idx % k8;       // c: float4 piece within the row
+                    xq[(int64_t) n * (K / 4) + c] = (q0 & 0xFF) | ((q1 & 0xFF) << 8) | ((q2 & 0xFF) << 16) | ((q3 & 0xFF) << 24);
+                    if ((c & 7) == 0) {
+                        xd[n * nbk + c / 8]   = h2f(f2h_bits(d));     // the CPU backend stores d as f16 and reads it back
+                        xsum[n * nbk + c / 8] = sum;
+                    }
+                }
             }
         }
     }
@@ -572,12 +795,12 @@ extern "C" const char * mi355x_mul_mat_kernel_name(const mi355x_tensor * src0, c
     }
 }
 
-// the GEMM with quantized weights rounds src1 to Q8_0 into `workspace` as f16 [ne13*ne12][N][K]; the GEMV does it in LDS
+// the GEMM with quantized weights quantizes src1 into `workspace`: per batch slice int8 [N][K], then f32 scales [K/32][N]
 extern "C" size_t mi355x_mul_mat_workspace_size(const mi355x_tensor * src0, const mi355x_tensor * src1) {
     if (!src0 || !src1) return 0;
     if (blck_size(src0->type) == 1 || src1->type != MI355X_TYPE_F32 || mm_path(src0, src1) != MM_GEMM) return 0;
-    const size_t n = (size_t) src1->ne[0] * src1->ne[1] * src1->ne[2] * src1->ne[3] * 2;
-    return (n + 255) / 256 * 256;
+    const size_t K = (size_t) src1->ne[0], N = (size_t) src1->ne[1];
+    return (round256(N * K) + round256(K / QK * N * 4)) * (size_t)(src1->ne[2] * src1->ne[3]);
 }
 
 extern "C" int mi355x_mul_mat(const mi355x_tensor * src0, const mi355x_tensor * src1, const mi355x_tensor * dst,
@@ -611,6 +834,8 @@ extern "C" int mi355x_mul_mat(const mi355x_tensor * src0, const mi355x_tensor * 
     a.e.flags = flags; a.e.scale = epi ? epi->scale : 1.0f;
     a.e.bias = epi ? (const float *) epi->bias : nullptr;
     a.e.residual = epi ? (const char *) epi->residual : nullptr;
+    a.e.gelu = nullptr;
+    if ((flags & MI355X_EPI_GELU) && !(a.e.gelu = gelu_table_device())) return MI355X_ERR_HIP;
 
     hipStream_t st = (hipStream_t) stream;
     const int64_t nbatch = a.ne12 * a.ne13;
@@ -626,16 +851,20 @@ extern "C" int mi355x_mul_mat(const mi355x_tensor * src0, const mi355x_tensor * 
         if (grid.y > 65535) return MI355X_ERR_UNSUPPORTED;
         if (quant && t1 == MI355X_TYPE_F32 && !(flags & MI355X_MM_EXACT_ACT)) {
             const size_t need = mi355x_mul_mat_workspace_size(src0, src1);
-            if (!workspace || workspace_size < need || (uintptr_t) workspace % 16 != 0) return MI355X_ERR_WORKSPACE;
+            if (!workspace || workspace_size < need || (uintptr_t) workspace % 256 != 0) return MI355X_ERR_WORKSPACE;
+            const int64_t xd_off = (int64_t) round256((size_t)(a.N * a.K));
+            const int64_t slice  = xd_off + (int64_t) round256((size_t)(a.K / QK * a.N * 4));
             if (!(flags & MI355X_MM_WS_READY)) {
                 const int64_t threads = a.K / 4 * a.N;
                 dim3 qgrid((unsigned)((threads + 255) / 256), (unsigned) nbatch);
-                k_round_act_q8_0<<<qgrid, 256, 0, st>>>(a.x, (half_t *) workspace, a.K, a.N, a.x_nb1, a.x_nb2, a.ne12, a.x_nb3);
+                k_quantize_act<<<qgrid, 256, 0, st>>>(a.x, (char *) workspace, a.K, a.N, a.x_nb1, a.x_nb2, a.ne12, a.x_nb3, slice, xd_off);
             }
-            a.x = (const char *) workspace;
-            a.x_nb1 = a.K * 2; a.x_nb2 = a.N * a.K * 2; a.x_nb3 = a.ne12 * a.N * a.K * 2;
-            if (t0 == MI355X_TYPE_Q5_0) k_gemm_mfma<MI355X_TYPE_Q5_0, MI355X_TYPE_F16><<<grid, 256, 0, st>>>(a);
-            else                        k_gemm_mfma<MI355X_TYPE_Q8_0, MI355X_TYPE_F16><<<grid, 256, 0, st>>>(a);
+            i8_args ia;
+            ia.m = a;
+            ia.m.x = (const char *) workspace; ia.m.x_nb1 = a.K; ia.m.x_nb2 = slice; ia.m.x_nb3 = slice * a.ne12;
+            ia.xd = (const char *) workspace + xd_off; ia.xd_slice = slice;
+            if (t0 == MI355X_TYPE_Q5_0) k_gemm_i8<MI355X_TYPE_Q5_0><<<grid, 256, 0, st>>>(ia);
+            else                        k_gemm_i8<MI355X_TYPE_Q8_0><<<grid, 256, 0, st>>>(ia);
             return launch_status();
         }
         if (t1 == MI355X_TYPE_F16) {

@@ -22,7 +22,14 @@ __global__ void k_norm(tview s, tview d, int64_t nrows, float eps, const float *
 
     if (IN_REGS) {
         const int n4 = (int)(ne0 / 4);
-        float4 v[NORM_MAX_V4];
+        float4 v[NORM_MAX_V4], ww[NORM_MAX_V4], bb[NORM_MAX_V4];
+        // the affine vectors are fetched together with the row, not after the two reductions
+#pragma unroll
+        for (int j = 0; j < NORM_MAX_V4; ++j) {
+            const int c = lane + j * WAVE;
+            ww[j] = make_float4(1.f, 1.f, 1.f, 1.f); bb[j] = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (c < n4) { if (w) ww[j] = ((const float4 *) w)[c]; if (b) bb[j] = ((const float4 *) b)[c]; }
+        }
         float sum = 0.0f;
 #pragma unroll
         for (int j = 0; j < NORM_MAX_V4; ++j) {
@@ -45,8 +52,8 @@ __global__ void k_norm(tview s, tview d, int64_t nrows, float eps, const float *
             const int c = lane + j * WAVE;
             if (c < n4) {
                 float4 r = { v[j].x * scale, v[j].y * scale, v[j].z * scale, v[j].w * scale };
-                if (w) { const float4 ww = ((const float4 *) w)[c]; r.x *= ww.x; r.y *= ww.y; r.z *= ww.z; r.w *= ww.w; }
-                if (b) { const float4 bb = ((const float4 *) b)[c]; r.x += bb.x; r.y += bb.y; r.z += bb.z; r.w += bb.w; }
+                if (w) { r.x *= ww[j].x; r.y *= ww[j].y; r.z *= ww[j].z; r.w *= ww[j].w; }
+                if (b) { r.x += bb[j].x; r.y += bb[j].y; r.z += bb[j].z; r.w += bb[j].w; }
                 ((float4 *) y)[c] = r;
             }
         }
