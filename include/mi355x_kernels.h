@@ -62,8 +62,10 @@ enum mi355x_epilogue_flags {
     MI355X_EPI_OUT_F16  = 32,  /* dst is f16 instead of f32 (ggml CPY f32->f16 folded in)                      */
     /* not epilogue parts, but options of the same call: */
     MI355X_MM_EXACT_ACT = 64,  /* GEMM path: keep src1 at f16 precision instead of rounding it to Q8_0 first   */
-    MI355X_MM_WS_READY  = 128, /* GEMM path: `workspace` already holds the Q8_0-rounded src1 of this call
-                                  (left there by the previous call with the same src1): skip the rounding pass */
+    MI355X_MM_WS_READY  = 128, /* GEMM path: `workspace` already holds the f16 image of this call's src1 (left
+                                  there by the previous call with the same src1): skip the conversion pass     */
+    MI355X_MM_ACT_Q8_0  = 256, /* GEMM path, F16 src0 that is the f16 image (mi355x_dequantize_row_f16) of a
+                                  quantized weight: round src1 to Q8_0 as for the quantized weight itself      */
 };
 
 typedef struct mi355x_epilogue {
@@ -85,6 +87,8 @@ MI355X_API const char * mi355x_status_string(int status);
  * dequantize_row_q5_0 / dequantize_row_q8_0 (ggml/src/ggml-quants.c:296-319, 349-363): y[i] = d * q,
  * bit-exact.  `k` weights (multiple of 32) from `src` (device) to f32 `dst` (device). */
 MI355X_API int mi355x_dequantize_row(int type, const void * src, float * dst, int64_t k, void * stream);
+/* the same rows as f16: y[i] = f16(d * q), the exact product rounded once to nearest even */
+MI355X_API int mi355x_dequantize_row_f16(int type, const void * src, void * dst, int64_t k, void * stream);
 
 /* quantize_row_q8_0 of the CPU backend's AVX2 build (ggml/src/ggml-cpu/ggml-cpu-quants.c:738,808-865):
  * per 32 values d = amax/127 stored as f16, q = round-to-nearest-even(x * (127/amax)).  `k` multiple of 32. */
@@ -98,10 +102,13 @@ MI355X_API int mi355x_quantize_row_q8_0(const float * src, void * dst, int64_t k
  * Columns n <= MI355X_GEMV_MAX_COLS with a quantized src0 take the HBM-streaming GEMV path, which
  * quantizes src1 to Q8_0 (in LDS) exactly like the CPU backend does (ggml-cpu.c:1328-1363) and
  * accumulates integer block dot products like ggml_vec_dot_q5_0_q8_0 / ggml_vec_dot_q8_0_q8_0
- * (ggml-cpu-quants.c:2930, 3597).  Everything else runs the MFMA GEMM (weights dequantized to f16 on the
- * way into LDS, f32 accumulation).  With quantized weights the GEMM, too, first rounds src1 to Q8_0 — one
- * pass that writes d*q as f16 into `workspace` (size from mi355x_mul_mat_workspace_size) — because that
- * rounding is part of what the reference computes; MI355X_MM_EXACT_ACT turns it off. */
+ * (ggml-cpu-quants.c:2930, 3597).  Everything else runs the MFMA GEMM: f16 operands, f32 accumulation.
+ * Its operands are brought to dense f16 rows in `workspace` (256-byte aligned, size from
+ * mi355x_mul_mat_workspace_size) by one pass each: an F32 src1 first, then a src0 that is not F16 (blocks
+ * expanded to f16(d*q)).  With quantized weights the src1 pass also rounds to Q8_0 — it writes f16(d*q) of
+ * the Q8_0 blocks — because that rounding is part of what the reference computes; MI355X_MM_EXACT_ACT turns
+ * it off.  A caller that reuses a quantized weight keeps its f16 image (mi355x_dequantize_row_f16) and
+ * passes that as an F16 src0 with MI355X_MM_ACT_Q8_0, which skips the src0 pass. */
 #define MI355X_GEMV_MAX_COLS 8
 /* name of the kernel mi355x_mul_mat would launch for these operands ("mul_mat.gemm_q5_0", "mul_mat.gemv_q8_0", ...);
  * a static string, used to label profiles */

@@ -24,7 +24,7 @@ BLOCK_BYTES = {Q5_0: 22, Q8_0: 34}
 
 # enum mi355x_epilogue_flags
 EPI_BIAS, EPI_GELU, EPI_SCALE, EPI_RESIDUAL, EPI_BIAS_COL, EPI_OUT_F16 = 1, 2, 4, 8, 16, 32
-MM_EXACT_ACT, MM_WS_READY = 64, 128
+MM_EXACT_ACT, MM_WS_READY, MM_ACT_Q8_0 = 64, 128, 256
 # enum mi355x_fa_mode
 FA_F16_SEQ, FA_F32 = 0, 1
 
@@ -59,6 +59,7 @@ def kernels() -> C.CDLL:
             "mi355x_device_is_gfx950": (C.c_int, [C.c_int]),
             "mi355x_status_string": (C.c_char_p, [C.c_int]),
             "mi355x_dequantize_row": (C.c_int, [C.c_int, P, P, C.c_int64, P]),
+            "mi355x_dequantize_row_f16": (C.c_int, [C.c_int, P, P, C.c_int64, P]),
             "mi355x_quantize_row_q8_0": (C.c_int, [P, P, C.c_int64, P]),
             "mi355x_mul_mat_kernel_name": (C.c_char_p, [T, T]),
             "mi355x_mul_mat_workspace_size": (C.c_size_t, [T, T]),

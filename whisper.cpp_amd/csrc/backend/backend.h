@@ -34,11 +34,31 @@ struct mi355x_device_ctx {
     std::string description;   // marketing name from the driver
 };
 
+// f16 image of a quantized weight tensor (rows of f16(d * q)), operand of the MFMA GEMM
+struct mi355x_weight_image {
+    void * f16;        // device memory, ne0 * ne1 halves
+    size_t src_bytes;  // bytes of the tensor it mirrors
+    int    type;
+    int64_t ne0, ne1;
+};
+
 struct mi355x_buffer_ctx {
     int    device;
     void * base;
     size_t size;
+    // Weight buffers keep, next to a Q5_0 / Q8_0 matrix that is multiplied with many columns at once, its f16 image:
+    // 2 bytes per weight more HBM, so that the GEMM streams matrix-core operands instead of unpacking the same blocks
+    // in every workgroup and on every call.  Keyed by the tensor's data address; anything that writes into the buffer
+    // drops the images it overlaps.
+    std::mutex                               image_mutex;
+    std::map<uintptr_t, mi355x_weight_image> images;
+
+    const void * weight_image(const struct ggml_tensor * w, hipStream_t stream);   // NULL: none could be made
+    void         drop_images(const void * begin, size_t size);
+    void         drop_all_images();
 };
+
+bool mi355x_buffer_is_ours(ggml_backend_buffer_t buffer);
 
 struct mi355x_kernel_stat {
     int64_t calls = 0;
@@ -60,6 +80,7 @@ struct mi355x_backend_ctx {
     bool        fuse    = true;
     bool        profile = false;
     bool        debug   = false;   // log what every MUL_MAT launch folds in (GGML_MI355X_DEBUG=1)
+    bool        weight_images = true;   // keep f16 images of quantized GEMM weights (GGML_MI355X_WEIGHT_IMAGES=0 turns it off)
     bool        exact   = false;   // true: f32 attention accumulators and un-rounded GEMM activations instead of the
                                    // reference's f16-sequential / Q8_0-rounded arithmetic
 
@@ -67,6 +88,7 @@ struct mi355x_backend_ctx {
     void *       ws       = nullptr;
     size_t       ws_size  = 0;
     const void * ws_x     = nullptr;
+    int          ws_x_mode = 0;
     int64_t      ws_x_ne[4] = {0, 0, 0, 0};
     size_t       ws_x_nb[4] = {0, 0, 0, 0};
     bool         reserve_workspace(size_t size);

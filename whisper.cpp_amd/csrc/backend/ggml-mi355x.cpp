@@ -35,10 +35,49 @@ static bool env_flag(const char * name, bool dflt) {
 // buffer  (ggml_backend_buffer_i, ggml-backend-impl.h:41-58)
 // ------------------------------------------------------------------------------------------------------
 
+const void * mi355x_buffer_ctx::weight_image(const struct ggml_tensor * w, hipStream_t stream) {
+    std::lock_guard<std::mutex> lock(image_mutex);
+    const uintptr_t key = (uintptr_t) w->data;
+    auto it = images.find(key);
+    if (it != images.end()) {
+        const mi355x_weight_image & im = it->second;
+        if (im.type == (int) w->type && im.ne0 == w->ne[0] && im.ne1 == w->ne[1]) return im.f16;
+        (void) hipFree(im.f16);                       // same address, another tensor: the buffer was laid out anew
+        images.erase(it);
+    }
+    mi355x_weight_image im = { nullptr, ggml_nbytes(w), (int) w->type, w->ne[0], w->ne[1] };
+    const int64_t n = w->ne[0] * w->ne[1];
+    if (hipMalloc(&im.f16, (size_t) n * 2) != hipSuccess || !im.f16) {
+        (void) hipGetLastError();
+        static bool warned = false;
+        if (!warned) { warned = true; GGML_LOG_WARN("ggml-mi355x: no memory for the f16 image of %s (%.1f MiB); its blocks are unpacked on every call\n", w->name, n * 2 / 1048576.0); }
+        return nullptr;
+    }
+    if (mi355x_dequantize_row_f16((int) w->type, w->data, im.f16, n, stream) != MI355X_OK) { (void) hipFree(im.f16); return nullptr; }
+    images.emplace(key, im);
+    return im.f16;
+}
+
+void mi355x_buffer_ctx::drop_images(const void * begin, size_t nbytes) {
+    std::lock_guard<std::mutex> lock(image_mutex);
+    const uintptr_t b = (uintptr_t) begin, e = b + nbytes;
+    for (auto it = images.begin(); it != images.end();) {
+        if (it->first < e && b < it->first + it->second.src_bytes) { (void) hipFree(it->second.f16); it = images.erase(it); }   // hipFree waits for the device
+        else ++it;
+    }
+}
+
+void mi355x_buffer_ctx::drop_all_images() {
+    std::lock_guard<std::mutex> lock(image_mutex);
+    for (auto & kv : images) (void) hipFree(kv.second.f16);
+    images.clear();
+}
+
 static void buffer_free(ggml_backend_buffer_t buffer) {
     mi355x_buffer_ctx * ctx = (mi355x_buffer_ctx *) buffer->context;
     HIP_TRY(hipSetDevice(ctx->device), (void) 0);
     HIP_TRY(hipDeviceSynchronize(), (void) 0);
+    ctx->drop_all_images();
     HIP_TRY(hipFree(ctx->base), (void) 0);
     delete ctx;
 }
@@ -57,6 +96,7 @@ static enum ggml_status buffer_init_tensor(ggml_backend_buffer_t, struct ggml_te
 static void buffer_memset_tensor(ggml_backend_buffer_t buffer, struct ggml_tensor * tensor, uint8_t value, size_t offset, size_t size) {
     mi355x_buffer_ctx * ctx = (mi355x_buffer_ctx *) buffer->context;
     HIP_TRY(hipSetDevice(ctx->device), return);
+    if (!ctx->images.empty()) ctx->drop_images((char *) tensor->data + offset, size);
     HIP_TRY(hipMemset((char *) tensor->data + offset, value, size), return);
     HIP_TRY(hipStreamSynchronize(nullptr), return);
 }
@@ -64,6 +104,7 @@ static void buffer_memset_tensor(ggml_backend_buffer_t buffer, struct ggml_tenso
 static void buffer_set_tensor(ggml_backend_buffer_t buffer, struct ggml_tensor * tensor, const void * data, size_t offset, size_t size) {
     mi355x_buffer_ctx * ctx = (mi355x_buffer_ctx *) buffer->context;
     HIP_TRY(hipSetDevice(ctx->device), return);
+    if (!ctx->images.empty()) ctx->drop_images((char *) tensor->data + offset, size);
     HIP_TRY(hipMemcpy((char *) tensor->data + offset, data, size, hipMemcpyHostToDevice), return);
 }
 
@@ -74,12 +115,14 @@ static void buffer_get_tensor(ggml_backend_buffer_t buffer, const struct ggml_te
 }
 
 static bool buffer_is_mi355x(ggml_backend_buffer_t buffer) { return buffer && buffer->iface.get_base == buffer_get_base; }
+bool mi355x_buffer_is_ours(ggml_backend_buffer_t buffer) { return buffer_is_mi355x(buffer); }
 
 static bool buffer_cpy_tensor(ggml_backend_buffer_t buffer, const struct ggml_tensor * src, struct ggml_tensor * dst) {
     mi355x_buffer_ctx * ctx = (mi355x_buffer_ctx *) buffer->context;
     ggml_backend_buffer_t sbuf = src->view_src ? src->view_src->buffer : src->buffer;
     if (!ggml_is_contiguous(src) || !ggml_is_contiguous(dst) || ggml_nbytes(src) != ggml_nbytes(dst)) return false;
     HIP_TRY(hipSetDevice(ctx->device), return false);
+    if (!ctx->images.empty()) ctx->drop_images(dst->data, ggml_nbytes(dst));
     if (buffer_is_mi355x(sbuf)) {
         HIP_TRY(hipMemcpy(dst->data, src->data, ggml_nbytes(src), hipMemcpyDeviceToDevice), return false);
         HIP_TRY(hipStreamSynchronize(nullptr), return false);
@@ -95,6 +138,7 @@ static bool buffer_cpy_tensor(ggml_backend_buffer_t buffer, const struct ggml_te
 static void buffer_clear(ggml_backend_buffer_t buffer, uint8_t value) {
     mi355x_buffer_ctx * ctx = (mi355x_buffer_ctx *) buffer->context;
     HIP_TRY(hipSetDevice(ctx->device), return);
+    ctx->drop_all_images();
     HIP_TRY(hipMemset(ctx->base, value, ctx->size), return);
     HIP_TRY(hipDeviceSynchronize(), return);
 }
@@ -130,7 +174,8 @@ static ggml_backend_buffer_t buft_alloc_buffer(ggml_backend_buffer_type_t buft, 
         GGML_LOG_ERROR("ggml-mi355x: allocating %.2f MiB on device %d failed: %s\n", alloc / 1048576.0, dev->device, hipGetErrorString(err));
         return NULL;
     }
-    mi355x_buffer_ctx * ctx = new mi355x_buffer_ctx{ dev->device, base, size };
+    mi355x_buffer_ctx * ctx = new mi355x_buffer_ctx;
+    ctx->device = dev->device; ctx->base = base; ctx->size = size;
     return ggml_backend_buffer_init(buft, mi355x_buffer_iface, ctx, size);
 }
 
@@ -205,6 +250,11 @@ static void backend_free(ggml_backend_t backend) {
 static void backend_set_tensor_async(ggml_backend_t backend, struct ggml_tensor * tensor, const void * data, size_t offset, size_t size) {
     mi355x_backend_ctx * ctx = (mi355x_backend_ctx *) backend->context;
     HIP_TRY(hipSetDevice(ctx->device), return);
+    ggml_backend_buffer_t buf = tensor->view_src ? tensor->view_src->buffer : tensor->buffer;
+    if (buffer_is_mi355x(buf)) {
+        mi355x_buffer_ctx * bctx = (mi355x_buffer_ctx *) buf->context;
+        if (!bctx->images.empty()) bctx->drop_images((char *) tensor->data + offset, size);
+    }
     HIP_TRY(hipMemcpyAsync((char *) tensor->data + offset, data, size, hipMemcpyHostToDevice, ctx->stream), return);
 }
 
@@ -267,6 +317,7 @@ static ggml_backend_t device_init_backend(ggml_backend_dev_t dev, const char *) 
     ctx->fuse    = env_flag("GGML_MI355X_FUSE", true);
     ctx->profile = env_flag("GGML_MI355X_PROFILE", false);
     ctx->exact   = env_flag("GGML_MI355X_EXACT", false);
+    ctx->weight_images = env_flag("GGML_MI355X_WEIGHT_IMAGES", true);
     ctx->debug   = env_flag("GGML_MI355X_DEBUG", false);
     // default priority, blocking with respect to the null stream used by the buffer-level copies
     HIP_TRY(hipStreamCreate(&ctx->stream), { delete ctx; return NULL; });

@@ -264,23 +264,39 @@ struct graph_runner {
         const double flops = 2.0 * mm->ne[0] * mm->ne[1] * w->ne[0] * batch;
         const double bytes = nbytes_of(w) + nbytes_of(x) + (double) ggml_nelements(mm) * ((epi.flags & MI355X_EPI_OUT_F16) ? 2 : 4) +
                              ((epi.flags & MI355X_EPI_RESIDUAL) ? nbytes_of(mm) : 0.0);
-        // the GEMM rounds src1 to Q8_0 into the workspace first; consecutive MUL_MATs over the same activations
-        // (Q, K, V projections) share that copy
+        const char * kernel_name = mi355x_mul_mat_kernel_name(&vw, &vx);
         if (ctx->exact) epi.flags |= MI355X_MM_EXACT_ACT;
-        const size_t need = ctx->exact ? 0 : mi355x_mul_mat_workspace_size(&vw, &vx);
+        // a quantized weight matrix that meets many columns is multiplied through its f16 image, kept beside it in HBM
+        if (ctx->weight_images && ggml_is_quantized(w->type) && w->ne[2] == 1 && w->ne[3] == 1 && ggml_is_contiguous(w) && !w->view_src &&
+            w->buffer && w->buffer->usage == GGML_BACKEND_BUFFER_USAGE_WEIGHTS && mi355x_buffer_is_ours(w->buffer) &&
+            strncmp(kernel_name, "mul_mat.gemm", 12) == 0) {
+            const void * image = ((mi355x_buffer_ctx *) w->buffer->context)->weight_image(w, ctx->stream);
+            if (image) {
+                vw.data = (void *) image; vw.type = MI355X_TYPE_F16;
+                vw.nb[0] = 2; vw.nb[1] = 2 * (size_t) w->ne[0]; vw.nb[2] = vw.nb[1] * (size_t) w->ne[1]; vw.nb[3] = vw.nb[2];
+                epi.flags |= MI355X_MM_ACT_Q8_0;
+            }
+        }
+        // the GEMM first brings src1 to f16 (rounded to Q8_0 on the way when the weights are quantized) in the workspace;
+        // consecutive MUL_MATs over the same activations (Q, K, V projections) share that copy
+        const size_t need = mi355x_mul_mat_workspace_size(&vw, &vx);
         if (need) {
             if (!ctx->reserve_workspace(need)) { status = MI355X_ERR_WORKSPACE; return used; }
-            const bool hit = ctx->ws_x == x->data && memcmp(ctx->ws_x_ne, x->ne, sizeof(x->ne)) == 0 && memcmp(ctx->ws_x_nb, x->nb, sizeof(x->nb)) == 0;
-            if (hit) epi.flags |= MI355X_MM_WS_READY;
-            ctx->ws_x = x->data; memcpy(ctx->ws_x_ne, x->ne, sizeof(x->ne)); memcpy(ctx->ws_x_nb, x->nb, sizeof(x->nb));
-            cached_x = x;
+            if (x->type == GGML_TYPE_F32) {
+                const int mode = (ggml_is_quantized(w->type) && !ctx->exact) ? 1 : 0;       // 1: rounded to Q8_0
+                const bool hit = ctx->ws_x == x->data && ctx->ws_x_mode == mode && memcmp(ctx->ws_x_ne, x->ne, sizeof(x->ne)) == 0 &&
+                                 memcmp(ctx->ws_x_nb, x->nb, sizeof(x->nb)) == 0;
+                if (hit) epi.flags |= MI355X_MM_WS_READY;
+                ctx->ws_x = x->data; ctx->ws_x_mode = mode; memcpy(ctx->ws_x_ne, x->ne, sizeof(x->ne)); memcpy(ctx->ws_x_nb, x->nb, sizeof(x->nb));
+                cached_x = x;
+            }
         }
         if (ctx->debug) {
-            GGML_LOG_INFO("ggml-mi355x: %s %s [%lld x %lld x %lld] folds %d nodes, flags 0x%x\n", mi355x_mul_mat_kernel_name(&vw, &vx), mm->name,
+            GGML_LOG_INFO("ggml-mi355x: %s %s [%lld x %lld x %lld] folds %d nodes, flags 0x%x\n", kernel_name, mm->name,
                           (long long) mm->ne[0], (long long) mm->ne[1], (long long) w->ne[0], used, epi.flags);
         }
         {
-            launch_scope ls(ctx, mi355x_mul_mat_kernel_name(&vw, &vx), bytes, flops);
+            launch_scope ls(ctx, kernel_name, bytes, flops);
             status = mi355x_mul_mat(&vw, &vx, &vd, epi.flags ? &epi : nullptr, ctx->ws, ctx->ws_size, ctx->stream);
         }
         note_write(out);

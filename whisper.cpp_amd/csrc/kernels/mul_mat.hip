@@ -15,6 +15,7 @@
 //                     ggml_vec_dot_q8_0_q8_0 / ggml_vec_dot_q5_0_q8_0 (ggml-cpu-quants.c:3597, 2930).
 //   * k_mul_mat_generic — any strides / K; one wavefront per output row, f32 FMA.
 #include "common.h"
+#include <stdlib.h>
 
 typedef uint32_t __attribute__((aligned(2))) u32a2;
 struct __attribute__((packed, aligned(2))) u128a2 { uint32_t x, y, z, w; };
@@ -38,6 +39,55 @@ __device__ __forceinline__ float apply_epilogue(float v, const epi_args & e, int
     if (e.flags & MI355X_EPI_SCALE)    v *= e.scale;
     if (e.flags & MI355X_EPI_RESIDUAL) v += *(const float *)(e.residual + res_off);
     return v;
+}
+
+// The same for the 16 registers of one 32x32 accumulator patch (column m, rows n[0..15]) and the stores.  All loads of
+// one kind are issued together before their first use; rows beyond N and columns beyond M are computed from clamped
+// addresses and not stored.
+__device__ __forceinline__ void patch_epilogue(float16_t v, const epi_args & e, char * db, int64_t batch_off, int64_t d_nb1,
+                                               int64_t m, int64_t M, const int64_t (&n)[16], int64_t N) {
+    const bool    m_ok = m < M;
+    const int64_t mc   = m_ok ? m : M - 1;
+    int64_t nc[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) nc[i] = n[i] < N ? n[i] : N - 1;
+    if (e.flags & MI355X_EPI_BIAS) {
+        const float b = e.bias[mc];
+#pragma unroll
+        for (int i = 0; i < 16; ++i) v[i] += b;
+    }
+    if (e.flags & MI355X_EPI_BIAS_COL) {
+        float b[16];
+#pragma unroll
+        for (int i = 0; i < 16; ++i) b[i] = e.bias[nc[i]];
+#pragma unroll
+        for (int i = 0; i < 16; ++i) v[i] += b[i];
+    }
+    if (e.flags & MI355X_EPI_GELU) {
+        uint16_t t[16];
+#pragma unroll
+        for (int i = 0; i < 16; ++i) t[i] = e.gelu[f2h_bits(v[i])];
+#pragma unroll
+        for (int i = 0; i < 16; ++i) v[i] = v[i] <= -10.0f ? 0.0f : v[i] >= 10.0f ? v[i] : h2f(t[i]);
+    }
+    if (e.flags & MI355X_EPI_SCALE) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) v[i] *= e.scale;
+    }
+    if (e.flags & MI355X_EPI_RESIDUAL) {
+        float r[16];
+#pragma unroll
+        for (int i = 0; i < 16; ++i) r[i] = *(const float *)(e.residual + batch_off + nc[i] * d_nb1 + mc * 4);
+#pragma unroll
+        for (int i = 0; i < 16; ++i) v[i] += r[i];
+    }
+    if (e.flags & MI355X_EPI_OUT_F16) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) if (m_ok && n[i] < N) *(half_t *)(db + n[i] * d_nb1 + m * 2) = (half_t) v[i];
+    } else {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) if (m_ok && n[i] < N) *(float *)(db + n[i] * d_nb1 + m * 4) = v[i];
+    }
 }
 
 struct mm_args {
@@ -102,440 +152,251 @@ __device__ __forceinline__ void q8_0_to_half32(uint32_t d_bits, const uint32_t q
 }
 
 // ------------------------------------------------------------------------------------------------------
-// MFMA GEMM
+// MFMA GEMM: operand conversion passes + one f16 x f16 -> f32 kernel
+//
+// Both operands reach the matrix cores as dense f16 rows [rows][K]:
+//   * src1 (F32) is converted by k_x_to_f16.  For quantized weights the CPU backend first rounds src1 to Q8_0
+//     (ggml-cpu.c:1328-1363, quantize_row_q8_0 ggml-cpu-quants.c:808-865): the pass reproduces that rounding —
+//     block amax, id = 127/amax, round half to even, d stored as f16 — and writes f16(q * d).  For F16 / F32
+//     weights (or when the caller asks for un-rounded activations) it is a plain f32 -> f16 conversion, which is
+//     what the CPU backend does for F16 weights.
+//   * src0 blocks are expanded by k_w_to_f16 to f16(d * q) unless src0 already is F16.  A caller that multiplies by
+//     the same weights many times keeps that f16 image itself and passes it as an F16 src0 with MI355X_MM_ACT_Q8_0.
 // ------------------------------------------------------------------------------------------------------
 
-#define GB_M 128      // W rows per block
-#define GB_N 128      // X rows per block
-#define GB_K 64
-#define GB_LD (GB_K + 8)   // LDS row pitch in halves: 144 B, so 8 consecutive rows start 4 banks apart
+static inline size_t round256(size_t n) { return (n + 255) / 256 * 256; }
 
-// per-thread staging registers for one K step
-template <int T0> struct w_frag;
-template <> struct w_frag<MI355X_TYPE_Q5_0> { uint32_t d, qh, qs[4]; };
-template <> struct w_frag<MI355X_TYPE_Q8_0> { uint32_t d, qs[8]; };
-template <> struct w_frag<MI355X_TYPE_F16>  { uint4 h[4]; };
-template <> struct w_frag<MI355X_TYPE_F32>  { float4 f[8]; };
-template <int T1> struct x_frag;
-template <> struct x_frag<MI355X_TYPE_F32>  { float4 f[8]; };
-template <> struct x_frag<MI355X_TYPE_F16>  { uint4 h[4]; };
-
-// thread t stages W row t/2, k-half t%2 (32 weights)
+// one thread per 32 weights
 template <int T0>
-__device__ __forceinline__ void load_w(w_frag<T0> & f, const char * wrow, bool row_ok, int64_t k0, int64_t K) {
-    const int kh = threadIdx.x & 1;
-    const int64_t k = k0 + kh * 32;
-    if constexpr (T0 == MI355X_TYPE_Q5_0) {
-        if (row_ok && k < K) {
-            const uint8_t * b = (const uint8_t *) wrow + (k / QK) * 22;
-            f.d  = *(const uint16_t *) b;
-            f.qh = *(const u32a2 *)(b + 2);
-            const u128a2 q = *(const u128a2 *)(b + 6);
-            f.qs[0] = q.x; f.qs[1] = q.y; f.qs[2] = q.z; f.qs[3] = q.w;
-        } else {
-            f.d = 0; f.qh = 0; f.qs[0] = f.qs[1] = f.qs[2] = f.qs[3] = 0;
-        }
-    } else if constexpr (T0 == MI355X_TYPE_Q8_0) {
-        if (row_ok && k < K) {
-            const uint8_t * b = (const uint8_t *) wrow + (k / QK) * 34;
-            f.d = *(const uint16_t *) b;
-            const u128a2 q0 = *(const u128a2 *)(b + 2);
-            const u128a2 q1 = *(const u128a2 *)(b + 18);
-            f.qs[0] = q0.x; f.qs[1] = q0.y; f.qs[2] = q0.z; f.qs[3] = q0.w;
-            f.qs[4] = q1.x; f.qs[5] = q1.y; f.qs[6] = q1.z; f.qs[7] = q1.w;
-        } else {
-            f.d = 0;
-#pragma unroll
-            for (int i = 0; i < 8; ++i) f.qs[i] = 0;
-        }
-    } else if constexpr (T0 == MI355X_TYPE_F16) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int64_t kk = k + 8 * i;
-            f.h[i] = (row_ok && kk < K) ? *(const uint4 *)(wrow + kk * 2) : make_uint4(0, 0, 0, 0);
-        }
-    } else {
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            const int64_t kk = k + 4 * i;
-            f.f[i] = (row_ok && kk < K) ? *(const float4 *)(wrow + kk * 4) : make_float4(0.f, 0.f, 0.f, 0.f);
-        }
-    }
-}
-
-__device__ __forceinline__ half4_t f4_to_h4(float4 v) {
-    half4_t h = { (half_t) v.x, (half_t) v.y, (half_t) v.z, (half_t) v.w };
-    return h;
-}
-
-template <int T0>
-__device__ __forceinline__ void store_w(const w_frag<T0> & f, half_t * ws) {
-    half_t * p = ws + (threadIdx.x >> 1) * GB_LD + (threadIdx.x & 1) * 32;
+__global__ void k_w_to_f16(const char * __restrict__ w, half_t * __restrict__ out, int64_t K, int64_t M, int64_t w_nb1, int64_t w_nb2,
+                           int64_t ne02, int64_t w_nb3, int64_t slice_halves) {
+    const int64_t t   = (int64_t) blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t nbk = K / QK;
+    if (t >= nbk * M) return;
+    const int64_t m = t / nbk, kb = t % nbk, b = blockIdx.y;
+    const uint8_t * row = (const uint8_t *) w + m * w_nb1 + (b % ne02) * w_nb2 + (b / ne02) * w_nb3;
     half8_t o[4];
     if constexpr (T0 == MI355X_TYPE_Q5_0) {
-        q5_0_to_half32(f.d, f.qh, f.qs, o);
+        const uint8_t * p = row + kb * 22;
+        const u128a2 q = *(const u128a2 *)(p + 6);
+        const uint32_t qs[4] = { q.x, q.y, q.z, q.w };
+        q5_0_to_half32(*(const uint16_t *) p, *(const u32a2 *)(p + 2), qs, o);
     } else if constexpr (T0 == MI355X_TYPE_Q8_0) {
-        q8_0_to_half32(f.d, f.qs, o);
-    } else if constexpr (T0 == MI355X_TYPE_F16) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) __builtin_memcpy(&o[i], &f.h[i], 16);
+        const uint8_t * p = row + kb * 34;
+        const u128a2 q0 = *(const u128a2 *)(p + 2), q1 = *(const u128a2 *)(p + 18);
+        const uint32_t qs[8] = { q0.x, q0.y, q0.z, q0.w, q1.x, q1.y, q1.z, q1.w };
+        q8_0_to_half32(*(const uint16_t *) p, qs, o);
     } else {
+        const float4 * p = (const float4 *)(row + kb * QK * 4);
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            const half4_t a = f4_to_h4(f.f[2*i]), b = f4_to_h4(f.f[2*i + 1]);
-            o[i] = (half8_t){ a[0], a[1], a[2], a[3], b[0], b[1], b[2], b[3] };
+            const float4 u = p[2*i], v = p[2*i + 1];
+            o[i] = (half8_t){ (half_t) u.x, (half_t) u.y, (half_t) u.z, (half_t) u.w, (half_t) v.x, (half_t) v.y, (half_t) v.z, (half_t) v.w };
         }
     }
+    half8_t * dst = (half8_t *)(out + b * slice_halves + m * K + kb * QK);
 #pragma unroll
-    for (int i = 0; i < 4; ++i) *(half8_t *)(p + 8 * i) = o[i];
+    for (int i = 0; i < 4; ++i) dst[i] = o[i];
 }
 
-// X tile, F32: thread t covers float4 column t%16 of rows t/16 + 16 i (i < 8)
-// X tile, F16: thread t covers 8-half column t%8 of rows t/8 + 32 i (i < 4)
-template <int T1>
-__device__ __forceinline__ void load_x(x_frag<T1> & f, const char * xb, int64_t x_nb1, int64_t n0, int64_t N, int64_t k0, int64_t K) {
-    if constexpr (T1 == MI355X_TYPE_F32) {
-        const int c = threadIdx.x & 15, r = threadIdx.x >> 4;
-        const int64_t k = k0 + 4 * c;
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            const int64_t n = n0 + r + 16 * i;
-            f.f[i] = (n < N && k < K) ? *(const float4 *)(xb + n * x_nb1 + k * 4) : make_float4(0.f, 0.f, 0.f, 0.f);
-        }
+// 8 lanes per 32 values, 4 each
+template <bool Q8>
+__global__ void k_x_to_f16(const char * __restrict__ x, half_t * __restrict__ out, int64_t K, int64_t N,
+                           int64_t x_nb1, int64_t x_nb2, int64_t ne12, int64_t x_nb3, int64_t slice_halves) {
+    const int64_t t  = (int64_t) blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t k4 = K / 4;
+    const int64_t b  = blockIdx.y;
+    if (t >= k4 * N) return;                                                // whole 8-lane groups leave together (K % 32 == 0 when Q8)
+    const int64_t n = t / k4, c = t % k4;
+    const float4 v = *(const float4 *)(x + n * x_nb1 + (b % ne12) * x_nb2 + (b / ne12) * x_nb3 + c * 16);
+    half4_t h;
+    if (Q8) {
+        float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
+        amax = fmaxf(amax, __shfl_xor(amax, 1, 8));
+        amax = fmaxf(amax, __shfl_xor(amax, 2, 8));
+        amax = fmaxf(amax, __shfl_xor(amax, 4, 8));
+        const float id = amax != 0.0f ? 127.0f / amax : 0.0f;
+        const float d  = h2f(f2h_bits(amax / 127.0f));                      // the scale goes through f16, like block_q8_0.d
+        h = (half4_t){ (half_t)(rintf(v.x * id) * d), (half_t)(rintf(v.y * id) * d), (half_t)(rintf(v.z * id) * d), (half_t)(rintf(v.w * id) * d) };
     } else {
-        const int c = threadIdx.x & 7, r = threadIdx.x >> 3;
-        const int64_t k = k0 + 8 * c;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int64_t n = n0 + r + 32 * i;
-            f.h[i] = (n < N && k < K) ? *(const uint4 *)(xb + n * x_nb1 + k * 2) : make_uint4(0, 0, 0, 0);
-        }
+        h = (half4_t){ (half_t) v.x, (half_t) v.y, (half_t) v.z, (half_t) v.w };
     }
-}
-template <int T1>
-__device__ __forceinline__ void store_x(const x_frag<T1> & f, half_t * xs) {
-    if constexpr (T1 == MI355X_TYPE_F32) {
-        const int c = threadIdx.x & 15, r = threadIdx.x >> 4;
-#pragma unroll
-        for (int i = 0; i < 8; ++i) *(half4_t *)(xs + (r + 16 * i) * GB_LD + 4 * c) = f4_to_h4(f.f[i]);
-    } else {
-        const int c = threadIdx.x & 7, r = threadIdx.x >> 3;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) *(uint4 *)(xs + (r + 32 * i) * GB_LD + 8 * c) = f.h[i];
-    }
+    *(half4_t *)(out + b * slice_halves + n * K + c * 4) = h;
 }
 
-template <int T0, int T1>
-__global__ void __launch_bounds__(256, 2) k_gemm_mfma(mm_args a) {
-    __shared__ __attribute__((aligned(16))) half_t xs[GB_N * GB_LD];
-    __shared__ __attribute__((aligned(16))) half_t ws[GB_M * GB_LD];
+// f16 x f16 -> f32 GEMM.  256 threads = 4 wavefronts in a 2 x 2 grid; a wavefront owns TI x TJ accumulator patches of
+// 32 (src1 rows, n) x 32 (weight rows, m), each a v_mfma_f32_32x32x16_f16 chain.  src1 rows are the MFMA A operand and
+// weight rows the B operand, so a lane's accumulator column is an m index and every store instruction writes 32
+// consecutive values of a dst row.  K advances 64 at a time through two LDS buffers: while the matrix cores work on
+// step s, the global loads of step s+2 are in flight and step s+1 moves from registers to the other buffer, with one
+// barrier per step.  LDS rows are padded to 144 B so that the 16-byte operand reads of 16 consecutive rows hit
+// distinct banks.
+#define GB_K  64
+#define GB_LD (GB_K + 8)
 
-    const int64_t m0 = (int64_t) blockIdx.x * GB_M;
-    const int64_t n0 = (int64_t) blockIdx.y * GB_N;
-    const int64_t b2 = blockIdx.z % a.ne12, b3 = blockIdx.z / a.ne12;
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+template <int TI, int TJ, int S, bool KTAIL>     // KTAIL: K is not a multiple of 64 (but of 8)
+__global__ void __launch_bounds__(256) k_gemm_f16(mm_args a, int tiles_m, int tiles_n) {
+    constexpr int BN = 64 * TI, BM = 64 * TJ;
+    constexpr int XR = BN / 32, WR = BM / 32;          // 16-byte pieces per thread and step
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    half_t * xs_base = (half_t *) smem;                // [2][BN * GB_LD]
+    half_t * ws_base = xs_base + 2 * BN * GB_LD;       // [2][BM * GB_LD]
+
+    // Workgroups are dealt round-robin to the 8 XCDs, each with its own L2.  Give every XCD one contiguous run of
+    // tiles (m fastest), so that the X rows and the W rows it touches are shared inside that L2.
+    const int nblk = tiles_m * tiles_n;
+    const int xcd = blockIdx.x % 8, q = nblk / 8, r = nblk % 8;
+    const int tile = xcd * q + (xcd < r ? xcd : r) + blockIdx.x / 8;
+    const int64_t m0 = (int64_t)(tile % tiles_m) * BM;
+    const int64_t n0 = (int64_t)(tile / tiles_m) * BN;
+    const int64_t b2 = blockIdx.y % a.ne12, b3 = blockIdx.y / a.ne12;
 
     const char * wb = a.w + (b2 / a.r2) * a.w_nb2 + (b3 / a.r3) * a.w_nb3;
     const char * xb = a.x + b2 * a.x_nb2 + b3 * a.x_nb3;
     char *       db = a.d + b2 * a.d_nb2 + b3 * a.d_nb3;
 
-    const int64_t wm     = m0 + (threadIdx.x >> 1);
-    const bool    w_ok   = wm < a.M;
-    const char *  wrow   = wb + (w_ok ? wm : 0) * a.w_nb1;
+    const int tid = threadIdx.x;
+    const int lc = tid & 7, lr = tid >> 3;             // piece column (8 halves) and first row of this thread
+    // rows beyond N / M are read from the last valid row: what they produce is never stored
+    const char * xp[XR]; const char * wp[WR];
+#pragma unroll
+    for (int i = 0; i < XR; ++i) { const int64_t n = n0 + lr + 32 * i; xp[i] = xb + (n < a.N ? n : a.N - 1) * a.x_nb1 + lc * 16; }
+#pragma unroll
+    for (int i = 0; i < WR; ++i) { const int64_t m = m0 + lr + 32 * i; wp[i] = wb + (m < a.M ? m : a.M - 1) * a.w_nb1 + lc * 16; }
 
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int wn = (wave >> 1) * 64, wmo = (wave & 1) * 64;   // wave patch origin inside the tile
+    // S steps of operands are in flight in registers (slot = step % S)
+    u32x4 xrs[S][XR], wrs[S][WR];
+    auto load = [&](u32x4 (&xr)[XR], u32x4 (&wr)[WR], int64_t k0) __attribute__((always_inline)) {
+        if (KTAIL) {                                   // pieces beyond K are read from k = 0 and zeroed
+            const bool kok = k0 + 8 * lc < a.K;
+            const int64_t ko = kok ? k0 * 2 : -(int64_t) lc * 16;
+#pragma unroll
+            for (int i = 0; i < XR; ++i) { const u32x4 v = *(const u32x4 *)(xp[i] + ko); xr[i] = kok ? v : (u32x4){0, 0, 0, 0}; }
+#pragma unroll
+            for (int i = 0; i < WR; ++i) { const u32x4 v = *(const u32x4 *)(wp[i] + ko); wr[i] = kok ? v : (u32x4){0, 0, 0, 0}; }
+        } else {
+#pragma unroll
+            for (int i = 0; i < XR; ++i) xr[i] = *(const u32x4 *)(xp[i] + k0 * 2);
+#pragma unroll
+            for (int i = 0; i < WR; ++i) wr[i] = *(const u32x4 *)(wp[i] + k0 * 2);
+        }
+    };
+    auto store = [&](const u32x4 (&xr)[XR], const u32x4 (&wr)[WR], int buf) __attribute__((always_inline)) {
+        half_t * xs = xs_base + buf * BN * GB_LD, * ws = ws_base + buf * BM * GB_LD;
+#pragma unroll
+        for (int i = 0; i < XR; ++i) *(u32x4 *)(xs + (lr + 32 * i) * GB_LD + 8 * lc) = xr[i];
+#pragma unroll
+        for (int i = 0; i < WR; ++i) *(u32x4 *)(ws + (lr + 32 * i) * GB_LD + 8 * lc) = wr[i];
+    };
+
+    const int lane = tid & 63, wave = tid >> 6;
+    const int wn = (wave >> 1) * 32 * TI, wmo = (wave & 1) * 32 * TJ;   // wave patch origin inside the tile
     const int l32 = lane & 31, g = lane >> 5;
 
-    float16_t acc[2][2];
+    float16_t acc[TI][TJ];
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < TI; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
+        for (int j = 0; j < TJ; ++j)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+            for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
 
-    w_frag<T0> wf;
-    x_frag<T1> xf;
-    load_w<T0>(wf, wrow, w_ok, 0, a.K);
-    load_x<T1>(xf, xb, a.x_nb1, n0, a.N, 0, a.K);
-
-    for (int64_t k0 = 0; k0 < a.K; k0 += GB_K) {
-        store_w<T0>(wf, ws);
-        store_x<T1>(xf, xs);
-        __syncthreads();
-        if (k0 + GB_K < a.K) {
-            load_w<T0>(wf, wrow, w_ok, k0 + GB_K, a.K);
-            load_x<T1>(xf, xb, a.x_nb1, n0, a.N, k0 + GB_K, a.K);
-        }
-#pragma unroll
-        for (int kk = 0; kk < GB_K / 16; ++kk) {
-            half8_t av[2], bv[2];
-#pragma unroll
-            for (int i = 0; i < 2; ++i) av[i] = *(const half8_t *)(xs + (wn  + 32 * i + l32) * GB_LD + kk * 16 + 8 * g);
-#pragma unroll
-            for (int j = 0; j < 2; ++j) bv[j] = *(const half8_t *)(ws + (wmo + 32 * j + l32) * GB_LD + kk * 16 + 8 * g);
-#pragma unroll
-            for (int i = 0; i < 2; ++i)
-#pragma unroll
-                for (int j = 0; j < 2; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(av[i], bv[j], acc[i][j], 0, 0, 0);
-        }
-        __syncthreads();
-    }
-
-    // accumulator register r of a 32x32 patch: row (= n) 8*(r/4) + 4*g + r%4, column (= m) lane%32
-    const bool out_f16 = a.e.flags & MI355X_EPI_OUT_F16;
-#pragma unroll
-    for (int i = 0; i < 2; ++i) {
-#pragma unroll
-        for (int j = 0; j < 2; ++j) {
-            const int64_t m = m0 + wmo + 32 * j + l32;
-            if (m >= a.M) continue;
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int64_t n = n0 + wn + 32 * i + 8 * (r >> 2) + 4 * g + (r & 3);
-                if (n >= a.N) continue;
-                const int64_t res_off = (b2 * a.d_nb2 + b3 * a.d_nb3) + n * a.d_nb1 + m * 4;
-                const float v = apply_epilogue(acc[i][j][r], a.e, m, n, res_off);
-                if (out_f16) *(half_t *)(db + n * a.d_nb1 + m * 2) = (half_t) v;
-                else         *(float  *)(db + n * a.d_nb1 + m * 4) = v;
-            }
-        }
-    }
-}
-
-// ------------------------------------------------------------------------------------------------------
-// Quantized-weight GEMM on the int8 matrix cores.
-//
-// ggml's MUL_MAT with Q5_0 / Q8_0 weights is, by definition of the CPU backend, an integer computation
-// (ggml-cpu.c:1328-1363 converts src1 to Q8_0 with quantize_row_q8_0; ggml_vec_dot_q5_0_q8_0 / ggml_vec_dot_q8_0_q8_0,
-// ggml-cpu-quants.c:2930, 3597, then form per 32-value block the exact integer dot product of the quants and add
-// it, times d_w * d_x, to an f32 sum).  The kernel does exactly that: one pass quantizes src1 (k_quantize_act), then
-// each 32x32 accumulator patch takes one v_mfma_i32_32x32x32_i8 per block — K = 32 is one quant block — and the
-// exact i32 block sums are folded into f32 accumulators with the outer product of the block scales.
-//
-// Tile 128 (src1 rows) x 128 (weight rows) x 64 (two blocks), 4 wavefronts as 2 x 2, LDS double-buffered: the
-// global loads of step s+2 and the nibble unpacking / LDS stores of step s+1 are issued in the same basic block as
-// the MFMAs and scale FMAs of step s.
-// ------------------------------------------------------------------------------------------------------
-
-typedef int v4i_t  __attribute__((ext_vector_type(4)));
-typedef int v16i_t __attribute__((ext_vector_type(16)));
-
-static inline size_t round256(size_t n) { return (n + 255) / 256 * 256; }
-
-// workspace of one batch slice: int8 quants [N][K], then f32 block scales [K/32][N]
-__global__ void k_quantize_act(const char * __restrict__ x, char * __restrict__ ws, int64_t K, int64_t N,
-                               int64_t x_nb1, int64_t x_nb2, int64_t ne12, int64_t x_nb3, int64_t slice_bytes, int64_t xd_off) {
-    const int64_t t  = (int64_t) blockIdx.x * blockDim.x + threadIdx.x;     // 8 lanes per block of 32 values, 4 values each
-    const int64_t k4 = K / 4;
-    const int64_t b  = blockIdx.y;
-    if (t >= k4 * N) return;                                                // whole 8-lane groups leave together
-    const int64_t n = t / k4, c = t % k4;
-    const float4 v = *(const float4 *)(x + n * x_nb1 + (b % ne12) * x_nb2 + (b / ne12) * x_nb3 + c * 16);
-    float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
-    amax = fmaxf(amax, __shfl_xor(amax, 1, 8));
-    amax = fmaxf(amax, __shfl_xor(amax, 2, 8));
-    amax = fmaxf(amax, __shfl_xor(amax, 4, 8));
-    const float id = amax != 0.0f ? 127.0f / amax : 0.0f;
-    const int q0 = (int) rintf(v.x * id), q1 = (int) rintf(v.y * id), q2 = (int) rintf(v.z * id), q3 = (int) rintf(v.w * id);
-    char * slice = ws + b * slice_bytes;
-    *(int32_t *)(slice + n * K + c * 4) = (q0 & 0xFF) | ((q1 & 0xFF) << 8) | ((q2 & 0xFF) << 16) | ((q3 & 0xFF) << 24);
-    if ((c & 7) == 0) ((float *)(slice + xd_off))[(c / 8) * N + n] = h2f(f2h_bits(amax / 127.0f));   // the scale goes through f16, like block_q8_0.d
-}
-
-#define I8_N   128
-#define I8_M   128
-#define I8_K   64            // two quant blocks per step
-#define I8_LD  80            // byte pitch of the quant tiles: 64 + 16, so that 8 consecutive rows start 4 banks apart
-
-struct i8_args {
-    mm_args m;               // x = workspace quants of this launch, x_nb* describe them; w / d as usual
-    const char * xd;         // block scales [K/32][N] of batch slice 0
-    int64_t xd_slice;        // bytes between batch slices
-};
-
-template <int T0> struct wq_frag;
-template <> struct wq_frag<MI355X_TYPE_Q5_0> { uint32_t d, qh, qs[4]; };
-template <> struct wq_frag<MI355X_TYPE_Q8_0> { uint32_t d, qs[8]; };
-
-template <int T0>
-__device__ __forceinline__ void i8_load_w(wq_frag<T0> & f, const char * wrow, bool row_ok, int64_t k0, int64_t K) {
-    const int64_t k = k0 + (threadIdx.x & 1) * 32;
-    if constexpr (T0 == MI355X_TYPE_Q5_0) {
-        if (row_ok && k < K) {
-            const uint8_t * b = (const uint8_t *) wrow + (k / QK) * 22;
-            f.d  = *(const uint16_t *) b;
-            f.qh = *(const u32a2 *)(b + 2);
-            const u128a2 q = *(const u128a2 *)(b + 6);
-            f.qs[0] = q.x; f.qs[1] = q.y; f.qs[2] = q.z; f.qs[3] = q.w;
-        } else { f.d = 0; f.qh = 0; f.qs[0] = f.qs[1] = f.qs[2] = f.qs[3] = 0; }
-    } else {
-        if (row_ok && k < K) {
-            const uint8_t * b = (const uint8_t *) wrow + (k / QK) * 34;
-            f.d = *(const uint16_t *) b;
-            const u128a2 q0 = *(const u128a2 *)(b + 2), q1 = *(const u128a2 *)(b + 18);
-            f.qs[0] = q0.x; f.qs[1] = q0.y; f.qs[2] = q0.z; f.qs[3] = q0.w;
-            f.qs[4] = q1.x; f.qs[5] = q1.y; f.qs[6] = q1.z; f.qs[7] = q1.w;
-        } else {
-            f.d = 0;
-#pragma unroll
-            for (int i = 0; i < 8; ++i) f.qs[i] = 0;
-        }
-    }
-}
-
-// block -> 32 signed bytes in weight order, plus the f32 scale
-template <int T0>
-__device__ __forceinline__ void i8_store_w(const wq_frag<T0> & f, char * wq_s, float * wd_s) {
-    const int row = threadIdx.x >> 1, blk = threadIdx.x & 1;
-    uint32_t o[8];
-    if constexpr (T0 == MI355X_TYPE_Q5_0) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            // q - 16 as a signed byte: the nibble, with 0xF0 on top where the fifth bit is clear
-            const uint32_t lo_h = ((~(f.qh >> (4*i))      & 0xFu) * 0x00204081u) & 0x01010101u;
-            const uint32_t hi_h = ((~(f.qh >> (16 + 4*i)) & 0xFu) * 0x00204081u) & 0x01010101u;
-            o[i]     = (f.qs[i] & 0x0F0F0F0Fu)        | (lo_h * 0xF0u);
-            o[4 + i] = ((f.qs[i] >> 4) & 0x0F0F0F0Fu) | (hi_h * 0xF0u);
-        }
-    } else {
-#pragma unroll
-        for (int i = 0; i < 8; ++i) o[i] = f.qs[i];
-    }
-    uint4 * p = (uint4 *)(wq_s + row * I8_LD + blk * 32);
-    p[0] = make_uint4(o[0], o[1], o[2], o[3]);
-    p[1] = make_uint4(o[4], o[5], o[6], o[7]);
-    wd_s[blk * I8_M + row] = h2f((uint16_t) f.d);
-}
-
-struct xq_frag { uint32_t q[8]; float d; };
-
-__device__ __forceinline__ void i8_load_x(xq_frag & f, const char * xq, const float * xd, int64_t n0, int64_t N, int64_t k0, int64_t K) {
-    const int row = threadIdx.x >> 1, half = threadIdx.x & 1;
-    const int64_t n = n0 + row, k = k0 + half * 32;
-    if (n < N && k < K) {
-        const uint4 * p = (const uint4 *)(xq + n * K + k);
-        const uint4 v0 = p[0], v1 = p[1];
-        f.q[0] = v0.x; f.q[1] = v0.y; f.q[2] = v0.z; f.q[3] = v0.w; f.q[4] = v1.x; f.q[5] = v1.y; f.q[6] = v1.z; f.q[7] = v1.w;
-    } else {
-#pragma unroll
-        for (int i = 0; i < 8; ++i) f.q[i] = 0;
-    }
-    // scales: thread t -> block t / 128 of this step, row t % 128
-    const int64_t sn = n0 + (threadIdx.x & 127), sk = k0 + (threadIdx.x >> 7) * 32;
-    f.d = (sn < N && sk < K) ? xd[(sk / QK) * N + sn] : 0.0f;
-}
-__device__ __forceinline__ void i8_store_x(const xq_frag & f, char * xq_s, float * xd_s) {
-    uint4 * p = (uint4 *)(xq_s + (threadIdx.x >> 1) * I8_LD + (threadIdx.x & 1) * 32);
-    p[0] = make_uint4(f.q[0], f.q[1], f.q[2], f.q[3]);
-    p[1] = make_uint4(f.q[4], f.q[5], f.q[6], f.q[7]);
-    xd_s[threadIdx.x] = f.d;               // [blk][row]
-}
-
-template <int T0>
-__global__ void __launch_bounds__(256, 2) k_gemm_i8(i8_args ia) {
-    const mm_args & a = ia.m;
-    __shared__ __attribute__((aligned(16))) char  xq_s[2][I8_N * I8_LD];
-    __shared__ __attribute__((aligned(16))) char  wq_s[2][I8_M * I8_LD];
-    __shared__ __attribute__((aligned(16))) float xd_s[2][2 * I8_N];
-    __shared__ __attribute__((aligned(16))) float wd_s[2][2 * I8_M];
-
-    const int64_t m0 = (int64_t) blockIdx.x * I8_M, n0 = (int64_t) blockIdx.y * I8_N;
-    const int64_t bz = blockIdx.z, b2 = bz % a.ne12, b3 = bz / a.ne12;
-    const char *  wb = a.w + (b2 / a.r2) * a.w_nb2 + (b3 / a.r3) * a.w_nb3;
-    const char *  xq = a.x + bz * a.x_nb2;
-    const float * xd = (const float *)(ia.xd + bz * ia.xd_slice);
-    char *        db = a.d + b2 * a.d_nb2 + b3 * a.d_nb3;
-
-    const int64_t wm   = m0 + (threadIdx.x >> 1);
-    const bool    w_ok = wm < a.M;
-    const char *  wrow = wb + (w_ok ? wm : 0) * a.w_nb1;
-
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int wn = (wave >> 1) * 64, wmo = (wave & 1) * 64, l32 = lane & 31, g = lane >> 5;
-
-    float16_t acc[2][2];
-#pragma unroll
-    for (int i = 0; i < 2; ++i)
-#pragma unroll
-        for (int j = 0; j < 2; ++j)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
-
-    wq_frag<T0> wf;
-    xq_frag     xf;
-    i8_load_w<T0>(wf, wrow, w_ok, 0, a.K);
-    i8_load_x(xf, xq, xd, n0, a.N, 0, a.K);
-    i8_store_w<T0>(wf, wq_s[0], wd_s[0]);
-    i8_store_x(xf, xq_s[0], xd_s[0]);
-    if (I8_K < a.K) { i8_load_w<T0>(wf, wrow, w_ok, I8_K, a.K); i8_load_x(xf, xq, xd, n0, a.N, I8_K, a.K); }
+    const int KT = (int)((a.K + GB_K - 1) / GB_K);
+    load(xrs[0], wrs[0], 0);
+    if (1 < KT) load(xrs[1], wrs[1], GB_K);
+    if (S > 2) { if (2 < KT) load(xrs[2 % S], wrs[2 % S], 2 * GB_K); if (3 < KT) load(xrs[3 % S], wrs[3 % S], 3 * GB_K); }
+    if (S > 4) { if (4 < KT) load(xrs[4 % S], wrs[4 % S], 4 * GB_K); if (5 < KT) load(xrs[5 % S], wrs[5 % S], 5 * GB_K); }
+    store(xrs[0], wrs[0], 0);
+    if (S < KT) load(xrs[0], wrs[0], (int64_t) S * GB_K);
     __syncthreads();
 
-    int buf = 0;
-    for (int64_t k0 = 0; k0 < a.K; k0 += I8_K, buf ^= 1) {
-        if (k0 + I8_K < a.K) {                      // stage s+1 goes to the other buffer (its last readers passed the barrier)
-            i8_store_w<T0>(wf, wq_s[buf ^ 1], wd_s[buf ^ 1]);
-            i8_store_x(xf, xq_s[buf ^ 1], xd_s[buf ^ 1]);
+    auto step = [&](int kt, int buf, u32x4 (&xr)[XR], u32x4 (&wr)[WR]) __attribute__((always_inline)) {   // xr / wr: slot of step kt + 1
+        const half_t * xs = xs_base + buf * BN * GB_LD + (wn  + l32) * GB_LD + 8 * g;
+        const half_t * ws = ws_base + buf * BM * GB_LD + (wmo + l32) * GB_LD + 8 * g;
+#pragma unroll
+        for (int kk = 0; kk < GB_K / 16; ++kk) {
+            half8_t av[TI], bv[TJ];
+#pragma unroll
+            for (int i = 0; i < TI; ++i) av[i] = *(const half8_t *)(xs + 32 * i * GB_LD + kk * 16);
+#pragma unroll
+            for (int j = 0; j < TJ; ++j) bv[j] = *(const half8_t *)(ws + 32 * j * GB_LD + kk * 16);
+#pragma unroll
+            for (int i = 0; i < TI; ++i)
+#pragma unroll
+                for (int j = 0; j < TJ; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(av[i], bv[j], acc[i][j], 0, 0, 0);
         }
-        if (k0 + 2 * I8_K < a.K) { i8_load_w<T0>(wf, wrow, w_ok, k0 + 2 * I8_K, a.K); i8_load_x(xf, xq, xd, n0, a.N, k0 + 2 * I8_K, a.K); }
-
-        const char *  xs = xq_s[buf]; const char * ws = wq_s[buf];
-        const float * xds = xd_s[buf]; const float * wds = wd_s[buf];
-#pragma unroll
-        for (int blk = 0; blk < 2; ++blk) {
-            v4i_t av[2], bv[2];
-            float dw[2];
-            float4 dx[2][4];
-#pragma unroll
-            for (int i = 0; i < 2; ++i) {
-                av[i] = *(const v4i_t *)(xs + (wn + 32 * i + l32) * I8_LD + blk * 32 + 16 * g);
-#pragma unroll
-                for (int q = 0; q < 4; ++q) dx[i][q] = *(const float4 *)(xds + blk * I8_N + wn + 32 * i + 8 * q + 4 * g);
-            }
-#pragma unroll
-            for (int j = 0; j < 2; ++j) {
-                bv[j] = *(const v4i_t *)(ws + (wmo + 32 * j + l32) * I8_LD + blk * 32 + 16 * g);
-                dw[j] = wds[blk * I8_M + wmo + 32 * j + l32];
-            }
-#pragma unroll
-            for (int i = 0; i < 2; ++i)
-#pragma unroll
-                for (int j = 0; j < 2; ++j) {
-                    v16i_t c;
-#pragma unroll
-                    for (int r = 0; r < 16; ++r) c[r] = 0;
-                    c = __builtin_amdgcn_mfma_i32_32x32x32_i8(av[i], bv[j], c, 0, 0, 0);
-#pragma unroll
-                    for (int q = 0; q < 4; ++q) {
-                        acc[i][j][4*q + 0] += (float) c[4*q + 0] * (dx[i][q].x * dw[j]);
-                        acc[i][j][4*q + 1] += (float) c[4*q + 1] * (dx[i][q].y * dw[j]);
-                        acc[i][j][4*q + 2] += (float) c[4*q + 2] * (dx[i][q].z * dw[j]);
-                        acc[i][j][4*q + 3] += (float) c[4*q + 3] * (dx[i][q].w * dw[j]);
-                    }
-                }
+        if (kt + 1 < KT) {
+            store(xr, wr, buf ^ 1);                     // the last readers of that buffer passed the previous barrier
+            if (kt + 1 + S < KT) load(xr, wr, (int64_t)(kt + 1 + S) * GB_K);
         }
         __syncthreads();
-    }
-
-    const bool out_f16 = a.e.flags & MI355X_EPI_OUT_F16;
-#pragma unroll
-    for (int i = 0; i < 2; ++i) {
-#pragma unroll
-        for (int j = 0; j < 2; ++j) {
-            const int64_t m = m0 + wmo + 32 * j + l32;
-            if (m >= a.M) continue;
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int64_t n = n0 + wn + 32 * i + 8 * (r >> 2) + 4 * g + (r & 3);
-                if (n >= a.N) continue;
-                const int64_t res_off = (b2 * a.d_nb2 + b3 * a.d_nb3) + n * a.d_nb1 + m * 4;
-                const float v = apply_epilogue(acc[i][j][r], a.e, m, n, res_off);
-                if (out_f16) *(half_t *)(db + n * a.d_nb1 + m * 2) = (half_t) v;
-                else         *(float  *)(db + n * a.d_nb1 + m * 4) = v;
-            }
+    };
+    for (int kt0 = 0; kt0 < KT; kt0 += S) {             // S is even: the LDS buffer of a step is the parity of its slot
+        if (kt0 + 0 < KT) step(kt0 + 0, 0, xrs[1 % S], wrs[1 % S]);
+        if (kt0 + 1 < KT) step(kt0 + 1, 1, xrs[2 % S], wrs[2 % S]);
+        if (S > 2) {
+            if (kt0 + 2 < KT) step(kt0 + 2, 0, xrs[3 % S], wrs[3 % S]);
+            if (kt0 + 3 < KT) step(kt0 + 3, 1, xrs[4 % S], wrs[4 % S]);
+        }
+        if (S > 4) {
+            if (kt0 + 4 < KT) step(kt0 + 4, 0, xrs[5 % S], wrs[5 % S]);
+            if (kt0 + 5 < KT) step(kt0 + 5, 1, xrs[6 % S], wrs[6 % S]);
         }
     }
+
+    // accumulator register e of a 32x32 patch: row (= n) 8*(e/4) + 4*g + e%4, column (= m) lane%32
+    const int64_t batch_off = b2 * a.d_nb2 + b3 * a.d_nb3;
+#pragma unroll
+    for (int i = 0; i < TI; ++i) {
+        int64_t n[16];
+#pragma unroll
+        for (int e = 0; e < 16; ++e) n[e] = n0 + wn + 32 * i + 8 * (e >> 2) + 4 * g + (e & 3);
+#pragma unroll
+        for (int j = 0; j < TJ; ++j)
+            patch_epilogue(acc[i][j], a.e, db, batch_off, a.d_nb1, m0 + wmo + 32 * j + l32, a.M, n, a.N);
+    }
+}
+
+template <int TI, int TJ, int S, bool KTAIL>
+static int launch_gemm_f16_k(const mm_args & a, hipStream_t st) {
+    static_assert(S % 2 == 0, "the LDS buffer index is the parity of the register slot");
+    constexpr int BN = 64 * TI, BM = 64 * TJ;
+    constexpr size_t lds = (size_t) 2 * (BN + BM) * GB_LD * sizeof(half_t);
+    static bool configured[64];                         // per device: kernels may use more than the default 64 KB of LDS
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return MI355X_ERR_HIP;
+    if (!configured[dev]) {
+        if (hipFuncSetAttribute((const void *) k_gemm_f16<TI, TJ, S, KTAIL>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds) != hipSuccess) return MI355X_ERR_HIP;
+        configured[dev] = true;
+    }
+    const int64_t tm = (a.M + BM - 1) / BM, tn = (a.N + BN - 1) / BN;
+    if (tm * tn > 0x7fffffff) return MI355X_ERR_UNSUPPORTED;
+    dim3 grid((unsigned)(tm * tn), (unsigned)(a.ne12 * a.ne13));
+    k_gemm_f16<TI, TJ, S, KTAIL><<<grid, 256, lds, st>>>(a, (int) tm, (int) tn);
+    return launch_status();
+}
+static int g_stages = -1;
+template <int TI, int TJ>
+static int launch_gemm_f16(const mm_args & a, hipStream_t st) {
+    if (g_stages < 0) { const char * e = getenv("MI355X_GEMM_STAGES"); g_stages = e ? atoi(e) : 4; }
+    if (a.K % GB_K) return launch_gemm_f16_k<TI, TJ, 2, true>(a, st);
+    switch (g_stages) {
+        case 2:  return launch_gemm_f16_k<TI, TJ, 2, false>(a, st);
+        case 6:  return launch_gemm_f16_k<TI, TJ, 6, false>(a, st);
+        default: return launch_gemm_f16_k<TI, TJ, 4, false>(a, st);
+    }
+}
+
+// tile shape: the largest whose grid still covers the 256 CUs about twice
+static int launch_gemm_f16_auto(const mm_args & a, hipStream_t st) {
+    const int64_t nb = a.ne12 * a.ne13;
+    auto blocks = [&](int bn, int bm) { return ((a.N + bn - 1) / bn) * ((a.M + bm - 1) / bm) * nb; };
+    if (blocks(128, 128) >= 384) return launch_gemm_f16<2, 2>(a, st);
+    if (blocks(128, 64)  >= 192 || a.N > 64) return launch_gemm_f16<2, 1>(a, st);
+    return launch_gemm_f16<1, 1>(a, st);
 }
 
 // ------------------------------------------------------------------------------------------------------
@@ -603,6 +464,23 @@ __global__ void __launch_bounds__(256) k_gemv_q(mm_args a) {
 #pragma unroll
     for (int n = 0; n < NC; ++n) acc[n] = 0.0f;
 
+    // the epilogue operands of the lane that will store are fetched now, under the weight stream
+    const bool writer = row_ok && j == 0;
+    float e_bias = 0.0f, e_bcol[NC], e_res[NC];
+#pragma unroll
+    for (int n = 0; n < NC; ++n) { e_bcol[n] = 0.0f; e_res[n] = 0.0f; }
+    if (writer) {
+        if (a.e.flags & MI355X_EPI_BIAS) e_bias = a.e.bias[row];
+        if (a.e.flags & MI355X_EPI_BIAS_COL) {
+#pragma unroll
+            for (int n = 0; n < NC; ++n) e_bcol[n] = a.e.bias[n];
+        }
+        if (a.e.flags & MI355X_EPI_RESIDUAL) {
+#pragma unroll
+            for (int n = 0; n < NC; ++n) e_res[n] = *(const float *)(a.e.residual + n * a.d_nb1 + row * 4);
+        }
+    }
+
     if (row_ok) {
         for (int kb = j; kb < nbk; kb += LPR) {
             uint32_t q[8];
@@ -649,11 +527,14 @@ __global__ void __launch_bounds__(256) k_gemv_q(mm_args a) {
 #pragma unroll
         for (int o = LPR / 2; o > 0; o >>= 1) acc[n] += __shfl_xor(acc[n], o, LPR);
     }
-    if (row_ok && j == 0) {
+    if (writer) {
         const bool out_f16 = a.e.flags & MI355X_EPI_OUT_F16;
 #pragma unroll
         for (int n = 0; n < NC; ++n) {
-            const float v = apply_epilogue(acc[n], a.e, row, n, n * a.d_nb1 + row * 4);
+            float v = acc[n] + e_bias + e_bcol[n];          // at most one of the two biases is set
+            if (a.e.flags & MI355X_EPI_GELU)     v  = gelu_f32(v, a.e.gelu);
+            if (a.e.flags & MI355X_EPI_SCALE)    v *= a.e.scale;
+            if (a.e.flags & MI355X_EPI_RESIDUAL) v += e_res[n];
             if (out_f16) *(half_t *)(a.d + n * a.d_nb1 + row * 2) = (half_t) v;
             else         *(float  *)(a.d + n * a.d_nb1 + row * 4) = v;
         }
@@ -775,12 +656,11 @@ static int mm_path(const mi355x_tensor * src0, const mi355x_tensor * src1) {
         return MM_GEMV;
     }
     bool fast = N > MI355X_GEMV_MAX_COLS || !quant;
-    if (N <= 2) fast = false;                         // a 128-wide tile for one or two columns is mostly padding
-    if (t1 == MI355X_TYPE_F32) fast = fast && aligned16(src1) && K % 4 == 0;
-    else                       fast = fast && aligned16(src1) && K % 8 == 0 && t0 == MI355X_TYPE_F16;
-    if (t0 == MI355X_TYPE_F16) fast = fast && aligned16(src0) && K % 8 == 0;
-    if (t0 == MI355X_TYPE_F32) fast = fast && aligned16(src0) && K % 4 == 0;
+    if (N <= 2) fast = false;                         // a 64-wide tile for one or two columns is mostly padding
+    fast = fast && aligned16(src1) && K % 8 == 0;
     if (quant)                 fast = fast && w_al2;
+    else if (t0 == MI355X_TYPE_F16) fast = fast && aligned16(src0);
+    else                       fast = fast && aligned16(src0) && K % QK == 0;
     return fast ? MM_GEMM : MM_GENERIC;
 }
 
@@ -795,12 +675,29 @@ extern "C" const char * mi355x_mul_mat_kernel_name(const mi355x_tensor * src0, c
     }
 }
 
-// the GEMM with quantized weights quantizes src1 into `workspace`: per batch slice int8 [N][K], then f32 scales [K/32][N]
+// workspace of the GEMM path: f16 image of src1 (when src1 is F32), then f16 image of src0 (when src0 is not F16), each
+// batch slice rounded up to 256 bytes
+static size_t x16_bytes(const mi355x_tensor * src1) {
+    return src1->type == MI355X_TYPE_F32 ? round256((size_t) src1->ne[0] * src1->ne[1] * 2) * (size_t)(src1->ne[2] * src1->ne[3]) : 0;
+}
+static size_t w16_bytes(const mi355x_tensor * src0) {
+    return src0->type != MI355X_TYPE_F16 ? round256((size_t) src0->ne[0] * src0->ne[1] * 2) * (size_t)(src0->ne[2] * src0->ne[3]) : 0;
+}
 extern "C" size_t mi355x_mul_mat_workspace_size(const mi355x_tensor * src0, const mi355x_tensor * src1) {
-    if (!src0 || !src1) return 0;
-    if (blck_size(src0->type) == 1 || src1->type != MI355X_TYPE_F32 || mm_path(src0, src1) != MM_GEMM) return 0;
-    const size_t K = (size_t) src1->ne[0], N = (size_t) src1->ne[1];
-    return (round256(N * K) + round256(K / QK * N * 4)) * (size_t)(src1->ne[2] * src1->ne[3]);
+    if (!src0 || !src1 || mm_path(src0, src1) != MM_GEMM) return 0;
+    return x16_bytes(src1) + w16_bytes(src0);
+}
+
+extern "C" int mi355x_dequantize_row_f16(int type, const void * src, void * dst, int64_t k, void * stream) {
+    if (!src || !dst || k < 0 || k % QK != 0 || (uintptr_t) src % 2 != 0 || (uintptr_t) dst % 16 != 0) return MI355X_ERR_INVALID;
+    if (k == 0) return MI355X_OK;
+    if (k / QK > 0x7fffffff * (int64_t) 256) return MI355X_ERR_UNSUPPORTED;
+    hipStream_t st = (hipStream_t) stream;
+    const unsigned grid = (unsigned)((k / QK + 255) / 256);
+    if      (type == MI355X_TYPE_Q5_0) k_w_to_f16<MI355X_TYPE_Q5_0><<<grid, 256, 0, st>>>((const char *) src, (half_t *) dst, k, 1, 0, 0, 1, 0, 0);
+    else if (type == MI355X_TYPE_Q8_0) k_w_to_f16<MI355X_TYPE_Q8_0><<<grid, 256, 0, st>>>((const char *) src, (half_t *) dst, k, 1, 0, 0, 1, 0, 0);
+    else return MI355X_ERR_UNSUPPORTED;
+    return launch_status();
 }
 
 extern "C" int mi355x_mul_mat(const mi355x_tensor * src0, const mi355x_tensor * src1, const mi355x_tensor * dst,
@@ -821,6 +718,7 @@ extern "C" int mi355x_mul_mat(const mi355x_tensor * src0, const mi355x_tensor * 
     if (src0->nb[0] != type_size(t0) || src1->nb[0] != type_size(t1) || dst->nb[0] != type_size(td)) return MI355X_ERR_UNSUPPORTED;
     if (blck_size(t0) > 1 && a.K % QK != 0) return MI355X_ERR_INVALID;
     if ((flags & (MI355X_EPI_BIAS | MI355X_EPI_BIAS_COL)) && !epi->bias) return MI355X_ERR_INVALID;
+    if ((flags & MI355X_EPI_BIAS) && (flags & MI355X_EPI_BIAS_COL)) return MI355X_ERR_INVALID;      // there is one bias pointer
     if ((flags & MI355X_EPI_RESIDUAL) && !epi->residual) return MI355X_ERR_INVALID;
     if ((flags & MI355X_EPI_RESIDUAL) && (flags & MI355X_EPI_OUT_F16)) return MI355X_ERR_UNSUPPORTED;
     if (a.M == 0 || a.N == 0 || dst->ne[2] * dst->ne[3] == 0) return MI355X_OK;
@@ -847,35 +745,32 @@ extern "C" int mi355x_mul_mat(const mi355x_tensor * src0, const mi355x_tensor * 
         return t0 == MI355X_TYPE_Q8_0 ? launch_gemv_n<MI355X_TYPE_Q8_0>(a, st) : launch_gemv_n<MI355X_TYPE_Q5_0>(a, st);
     }
     if (path == MM_GEMM) {
-        dim3 grid((unsigned)((a.M + GB_M - 1) / GB_M), (unsigned)((a.N + GB_N - 1) / GB_N), (unsigned) nbatch);
-        if (grid.y > 65535) return MI355X_ERR_UNSUPPORTED;
-        if (quant && t1 == MI355X_TYPE_F32 && !(flags & MI355X_MM_EXACT_ACT)) {
-            const size_t need = mi355x_mul_mat_workspace_size(src0, src1);
-            if (!workspace || workspace_size < need || (uintptr_t) workspace % 256 != 0) return MI355X_ERR_WORKSPACE;
-            const int64_t xd_off = (int64_t) round256((size_t)(a.N * a.K));
-            const int64_t slice  = xd_off + (int64_t) round256((size_t)(a.K / QK * a.N * 4));
+        const size_t xbytes = x16_bytes(src1), wbytes = w16_bytes(src0);
+        if (xbytes + wbytes > 0 && (!workspace || workspace_size < xbytes + wbytes || (uintptr_t) workspace % 256 != 0)) return MI355X_ERR_WORKSPACE;
+        mm_args g = a;
+        if (xbytes) {
+            const int64_t slice = (int64_t) round256((size_t)(a.N * a.K * 2));
             if (!(flags & MI355X_MM_WS_READY)) {
-                const int64_t threads = a.K / 4 * a.N;
-                dim3 qgrid((unsigned)((threads + 255) / 256), (unsigned) nbatch);
-                k_quantize_act<<<qgrid, 256, 0, st>>>(a.x, (char *) workspace, a.K, a.N, a.x_nb1, a.x_nb2, a.ne12, a.x_nb3, slice, xd_off);
+                dim3 qgrid((unsigned)((a.K / 4 * a.N + 255) / 256), (unsigned) nbatch);
+                const bool q8 = (quant || (flags & MI355X_MM_ACT_Q8_0)) && !(flags & MI355X_MM_EXACT_ACT);
+                if (q8 && a.K % QK != 0) return MI355X_ERR_INVALID;
+                if (q8) k_x_to_f16<true ><<<qgrid, 256, 0, st>>>(a.x, (half_t *) workspace, a.K, a.N, a.x_nb1, a.x_nb2, a.ne12, a.x_nb3, slice / 2);
+                else    k_x_to_f16<false><<<qgrid, 256, 0, st>>>(a.x, (half_t *) workspace, a.K, a.N, a.x_nb1, a.x_nb2, a.ne12, a.x_nb3, slice / 2);
             }
-            i8_args ia;
-            ia.m = a;
-            ia.m.x = (const char *) workspace; ia.m.x_nb1 = a.K; ia.m.x_nb2 = slice; ia.m.x_nb3 = slice * a.ne12;
-            ia.xd = (const char *) workspace + xd_off; ia.xd_slice = slice;
-            if (t0 == MI355X_TYPE_Q5_0) k_gemm_i8<MI355X_TYPE_Q5_0><<<grid, 256, 0, st>>>(ia);
-            else                        k_gemm_i8<MI355X_TYPE_Q8_0><<<grid, 256, 0, st>>>(ia);
-            return launch_status();
+            g.x = (const char *) workspace; g.x_nb1 = a.K * 2; g.x_nb2 = slice; g.x_nb3 = slice * a.ne12;
         }
-        if (t1 == MI355X_TYPE_F16) {
-            k_gemm_mfma<MI355X_TYPE_F16, MI355X_TYPE_F16><<<grid, 256, 0, st>>>(a);
-        } else switch (t0) {
-            case MI355X_TYPE_Q5_0: k_gemm_mfma<MI355X_TYPE_Q5_0, MI355X_TYPE_F32><<<grid, 256, 0, st>>>(a); break;
-            case MI355X_TYPE_Q8_0: k_gemm_mfma<MI355X_TYPE_Q8_0, MI355X_TYPE_F32><<<grid, 256, 0, st>>>(a); break;
-            case MI355X_TYPE_F16:  k_gemm_mfma<MI355X_TYPE_F16,  MI355X_TYPE_F32><<<grid, 256, 0, st>>>(a); break;
-            default:               k_gemm_mfma<MI355X_TYPE_F32,  MI355X_TYPE_F32><<<grid, 256, 0, st>>>(a); break;
+        if (wbytes) {
+            const int64_t slice = (int64_t) round256((size_t)(a.M * a.K * 2));
+            half_t * w16 = (half_t *)((char *) workspace + xbytes);
+            dim3 wgrid((unsigned)((a.K / QK * a.M + 255) / 256), (unsigned)(src0->ne[2] * src0->ne[3]));
+            switch (t0) {
+                case MI355X_TYPE_Q5_0: k_w_to_f16<MI355X_TYPE_Q5_0><<<wgrid, 256, 0, st>>>(a.w, w16, a.K, a.M, a.w_nb1, a.w_nb2, src0->ne[2], a.w_nb3, slice / 2); break;
+                case MI355X_TYPE_Q8_0: k_w_to_f16<MI355X_TYPE_Q8_0><<<wgrid, 256, 0, st>>>(a.w, w16, a.K, a.M, a.w_nb1, a.w_nb2, src0->ne[2], a.w_nb3, slice / 2); break;
+                default:               k_w_to_f16<MI355X_TYPE_F32 ><<<wgrid, 256, 0, st>>>(a.w, w16, a.K, a.M, a.w_nb1, a.w_nb2, src0->ne[2], a.w_nb3, slice / 2); break;
+            }
+            g.w = (const char *) w16; g.w_nb1 = a.K * 2; g.w_nb2 = slice; g.w_nb3 = slice * src0->ne[2];
         }
-        return launch_status();
+        return launch_gemm_f16_auto(g, st);
     }
 
     if (a.M > 0x7fffffff || (a.N + 7) / 8 > 65535) return MI355X_ERR_UNSUPPORTED;
