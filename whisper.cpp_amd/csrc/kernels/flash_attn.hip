@@ -21,6 +21,8 @@
 
 #define FA_D 64
 
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
 struct fa_args {
     const char * q; const char * k; const char * v; const char * mask; char * d;
     int64_t N, KV, H;
@@ -109,6 +111,27 @@ __global__ void __launch_bounds__(256) k_fattn_vec(fa_args a) {
 //   VKQ16 = f16(fma(f32(v), vs, f32(VKQ16)))  (ggml_vec_mad_f16: fma in f32, stored as f16)
 __device__ __forceinline__ half_t seq_scale(half_t acc, float ms) { return (half_t)((float) acc * ms); }
 __device__ __forceinline__ half_t seq_mad(half_t acc, half_t v, float vs) { return (half_t) __builtin_fmaf((float) v, vs, (float) acc); }
+
+// The same two steps on a pair of accumulators: two full-rate v_fma_mix_f32 (f16 and f32 sources, fma rounded to f32)
+// and one v_cvt_pk_f16_f32 (round to nearest even) per pair — the reference's f32 fma followed by GGML_FP32_TO_FP16,
+// both roundings included.  Spelled out as instructions because the compiler otherwise mixes in v_fma_mixlo/hi_f16,
+// which issue at half rate on gfx950 and round the exact fma once (a last-bit difference from the reference's two steps).
+__device__ __forceinline__ half2_t seq_mad2(half2_t acc, half2_t v, float vs) {
+    float lo, hi;
+    half2_t r;
+    asm("v_fma_mix_f32 %0, %2, %3, %4 op_sel_hi:[1,0,1]\n\t"
+        "v_fma_mix_f32 %1, %2, %3, %4 op_sel:[1,0,1] op_sel_hi:[1,0,1]" : "=&v"(lo), "=&v"(hi) : "v"(v), "v"(vs), "v"(acc));
+    asm("v_cvt_pk_f16_f32 %0, %1, %2" : "=v"(r) : "v"(lo), "v"(hi));
+    return r;
+}
+__device__ __forceinline__ half2_t seq_scale2(half2_t acc, float ms) {
+    float lo, hi;
+    half2_t r;
+    asm("v_fma_mix_f32 %0, %2, %3, 0 op_sel_hi:[1,0,0]\n\t"
+        "v_fma_mix_f32 %1, %2, %3, 0 op_sel:[1,0,0] op_sel_hi:[1,0,0]" : "=&v"(lo), "=&v"(hi) : "v"(acc), "v"(ms));
+    asm("v_cvt_pk_f16_f32 %0, %1, %2" : "=v"(r) : "v"(lo), "v"(hi));
+    return r;
+}
 
 // softmax factors of a run of scores that continues a running maximum M:  s[i] -> vs[i], ms[i]; also the run's
 // contribution to the softmax denominator as (P, A): S_after = S_before * P + A
@@ -249,22 +272,42 @@ __global__ void __launch_bounds__(256) k_fattn_seq_row(fa_args a, int kv_pad) {
 
 // ------------------------------------------------------------------------------------------------------
 // k_fattn_seq_tile: 64 queries per block, 64 keys per step
+//
+// Per step: (1) K tile -> LDS, S = Q K^T on the matrix cores, scores -> LDS; (2) thread (query, 16-key run) turns the
+// scores into one factor per (query, key): f = vs = exp(s - M_k) when the running maximum stands, f = -ms =
+// -exp(M_{k-1} - M_k) when key k raises it (then vs is exactly 1); (3) the chains: lane = query, wavefront = 16 of the
+// 64 d.  All lanes of a wavefront then want the same 16 V values per key: two broadcast LDS reads; the factors come
+// four keys per LDS read.  Per key and lane that leaves the 16 fma + 8 pack instructions the reference's rounding
+// sequence dictates; a rescale is only looked for once per four keys.
 // ------------------------------------------------------------------------------------------------------
 
 #define T_Q   64
 #define T_KV  64
 #define T_LDH (FA_D + 8)      // f16 pitch of the Q and K tiles (144 B rows: conflict-free b128 reads for the MFMA operands)
-#define T_LDS (T_KV + 1)      // f32 pitch of the factor tiles
+#define T_LDF (T_KV + 4)      // f32 pitch of the factor tile (272 B rows: conflict-free b128 reads with lane = row)
+
+// exp(x) for x <= 0 to about 1 ulp: 2^(x log2 e) with the rounding error of the product fed back in
+__device__ __forceinline__ float exp_neg(float x) {
+    if (x < -104.0f) return 0.0f;                         // below the smallest denormal; also x = -inf (first key of a row)
+    const float l2e_hi = 1.44269502e+0f, l2e_lo = 1.92596299e-8f;
+    const float t = x * l2e_hi;
+    float e = __builtin_fmaf(x, l2e_hi, -t);
+    e = __builtin_fmaf(x, l2e_lo, e);
+    const float r = __builtin_amdgcn_exp2f(t);
+    return __builtin_fmaf(r, e * 0.693147182f, r);
+}
+
+typedef const uint32_t __attribute__((address_space(4))) * const_u32_ptr;   // read-only data: uniform loads become scalar loads
 
 __global__ void __launch_bounds__(256) k_fattn_seq_tile(fa_args a) {
     __shared__ __attribute__((aligned(16))) half_t q_s[T_Q * T_LDH];
     __shared__ __attribute__((aligned(16))) half_t k_s[T_KV * T_LDH];
     __shared__ __attribute__((aligned(16))) half_t v_s[T_KV * FA_D];
-    __shared__ float vs_s[T_Q * T_LDS];
-    __shared__ float ms_s[T_Q * T_LDS];
+    __shared__ __attribute__((aligned(16))) float  f_s[T_Q * T_LDF];
     __shared__ float m_run[T_Q], s_run[T_Q];
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int64_t n0 = (int64_t) blockIdx.x * T_Q, h = blockIdx.y, i3 = blockIdx.z;
     const char * qb = a.q + h * a.q_nb2 + i3 * a.q_nb3;
     const char * kb = a.k + (h / a.hk_ratio) * a.k_nb2 + (i3 / a.k_ne3_ratio) * a.k_nb3;
@@ -283,34 +326,38 @@ __global__ void __launch_bounds__(256) k_fattn_seq_tile(fa_args a) {
         }
     }
     if (tid < T_Q) { m_run[tid] = -INFINITY; s_run[tid] = 0.0f; }
-    __syncthreads();
 
-    // accumulation role: wavefront w owns queries 16w .. 16w+15, 4 lanes per query, 16 d each
-    const int aq = wave * 16 + (lane >> 2), ad = (lane & 3) * 16;
-    half_t acc[16];
+    // chain role: lane = query, this wavefront's d slice
+    const int d0 = wave * 16;
+    half2_t acc2[8];                                       // 16 f16 accumulators, two per register
 #pragma unroll
-    for (int e = 0; e < 16; ++e) acc[e] = (half_t) 0.0f;
+    for (int e = 0; e < 8; ++e) acc2[e] = (half2_t){ (half_t) 0.0f, (half_t) 0.0f };
 
     // score role: wavefront w computes the 32x32 patch (queries 32*(w/2).., keys 32*(w%2)..)
     const int sq = (wave >> 1) * 32, sk = (wave & 1) * 32, l32 = lane & 31, g = lane >> 5;
 
+    // K / V tile staging: thread t: row t/4, 32 bytes of each; the next tile is in flight while this one is worked on
+    const int kr = tid >> 2, kc = (tid & 3) * 16;
+    u32x4 kreg0, kreg1, vreg0, vreg1;
+    auto load_kv = [&](int64_t key0) __attribute__((always_inline)) {
+        const int64_t key = key0 + kr < a.KV ? key0 + kr : a.KV - 1;      // rows past the end repeat the last key; their scores are masked
+        const u32x4 * kp = (const u32x4 *)(kb + key * a.k_nb1 + kc * 2);
+        const u32x4 * vp = (const u32x4 *)(vb + key * a.v_nb1 + kc * 2);
+        kreg0 = kp[0]; kreg1 = kp[1]; vreg0 = vp[0]; vreg1 = vp[1];
+    };
+    load_kv(0);
+
     for (int64_t key0 = 0; key0 < a.KV; key0 += T_KV) {
-        // ---- stage K and V: thread t: row t/4, 32 bytes -----------------------------------------------------------------
-        {
-            const int r = tid >> 2, c = (tid & 3) * 16;
-            const int64_t key = key0 + r;
-            uint4 k0 = make_uint4(0, 0, 0, 0), k1 = k0, v0 = k0, v1 = k0;
-            if (key < a.KV) {
-                const uint4 * kp = (const uint4 *)(kb + key * a.k_nb1 + c * 2);
-                const uint4 * vp = (const uint4 *)(vb + key * a.v_nb1 + c * 2);
-                k0 = kp[0]; k1 = kp[1]; v0 = vp[0]; v1 = vp[1];
-            }
-            *(uint4 *)(k_s + r * T_LDH + c) = k0; *(uint4 *)(k_s + r * T_LDH + c + 8) = k1;
-            *(uint4 *)(v_s + r * FA_D + c)  = v0; *(uint4 *)(v_s + r * FA_D + c + 8)  = v1;
-        }
-        __syncthreads();
+        __syncthreads();                                   // the previous step's chains are done with v_s and f_s
+        *(u32x4 *)(k_s + kr * T_LDH + kc) = kreg0; *(u32x4 *)(k_s + kr * T_LDH + kc + 8) = kreg1;
+        *(u32x4 *)(v_s + kr * FA_D  + kc) = vreg0; *(u32x4 *)(v_s + kr * FA_D  + kc + 8) = vreg1;
+        __syncthreads();                                   // K / V tile (and, first time, Q tile) visible
+        if (key0 + T_KV < a.KV) load_kv(key0 + T_KV);
 
         // ---- scores: S = Q K^T on the matrix cores ------------------------------------------------------------------------------
+#ifdef FA_DBG_SKIP_SCORES
+        if (a.scale > 1e30f)
+#endif
         {
             float16_t c16;
 #pragma unroll
@@ -322,28 +369,37 @@ __global__ void __launch_bounds__(256) k_fattn_seq_tile(fa_args a) {
                 c16 = __builtin_amdgcn_mfma_f32_32x32x16_f16(av, bv, c16, 0, 0, 0);
             }
             const int64_t key = key0 + sk + l32;                  // accumulator column = key, rows = queries
+            const bool key_ok = key < a.KV;
+            float mv[16];
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const int qi = sq + 8 * (r >> 2) + 4 * g + (r & 3);
-                float s = -INFINITY;
-                if (key < a.KV) {
-                    float mv = 0.0f;
-                    if (a.mask && n0 + qi < a.N) mv = (float) *(const half_t *)(a.mask + (n0 + qi) * a.m_nb1 + key * 2);
-                    s = __fadd_rn(__fmul_rn(c16[r], a.scale), mv);
+                mv[r] = 0.0f;
+                if (a.mask) {
+                    const int64_t n = n0 + qi < a.N ? n0 + qi : a.N - 1;
+                    mv[r] = (float) *(const half_t *)(a.mask + n * a.m_nb1 + (key_ok ? key : a.KV - 1) * 2);
                 }
-                vs_s[qi * T_LDS + sk + l32] = s;
+            }
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int qi = sq + 8 * (r >> 2) + 4 * g + (r & 3);
+                f_s[qi * T_LDF + sk + l32] = key_ok ? __fadd_rn(__fmul_rn(c16[r], a.scale), mv[r]) : -INFINITY;
             }
         }
         __syncthreads();
 
-        // ---- softmax factors: thread t: query t/4, keys 16*(t%4) .. +15 ------------------------------------------------------------
+        // ---- factors: thread t: query t/4, keys 16*(t%4) .. +15 ---------------------------------------------------------------------
+#ifdef FA_DBG_SKIP_FACTORS
+        if (a.scale > 1e30f)
+#endif
         {
             const int qi = tid >> 2, sgm = tid & 3;
-            float * sp = vs_s + qi * T_LDS + sgm * 16;
-            float * mp = ms_s + qi * T_LDS + sgm * 16;
+            float4 * fp = (float4 *)(f_s + qi * T_LDF + sgm * 16);
             float sv[16], lmax = -INFINITY;
 #pragma unroll
-            for (int i = 0; i < 16; ++i) { sv[i] = sp[i]; lmax = fmaxf(lmax, sv[i]); }
+            for (int i = 0; i < 4; ++i) { const float4 t = fp[i]; sv[4*i] = t.x; sv[4*i+1] = t.y; sv[4*i+2] = t.z; sv[4*i+3] = t.w; }
+#pragma unroll
+            for (int i = 0; i < 16; ++i) lmax = fmaxf(lmax, sv[i]);
             float M = m_run[qi];
             const float S0 = s_run[qi];
             const int base = lane & ~3;
@@ -351,13 +407,23 @@ __global__ void __launch_bounds__(256) k_fattn_seq_tile(fa_args a) {
             if (sgm > 0) M = fmaxf(M, m0);
             if (sgm > 1) M = fmaxf(M, m1);
             if (sgm > 2) M = fmaxf(M, m2);
+            // this run's effect on the softmax denominator: S_after = S_before * P + A
             float P = 1.0f, A = 0.0f;
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
-                float vs, ms;
-                seq_factors(sv[i], M, vs, ms, P, A);
-                sp[i] = vs; mp[i] = ms;
+                // one exp serves both cases: a new maximum (ms = exp(M - s), 0 for the first key; vs = 1) and a standing
+                // one (vs = exp(s - M); masked keys, s = -inf, get vs = 0, a no-op on the accumulator)
+                const float s = sv[i];
+                const bool  raised = s > M;
+                const float x = raised ? M - s : s - M;    // <= 0; -inf - -inf (masked key before any other) is NaN ...
+                const float ex = s == -INFINITY ? 0.0f : exp_neg(x);                          // ... and never used
+                const float ms = raised ? ex : 1.0f, vs = raised ? 1.0f : ex;
+                M = raised ? s : M;
+                P *= ms; A = A * ms + vs;
+                sv[i] = raised ? -ex : ex;                 // -0.0 keeps the sign
             }
+#pragma unroll
+            for (int i = 0; i < 4; ++i) fp[i] = make_float4(sv[4*i], sv[4*i+1], sv[4*i+2], sv[4*i+3]);
             // fold the four runs of this query in key order
             const float P1 = __shfl(P, base + 1, WAVE), A1 = __shfl(A, base + 1, WAVE);
             const float P2 = __shfl(P, base + 2, WAVE), A2 = __shfl(A, base + 2, WAVE);
@@ -372,32 +438,85 @@ __global__ void __launch_bounds__(256) k_fattn_seq_tile(fa_args a) {
         __syncthreads();
 
         // ---- the sequential f16 chains over this tile's keys -----------------------------------------------------------------------------
+#ifdef FA_DBG_SKIP_CHAIN
+        if (a.scale > 1e30f)
+#endif
         {
-            const float * vsp = vs_s + aq * T_LDS;
-            const float * msp = ms_s + aq * T_LDS;
-#pragma unroll 4
-            for (int key = 0; key < T_KV; ++key) {
-                const float vs = vsp[key], ms = msp[key];
-                const half8_t va = *(const half8_t *)(v_s + key * FA_D + ad);
-                const half8_t vb8 = *(const half8_t *)(v_s + key * FA_D + ad + 8);
-                if (__any(ms != 1.0f)) {
+            const int nk = (int)(a.KV - key0 < T_KV ? a.KV - key0 : T_KV);       // uniform
+            const float4 * fp = (const float4 *)(f_s + lane * T_LDF);
+            const half8_t * vp = (const half8_t *)(v_s + d0);                    // + key * FA_D halves = 8 of these
+            // one group = four keys: their factors (one b128 read) and their V values (two broadcast b128 reads per key);
+            // the next group is read while this one is consumed
+            struct group { float4 f; half8_t v[4][2]; };
+            auto gload = [&](group & gr, int k4) __attribute__((always_inline)) {
+                gr.f = fp[k4 >> 2];
 #pragma unroll
-                    for (int e = 0; e < 16; ++e) acc[e] = seq_scale(acc[e], ms);     // lanes with ms == 1 keep their value exactly
+                for (int j = 0; j < 4; ++j) { gr.v[j][0] = vp[(k4 + j) * 8]; gr.v[j][1] = vp[(k4 + j) * 8 + 1]; }
+            };
+            auto chain4 = [&](const group & gr, int k4) __attribute__((always_inline)) {
+                const float fk[4] = { gr.f.x, gr.f.y, gr.f.z, gr.f.w };
+                const uint32_t sign = (__float_as_uint(fk[0]) | __float_as_uint(fk[1]) | __float_as_uint(fk[2]) | __float_as_uint(fk[3])) >> 31;
+                if (__any(sign)) {                         // some query's maximum moved within these keys: rescale its accumulators
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        if (k4 + j < nk) {
+                            const bool raised = __float_as_uint(fk[j]) >> 31;
+                            const float ms = raised ? -fk[j] : 1.0f, vs = raised ? 1.0f : fk[j];
+                            if (__any(raised)) {
+#pragma unroll
+                                for (int e = 0; e < 8; ++e) acc2[e] = seq_scale2(acc2[e], ms);   // ms == 1 leaves the value as it is
+                            }
+#pragma unroll
+                            for (int e = 0; e < 8; ++e) {
+                                const half8_t v8 = gr.v[j][e >> 2];
+                                acc2[e] = seq_mad2(acc2[e], (half2_t){ v8[2 * (e & 3)], v8[2 * (e & 3) + 1] }, vs);
+                            }
+                        }
+                    }
+                } else {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        if (k4 + j < nk) {
+#pragma unroll
+                            for (int e = 0; e < 8; ++e) {
+                                const half8_t v8 = gr.v[j][e >> 2];
+                                acc2[e] = seq_mad2(acc2[e], (half2_t){ v8[2 * (e & 3)], v8[2 * (e & 3) + 1] }, fk[j]);
+                            }
+                        }
+                    }
                 }
-#pragma unroll
-                for (int e = 0; e < 8; ++e) { acc[e] = seq_mad(acc[e], va[e], vs); acc[8 + e] = seq_mad(acc[8 + e], vb8[e], vs); }
+            };
+            // arrived(): first use of a group, placed before the next group's reads are issued, so that the wait it
+            // implies only covers reads that have had four keys' worth of time
+            auto arrived = [&](const group & gr) __attribute__((always_inline)) {
+                asm volatile("" :: "v"(gr.f.x), "v"(gr.v[3][1]));
+                __builtin_amdgcn_sched_barrier(0);
+            };
+            group ga, gb;
+            gload(ga, 0);
+            for (int k4 = 0; k4 < nk; k4 += 8) {
+                arrived(ga);
+                if (k4 + 4 < nk) gload(gb, k4 + 4);
+                __builtin_amdgcn_sched_barrier(0);
+                chain4(ga, k4);
+                if (k4 + 4 < nk) {
+                    arrived(gb);
+                    if (k4 + 8 < nk) gload(ga, k4 + 8);
+                    __builtin_amdgcn_sched_barrier(0);
+                    chain4(gb, k4 + 4);
+                }
             }
         }
-        __syncthreads();
     }
 
-    const int64_t n = n0 + aq;
+    const int64_t n = n0 + lane;
     if (n < a.N) {
-        const float inv = 1.0f / s_run[aq];
-        float * dp = (float *) a.d + ((i3 * a.N + n) * a.H + h) * FA_D + ad;
+        const float inv = 1.0f / s_run[lane];
+        float * dp = (float *) a.d + ((i3 * a.N + n) * a.H + h) * FA_D + d0;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            float4 o = { (float) acc[4*i] * inv, (float) acc[4*i + 1] * inv, (float) acc[4*i + 2] * inv, (float) acc[4*i + 3] * inv };
+            const half2_t p0 = acc2[2*i], p1 = acc2[2*i + 1];
+            float4 o = { (float) p0[0] * inv, (float) p0[1] * inv, (float) p1[0] * inv, (float) p1[1] * inv };
             *(float4 *)(dp + 4 * i) = o;
         }
     }
