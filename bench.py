@@ -6,9 +6,9 @@ A step is one whisper_encode() of a synthetic log-mel window (conv stem + 32 enc
 K/V of all decoder layers), timed with the window already resident in host memory; weights, KV caches and all
 intermediates live in HBM.  W untimed steps, then exactly K timed ones.
 
-Prints one JSON line.  `roofline` is for the dominant kernel of that step (the Q5_0 MFMA GEMM): algorithmic FLOPs of
-the launches divided by their durations, measured with HIP events on the backend's stream in a second pass over the
-same workload.  `cpu_baseline` is the reference's own ggml CPU backend (oracle/_ref) on the same model file and the
+Prints one JSON line.  `roofline` is for the kernel that takes most of that step: algorithmic FLOPs (or bytes) of its
+launches divided by their durations, measured with HIP events on the backend's stream in a second pass over the same
+workload; `kernel_rooflines` lists the same for every kernel with 30 or more launches per step.  `cpu_baseline` is the reference's own ggml CPU backend (oracle/_ref) on the same model file and the
 same window, on the host cores of this box.
 """
 from __future__ import annotations
@@ -57,6 +57,33 @@ def model_file(arch: str, ftype: str) -> str:
     return str(path)
 
 
+# HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled by the same counters over a 256 MiB copy:
+# x2 KiB and x1 KiB), for the large-v3 encoder shapes; the summary with the commands is under profiles/
+MEASURED_TRAFFIC_MB = {"mul_mat.gemm_q5_0": 47.4 + 5.5, "flash_attn.seq_tile": 70.9 + 7.7}
+
+# kernels that live on the matrix cores (bound "mfma"); everything else streams memory (bound "hbm")
+MFMA_KERNELS = ("mul_mat.gemm_", "flash_attn.seq_tile")
+
+
+def kernel_roofline(name: str, k: dict) -> dict:
+    """achieved = algorithmic flops (or bytes) of the launches / their summed durations"""
+    sec = k["ms"] * 1e-3
+    out = {"kernel": name, "launches": k["calls"], "avg_launch_us": round(1e3 * k["ms"] / k["calls"], 3)}
+    if name.startswith(MFMA_KERNELS) and k["flops"] > 0:
+        achieved = k["flops"] / sec / 1e12
+        out.update({"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_MFMA_F16_TFLOPS, "unit": "TFLOP/s",
+                    "frac": round(achieved / PEAK_MFMA_F16_TFLOPS, 5),
+                    "algorithmic_gflop_per_launch": round(k["flops"] / k["calls"] / 1e9, 4)})
+    else:
+        achieved = k["bytes"] / sec / 1e9
+        out.update({"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                    "frac": round(achieved / PEAK_HBM_GBS, 5),
+                    "algorithmic_mb_per_launch": round(k["bytes"] / k["calls"] / 1e6, 4)})
+    t = MEASURED_TRAFFIC_MB.get(name)
+    out["traffic"] = round(t * 1e6) if t else None
+    return out
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -79,21 +106,16 @@ def main() -> int:
                        "--warmup", str(a.warmup), "--profile-reps", "3", "--threads", str(a.threads)])
     ms_per_step = enc["ms_per_step"]
 
+    # per-kernel figures from HIP events on the backend's stream (three extra windows, not part of the timing above)
     kernels = {k["kernel"]: k for k in enc["kernels"]}
+    breakdown, rooflines = {}, {}
+    tot = sum(k["ms"] for k in kernels.values()) or 1.0
+    for n, k in sorted(kernels.items(), key=lambda kv: -kv[1]["ms"]):
+        breakdown[n] = {"launches_per_step": k["calls"] / enc["profile_reps"], "ms_per_step": round(k["ms"] / enc["profile_reps"], 4),
+                        "share": round(k["ms"] / tot, 4)}
+        rooflines[n] = kernel_roofline(n, k)
     dom_name = max(kernels, key=lambda n: kernels[n]["ms"]) if kernels else None
-    roofline = None
-    breakdown = {}
-    if dom_name:
-        tot = sum(k["ms"] for k in kernels.values())
-        for n, k in sorted(kernels.items(), key=lambda kv: -kv[1]["ms"]):
-            breakdown[n] = {"launches_per_step": k["calls"] / enc["profile_reps"], "ms_per_step": round(k["ms"] / enc["profile_reps"], 4),
-                            "share": round(k["ms"] / tot, 4)}
-        gemm = kernels.get("mul_mat.gemm_q5_0", kernels[dom_name])
-        achieved = gemm["flops"] / (gemm["ms"] * 1e-3) / 1e12
-        roofline = {"kernel": "mul_mat.gemm_q5_0" if "mul_mat.gemm_q5_0" in kernels else dom_name, "bound": "mfma",
-                    "achieved": round(achieved, 2), "peak": PEAK_MFMA_F16_TFLOPS, "unit": "TFLOP/s", "frac": round(achieved / PEAK_MFMA_F16_TFLOPS, 5),
-                    "traffic": None, "launches": gemm["calls"], "avg_launch_us": round(1e3 * gemm["ms"] / gemm["calls"], 3),
-                    "algorithmic_gflop_per_launch": round(gemm["flops"] / gemm["calls"] / 1e9, 4)}
+    roofline = rooflines.get(dom_name)
 
     # ---- decode: 224 five-token steps (the shape of a 5-beam search step) on large-v3-turbo Q8_0 ----------------------------
     dec = run_harness(["bench", "--model", dec_model, "--what", "decoder", "--backend", "gpu", "--reps", "3", "--warmup", "2",
@@ -103,9 +125,9 @@ def main() -> int:
     decode = {"model": "large-v3-turbo Q8_0", "steps": dec["steps"], "beams": dec["batch"], "ms_per_step": round(dec["ms_per_step"], 4),
               "steps_per_s": round(dec["steps_per_s"], 1), "beam_tokens_per_s": round(dec["batch_tokens_per_s"], 1)}
     if gemv:
-        gbs = gemv["bytes"] / (gemv["ms"] * 1e-3) / 1e9
-        decode["gemv_roofline"] = {"kernel": "mul_mat.gemv_q8_0", "bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                                   "frac": round(gbs / PEAK_HBM_GBS, 4), "avg_launch_us": round(1e3 * gemv["ms"] / gemv["calls"], 3)}
+        decode["gemv_roofline"] = kernel_roofline("mul_mat.gemv_q8_0", gemv)
+    decode["kernel_breakdown"] = {n: {"launches_per_step": k["calls"] / dec["steps"], "ms_per_step": round(k["ms"] / dec["steps"], 4)}
+                                  for n, k in sorted(dk.items(), key=lambda kv: -kv[1]["ms"])[:6]}
 
     # ---- CPU baseline: the reference's ggml CPU backend, same model file, same window ------------------------------------------
     cpu_baseline = None
@@ -140,6 +162,7 @@ def main() -> int:
         "decode": decode,
         "kernel_breakdown": breakdown,
         "roofline": roofline,
+        "kernel_rooflines": [r for r in rooflines.values() if r["launches"] / enc["profile_reps"] >= 30],
         "cpu_baseline": cpu_baseline,
     }
     print(json.dumps(out))

@@ -66,6 +66,9 @@ enum mi355x_epilogue_flags {
                                   there by the previous call with the same src1): skip the conversion pass     */
     MI355X_MM_ACT_Q8_0  = 256, /* GEMM path, F16 src0 that is the f16 image (mi355x_dequantize_row_f16) of a
                                   quantized weight: round src1 to Q8_0 as for the quantized weight itself      */
+    MI355X_MM_PREPARE_ONLY = 512, /* GEMM path: run only the src1 conversion pass into `workspace` and return; the
+                                  product itself then follows in a second call with MI355X_MM_WS_READY (lets a
+                                  caller time or overlap the two separately); a no-op on the other paths       */
 };
 
 typedef struct mi355x_epilogue {

@@ -336,6 +336,65 @@ def test_cpy_get_rows_im2col_softmax_concat(pkg, oracle, gpu):
     assert np.array_equal(gpu.down(d_o), np.concatenate([a, b], axis=0))
 
 
+# ------------------------------------------------------------------------------------------------------------------
+# the committed vectors of the reference's CPU backend (tests/golden), on the GPU box where the reference does not exist
+# ------------------------------------------------------------------------------------------------------------------
+
+@pytest.fixture(scope="module")
+def vec():
+    from pathlib import Path
+    return np.load(Path(__file__).resolve().parent / "golden" / "cpu_backend_vectors.npz", allow_pickle=False)
+
+
+@pytest.mark.parametrize("name", ["q5_0", "q8_0"])
+def test_golden_dequantize_and_mul_mat(pkg, oracle, gpu, vec, name):
+    t = getattr(pkg, name.upper())
+    blocks = vec[f"quant_{name}_blocks"]
+    d_b = gpu.up(blocks)
+    d_y = torch.empty(blocks.shape[0] * 128, dtype=torch.float32, device=gpu.dev)
+    pkg.check(pkg.kernels().mi355x_dequantize_row(t, d_b.data_ptr(), d_y.data_ptr(), d_y.numel(), gpu.stream))
+    assert np.array_equal(gpu.down(d_y).view(np.uint32), vec[f"dequant_{name}"].reshape(-1).view(np.uint32))       # bit-exact
+    for n in (1, 5, 40):
+        got, kernel = run_mul_mat(pkg, gpu, t, vec[f"mul_mat_{name}_w"], vec[f"mul_mat_{name}_x_n{n}"], 128, 48)
+        # north-star bound 5e-4; the GEMV forms the reference's integers (1e-10), the GEMM rounds d*q to f16 (1e-6)
+        assert oracle.nmse(got, vec[f"mul_mat_{name}_y_n{n}"]) <= (1e-10 if "gemv" in kernel else 1e-6), kernel
+
+
+def test_golden_activation_quantizer(pkg, gpu, vec):
+    x = vec["act_q8_0_input"]
+    d_x = gpu.up(x)
+    d_q = torch.empty(x.size // 32 * 34, dtype=torch.uint8, device=gpu.dev)
+    pkg.check(pkg.kernels().mi355x_quantize_row_q8_0(d_x.data_ptr(), d_q.data_ptr(), x.size, gpu.stream))
+    assert np.array_equal(gpu.down(d_q).reshape(x.shape[0], -1), vec["act_q8_0_blocks"])
+
+
+@pytest.mark.parametrize("name", ["enc", "dec"])
+def test_golden_flash_attn(pkg, oracle, gpu, vec, name):
+    mask = vec[f"fa_{name}_mask"] if f"fa_{name}_mask" in vec else None
+    got, _ = run_fa(pkg, gpu, vec[f"fa_{name}_q"], vec[f"fa_{name}_k"], vec[f"fa_{name}_v"], mask, float(vec[f"fa_{name}_scale"]), pkg.FA_F16_SEQ)
+    assert oracle.nmse(got, vec[f"fa_{name}_y"]) <= 1e-6           # north-star bound 5e-4
+
+
+def test_golden_norm_gelu_soft_max(pkg, oracle, gpu, vec):
+    lib = pkg.kernels()
+    for op, x, want, tol in (("norm", vec["norm_x"], vec["norm_y"], 1e-12), ("gelu", vec["gelu_x"], vec["gelu_y"], 0.0),
+                             ("soft_max", vec["soft_max_x"], vec["soft_max_y"], 1e-12)):
+        d_x = gpu.up(x)
+        d_y = torch.empty_like(d_x)
+        tx, ty = pkg.tensor(d_x, pkg.F32), pkg.tensor(d_y, pkg.F32)
+        if op == "norm":
+            pkg.check(lib.mi355x_norm(tx, ty, 1e-5, None, None, gpu.stream))
+        elif op == "gelu":
+            pkg.check(lib.mi355x_gelu(tx, ty, gpu.stream))
+        else:
+            pkg.check(lib.mi355x_soft_max(tx, None, ty, float(vec["soft_max_scale"]), gpu.stream))
+        got = gpu.down(d_y)
+        if tol == 0.0:
+            assert np.array_equal(got, want), op                 # the f16 table makes GELU reproducible bit for bit
+        else:
+            assert oracle.nmse(got, want) <= tol, op
+
+
 def test_smoke_entry_point():
     import __graft_entry__ as entry
     entry.smoke()

@@ -295,6 +295,17 @@ struct graph_runner {
             GGML_LOG_INFO("ggml-mi355x: %s %s [%lld x %lld x %lld] folds %d nodes, flags 0x%x\n", kernel_name, mm->name,
                           (long long) mm->ne[0], (long long) mm->ne[1], (long long) w->ne[0], used, epi.flags);
         }
+        // the activation conversion is a kernel of its own: run (and time) it apart from the product
+        if (need && x->type == GGML_TYPE_F32 && !(epi.flags & MI355X_MM_WS_READY)) {
+            mi355x_epilogue prep = epi;
+            prep.flags |= MI355X_MM_PREPARE_ONLY;
+            {
+                launch_scope ls(ctx, "mul_mat.src1_to_f16", nbytes_of(x) * 1.5, 0.0);
+                status = mi355x_mul_mat(&vw, &vx, &vd, &prep, ctx->ws, ctx->ws_size, ctx->stream);
+            }
+            if (status != MI355X_OK) return used;
+            epi.flags |= MI355X_MM_WS_READY;
+        }
         {
             launch_scope ls(ctx, kernel_name, bytes, flops);
             status = mi355x_mul_mat(&vw, &vx, &vd, epi.flags ? &epi : nullptr, ctx->ws, ctx->ws_size, ctx->stream);

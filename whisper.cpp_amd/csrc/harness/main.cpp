@@ -583,8 +583,41 @@ static int cmd_bench(const args & a) {
     return 0;
 }
 
+// ---------------------------------------------------------------------------------------------------------------
+// copy: a plain device copy of known size (one CPY node, f32 -> f32, contiguous) — the yardstick the memory-traffic
+// counters of a profiler are scaled by
+// ---------------------------------------------------------------------------------------------------------------
+
+static int cmd_copy(const args & a) {
+    const int64_t mib = a.num("mib", 256), reps = a.num("reps", 5);
+    ggml_backend_reg_t reg = load_plugin(true);
+    if (!reg) { printf("{\"error\": \"no MI355X backend\"}\n"); return 2; }
+    ggml_backend_t be = ggml_backend_dev_init(ggml_backend_reg_dev_get(reg, 0), nullptr);
+    if (!be) return 1;
+    ggml_init_params ip = { ggml_tensor_overhead() * 8 + ggml_graph_overhead(), nullptr, true };
+    ggml_context * ctx = ggml_init(ip);
+    const int64_t n = mib * 1024 * 1024 / 4;
+    ggml_tensor * src = ggml_new_tensor_1d(ctx, GGML_TYPE_F32, n), * dst = ggml_new_tensor_1d(ctx, GGML_TYPE_F32, n);
+    ggml_tensor * cp = ggml_cpy(ctx, src, dst);
+    ggml_cgraph * gf = ggml_new_graph(ctx);
+    ggml_build_forward_expand(gf, cp);
+    ggml_backend_buffer_t buf = ggml_backend_alloc_ctx_tensors(ctx, be);
+    if (!buf) return 1;
+    ggml_backend_buffer_clear(buf, 0);
+    if (ggml_backend_graph_compute(be, gf) != GGML_STATUS_SUCCESS) return 1;
+    const double t0 = now_ms();
+    for (int i = 0; i < reps; ++i) if (ggml_backend_graph_compute(be, gf) != GGML_STATUS_SUCCESS) return 1;
+    const double ms = (now_ms() - t0) / (double) reps;
+    printf("{\"copy\": \"f32 contiguous\", \"bytes_read\": %lld, \"bytes_written\": %lld, \"launches\": %lld, \"ms_per_launch\": %.4f, \"gb_per_s\": %.1f}\n",
+           (long long)(n * 4), (long long)(n * 4), (long long)(reps + 1), ms, 2.0 * n * 4 / ms / 1e6);
+    ggml_backend_buffer_free(buf);
+    ggml_free(ctx);
+    ggml_backend_free(be);
+    return 0;
+}
+
 int main(int argc, char ** argv) {
-    if (argc < 2) { fprintf(stderr, "usage: %s info|gen|selftest|ops|model|verify|bench [options]\n", argv[0]); return 2; }
+    if (argc < 2) { fprintf(stderr, "usage: %s info|gen|selftest|ops|model|verify|bench|copy [options]\n", argv[0]); return 2; }
     ggml_log_set(quiet_log, nullptr);
     whisper_log_set(quiet_log, nullptr);
     const std::string cmd = argv[1];
@@ -596,6 +629,7 @@ int main(int argc, char ** argv) {
     if (cmd == "model") return cmd_model(a);
     if (cmd == "verify") return cmd_verify(a);
     if (cmd == "bench") return cmd_bench(a);
+    if (cmd == "copy")  return cmd_copy(a);
     fprintf(stderr, "unknown command %s\n", cmd.c_str());
     return 2;
 }

@@ -722,6 +722,7 @@ extern "C" int mi355x_mul_mat(const mi355x_tensor * src0, const mi355x_tensor * 
     if ((flags & MI355X_EPI_RESIDUAL) && !epi->residual) return MI355X_ERR_INVALID;
     if ((flags & MI355X_EPI_RESIDUAL) && (flags & MI355X_EPI_OUT_F16)) return MI355X_ERR_UNSUPPORTED;
     if (a.M == 0 || a.N == 0 || dst->ne[2] * dst->ne[3] == 0) return MI355X_OK;
+    if ((flags & MI355X_MM_PREPARE_ONLY) && mm_path(src0, src1) != MM_GEMM) return MI355X_OK;      // nothing to prepare
 
     a.w = (const char *) src0->data; a.x = (const char *) src1->data; a.d = (char *) dst->data;
     a.w_nb1 = src0->nb[1]; a.w_nb2 = src0->nb[2]; a.w_nb3 = src0->nb[3];
@@ -759,6 +760,7 @@ extern "C" int mi355x_mul_mat(const mi355x_tensor * src0, const mi355x_tensor * 
             }
             g.x = (const char *) workspace; g.x_nb1 = a.K * 2; g.x_nb2 = slice; g.x_nb3 = slice * a.ne12;
         }
+        if (flags & MI355X_MM_PREPARE_ONLY) return launch_status();
         if (wbytes) {
             const int64_t slice = (int64_t) round256((size_t)(a.M * a.K * 2));
             half_t * w16 = (half_t *)((char *) workspace + xbytes);
