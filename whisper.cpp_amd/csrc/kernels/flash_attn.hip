@@ -117,6 +117,10 @@ __device__ __forceinline__ half_t seq_mad(half_t acc, half_t v, float vs) { retu
 // both roundings included.  Spelled out as instructions because the compiler otherwise mixes in v_fma_mixlo/hi_f16,
 // which issue at half rate on gfx950 and round the exact fma once (a last-bit difference from the reference's two steps).
 __device__ __forceinline__ half2_t seq_mad2(half2_t acc, half2_t v, float vs) {
+#ifdef FA_DBG_MIXLO
+    asm("v_fma_mixlo_f16 %0, %1, %2, %0 op_sel_hi:[1,0,1]\n\tv_fma_mixhi_f16 %0, %1, %2, %0 op_sel:[1,0,1] op_sel_hi:[1,0,1]" : "+v"(acc) : "v"(v), "v"(vs));
+    return acc;
+#endif
     float lo, hi;
     half2_t r;
     asm("v_fma_mix_f32 %0, %2, %3, %4 op_sel_hi:[1,0,1]\n\t"
@@ -151,6 +155,7 @@ __device__ __forceinline__ void seq_factors(float s, float & M, float & vs, floa
 // ------------------------------------------------------------------------------------------------------
 
 #define ROW_CHUNK 64
+#define ROW_STAGE 256     // keys staged per step = threads per workgroup
 
 __global__ void __launch_bounds__(256) k_fattn_seq_row(fa_args a, int kv_pad) {
     extern __shared__ __attribute__((aligned(16))) float sm[];
@@ -230,44 +235,90 @@ __global__ void __launch_bounds__(256) k_fattn_seq_row(fa_args a, int kv_pad) {
         s_total = S;
     }
     __syncthreads();
-    if (wave != 0) return;
 
     // ---- the sequential f16 chain: lane = d -----------------------------------------------------------------------------------
-    // 64 keys at a time: their V values sit in registers (the next 64 are in flight while these are consumed), their
-    // factors are read once, one per lane, and handed to the chain through v_readlane, so that the dependent part of
-    // every step is a single v_fma_mixlo_f16.
-    half_t acc = (half_t) 0.0f;
-    const char * vcol = vb + lane * 2;
-    half_t va[ROW_CHUNK], vn[ROW_CHUNK];
-    auto load_chunk = [&](half_t * dst, int key0) {
+    // One wavefront walks the keys; with nothing else running on its SIMD the time of a key is the latency of its
+    // dependent instructions, so the common case is straight-line code of two per key: v_fma_mix_f32 (f16 V, f32
+    // factor, f16 accumulator -> f32) and v_cvt_f16_f32 — the reference's f32 fma and its f16 store.  The factors are
+    // read once per 64 keys, one per lane (vs, or -ms where the key raises the maximum: then vs is 1), and reach the
+    // chain as scalar operands through v_readlane.  V is staged by the whole workgroup: 256 keys (rows of 128 B) per
+    // step into one of two LDS buffers, the next step's rows in flight meanwhile, so the walker never waits on HBM.
+    half_t * v_lds = (half_t *)(sm + 2 * kv_pad);          // [2][ROW_STAGE][FA_D]
+    u32x4 vrow[8];
+    auto load_rows = [&](int key0) __attribute__((always_inline)) {
+        const int key = key0 + tid;
+        const u32x4 * src = (const u32x4 *)(vb + (int64_t)(key < KV ? key : KV - 1) * a.v_nb1);
 #pragma unroll
-        for (int j = 0; j < ROW_CHUNK; ++j) {
-            const int key = key0 + j;
-            dst[j] = key < KV ? *(const half_t *)(vcol + (int64_t) key * a.v_nb1) : (half_t) 0.0f;
+        for (int i = 0; i < 8; ++i) vrow[i] = key < KV ? src[i] : (u32x4){0, 0, 0, 0};
+    };
+    auto store_rows = [&](int buf) __attribute__((always_inline)) {
+        u32x4 * dst = (u32x4 *)(v_lds + ((size_t) buf * ROW_STAGE + tid) * FA_D);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) dst[i] = vrow[i];
+    };
+
+    uint32_t acc = 0;                                      // f16 accumulator in the low half
+    auto mad = [&](half_t v, uint32_t vs_bits) __attribute__((always_inline)) {
+        float t;
+        asm("v_fma_mix_f32 %0, %1, %2, %3 op_sel_hi:[1,0,1]" : "=v"(t) : "v"(v), "s"(vs_bits), "v"(acc));
+        asm("v_cvt_f16_f32 %0, %1" : "=v"(acc) : "v"(t));
+    };
+    auto read_chunk = [&](half_t * dst, const half_t * vbuf, int k0) __attribute__((always_inline)) {
+#pragma unroll
+        for (int j = 0; j < ROW_CHUNK; ++j) dst[j] = vbuf[(k0 + j) * FA_D + lane];
+    };
+    auto run_chunk = [&](const half_t * v, int key0) __attribute__((always_inline)) {
+        const float vs_f = vs_s[key0 + lane], ms_f = ms_s[key0 + lane];
+        const bool  raised_l = ms_f != 1.0f;
+        const uint32_t f_l = __float_as_uint(raised_l ? -ms_f : vs_f);
+        const uint64_t raised = __ballot(raised_l);        // uniform: which of the 64 keys move the maximum
+        if (raised == 0) {
+#pragma unroll
+            for (int j = 0; j < ROW_CHUNK; ++j) mad(v[j], __builtin_amdgcn_readlane(f_l, j));   // masked keys: vs = 0 leaves acc as it is
+        } else {
+#pragma unroll
+            for (int j = 0; j < ROW_CHUNK; ++j) {
+                uint32_t f = __builtin_amdgcn_readlane(f_l, j);
+                if ((raised >> j) & 1) {                   // scalar condition
+                    float t;
+                    asm("v_fma_mix_f32 %0, %1, %2, 0 op_sel_hi:[1,0,0]" : "=v"(t) : "v"(acc), "s"(f ^ 0x80000000u));
+                    asm("v_cvt_f16_f32 %0, %1" : "=v"(acc) : "v"(t));
+                    f = 0x3f800000u;                       // vs = 1
+                }
+                mad(v[j], f);
+            }
         }
     };
-    auto run_chunk = [&](const half_t * v, int key0) {
-        const int vs_l = __float_as_int(vs_s[key0 + lane]), ms_l = __float_as_int(ms_s[key0 + lane]);
-#pragma unroll
-        for (int j = 0; j < ROW_CHUNK; ++j) {
-            const float vs = __int_as_float(__builtin_amdgcn_readlane(vs_l, j));
-            const float ms = __int_as_float(__builtin_amdgcn_readlane(ms_l, j));
-            if (ms != 1.0f) acc = seq_scale(acc, ms);      // scalar condition: uniform across the wavefront
-            if (vs != 0.0f) acc = seq_mad(acc, v[j], vs);
-        }
-    };
-    load_chunk(va, 0);
-    for (int key0 = 0; key0 < kv_pad; key0 += 2 * ROW_CHUNK) {
-        const bool more = key0 + ROW_CHUNK < kv_pad;
-        if (more) load_chunk(vn, key0 + ROW_CHUNK);
-        run_chunk(va, key0);
-        if (more) {
-            if (key0 + 2 * ROW_CHUNK < kv_pad) load_chunk(va, key0 + 2 * ROW_CHUNK);
-            run_chunk(vn, key0 + ROW_CHUNK);
+
+    load_rows(0);
+    int buf = 0;
+    for (int key0 = 0; key0 < kv_pad; key0 += ROW_STAGE, buf ^= 1) {
+        store_rows(buf);
+        __syncthreads();       // rows visible; the buffer written next time was last read before the previous barrier
+        if (key0 + ROW_STAGE < kv_pad) load_rows(key0 + ROW_STAGE);
+#ifdef FA_DBG_SKIP_ROWCHAIN
+        if (a.scale > 1e30f)
+#endif
+        if (wave == 0) {
+            const half_t * vbuf = v_lds + (size_t) buf * ROW_STAGE * FA_D;
+            const int nk = min(ROW_STAGE, kv_pad - key0);                   // multiple of ROW_CHUNK
+            half_t va[ROW_CHUNK], vn[ROW_CHUNK];
+            read_chunk(va, vbuf, 0);
+            for (int k0 = 0; k0 < nk; k0 += 2 * ROW_CHUNK) {
+                const bool more = k0 + ROW_CHUNK < nk;
+                if (more) read_chunk(vn, vbuf, k0 + ROW_CHUNK);
+                run_chunk(va, key0 + k0);
+                if (more) {
+                    if (k0 + 2 * ROW_CHUNK < nk) read_chunk(va, vbuf, k0 + 2 * ROW_CHUNK);
+                    run_chunk(vn, key0 + k0 + ROW_CHUNK);
+                }
+            }
         }
     }
+    if (wave != 0) return;
+    half_t acc_h; { const uint16_t t16 = (uint16_t) acc; __builtin_memcpy(&acc_h, &t16, 2); }
     float * dp = (float *) a.d + ((i3 * a.N + n) * a.H + h) * FA_D;
-    dp[lane] = (float) acc * (1.0f / s_total);
+    dp[lane] = (float) acc_h * (1.0f / s_total);
 }
 
 // ------------------------------------------------------------------------------------------------------
@@ -592,7 +643,15 @@ extern "C" int mi355x_flash_attn_ext(const mi355x_tensor * q, const mi355x_tenso
         case FA_K_SEQ_ROW: {
             const int kv_pad = (int)((KV + ROW_CHUNK - 1) / ROW_CHUNK * ROW_CHUNK);
             dim3 grid((unsigned) N, (unsigned) H, (unsigned) q->ne[3]);
-            k_fattn_seq_row<<<grid, 256, (size_t) kv_pad * 8, st>>>(a, kv_pad);
+            const size_t lds = (size_t) kv_pad * 8 + (size_t) 2 * ROW_STAGE * FA_D * sizeof(half_t);   // factors + two V stages
+            static bool configured[64];                    // per device: more than the default 64 KB of dynamic LDS
+            int dev = 0;
+            if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return MI355X_ERR_HIP;
+            if (!configured[dev]) {
+                if (hipFuncSetAttribute((const void *) k_fattn_seq_row, hipFuncAttributeMaxDynamicSharedMemorySize, SEQ_ROW_MAX_KV * 8 + 2 * ROW_STAGE * FA_D * 2) != hipSuccess) return MI355X_ERR_HIP;
+                configured[dev] = true;
+            }
+            k_fattn_seq_row<<<grid, 256, lds, st>>>(a, kv_pad);
         } break;
         case FA_K_SEQ_TILE: {
             const int64_t gx = (N + T_Q - 1) / T_Q;

@@ -403,6 +403,25 @@ static int launch_gemm_f16_auto(const mm_args & a, hipStream_t st) {
 // quantized GEMV (N <= 8)
 // ------------------------------------------------------------------------------------------------------
 
+// one weight block as loaded: scale bits, (Q5_0: high bits,) quants
+template <int T0> struct wraw { uint32_t d, qh, q[T0 == MI355X_TYPE_Q8_0 ? 8 : 4]; };
+template <int T0>
+__device__ __forceinline__ wraw<T0> load_wraw(const uint8_t * wrow, int kb) {
+    wraw<T0> r;
+    if constexpr (T0 == MI355X_TYPE_Q8_0) {
+        const uint8_t * b = wrow + (int64_t) kb * 34;
+        r.d = *(const uint16_t *) b; r.qh = 0;
+        const u128a2 q0 = *(const u128a2 *)(b + 2), q1 = *(const u128a2 *)(b + 18);
+        r.q[0] = q0.x; r.q[1] = q0.y; r.q[2] = q0.z; r.q[3] = q0.w; r.q[4] = q1.x; r.q[5] = q1.y; r.q[6] = q1.z; r.q[7] = q1.w;
+    } else {
+        const uint8_t * b = wrow + (int64_t) kb * 22;
+        r.d = *(const uint16_t *) b; r.qh = *(const u32a2 *)(b + 2);
+        const u128a2 qs = *(const u128a2 *)(b + 6);
+        r.q[0] = qs.x; r.q[1] = qs.y; r.q[2] = qs.z; r.q[3] = qs.w;
+    }
+    return r;
+}
+
 // LDS: int32 xq[NC][K/4] | float xd[NC][K/32] | int32 xsum[NC][K/32]
 template <int T0, int NC, int LPR>
 __global__ void __launch_bounds__(256) k_gemv_q(mm_args a) {
@@ -412,6 +431,39 @@ __global__ void __launch_bounds__(256) k_gemv_q(mm_args a) {
     int32_t * xq   = (int32_t *) smem;
     float *   xd   = (float *)(smem + (size_t) NC * K);
     int32_t * xsum = (int32_t *)(smem + (size_t) NC * K + (size_t) NC * nbk * 4);
+
+    constexpr int RPW = WAVE / LPR;                 // rows per wavefront
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int j = lane % LPR, r = lane / LPR;
+    const int64_t row = (int64_t) blockIdx.x * (4 * RPW) + wave * RPW + r;
+    const bool row_ok = row < a.M;
+    const uint8_t * wrow = (const uint8_t *) a.w + (row_ok ? row : 0) * a.w_nb1;
+
+    float acc[NC];
+#pragma unroll
+    for (int n = 0; n < NC; ++n) acc[n] = 0.0f;
+
+    // the epilogue operands of the lane that will store are fetched now, under the weight stream
+    const bool writer = row_ok && j == 0;
+    float e_bias = 0.0f, e_bcol[NC], e_res[NC];
+#pragma unroll
+    for (int n = 0; n < NC; ++n) { e_bcol[n] = 0.0f; e_res[n] = 0.0f; }
+    if (writer) {
+        if (a.e.flags & MI355X_EPI_BIAS) e_bias = a.e.bias[row];
+        if (a.e.flags & MI355X_EPI_BIAS_COL) {
+#pragma unroll
+            for (int n = 0; n < NC; ++n) e_bcol[n] = a.e.bias[n];
+        }
+        if (a.e.flags & MI355X_EPI_RESIDUAL) {
+#pragma unroll
+            for (int n = 0; n < NC; ++n) e_res[n] = *(const float *)(a.e.residual + n * a.d_nb1 + row * 4);
+        }
+    }
+
+    // this lane's first weight block is requested before the activations are touched: the two HBM round trips of the
+    // kernel (activations, weights) overlap instead of following each other
+    wraw<T0> blk;
+    if (row_ok && j < nbk) blk = load_wraw<T0>(wrow, j);
 
     // --- quantize X: 8 lanes per 32-value block, round-to-nearest-even like _mm256_round_ps(_MM_ROUND_NEAREST).
     // Eight independent loads per thread are in flight before the first is consumed.
@@ -453,55 +505,20 @@ __global__ void __launch_bounds__(256) k_gemv_q(mm_args a) {
     }
     __syncthreads();
 
-    constexpr int RPW = WAVE / LPR;                 // rows per wavefront
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int j = lane % LPR, r = lane / LPR;
-    const int64_t row = (int64_t) blockIdx.x * (4 * RPW) + wave * RPW + r;
-    const bool row_ok = row < a.M;
-    const uint8_t * wrow = (const uint8_t *) a.w + (row_ok ? row : 0) * a.w_nb1;
-
-    float acc[NC];
-#pragma unroll
-    for (int n = 0; n < NC; ++n) acc[n] = 0.0f;
-
-    // the epilogue operands of the lane that will store are fetched now, under the weight stream
-    const bool writer = row_ok && j == 0;
-    float e_bias = 0.0f, e_bcol[NC], e_res[NC];
-#pragma unroll
-    for (int n = 0; n < NC; ++n) { e_bcol[n] = 0.0f; e_res[n] = 0.0f; }
-    if (writer) {
-        if (a.e.flags & MI355X_EPI_BIAS) e_bias = a.e.bias[row];
-        if (a.e.flags & MI355X_EPI_BIAS_COL) {
-#pragma unroll
-            for (int n = 0; n < NC; ++n) e_bcol[n] = a.e.bias[n];
-        }
-        if (a.e.flags & MI355X_EPI_RESIDUAL) {
-#pragma unroll
-            for (int n = 0; n < NC; ++n) e_res[n] = *(const float *)(a.e.residual + n * a.d_nb1 + row * 4);
-        }
-    }
-
     if (row_ok) {
         for (int kb = j; kb < nbk; kb += LPR) {
+            const wraw<T0> cur = blk;
+            if (kb + LPR < nbk) blk = load_wraw<T0>(wrow, kb + LPR);      // next block in flight under this one's dot products
             uint32_t q[8];
-            float dw;
+            const float dw = h2f((uint16_t) cur.d);
             if constexpr (T0 == MI355X_TYPE_Q8_0) {
-                const uint8_t * b = wrow + (int64_t) kb * 34;
-                dw = h2f(*(const uint16_t *) b);
-                const u128a2 q0 = *(const u128a2 *)(b + 2);
-                const u128a2 q1 = *(const u128a2 *)(b + 18);
-                q[0] = q0.x; q[1] = q0.y; q[2] = q0.z; q[3] = q0.w;
-                q[4] = q1.x; q[5] = q1.y; q[6] = q1.z; q[7] = q1.w;
+#pragma unroll
+                for (int i = 0; i < 8; ++i) q[i] = cur.q[i];
             } else {
-                const uint8_t * b = wrow + (int64_t) kb * 22;
-                dw = h2f(*(const uint16_t *) b);
-                const uint32_t qh = *(const u32a2 *)(b + 2);
-                const u128a2 qs = *(const u128a2 *)(b + 6);
-                const uint32_t s[4] = { qs.x, qs.y, qs.z, qs.w };
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {     // unsigned 5-bit values; the -16 is applied through xsum
-                    q[i]     = (s[i] & 0x0F0F0F0Fu)        | spread4_to_bit4((qh >> (4*i))      & 0xFu);
-                    q[4 + i] = ((s[i] >> 4) & 0x0F0F0F0Fu) | spread4_to_bit4((qh >> (16 + 4*i)) & 0xFu);
+                    q[i]     = (cur.q[i] & 0x0F0F0F0Fu)        | spread4_to_bit4((cur.qh >> (4*i))      & 0xFu);
+                    q[4 + i] = ((cur.q[i] >> 4) & 0x0F0F0F0Fu) | spread4_to_bit4((cur.qh >> (16 + 4*i)) & 0xFu);
                 }
             }
 #pragma unroll
