@@ -156,6 +156,12 @@ MI355X_API int mi355x_gelu(const mi355x_tensor * src, const mi355x_tensor * dst,
  * src/whisper.cpp:2116-2121).  All F32. */
 MI355X_API int mi355x_norm(const mi355x_tensor * src, const mi355x_tensor * dst, float eps,
                            const float * w, const float * b, void * stream);
+/* The same, and in the same pass the result's image for the MFMA GEMM: rounded to Q8_0 as quantize_row_q8_0 does
+ * (ggml-cpu-quants.c:808-865) and stored as f16(q * d), dense [rows][ne0], at `x16` — what mi355x_mul_mat's src1
+ * conversion pass would write into its workspace (then pass MI355X_MM_WS_READY).  ne0 multiple of 32 and at most 2048,
+ * 16-byte aligned rows; MI355X_ERR_UNSUPPORTED otherwise. */
+MI355X_API int mi355x_norm_emit_f16(const mi355x_tensor * src, const mi355x_tensor * dst, float eps, const float * w, const float * b,
+                                    void * x16, void * stream);
 
 /* SOFT_MAX (ggml/src/ggml-cpu/ops.cpp:4641-4737), max_bias = 0: softmax(scale * x + mask) over ne0.
  * mask F32 or F16 [ne0, >= ne1], broadcast over ne2/ne3, or NULL. */

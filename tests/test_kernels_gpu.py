@@ -266,6 +266,17 @@ def test_norm_and_affine(pkg, oracle, gpu):
         d_w, d_b = gpu.up(w), gpu.up(b)
         pkg.check(lib.mi355x_norm(pkg.tensor(d_x, pkg.F32), pkg.tensor(d_y, pkg.F32), 1e-5, d_w.data_ptr(), d_b.data_ptr(), gpu.stream))
         assert oracle.nmse(gpu.down(d_y), want * w + b) <= 1e-10
+        # the variant that also leaves the GEMM's activation image: the Q8_0 rounding of what it just wrote, as f16(q * d)
+        d_h = torch.zeros(shape, dtype=torch.float16, device=gpu.dev)
+        rc = lib.mi355x_norm_emit_f16(pkg.tensor(d_x, pkg.F32), pkg.tensor(d_y, pkg.F32), 1e-5, d_w.data_ptr(), d_b.data_ptr(), d_h.data_ptr(), gpu.stream)
+        if shape[1] % 32 == 0 and shape[1] <= 2048:
+            pkg.check(rc)
+            y = gpu.down(d_y)
+            assert oracle.nmse(y, want * w + b) <= 1e-10
+            image = oracle.dequantize(oracle.Q8_0, oracle.quantize(oracle.Q8_0, y, act=True), shape[1]).reshape(shape)
+            assert np.array_equal(gpu.down(d_h, np.uint16), oracle.f32_to_f16_bits(image))
+        else:
+            assert rc == -1                      # unsupported shapes say so; the caller falls back to the plain kernel
 
 
 def test_gelu_scale_binary(pkg, oracle, gpu):

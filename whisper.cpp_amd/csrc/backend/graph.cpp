@@ -332,9 +332,33 @@ struct graph_runner {
             }
         }
         mi355x_tensor vs = to_view(nm->src[0]), vd = to_view(out);
-        launch_scope ls(ctx, used == 3 ? "norm_affine" : "norm", nbytes_of(nm->src[0]) + nbytes_of(out), 0.0);
-        status = mi355x_norm(&vs, &vd, eps, w, b, ctx->stream);
+        // When everything that reads the result is a many-column product with quantized weights, the kernel also leaves
+        // the Q8_0-rounded f16 image those products want in the workspace, and they skip their conversion pass.
+        bool emit = false;
+        if (ctx->fuse && !ctx->exact && out->ne[2] == 1 && out->ne[3] == 1 && out->ne[1] > MI355X_GEMV_MAX_COLS && out->ne[0] % 32 == 0 &&
+            out->ne[0] <= 2048 && ggml_is_contiguous(out) && !(out->flags & GGML_TENSOR_FLAG_OUTPUT)) {
+            auto it = readers.find(out);
+            int want = it == readers.end() ? 0 : it->second, seen = 0;
+            for (int j = i + used; j < g->n_nodes && want > 0; ++j) {
+                const ggml_tensor * n = g->nodes[j];
+                bool reads = false;
+                for (int k = 0; k < GGML_MAX_SRC; ++k) reads = reads || n->src[k] == out;
+                if (!reads && n->view_src != out) continue;
+                if (n->op == GGML_OP_MUL_MAT && n->src[1] == out && n->src[0] != out && ggml_is_quantized(n->src[0]->type)) ++seen; else { seen = -1; break; }
+                if (seen == want) break;
+            }
+            emit = want > 0 && seen == want && ctx->reserve_workspace((size_t)(out->ne[0] * out->ne[1] * 2 + 256));
+        }
+        {
+            launch_scope ls(ctx, used == 3 ? (emit ? "norm_affine_emit" : "norm_affine") : "norm", nbytes_of(nm->src[0]) + nbytes_of(out) * (emit ? 1.5 : 1.0), 0.0);
+            status = emit ? mi355x_norm_emit_f16(&vs, &vd, eps, w, b, ctx->ws, ctx->stream) : mi355x_norm(&vs, &vd, eps, w, b, ctx->stream);
+        }
+        if (emit && status == MI355X_ERR_UNSUPPORTED) { emit = false; status = mi355x_norm(&vs, &vd, eps, w, b, ctx->stream); }
         note_write(out);
+        if (emit && status == MI355X_OK) {
+            ctx->ws_x = out->data; ctx->ws_x_mode = 1; memcpy(ctx->ws_x_ne, out->ne, sizeof(out->ne)); memcpy(ctx->ws_x_nb, out->nb, sizeof(out->nb));
+            cached_x = out;
+        }
         return used;
     }
 

@@ -217,7 +217,8 @@ __global__ void k_x_to_f16(const char * __restrict__ x, half_t * __restrict__ ou
         amax = fmaxf(amax, __shfl_xor(amax, 4, 8));
         const float id = amax != 0.0f ? 127.0f / amax : 0.0f;
         const float d  = h2f(f2h_bits(amax / 127.0f));                      // the scale goes through f16, like block_q8_0.d
-        h = (half4_t){ (half_t)(rintf(v.x * id) * d), (half_t)(rintf(v.y * id) * d), (half_t)(rintf(v.z * id) * d), (half_t)(rintf(v.w * id) * d) };
+        // (+ 0.0f: a quant that rounds to -0 is the integer 0, whose product with d is +0)
+        h = (half4_t){ (half_t)((rintf(v.x * id) + 0.0f) * d), (half_t)((rintf(v.y * id) + 0.0f) * d), (half_t)((rintf(v.z * id) + 0.0f) * d), (half_t)((rintf(v.w * id) + 0.0f) * d) };
     } else {
         h = (half4_t){ (half_t) v.x, (half_t) v.y, (half_t) v.z, (half_t) v.w };
     }

@@ -10,8 +10,11 @@
 // NORM (ggml/src/ggml-cpu/ops.cpp:3109-3158): mean, then variance of the centred values, then scale.
 // ------------------------------------------------------------------------------------------------------
 
-template <bool IN_REGS>
-__global__ void k_norm(tview s, tview d, int64_t nrows, float eps, const float * __restrict__ w, const float * __restrict__ b) {
+// EMIT: also write the row as the MFMA GEMM wants its activations — rounded to Q8_0 like quantize_row_q8_0
+// (ggml-cpu-quants.c:808-865: block amax, id = 127/amax, round half to even, d through f16) and stored as f16(q * d),
+// dense [nrows][ne0] — so that the products that follow need no conversion pass of their own.
+template <bool IN_REGS, bool EMIT>
+__global__ void k_norm(tview s, tview d, int64_t nrows, float eps, const float * __restrict__ w, const float * __restrict__ b, half_t * __restrict__ x16) {
     const int     lane = threadIdx.x % WAVE;
     const int64_t row  = (int64_t) blockIdx.x * ROWS_PER_BLOCK + threadIdx.x / WAVE;
     if (row >= nrows) return;
@@ -55,6 +58,16 @@ __global__ void k_norm(tview s, tview d, int64_t nrows, float eps, const float *
                 if (w) { r.x *= ww[j].x; r.y *= ww[j].y; r.z *= ww[j].z; r.w *= ww[j].w; }
                 if (b) { r.x += bb[j].x; r.y += bb[j].y; r.z += bb[j].z; r.w += bb[j].w; }
                 ((float4 *) y)[c] = r;
+                if (EMIT) {                                // a 32-value block = 8 consecutive lanes (ne0 % 32 == 0: they are all here)
+                    float amax = fmaxf(fmaxf(fabsf(r.x), fabsf(r.y)), fmaxf(fabsf(r.z), fabsf(r.w)));
+                    amax = fmaxf(amax, __shfl_xor(amax, 1, 8));
+                    amax = fmaxf(amax, __shfl_xor(amax, 2, 8));
+                    amax = fmaxf(amax, __shfl_xor(amax, 4, 8));
+                    const float id = amax != 0.0f ? 127.0f / amax : 0.0f;
+                    const float dq = h2f(f2h_bits(amax / 127.0f));
+                    const half4_t h = { (half_t)((rintf(r.x * id) + 0.0f) * dq), (half_t)((rintf(r.y * id) + 0.0f) * dq), (half_t)((rintf(r.z * id) + 0.0f) * dq), (half_t)((rintf(r.w * id) + 0.0f) * dq) };
+                    *(half4_t *)(x16 + row * ne0 + 4 * (int64_t) c) = h;
+                }
             }
         }
     } else {
@@ -73,7 +86,18 @@ __global__ void k_norm(tview s, tview d, int64_t nrows, float eps, const float *
     }
 }
 
+static int norm_impl(const mi355x_tensor * src, const mi355x_tensor * dst, float eps, const float * w, const float * b, void * x16, void * stream);
+
 extern "C" int mi355x_norm(const mi355x_tensor * src, const mi355x_tensor * dst, float eps, const float * w, const float * b, void * stream) {
+    return norm_impl(src, dst, eps, w, b, nullptr, stream);
+}
+
+extern "C" int mi355x_norm_emit_f16(const mi355x_tensor * src, const mi355x_tensor * dst, float eps, const float * w, const float * b, void * x16, void * stream) {
+    if (!x16 || (uintptr_t) x16 % 8 != 0) return MI355X_ERR_INVALID;
+    return norm_impl(src, dst, eps, w, b, x16, stream);
+}
+
+static int norm_impl(const mi355x_tensor * src, const mi355x_tensor * dst, float eps, const float * w, const float * b, void * x16, void * stream) {
     if (!src || !dst || !(eps >= 0.0f)) return MI355X_ERR_INVALID;
     if (src->type != MI355X_TYPE_F32 || dst->type != MI355X_TYPE_F32) return MI355X_ERR_UNSUPPORTED;
     if (!same_shape(src, dst) || src->nb[0] != 4 || dst->nb[0] != 4) return MI355X_ERR_INVALID;
@@ -88,8 +112,13 @@ extern "C" int mi355x_norm(const mi355x_tensor * src, const mi355x_tensor * dst,
     const bool in_regs = src->ne[0] % 4 == 0 && src->ne[0] <= 4 * WAVE * NORM_MAX_V4 &&
                          al16(src->data, src->nb) && al16(dst->data, dst->nb) &&
                          (uintptr_t) w % 16 == 0 && (uintptr_t) b % 16 == 0;
-    if (in_regs) k_norm<true ><<<(unsigned) grid, ROWS_PER_BLOCK * WAVE, 0, st>>>(make_view(src), make_view(dst), nrows, eps, w, b);
-    else         k_norm<false><<<(unsigned) grid, ROWS_PER_BLOCK * WAVE, 0, st>>>(make_view(src), make_view(dst), nrows, eps, w, b);
+    if (x16) {                                             // only the register-resident form emits, and only whole blocks
+        if (!in_regs || src->ne[0] % QK != 0) return MI355X_ERR_UNSUPPORTED;
+        k_norm<true, true><<<(unsigned) grid, ROWS_PER_BLOCK * WAVE, 0, st>>>(make_view(src), make_view(dst), nrows, eps, w, b, (half_t *) x16);
+        return launch_status();
+    }
+    if (in_regs) k_norm<true,  false><<<(unsigned) grid, ROWS_PER_BLOCK * WAVE, 0, st>>>(make_view(src), make_view(dst), nrows, eps, w, b, nullptr);
+    else         k_norm<false, false><<<(unsigned) grid, ROWS_PER_BLOCK * WAVE, 0, st>>>(make_view(src), make_view(dst), nrows, eps, w, b, nullptr);
     return launch_status();
 }
 
