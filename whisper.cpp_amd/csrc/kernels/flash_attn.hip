@@ -117,10 +117,6 @@ __device__ __forceinline__ half_t seq_mad(half_t acc, half_t v, float vs) { retu
 // both roundings included.  Spelled out as instructions because the compiler otherwise mixes in v_fma_mixlo/hi_f16,
 // which issue at half rate on gfx950 and round the exact fma once (a last-bit difference from the reference's two steps).
 __device__ __forceinline__ half2_t seq_mad2(half2_t acc, half2_t v, float vs) {
-#ifdef FA_DBG_MIXLO
-    asm("v_fma_mixlo_f16 %0, %1, %2, %0 op_sel_hi:[1,0,1]\n\tv_fma_mixhi_f16 %0, %1, %2, %0 op_sel:[1,0,1] op_sel_hi:[1,0,1]" : "+v"(acc) : "v"(v), "v"(vs));
-    return acc;
-#endif
     float lo, hi;
     half2_t r;
     asm("v_fma_mix_f32 %0, %2, %3, %4 op_sel_hi:[1,0,1]\n\t"
@@ -296,9 +292,6 @@ __global__ void __launch_bounds__(256) k_fattn_seq_row(fa_args a, int kv_pad) {
         store_rows(buf);
         __syncthreads();       // rows visible; the buffer written next time was last read before the previous barrier
         if (key0 + ROW_STAGE < kv_pad) load_rows(key0 + ROW_STAGE);
-#ifdef FA_DBG_SKIP_ROWCHAIN
-        if (a.scale > 1e30f)
-#endif
         if (wave == 0) {
             const half_t * vbuf = v_lds + (size_t) buf * ROW_STAGE * FA_D;
             const int nk = min(ROW_STAGE, kv_pad - key0);                   // multiple of ROW_CHUNK
@@ -406,9 +399,6 @@ __global__ void __launch_bounds__(256) k_fattn_seq_tile(fa_args a) {
         if (key0 + T_KV < a.KV) load_kv(key0 + T_KV);
 
         // ---- scores: S = Q K^T on the matrix cores ------------------------------------------------------------------------------
-#ifdef FA_DBG_SKIP_SCORES
-        if (a.scale > 1e30f)
-#endif
         {
             float16_t c16;
 #pragma unroll
@@ -440,9 +430,6 @@ __global__ void __launch_bounds__(256) k_fattn_seq_tile(fa_args a) {
         __syncthreads();
 
         // ---- factors: thread t: query t/4, keys 16*(t%4) .. +15 ---------------------------------------------------------------------
-#ifdef FA_DBG_SKIP_FACTORS
-        if (a.scale > 1e30f)
-#endif
         {
             const int qi = tid >> 2, sgm = tid & 3;
             float4 * fp = (float4 *)(f_s + qi * T_LDF + sgm * 16);
@@ -489,9 +476,6 @@ __global__ void __launch_bounds__(256) k_fattn_seq_tile(fa_args a) {
         __syncthreads();
 
         // ---- the sequential f16 chains over this tile's keys -----------------------------------------------------------------------------
-#ifdef FA_DBG_SKIP_CHAIN
-        if (a.scale > 1e30f)
-#endif
         {
             const int nk = (int)(a.KV - key0 < T_KV ? a.KV - key0 : T_KV);       // uniform
             const float4 * fp = (const float4 *)(f_s + lane * T_LDF);

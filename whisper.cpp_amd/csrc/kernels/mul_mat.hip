@@ -231,13 +231,16 @@ __global__ void k_x_to_f16(const char * __restrict__ x, half_t * __restrict__ ou
 // consecutive values of a dst row.  K advances 64 at a time through two LDS buffers: while the matrix cores work on
 // step s, the global loads of step s+2 are in flight and step s+1 moves from registers to the other buffer, with one
 // barrier per step.  LDS rows are padded to 144 B so that the 16-byte operand reads of 16 consecutive rows hit
-// distinct banks.
+// distinct banks.  What bounds the kernel is LDS throughput: ds_read_b128 returns about 64 B per clock and CU on this
+// part (one 32x32x16 operand per 16 clocks, while the four SIMDs could consume eight in that time), so with 64x64
+// accumulator patches per wavefront — one operand read per matrix instruction — plus the staging writes, the matrix cores
+// wait for LDS about half of the time.
 #define GB_K  64
 #define GB_LD (GB_K + 8)
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
-template <int TI, int TJ, int S, bool KTAIL>     // KTAIL: K is not a multiple of 64 (but of 8)
+template <int TI, int TJ, int S, bool KTAIL, bool FULL>     // KTAIL: K is not a multiple of 64 (but of 8); FULL: K / 64 is a multiple of S
 __global__ void __launch_bounds__(256) k_gemm_f16(mm_args a, int tiles_m, int tiles_n) {
     constexpr int BN = 64 * TI, BM = 64 * TJ;
     constexpr int XR = BN / 32, WR = BM / 32;          // 16-byte pieces per thread and step
@@ -305,46 +308,89 @@ __global__ void __launch_bounds__(256) k_gemm_f16(mm_args a, int tiles_m, int ti
             for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
 
     const int KT = (int)((a.K + GB_K - 1) / GB_K);
-    load(xrs[0], wrs[0], 0);
-    if (1 < KT) load(xrs[1], wrs[1], GB_K);
-    if (S > 2) { if (2 < KT) load(xrs[2 % S], wrs[2 % S], 2 * GB_K); if (3 < KT) load(xrs[3 % S], wrs[3 % S], 3 * GB_K); }
-    if (S > 4) { if (4 < KT) load(xrs[4 % S], wrs[4 % S], 4 * GB_K); if (5 < KT) load(xrs[5 % S], wrs[5 % S], 5 * GB_K); }
-    store(xrs[0], wrs[0], 0);
-    if (S < KT) load(xrs[0], wrs[0], (int64_t) S * GB_K);
-    __syncthreads();
-
-    auto step = [&](int kt, int buf, u32x4 (&xr)[XR], u32x4 (&wr)[WR]) __attribute__((always_inline)) {   // xr / wr: slot of step kt + 1
+    // one K step: the operand fragments of sub-step kk + 1 are read from LDS while the matrix cores work on kk
+    auto mma = [&](int buf) __attribute__((always_inline)) {
         const half_t * xs = xs_base + buf * BN * GB_LD + (wn  + l32) * GB_LD + 8 * g;
         const half_t * ws = ws_base + buf * BM * GB_LD + (wmo + l32) * GB_LD + 8 * g;
+        half8_t av[2][TI], bv[2][TJ];
+#pragma unroll
+        for (int i = 0; i < TI; ++i) av[0][i] = *(const half8_t *)(xs + 32 * i * GB_LD);
+#pragma unroll
+        for (int j = 0; j < TJ; ++j) bv[0][j] = *(const half8_t *)(ws + 32 * j * GB_LD);
 #pragma unroll
         for (int kk = 0; kk < GB_K / 16; ++kk) {
-            half8_t av[TI], bv[TJ];
+            const int c = kk & 1, nx = c ^ 1;
+            if (kk + 1 < GB_K / 16) {
 #pragma unroll
-            for (int i = 0; i < TI; ++i) av[i] = *(const half8_t *)(xs + 32 * i * GB_LD + kk * 16);
+                for (int i = 0; i < TI; ++i) av[nx][i] = *(const half8_t *)(xs + 32 * i * GB_LD + (kk + 1) * 16);
 #pragma unroll
-            for (int j = 0; j < TJ; ++j) bv[j] = *(const half8_t *)(ws + 32 * j * GB_LD + kk * 16);
+                for (int j = 0; j < TJ; ++j) bv[nx][j] = *(const half8_t *)(ws + 32 * j * GB_LD + (kk + 1) * 16);
+            }
 #pragma unroll
             for (int i = 0; i < TI; ++i)
 #pragma unroll
                 for (int j = 0; j < TJ; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(av[i], bv[j], acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(av[c][i], bv[c][j], acc[i][j], 0, 0, 0);
+            if (kk + 1 < GB_K / 16) {
+                // issue order: one LDS read after each of the first matrix instructions of this sub-step
+#pragma unroll
+                for (int r = 0; r < TI + TJ; ++r) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // 1 MFMA
+                    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);   // 1 DS read
+                }
+            }
         }
-        if (kt + 1 < KT) {
-            store(xr, wr, buf ^ 1);                     // the last readers of that buffer passed the previous barrier
-            if (kt + 1 + S < KT) load(xr, wr, (int64_t)(kt + 1 + S) * GB_K);
-        }
-        __syncthreads();
     };
-    for (int kt0 = 0; kt0 < KT; kt0 += S) {             // S is even: the LDS buffer of a step is the parity of its slot
-        if (kt0 + 0 < KT) step(kt0 + 0, 0, xrs[1 % S], wrs[1 % S]);
-        if (kt0 + 1 < KT) step(kt0 + 1, 1, xrs[2 % S], wrs[2 % S]);
-        if (S > 2) {
-            if (kt0 + 2 < KT) step(kt0 + 2, 0, xrs[3 % S], wrs[3 % S]);
-            if (kt0 + 3 < KT) step(kt0 + 3, 1, xrs[4 % S], wrs[4 % S]);
+    if constexpr (FULL) {
+        // The number of steps is a multiple of S: every step stores and loads unconditionally (beyond the end it re-reads
+        // the last step's operands, which nobody consumes).  With no load behind a branch the compiler knows how many
+        // are outstanding at every point and waits for exactly the oldest slot — with conditional loads it has to assume
+        // the younger ones were never issued, waits for all of them, and the ring degenerates to one step in flight.
+        const int last = KT - 1;
+#pragma unroll
+        for (int st = 0; st < S; ++st) load(xrs[st], wrs[st], (int64_t) st * GB_K);
+        store(xrs[0], wrs[0], 0);
+        load(xrs[0], wrs[0], (int64_t) min(S, last) * GB_K);
+        __syncthreads();
+        auto step = [&](int kt, int buf, u32x4 (&xr)[XR], u32x4 (&wr)[WR]) __attribute__((always_inline)) {   // xr / wr: slot of step kt + 1
+            mma(buf);
+            store(xr, wr, buf ^ 1);                     // the last readers of that buffer passed the previous barrier
+            load(xr, wr, (int64_t) min(kt + 1 + S, last) * GB_K);
+            __syncthreads();
+        };
+        for (int kt0 = 0; kt0 < KT; kt0 += S) {         // S is even: the LDS buffer of a step is the parity of its slot
+            step(kt0 + 0, 0, xrs[1 % S], wrs[1 % S]);
+            step(kt0 + 1, 1, xrs[2 % S], wrs[2 % S]);
+            if (S > 2) { step(kt0 + 2, 0, xrs[3 % S], wrs[3 % S]); step(kt0 + 3, 1, xrs[4 % S], wrs[4 % S]); }
+            if (S > 4) { step(kt0 + 4, 0, xrs[5 % S], wrs[5 % S]); step(kt0 + 5, 1, xrs[6 % S], wrs[6 % S]); }
         }
-        if (S > 4) {
-            if (kt0 + 4 < KT) step(kt0 + 4, 0, xrs[5 % S], wrs[5 % S]);
-            if (kt0 + 5 < KT) step(kt0 + 5, 1, xrs[6 % S], wrs[6 % S]);
+    } else {
+        load(xrs[0], wrs[0], 0);
+        if (1 < KT) load(xrs[1], wrs[1], GB_K);
+        if (S > 2) { if (2 < KT) load(xrs[2 % S], wrs[2 % S], 2 * GB_K); if (3 < KT) load(xrs[3 % S], wrs[3 % S], 3 * GB_K); }
+        if (S > 4) { if (4 < KT) load(xrs[4 % S], wrs[4 % S], 4 * GB_K); if (5 < KT) load(xrs[5 % S], wrs[5 % S], 5 * GB_K); }
+        store(xrs[0], wrs[0], 0);
+        if (S < KT) load(xrs[0], wrs[0], (int64_t) S * GB_K);
+        __syncthreads();
+        auto step = [&](int kt, int buf, u32x4 (&xr)[XR], u32x4 (&wr)[WR]) __attribute__((always_inline)) {
+            mma(buf);
+            if (kt + 1 < KT) {
+                store(xr, wr, buf ^ 1);
+                if (kt + 1 + S < KT) load(xr, wr, (int64_t)(kt + 1 + S) * GB_K);
+            }
+            __syncthreads();
+        };
+        for (int kt0 = 0; kt0 < KT; kt0 += S) {
+            if (kt0 + 0 < KT) step(kt0 + 0, 0, xrs[1 % S], wrs[1 % S]);
+            if (kt0 + 1 < KT) step(kt0 + 1, 1, xrs[2 % S], wrs[2 % S]);
+            if (S > 2) {
+                if (kt0 + 2 < KT) step(kt0 + 2, 0, xrs[3 % S], wrs[3 % S]);
+                if (kt0 + 3 < KT) step(kt0 + 3, 1, xrs[4 % S], wrs[4 % S]);
+            }
+            if (S > 4) {
+                if (kt0 + 4 < KT) step(kt0 + 4, 0, xrs[5 % S], wrs[5 % S]);
+                if (kt0 + 5 < KT) step(kt0 + 5, 1, xrs[6 % S], wrs[6 % S]);
+            }
         }
     }
 
@@ -361,7 +407,7 @@ __global__ void __launch_bounds__(256) k_gemm_f16(mm_args a, int tiles_m, int ti
     }
 }
 
-template <int TI, int TJ, int S, bool KTAIL>
+template <int TI, int TJ, int S, bool KTAIL, bool FULL>
 static int launch_gemm_f16_k(const mm_args & a, hipStream_t st) {
     static_assert(S % 2 == 0, "the LDS buffer index is the parity of the register slot");
     constexpr int BN = 64 * TI, BM = 64 * TJ;
@@ -370,25 +416,22 @@ static int launch_gemm_f16_k(const mm_args & a, hipStream_t st) {
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return MI355X_ERR_HIP;
     if (!configured[dev]) {
-        if (hipFuncSetAttribute((const void *) k_gemm_f16<TI, TJ, S, KTAIL>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds) != hipSuccess) return MI355X_ERR_HIP;
+        if (hipFuncSetAttribute((const void *) k_gemm_f16<TI, TJ, S, KTAIL, FULL>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds) != hipSuccess) return MI355X_ERR_HIP;
         configured[dev] = true;
     }
     const int64_t tm = (a.M + BM - 1) / BM, tn = (a.N + BN - 1) / BN;
     if (tm * tn > 0x7fffffff) return MI355X_ERR_UNSUPPORTED;
     dim3 grid((unsigned)(tm * tn), (unsigned)(a.ne12 * a.ne13));
-    k_gemm_f16<TI, TJ, S, KTAIL><<<grid, 256, lds, st>>>(a, (int) tm, (int) tn);
+    k_gemm_f16<TI, TJ, S, KTAIL, FULL><<<grid, 256, lds, st>>>(a, (int) tm, (int) tn);
     return launch_status();
 }
-static int g_stages = -1;
 template <int TI, int TJ>
 static int launch_gemm_f16(const mm_args & a, hipStream_t st) {
-    if (g_stages < 0) { const char * e = getenv("MI355X_GEMM_STAGES"); g_stages = e ? atoi(e) : 4; }
-    if (a.K % GB_K) return launch_gemm_f16_k<TI, TJ, 2, true>(a, st);
-    switch (g_stages) {
-        case 2:  return launch_gemm_f16_k<TI, TJ, 2, false>(a, st);
-        case 6:  return launch_gemm_f16_k<TI, TJ, 6, false>(a, st);
-        default: return launch_gemm_f16_k<TI, TJ, 4, false>(a, st);
-    }
+    if (a.K % GB_K) return launch_gemm_f16_k<TI, TJ, 2, true, false>(a, st);
+    const int64_t kt = a.K / GB_K;
+    if (kt % 4 == 0) return launch_gemm_f16_k<TI, TJ, 4, false, true>(a, st);
+    if (kt % 2 == 0) return launch_gemm_f16_k<TI, TJ, 2, false, true>(a, st);
+    return launch_gemm_f16_k<TI, TJ, 4, false, false>(a, st);
 }
 
 // tile shape: the largest whose grid still covers the 256 CUs about twice
@@ -433,33 +476,34 @@ __global__ void __launch_bounds__(256) k_gemv_q(mm_args a) {
     float *   xd   = (float *)(smem + (size_t) NC * K);
     int32_t * xsum = (int32_t *)(smem + (size_t) NC * K + (size_t) NC * nbk * 4);
 
+    // A workgroup takes every gridDim.x-th group of 4 * (64 / LPR) rows; the activations are quantized once for all of them.
     constexpr int RPW = WAVE / LPR;                 // rows per wavefront
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int j = lane % LPR, r = lane / LPR;
-    const int64_t row = (int64_t) blockIdx.x * (4 * RPW) + wave * RPW + r;
-    const bool row_ok = row < a.M;
+    const int64_t n_groups = (a.M + 4 * RPW - 1) / (4 * RPW);
+    int64_t group = blockIdx.x;
+    int64_t row = group * (4 * RPW) + wave * RPW + r;
+    bool row_ok = row < a.M;
     const uint8_t * wrow = (const uint8_t *) a.w + (row_ok ? row : 0) * a.w_nb1;
 
-    float acc[NC];
-#pragma unroll
-    for (int n = 0; n < NC; ++n) acc[n] = 0.0f;
-
-    // the epilogue operands of the lane that will store are fetched now, under the weight stream
-    const bool writer = row_ok && j == 0;
+    // the epilogue operands of the lane that will store are fetched early, under the weight stream
     float e_bias = 0.0f, e_bcol[NC], e_res[NC];
 #pragma unroll
     for (int n = 0; n < NC; ++n) { e_bcol[n] = 0.0f; e_res[n] = 0.0f; }
-    if (writer) {
-        if (a.e.flags & MI355X_EPI_BIAS) e_bias = a.e.bias[row];
-        if (a.e.flags & MI355X_EPI_BIAS_COL) {
+    auto fetch_epilogue = [&]() __attribute__((always_inline)) {
+        if (row_ok && j == 0) {
+            if (a.e.flags & MI355X_EPI_BIAS) e_bias = a.e.bias[row];
+            if (a.e.flags & MI355X_EPI_BIAS_COL) {
 #pragma unroll
-            for (int n = 0; n < NC; ++n) e_bcol[n] = a.e.bias[n];
-        }
-        if (a.e.flags & MI355X_EPI_RESIDUAL) {
+                for (int n = 0; n < NC; ++n) e_bcol[n] = a.e.bias[n];
+            }
+            if (a.e.flags & MI355X_EPI_RESIDUAL) {
 #pragma unroll
-            for (int n = 0; n < NC; ++n) e_res[n] = *(const float *)(a.e.residual + n * a.d_nb1 + row * 4);
+                for (int n = 0; n < NC; ++n) e_res[n] = *(const float *)(a.e.residual + n * a.d_nb1 + row * 4);
+            }
         }
-    }
+    };
+    fetch_epilogue();
 
     // this lane's first weight block is requested before the activations are touched: the two HBM round trips of the
     // kernel (activations, weights) overlap instead of following each other
@@ -506,56 +550,78 @@ __global__ void __launch_bounds__(256) k_gemv_q(mm_args a) {
     }
     __syncthreads();
 
-    if (row_ok) {
-        for (int kb = j; kb < nbk; kb += LPR) {
-            const wraw<T0> cur = blk;
-            if (kb + LPR < nbk) blk = load_wraw<T0>(wrow, kb + LPR);      // next block in flight under this one's dot products
-            uint32_t q[8];
-            const float dw = h2f((uint16_t) cur.d);
-            if constexpr (T0 == MI355X_TYPE_Q8_0) {
+    for (;;) {
+        float acc[NC];
 #pragma unroll
-                for (int i = 0; i < 8; ++i) q[i] = cur.q[i];
-            } else {
+        for (int n = 0; n < NC; ++n) acc[n] = 0.0f;
+        if (row_ok) {
+            for (int kb = j; kb < nbk; kb += LPR) {
+                const wraw<T0> cur = blk;
+                if (kb + LPR < nbk) blk = load_wraw<T0>(wrow, kb + LPR);      // next block in flight under this one's dot products
+                uint32_t q[8];
+                const float dw = h2f((uint16_t) cur.d);
+                if constexpr (T0 == MI355X_TYPE_Q8_0) {
 #pragma unroll
-                for (int i = 0; i < 4; ++i) {     // unsigned 5-bit values; the -16 is applied through xsum
-                    q[i]     = (cur.q[i] & 0x0F0F0F0Fu)        | spread4_to_bit4((cur.qh >> (4*i))      & 0xFu);
-                    q[4 + i] = ((cur.q[i] >> 4) & 0x0F0F0F0Fu) | spread4_to_bit4((cur.qh >> (16 + 4*i)) & 0xFu);
+                    for (int i = 0; i < 8; ++i) q[i] = cur.q[i];
+                } else {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {     // unsigned 5-bit values; the -16 is applied through xsum
+                        q[i]     = (cur.q[i] & 0x0F0F0F0Fu)        | spread4_to_bit4((cur.qh >> (4*i))      & 0xFu);
+                        q[4 + i] = ((cur.q[i] >> 4) & 0x0F0F0F0Fu) | spread4_to_bit4((cur.qh >> (16 + 4*i)) & 0xFu);
+                    }
+                }
+#pragma unroll
+                for (int n = 0; n < NC; ++n) {
+                    const int4 x0 = *(const int4 *)(xq + (int64_t) n * (K / 4) + kb * 8);
+                    const int4 x1 = *(const int4 *)(xq + (int64_t) n * (K / 4) + kb * 8 + 4);
+                    int s = 0;
+                    s = __builtin_amdgcn_sdot4((int) q[0], x0.x, s, false);
+                    s = __builtin_amdgcn_sdot4((int) q[1], x0.y, s, false);
+                    s = __builtin_amdgcn_sdot4((int) q[2], x0.z, s, false);
+                    s = __builtin_amdgcn_sdot4((int) q[3], x0.w, s, false);
+                    s = __builtin_amdgcn_sdot4((int) q[4], x1.x, s, false);
+                    s = __builtin_amdgcn_sdot4((int) q[5], x1.y, s, false);
+                    s = __builtin_amdgcn_sdot4((int) q[6], x1.z, s, false);
+                    s = __builtin_amdgcn_sdot4((int) q[7], x1.w, s, false);
+                    if constexpr (T0 == MI355X_TYPE_Q5_0) s -= 16 * xsum[n * nbk + kb];
+                    acc[n] += (float) s * (dw * xd[n * nbk + kb]);
                 }
             }
-#pragma unroll
-            for (int n = 0; n < NC; ++n) {
-                const int4 x0 = *(const int4 *)(xq + (int64_t) n * (K / 4) + kb * 8);
-                const int4 x1 = *(const int4 *)(xq + (int64_t) n * (K / 4) + kb * 8 + 4);
-                int s = 0;
-                s = __builtin_amdgcn_sdot4((int) q[0], x0.x, s, false);
-                s = __builtin_amdgcn_sdot4((int) q[1], x0.y, s, false);
-                s = __builtin_amdgcn_sdot4((int) q[2], x0.z, s, false);
-                s = __builtin_amdgcn_sdot4((int) q[3], x0.w, s, false);
-                s = __builtin_amdgcn_sdot4((int) q[4], x1.x, s, false);
-                s = __builtin_amdgcn_sdot4((int) q[5], x1.y, s, false);
-                s = __builtin_amdgcn_sdot4((int) q[6], x1.z, s, false);
-                s = __builtin_amdgcn_sdot4((int) q[7], x1.w, s, false);
-                if constexpr (T0 == MI355X_TYPE_Q5_0) s -= 16 * xsum[n * nbk + kb];
-                acc[n] += (float) s * (dw * xd[n * nbk + kb]);
-            }
         }
-    }
+        // this group's results are complete in registers; request the next group's first block before reducing and storing
+        const int64_t done_row = row;
+        const bool done_writer = row_ok && j == 0;
+        const float o_bias = e_bias;
+        float o_bcol[NC], o_res[NC];
 #pragma unroll
-    for (int n = 0; n < NC; ++n) {
-#pragma unroll
-        for (int o = LPR / 2; o > 0; o >>= 1) acc[n] += __shfl_xor(acc[n], o, LPR);
-    }
-    if (writer) {
-        const bool out_f16 = a.e.flags & MI355X_EPI_OUT_F16;
+        for (int n = 0; n < NC; ++n) { o_bcol[n] = e_bcol[n]; o_res[n] = e_res[n]; }
+        group += gridDim.x;
+        const bool more = group < n_groups;                 // uniform
+        if (more) {
+            row = group * (4 * RPW) + wave * RPW + r;
+            row_ok = row < a.M;
+            wrow = (const uint8_t *) a.w + (row_ok ? row : 0) * a.w_nb1;
+            if (row_ok && j < nbk) blk = load_wraw<T0>(wrow, j);
+            fetch_epilogue();
+        }
 #pragma unroll
         for (int n = 0; n < NC; ++n) {
-            float v = acc[n] + e_bias + e_bcol[n];          // at most one of the two biases is set
-            if (a.e.flags & MI355X_EPI_GELU)     v  = gelu_f32(v, a.e.gelu);
-            if (a.e.flags & MI355X_EPI_SCALE)    v *= a.e.scale;
-            if (a.e.flags & MI355X_EPI_RESIDUAL) v += e_res[n];
-            if (out_f16) *(half_t *)(a.d + n * a.d_nb1 + row * 2) = (half_t) v;
-            else         *(float  *)(a.d + n * a.d_nb1 + row * 4) = v;
+#pragma unroll
+            for (int o = LPR / 2; o > 0; o >>= 1) acc[n] += __shfl_xor(acc[n], o, LPR);
         }
+        if (done_writer) {
+            const bool out_f16 = a.e.flags & MI355X_EPI_OUT_F16;
+#pragma unroll
+            for (int n = 0; n < NC; ++n) {
+                float v = acc[n] + o_bias + o_bcol[n];          // at most one of the two biases is set
+                if (a.e.flags & MI355X_EPI_GELU)     v  = gelu_f32(v, a.e.gelu);
+                if (a.e.flags & MI355X_EPI_SCALE)    v *= a.e.scale;
+                if (a.e.flags & MI355X_EPI_RESIDUAL) v += o_res[n];
+                if (out_f16) *(half_t *)(a.d + n * a.d_nb1 + done_row * 2) = (half_t) v;
+                else         *(float  *)(a.d + n * a.d_nb1 + done_row * 4) = v;
+            }
+        }
+        if (!more) break;
     }
 }
 
@@ -633,7 +699,11 @@ static int launch_gemv(const mm_args & a, hipStream_t st) {
     int lpr = 8;
     while (lpr < 64 && a.M * lpr / 256 < 512) lpr *= 2;
     const int rows_per_wg = 4 * (WAVE / lpr);
-    const unsigned grid = (unsigned)((a.M + rows_per_wg - 1) / rows_per_wg);
+    // a workgroup walks several row groups when there are more than three per CU, so that the activations are quantized
+    // fewer times; the groups are dealt out evenly
+    const int64_t n_groups = (a.M + rows_per_wg - 1) / rows_per_wg;
+    const int64_t rounds   = (n_groups + 767) / 768;
+    const unsigned grid    = (unsigned)((n_groups + rounds - 1) / rounds);
     switch (lpr) {
         case 8:  k_gemv_q<T0, NC, 8 ><<<grid, 256, lds, st>>>(a); break;
         case 16: k_gemv_q<T0, NC, 16><<<grid, 256, lds, st>>>(a); break;
