@@ -120,6 +120,21 @@ MI355X_API size_t mi355x_mul_mat_workspace_size(const mi355x_tensor * src0, cons
 MI355X_API int    mi355x_mul_mat(const mi355x_tensor * src0, const mi355x_tensor * src1, const mi355x_tensor * dst,
                                  const mi355x_epilogue * epi, void * workspace, size_t workspace_size, void * stream);
 
+/* Several MUL_MATs over the same src1 in one launch (a layer's Q, K and V projections; the cross-attention K and V of all
+ * decoder layers): the same arithmetic as `count` calls of mi355x_mul_mat, item by item, but one grid that fills the
+ * device where a single 1280-row product covers half of it.  No counterpart in the reference, whose graphs issue these
+ * products one node at a time.  Only the shape this exists for: every src0 a dense 2-d F16 matrix of the same size (e.g.
+ * the f16 images of quantized weights, with MI355X_MM_ACT_Q8_0 in `flags`), K a multiple of 256, more than 8 columns,
+ * count <= 64; anything else returns MI355X_ERR_UNSUPPORTED and the caller issues single calls.
+ * `flags`: MI355X_MM_* options common to all items; the items' epilogues carry MI355X_EPI_* only. */
+typedef struct mi355x_mul_mat_item {
+    const mi355x_tensor *   src0;
+    const mi355x_tensor *   dst;
+    const mi355x_epilogue * epi;     /* may be NULL */
+} mi355x_mul_mat_item;
+MI355X_API int    mi355x_mul_mat_group(const mi355x_mul_mat_item * items, int count, const mi355x_tensor * src1, int flags,
+                                       void * workspace, size_t workspace_size, void * stream);
+
 /* FLASH_ATTN_EXT --------------------------------------------------------------------------------------
  * ggml_compute_forward_flash_attn_ext_f16 (ggml/src/ggml-cpu/ops.cpp:6638-6851), max_bias = 0 and
  * logit_softcap = 0 (the only values whisper uses):

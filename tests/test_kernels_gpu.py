@@ -161,6 +161,48 @@ def test_mul_mat_epilogues(pkg, oracle, gpu):
         assert oracle.nmse(got, base + colbias[:, None]) <= 1e-6
 
 
+def test_mul_mat_group_equals_single_calls(pkg, oracle, gpu):
+    # three products over the same activations (the shape of a layer's Q, K, V projections) as one launch: same bits as
+    # three calls, each with its own epilogue and destination type
+    lib = pkg.kernels()
+    k, m, n = 512, 384, 200
+    x = rnd((n, k))
+    d_x = gpu.up(x)
+    tx = pkg.tensor(d_x, pkg.F32)
+    images, singles, grouped, items, keep = [], [], [], (pkg.MulMatItem * 3)(), []
+    specs = [(pkg.EPI_BIAS, torch.float32), (0, torch.float32), (pkg.EPI_BIAS | pkg.EPI_OUT_F16, torch.float16)]
+    for i, (flags, dt) in enumerate(specs):
+        blocks = oracle.quantize(pkg.Q5_0, rnd((m, k), 0.02))
+        d_b = gpu.up(blocks)
+        img = torch.empty((m, k), dtype=torch.float16, device=gpu.dev)
+        pkg.check(lib.mi355x_dequantize_row_f16(pkg.Q5_0, d_b.data_ptr(), img.data_ptr(), m * k, gpu.stream))
+        bias = gpu.up(rnd((m,), 0.5))
+        epi = pkg.Epilogue(); epi.flags, epi.scale, epi.bias = flags, 1.0, bias.data_ptr()
+        tw = pkg.tensor(img, pkg.F16)
+        y1, y2 = torch.zeros((n, m), dtype=dt, device=gpu.dev), torch.zeros((n, m), dtype=dt, device=gpu.dev)
+        t1, t2 = pkg.tensor(y1, pkg.F16 if dt == torch.float16 else pkg.F32), pkg.tensor(y2, pkg.F16 if dt == torch.float16 else pkg.F32)
+        keep += [d_b, img, bias, epi, tw, t1, t2]
+        images.append(tw); singles.append((y1, t1, epi)); grouped.append(y2)
+        items[i].src0, items[i].dst, items[i].epi = C.pointer(tw), C.pointer(t2), C.pointer(epi)
+    need = lib.mi355x_mul_mat_workspace_size(images[0], tx)
+    ws = torch.empty(max(need, 256), dtype=torch.uint8, device=gpu.dev)
+    for tw, (y1, t1, epi) in zip(images, singles):
+        one = pkg.Epilogue(); one.flags, one.scale, one.bias = epi.flags | pkg.MM_ACT_Q8_0, 1.0, epi.bias
+        pkg.check(lib.mi355x_mul_mat(tw, tx, t1, C.byref(one), ws.data_ptr(), need, gpu.stream))
+    rc = lib.mi355x_mul_mat_group(items, 3, tx, pkg.MM_ACT_Q8_0, ws.data_ptr(), need, gpu.stream)
+    pkg.check(rc, "mul_mat_group")
+    for (y1, _, _), y2 in zip(singles, grouped):
+        assert torch.equal(y1, y2)
+    assert float(grouped[1].abs().sum()) > 0
+    # shapes outside its one purpose are declined, not mis-computed: K = 96 is no multiple of 256
+    small = torch.zeros((m, 96), dtype=torch.float16, device=gpu.dev)
+    xs = torch.zeros((n, 96), dtype=torch.float32, device=gpu.dev)
+    it = (pkg.MulMatItem * 1)()
+    tws, tds = pkg.tensor(small, pkg.F16), pkg.tensor(grouped[1], pkg.F32)
+    it[0].src0, it[0].dst, it[0].epi = C.pointer(tws), C.pointer(tds), None
+    assert lib.mi355x_mul_mat_group(it, 1, pkg.tensor(xs, pkg.F32), 0, ws.data_ptr(), need, gpu.stream) == -1
+
+
 def test_mul_mat_rejects_bad_arguments(pkg, gpu):
     lib = pkg.kernels()
     d_w = torch.zeros(22 * 4, dtype=torch.uint8, device=gpu.dev)

@@ -191,13 +191,21 @@ struct graph_runner {
 
     ggml_tensor * node_at(int i) const { return i < g->n_nodes ? g->nodes[i] : nullptr; }
 
-    // ---- MUL_MAT and what can be folded behind it; returns the number of nodes consumed --------------
-    int run_mul_mat(int i, int & status) {
+    // ---- MUL_MAT and what can be folded behind it --------------------------------------------------------
+    struct mm_chain {
+        ggml_tensor *       mm;
+        const ggml_tensor * w, * x;
+        mi355x_epilogue     epi;
+        ggml_tensor *       out;       // tensor that receives the fused result
+        int                 used;      // nodes consumed, starting at the MUL_MAT
+    };
+
+    mm_chain plan_chain(int i) const {
         ggml_tensor * mm = g->nodes[i];
         const ggml_tensor * w = mm->src[0], * x = mm->src[1];
         mi355x_epilogue epi = { 0, 1.0f, nullptr, nullptr };
         ggml_tensor * last = mm;       // node whose value the fused kernel produces
-        ggml_tensor * out  = mm;       // tensor that receives it
+        ggml_tensor * out  = mm;
         int used = 1;
 
         if (ctx->fuse && mm->ne[2] == 1 && mm->ne[3] == 1 && ggml_is_contiguous(mm)) {
@@ -253,65 +261,139 @@ struct graph_runner {
                 epi = { 0, 1.0f, nullptr, nullptr }; out = mm; used = 1;
             }
         }
+        return { mm, w, x, epi, out, used };
+    }
 
-        mi355x_tensor vw = to_view(w), vx = to_view(x), vd = to_view(mm);
-        vd.data = out->data;
-        if (epi.flags & MI355X_EPI_OUT_F16) {
-            vd.type = MI355X_TYPE_F16;
-            vd.nb[0] = 2; vd.nb[1] = 2 * (size_t) mm->ne[0]; vd.nb[2] = vd.nb[1] * mm->ne[1]; vd.nb[3] = vd.nb[2];
+    // operand descriptors of a planned chain; a quantized weight matrix that meets many columns is replaced by its f16
+    // image, kept beside it in HBM (then MI355X_MM_ACT_Q8_0 goes into `mm_flags`)
+    struct mm_operands { mi355x_tensor vw, vx, vd; int mm_flags; const char * kernel_name; };
+    mm_operands describe(const mm_chain & c) const {
+        mm_operands o;
+        o.vw = to_view(c.w); o.vx = to_view(c.x); o.vd = to_view(c.mm);
+        o.vd.data = c.out->data;
+        if (c.epi.flags & MI355X_EPI_OUT_F16) {
+            o.vd.type = MI355X_TYPE_F16;
+            o.vd.nb[0] = 2; o.vd.nb[1] = 2 * (size_t) c.mm->ne[0]; o.vd.nb[2] = o.vd.nb[1] * c.mm->ne[1]; o.vd.nb[3] = o.vd.nb[2];
         }
-        const double batch = (double) mm->ne[2] * mm->ne[3];
-        const double flops = 2.0 * mm->ne[0] * mm->ne[1] * w->ne[0] * batch;
-        const double bytes = nbytes_of(w) + nbytes_of(x) + (double) ggml_nelements(mm) * ((epi.flags & MI355X_EPI_OUT_F16) ? 2 : 4) +
-                             ((epi.flags & MI355X_EPI_RESIDUAL) ? nbytes_of(mm) : 0.0);
-        const char * kernel_name = mi355x_mul_mat_kernel_name(&vw, &vx);
-        if (ctx->exact) epi.flags |= MI355X_MM_EXACT_ACT;
-        // a quantized weight matrix that meets many columns is multiplied through its f16 image, kept beside it in HBM
+        o.kernel_name = mi355x_mul_mat_kernel_name(&o.vw, &o.vx);
+        o.mm_flags = ctx->exact ? MI355X_MM_EXACT_ACT : 0;
+        const ggml_tensor * w = c.w;
         if (ctx->weight_images && ggml_is_quantized(w->type) && w->ne[2] == 1 && w->ne[3] == 1 && ggml_is_contiguous(w) && !w->view_src &&
             w->buffer && w->buffer->usage == GGML_BACKEND_BUFFER_USAGE_WEIGHTS && mi355x_buffer_is_ours(w->buffer) &&
-            strncmp(kernel_name, "mul_mat.gemm", 12) == 0) {
+            strncmp(o.kernel_name, "mul_mat.gemm", 12) == 0) {
             const void * image = ((mi355x_buffer_ctx *) w->buffer->context)->weight_image(w, ctx->stream);
             if (image) {
-                vw.data = (void *) image; vw.type = MI355X_TYPE_F16;
-                vw.nb[0] = 2; vw.nb[1] = 2 * (size_t) w->ne[0]; vw.nb[2] = vw.nb[1] * (size_t) w->ne[1]; vw.nb[3] = vw.nb[2];
-                epi.flags |= MI355X_MM_ACT_Q8_0;
+                o.vw.data = (void *) image; o.vw.type = MI355X_TYPE_F16;
+                o.vw.nb[0] = 2; o.vw.nb[1] = 2 * (size_t) w->ne[0]; o.vw.nb[2] = o.vw.nb[1] * (size_t) w->ne[1]; o.vw.nb[3] = o.vw.nb[2];
+                o.mm_flags |= MI355X_MM_ACT_Q8_0;
             }
         }
-        // the GEMM first brings src1 to f16 (rounded to Q8_0 on the way when the weights are quantized) in the workspace;
-        // consecutive MUL_MATs over the same activations (Q, K, V projections) share that copy
-        const size_t need = mi355x_mul_mat_workspace_size(&vw, &vx);
-        if (need) {
-            if (!ctx->reserve_workspace(need)) { status = MI355X_ERR_WORKSPACE; return used; }
-            if (x->type == GGML_TYPE_F32) {
-                const int mode = (ggml_is_quantized(w->type) && !ctx->exact) ? 1 : 0;       // 1: rounded to Q8_0
-                const bool hit = ctx->ws_x == x->data && ctx->ws_x_mode == mode && memcmp(ctx->ws_x_ne, x->ne, sizeof(x->ne)) == 0 &&
-                                 memcmp(ctx->ws_x_nb, x->nb, sizeof(x->nb)) == 0;
-                if (hit) epi.flags |= MI355X_MM_WS_READY;
-                ctx->ws_x = x->data; ctx->ws_x_mode = mode; memcpy(ctx->ws_x_ne, x->ne, sizeof(x->ne)); memcpy(ctx->ws_x_nb, x->nb, sizeof(x->nb));
-                cached_x = x;
-            }
+        return o;
+    }
+
+    // The GEMM first brings src1 to f16 (rounded to Q8_0 on the way when the weights are quantized) in the workspace;
+    // consecutive MUL_MATs over the same activations share that copy.  Runs (and times) the conversion when the workspace
+    // does not hold it yet; returns the MM flags to add (WS_READY), or -1 with `status` set.
+    int prepare_src1(const mm_chain & c, const mm_operands & o, size_t need, int & status) {
+        if (!need) return 0;
+        if (!ctx->reserve_workspace(need)) { status = MI355X_ERR_WORKSPACE; return -1; }
+        const ggml_tensor * x = c.x;
+        if (x->type != GGML_TYPE_F32) return 0;
+        const int mode = (ggml_is_quantized(c.w->type) && !ctx->exact) ? 1 : 0;       // 1: rounded to Q8_0
+        const bool hit = ctx->ws_x == x->data && ctx->ws_x_mode == mode && memcmp(ctx->ws_x_ne, x->ne, sizeof(x->ne)) == 0 &&
+                         memcmp(ctx->ws_x_nb, x->nb, sizeof(x->nb)) == 0;
+        ctx->ws_x = x->data; ctx->ws_x_mode = mode; memcpy(ctx->ws_x_ne, x->ne, sizeof(x->ne)); memcpy(ctx->ws_x_nb, x->nb, sizeof(x->nb));
+        cached_x = x;
+        if (!hit) {
+            mi355x_epilogue prep = c.epi;                 // same call as the product itself, stopped after the conversion
+            prep.flags |= o.mm_flags | MI355X_MM_PREPARE_ONLY;
+            launch_scope ls(ctx, "mul_mat.src1_to_f16", nbytes_of(x) * 1.5, 0.0);
+            status = mi355x_mul_mat(&o.vw, &o.vx, &o.vd, &prep, ctx->ws, ctx->ws_size, ctx->stream);
+            if (status != MI355X_OK) return -1;
         }
+        return MI355X_MM_WS_READY;
+    }
+
+    static double chain_flops(const mm_chain & c) { return 2.0 * c.mm->ne[0] * c.mm->ne[1] * c.w->ne[0] * (double) c.mm->ne[2] * c.mm->ne[3]; }
+    static double chain_bytes(const mm_chain & c) {
+        return nbytes_of(c.w) + nbytes_of(c.x) + (double) ggml_nelements(c.mm) * ((c.epi.flags & MI355X_EPI_OUT_F16) ? 2 : 4) +
+               ((c.epi.flags & MI355X_EPI_RESIDUAL) ? nbytes_of(c.mm) : 0.0);
+    }
+
+    // Products that follow each other over the same activations with weights of one shape (Q, K, V of a layer; the
+    // cross-attention K / V of all decoder layers) go out as one launch.  Returns the nodes consumed, 0 if no group formed.
+    int run_mul_mat_group(int i, const mm_chain & first, const mm_operands & o0, int & status) {
+        if (!ctx->fuse || o0.vw.type != MI355X_TYPE_F16 || strncmp(o0.kernel_name, "mul_mat.gemm", 12) != 0) return 0;
+        if (first.mm->ne[2] != 1 || first.mm->ne[3] != 1 || first.w->ne[0] % 256 != 0) return 0;
+        std::vector<mm_chain>    chains{ first };
+        std::vector<mm_operands> ops{ o0 };
+        int end = i + first.used;                       // first node after the group
+        while ((int) chains.size() < 64) {
+            int j = end;
+            while (node_at(j) && (is_view_op(node_at(j)->op) || ggml_is_empty(node_at(j)))) ++j;
+            ggml_tensor * n = node_at(j);
+            if (!n || n->op != GGML_OP_MUL_MAT || n->src[1] != first.x || n->src[0]->type != first.w->type ||
+                !ggml_are_same_shape(n->src[0], first.w) || !ggml_are_same_shape(n, first.mm)) break;
+            mm_chain c = plan_chain(j);
+            mm_operands o = describe(c);
+            if (o.vw.type != MI355X_TYPE_F16 || o.mm_flags != o0.mm_flags || o.vw.nb[1] != o0.vw.nb[1]) break;
+            // nothing in the group may read what another member writes
+            bool clash = false;
+            for (const mm_chain & p : chains) {
+                clash = clash || ranges_overlap(c.out, p.out) || ranges_overlap(p.out, c.w);
+                for (int k = j; k < j + c.used; ++k)
+                    for (int s = 0; s < GGML_MAX_SRC; ++s)
+                        if (g->nodes[k]->src[s] && !is_view_op(g->nodes[k]->op)) clash = clash || ranges_overlap(p.out, g->nodes[k]->src[s]);
+            }
+            if (clash) break;
+            chains.push_back(c); ops.push_back(o);
+            end = j + c.used;
+        }
+        if (chains.size() < 2) return 0;
+
+        const size_t need = mi355x_mul_mat_workspace_size(&o0.vw, &o0.vx);
+        const int ready = prepare_src1(first, o0, need, status);
+        if (ready < 0) return end - i;
+        std::vector<mi355x_mul_mat_item> items(chains.size());
+        double flops = 0.0, bytes = 0.0;
+        for (size_t k = 0; k < chains.size(); ++k) {
+            items[k] = { &ops[k].vw, &ops[k].vd, &chains[k].epi };
+            flops += chain_flops(chains[k]); bytes += chain_bytes(chains[k]) - (k ? nbytes_of(first.x) : 0.0);
+        }
+        int rc;
+        {
+            launch_scope ls(ctx, "mul_mat.gemm_group", bytes, flops);
+            rc = mi355x_mul_mat_group(items.data(), (int) items.size(), &o0.vx, o0.mm_flags | ready, ctx->ws, ctx->ws_size, ctx->stream);
+        }
+        if (rc == MI355X_ERR_UNSUPPORTED) return 0;     // the single-product path takes them one by one
+        status = rc;
+        if (ctx->debug) GGML_LOG_INFO("ggml-mi355x: mul_mat.gemm_group of %zu starting at %s, %d nodes\n", chains.size(), first.mm->name, end - i);
+        for (const mm_chain & c : chains) note_write(c.out);
+        return end - i;
+    }
+
+    // returns the number of nodes consumed
+    int run_mul_mat(int i, int & status) {
+        const mm_chain c = plan_chain(i);
+        mm_operands o = describe(c);
+        if (const int grouped = run_mul_mat_group(i, c, o, status)) return grouped;
+
+        mi355x_epilogue epi = c.epi;
+        epi.flags |= o.mm_flags;
+        const size_t need = mi355x_mul_mat_workspace_size(&o.vw, &o.vx);
+        const int ready = prepare_src1(c, o, need, status);
+        if (ready < 0) return c.used;
+        epi.flags |= ready;
         if (ctx->debug) {
-            GGML_LOG_INFO("ggml-mi355x: %s %s [%lld x %lld x %lld] folds %d nodes, flags 0x%x\n", kernel_name, mm->name,
-                          (long long) mm->ne[0], (long long) mm->ne[1], (long long) w->ne[0], used, epi.flags);
-        }
-        // the activation conversion is a kernel of its own: run (and time) it apart from the product
-        if (need && x->type == GGML_TYPE_F32 && !(epi.flags & MI355X_MM_WS_READY)) {
-            mi355x_epilogue prep = epi;
-            prep.flags |= MI355X_MM_PREPARE_ONLY;
-            {
-                launch_scope ls(ctx, "mul_mat.src1_to_f16", nbytes_of(x) * 1.5, 0.0);
-                status = mi355x_mul_mat(&vw, &vx, &vd, &prep, ctx->ws, ctx->ws_size, ctx->stream);
-            }
-            if (status != MI355X_OK) return used;
-            epi.flags |= MI355X_MM_WS_READY;
+            GGML_LOG_INFO("ggml-mi355x: %s %s [%lld x %lld x %lld] folds %d nodes, flags 0x%x\n", o.kernel_name, c.mm->name,
+                          (long long) c.mm->ne[0], (long long) c.mm->ne[1], (long long) c.w->ne[0], c.used, epi.flags);
         }
         {
-            launch_scope ls(ctx, kernel_name, bytes, flops);
-            status = mi355x_mul_mat(&vw, &vx, &vd, epi.flags ? &epi : nullptr, ctx->ws, ctx->ws_size, ctx->stream);
+            launch_scope ls(ctx, o.kernel_name, chain_bytes(c), chain_flops(c));
+            status = mi355x_mul_mat(&o.vw, &o.vx, &o.vd, epi.flags ? &epi : nullptr, ctx->ws, ctx->ws_size, ctx->stream);
         }
-        note_write(out);
-        return used;
+        note_write(c.out);
+        return c.used;
     }
 
     // ---- NORM [-> MUL(w) -> ADD(b)] ---------------------------------------------------------------------

@@ -241,7 +241,8 @@ __global__ void k_x_to_f16(const char * __restrict__ x, half_t * __restrict__ ou
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 template <int TI, int TJ, int S, bool KTAIL, bool FULL>     // KTAIL: K is not a multiple of 64 (but of 8); FULL: K / 64 is a multiple of S
-__global__ void __launch_bounds__(256) k_gemm_f16(mm_args a, int tiles_m, int tiles_n) {
+__device__ __forceinline__ void gemm_f16_tile(const mm_args & a, int tiles_m, int tiles_n, const char * wb, const char * xb, char * db,
+                                              const epi_args & epi, int64_t batch_off, int64_t d_nb1) {
     constexpr int BN = 64 * TI, BM = 64 * TJ;
     constexpr int XR = BN / 32, WR = BM / 32;          // 16-byte pieces per thread and step
     extern __shared__ __attribute__((aligned(16))) char smem[];
@@ -255,11 +256,6 @@ __global__ void __launch_bounds__(256) k_gemm_f16(mm_args a, int tiles_m, int ti
     const int tile = xcd * q + (xcd < r ? xcd : r) + blockIdx.x / 8;
     const int64_t m0 = (int64_t)(tile % tiles_m) * BM;
     const int64_t n0 = (int64_t)(tile / tiles_m) * BN;
-    const int64_t b2 = blockIdx.y % a.ne12, b3 = blockIdx.y / a.ne12;
-
-    const char * wb = a.w + (b2 / a.r2) * a.w_nb2 + (b3 / a.r3) * a.w_nb3;
-    const char * xb = a.x + b2 * a.x_nb2 + b3 * a.x_nb3;
-    char *       db = a.d + b2 * a.d_nb2 + b3 * a.d_nb3;
 
     const int tid = threadIdx.x;
     const int lc = tid & 7, lr = tid >> 3;             // piece column (8 halves) and first row of this thread
@@ -395,7 +391,6 @@ __global__ void __launch_bounds__(256) k_gemm_f16(mm_args a, int tiles_m, int ti
     }
 
     // accumulator register e of a 32x32 patch: row (= n) 8*(e/4) + 4*g + e%4, column (= m) lane%32
-    const int64_t batch_off = b2 * a.d_nb2 + b3 * a.d_nb3;
 #pragma unroll
     for (int i = 0; i < TI; ++i) {
         int64_t n[16];
@@ -403,8 +398,30 @@ __global__ void __launch_bounds__(256) k_gemm_f16(mm_args a, int tiles_m, int ti
         for (int e = 0; e < 16; ++e) n[e] = n0 + wn + 32 * i + 8 * (e >> 2) + 4 * g + (e & 3);
 #pragma unroll
         for (int j = 0; j < TJ; ++j)
-            patch_epilogue(acc[i][j], a.e, db, batch_off, a.d_nb1, m0 + wmo + 32 * j + l32, a.M, n, a.N);
+            patch_epilogue(acc[i][j], epi, db, batch_off, d_nb1, m0 + wmo + 32 * j + l32, a.M, n, a.N);
     }
+}
+
+template <int TI, int TJ, int S, bool KTAIL, bool FULL>
+__global__ void __launch_bounds__(256) k_gemm_f16(mm_args a, int tiles_m, int tiles_n) {
+    const int64_t b2 = blockIdx.y % a.ne12, b3 = blockIdx.y / a.ne12;
+    gemm_f16_tile<TI, TJ, S, KTAIL, FULL>(a, tiles_m, tiles_n, a.w + (b2 / a.r2) * a.w_nb2 + (b3 / a.r3) * a.w_nb3, a.x + b2 * a.x_nb2 + b3 * a.x_nb3,
+                                          a.d + b2 * a.d_nb2 + b3 * a.d_nb3, a.e, b2 * a.d_nb2 + b3 * a.d_nb3, a.d_nb1);
+}
+
+// Several products over the same src1 in one launch (the Q, K and V projections of a layer; the cross-attention K and V
+// of all decoder layers): blockIdx.y picks the weights, the destination and the epilogue.  One launch of 3 x 120 or
+// 64 x 120 tiles fills 256 CUs where 120 tiles at a time leave half of them idle.
+#define MM_GROUP_MAX 64
+struct mm_group_entry { const char * w; char * d; const float * bias; const char * residual; int64_t d_nb1; int flags; float scale; };
+struct mm_group { mm_group_entry e[MM_GROUP_MAX]; };
+
+template <int TI, int TJ, int S>
+__global__ void __launch_bounds__(256) k_gemm_f16_group(mm_args a, int tiles_m, int tiles_n, mm_group grp) {
+    const mm_group_entry & ge = grp.e[blockIdx.y];
+    epi_args e;
+    e.flags = ge.flags; e.scale = ge.scale; e.bias = ge.bias; e.residual = ge.residual; e.gelu = a.e.gelu;
+    gemm_f16_tile<TI, TJ, S, false, true>(a, tiles_m, tiles_n, ge.w, a.x, ge.d, e, 0, ge.d_nb1);
 }
 
 template <int TI, int TJ, int S, bool KTAIL, bool FULL>
@@ -432,6 +449,24 @@ static int launch_gemm_f16(const mm_args & a, hipStream_t st) {
     if (kt % 4 == 0) return launch_gemm_f16_k<TI, TJ, 4, false, true>(a, st);
     if (kt % 2 == 0) return launch_gemm_f16_k<TI, TJ, 2, false, true>(a, st);
     return launch_gemm_f16_k<TI, TJ, 4, false, false>(a, st);
+}
+
+template <int TI, int TJ>
+static int launch_gemm_f16_group(const mm_args & a, const mm_group & grp, int count, hipStream_t st) {
+    constexpr int BN = 64 * TI, BM = 64 * TJ;
+    constexpr size_t lds = (size_t) 2 * (BN + BM) * GB_LD * sizeof(half_t);
+    static bool configured[64];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return MI355X_ERR_HIP;
+    if (!configured[dev]) {
+        if (hipFuncSetAttribute((const void *) k_gemm_f16_group<TI, TJ, 4>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds) != hipSuccess) return MI355X_ERR_HIP;
+        configured[dev] = true;
+    }
+    const int64_t tm = (a.M + BM - 1) / BM, tn = (a.N + BN - 1) / BN;
+    if (tm * tn > 0x7fffffff) return MI355X_ERR_UNSUPPORTED;
+    dim3 grid((unsigned)(tm * tn), (unsigned) count);
+    k_gemm_f16_group<TI, TJ, 4><<<grid, 256, lds, st>>>(a, (int) tm, (int) tn, grp);
+    return launch_status();
 }
 
 // tile shape: the largest whose grid still covers the 256 CUs about twice
@@ -774,6 +809,61 @@ static size_t w16_bytes(const mi355x_tensor * src0) {
 extern "C" size_t mi355x_mul_mat_workspace_size(const mi355x_tensor * src0, const mi355x_tensor * src1) {
     if (!src0 || !src1 || mm_path(src0, src1) != MM_GEMM) return 0;
     return x16_bytes(src1) + w16_bytes(src0);
+}
+
+extern "C" int mi355x_mul_mat_group(const mi355x_mul_mat_item * items, int count, const mi355x_tensor * src1, int flags,
+                                    void * workspace, size_t workspace_size, void * stream) {
+    if (!items || !src1 || count < 1) return MI355X_ERR_INVALID;
+    if (count > MM_GROUP_MAX) return MI355X_ERR_UNSUPPORTED;
+    const mi355x_tensor * w0 = items[0].src0;
+    if (!w0 || !items[0].dst) return MI355X_ERR_INVALID;
+    // one shape of problem only: dense f16 weights (or weight images), 2-d, K a multiple of 256, the MFMA GEMM path
+    if (w0->type != MI355X_TYPE_F16 || (src1->type != MI355X_TYPE_F32 && src1->type != MI355X_TYPE_F16)) return MI355X_ERR_UNSUPPORTED;
+    if (src1->ne[2] != 1 || src1->ne[3] != 1 || w0->ne[2] != 1 || w0->ne[3] != 1) return MI355X_ERR_UNSUPPORTED;
+    if (mm_path(w0, src1) != MM_GEMM || w0->ne[0] % (4 * GB_K) != 0) return MI355X_ERR_UNSUPPORTED;
+    mm_args a;
+    a.K = w0->ne[0]; a.M = w0->ne[1]; a.N = src1->ne[1];
+    if (src1->ne[0] != a.K || w0->nb[0] != 2 || src1->nb[0] != type_size(src1->type)) return MI355X_ERR_INVALID;
+    if (a.M == 0 || a.N == 0) return MI355X_OK;
+    mm_group grp;
+    bool any_gelu = false;
+    for (int i = 0; i < count; ++i) {
+        const mi355x_tensor * w = items[i].src0, * d = items[i].dst;
+        const mi355x_epilogue * e = items[i].epi;
+        if (!w || !d) return MI355X_ERR_INVALID;
+        if (w->type != MI355X_TYPE_F16 || w->ne[0] != a.K || w->ne[1] != a.M || w->ne[2] != 1 || w->ne[3] != 1 || w->nb[0] != 2 || w->nb[1] != w0->nb[1] || !aligned16(w)) return MI355X_ERR_UNSUPPORTED;
+        const int ef = e ? (e->flags & 63) : 0;
+        const int td = (ef & MI355X_EPI_OUT_F16) ? MI355X_TYPE_F16 : MI355X_TYPE_F32;
+        if (d->type != td || d->ne[0] != a.M || d->ne[1] != a.N || d->ne[2] != 1 || d->ne[3] != 1 || d->nb[0] != type_size(td) || d->nb[1] % 4 != 0) return MI355X_ERR_UNSUPPORTED;
+        if ((ef & (MI355X_EPI_BIAS | MI355X_EPI_BIAS_COL)) && !e->bias) return MI355X_ERR_INVALID;
+        if ((ef & MI355X_EPI_BIAS) && (ef & MI355X_EPI_BIAS_COL)) return MI355X_ERR_INVALID;
+        if ((ef & MI355X_EPI_RESIDUAL) && (!e->residual || (ef & MI355X_EPI_OUT_F16))) return MI355X_ERR_INVALID;
+        any_gelu = any_gelu || (ef & MI355X_EPI_GELU);
+        grp.e[i] = { (const char *) w->data, (char *) d->data, e ? (const float *) e->bias : nullptr, e ? (const char *) e->residual : nullptr, (int64_t) d->nb[1], ef, e ? e->scale : 1.0f };
+    }
+    a.w = (const char *) w0->data; a.x = (const char *) src1->data; a.d = (char *) items[0].dst->data;
+    a.w_nb1 = w0->nb[1]; a.w_nb2 = a.w_nb3 = 0;
+    a.x_nb1 = src1->nb[1]; a.x_nb2 = a.x_nb3 = 0;
+    a.d_nb1 = items[0].dst->nb[1]; a.d_nb2 = a.d_nb3 = 0;
+    a.ne12 = a.ne13 = a.r2 = a.r3 = 1;
+    a.e.flags = 0; a.e.scale = 1.0f; a.e.bias = nullptr; a.e.residual = nullptr; a.e.gelu = nullptr;
+    if (any_gelu && !(a.e.gelu = gelu_table_device())) return MI355X_ERR_HIP;
+    hipStream_t st = (hipStream_t) stream;
+
+    const size_t xbytes = x16_bytes(src1);
+    if (xbytes) {
+        if (!workspace || workspace_size < xbytes || (uintptr_t) workspace % 256 != 0) return MI355X_ERR_WORKSPACE;
+        if (!(flags & MI355X_MM_WS_READY)) {
+            dim3 qgrid((unsigned)((a.K / 4 * a.N + 255) / 256), 1);
+            const bool q8 = (flags & MI355X_MM_ACT_Q8_0) && !(flags & MI355X_MM_EXACT_ACT);
+            if (q8) k_x_to_f16<true ><<<qgrid, 256, 0, st>>>(a.x, (half_t *) workspace, a.K, a.N, a.x_nb1, 0, 1, 0, 0);
+            else    k_x_to_f16<false><<<qgrid, 256, 0, st>>>(a.x, (half_t *) workspace, a.K, a.N, a.x_nb1, 0, 1, 0, 0);
+        }
+        a.x = (const char *) workspace; a.x_nb1 = a.K * 2;
+    }
+    if (flags & MI355X_MM_PREPARE_ONLY) return launch_status();
+    const int64_t blocks22 = ((a.N + 127) / 128) * ((a.M + 127) / 128) * count;
+    return blocks22 >= 300 ? launch_gemm_f16_group<2, 2>(a, grp, count, st) : launch_gemm_f16_group<2, 1>(a, grp, count, st);
 }
 
 extern "C" int mi355x_dequantize_row_f16(int type, const void * src, void * dst, int64_t k, void * stream) {
