@@ -67,6 +67,17 @@ def test_every_node_of_the_whisper_graphs(harness, models, key):
     assert {"FLASH_ATTN_EXT", "NORM", "GET_ROWS", "IM2COL"} <= ops
 
 
+def test_default_attention_graphs_without_flash_attn(harness, models):
+    # whisper.cpp's default (flash_attn = false, src/whisper.cpp:3620): KQ and KQV as batched MUL_MATs over permuted
+    # operands, SOFT_MAX with an f32 mask, strided copies into the V cache
+    rc, rows = run_harness(harness, ["model", "--model", models[("base", "q5_0")], "--steps", "8", "--no-flash-attn"], timeout=900)
+    s = rows[-1]
+    assert rc == 0 and s["pass"] and s["ids_identical"] == 8 and s["worst_logits_nmse"] <= 1e-3, s
+    rc, rows = run_harness(harness, ["verify", "--model", models[("base", "q5_0")], "--steps", "2", "--no-flash-attn"], timeout=1200)
+    assert rc == 0 and rows[-1]["pass"], [r for r in rows if "bad_node" in r]
+    assert "SOFT_MAX" in {r["op"] for r in rows if "phase" in r}
+
+
 @pytest.mark.parametrize("key,steps", [(("base", "q5_0"), 32), (("base", "q8_0"), 32), (("base", "f16"), 32),
                                        (("large-v3", "q5_0"), 32), (("large-v3-turbo", "q8_0"), 32)])
 def test_whole_model_logits_and_greedy_ids(harness, models, key, steps):

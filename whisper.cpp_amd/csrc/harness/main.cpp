@@ -343,10 +343,12 @@ static int cmd_gen(const args & a) {
 // whisper contexts
 // ---------------------------------------------------------------------------------------------------------------
 
+static bool g_flash_attn = true;   // --no-flash-attn: whisper.cpp's default graphs (KQ MUL_MAT, SOFT_MAX, KQV MUL_MAT; src/whisper.cpp:3620)
+
 static whisper_context * open_model(const std::string & path, bool use_gpu) {
     whisper_context_params cp = whisper_context_default_params();
     cp.use_gpu    = use_gpu;
-    cp.flash_attn = true;      // the FLASH_ATTN_EXT graphs are the ones under test (default is off, src/whisper.cpp:3620)
+    cp.flash_attn = g_flash_attn;
     return whisper_init_from_file_with_params(path.c_str(), cp);
 }
 
@@ -622,6 +624,7 @@ int main(int argc, char ** argv) {
     whisper_log_set(quiet_log, nullptr);
     const std::string cmd = argv[1];
     const args a = parse_args(argc, argv, 2);
+    if (a.has("no-flash-attn")) g_flash_attn = false;
     if (cmd == "info")  return cmd_info(a);
     if (cmd == "gen")   return cmd_gen(a);
     if (cmd == "selftest") return cmd_selftest(a);
