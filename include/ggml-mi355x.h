@@ -53,8 +53,12 @@ GGML_BACKEND_API int                ggml_backend_score(void);
  * "profile" (0/1: bracket every kernel with HIP events on the backend's stream, default 0),
  * "exact" (0/1, default 0: 0 reproduces the two roundings that the reference's CPU backend applies — Q8_0-rounded
  * activations in front of quantized MUL_MAT, f16 key-by-key V accumulation in FLASH_ATTN_EXT; 1 keeps f16 activations
- * and f32 accumulators, which is closer to exact arithmetic and further from the reference).
- * The environment variables GGML_MI355X_FUSE, GGML_MI355X_PROFILE and GGML_MI355X_EXACT give the initial values.
+ * and f32 accumulators, which is closer to exact arithmetic and further from the reference),
+ * "fa_packed" (0/1, default 0: 1 lets FLASH_ATTN_EXT over more than 8 queries accumulate V with f16 fused multiply-adds,
+ * the arithmetic of the reference's Arm fp16 build, simd-mappings.h:67-78, instead of the x86 build's f32 fma + f16
+ * store: a third of the accumulation work, about 1e-7 NMSE away).
+ * The environment variables GGML_MI355X_FUSE, GGML_MI355X_PROFILE, GGML_MI355X_EXACT and GGML_MI355X_FA_PACKED give the
+ * initial values.
  * backend == NULL addresses every live MI355X backend of the process (a host such as whisper.cpp keeps its
  * backends private). */
 typedef int (*ggml_backend_mi355x_set_option_t)(ggml_backend_t backend, const char * name, int value);

@@ -67,6 +67,18 @@ def test_every_node_of_the_whisper_graphs(harness, models, key):
     assert {"FLASH_ATTN_EXT", "NORM", "GET_ROWS", "IM2COL"} <= ops
 
 
+def test_packed_f16_attention_option_stays_within_the_bounds(harness, models):
+    # GGML_MI355X_FA_PACKED=1: encoder / prompt attention accumulates with f16 fused multiply-adds (the reference's Arm
+    # arithmetic); against the x86 CPU backend it must still meet the per-op and whole-model bounds
+    env = {"GGML_MI355X_FA_PACKED": "1"}
+    rc, rows = run_harness(harness, ["ops", "--quick", "--reps", "0", "--filter", "flash_attn"], env=env, timeout=900)
+    cases = [r for r in rows if "case" in r]
+    assert rc == 0 and cases and all(r["pass"] for r in cases), [r for r in cases if not r["pass"]]
+    rc, rows = run_harness(harness, ["model", "--model", models[("base", "q5_0")], "--steps", "16"], env=env, timeout=900)
+    s = rows[-1]
+    assert rc == 0 and s["pass"] and s["ids_identical"] == 16 and s["worst_logits_nmse"] <= 1e-3, s
+
+
 def test_default_attention_graphs_without_flash_attn(harness, models):
     # whisper.cpp's default (flash_attn = false, src/whisper.cpp:3620): KQ and KQV as batched MUL_MATs over permuted
     # operands, SOFT_MAX with an f32 mask, strided copies into the V cache

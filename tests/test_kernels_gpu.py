@@ -265,6 +265,24 @@ def test_flash_attn_reference_faithful(pkg, oracle, gpu, case):
     assert oracle.nmse(got, want) <= 1e-6      # same key order, same f16 accumulator: only exp() and dot-product ulps differ
 
 
+@pytest.mark.parametrize("case", [dict(H=2, N=70, KV=100), dict(H=3, N=200, KV=1536, flat=True, pad_from=1500), dict(H=2, N=100, KV=100, mask="causal")])
+def test_flash_attn_f16_fma_mode(pkg, oracle, gpu, case):
+    H, N, KV = case["H"], case["N"], case["KV"]
+    q, kb, vb = _attention_inputs(oracle, H, N, KV, case.get("flat", False), case.get("pad_from"))
+    mask = None
+    if "mask" in case:
+        m = np.full((-(-N // 64) * 64, KV), -np.inf, dtype=np.float32)
+        for r in range(N):
+            m[r, : KV - N + r + 1] = 0.0
+        mask = oracle.f32_to_f16_bits(m)
+    got, name = run_fa(pkg, gpu, q, kb, vb, mask, 0.125, pkg.FA_F16_PACKED)
+    assert name == "flash_attn.seq_tile_packed"
+    arm = oracle.flash_attn_ext(q, kb, vb, None if mask is None else mask[:N], 0.125, f16_fma=True)
+    x86 = oracle.flash_attn_ext(q, kb, vb, None if mask is None else mask[:N], 0.125)
+    assert oracle.nmse(got, arm) <= 1e-6       # the same f16 fma chain; exp() and dot-product ulps differ
+    assert oracle.nmse(got, x86) <= 5e-4       # north-star per-op bound against the arithmetic of the CPU build at hand
+
+
 def test_flash_attn_f32_mode_matches_float64(pkg, oracle, gpu):
     q, kb, vb = _attention_inputs(oracle, 2, 30, 300, flat=True, pad_from=280)
     got, name = run_fa(pkg, gpu, q, kb, vb, None, 0.125, pkg.FA_F32)

@@ -317,6 +317,7 @@ static ggml_backend_t device_init_backend(ggml_backend_dev_t dev, const char *) 
     ctx->fuse    = env_flag("GGML_MI355X_FUSE", true);
     ctx->profile = env_flag("GGML_MI355X_PROFILE", false);
     ctx->exact   = env_flag("GGML_MI355X_EXACT", false);
+    ctx->fa_packed = env_flag("GGML_MI355X_FA_PACKED", false);
     ctx->weight_images = env_flag("GGML_MI355X_WEIGHT_IMAGES", true);
     ctx->debug   = env_flag("GGML_MI355X_DEBUG", false);
     // default priority, blocking with respect to the null stream used by the buffer-level copies
@@ -399,12 +400,14 @@ static void ctx_synchronize(mi355x_backend_ctx * ctx) {
 static int set_option(ggml_backend_t backend, const char * name, int value) {
     if (!name || (backend && !ggml_backend_is_mi355x(backend))) return -1;
     const bool is_fuse = strcmp(name, "fuse") == 0, is_profile = strcmp(name, "profile") == 0, is_exact = strcmp(name, "exact") == 0;
-    if (!is_fuse && !is_profile && !is_exact) return -1;
+    const bool is_packed = strcmp(name, "fa_packed") == 0;
+    if (!is_fuse && !is_profile && !is_exact && !is_packed) return -1;
     std::lock_guard<std::mutex> lock(g_live_mutex);
     for (mi355x_backend_ctx * ctx : g_live) {
         if (backend && ctx != (mi355x_backend_ctx *) backend->context) continue;
         if (is_fuse) ctx->fuse = value != 0;
         else if (is_exact) ctx->exact = value != 0;
+        else if (is_packed) ctx->fa_packed = value != 0;
         else { ctx_synchronize(ctx); ctx->profile = value != 0; }
     }
     return 0;

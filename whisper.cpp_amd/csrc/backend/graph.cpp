@@ -514,7 +514,7 @@ struct graph_runner {
                 if (m) vm = to_view(m);
                 const double flops = 4.0 * s0->ne[1] * k->ne[1] * 64.0 * s0->ne[2] * s0->ne[3];
                 const double bytes = (double) ggml_nelements(s0) * 4 + 2.0 * (double) k->ne[0] * k->ne[1] * k->ne[2] * k->ne[3] * 2 + nbytes_of(n);
-                const int mode = ctx->exact ? MI355X_FA_F32 : MI355X_FA_F16_SEQ;
+                const int mode = ctx->exact ? MI355X_FA_F32 : ctx->fa_packed ? MI355X_FA_F16_PACKED : MI355X_FA_F16_SEQ;
                 launch_scope ls(ctx, mi355x_flash_attn_ext_kernel_name(&vq, &vk, mode), bytes, flops);
                 status = mi355x_flash_attn_ext(&vq, &vk, &vv, m ? &vm : nullptr, &vd, scale, mode, nullptr, 0, ctx->stream);
                 return 1;

@@ -343,6 +343,12 @@ __device__ __forceinline__ float exp_neg(float x) {
 
 typedef const uint32_t __attribute__((address_space(4))) * const_u32_ptr;   // read-only data: uniform loads become scalar loads
 
+// PACKED (MI355X_FA_F16_PACKED): the accumulation is the f16 fused multiply-add of the reference's Arm fp16 build instead
+// (GGML_F16_VEC_FMA = vfmaq_f16 on the factor converted to f16, GGML_F16_VEC_MUL for the rescale; simd-mappings.h:67-78,
+// vec.h:180-197, 295-310): one v_pk_fma_f16 per two accumulators.  A third of the arithmetic; LDS could not deliver the
+// V operands that fast as broadcast reads, so a wavefront holds the tile's V slice distributed over its lanes (lane =
+// key) and hands each key's eight registers to the packed fma as scalar operands through v_readlane.
+template <bool PACKED>
 __global__ void __launch_bounds__(256) k_fattn_seq_tile(fa_args a) {
     __shared__ __attribute__((aligned(16))) half_t q_s[T_Q * T_LDH];
     __shared__ __attribute__((aligned(16))) half_t k_s[T_KV * T_LDH];
@@ -459,6 +465,10 @@ __global__ void __launch_bounds__(256) k_fattn_seq_tile(fa_args a) {
                 M = raised ? s : M;
                 P *= ms; A = A * ms + vs;
                 sv[i] = raised ? -ex : ex;                 // -0.0 keeps the sign
+                if (PACKED) {                              // the factor as the f16 pair the packed fma takes
+                    const uint32_t hb = f2h_bits(sv[i]);
+                    sv[i] = __uint_as_float(hb | (hb << 16));
+                }
             }
 #pragma unroll
             for (int i = 0; i < 4; ++i) fp[i] = make_float4(sv[4*i], sv[4*i+1], sv[4*i+2], sv[4*i+3]);
@@ -476,7 +486,51 @@ __global__ void __launch_bounds__(256) k_fattn_seq_tile(fa_args a) {
         __syncthreads();
 
         // ---- the sequential f16 chains over this tile's keys -----------------------------------------------------------------------------
-        {
+        if constexpr (PACKED) {
+            const int nk = (int)(a.KV - key0 < T_KV ? a.KV - key0 : T_KV);       // uniform
+            const float4 * fp = (const float4 *)(f_s + lane * T_LDF);
+            uint32_t vk[8];                                                       // V[key = lane][d0 .. d0 + 15]
+            {
+                const u32x4 * vr = (const u32x4 *)(v_s + lane * FA_D + d0);
+                const u32x4 lo = vr[0], hi = vr[1];
+                vk[0] = lo.x; vk[1] = lo.y; vk[2] = lo.z; vk[3] = lo.w; vk[4] = hi.x; vk[5] = hi.y; vk[6] = hi.z; vk[7] = hi.w;
+            }
+            float4 fnext = fp[0];
+            for (int k4 = 0; k4 < nk; k4 += 4) {
+                const float4 f4 = fnext;
+                if (k4 + 4 < nk) fnext = fp[(k4 >> 2) + 1];
+                const uint32_t fk[4] = { __float_as_uint(f4.x), __float_as_uint(f4.y), __float_as_uint(f4.z), __float_as_uint(f4.w) };
+                const bool any_raised = __any((fk[0] | fk[1] | fk[2] | fk[3]) >> 31);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    if (k4 + j < nk) {
+                        half2_t f2; __builtin_memcpy(&f2, &fk[j], 4);
+                        if (any_raised) {
+                            const bool raised = fk[j] >> 31;
+                            if (__any(raised)) {
+                                const half2_t one = { (half_t) 1.0f, (half_t) 1.0f };
+                                const half2_t ms2 = raised ? -f2 : one;
+#pragma unroll
+                                for (int e = 0; e < 8; ++e) acc2[e] = acc2[e] * ms2;
+                                f2 = raised ? one : f2;
+                            }
+                        }
+                        // all eight scalar reads first, then the eight fmas: a scalar register written by the vector unit
+                        // needs two idle cycles before the vector unit may read it, paid once per key instead of per fma
+                        uint32_t vs8[8];
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) vs8[e] = (uint32_t) __builtin_amdgcn_readlane((int) vk[e], k4 + j);
+                        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) {
+                            half2_t v2; __builtin_memcpy(&v2, &vs8[e], 4);
+                            acc2[e] = __builtin_elementwise_fma(v2, f2, acc2[e]);
+                        }
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+                }
+            }
+        } else {
             const int nk = (int)(a.KV - key0 < T_KV ? a.KV - key0 : T_KV);       // uniform
             const float4 * fp = (const float4 *)(f_s + lane * T_LDF);
             const half8_t * vp = (const half8_t *)(v_s + d0);                    // + key * FA_D halves = 8 of these
@@ -576,7 +630,7 @@ extern "C" const char * mi355x_flash_attn_ext_kernel_name(const mi355x_tensor * 
     if (!q || !k) return "flash_attn.invalid";
     switch (fa_kernel(q, k, mode)) {
         case FA_K_SEQ_ROW:  return "flash_attn.seq_row";
-        case FA_K_SEQ_TILE: return "flash_attn.seq_tile";
+        case FA_K_SEQ_TILE: return mode == MI355X_FA_F16_PACKED ? "flash_attn.seq_tile_packed" : "flash_attn.seq_tile";
         default:            return "flash_attn.vec_f32";
     }
 }
@@ -591,7 +645,7 @@ extern "C" int mi355x_flash_attn_ext(const mi355x_tensor * q, const mi355x_tenso
                                      void * workspace, size_t workspace_size, void * stream) {
     (void) workspace; (void) workspace_size;
     if (!q || !k || !v || !dst) return MI355X_ERR_INVALID;
-    if (mode != MI355X_FA_F16_SEQ && mode != MI355X_FA_F32) return MI355X_ERR_INVALID;
+    if (mode != MI355X_FA_F16_SEQ && mode != MI355X_FA_F32 && mode != MI355X_FA_F16_PACKED) return MI355X_ERR_INVALID;
     if (q->type != MI355X_TYPE_F32 || k->type != MI355X_TYPE_F16 || v->type != MI355X_TYPE_F16 || dst->type != MI355X_TYPE_F32) return MI355X_ERR_UNSUPPORTED;
     if (q->ne[0] != FA_D || k->ne[0] != FA_D || v->ne[0] != FA_D) return MI355X_ERR_UNSUPPORTED;
     if (q->nb[0] != 4 || k->nb[0] != 2 || v->nb[0] != 2) return MI355X_ERR_UNSUPPORTED;
@@ -641,7 +695,8 @@ extern "C" int mi355x_flash_attn_ext(const mi355x_tensor * q, const mi355x_tenso
             const int64_t gx = (N + T_Q - 1) / T_Q;
             if (gx > 0x7fffffff) return MI355X_ERR_UNSUPPORTED;
             dim3 grid((unsigned) gx, (unsigned) H, (unsigned) q->ne[3]);
-            k_fattn_seq_tile<<<grid, 256, 0, st>>>(a);
+            if (mode == MI355X_FA_F16_PACKED) k_fattn_seq_tile<true ><<<grid, 256, 0, st>>>(a);
+            else                              k_fattn_seq_tile<false><<<grid, 256, 0, st>>>(a);
         } break;
         default: {
             const int64_t waves = N * H * q->ne[3];
