@@ -66,6 +66,9 @@ enum mi355x_epilogue_flags {
                                   there by the previous call with the same src1): skip the conversion pass     */
     MI355X_MM_ACT_Q8_0  = 256, /* GEMM path, F16 src0 that is the f16 image (mi355x_dequantize_row_f16) of a
                                   quantized weight: round src1 to Q8_0 as for the quantized weight itself      */
+    MI355X_EPI_EMIT_F16 = 1024, /* GEMM path, f32 dst with ne0 a multiple of 32: also write to `image` the rows of dst
+                                  rounded to Q8_0 like quantize_row_q8_0 and stored as f16(q * d), dense [N][M] — what
+                                  the src1 conversion pass of the MUL_MAT that reads dst next would produce            */
     MI355X_MM_PREPARE_ONLY = 512, /* GEMM path: run only the src1 conversion pass into `workspace` and return; the
                                   product itself then follows in a second call with MI355X_MM_WS_READY (lets a
                                   caller time or overlap the two separately); a no-op on the other paths       */
@@ -76,6 +79,7 @@ typedef struct mi355x_epilogue {
     float        scale;
     const void * bias;
     const void * residual;
+    void *       image;      /* MI355X_EPI_EMIT_F16 */
 } mi355x_epilogue;
 
 /* library / device ---------------------------------------------------------------------------------- */
@@ -148,7 +152,12 @@ MI355X_API int    mi355x_mul_mat_group(const mi355x_mul_mat_item * items, int co
  * with the softmax factor converted to f16 — the arithmetic of the reference's Arm fp16 build (GGML_F16_VEC_FMA =
  * vfmaq_f16, ggml/src/ggml-cpu/simd-mappings.h:67-78) rather than of its x86 build; about 1e-7 NMSE from the latter,
  * a third of the accumulation work.  It applies to more than 8 queries (fewer run as MI355X_FA_F16_SEQ). */
-enum mi355x_fa_mode { MI355X_FA_F16_SEQ = 0, MI355X_FA_F32 = 1, MI355X_FA_F16_PACKED = 2 };
+enum mi355x_fa_mode { MI355X_FA_F16_SEQ = 0, MI355X_FA_F32 = 1, MI355X_FA_F16_PACKED = 2,
+    /* or-ed into the mode: also write into `workspace` (16-byte aligned, N * H * ne3 * 64 halves) the image of dst that
+     * a following MUL_MAT with quantized weights wants — rows [N][H * 64] rounded to Q8_0 as quantize_row_q8_0 does and
+     * stored as f16(q * d) (then pass MI355X_MM_WS_READY there).  More than 8 queries, not MI355X_FA_F32;
+     * MI355X_ERR_UNSUPPORTED otherwise. */
+    MI355X_FA_EMIT_F16 = 0x100 };
 MI355X_API const char * mi355x_flash_attn_ext_kernel_name(const mi355x_tensor * q, const mi355x_tensor * k, int mode);
 MI355X_API size_t mi355x_flash_attn_ext_workspace_size(const mi355x_tensor * q, const mi355x_tensor * k);
 MI355X_API int    mi355x_flash_attn_ext(const mi355x_tensor * q, const mi355x_tensor * k, const mi355x_tensor * v,

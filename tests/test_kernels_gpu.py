@@ -161,6 +161,31 @@ def test_mul_mat_epilogues(pkg, oracle, gpu):
         assert oracle.nmse(got, base + colbias[:, None]) <= 1e-6
 
 
+def test_mul_mat_epilogue_emits_the_next_products_activation_image(pkg, oracle, gpu):
+    # MI355X_EPI_EMIT_F16: besides dst (here with bias and GELU, the FFN's first matrix), its rows rounded to Q8_0 as f16(q * d)
+    lib = pkg.kernels()
+    k, m, n = 256, 320, 150
+    blocks = oracle.quantize(pkg.Q5_0, rnd((m, k), 0.05))
+    x, bias = rnd((n, k)), rnd((m,), 0.5)
+    d_w, d_x, d_b = gpu.up(blocks), gpu.up(x), gpu.up(bias)
+    d_y = torch.zeros((n, m), dtype=torch.float32, device=gpu.dev)
+    d_h = torch.zeros((n, m), dtype=torch.float16, device=gpu.dev)
+    tw, tx, ty = pkg.tensor(d_w, pkg.Q5_0, ne=[k, m]), pkg.tensor(d_x, pkg.F32), pkg.tensor(d_y, pkg.F32)
+    need = lib.mi355x_mul_mat_workspace_size(tw, tx)
+    ws = torch.empty(need, dtype=torch.uint8, device=gpu.dev)
+    epi = pkg.Epilogue()
+    epi.flags, epi.scale, epi.bias, epi.image = pkg.EPI_BIAS | pkg.EPI_GELU | pkg.EPI_EMIT_F16, 1.0, d_b.data_ptr(), d_h.data_ptr()
+    pkg.check(lib.mi355x_mul_mat(tw, tx, ty, C.byref(epi), ws.data_ptr(), need, gpu.stream))
+    y = gpu.down(d_y)
+    assert oracle.nmse(y, oracle.gelu(oracle.mul_mat(pkg.Q5_0, blocks, x) + bias)) <= 1e-5
+    image = oracle.dequantize(oracle.Q8_0, oracle.quantize(oracle.Q8_0, y, act=True), m).reshape(n, m)
+    assert np.array_equal(gpu.down(d_h, np.uint16), oracle.f32_to_f16_bits(image))
+    # the GEMV path has no such epilogue
+    d_x5 = gpu.up(x[:5])
+    d_y5 = torch.zeros((5, m), dtype=torch.float32, device=gpu.dev)
+    assert lib.mi355x_mul_mat(tw, pkg.tensor(d_x5, pkg.F32), pkg.tensor(d_y5, pkg.F32), C.byref(epi), ws.data_ptr(), need, gpu.stream) == -1
+
+
 def test_mul_mat_group_equals_single_calls(pkg, oracle, gpu):
     # three products over the same activations (the shape of a layer's Q, K, V projections) as one launch: same bits as
     # three calls, each with its own epilogue and destination type
@@ -281,6 +306,27 @@ def test_flash_attn_f16_fma_mode(pkg, oracle, gpu, case):
     x86 = oracle.flash_attn_ext(q, kb, vb, None if mask is None else mask[:N], 0.125)
     assert oracle.nmse(got, arm) <= 1e-6       # the same f16 fma chain; exp() and dot-product ulps differ
     assert oracle.nmse(got, x86) <= 5e-4       # north-star per-op bound against the arithmetic of the CPU build at hand
+
+
+def test_flash_attn_emits_the_next_products_activation_image(pkg, oracle, gpu):
+    # MI355X_FA_EMIT_F16: besides dst, the rows [N][H * 64] rounded to Q8_0 and stored as f16(q * d)
+    H, N, KV = 4, 100, 130
+    q, kb, vb = _attention_inputs(oracle, H, N, KV)
+    d_q, d_k, d_v = gpu.up(q), gpu.up(kb), gpu.up(vb)
+    d_o = torch.empty((N, H, 64), dtype=torch.float32, device=gpu.dev)
+    d_h = torch.zeros((N, H * 64), dtype=torch.float16, device=gpu.dev)
+    tq, tk, tv, to = pkg.tensor(d_q, pkg.F32), pkg.tensor(d_k, pkg.F16), pkg.tensor(d_v, pkg.F16), pkg.tensor(d_o, pkg.F32)
+    lib = pkg.kernels()
+    pkg.check(lib.mi355x_flash_attn_ext(tq, tk, tv, None, to, 0.125, pkg.FA_F16_SEQ | pkg.FA_EMIT_F16, d_h.data_ptr(), d_h.numel() * 2, gpu.stream))
+    y = gpu.down(d_o).reshape(N, H * 64)
+    assert oracle.nmse(y, oracle.flash_attn_ext(q, kb, vb, None, 0.125).reshape(N, H * 64)) <= 1e-6
+    image = oracle.dequantize(oracle.Q8_0, oracle.quantize(oracle.Q8_0, y, act=True), H * 64).reshape(N, H * 64)
+    assert np.array_equal(gpu.down(d_h, np.uint16), oracle.f32_to_f16_bits(image))
+    # not for the few-query kernel, and not without room for the image
+    d_q5 = gpu.up(q[:, :5])
+    d_o5 = torch.empty((5, H, 64), dtype=torch.float32, device=gpu.dev)
+    assert lib.mi355x_flash_attn_ext(pkg.tensor(d_q5, pkg.F32), tk, tv, None, pkg.tensor(d_o5, pkg.F32), 0.125, pkg.FA_EMIT_F16, d_h.data_ptr(), d_h.numel() * 2, gpu.stream) == -1
+    assert lib.mi355x_flash_attn_ext(tq, tk, tv, None, to, 0.125, pkg.FA_EMIT_F16, d_h.data_ptr(), 64, gpu.stream) == -3
 
 
 def test_flash_attn_f32_mode_matches_float64(pkg, oracle, gpu):

@@ -24,9 +24,9 @@ BLOCK_BYTES = {Q5_0: 22, Q8_0: 34}
 
 # enum mi355x_epilogue_flags
 EPI_BIAS, EPI_GELU, EPI_SCALE, EPI_RESIDUAL, EPI_BIAS_COL, EPI_OUT_F16 = 1, 2, 4, 8, 16, 32
-MM_EXACT_ACT, MM_WS_READY, MM_ACT_Q8_0, MM_PREPARE_ONLY = 64, 128, 256, 512
+MM_EXACT_ACT, MM_WS_READY, MM_ACT_Q8_0, MM_PREPARE_ONLY, EPI_EMIT_F16 = 64, 128, 256, 512, 1024
 # enum mi355x_fa_mode
-FA_F16_SEQ, FA_F32, FA_F16_PACKED = 0, 1, 2
+FA_F16_SEQ, FA_F32, FA_F16_PACKED, FA_EMIT_F16 = 0, 1, 2, 0x100
 
 
 class Tensor(C.Structure):
@@ -36,7 +36,7 @@ class Tensor(C.Structure):
 
 class Epilogue(C.Structure):
     """struct mi355x_epilogue"""
-    _fields_ = [("flags", C.c_int32), ("scale", C.c_float), ("bias", C.c_void_p), ("residual", C.c_void_p)]
+    _fields_ = [("flags", C.c_int32), ("scale", C.c_float), ("bias", C.c_void_p), ("residual", C.c_void_p), ("image", C.c_void_p)]
 
 
 class MulMatItem(C.Structure):

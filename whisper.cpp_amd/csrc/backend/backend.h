@@ -87,8 +87,10 @@ struct mi355x_backend_ctx {
                                    // reference's f16-sequential / Q8_0-rounded arithmetic
 
     // scratch for the kernels (grow-only), and which activations its Q8_0-rounded copy currently mirrors
-    void *       ws       = nullptr;
-    size_t       ws_size  = 0;
+    void *       ws_base  = nullptr;   // the allocation: two slots of ws_size bytes
+    void *       ws       = nullptr;   // the current slot (where the cached activation image lives)
+    size_t       ws_size  = 0;         // bytes per slot
+    int          ws_slot  = 0;
     const void * ws_x     = nullptr;
     int          ws_x_mode = 0;
     int64_t      ws_x_ne[4] = {0, 0, 0, 0};

@@ -241,7 +241,7 @@ static void backend_free(ggml_backend_t backend) {
         }
     }
     for (hipEvent_t e : ctx->event_pool) (void) hipEventDestroy(e);
-    if (ctx->ws) (void) hipFree(ctx->ws);
+    if (ctx->ws_base) (void) hipFree(ctx->ws_base);
     if (ctx->stream) (void) hipStreamDestroy(ctx->stream);
     delete ctx;
     delete backend;

@@ -117,15 +117,18 @@ void mi355x_backend_ctx::drain_events() {
     pending.clear();
 }
 
+// Two slots of `size` bytes each: a product reads its activation image from one while its epilogue may already write the
+// next product's image into the other.
 bool mi355x_backend_ctx::reserve_workspace(size_t size) {
     if (size <= ws_size) return true;
     // the stream may still be reading the old block
     if (hipStreamSynchronize(stream) != hipSuccess) { (void) hipGetLastError(); return false; }
-    if (ws) (void) hipFree(ws);
-    ws = nullptr; ws_size = 0; ws_x = nullptr;
-    const size_t want = size + size / 2;
-    if (hipMalloc(&ws, want) != hipSuccess) { (void) hipGetLastError(); ws = nullptr; return false; }
+    if (ws_base) (void) hipFree(ws_base);
+    ws_base = nullptr; ws = nullptr; ws_size = 0; ws_x = nullptr; ws_slot = 0;
+    const size_t want = (size + size / 2 + 255) / 256 * 256;
+    if (hipMalloc(&ws_base, 2 * want) != hipSuccess) { (void) hipGetLastError(); ws_base = nullptr; return false; }
     ws_size = want;
+    ws = ws_base;
     return true;
 }
 
@@ -203,7 +206,7 @@ struct graph_runner {
     mm_chain plan_chain(int i) const {
         ggml_tensor * mm = g->nodes[i];
         const ggml_tensor * w = mm->src[0], * x = mm->src[1];
-        mi355x_epilogue epi = { 0, 1.0f, nullptr, nullptr };
+        mi355x_epilogue epi = { 0, 1.0f, nullptr, nullptr, nullptr };
         ggml_tensor * last = mm;       // node whose value the fused kernel produces
         ggml_tensor * out  = mm;
         int used = 1;
@@ -258,7 +261,7 @@ struct graph_runner {
             }
             // the folded result must not land on memory the kernel is still reading
             if (used > 1 && (ranges_overlap(out, x) || ranges_overlap(out, w))) {
-                epi = { 0, 1.0f, nullptr, nullptr }; out = mm; used = 1;
+                epi = { 0, 1.0f, nullptr, nullptr, nullptr }; out = mm; used = 1;
             }
         }
         return { mm, w, x, epi, out, used };
@@ -380,10 +383,18 @@ struct graph_runner {
 
         mi355x_epilogue epi = c.epi;
         epi.flags |= o.mm_flags;
-        const size_t need = mi355x_mul_mat_workspace_size(&o.vw, &o.vx);
+        size_t need = mi355x_mul_mat_workspace_size(&o.vw, &o.vx);
+        // when the result feeds nothing but products that round it to Q8_0 (the FFN's second matrix after the first), the
+        // epilogue writes that image into the workspace slot this product is not reading from
+        const ggml_tensor * key = nullptr;
+        if (!(epi.flags & MI355X_EPI_OUT_F16) && c.mm->ne[2] == 1 && c.mm->ne[3] == 1 && strncmp(o.kernel_name, "mul_mat.gemm", 12) == 0) {
+            key = image_consumer(c.out, i + c.used);
+            if (key) need = std::max(need, (size_t) ggml_nelements(c.out) * 2 + 256);
+        }
         const int ready = prepare_src1(c, o, need, status);
         if (ready < 0) return c.used;
         epi.flags |= ready;
+        if (key && ctx->ws_base) { epi.flags |= MI355X_EPI_EMIT_F16; epi.image = slot_ptr(ctx->ws_slot ^ 1); } else key = nullptr;
         if (ctx->debug) {
             GGML_LOG_INFO("ggml-mi355x: %s %s [%lld x %lld x %lld] folds %d nodes, flags 0x%x\n", o.kernel_name, c.mm->name,
                           (long long) c.mm->ne[0], (long long) c.mm->ne[1], (long long) c.w->ne[0], c.used, epi.flags);
@@ -391,9 +402,51 @@ struct graph_runner {
         {
             launch_scope ls(ctx, o.kernel_name, chain_bytes(c), chain_flops(c));
             status = mi355x_mul_mat(&o.vw, &o.vx, &o.vd, epi.flags ? &epi : nullptr, ctx->ws, ctx->ws_size, ctx->stream);
+            if (key && status == MI355X_ERR_UNSUPPORTED) {          // shapes the epilogue cannot emit for: plain product
+                epi.flags &= ~MI355X_EPI_EMIT_F16; key = nullptr;
+                status = mi355x_mul_mat(&o.vw, &o.vx, &o.vd, epi.flags ? &epi : nullptr, ctx->ws, ctx->ws_size, ctx->stream);
+            }
         }
         note_write(c.out);
+        if (key && status == MI355X_OK) workspace_holds(key, ctx->ws_slot ^ 1);
         return c.used;
+    }
+
+    // When everything that reads `out` (produced just before node `from`) — directly, or through one dense 2-d RESHAPE of
+    // it — is a many-column product with quantized weights, the producer can leave the Q8_0-rounded f16 image those
+    // products want in the workspace and they skip their conversion pass.  Returns the tensor the products name as src1.
+    const ggml_tensor * image_consumer(const ggml_tensor * out, int from) const {
+        if (!ctx->fuse || ctx->exact || (out->flags & GGML_TENSOR_FLAG_OUTPUT) || !ggml_is_contiguous(out)) return nullptr;
+        const ggml_tensor * key = out;
+        for (int hop = 0; hop < 2; ++hop) {
+            auto it = readers.find(key);
+            const int want = it == readers.end() ? 0 : it->second;
+            if (want == 0) return nullptr;
+            int seen = 0;
+            const ggml_tensor * reshape = nullptr;
+            for (int j = from; j < g->n_nodes && seen < want; ++j) {
+                const ggml_tensor * n = g->nodes[j];
+                bool reads = n->view_src == key;
+                for (int k = 0; k < GGML_MAX_SRC; ++k) reads = reads || n->src[k] == key;
+                if (!reads) continue;
+                ++seen;
+                if (n->op == GGML_OP_MUL_MAT && n->src[1] == key && n->src[0] != key && ggml_is_quantized(n->src[0]->type)) continue;
+                if (want == 1 && hop == 0 && n->op == GGML_OP_RESHAPE && n->src[0] == key && ggml_is_contiguous(n) && !(n->flags & GGML_TENSOR_FLAG_OUTPUT)) { reshape = n; continue; }
+                return nullptr;
+            }
+            if (seen != want) return nullptr;
+            if (!reshape) break;
+            key = reshape;
+        }
+        if (key->ne[2] != 1 || key->ne[3] != 1 || key->ne[1] <= MI355X_GEMV_MAX_COLS || key->ne[0] % 32 != 0) return nullptr;
+        return key;
+    }
+    void * slot_ptr(int slot) const { return (char *) ctx->ws_base + (size_t) slot * ctx->ws_size; }
+    // the image of `key` now sits in `slot`, which becomes the current one
+    void workspace_holds(const ggml_tensor * key, int slot) {
+        ctx->ws_slot = slot; ctx->ws = slot_ptr(slot);
+        ctx->ws_x = key->data; ctx->ws_x_mode = 1; memcpy(ctx->ws_x_ne, key->ne, sizeof(key->ne)); memcpy(ctx->ws_x_nb, key->nb, sizeof(key->nb));
+        cached_x = key;
     }
 
     // ---- NORM [-> MUL(w) -> ADD(b)] ---------------------------------------------------------------------
@@ -416,31 +469,15 @@ struct graph_runner {
         mi355x_tensor vs = to_view(nm->src[0]), vd = to_view(out);
         // When everything that reads the result is a many-column product with quantized weights, the kernel also leaves
         // the Q8_0-rounded f16 image those products want in the workspace, and they skip their conversion pass.
-        bool emit = false;
-        if (ctx->fuse && !ctx->exact && out->ne[2] == 1 && out->ne[3] == 1 && out->ne[1] > MI355X_GEMV_MAX_COLS && out->ne[0] % 32 == 0 &&
-            out->ne[0] <= 2048 && ggml_is_contiguous(out) && !(out->flags & GGML_TENSOR_FLAG_OUTPUT)) {
-            auto it = readers.find(out);
-            int want = it == readers.end() ? 0 : it->second, seen = 0;
-            for (int j = i + used; j < g->n_nodes && want > 0; ++j) {
-                const ggml_tensor * n = g->nodes[j];
-                bool reads = false;
-                for (int k = 0; k < GGML_MAX_SRC; ++k) reads = reads || n->src[k] == out;
-                if (!reads && n->view_src != out) continue;
-                if (n->op == GGML_OP_MUL_MAT && n->src[1] == out && n->src[0] != out && ggml_is_quantized(n->src[0]->type)) ++seen; else { seen = -1; break; }
-                if (seen == want) break;
-            }
-            emit = want > 0 && seen == want && ctx->reserve_workspace((size_t)(out->ne[0] * out->ne[1] * 2 + 256));
-        }
+        const ggml_tensor * key = out->ne[0] <= 2048 ? image_consumer(out, i + used) : nullptr;
+        bool emit = key && ctx->reserve_workspace((size_t)(out->ne[0] * out->ne[1] * 2 + 256));
         {
             launch_scope ls(ctx, used == 3 ? (emit ? "norm_affine_emit" : "norm_affine") : "norm", nbytes_of(nm->src[0]) + nbytes_of(out) * (emit ? 1.5 : 1.0), 0.0);
             status = emit ? mi355x_norm_emit_f16(&vs, &vd, eps, w, b, ctx->ws, ctx->stream) : mi355x_norm(&vs, &vd, eps, w, b, ctx->stream);
         }
         if (emit && status == MI355X_ERR_UNSUPPORTED) { emit = false; status = mi355x_norm(&vs, &vd, eps, w, b, ctx->stream); }
         note_write(out);
-        if (emit && status == MI355X_OK) {
-            ctx->ws_x = out->data; ctx->ws_x_mode = 1; memcpy(ctx->ws_x_ne, out->ne, sizeof(out->ne)); memcpy(ctx->ws_x_nb, out->nb, sizeof(out->nb));
-            cached_x = out;
-        }
+        if (emit && status == MI355X_OK) workspace_holds(key, ctx->ws_slot);
         return used;
     }
 
@@ -515,8 +552,17 @@ struct graph_runner {
                 const double flops = 4.0 * s0->ne[1] * k->ne[1] * 64.0 * s0->ne[2] * s0->ne[3];
                 const double bytes = (double) ggml_nelements(s0) * 4 + 2.0 * (double) k->ne[0] * k->ne[1] * k->ne[2] * k->ne[3] * 2 + nbytes_of(n);
                 const int mode = ctx->exact ? MI355X_FA_F32 : ctx->fa_packed ? MI355X_FA_F16_PACKED : MI355X_FA_F16_SEQ;
-                launch_scope ls(ctx, mi355x_flash_attn_ext_kernel_name(&vq, &vk, mode), bytes, flops);
-                status = mi355x_flash_attn_ext(&vq, &vk, &vv, m ? &vm : nullptr, &vd, scale, mode, nullptr, 0, ctx->stream);
+                const char * name = mi355x_flash_attn_ext_kernel_name(&vq, &vk, mode);
+                // the output projection that follows takes its Q8_0-rounded activations from the attention kernel itself
+                const ggml_tensor * key = strncmp(name, "flash_attn.seq_tile", 19) == 0 ? image_consumer(n, i + 1) : nullptr;
+                const size_t image_bytes = (size_t) ggml_nelements(n) * 2;
+                if (key && !ctx->reserve_workspace(image_bytes + 256)) key = nullptr;
+                {
+                    launch_scope ls(ctx, name, bytes + (key ? image_bytes : 0), flops);
+                    status = mi355x_flash_attn_ext(&vq, &vk, &vv, m ? &vm : nullptr, &vd, scale, mode | (key ? MI355X_FA_EMIT_F16 : 0),
+                                                   key ? ctx->ws : nullptr, key ? ctx->ws_size : 0, ctx->stream);
+                }
+                if (key && status == MI355X_OK) workspace_holds(key, ctx->ws_slot);
                 return 1;
             }
             case GGML_OP_CONCAT: {

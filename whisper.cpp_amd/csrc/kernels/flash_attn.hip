@@ -33,6 +33,7 @@ struct fa_args {
     int64_t hk_ratio, hv_ratio;      // q heads per k head / v head (broadcast)
     int64_t ne3, k_ne3_ratio, v_ne3_ratio;
     float scale;
+    half_t * x16;                    // when set: also the Q8_0-rounded f16 image of dst ([N][H * 64] rows), for the product that follows
 };
 
 // ------------------------------------------------------------------------------------------------------
@@ -599,14 +600,36 @@ __global__ void __launch_bounds__(256) k_fattn_seq_tile(fa_args a) {
     }
 
     const int64_t n = n0 + lane;
-    if (n < a.N) {
+    float o[16];
+    {
         const float inv = 1.0f / s_run[lane];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) { o[2*i] = (float) acc2[i][0] * inv; o[2*i + 1] = (float) acc2[i][1] * inv; }
+    }
+    if (n < a.N) {
         float * dp = (float *) a.d + ((i3 * a.N + n) * a.H + h) * FA_D + d0;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const half2_t p0 = acc2[2*i], p1 = acc2[2*i + 1];
-            float4 o = { (float) p0[0] * inv, (float) p0[1] * inv, (float) p1[0] * inv, (float) p1[1] * inv };
-            *(float4 *)(dp + 4 * i) = o;
+        for (int i = 0; i < 4; ++i) *(float4 *)(dp + 4 * i) = make_float4(o[4*i], o[4*i + 1], o[4*i + 2], o[4*i + 3]);
+    }
+    if (a.x16) {
+        // The projection that follows rounds these rows to Q8_0 (blocks of 32 along d: two wavefronts' slices of a query)
+        // before multiplying; write that image — f16(q * d), as quantize_row_q8_0 would produce q and d — here, so that it
+        // needs no pass of its own over the attention output.
+        float amax = 0.0f;
+#pragma unroll
+        for (int e = 0; e < 16; ++e) amax = fmaxf(amax, fabsf(o[e]));
+        __syncthreads();                                   // every chain is done with the factor tile
+        f_s[wave * T_Q + lane] = amax;
+        __syncthreads();
+        amax = fmaxf(amax, f_s[(wave ^ 1) * T_Q + lane]);
+        if (n < a.N) {
+            const float id = amax != 0.0f ? 127.0f / amax : 0.0f;
+            const float dq = h2f(f2h_bits(amax / 127.0f));
+            half8_t h0, h1;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) { h0[e] = (half_t)((rintf(o[e] * id) + 0.0f) * dq); h1[e] = (half_t)((rintf(o[8 + e] * id) + 0.0f) * dq); }
+            half8_t * xp = (half8_t *)(a.x16 + ((i3 * a.N + n) * a.H + h) * FA_D + d0);
+            xp[0] = h0; xp[1] = h1;
         }
     }
 }
@@ -643,8 +666,9 @@ extern "C" size_t mi355x_flash_attn_ext_workspace_size(const mi355x_tensor * q, 
 extern "C" int mi355x_flash_attn_ext(const mi355x_tensor * q, const mi355x_tensor * k, const mi355x_tensor * v,
                                      const mi355x_tensor * mask, const mi355x_tensor * dst, float scale, int mode,
                                      void * workspace, size_t workspace_size, void * stream) {
-    (void) workspace; (void) workspace_size;
     if (!q || !k || !v || !dst) return MI355X_ERR_INVALID;
+    const bool emit = mode & MI355X_FA_EMIT_F16;
+    mode &= ~MI355X_FA_EMIT_F16;
     if (mode != MI355X_FA_F16_SEQ && mode != MI355X_FA_F32 && mode != MI355X_FA_F16_PACKED) return MI355X_ERR_INVALID;
     if (q->type != MI355X_TYPE_F32 || k->type != MI355X_TYPE_F16 || v->type != MI355X_TYPE_F16 || dst->type != MI355X_TYPE_F32) return MI355X_ERR_UNSUPPORTED;
     if (q->ne[0] != FA_D || k->ne[0] != FA_D || v->ne[0] != FA_D) return MI355X_ERR_UNSUPPORTED;
@@ -675,6 +699,13 @@ extern "C" int mi355x_flash_attn_ext(const mi355x_tensor * q, const mi355x_tenso
     a.hk_ratio = H / k->ne[2]; a.hv_ratio = H / v->ne[2];
     a.ne3 = q->ne[3]; a.k_ne3_ratio = q->ne[3] / k->ne[3]; a.v_ne3_ratio = q->ne[3] / v->ne[3];
     a.scale = scale;
+    a.x16 = nullptr;
+    if (emit) {
+        // only the tile kernel in the reference's arithmetic writes the image; say so rather than silently skip it
+        if (fa_kernel(q, k, mode) != FA_K_SEQ_TILE || mode == MI355X_FA_F32) return MI355X_ERR_UNSUPPORTED;
+        if (!workspace || (uintptr_t) workspace % 16 != 0 || workspace_size < (size_t)(N * H * q->ne[3]) * FA_D * sizeof(half_t)) return MI355X_ERR_WORKSPACE;
+        a.x16 = (half_t *) workspace;
+    }
     hipStream_t st = (hipStream_t) stream;
 
     switch (fa_kernel(q, k, mode)) {

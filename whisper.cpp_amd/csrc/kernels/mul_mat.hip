@@ -30,6 +30,7 @@ struct epi_args {
     const float *bias;
     const char * residual;   // same strides as dst, f32
     const uint16_t * gelu;   // GELU table (device), set when MI355X_EPI_GELU is
+    half_t * image;          // MI355X_EPI_EMIT_F16: where the Q8_0-rounded f16 image of dst goes ([N][M] dense)
 };
 
 __device__ __forceinline__ float apply_epilogue(float v, const epi_args & e, int64_t m, int64_t n, int64_t res_off) {
@@ -44,6 +45,20 @@ __device__ __forceinline__ float apply_epilogue(float v, const epi_args & e, int
 // The same for the 16 registers of one 32x32 accumulator patch (column m, rows n[0..15]) and the stores.  All loads of
 // one kind are issued together before their first use; rows beyond N and columns beyond M are computed from clamped
 // addresses and not stored.
+// maximum over the 32 lanes of a half-wavefront, in every lane: four DPP steps inside the rows of 16 (a mirror pairs the
+// lanes as well as an exchange does, for a maximum) and one swizzle across the two rows
+__device__ __forceinline__ float half_wave_max(float x) {
+    auto dpp = [](float v, auto ctrl) __attribute__((always_inline)) {
+        return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), decltype(ctrl)::value, 0xf, 0xf, true));
+    };
+    x = fmaxf(x, dpp(x, std::integral_constant<int, 0xB1>()));    // quad_perm [1,0,3,2]
+    x = fmaxf(x, dpp(x, std::integral_constant<int, 0x4E>()));    // quad_perm [2,3,0,1]
+    x = fmaxf(x, dpp(x, std::integral_constant<int, 0x141>()));   // row_half_mirror
+    x = fmaxf(x, dpp(x, std::integral_constant<int, 0x140>()));   // row_mirror
+    return fmaxf(x, __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, x), 0x401F)));   // lane ^ 16
+}
+
+template <bool EMIT>
 __device__ __forceinline__ void patch_epilogue(float16_t v, const epi_args & e, char * db, int64_t batch_off, int64_t d_nb1,
                                                int64_t m, int64_t M, const int64_t (&n)[16], int64_t N) {
     const bool    m_ok = m < M;
@@ -87,6 +102,18 @@ __device__ __forceinline__ void patch_epilogue(float16_t v, const epi_args & e, 
     } else {
 #pragma unroll
         for (int i = 0; i < 16; ++i) if (m_ok && n[i] < N) *(float *)(db + n[i] * d_nb1 + m * 4) = v[i];
+    }
+    if (EMIT) {
+        // The product that reads dst next rounds its rows to Q8_0 first.  The 32 lanes of a half-wavefront hold 32
+        // consecutive m of one dst row — exactly one Q8_0 block (M % 32 == 0) — so the block maximum is a 5-step
+        // butterfly, and the image f16(q * d) is written here instead of by a pass of its own over dst.
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const float amax = half_wave_max(fabsf(v[i]));
+            const float id = amax != 0.0f ? 127.0f / amax : 0.0f;
+            const float dq = h2f(f2h_bits(amax / 127.0f));
+            if (m_ok && n[i] < N) e.image[n[i] * M + m] = (half_t)((rintf(v[i] * id) + 0.0f) * dq);
+        }
     }
 }
 
@@ -240,7 +267,9 @@ __global__ void k_x_to_f16(const char * __restrict__ x, half_t * __restrict__ ou
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
-template <int TI, int TJ, int S, bool KTAIL, bool FULL>     // KTAIL: K is not a multiple of 64 (but of 8); FULL: K / 64 is a multiple of S
+// KTAIL: K is not a multiple of 64 (but of 8); FULL: K / 64 is a multiple of S; EMIT: MI355X_EPI_EMIT_F16 (a kernel of its
+// own, because its epilogue needs more registers than two workgroups per CU leave)
+template <int TI, int TJ, int S, bool KTAIL, bool FULL, bool EMIT = false>
 __device__ __forceinline__ void gemm_f16_tile(const mm_args & a, int tiles_m, int tiles_n, const char * wb, const char * xb, char * db,
                                               const epi_args & epi, int64_t batch_off, int64_t d_nb1) {
     constexpr int BN = 64 * TI, BM = 64 * TJ;
@@ -398,14 +427,14 @@ __device__ __forceinline__ void gemm_f16_tile(const mm_args & a, int tiles_m, in
         for (int e = 0; e < 16; ++e) n[e] = n0 + wn + 32 * i + 8 * (e >> 2) + 4 * g + (e & 3);
 #pragma unroll
         for (int j = 0; j < TJ; ++j)
-            patch_epilogue(acc[i][j], epi, db, batch_off, d_nb1, m0 + wmo + 32 * j + l32, a.M, n, a.N);
+            patch_epilogue<EMIT>(acc[i][j], epi, db, batch_off, d_nb1, m0 + wmo + 32 * j + l32, a.M, n, a.N);
     }
 }
 
-template <int TI, int TJ, int S, bool KTAIL, bool FULL>
-__global__ void __launch_bounds__(256) k_gemm_f16(mm_args a, int tiles_m, int tiles_n) {
+template <int TI, int TJ, int S, bool KTAIL, bool FULL, bool EMIT>
+__global__ void __launch_bounds__(256, 2) k_gemm_f16(mm_args a, int tiles_m, int tiles_n) {
     const int64_t b2 = blockIdx.y % a.ne12, b3 = blockIdx.y / a.ne12;
-    gemm_f16_tile<TI, TJ, S, KTAIL, FULL>(a, tiles_m, tiles_n, a.w + (b2 / a.r2) * a.w_nb2 + (b3 / a.r3) * a.w_nb3, a.x + b2 * a.x_nb2 + b3 * a.x_nb3,
+    gemm_f16_tile<TI, TJ, S, KTAIL, FULL, EMIT>(a, tiles_m, tiles_n, a.w + (b2 / a.r2) * a.w_nb2 + (b3 / a.r3) * a.w_nb3, a.x + b2 * a.x_nb2 + b3 * a.x_nb3,
                                           a.d + b2 * a.d_nb2 + b3 * a.d_nb3, a.e, b2 * a.d_nb2 + b3 * a.d_nb3, a.d_nb1);
 }
 
@@ -420,11 +449,11 @@ template <int TI, int TJ, int S>
 __global__ void __launch_bounds__(256) k_gemm_f16_group(mm_args a, int tiles_m, int tiles_n, mm_group grp) {
     const mm_group_entry & ge = grp.e[blockIdx.y];
     epi_args e;
-    e.flags = ge.flags; e.scale = ge.scale; e.bias = ge.bias; e.residual = ge.residual; e.gelu = a.e.gelu;
+    e.flags = ge.flags; e.scale = ge.scale; e.bias = ge.bias; e.residual = ge.residual; e.gelu = a.e.gelu; e.image = nullptr;
     gemm_f16_tile<TI, TJ, S, false, true>(a, tiles_m, tiles_n, ge.w, a.x, ge.d, e, 0, ge.d_nb1);
 }
 
-template <int TI, int TJ, int S, bool KTAIL, bool FULL>
+template <int TI, int TJ, int S, bool KTAIL, bool FULL, bool EMIT = false>
 static int launch_gemm_f16_k(const mm_args & a, hipStream_t st) {
     static_assert(S % 2 == 0, "the LDS buffer index is the parity of the register slot");
     constexpr int BN = 64 * TI, BM = 64 * TJ;
@@ -433,17 +462,21 @@ static int launch_gemm_f16_k(const mm_args & a, hipStream_t st) {
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return MI355X_ERR_HIP;
     if (!configured[dev]) {
-        if (hipFuncSetAttribute((const void *) k_gemm_f16<TI, TJ, S, KTAIL, FULL>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds) != hipSuccess) return MI355X_ERR_HIP;
+        if (hipFuncSetAttribute((const void *) k_gemm_f16<TI, TJ, S, KTAIL, FULL, EMIT>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds) != hipSuccess) return MI355X_ERR_HIP;
         configured[dev] = true;
     }
     const int64_t tm = (a.M + BM - 1) / BM, tn = (a.N + BN - 1) / BN;
     if (tm * tn > 0x7fffffff) return MI355X_ERR_UNSUPPORTED;
     dim3 grid((unsigned)(tm * tn), (unsigned)(a.ne12 * a.ne13));
-    k_gemm_f16<TI, TJ, S, KTAIL, FULL><<<grid, 256, lds, st>>>(a, (int) tm, (int) tn);
+    k_gemm_f16<TI, TJ, S, KTAIL, FULL, EMIT><<<grid, 256, lds, st>>>(a, (int) tm, (int) tn);
     return launch_status();
 }
 template <int TI, int TJ>
 static int launch_gemm_f16(const mm_args & a, hipStream_t st) {
+    if (a.e.flags & MI355X_EPI_EMIT_F16) {
+        if (a.K % (2 * GB_K)) return MI355X_ERR_UNSUPPORTED;
+        return a.K % (4 * GB_K) == 0 ? launch_gemm_f16_k<TI, TJ, 4, false, true, true>(a, st) : launch_gemm_f16_k<TI, TJ, 2, false, true, true>(a, st);
+    }
     if (a.K % GB_K) return launch_gemm_f16_k<TI, TJ, 2, true, false>(a, st);
     const int64_t kt = a.K / GB_K;
     if (kt % 4 == 0) return launch_gemm_f16_k<TI, TJ, 4, false, true>(a, st);
@@ -832,6 +865,7 @@ extern "C" int mi355x_mul_mat_group(const mi355x_mul_mat_item * items, int count
         const mi355x_epilogue * e = items[i].epi;
         if (!w || !d) return MI355X_ERR_INVALID;
         if (w->type != MI355X_TYPE_F16 || w->ne[0] != a.K || w->ne[1] != a.M || w->ne[2] != 1 || w->ne[3] != 1 || w->nb[0] != 2 || w->nb[1] != w0->nb[1] || !aligned16(w)) return MI355X_ERR_UNSUPPORTED;
+        if (e && (e->flags & MI355X_EPI_EMIT_F16)) return MI355X_ERR_UNSUPPORTED;
         const int ef = e ? (e->flags & 63) : 0;
         const int td = (ef & MI355X_EPI_OUT_F16) ? MI355X_TYPE_F16 : MI355X_TYPE_F32;
         if (d->type != td || d->ne[0] != a.M || d->ne[1] != a.N || d->ne[2] != 1 || d->ne[3] != 1 || d->nb[0] != type_size(td) || d->nb[1] % 4 != 0) return MI355X_ERR_UNSUPPORTED;
@@ -846,7 +880,7 @@ extern "C" int mi355x_mul_mat_group(const mi355x_mul_mat_item * items, int count
     a.x_nb1 = src1->nb[1]; a.x_nb2 = a.x_nb3 = 0;
     a.d_nb1 = items[0].dst->nb[1]; a.d_nb2 = a.d_nb3 = 0;
     a.ne12 = a.ne13 = a.r2 = a.r3 = 1;
-    a.e.flags = 0; a.e.scale = 1.0f; a.e.bias = nullptr; a.e.residual = nullptr; a.e.gelu = nullptr;
+    a.e.flags = 0; a.e.scale = 1.0f; a.e.bias = nullptr; a.e.residual = nullptr; a.e.gelu = nullptr; a.e.image = nullptr;
     if (any_gelu && !(a.e.gelu = gelu_table_device())) return MI355X_ERR_HIP;
     hipStream_t st = (hipStream_t) stream;
 
@@ -913,6 +947,11 @@ extern "C" int mi355x_mul_mat(const mi355x_tensor * src0, const mi355x_tensor * 
     a.e.residual = epi ? (const char *) epi->residual : nullptr;
     a.e.gelu = nullptr;
     if ((flags & MI355X_EPI_GELU) && !(a.e.gelu = gelu_table_device())) return MI355X_ERR_HIP;
+    a.e.image = epi ? (half_t *) epi->image : nullptr;
+    if (flags & MI355X_EPI_EMIT_F16) {
+        if (!a.e.image || (flags & MI355X_EPI_OUT_F16)) return MI355X_ERR_INVALID;
+        if (a.M % QK != 0 || dst->ne[2] * dst->ne[3] != 1 || mm_path(src0, src1) != MM_GEMM) return MI355X_ERR_UNSUPPORTED;
+    }
 
     hipStream_t st = (hipStream_t) stream;
     const int64_t nbatch = a.ne12 * a.ne13;
