@@ -54,11 +54,15 @@ GGML_BACKEND_API int                ggml_backend_score(void);
  * "exact" (0/1, default 0: 0 reproduces the two roundings that the reference's CPU backend applies — Q8_0-rounded
  * activations in front of quantized MUL_MAT, f16 key-by-key V accumulation in FLASH_ATTN_EXT; 1 keeps f16 activations
  * and f32 accumulators, which is closer to exact arithmetic and further from the reference),
- * "fa_packed" (0/1, default 0: 1 lets FLASH_ATTN_EXT over more than 8 queries accumulate V with f16 fused multiply-adds,
- * the arithmetic of the reference's Arm fp16 build, simd-mappings.h:67-78, instead of the x86 build's f32 fma + f16
- * store: a third of the accumulation work, about 1e-7 NMSE away).
- * The environment variables GGML_MI355X_FUSE, GGML_MI355X_PROFILE, GGML_MI355X_EXACT and GGML_MI355X_FA_PACKED give the
- * initial values.
+ * "fa_accum" (0/1/2, default 0: how FLASH_ATTN_EXT over more than 8 queries accumulates V.  0: key by key with an f16
+ * accumulator, f32 fma + f16 store — the reference's x86 build, and the only setting that keeps whole-model logits within
+ * 1e-3 NMSE of the CPU backend.  1: f32 accumulators with both products on the matrix cores — six times faster, within
+ * the per-op bound, but the reference's f16 rounding is then missing and whole-model logits sit several 1e-3 away.
+ * 2: key by key with f16 fused multiply-adds, the arithmetic of the reference's Arm fp16 build, simd-mappings.h:67-78 —
+ * a third of the accumulation work, about 1e-7 NMSE per op away from the x86 build),
+ * "fa_packed" (0/1: the same as "fa_accum" 2/0).
+ * The environment variables GGML_MI355X_FUSE, GGML_MI355X_PROFILE, GGML_MI355X_EXACT, GGML_MI355X_FA_ACCUM and
+ * GGML_MI355X_FA_PACKED give the initial values.
  * backend == NULL addresses every live MI355X backend of the process (a host such as whisper.cpp keeps its
  * backends private). */
 typedef int (*ggml_backend_mi355x_set_option_t)(ggml_backend_t backend, const char * name, int value);

@@ -147,7 +147,8 @@ MI355X_API int    mi355x_mul_mat_group(const mi355x_mul_mat_item * items, int co
  * key), dst: F32 [D, H, N] contiguous.
  * mode: MI355X_FA_F16_SEQ accumulates V in f16, key by key in order, as the reference does (ops.cpp:6793-6807) —
  * with near-uniform attention over ~1500 keys that rounding sequence dominates the low bits of the result;
- * MI355X_FA_F32 accumulates in f32 (closer to exact arithmetic, further from the reference).
+ * MI355X_FA_F32 accumulates in f32 (closer to exact arithmetic, further from the reference); with more than 8 queries
+ * both products run on the matrix cores with the softmax probabilities as f16 operands.
  * MI355X_FA_F16_PACKED keeps the key order and the f16 accumulator but forms each step as one f16 fused multiply-add
  * with the softmax factor converted to f16 — the arithmetic of the reference's Arm fp16 build (GGML_F16_VEC_FMA =
  * vfmaq_f16, ggml/src/ggml-cpu/simd-mappings.h:67-78) rather than of its x86 build; about 1e-7 NMSE from the latter,
@@ -155,8 +156,7 @@ MI355X_API int    mi355x_mul_mat_group(const mi355x_mul_mat_item * items, int co
 enum mi355x_fa_mode { MI355X_FA_F16_SEQ = 0, MI355X_FA_F32 = 1, MI355X_FA_F16_PACKED = 2,
     /* or-ed into the mode: also write into `workspace` (16-byte aligned, N * H * ne3 * 64 halves) the image of dst that
      * a following MUL_MAT with quantized weights wants — rows [N][H * 64] rounded to Q8_0 as quantize_row_q8_0 does and
-     * stored as f16(q * d) (then pass MI355X_MM_WS_READY there).  More than 8 queries, not MI355X_FA_F32;
-     * MI355X_ERR_UNSUPPORTED otherwise. */
+     * stored as f16(q * d) (then pass MI355X_MM_WS_READY there).  More than 8 queries; MI355X_ERR_UNSUPPORTED otherwise. */
     MI355X_FA_EMIT_F16 = 0x100 };
 MI355X_API const char * mi355x_flash_attn_ext_kernel_name(const mi355x_tensor * q, const mi355x_tensor * k, int mode);
 MI355X_API size_t mi355x_flash_attn_ext_workspace_size(const mi355x_tensor * q, const mi355x_tensor * k);

@@ -329,15 +329,55 @@ def test_flash_attn_emits_the_next_products_activation_image(pkg, oracle, gpu):
     assert lib.mi355x_flash_attn_ext(tq, tk, tv, None, to, 0.125, pkg.FA_EMIT_F16, d_h.data_ptr(), 64, gpu.stream) == -3
 
 
-def test_flash_attn_f32_mode_matches_float64(pkg, oracle, gpu):
-    q, kb, vb = _attention_inputs(oracle, 2, 30, 300, flat=True, pad_from=280)
-    got, name = run_fa(pkg, gpu, q, kb, vb, None, 0.125, pkg.FA_F32)
-    assert name == "flash_attn.vec_f32"
+def _attention_float64(oracle, q, kb, vb, mask, scale):
     qf = oracle.f16_bits_to_f32(oracle.f32_to_f16_bits(q)).astype(np.float64)
-    s = np.einsum("hnd,hkd->hnk", qf, oracle.f16_bits_to_f32(kb).astype(np.float64)) * 0.125
+    s = np.einsum("hnd,hkd->hnk", qf, oracle.f16_bits_to_f32(kb).astype(np.float64)) * scale
+    if mask is not None:
+        s = s + oracle.f16_bits_to_f32(mask)[None, : q.shape[1]].astype(np.float64)
     p = np.exp(s - s.max(-1, keepdims=True)); p /= p.sum(-1, keepdims=True)
-    exact = np.einsum("hnk,hkd->nhd", p, oracle.f16_bits_to_f32(vb).astype(np.float64))
-    assert oracle.nmse(got, exact) <= 1e-9
+    return np.einsum("hnk,hkd->nhd", p, oracle.f16_bits_to_f32(vb).astype(np.float64))
+
+
+@pytest.mark.parametrize("case", [
+    dict(H=2, N=5, KV=300, flat=True, pad_from=280), dict(H=2, N=30, KV=300, flat=True, pad_from=280), dict(H=3, N=200, KV=1536, flat=True, pad_from=1500),
+    dict(H=2, N=70, KV=100), dict(H=2, N=9, KV=63), dict(H=2, N=33, KV=37, mask="beam"), dict(H=2, N=100, KV=100, mask="causal"),
+    dict(H=2, N=130, KV=448, mask="causal"), dict(H=1, N=64, KV=20)])
+def test_flash_attn_f32_mode_matches_float64(pkg, oracle, gpu, case):
+    # MI355X_FA_F32: f32 accumulators.  More than 8 queries: both products on the matrix cores, probabilities rounded to f16
+    # (relative 2^-11 each, averaged over the keys); otherwise plain f32 arithmetic.
+    H, N, KV = case["H"], case["N"], case["KV"]
+    q, kb, vb = _attention_inputs(oracle, H, N, KV, case.get("flat", False), case.get("pad_from"))
+    mask = None
+    if "mask" in case:
+        m = np.full((-(-N // 64) * 64, KV), -np.inf, dtype=np.float32)
+        for r in range(N):
+            if case["mask"] == "causal":
+                m[r, : KV - N + r + 1] = 0.0
+            else:
+                m[r, : (KV + 1) // 2] = 0.0
+                m[r, [c for c in range(KV) if c % N == r]] = 0.0
+        mask = oracle.f32_to_f16_bits(m)
+    got, name = run_fa(pkg, gpu, q, kb, vb, mask, 0.125, pkg.FA_F32)
+    assert name == ("flash_attn.mfma_f32" if N > 8 else "flash_attn.vec_f32")
+    assert np.isfinite(got).all()
+    exact = _attention_float64(oracle, q, kb, vb, mask, 0.125)
+    assert oracle.nmse(got, exact) <= (1e-7 if N > 8 else 1e-9)
+    # north-star per-op bound against the CPU backend's own arithmetic (f16 accumulator rounded after every key)
+    assert oracle.nmse(got, oracle.flash_attn_ext(q, kb, vb, None if mask is None else mask[:N], 0.125)) <= 5e-4
+
+
+def test_flash_attn_f32_mode_emits_the_activation_image(pkg, oracle, gpu):
+    H, N, KV = 4, 100, 130
+    q, kb, vb = _attention_inputs(oracle, H, N, KV)
+    d_q, d_k, d_v = gpu.up(q), gpu.up(kb), gpu.up(vb)
+    d_o = torch.empty((N, H, 64), dtype=torch.float32, device=gpu.dev)
+    d_h = torch.zeros((N, H * 64), dtype=torch.float16, device=gpu.dev)
+    tq, tk, tv, to = pkg.tensor(d_q, pkg.F32), pkg.tensor(d_k, pkg.F16), pkg.tensor(d_v, pkg.F16), pkg.tensor(d_o, pkg.F32)
+    pkg.check(pkg.kernels().mi355x_flash_attn_ext(tq, tk, tv, None, to, 0.125, pkg.FA_F32 | pkg.FA_EMIT_F16, d_h.data_ptr(), d_h.numel() * 2, gpu.stream))
+    y = gpu.down(d_o).reshape(N, H * 64)
+    assert oracle.nmse(y, _attention_float64(oracle, q, kb, vb, None, 0.125).reshape(N, H * 64)) <= 1e-7
+    image = oracle.dequantize(oracle.Q8_0, oracle.quantize(oracle.Q8_0, y, act=True), H * 64).reshape(N, H * 64)
+    assert np.array_equal(gpu.down(d_h, np.uint16), oracle.f32_to_f16_bits(image))
 
 
 def test_flash_attn_strided_views_like_whisper(pkg, oracle, gpu):

@@ -80,8 +80,9 @@ struct mi355x_backend_ctx {
     bool        fuse    = true;
     bool        profile = false;
     bool        debug   = false;   // log what every MUL_MAT launch folds in (GGML_MI355X_DEBUG=1)
-    bool        fa_packed = false;      // attention over more than 8 queries accumulates with f16 fused multiply-adds (the
-                                        // arithmetic of the reference's Arm fp16 build) instead of f32 fma + f16 store
+    int         fa_accum = 0;           // V accumulation of attention over more than 8 queries: 0 the reference's x86 sequence (f32 fma,
+                                        // f16 store, key by key), 1 f32 accumulators on the matrix cores, 2 f16 fused multiply-adds
+                                        // key by key (the reference's Arm fp16 build)
     bool        weight_images = true;   // keep f16 images of quantized GEMM weights (GGML_MI355X_WEIGHT_IMAGES=0 turns it off)
     bool        exact   = false;   // true: f32 attention accumulators and un-rounded GEMM activations instead of the
                                    // reference's f16-sequential / Q8_0-rounded arithmetic

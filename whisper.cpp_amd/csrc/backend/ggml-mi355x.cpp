@@ -317,7 +317,8 @@ static ggml_backend_t device_init_backend(ggml_backend_dev_t dev, const char *) 
     ctx->fuse    = env_flag("GGML_MI355X_FUSE", true);
     ctx->profile = env_flag("GGML_MI355X_PROFILE", false);
     ctx->exact   = env_flag("GGML_MI355X_EXACT", false);
-    ctx->fa_packed = env_flag("GGML_MI355X_FA_PACKED", false);
+    ctx->fa_accum = env_flag("GGML_MI355X_FA_PACKED", false) ? 2 : 0;
+    if (const char * e = getenv("GGML_MI355X_FA_ACCUM")) { const int v = atoi(e); if (v >= 0 && v <= 2) ctx->fa_accum = v; }
     ctx->weight_images = env_flag("GGML_MI355X_WEIGHT_IMAGES", true);
     ctx->debug   = env_flag("GGML_MI355X_DEBUG", false);
     // default priority, blocking with respect to the null stream used by the buffer-level copies
@@ -400,14 +401,16 @@ static void ctx_synchronize(mi355x_backend_ctx * ctx) {
 static int set_option(ggml_backend_t backend, const char * name, int value) {
     if (!name || (backend && !ggml_backend_is_mi355x(backend))) return -1;
     const bool is_fuse = strcmp(name, "fuse") == 0, is_profile = strcmp(name, "profile") == 0, is_exact = strcmp(name, "exact") == 0;
-    const bool is_packed = strcmp(name, "fa_packed") == 0;
-    if (!is_fuse && !is_profile && !is_exact && !is_packed) return -1;
+    const bool is_packed = strcmp(name, "fa_packed") == 0, is_accum = strcmp(name, "fa_accum") == 0;
+    if (!is_fuse && !is_profile && !is_exact && !is_packed && !is_accum) return -1;
+    if (is_accum && (value < 0 || value > 2)) return -1;
     std::lock_guard<std::mutex> lock(g_live_mutex);
     for (mi355x_backend_ctx * ctx : g_live) {
         if (backend && ctx != (mi355x_backend_ctx *) backend->context) continue;
         if (is_fuse) ctx->fuse = value != 0;
         else if (is_exact) ctx->exact = value != 0;
-        else if (is_packed) ctx->fa_packed = value != 0;
+        else if (is_packed) ctx->fa_accum = value != 0 ? 2 : 0;
+        else if (is_accum) ctx->fa_accum = value;
         else { ctx_synchronize(ctx); ctx->profile = value != 0; }
     }
     return 0;

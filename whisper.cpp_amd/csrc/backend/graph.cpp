@@ -551,10 +551,13 @@ struct graph_runner {
                 if (m) vm = to_view(m);
                 const double flops = 4.0 * s0->ne[1] * k->ne[1] * 64.0 * s0->ne[2] * s0->ne[3];
                 const double bytes = (double) ggml_nelements(s0) * 4 + 2.0 * (double) k->ne[0] * k->ne[1] * k->ne[2] * k->ne[3] * 2 + nbytes_of(n);
-                const int mode = ctx->exact ? MI355X_FA_F32 : ctx->fa_packed ? MI355X_FA_F16_PACKED : MI355X_FA_F16_SEQ;
+                // the accumulation option is for the many-query kernels; a decode step keeps the reference's sequence
+                const int accum = s0->ne[1] > 8 ? ctx->fa_accum : 0;
+                const int mode = ctx->exact || accum == 1 ? MI355X_FA_F32 : accum == 2 ? MI355X_FA_F16_PACKED : MI355X_FA_F16_SEQ;
                 const char * name = mi355x_flash_attn_ext_kernel_name(&vq, &vk, mode);
                 // the output projection that follows takes its Q8_0-rounded activations from the attention kernel itself
-                const ggml_tensor * key = strncmp(name, "flash_attn.seq_tile", 19) == 0 ? image_consumer(n, i + 1) : nullptr;
+                const bool emits = !ctx->exact && (strncmp(name, "flash_attn.seq_tile", 19) == 0 || strcmp(name, "flash_attn.mfma_f32") == 0);
+                const ggml_tensor * key = emits ? image_consumer(n, i + 1) : nullptr;
                 const size_t image_bytes = (size_t) ggml_nelements(n) * 2;
                 if (key && !ctx->reserve_workspace(image_bytes + 256)) key = nullptr;
                 {

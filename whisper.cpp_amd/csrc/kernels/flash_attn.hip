@@ -15,8 +15,10 @@
 //                                  v_fma_mixlo/hi_f16 chains against the LDS-staged V tile.
 //       k_fattn_seq_row    N <= 8: one block per (query, head): 256 threads score all keys and scan the maximum,
 //                                  one wavefront (lane = d) runs the chain with V streamed from global memory.
-//   MI355X_FA_F32          f32 accumulators, keys split across lanes (k_fattn_vec): closer to exact arithmetic,
-//                          not to the reference.
+//   MI355X_FA_F32          f32 accumulators: closer to exact arithmetic, not to the reference (whose f16 accumulator
+//                          loses about 1e-4 NMSE per attention, which whole-model logits then show as several 1e-3).
+//       k_fattn_mfma       N > 8:  both products on the matrix cores, online softmax, probabilities as f16 operands
+//       k_fattn_vec        N <= 8: one wavefront per (query, head), keys split across lanes
 #include "common.h"
 
 #define FA_D 64
@@ -635,16 +637,213 @@ __global__ void __launch_bounds__(256) k_fattn_seq_tile(fa_args a) {
 }
 
 // ------------------------------------------------------------------------------------------------------
+// N > 8, f32 accumulators on the matrix cores (MI355X_FA_F32).
+//
+// Both products run on v_mfma_f32_32x32x16_f16, transposed so that a lane owns one query throughout:
+//   S^T = K Q^T     (32 keys x 32 queries per wavefront; Q^T is the B operand and stays in registers for the whole kernel)
+//   O^T += V^T P^T  (64 d x 32 queries; P^T = exp2(S^T - m) leaves the accumulator registers of the first product in the
+//                    very lanes that need it as the B operand of the second, once the keys of a block are visited in the
+//                    order those registers hold them — the V^T operand is read from LDS in the same order)
+// so the running maximum and sum are per-lane scalars (one exchange with lane ^ 32 per tile) and the rescale of O is a
+// per-lane multiply.  A workgroup is 64 queries of one head; wavefront w takes queries 32 * (w / 2) and the keys
+// 32 * (w % 2) .. + 31 of each 64-key tile with a softmax state of its own, and the two states of a query are merged at
+// the end.  K tiles go to LDS as they are; V tiles are transposed on the way in (two keys packed per 32-bit store), both
+// double buffered with the next tile's global loads in flight.
+// ------------------------------------------------------------------------------------------------------
+
+#define M_Q   64
+#define M_KV  64
+#define M_LDK (FA_D + 8)      // f16 pitch of a K row
+#define M_LDV (M_KV + 4)      // f16 pitch of a V^T row (136 B: the b64 operand reads of 32 d-rows cover all banks once)
+#define LOG2E 1.44269504088896340736f
+
+__global__ void __launch_bounds__(256) k_fattn_mfma(fa_args a) {
+    __shared__ __attribute__((aligned(16))) half_t k_s[2][M_KV * M_LDK];
+    __shared__ __attribute__((aligned(16))) half_t vt_s[2][FA_D * M_LDV];
+
+    const int tid = threadIdx.x, lane = tid & 63, l32 = lane & 31, g = lane >> 5;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wq = (wave >> 1) * 32, wk = (wave & 1) * 32;
+    const int64_t n0 = (int64_t) blockIdx.x * M_Q, h = blockIdx.y, i3 = blockIdx.z;
+    const char * qb = a.q + h * a.q_nb2 + i3 * a.q_nb3;
+    const char * kb = a.k + (h / a.hk_ratio) * a.k_nb2 + (i3 / a.k_ne3_ratio) * a.k_nb3;
+    const char * vb = a.v + (h / a.hv_ratio) * a.v_nb2 + (i3 / a.v_ne3_ratio) * a.v_nb3;
+
+    // B operand of the first product: lane (query l32, half g) holds q[16 kk + 8 g .. + 7], rounded to f16 as the CPU backend does
+    const int64_t n  = n0 + wq + l32;
+    const int64_t nc = n < a.N ? n : a.N - 1;
+    half8_t qf[FA_D / 16];
+    {
+        const float * qp = (const float *)(qb + nc * a.q_nb1);
+#pragma unroll
+        for (int kk = 0; kk < FA_D / 16; ++kk) {
+            const float4 t0 = *(const float4 *)(qp + 16 * kk + 8 * g), t1 = *(const float4 *)(qp + 16 * kk + 8 * g + 4);
+            qf[kk] = (half8_t){ (half_t) t0.x, (half_t) t0.y, (half_t) t0.z, (half_t) t0.w, (half_t) t1.x, (half_t) t1.y, (half_t) t1.z, (half_t) t1.w };
+        }
+    }
+    const half_t * mrow = a.mask ? (const half_t *)(a.mask + nc * a.m_nb1) : nullptr;
+    const bool mask_al8 = (((uintptr_t) a.mask | (uintptr_t) a.m_nb1) & 7) == 0;      // rows of the mask can be read four keys at a time
+
+    // staging roles: K: thread t -> key t / 4, 32 bytes; V: thread t -> keys 2 (t / 8) and + 1, d 8 (t % 8) .. + 7
+    const int kr = tid >> 2, kc = (tid & 3) * 16;
+    const int vp = tid >> 3, vc = (tid & 7) * 8;
+    u32x4 kreg0, kreg1, vreg0, vreg1;
+    auto load_kv = [&](int64_t key0) __attribute__((always_inline)) {
+        const int64_t last = a.KV - 1;                    // rows past the end repeat the last key; their scores are masked
+        const int64_t kk = key0 + kr < last ? key0 + kr : last;
+        const int64_t v0 = key0 + 2 * vp < last ? key0 + 2 * vp : last, v1 = key0 + 2 * vp + 1 < last ? key0 + 2 * vp + 1 : last;
+        const u32x4 * kp = (const u32x4 *)(kb + kk * a.k_nb1 + kc * 2);
+        kreg0 = kp[0]; kreg1 = kp[1];
+        vreg0 = *(const u32x4 *)(vb + v0 * a.v_nb1 + vc * 2);
+        vreg1 = *(const u32x4 *)(vb + v1 * a.v_nb1 + vc * 2);
+    };
+    auto store_kv = [&](int b) __attribute__((always_inline)) {
+        *(u32x4 *)(k_s[b] + kr * M_LDK + kc) = kreg0; *(u32x4 *)(k_s[b] + kr * M_LDK + kc + 8) = kreg1;
+        uint32_t * vt = (uint32_t *)(vt_s[b] + vc * M_LDV) + vp;          // V^T[d = vc + j][keys 2 vp, 2 vp + 1]
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            vt[(2 * i    ) * (M_LDV / 2)] = (vreg0[i] & 0xffffu) | (vreg1[i] << 16);
+            vt[(2 * i + 1) * (M_LDV / 2)] = (vreg0[i] >> 16) | (vreg1[i] & 0xffff0000u);
+        }
+    };
+
+    float16_t o[2];
+#pragma unroll
+    for (int r = 0; r < 16; ++r) { o[0][r] = 0.0f; o[1][r] = 0.0f; }
+    float m = -1.0e30f, l = 0.0f;                          // log2 domain; finite so that a fully masked tile gives factors of 0, not NaN
+    const float c = a.scale * LOG2E;
+
+    const int nt = (int)((a.KV + M_KV - 1) / M_KV);
+    load_kv(0);
+    for (int t = 0; t < nt; ++t) {
+        const int b = t & 1;
+        const int64_t key0 = (int64_t) t * M_KV;
+        store_kv(b);
+        __syncthreads();                                   // tile t visible; everyone is done with tile t - 1, whose buffer the next store reuses
+        if (t + 1 < nt) load_kv(key0 + M_KV);
+
+        float16_t sc;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) sc[r] = 0.0f;
+#pragma unroll
+        for (int kk = 0; kk < FA_D / 16; ++kk) {
+            const half8_t av = *(const half8_t *)(k_s[b] + (wk + l32) * M_LDK + 16 * kk + 8 * g);
+            sc = __builtin_amdgcn_mfma_f32_32x32x16_f16(av, qf[kk], sc, 0, 0, 0);
+        }
+        // register r: key key0 + wk + 8 (r / 4) + 4 g + r % 4, query l32
+        float tv[16];
+        if (mrow) {
+            half4_t mk[4];
+#pragma unroll
+            for (int q4 = 0; q4 < 4; ++q4) {
+                const int64_t key = key0 + wk + 8 * q4 + 4 * g;
+                if (mask_al8 && key + 3 < a.KV) mk[q4] = *(const half4_t *)(mrow + key);
+                else {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) mk[q4][e] = mrow[key + e < a.KV ? key + e : a.KV - 1];   // past the end: masked below
+                }
+            }
+#pragma unroll
+            for (int r = 0; r < 16; ++r) tv[r] = __builtin_fmaf(sc[r], c, (float) mk[r >> 2][r & 3] * LOG2E);
+        } else {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) tv[r] = sc[r] * c;
+        }
+        if (key0 + M_KV > a.KV) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) if (key0 + wk + 8 * (r >> 2) + 4 * g + (r & 3) >= a.KV) tv[r] = -INFINITY;
+        }
+        float tmax = tv[0];
+#pragma unroll
+        for (int r = 1; r < 16; ++r) tmax = fmaxf(tmax, tv[r]);
+        tmax = fmaxf(tmax, __shfl_xor(tmax, 32, WAVE));
+        const float m_new = fmaxf(m, tmax);
+        if (__any(m_new > m)) {
+            const float alpha = __builtin_amdgcn_exp2f(m - m_new);
+            l *= alpha;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) { o[0][r] *= alpha; o[1][r] *= alpha; }
+            m = m_new;
+        }
+        half8_t ph[2];
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const float p = __builtin_amdgcn_exp2f(tv[r] - m);
+            l += p;
+            ph[r >> 3][r & 7] = (half_t) p;
+        }
+#pragma unroll
+        for (int db = 0; db < 2; ++db) {
+#pragma unroll
+            for (int ks = 0; ks < 2; ++ks) {
+                const half_t * vr = vt_s[b] + (32 * db + l32) * M_LDV + wk + 16 * ks + 4 * g;
+                const half4_t lo = *(const half4_t *) vr, hi = *(const half4_t *)(vr + 8);
+                const half8_t av = { lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3] };
+                o[db] = __builtin_amdgcn_mfma_f32_32x32x16_f16(av, ph[ks], o[db], 0, 0, 0);
+            }
+        }
+    }
+    l += __shfl_xor(l, 32, WAVE);
+
+    // merge the two key halves of each query: this wavefront finishes d block (wave & 1) and hands the other block over
+    __syncthreads();                                       // the tiles are no longer needed
+    float * xch = (float *) k_s;                           // [wave][16][64] f32 = 16 KB of the 18 KB
+    float * ml  = (float *) vt_s;                          // [wave][2][64]
+    const bool odd = wave & 1;
+    const float16_t mine = odd ? o[1] : o[0], send = odd ? o[0] : o[1];
+#pragma unroll
+    for (int r = 0; r < 16; ++r) xch[(wave * 16 + r) * 64 + lane] = send[r];
+    ml[(wave * 2 + 0) * 64 + lane] = m; ml[(wave * 2 + 1) * 64 + lane] = l;
+    __syncthreads();
+    const int pw = wave ^ 1;
+    const float pm = ml[(pw * 2 + 0) * 64 + lane], pl = ml[(pw * 2 + 1) * 64 + lane];
+    const float mm = fmaxf(m, pm);
+    const float fa = __builtin_amdgcn_exp2f(m - mm), fb = __builtin_amdgcn_exp2f(pm - mm);
+    const float inv = 1.0f / (l * fa + pl * fb);
+    float out[16];
+#pragma unroll
+    for (int r = 0; r < 16; ++r) out[r] = (mine[r] * fa + xch[(pw * 16 + r) * 64 + lane] * fb) * inv;
+
+    // out[r]: d = 32 (wave & 1) + 8 (r / 4) + 4 g + r % 4 of query n
+    const int64_t row = ((i3 * a.N + n) * a.H + h) * FA_D + 32 * (wave & 1) + 4 * g;
+    if (n < a.N) {
+        float * dp = (float *) a.d + row;
+#pragma unroll
+        for (int q4 = 0; q4 < 4; ++q4) *(float4 *)(dp + 8 * q4) = make_float4(out[4*q4], out[4*q4 + 1], out[4*q4 + 2], out[4*q4 + 3]);
+    }
+    if (a.x16) {
+        // the Q8_0-rounded image for the projection that follows: one block = the 32 d of this wavefront's block of a query,
+        // half of them here and half in lane ^ 32
+        float amax = 0.0f;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) amax = fmaxf(amax, fabsf(out[r]));
+        amax = fmaxf(amax, __shfl_xor(amax, 32, WAVE));
+        if (n < a.N) {
+            const float id = amax != 0.0f ? 127.0f / amax : 0.0f;
+            const float dq = h2f(f2h_bits(amax / 127.0f));
+            half_t * xp = a.x16 + row;
+#pragma unroll
+            for (int q4 = 0; q4 < 4; ++q4) {
+                half4_t hv;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) hv[e] = (half_t)((rintf(out[4*q4 + e] * id) + 0.0f) * dq);
+                *(half4_t *)(xp + 8 * q4) = hv;
+            }
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------------------
 // host dispatch
 // ------------------------------------------------------------------------------------------------------
 
 #define SEQ_ROW_MAX_N   8
 #define SEQ_ROW_MAX_KV  7168      // two f32 arrays of that many keys stay under 64 KB of LDS
 
-enum { FA_K_VEC = 0, FA_K_SEQ_ROW = 1, FA_K_SEQ_TILE = 2 };
+enum { FA_K_VEC = 0, FA_K_SEQ_ROW = 1, FA_K_SEQ_TILE = 2, FA_K_MFMA = 3 };
 
 static int fa_kernel(const mi355x_tensor * q, const mi355x_tensor * k, int mode) {
-    if (mode == MI355X_FA_F32) return FA_K_VEC;
+    if (mode == MI355X_FA_F32) return q->ne[1] > SEQ_ROW_MAX_N ? FA_K_MFMA : FA_K_VEC;
     if (q->ne[1] <= SEQ_ROW_MAX_N && k->ne[1] <= SEQ_ROW_MAX_KV) return FA_K_SEQ_ROW;
     return FA_K_SEQ_TILE;
 }
@@ -654,6 +853,7 @@ extern "C" const char * mi355x_flash_attn_ext_kernel_name(const mi355x_tensor * 
     switch (fa_kernel(q, k, mode)) {
         case FA_K_SEQ_ROW:  return "flash_attn.seq_row";
         case FA_K_SEQ_TILE: return mode == MI355X_FA_F16_PACKED ? "flash_attn.seq_tile_packed" : "flash_attn.seq_tile";
+        case FA_K_MFMA:     return "flash_attn.mfma_f32";
         default:            return "flash_attn.vec_f32";
     }
 }
@@ -701,8 +901,8 @@ extern "C" int mi355x_flash_attn_ext(const mi355x_tensor * q, const mi355x_tenso
     a.scale = scale;
     a.x16 = nullptr;
     if (emit) {
-        // only the tile kernel in the reference's arithmetic writes the image; say so rather than silently skip it
-        if (fa_kernel(q, k, mode) != FA_K_SEQ_TILE || mode == MI355X_FA_F32) return MI355X_ERR_UNSUPPORTED;
+        // only the tile kernels write the image; say so rather than silently skip it
+        if (fa_kernel(q, k, mode) != FA_K_SEQ_TILE && fa_kernel(q, k, mode) != FA_K_MFMA) return MI355X_ERR_UNSUPPORTED;
         if (!workspace || (uintptr_t) workspace % 16 != 0 || workspace_size < (size_t)(N * H * q->ne[3]) * FA_D * sizeof(half_t)) return MI355X_ERR_WORKSPACE;
         a.x16 = (half_t *) workspace;
     }
@@ -728,6 +928,11 @@ extern "C" int mi355x_flash_attn_ext(const mi355x_tensor * q, const mi355x_tenso
             dim3 grid((unsigned) gx, (unsigned) H, (unsigned) q->ne[3]);
             if (mode == MI355X_FA_F16_PACKED) k_fattn_seq_tile<true ><<<grid, 256, 0, st>>>(a);
             else                              k_fattn_seq_tile<false><<<grid, 256, 0, st>>>(a);
+        } break;
+        case FA_K_MFMA: {
+            const int64_t gx = (N + M_Q - 1) / M_Q;
+            if (gx > 0x7fffffff) return MI355X_ERR_UNSUPPORTED;
+            k_fattn_mfma<<<dim3((unsigned) gx, (unsigned) H, (unsigned) q->ne[3]), 256, 0, st>>>(a);
         } break;
         default: {
             const int64_t waves = N * H * q->ne[3];
