@@ -190,6 +190,13 @@ MI355X_API int mi355x_norm(const mi355x_tensor * src, const mi355x_tensor * dst,
  * 16-byte aligned rows; MI355X_ERR_UNSUPPORTED otherwise. */
 MI355X_API int mi355x_norm_emit_f16(const mi355x_tensor * src, const mi355x_tensor * dst, float eps, const float * w, const float * b,
                                     void * x16, void * stream);
+/* The same for the few-column product (N <= 8) over quantized weights: the result quantized to Q8_0 itself, in the layout
+ * mi355x_mul_mat's quantization pass writes into its workspace for that path —
+ *   int8 q[rows][ne0] | float d[rows][ne0/32] (the f16-rounded scales) | int32 s[rows][ne0/32] (sum of a block's quants)
+ * — at `q8` (16-byte aligned, mi355x_mul_mat_workspace_size bytes of the product that follows).  2-d src; otherwise the
+ * conditions of mi355x_norm_emit_f16. */
+MI355X_API int mi355x_norm_emit_q8_0(const mi355x_tensor * src, const mi355x_tensor * dst, float eps, const float * w, const float * b,
+                                     void * q8, void * stream);
 
 /* SOFT_MAX (ggml/src/ggml-cpu/ops.cpp:4641-4737), max_bias = 0: softmax(scale * x + mask) over ne0.
  * mask F32 or F16 [ne0, >= ne1], broadcast over ne2/ne3, or NULL. */

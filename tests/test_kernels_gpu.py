@@ -48,7 +48,7 @@ def gpu(pkg):
     return G
 
 
-def run_mul_mat(pkg, gpu, wtype, wdata, x, k, m, flags=0, bias=None, resid=None, scale=1.0, out_f16=False):
+def run_mul_mat(pkg, gpu, wtype, wdata, x, k, m, flags=0, bias=None, resid=None, scale=1.0, out_f16=False, workspace=True):
     lib = pkg.kernels()
     d_w, d_x = gpu.up(wdata), gpu.up(x)
     n = x.shape[0]
@@ -56,7 +56,7 @@ def run_mul_mat(pkg, gpu, wtype, wdata, x, k, m, flags=0, bias=None, resid=None,
     tw = pkg.tensor(d_w, wtype, ne=[k, m])
     tx = pkg.tensor(d_x, pkg.F32)
     ty = pkg.tensor(d_y, pkg.F16 if out_f16 else pkg.F32)
-    ws_size = lib.mi355x_mul_mat_workspace_size(tw, tx)
+    ws_size = lib.mi355x_mul_mat_workspace_size(tw, tx) if workspace else 0
     ws = torch.empty(max(ws_size, 16), dtype=torch.uint8, device=gpu.dev)
     epi = pkg.Epilogue()
     epi.flags, epi.scale = flags | (pkg.EPI_OUT_F16 if out_f16 else 0), scale
@@ -117,6 +117,43 @@ def test_mul_mat_quantized(pkg, oracle, gpu, wtype, shape):
         got = got[:, sel]
     # both paths reproduce the reference's Q8_0 rounding of the activations: NMSE <= 1e-6 (GEMV: integer dot products, <= 1e-10)
     assert oracle.nmse(got, want) <= (1e-10 if n <= 8 else 1e-6)
+    if n <= 8:
+        # without a workspace every workgroup quantizes the activations for itself: the same integers, another summation order
+        alone, _ = run_mul_mat(pkg, gpu, t, blocks, x, k, m, workspace=False)
+        assert oracle.nmse(alone if n * m * k <= 2e9 else alone[:, sel], want) <= 1e-10
+
+
+def test_gemv_over_activations_quantized_ahead(pkg, oracle, gpu):
+    # MI355X_MM_PREPARE_ONLY leaves the quantized activations in the workspace; products over them pass MI355X_MM_WS_READY
+    lib = pkg.kernels()
+    k, n = 1280, 5
+    x = rnd((n, k))
+    d_x = gpu.up(x)
+    tx = pkg.tensor(d_x, pkg.F32)
+    mats = [(pkg.Q8_0, 1280), (pkg.Q8_0, 640), (pkg.Q5_0, 5120)]
+    ws = None
+    for step, (t, m) in enumerate(mats):
+        blocks = oracle.quantize(t, rnd((m, k), 0.02))
+        d_w = gpu.up(blocks)
+        tw = pkg.tensor(d_w, t, ne=[k, m])
+        need = lib.mi355x_mul_mat_workspace_size(tw, tx)
+        assert need >= n * k + n * (k // 32) * 8
+        epi = pkg.Epilogue()
+        if ws is None:
+            ws = torch.zeros(need, dtype=torch.uint8, device=gpu.dev)
+            epi.flags = pkg.MM_PREPARE_ONLY
+            pkg.check(lib.mi355x_mul_mat(tw, tx, pkg.tensor(torch.empty((n, m), device=gpu.dev), pkg.F32), C.byref(epi), ws.data_ptr(), need, gpu.stream))
+            image = gpu.down(ws)
+            q = oracle.quantize(oracle.Q8_0, x, act=True).reshape(n, k // 32, 34)
+            assert np.array_equal(image[: n * k].reshape(n, k // 32, 32), q[:, :, 2:])
+            scales = image[n * k : n * k + n * (k // 32) * 4].view(np.float32).reshape(n, k // 32)
+            assert np.array_equal(scales, oracle.f16_bits_to_f32(q[:, :, :2].copy().view(np.uint16)[..., 0]))
+        assert need <= ws.numel()
+        d_y = torch.zeros((n, m), dtype=torch.float32, device=gpu.dev)
+        epi.flags = pkg.MM_WS_READY
+        d_x.zero_() if step == len(mats) - 1 else None      # the last product must not look at src1 any more
+        pkg.check(lib.mi355x_mul_mat(tw, tx, pkg.tensor(d_y, pkg.F32), C.byref(epi), ws.data_ptr(), need, gpu.stream))
+        assert oracle.nmse(gpu.down(d_y), oracle.mul_mat(t, blocks, x)) <= 1e-10
 
 
 @pytest.mark.parametrize("wtype", ["F16", "F32"])
@@ -423,6 +460,21 @@ def test_norm_and_affine(pkg, oracle, gpu):
             assert np.array_equal(gpu.down(d_h, np.uint16), oracle.f32_to_f16_bits(image))
         else:
             assert rc == -1                      # unsupported shapes say so; the caller falls back to the plain kernel
+        # and the variant for the few-column product: Q8_0 itself, quants | scales | block sums
+        n, k = shape
+        d_q = torch.zeros(n * k + n * (k // 32 + 1) * 8, dtype=torch.uint8, device=gpu.dev)
+        rc = lib.mi355x_norm_emit_q8_0(pkg.tensor(d_x, pkg.F32), pkg.tensor(d_y, pkg.F32), 1e-5, d_w.data_ptr(), d_b.data_ptr(), d_q.data_ptr(), gpu.stream)
+        if k % 32 == 0 and k <= 2048:
+            pkg.check(rc)
+            y, image = gpu.down(d_y), gpu.down(d_q)
+            q = oracle.quantize(oracle.Q8_0, y, act=True).reshape(n, k // 32, 34)
+            assert np.array_equal(image[: n * k].reshape(n, k // 32, 32), q[:, :, 2:])
+            assert np.array_equal(image[n * k : n * k + n * (k // 32) * 4].view(np.float32).reshape(n, k // 32),
+                                  oracle.f16_bits_to_f32(q[:, :, :2].copy().view(np.uint16)[..., 0]))
+            sums = image[n * k + n * (k // 32) * 4 : n * k + n * (k // 32) * 8].view(np.int32).reshape(n, k // 32)
+            assert np.array_equal(sums, q[:, :, 2:].view(np.int8).astype(np.int32).sum(-1))
+        else:
+            assert rc == -1
 
 
 def test_gelu_scale_binary(pkg, oracle, gpu):

@@ -78,6 +78,7 @@ def kernels() -> C.CDLL:
             "mi355x_gelu": (C.c_int, [T, T, P]),
             "mi355x_norm": (C.c_int, [T, T, C.c_float, P, P, P]),
             "mi355x_norm_emit_f16": (C.c_int, [T, T, C.c_float, P, P, P, P]),
+            "mi355x_norm_emit_q8_0": (C.c_int, [T, T, C.c_float, P, P, P, P]),
             "mi355x_soft_max": (C.c_int, [T, T, T, C.c_float, P]),
             "mi355x_cpy": (C.c_int, [T, T, P]),
             "mi355x_get_rows": (C.c_int, [T, T, T, P]),

@@ -294,15 +294,17 @@ struct graph_runner {
         return o;
     }
 
-    // The GEMM first brings src1 to f16 (rounded to Q8_0 on the way when the weights are quantized) in the workspace;
-    // consecutive MUL_MATs over the same activations share that copy.  Runs (and times) the conversion when the workspace
+    // The GEMM first brings src1 to f16 (rounded to Q8_0 on the way when the weights are quantized) in the workspace, the
+    // few-column product over quantized weights brings it to Q8_0; consecutive MUL_MATs over the same activations share
+    // that copy.  Runs (and times) the conversion when the workspace
     // does not hold it yet; returns the MM flags to add (WS_READY), or -1 with `status` set.
     int prepare_src1(const mm_chain & c, const mm_operands & o, size_t need, int & status) {
         if (!need) return 0;
         if (!ctx->reserve_workspace(need)) { status = MI355X_ERR_WORKSPACE; return -1; }
         const ggml_tensor * x = c.x;
         if (x->type != GGML_TYPE_F32) return 0;
-        const int mode = (ggml_is_quantized(c.w->type) && !ctx->exact) ? 1 : 0;       // 1: rounded to Q8_0
+        const bool gemv = strncmp(o.kernel_name, "mul_mat.gemv", 12) == 0;
+        const int mode = gemv ? 2 : (ggml_is_quantized(c.w->type) && !ctx->exact) ? 1 : 0;       // 1: f16 rounded to Q8_0, 2: Q8_0 itself
         const bool hit = ctx->ws_x == x->data && ctx->ws_x_mode == mode && memcmp(ctx->ws_x_ne, x->ne, sizeof(x->ne)) == 0 &&
                          memcmp(ctx->ws_x_nb, x->nb, sizeof(x->nb)) == 0;
         ctx->ws_x = x->data; ctx->ws_x_mode = mode; memcpy(ctx->ws_x_ne, x->ne, sizeof(x->ne)); memcpy(ctx->ws_x_nb, x->nb, sizeof(x->nb));
@@ -310,7 +312,7 @@ struct graph_runner {
         if (!hit) {
             mi355x_epilogue prep = c.epi;                 // same call as the product itself, stopped after the conversion
             prep.flags |= o.mm_flags | MI355X_MM_PREPARE_ONLY;
-            launch_scope ls(ctx, "mul_mat.src1_to_f16", nbytes_of(x) * 1.5, 0.0);
+            launch_scope ls(ctx, gemv ? "mul_mat.src1_to_q8_0" : "mul_mat.src1_to_f16", nbytes_of(x) * (gemv ? 1.3125 : 1.5), 0.0);
             status = mi355x_mul_mat(&o.vw, &o.vx, &o.vd, &prep, ctx->ws, ctx->ws_size, ctx->stream);
             if (status != MI355X_OK) return -1;
         }
@@ -415,7 +417,8 @@ struct graph_runner {
     // When everything that reads `out` (produced just before node `from`) — directly, or through one dense 2-d RESHAPE of
     // it — is a many-column product with quantized weights, the producer can leave the Q8_0-rounded f16 image those
     // products want in the workspace and they skip their conversion pass.  Returns the tensor the products name as src1.
-    const ggml_tensor * image_consumer(const ggml_tensor * out, int from) const {
+    // `few`: the same question for the few-column products, which read their activations as Q8_0 from the workspace.
+    const ggml_tensor * image_consumer(const ggml_tensor * out, int from, bool few = false) const {
         if (!ctx->fuse || ctx->exact || (out->flags & GGML_TENSOR_FLAG_OUTPUT) || !ggml_is_contiguous(out)) return nullptr;
         const ggml_tensor * key = out;
         for (int hop = 0; hop < 2; ++hop) {
@@ -430,7 +433,12 @@ struct graph_runner {
                 for (int k = 0; k < GGML_MAX_SRC; ++k) reads = reads || n->src[k] == key;
                 if (!reads) continue;
                 ++seen;
-                if (n->op == GGML_OP_MUL_MAT && n->src[1] == key && n->src[0] != key && ggml_is_quantized(n->src[0]->type)) continue;
+                if (n->op == GGML_OP_MUL_MAT && n->src[1] == key && n->src[0] != key && ggml_is_quantized(n->src[0]->type)) {
+                    if (!few) continue;
+                    mi355x_tensor vw = to_view(n->src[0]), vx = to_view(key);
+                    if (mi355x_mul_mat_workspace_size(&vw, &vx) > 0 && strncmp(mi355x_mul_mat_kernel_name(&vw, &vx), "mul_mat.gemv", 12) == 0) continue;
+                    return nullptr;
+                }
                 if (want == 1 && hop == 0 && n->op == GGML_OP_RESHAPE && n->src[0] == key && ggml_is_contiguous(n) && !(n->flags & GGML_TENSOR_FLAG_OUTPUT)) { reshape = n; continue; }
                 return nullptr;
             }
@@ -438,14 +446,14 @@ struct graph_runner {
             if (!reshape) break;
             key = reshape;
         }
-        if (key->ne[2] != 1 || key->ne[3] != 1 || key->ne[1] <= MI355X_GEMV_MAX_COLS || key->ne[0] % 32 != 0) return nullptr;
+        if (key->ne[2] != 1 || key->ne[3] != 1 || (key->ne[1] <= MI355X_GEMV_MAX_COLS) != few || key->ne[0] % 32 != 0) return nullptr;
         return key;
     }
     void * slot_ptr(int slot) const { return (char *) ctx->ws_base + (size_t) slot * ctx->ws_size; }
     // the image of `key` now sits in `slot`, which becomes the current one
-    void workspace_holds(const ggml_tensor * key, int slot) {
+    void workspace_holds(const ggml_tensor * key, int slot, int mode = 1) {
         ctx->ws_slot = slot; ctx->ws = slot_ptr(slot);
-        ctx->ws_x = key->data; ctx->ws_x_mode = 1; memcpy(ctx->ws_x_ne, key->ne, sizeof(key->ne)); memcpy(ctx->ws_x_nb, key->nb, sizeof(key->nb));
+        ctx->ws_x = key->data; ctx->ws_x_mode = mode; memcpy(ctx->ws_x_ne, key->ne, sizeof(key->ne)); memcpy(ctx->ws_x_nb, key->nb, sizeof(key->nb));
         cached_x = key;
     }
 
@@ -469,15 +477,20 @@ struct graph_runner {
         mi355x_tensor vs = to_view(nm->src[0]), vd = to_view(out);
         // When everything that reads the result is a many-column product with quantized weights, the kernel also leaves
         // the Q8_0-rounded f16 image those products want in the workspace, and they skip their conversion pass.
+        // (A decode step's few-column products read Q8_0 itself; then the kernel leaves that.)
         const ggml_tensor * key = out->ne[0] <= 2048 ? image_consumer(out, i + used) : nullptr;
-        bool emit = key && ctx->reserve_workspace((size_t)(out->ne[0] * out->ne[1] * 2 + 256));
+        int mode = 1;
+        if (!key && out->ne[0] <= 2048 && (key = image_consumer(out, i + used, true))) mode = 2;
+        const size_t image_bytes = mode == 1 ? (size_t)(out->ne[0] * out->ne[1] * 2) : (size_t)(out->ne[0] * out->ne[1] + out->ne[0] / 32 * out->ne[1] * 8);
+        bool emit = key && ctx->reserve_workspace(image_bytes + 256);
         {
-            launch_scope ls(ctx, used == 3 ? (emit ? "norm_affine_emit" : "norm_affine") : "norm", nbytes_of(nm->src[0]) + nbytes_of(out) * (emit ? 1.5 : 1.0), 0.0);
-            status = emit ? mi355x_norm_emit_f16(&vs, &vd, eps, w, b, ctx->ws, ctx->stream) : mi355x_norm(&vs, &vd, eps, w, b, ctx->stream);
+            launch_scope ls(ctx, used == 3 ? (emit ? "norm_affine_emit" : "norm_affine") : "norm", nbytes_of(nm->src[0]) + nbytes_of(out) + (emit ? image_bytes : 0), 0.0);
+            status = !emit ? mi355x_norm(&vs, &vd, eps, w, b, ctx->stream)
+                   : mode == 1 ? mi355x_norm_emit_f16(&vs, &vd, eps, w, b, ctx->ws, ctx->stream) : mi355x_norm_emit_q8_0(&vs, &vd, eps, w, b, ctx->ws, ctx->stream);
         }
         if (emit && status == MI355X_ERR_UNSUPPORTED) { emit = false; status = mi355x_norm(&vs, &vd, eps, w, b, ctx->stream); }
         note_write(out);
-        if (emit && status == MI355X_OK) workspace_holds(key, ctx->ws_slot);
+        if (emit && status == MI355X_OK) workspace_holds(key, ctx->ws_slot, mode);
         return used;
     }
 

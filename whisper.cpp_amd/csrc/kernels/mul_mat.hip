@@ -534,6 +534,50 @@ __device__ __forceinline__ wraw<T0> load_wraw(const uint8_t * wrow, int kb) {
     return r;
 }
 
+// X -> Q8_0 in LDS (int32 xq[NC][K/4] | float xd[NC][K/32] | int32 xsum[NC][K/32]) by the 256 threads of a workgroup
+template <int NC>
+__device__ __forceinline__ void quantize_x_to_lds(const mm_args & a, int32_t * xq, float * xd, int32_t * xsum, int nbk) {
+    const int64_t K = a.K;
+    // --- quantize X: 8 lanes per 32-value block, round-to-nearest-even like _mm256_round_ps(_MM_ROUND_NEAREST).
+    // Eight independent loads per thread are in flight before the first is consumed.
+    {
+        const int total = NC * nbk * 8;                         // float4 pieces
+        const int k8 = nbk * 8;
+        for (int base = 0; base < total; base += 256 * 8) {
+            float4 v[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const int idx = base + u * 256 + (int) threadIdx.x;
+                v[u] = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (idx < total) v[u] = *(const float4 *)(a.x + (int64_t)(idx / k8) * a.x_nb1 + (int64_t)(idx % k8) * 16);
+            }
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const int idx = base + u * 256 + (int) threadIdx.x;      // lanes 8i .. 8i+7 share a block
+                float amax = fmaxf(fmaxf(fabsf(v[u].x), fabsf(v[u].y)), fmaxf(fabsf(v[u].z), fabsf(v[u].w)));
+                amax = fmaxf(amax, __shfl_xor(amax, 1, 8));
+                amax = fmaxf(amax, __shfl_xor(amax, 2, 8));
+                amax = fmaxf(amax, __shfl_xor(amax, 4, 8));
+                const float d  = amax / 127.0f;
+                const float id = amax != 0.0f ? 127.0f / amax : 0.0f;
+                const int q0 = (int) rintf(v[u].x * id), q1 = (int) rintf(v[u].y * id), q2 = (int) rintf(v[u].z * id), q3 = (int) rintf(v[u].w * id);
+                int sum = q0 + q1 + q2 + q3;
+                sum += __shfl_xor(sum, 1, 8);
+                sum += __shfl_xor(sum, 2, 8);
+                sum += __shfl_xor(sum, 4, 8);
+                if (idx < total) {
+                    const int n = idx / k8, c = idx % k8;       // c: float4 piece within the row
+                    xq[(int64_t) n * (K / 4) + c] = (q0 & 0xFF) | ((q1 & 0xFF) << 8) | ((q2 & 0xFF) << 16) | ((q3 & 0xFF) << 24);
+                    if ((c & 7) == 0) {
+                        xd[n * nbk + c / 8]   = h2f(f2h_bits(d));     // the CPU backend stores d as f16 and reads it back
+                        xsum[n * nbk + c / 8] = sum;
+                    }
+                }
+            }
+        }
+    }
+}
+
 // LDS: int32 xq[NC][K/4] | float xd[NC][K/32] | int32 xsum[NC][K/32]
 template <int T0, int NC, int LPR>
 __global__ void __launch_bounds__(256) k_gemv_q(mm_args a) {
@@ -578,44 +622,7 @@ __global__ void __launch_bounds__(256) k_gemv_q(mm_args a) {
     wraw<T0> blk;
     if (row_ok && j < nbk) blk = load_wraw<T0>(wrow, j);
 
-    // --- quantize X: 8 lanes per 32-value block, round-to-nearest-even like _mm256_round_ps(_MM_ROUND_NEAREST).
-    // Eight independent loads per thread are in flight before the first is consumed.
-    {
-        const int total = NC * nbk * 8;                         // float4 pieces
-        const int k8 = nbk * 8;
-        for (int base = 0; base < total; base += 256 * 8) {
-            float4 v[8];
-#pragma unroll
-            for (int u = 0; u < 8; ++u) {
-                const int idx = base + u * 256 + (int) threadIdx.x;
-                v[u] = make_float4(0.f, 0.f, 0.f, 0.f);
-                if (idx < total) v[u] = *(const float4 *)(a.x + (int64_t)(idx / k8) * a.x_nb1 + (int64_t)(idx % k8) * 16);
-            }
-#pragma unroll
-            for (int u = 0; u < 8; ++u) {
-                const int idx = base + u * 256 + (int) threadIdx.x;      // lanes 8i .. 8i+7 share a block
-                float amax = fmaxf(fmaxf(fabsf(v[u].x), fabsf(v[u].y)), fmaxf(fabsf(v[u].z), fabsf(v[u].w)));
-                amax = fmaxf(amax, __shfl_xor(amax, 1, 8));
-                amax = fmaxf(amax, __shfl_xor(amax, 2, 8));
-                amax = fmaxf(amax, __shfl_xor(amax, 4, 8));
-                const float d  = amax / 127.0f;
-                const float id = amax != 0.0f ? 127.0f / amax : 0.0f;
-                const int q0 = (int) rintf(v[u].x * id), q1 = (int) rintf(v[u].y * id), q2 = (int) rintf(v[u].z * id), q3 = (int) rintf(v[u].w * id);
-                int sum = q0 + q1 + q2 + q3;
-                sum += __shfl_xor(sum, 1, 8);
-                sum += __shfl_xor(sum, 2, 8);
-                sum += __shfl_xor(sum, 4, 8);
-                if (idx < total) {
-                    const int n = idx / k8, c = idx % k8;       // c: float4 piece within the row
-                    xq[(int64_t) n * (K / 4) + c] = (q0 & 0xFF) | ((q1 & 0xFF) << 8) | ((q2 & 0xFF) << 16) | ((q3 & 0xFF) << 24);
-                    if ((c & 7) == 0) {
-                        xd[n * nbk + c / 8]   = h2f(f2h_bits(d));     // the CPU backend stores d as f16 and reads it back
-                        xsum[n * nbk + c / 8] = sum;
-                    }
-                }
-            }
-        }
-    }
+    quantize_x_to_lds<NC>(a, xq, xd, xsum, nbk);
     __syncthreads();
 
     for (;;) {
@@ -677,6 +684,188 @@ __global__ void __launch_bounds__(256) k_gemv_q(mm_args a) {
 #pragma unroll
             for (int o = LPR / 2; o > 0; o >>= 1) acc[n] += __shfl_xor(acc[n], o, LPR);
         }
+        if (done_writer) {
+            const bool out_f16 = a.e.flags & MI355X_EPI_OUT_F16;
+#pragma unroll
+            for (int n = 0; n < NC; ++n) {
+                float v = acc[n] + o_bias + o_bcol[n];          // at most one of the two biases is set
+                if (a.e.flags & MI355X_EPI_GELU)     v  = gelu_f32(v, a.e.gelu);
+                if (a.e.flags & MI355X_EPI_SCALE)    v *= a.e.scale;
+                if (a.e.flags & MI355X_EPI_RESIDUAL) v += o_res[n];
+                if (out_f16) *(half_t *)(a.d + n * a.d_nb1 + done_row * 2) = (half_t) v;
+                else         *(float  *)(a.d + n * a.d_nb1 + done_row * 4) = v;
+            }
+        }
+        if (!more) break;
+    }
+}
+
+// sum over the LPR lanes of a row, in every lane: DPP steps inside the rows of 16 (a mirror pairs the lanes as well as an
+// exchange does, for a sum), a swizzle across two rows, a permute across the halves of the wavefront
+template <int LPR>
+__device__ __forceinline__ float lanes_sum(float x) {
+    auto dpp = [](float v, auto ctrl) __attribute__((always_inline)) {
+        return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), decltype(ctrl)::value, 0xf, 0xf, true));
+    };
+    x += dpp(x, std::integral_constant<int, 0xB1>());                   // quad_perm [1,0,3,2]
+    x += dpp(x, std::integral_constant<int, 0x4E>());                   // quad_perm [2,3,0,1]
+    x += dpp(x, std::integral_constant<int, 0x141>());                  // row_half_mirror
+    if (LPR >= 16) x += dpp(x, std::integral_constant<int, 0x140>());   // row_mirror
+    if (LPR >= 32) x += __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, x), 0x401F));   // lane ^ 16
+    if (LPR >= 64) x += __shfl_xor(x, 32, WAVE);
+    return x;
+}
+
+// Activations quantized ahead of the product, once for every product that reads them:
+//   int8 xq[N][K] | float xd[N][K/32] (the f16-rounded block scales) | int32 xsum[N][K/32] (sum of a block's quants)
+// One thread per four values, eight lanes per block; rounding as quantize_row_q8_0 (ggml-cpu-quants.c:808-865).
+__global__ void __launch_bounds__(256) k_quantize_x_q8(const char * __restrict__ x, int64_t x_nb1, int64_t K, int64_t N, char * __restrict__ ws) {
+    const int64_t k4 = K / 4, nbk = K / QK;
+    const int64_t idx = (int64_t) blockIdx.x * 256 + threadIdx.x;          // K % 32 == 0: the 8 lanes of a block are in or out together
+    if (idx >= N * k4) return;
+    const int64_t n = idx / k4, c = idx % k4;
+    const float4 v = *(const float4 *)(x + n * x_nb1 + c * 16);
+    float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
+    amax = fmaxf(amax, __shfl_xor(amax, 1, 8));
+    amax = fmaxf(amax, __shfl_xor(amax, 2, 8));
+    amax = fmaxf(amax, __shfl_xor(amax, 4, 8));
+    const float d  = amax / 127.0f;
+    const float id = amax != 0.0f ? 127.0f / amax : 0.0f;
+    const int q0 = (int) rintf(v.x * id), q1 = (int) rintf(v.y * id), q2 = (int) rintf(v.z * id), q3 = (int) rintf(v.w * id);
+    int sum = q0 + q1 + q2 + q3;
+    sum += __shfl_xor(sum, 1, 8);
+    sum += __shfl_xor(sum, 2, 8);
+    sum += __shfl_xor(sum, 4, 8);
+    int32_t * xq   = (int32_t *) ws;
+    float *   xd   = (float *)(ws + N * K);
+    int32_t * xsum = (int32_t *)(ws + N * K + N * nbk * 4);
+    xq[n * k4 + c] = (q0 & 0xFF) | ((q1 & 0xFF) << 8) | ((q2 & 0xFF) << 16) | ((q3 & 0xFF) << 24);
+    if ((c & 7) == 0) {
+        xd[n * nbk + c / 8]   = h2f(f2h_bits(d));          // the CPU backend stores d as f16 and reads it back
+        xsum[n * nbk + c / 8] = sum;
+    }
+}
+
+// The product over activations quantized ahead (a.x: the layout above, NC rows).  Lane j of a row's LPR lanes owns blocks
+// j, j + LPR, ... (NB of them) of EVERY row it visits, so its slices of the activations are read once and stay in
+// registers while the workgroup walks its row groups: the loop is weight loads and integer dot products only.  With
+// the activations in LDS, their reads (NC x 32 bytes per 34-byte block) are what bounds the kernel, and quantizing them
+// in every workgroup costs more than the product itself once K is large.
+template <int T0, int NC, int LPR, int NB>
+__global__ void __launch_bounds__(256) k_gemv_qr(mm_args a) {
+    const int64_t K = a.K;
+    const int nbk = (int)(K / QK);
+    const int32_t * xq   = (const int32_t *) a.x;
+    const float *   xd   = (const float *)(a.x + (size_t) NC * K);
+    const int32_t * xsum = (const int32_t *)(a.x + (size_t) NC * K + (size_t) NC * nbk * 4);
+
+    constexpr int RPW = WAVE / LPR;                 // rows per wavefront
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int j = lane % LPR, r = lane / LPR;
+    const int64_t n_groups = (a.M + 4 * RPW - 1) / (4 * RPW);
+    int64_t group = blockIdx.x;
+    int64_t row = group * (4 * RPW) + wave * RPW + r;
+    bool row_ok = row < a.M;
+    const uint8_t * wrow = (const uint8_t *) a.w + (row_ok ? row : 0) * a.w_nb1;
+
+    // the first row's blocks are requested first; a lane whose block index lies beyond the row keeps an all-zero block
+    wraw<T0> blk[NB];
+#pragma unroll
+    for (int b = 0; b < NB; ++b) {
+        blk[b].d = 0; blk[b].qh = 0;
+#pragma unroll
+        for (int i = 0; i < (T0 == MI355X_TYPE_Q8_0 ? 8 : 4); ++i) blk[b].q[i] = 0;
+    }
+    auto load_blocks = [&]() __attribute__((always_inline)) {
+#pragma unroll
+        for (int b = 0; b < NB; ++b) if (j + b * LPR < nbk) blk[b] = load_wraw<T0>(wrow, j + b * LPR);
+    };
+    load_blocks();
+
+    int32_t xr[NC][NB][8];
+    float   xs[NC][NB];          // scale of the block
+    int32_t xo[NC][NB];          // 16 x sum of its quants (Q5_0 weights are stored with an offset of 16)
+#pragma unroll
+    for (int n = 0; n < NC; ++n) {
+#pragma unroll
+        for (int b = 0; b < NB; ++b) {
+            const int kb = j + b * LPR < nbk ? j + b * LPR : 0;
+            const int4 x0 = *(const int4 *)(xq + (int64_t) n * (K / 4) + kb * 8), x1 = *(const int4 *)(xq + (int64_t) n * (K / 4) + kb * 8 + 4);
+            xr[n][b][0] = x0.x; xr[n][b][1] = x0.y; xr[n][b][2] = x0.z; xr[n][b][3] = x0.w;
+            xr[n][b][4] = x1.x; xr[n][b][5] = x1.y; xr[n][b][6] = x1.z; xr[n][b][7] = x1.w;
+            xs[n][b] = xd[n * nbk + kb];
+            xo[n][b] = T0 == MI355X_TYPE_Q5_0 ? 16 * xsum[n * nbk + kb] : 0;
+        }
+    }
+
+    // the epilogue operands of the lane that will store are fetched early, under the weight stream
+    float e_bias = 0.0f, e_bcol[NC], e_res[NC];
+#pragma unroll
+    for (int n = 0; n < NC; ++n) { e_bcol[n] = 0.0f; e_res[n] = 0.0f; }
+    auto fetch_epilogue = [&]() __attribute__((always_inline)) {
+        if (row_ok && j == 0) {
+            if (a.e.flags & MI355X_EPI_BIAS) e_bias = a.e.bias[row];
+            if (a.e.flags & MI355X_EPI_BIAS_COL) {
+#pragma unroll
+                for (int n = 0; n < NC; ++n) e_bcol[n] = a.e.bias[n];
+            }
+            if (a.e.flags & MI355X_EPI_RESIDUAL) {
+#pragma unroll
+                for (int n = 0; n < NC; ++n) e_res[n] = *(const float *)(a.e.residual + n * a.d_nb1 + row * 4);
+            }
+        }
+    };
+    fetch_epilogue();
+
+    for (;;) {
+        wraw<T0> cur[NB];
+#pragma unroll
+        for (int b = 0; b < NB; ++b) cur[b] = blk[b];
+        const int64_t done_row = row;
+        const bool done_writer = row_ok && j == 0;
+        const float o_bias = e_bias;
+        float o_bcol[NC], o_res[NC];
+#pragma unroll
+        for (int n = 0; n < NC; ++n) { o_bcol[n] = e_bcol[n]; o_res[n] = e_res[n]; }
+        // the next row's blocks and epilogue operands travel while this row is worked on
+        group += gridDim.x;
+        const bool more = group < n_groups;                 // uniform
+        if (more) {
+            row = group * (4 * RPW) + wave * RPW + r;
+            row_ok = row < a.M;
+            wrow = (const uint8_t *) a.w + (row_ok ? row : 0) * a.w_nb1;
+            load_blocks();
+            fetch_epilogue();
+        }
+
+        float acc[NC];
+#pragma unroll
+        for (int n = 0; n < NC; ++n) acc[n] = 0.0f;
+#pragma unroll
+        for (int b = 0; b < NB; ++b) {
+            uint32_t q[8];
+            const float dw = h2f((uint16_t) cur[b].d);
+            if constexpr (T0 == MI355X_TYPE_Q8_0) {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) q[i] = cur[b].q[i];
+            } else {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    q[i]     = (cur[b].q[i] & 0x0F0F0F0Fu)        | spread4_to_bit4((cur[b].qh >> (4*i))      & 0xFu);
+                    q[4 + i] = ((cur[b].q[i] >> 4) & 0x0F0F0F0Fu) | spread4_to_bit4((cur[b].qh >> (16 + 4*i)) & 0xFu);
+                }
+            }
+#pragma unroll
+            for (int n = 0; n < NC; ++n) {
+                int s = 0;
+#pragma unroll
+                for (int i = 0; i < 8; ++i) s = __builtin_amdgcn_sdot4((int) q[i], xr[n][b][i], s, false);
+                if constexpr (T0 == MI355X_TYPE_Q5_0) s -= xo[n][b];
+                acc[n] += (float) s * (dw * xs[n][b]);
+            }
+        }
+#pragma unroll
+        for (int n = 0; n < NC; ++n) acc[n] = lanes_sum<LPR>(acc[n]);
         if (done_writer) {
             const bool out_f16 = a.e.flags & MI355X_EPI_OUT_F16;
 #pragma unroll
@@ -760,6 +949,68 @@ static bool aligned16(const mi355x_tensor * t) {
     return (uintptr_t) t->data % 16 == 0 && t->nb[1] % 16 == 0 && t->nb[2] % 16 == 0 && t->nb[3] % 16 == 0;
 }
 
+// Register-resident variant: LPR = 16, 32 or 64 lanes per row with NB <= 3 blocks per lane and N * NB <= 15 block slices of
+// activations (120 registers).  The fewest lanes per row that still give 512 workgroups (few lanes per row = few idle
+// lanes when the blocks of a row do not divide evenly), else the most.  Returns LPR, 0 when the shape does not fit.
+static int gemv_r_lanes(int64_t M, int64_t N, int64_t K) {
+    const int64_t nbk = K / QK;
+    int best = 0;
+    for (int lpr = 64; lpr >= 16; lpr /= 2) {
+        const int64_t nb = (nbk + lpr - 1) / lpr;
+        if (nb > 3 || nb * N > 15) break;
+        if (best == 0 || M * lpr / 256 >= 512) best = lpr;
+    }
+    return best;
+}
+// bytes of the quantized activations the register variant reads (0: the shape runs with in-kernel quantization)
+static size_t gemv_ws_bytes(const mi355x_tensor * src0, const mi355x_tensor * src1) {
+    const int64_t K = src0->ne[0], N = src1->ne[1];
+    if (!gemv_r_lanes(src0->ne[1], N, K)) return 0;
+    return round256((size_t)(N * K + N * (K / QK) * 8));
+}
+
+template <int T0, int NC, int LPR>
+static int launch_gemv_r_nb(const mm_args & a, int nb, unsigned grid, hipStream_t st) {
+    switch (nb) {
+        case 1: k_gemv_qr<T0, NC, LPR, 1><<<grid, 256, 0, st>>>(a); return launch_status();
+        case 2: if constexpr (NC * 2 <= 15) { k_gemv_qr<T0, NC, LPR, 2><<<grid, 256, 0, st>>>(a); return launch_status(); } break;
+        case 3: if constexpr (NC * 3 <= 15) { k_gemv_qr<T0, NC, LPR, 3><<<grid, 256, 0, st>>>(a); return launch_status(); } break;
+    }
+    return MI355X_ERR_UNSUPPORTED;
+}
+template <int T0, int NC>
+static int launch_gemv_r(const mm_args & a, hipStream_t st) {
+    const int lpr = gemv_r_lanes(a.M, NC, a.K);
+    if (!lpr) return MI355X_ERR_UNSUPPORTED;
+    const int nb = (int)((a.K / QK + lpr - 1) / lpr);
+    const int rows_per_wg = 4 * (WAVE / lpr);
+    const int64_t n_groups = (a.M + rows_per_wg - 1) / rows_per_wg;
+    // one resident set of workgroups (the registers allow 4 per CU with one block per lane, else 2), each walking its
+    // share of the row groups: a second, partly filled set would double the time
+    const int64_t resident = 256 * (nb == 1 ? 4 : 2);
+    const int64_t rounds   = (n_groups + resident - 1) / resident;
+    const unsigned grid    = (unsigned)((n_groups + rounds - 1) / rounds);
+    switch (lpr) {
+        case 16: return launch_gemv_r_nb<T0, NC, 16>(a, nb, grid, st);
+        case 32: return launch_gemv_r_nb<T0, NC, 32>(a, nb, grid, st);
+        default: return launch_gemv_r_nb<T0, NC, 64>(a, nb, grid, st);
+    }
+}
+template <int T0>
+static int launch_gemv_r_n(const mm_args & a, hipStream_t st) {
+    switch (a.N) {
+        case 1: return launch_gemv_r<T0, 1>(a, st);
+        case 2: return launch_gemv_r<T0, 2>(a, st);
+        case 3: return launch_gemv_r<T0, 3>(a, st);
+        case 4: return launch_gemv_r<T0, 4>(a, st);
+        case 5: return launch_gemv_r<T0, 5>(a, st);
+        case 6: return launch_gemv_r<T0, 6>(a, st);
+        case 7: return launch_gemv_r<T0, 7>(a, st);
+        case 8: return launch_gemv_r<T0, 8>(a, st);
+    }
+    return MI355X_ERR_INVALID;
+}
+
 template <int T0, int NC>
 static int launch_gemv(const mm_args & a, hipStream_t st) {
     const size_t lds = (size_t) NC * a.K + (size_t) NC * (a.K / QK) * 8;
@@ -840,7 +1091,10 @@ static size_t w16_bytes(const mi355x_tensor * src0) {
     return src0->type != MI355X_TYPE_F16 ? round256((size_t) src0->ne[0] * src0->ne[1] * 2) * (size_t)(src0->ne[2] * src0->ne[3]) : 0;
 }
 extern "C" size_t mi355x_mul_mat_workspace_size(const mi355x_tensor * src0, const mi355x_tensor * src1) {
-    if (!src0 || !src1 || mm_path(src0, src1) != MM_GEMM) return 0;
+    if (!src0 || !src1) return 0;
+    const int path = mm_path(src0, src1);
+    if (path == MM_GEMV) return gemv_ws_bytes(src0, src1);
+    if (path != MM_GEMM) return 0;
     return x16_bytes(src1) + w16_bytes(src0);
 }
 
@@ -934,7 +1188,7 @@ extern "C" int mi355x_mul_mat(const mi355x_tensor * src0, const mi355x_tensor * 
     if ((flags & MI355X_EPI_RESIDUAL) && !epi->residual) return MI355X_ERR_INVALID;
     if ((flags & MI355X_EPI_RESIDUAL) && (flags & MI355X_EPI_OUT_F16)) return MI355X_ERR_UNSUPPORTED;
     if (a.M == 0 || a.N == 0 || dst->ne[2] * dst->ne[3] == 0) return MI355X_OK;
-    if ((flags & MI355X_MM_PREPARE_ONLY) && mm_path(src0, src1) != MM_GEMM) return MI355X_OK;      // nothing to prepare
+    if ((flags & MI355X_MM_PREPARE_ONLY) && mm_path(src0, src1) == MM_GENERIC) return MI355X_OK;   // nothing to prepare
 
     a.w = (const char *) src0->data; a.x = (const char *) src1->data; a.d = (char *) dst->data;
     a.w_nb1 = src0->nb[1]; a.w_nb2 = src0->nb[2]; a.w_nb3 = src0->nb[3];
@@ -960,6 +1214,20 @@ extern "C" int mi355x_mul_mat(const mi355x_tensor * src0, const mi355x_tensor * 
     const int path = mm_path(src0, src1);
     const bool quant = blck_size(t0) > 1;
     if (path == MM_GEMV) {
+        // with a workspace: activations quantized once (skipped when the caller says they are there), then the product
+        // with them in registers; without: every workgroup quantizes them into LDS for itself
+        const size_t need = gemv_ws_bytes(src0, src1);
+        if (need && workspace && workspace_size >= need && (uintptr_t) workspace % 16 == 0) {
+            if (!(flags & MI355X_MM_WS_READY)) {
+                k_quantize_x_q8<<<(unsigned)((a.N * (a.K / 4) + 255) / 256), 256, 0, st>>>(a.x, a.x_nb1, a.K, a.N, (char *) workspace);
+                if (const int rc = launch_status()) return rc;
+            }
+            if (flags & MI355X_MM_PREPARE_ONLY) return MI355X_OK;
+            mm_args g = a;
+            g.x = (const char *) workspace;
+            return t0 == MI355X_TYPE_Q8_0 ? launch_gemv_r_n<MI355X_TYPE_Q8_0>(g, st) : launch_gemv_r_n<MI355X_TYPE_Q5_0>(g, st);
+        }
+        if (flags & MI355X_MM_PREPARE_ONLY) return MI355X_OK;
         return t0 == MI355X_TYPE_Q8_0 ? launch_gemv_n<MI355X_TYPE_Q8_0>(a, st) : launch_gemv_n<MI355X_TYPE_Q5_0>(a, st);
     }
     if (path == MM_GEMM) {

@@ -13,7 +13,9 @@
 // EMIT: also write the row as the MFMA GEMM wants its activations — rounded to Q8_0 like quantize_row_q8_0
 // (ggml-cpu-quants.c:808-865: block amax, id = 127/amax, round half to even, d through f16) and stored as f16(q * d),
 // dense [nrows][ne0] — so that the products that follow need no conversion pass of their own.
-template <bool IN_REGS, bool EMIT>
+// EMIT == 2: the row quantized to Q8_0 itself, in the layout the few-column product reads its activations from
+// (int8 q[nrows][ne0] | float d[nrows][ne0/32] | int32 sum of a block's quants).
+template <bool IN_REGS, int EMIT>
 __global__ void k_norm(tview s, tview d, int64_t nrows, float eps, const float * __restrict__ w, const float * __restrict__ b, half_t * __restrict__ x16) {
     const int     lane = threadIdx.x % WAVE;
     const int64_t row  = (int64_t) blockIdx.x * ROWS_PER_BLOCK + threadIdx.x / WAVE;
@@ -65,8 +67,23 @@ __global__ void k_norm(tview s, tview d, int64_t nrows, float eps, const float *
                     amax = fmaxf(amax, __shfl_xor(amax, 4, 8));
                     const float id = amax != 0.0f ? 127.0f / amax : 0.0f;
                     const float dq = h2f(f2h_bits(amax / 127.0f));
-                    const half4_t h = { (half_t)((rintf(r.x * id) + 0.0f) * dq), (half_t)((rintf(r.y * id) + 0.0f) * dq), (half_t)((rintf(r.z * id) + 0.0f) * dq), (half_t)((rintf(r.w * id) + 0.0f) * dq) };
-                    *(half4_t *)(x16 + row * ne0 + 4 * (int64_t) c) = h;
+                    if (EMIT == 1) {
+                        const half4_t h = { (half_t)((rintf(r.x * id) + 0.0f) * dq), (half_t)((rintf(r.y * id) + 0.0f) * dq), (half_t)((rintf(r.z * id) + 0.0f) * dq), (half_t)((rintf(r.w * id) + 0.0f) * dq) };
+                        *(half4_t *)(x16 + row * ne0 + 4 * (int64_t) c) = h;
+                    } else {
+                        const int q0 = (int) rintf(r.x * id), q1 = (int) rintf(r.y * id), q2 = (int) rintf(r.z * id), q3 = (int) rintf(r.w * id);
+                        int qsum = q0 + q1 + q2 + q3;
+                        qsum += __shfl_xor(qsum, 1, 8);
+                        qsum += __shfl_xor(qsum, 2, 8);
+                        qsum += __shfl_xor(qsum, 4, 8);
+                        char * q8 = (char *) x16;
+                        const int64_t nbk = ne0 / 32;
+                        ((int32_t *) q8)[row * (ne0 / 4) + c] = (q0 & 0xFF) | ((q1 & 0xFF) << 8) | ((q2 & 0xFF) << 16) | ((q3 & 0xFF) << 24);
+                        if ((c & 7) == 0) {
+                            ((float *)(q8 + nrows * ne0))[row * nbk + c / 8] = dq;
+                            ((int32_t *)(q8 + nrows * ne0 + nrows * nbk * 4))[row * nbk + c / 8] = qsum;
+                        }
+                    }
                 }
             }
         }
@@ -86,18 +103,23 @@ __global__ void k_norm(tview s, tview d, int64_t nrows, float eps, const float *
     }
 }
 
-static int norm_impl(const mi355x_tensor * src, const mi355x_tensor * dst, float eps, const float * w, const float * b, void * x16, void * stream);
+static int norm_impl(const mi355x_tensor * src, const mi355x_tensor * dst, float eps, const float * w, const float * b, void * x16, int emit, void * stream);
 
 extern "C" int mi355x_norm(const mi355x_tensor * src, const mi355x_tensor * dst, float eps, const float * w, const float * b, void * stream) {
-    return norm_impl(src, dst, eps, w, b, nullptr, stream);
+    return norm_impl(src, dst, eps, w, b, nullptr, 0, stream);
 }
 
 extern "C" int mi355x_norm_emit_f16(const mi355x_tensor * src, const mi355x_tensor * dst, float eps, const float * w, const float * b, void * x16, void * stream) {
     if (!x16 || (uintptr_t) x16 % 8 != 0) return MI355X_ERR_INVALID;
-    return norm_impl(src, dst, eps, w, b, x16, stream);
+    return norm_impl(src, dst, eps, w, b, x16, 1, stream);
+}
+extern "C" int mi355x_norm_emit_q8_0(const mi355x_tensor * src, const mi355x_tensor * dst, float eps, const float * w, const float * b, void * q8, void * stream) {
+    if (!q8 || (uintptr_t) q8 % 16 != 0) return MI355X_ERR_INVALID;
+    if (src && (src->ne[2] != 1 || src->ne[3] != 1)) return MI355X_ERR_UNSUPPORTED;
+    return norm_impl(src, dst, eps, w, b, q8, 2, stream);
 }
 
-static int norm_impl(const mi355x_tensor * src, const mi355x_tensor * dst, float eps, const float * w, const float * b, void * x16, void * stream) {
+static int norm_impl(const mi355x_tensor * src, const mi355x_tensor * dst, float eps, const float * w, const float * b, void * x16, int emit, void * stream) {
     if (!src || !dst || !(eps >= 0.0f)) return MI355X_ERR_INVALID;
     if (src->type != MI355X_TYPE_F32 || dst->type != MI355X_TYPE_F32) return MI355X_ERR_UNSUPPORTED;
     if (!same_shape(src, dst) || src->nb[0] != 4 || dst->nb[0] != 4) return MI355X_ERR_INVALID;
@@ -114,11 +136,12 @@ static int norm_impl(const mi355x_tensor * src, const mi355x_tensor * dst, float
                          (uintptr_t) w % 16 == 0 && (uintptr_t) b % 16 == 0;
     if (x16) {                                             // only the register-resident form emits, and only whole blocks
         if (!in_regs || src->ne[0] % QK != 0) return MI355X_ERR_UNSUPPORTED;
-        k_norm<true, true><<<(unsigned) grid, ROWS_PER_BLOCK * WAVE, 0, st>>>(make_view(src), make_view(dst), nrows, eps, w, b, (half_t *) x16);
+        if (emit == 2) k_norm<true, 2><<<(unsigned) grid, ROWS_PER_BLOCK * WAVE, 0, st>>>(make_view(src), make_view(dst), nrows, eps, w, b, (half_t *) x16);
+        else           k_norm<true, 1><<<(unsigned) grid, ROWS_PER_BLOCK * WAVE, 0, st>>>(make_view(src), make_view(dst), nrows, eps, w, b, (half_t *) x16);
         return launch_status();
     }
-    if (in_regs) k_norm<true,  false><<<(unsigned) grid, ROWS_PER_BLOCK * WAVE, 0, st>>>(make_view(src), make_view(dst), nrows, eps, w, b, nullptr);
-    else         k_norm<false, false><<<(unsigned) grid, ROWS_PER_BLOCK * WAVE, 0, st>>>(make_view(src), make_view(dst), nrows, eps, w, b, nullptr);
+    if (in_regs) k_norm<true,  0><<<(unsigned) grid, ROWS_PER_BLOCK * WAVE, 0, st>>>(make_view(src), make_view(dst), nrows, eps, w, b, nullptr);
+    else         k_norm<false, 0><<<(unsigned) grid, ROWS_PER_BLOCK * WAVE, 0, st>>>(make_view(src), make_view(dst), nrows, eps, w, b, nullptr);
     return launch_status();
 }
 
