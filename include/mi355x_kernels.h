@@ -157,7 +157,11 @@ enum mi355x_fa_mode { MI355X_FA_F16_SEQ = 0, MI355X_FA_F32 = 1, MI355X_FA_F16_PA
     /* or-ed into the mode: also write into `workspace` (16-byte aligned, N * H * ne3 * 64 halves) the image of dst that
      * a following MUL_MAT with quantized weights wants — rows [N][H * 64] rounded to Q8_0 as quantize_row_q8_0 does and
      * stored as f16(q * d) (then pass MI355X_MM_WS_READY there).  More than 8 queries; MI355X_ERR_UNSUPPORTED otherwise. */
-    MI355X_FA_EMIT_F16 = 0x100 };
+    MI355X_FA_EMIT_F16 = 0x100,
+    /* or-ed into the mode, at most 8 queries (the f16-sequential kernel of a decode step): also write into `workspace`
+     * (16-byte aligned) the rows [N * ne3][H * 64] of dst quantized to Q8_0, in the layout the few-column mi355x_mul_mat
+     * reads its activations from (see mi355x_norm_emit_q8_0); MI355X_ERR_UNSUPPORTED for other kernels. */
+    MI355X_FA_EMIT_Q8_0 = 0x200 };
 MI355X_API const char * mi355x_flash_attn_ext_kernel_name(const mi355x_tensor * q, const mi355x_tensor * k, int mode);
 MI355X_API size_t mi355x_flash_attn_ext_workspace_size(const mi355x_tensor * q, const mi355x_tensor * k);
 MI355X_API int    mi355x_flash_attn_ext(const mi355x_tensor * q, const mi355x_tensor * k, const mi355x_tensor * v,

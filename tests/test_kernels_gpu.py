@@ -366,6 +366,30 @@ def test_flash_attn_emits_the_next_products_activation_image(pkg, oracle, gpu):
     assert lib.mi355x_flash_attn_ext(tq, tk, tv, None, to, 0.125, pkg.FA_EMIT_F16, d_h.data_ptr(), 64, gpu.stream) == -3
 
 
+def test_flash_attn_few_queries_emit_q8_0(pkg, oracle, gpu):
+    # MI355X_FA_EMIT_Q8_0: a decode step's attention leaves its rows [N][H * 64] quantized for the projection that follows
+    H, N, KV = 6, 5, 200
+    q, kb, vb = _attention_inputs(oracle, H, N, KV)
+    d_q, d_k, d_v = gpu.up(q), gpu.up(kb), gpu.up(vb)
+    d_o = torch.empty((N, H, 64), dtype=torch.float32, device=gpu.dev)
+    k = H * 64
+    d_w = torch.zeros(N * k + N * (k // 32) * 8, dtype=torch.uint8, device=gpu.dev)
+    tq, tk, tv, to = pkg.tensor(d_q, pkg.F32), pkg.tensor(d_k, pkg.F16), pkg.tensor(d_v, pkg.F16), pkg.tensor(d_o, pkg.F32)
+    lib = pkg.kernels()
+    pkg.check(lib.mi355x_flash_attn_ext(tq, tk, tv, None, to, 0.125, pkg.FA_F16_SEQ | pkg.FA_EMIT_Q8_0, d_w.data_ptr(), d_w.numel(), gpu.stream))
+    y, image = gpu.down(d_o).reshape(N, k), gpu.down(d_w)
+    assert oracle.nmse(y, oracle.flash_attn_ext(q, kb, vb, None, 0.125).reshape(N, k)) <= 1e-6
+    want = oracle.quantize(oracle.Q8_0, y, act=True).reshape(N, k // 32, 34)
+    assert np.array_equal(image[: N * k].reshape(N, k // 32, 32), want[:, :, 2:])
+    assert np.array_equal(image[N * k : N * k + N * (k // 32) * 4].view(np.float32).reshape(N, k // 32),
+                          oracle.f16_bits_to_f32(want[:, :, :2].copy().view(np.uint16)[..., 0]))
+    assert np.array_equal(image[N * k + N * (k // 32) * 4 :].view(np.int32).reshape(N, k // 32), want[:, :, 2:].view(np.int8).astype(np.int32).sum(-1))
+    # the many-query kernels do not write this form
+    d_q9 = gpu.up(rnd((H, 9, 64)))
+    d_o9 = torch.empty((9, H, 64), dtype=torch.float32, device=gpu.dev)
+    assert lib.mi355x_flash_attn_ext(pkg.tensor(d_q9, pkg.F32), tk, tv, None, pkg.tensor(d_o9, pkg.F32), 0.125, pkg.FA_EMIT_Q8_0, d_w.data_ptr(), d_w.numel(), gpu.stream) == -1
+
+
 def _attention_float64(oracle, q, kb, vb, mask, scale):
     qf = oracle.f16_bits_to_f32(oracle.f32_to_f16_bits(q)).astype(np.float64)
     s = np.einsum("hnd,hkd->hnk", qf, oracle.f16_bits_to_f32(kb).astype(np.float64)) * scale

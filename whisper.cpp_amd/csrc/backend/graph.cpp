@@ -571,14 +571,18 @@ struct graph_runner {
                 // the output projection that follows takes its Q8_0-rounded activations from the attention kernel itself
                 const bool emits = !ctx->exact && (strncmp(name, "flash_attn.seq_tile", 19) == 0 || strcmp(name, "flash_attn.mfma_f32") == 0);
                 const ggml_tensor * key = emits ? image_consumer(n, i + 1) : nullptr;
-                const size_t image_bytes = (size_t) ggml_nelements(n) * 2;
+                // (a decode step's projection reads Q8_0 itself, written by the few-query kernel)
+                int form = 1;
+                if (!key && !ctx->exact && strcmp(name, "flash_attn.seq_row") == 0 && (key = image_consumer(n, i + 1, true))) form = 2;
+                const size_t image_bytes = form == 1 ? (size_t) ggml_nelements(n) * 2 : (size_t) ggml_nelements(n) / 32 * 40;
                 if (key && !ctx->reserve_workspace(image_bytes + 256)) key = nullptr;
                 {
                     launch_scope ls(ctx, name, bytes + (key ? image_bytes : 0), flops);
-                    status = mi355x_flash_attn_ext(&vq, &vk, &vv, m ? &vm : nullptr, &vd, scale, mode | (key ? MI355X_FA_EMIT_F16 : 0),
+                    status = mi355x_flash_attn_ext(&vq, &vk, &vv, m ? &vm : nullptr, &vd, scale,
+                                                   mode | (!key ? 0 : form == 1 ? MI355X_FA_EMIT_F16 : MI355X_FA_EMIT_Q8_0),
                                                    key ? ctx->ws : nullptr, key ? ctx->ws_size : 0, ctx->stream);
                 }
-                if (key && status == MI355X_OK) workspace_holds(key, ctx->ws_slot);
+                if (key && status == MI355X_OK) workspace_holds(key, ctx->ws_slot, form);
                 return 1;
             }
             case GGML_OP_CONCAT: {

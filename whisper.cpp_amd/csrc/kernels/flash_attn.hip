@@ -314,7 +314,28 @@ __global__ void __launch_bounds__(256) k_fattn_seq_row(fa_args a, int kv_pad) {
     if (wave != 0) return;
     half_t acc_h; { const uint16_t t16 = (uint16_t) acc; __builtin_memcpy(&acc_h, &t16, 2); }
     float * dp = (float *) a.d + ((i3 * a.N + n) * a.H + h) * FA_D;
-    dp[lane] = (float) acc_h * (1.0f / s_total);
+    const float o = (float) acc_h * (1.0f / s_total);
+    dp[lane] = o;
+    if (a.x16) {
+        // MI355X_FA_EMIT_Q8_0: the projection that follows reads its activations as Q8_0 (rows [N][H * 64]: int8 quants |
+        // f32 scales | int32 block sums); this wavefront holds two blocks of one row, one per 32 lanes
+        float amax = fabsf(o);
+#pragma unroll
+        for (int s = 1; s < 32; s <<= 1) amax = fmaxf(amax, __shfl_xor(amax, s, 32));
+        const float id = amax != 0.0f ? 127.0f / amax : 0.0f;
+        const int q = (int) rintf(o * id);
+        int qsum = q;
+#pragma unroll
+        for (int s = 1; s < 32; s <<= 1) qsum += __shfl_xor(qsum, s, 32);
+        char * q8 = (char *) a.x16;
+        const int64_t K = a.H * FA_D, nbk = K / 32, rows = a.N * a.ne3, rowi = i3 * a.N + n;
+        ((int8_t *) q8)[rowi * K + h * FA_D + lane] = (int8_t) q;
+        if ((lane & 31) == 0) {
+            const int64_t blk = rowi * nbk + h * 2 + (lane >> 5);
+            ((float *)(q8 + rows * K))[blk] = h2f(f2h_bits(amax / 127.0f));
+            ((int32_t *)(q8 + rows * K + rows * nbk * 4))[blk] = qsum;
+        }
+    }
 }
 
 // ------------------------------------------------------------------------------------------------------
@@ -867,8 +888,9 @@ extern "C" int mi355x_flash_attn_ext(const mi355x_tensor * q, const mi355x_tenso
                                      const mi355x_tensor * mask, const mi355x_tensor * dst, float scale, int mode,
                                      void * workspace, size_t workspace_size, void * stream) {
     if (!q || !k || !v || !dst) return MI355X_ERR_INVALID;
-    const bool emit = mode & MI355X_FA_EMIT_F16;
-    mode &= ~MI355X_FA_EMIT_F16;
+    const bool emit = mode & MI355X_FA_EMIT_F16, emit_q8 = mode & MI355X_FA_EMIT_Q8_0;
+    mode &= ~(MI355X_FA_EMIT_F16 | MI355X_FA_EMIT_Q8_0);
+    if (emit && emit_q8) return MI355X_ERR_INVALID;
     if (mode != MI355X_FA_F16_SEQ && mode != MI355X_FA_F32 && mode != MI355X_FA_F16_PACKED) return MI355X_ERR_INVALID;
     if (q->type != MI355X_TYPE_F32 || k->type != MI355X_TYPE_F16 || v->type != MI355X_TYPE_F16 || dst->type != MI355X_TYPE_F32) return MI355X_ERR_UNSUPPORTED;
     if (q->ne[0] != FA_D || k->ne[0] != FA_D || v->ne[0] != FA_D) return MI355X_ERR_UNSUPPORTED;
@@ -904,6 +926,13 @@ extern "C" int mi355x_flash_attn_ext(const mi355x_tensor * q, const mi355x_tenso
         // only the tile kernels write the image; say so rather than silently skip it
         if (fa_kernel(q, k, mode) != FA_K_SEQ_TILE && fa_kernel(q, k, mode) != FA_K_MFMA) return MI355X_ERR_UNSUPPORTED;
         if (!workspace || (uintptr_t) workspace % 16 != 0 || workspace_size < (size_t)(N * H * q->ne[3]) * FA_D * sizeof(half_t)) return MI355X_ERR_WORKSPACE;
+        a.x16 = (half_t *) workspace;
+    }
+    if (emit_q8) {
+        // the few-query kernel writes the Q8_0 form
+        if (fa_kernel(q, k, mode) != FA_K_SEQ_ROW) return MI355X_ERR_UNSUPPORTED;
+        const size_t rows = (size_t)(N * q->ne[3]), K = (size_t) H * FA_D;
+        if (!workspace || (uintptr_t) workspace % 16 != 0 || workspace_size < rows * K + rows * (K / 32) * 8) return MI355X_ERR_WORKSPACE;
         a.x16 = (half_t *) workspace;
     }
     hipStream_t st = (hipStream_t) stream;
