@@ -59,7 +59,9 @@ def model_file(arch: str, ftype: str) -> str:
 
 # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled by the same counters over a 256 MiB copy:
 # x2 KiB and x1 KiB), for the large-v3 encoder shapes; the summary with the commands is under profiles/
-MEASURED_TRAFFIC_MB = {"mul_mat.gemm_q5_0": 47.4 + 5.5, "flash_attn.seq_tile": 70.9 + 7.7}
+# (mul_mat.gemm_q5_0 averages its two templates: 64 launches of 86.7 + 7.7 MB and 32 of 149.0 + 48.4 MB per window)
+MEASURED_TRAFFIC_MB = {"mul_mat.gemm_q5_0": (64 * (86.7 + 7.7) + 32 * (149.0 + 48.4)) / 96, "flash_attn.seq_tile": 70.9 + 11.5,
+                       "mul_mat.gemm_group": 144.3 + 23.1, "norm_affine_emit": 9.1 + 13.8}
 
 # kernels that live on the matrix cores (bound "mfma"); everything else streams memory (bound "hbm")
 MFMA_KERNELS = ("mul_mat.gemm_", "flash_attn.seq_tile")
@@ -116,6 +118,10 @@ def main() -> int:
         rooflines[n] = kernel_roofline(n, k)
     dom_name = max(kernels, key=lambda n: kernels[n]["ms"]) if kernels else None
     roofline = rooflines.get(dom_name)
+    if roofline and dom_name == "flash_attn.seq_tile":
+        roofline["note"] = ("priced against the dense f16 matrix-core peak as the brief asks; the matrix cores only form the scores. "
+                            "The reference accumulates V key by key in f16 (f32 fma, f16 store), and reproducing that takes 1.5 vector "
+                            "instructions per (query, key, d): 110 us per launch at the vector units' issue rate, which is the bound that applies")
 
     # ---- the same window with the packed f16 attention option (an optional arithmetic, reported beside the headline) -------
     packed = run_harness(["bench", "--model", enc_model, "--what", "encoder", "--backend", "gpu", "--reps", str(a.steps),
@@ -129,11 +135,15 @@ def main() -> int:
     dec = run_harness(["bench", "--model", dec_model, "--what", "decoder", "--backend", "gpu", "--reps", "3", "--warmup", "2",
                        "--steps", "224", "--batch", "5", "--profile", "--threads", str(a.threads)])
     dk = {k["kernel"]: k for k in dec["kernels"]}
-    gemv = dk.get("mul_mat.gemv_q8_0")
+    gemv = dk.get("mul_mat.gemv_q8_0.vocab")     # the logits product, 70.5 MB of Q8_0 blocks: the one GEMV that bandwidth bounds
     decode = {"model": "large-v3-turbo Q8_0", "steps": dec["steps"], "beams": dec["batch"], "ms_per_step": round(dec["ms_per_step"], 4),
               "steps_per_s": round(dec["steps_per_s"], 1), "beam_tokens_per_s": round(dec["batch_tokens_per_s"], 1)}
     if gemv:
-        decode["gemv_roofline"] = kernel_roofline("mul_mat.gemv_q8_0", gemv)
+        decode["gemv_roofline"] = kernel_roofline("mul_mat.gemv_q8_0.vocab", gemv)
+        decode["gemv_roofline"]["traffic"] = round(70.7e6 + 1.3e6)
+    if dk.get("mul_mat.gemv_q8_0"):
+        # the 32 products per step over 1.7 ... 7 MB matrices: over in the launch-to-store latency of a small kernel
+        decode["gemv_small_roofline"] = kernel_roofline("mul_mat.gemv_q8_0", dk["mul_mat.gemv_q8_0"])
     decode["kernel_breakdown"] = {n: {"launches_per_step": k["calls"] / dec["steps"], "ms_per_step": round(k["ms"] / dec["steps"], 4)}
                                   for n, k in sorted(dk.items(), key=lambda kv: -kv[1]["ms"])[:6]}
 
