@@ -4,7 +4,7 @@
 #include "common.h"
 
 #define ROWS_PER_BLOCK 4
-#define NORM_MAX_V4    8      // rows up to 64*4*8 = 2048 floats are held in registers between the passes
+#define NORM_MAX_V4    8      // rows up to 64*4*8 = 2048 floats are held in registers between the passes (NV = float4s per lane)
 
 // ------------------------------------------------------------------------------------------------------
 // NORM (ggml/src/ggml-cpu/ops.cpp:3109-3158): mean, then variance of the centred values, then scale.
@@ -15,8 +15,8 @@
 // dense [nrows][ne0] — so that the products that follow need no conversion pass of their own.
 // EMIT == 2: the row quantized to Q8_0 itself, in the layout the few-column product reads its activations from
 // (int8 q[nrows][ne0] | float d[nrows][ne0/32] | int32 sum of a block's quants).
-template <bool IN_REGS, int EMIT>
-__global__ void k_norm(tview s, tview d, int64_t nrows, float eps, const float * __restrict__ w, const float * __restrict__ b, half_t * __restrict__ x16) {
+template <int NV, int EMIT>
+__global__ void __launch_bounds__(ROWS_PER_BLOCK * WAVE) k_norm(tview s, tview d, int64_t nrows, float eps, const float * __restrict__ w, const float * __restrict__ b, half_t * __restrict__ x16) {
     const int     lane = threadIdx.x % WAVE;
     const int64_t row  = (int64_t) blockIdx.x * ROWS_PER_BLOCK + threadIdx.x / WAVE;
     if (row >= nrows) return;
@@ -25,26 +25,26 @@ __global__ void k_norm(tview s, tview d, int64_t nrows, float eps, const float *
     float *       y = (float *)(d.p + i1*d.nb1 + i2*d.nb2 + i3*d.nb3);
     const int64_t ne0 = s.ne0;
 
-    if (IN_REGS) {
+    if (NV > 0) {
         const int n4 = (int)(ne0 / 4);
-        float4 v[NORM_MAX_V4], ww[NORM_MAX_V4], bb[NORM_MAX_V4];
+        float4 v[NV ? NV : 1], ww[NV ? NV : 1], bb[NV ? NV : 1];
         // the affine vectors are fetched together with the row, not after the two reductions
 #pragma unroll
-        for (int j = 0; j < NORM_MAX_V4; ++j) {
+        for (int j = 0; j < NV; ++j) {
             const int c = lane + j * WAVE;
             ww[j] = make_float4(1.f, 1.f, 1.f, 1.f); bb[j] = make_float4(0.f, 0.f, 0.f, 0.f);
             if (c < n4) { if (w) ww[j] = ((const float4 *) w)[c]; if (b) bb[j] = ((const float4 *) b)[c]; }
         }
         float sum = 0.0f;
 #pragma unroll
-        for (int j = 0; j < NORM_MAX_V4; ++j) {
+        for (int j = 0; j < NV; ++j) {
             const int c = lane + j * WAVE;
             if (c < n4) { v[j] = ((const float4 *) x)[c]; sum += (v[j].x + v[j].y) + (v[j].z + v[j].w); }
         }
         const float mean = wave_sum(sum) / (float) ne0;
         float sum2 = 0.0f;
 #pragma unroll
-        for (int j = 0; j < NORM_MAX_V4; ++j) {
+        for (int j = 0; j < NV; ++j) {
             const int c = lane + j * WAVE;
             if (c < n4) {
                 v[j].x -= mean; v[j].y -= mean; v[j].z -= mean; v[j].w -= mean;
@@ -53,7 +53,7 @@ __global__ void k_norm(tview s, tview d, int64_t nrows, float eps, const float *
         }
         const float scale = 1.0f / sqrtf(wave_sum(sum2) / (float) ne0 + eps);
 #pragma unroll
-        for (int j = 0; j < NORM_MAX_V4; ++j) {
+        for (int j = 0; j < NV; ++j) {
             const int c = lane + j * WAVE;
             if (c < n4) {
                 float4 r = { v[j].x * scale, v[j].y * scale, v[j].z * scale, v[j].w * scale };
@@ -134,14 +134,29 @@ static int norm_impl(const mi355x_tensor * src, const mi355x_tensor * dst, float
     const bool in_regs = src->ne[0] % 4 == 0 && src->ne[0] <= 4 * WAVE * NORM_MAX_V4 &&
                          al16(src->data, src->nb) && al16(dst->data, dst->nb) &&
                          (uintptr_t) w % 16 == 0 && (uintptr_t) b % 16 == 0;
-    if (x16) {                                             // only the register-resident form emits, and only whole blocks
-        if (!in_regs || src->ne[0] % QK != 0) return MI355X_ERR_UNSUPPORTED;
-        if (emit == 2) k_norm<true, 2><<<(unsigned) grid, ROWS_PER_BLOCK * WAVE, 0, st>>>(make_view(src), make_view(dst), nrows, eps, w, b, (half_t *) x16);
-        else           k_norm<true, 1><<<(unsigned) grid, ROWS_PER_BLOCK * WAVE, 0, st>>>(make_view(src), make_view(dst), nrows, eps, w, b, (half_t *) x16);
-        return launch_status();
+    // the register-resident form is compiled per row length (float4s per lane), so that a 1280-wide row runs five
+    // iterations' worth of code, not eight guarded ones: these kernels are latency, not bandwidth, when the rows are few
+    const int nv = in_regs ? (int)((src->ne[0] / 4 + WAVE - 1) / WAVE) : 0;
+    if (x16 && (!in_regs || src->ne[0] % QK != 0)) return MI355X_ERR_UNSUPPORTED;      // only that form emits, and only whole blocks
+    const tview vs = make_view(src), vd = make_view(dst);
+    const unsigned g = (unsigned) grid, t = ROWS_PER_BLOCK * WAVE;
+#define NORM_LAUNCH(NV) \
+    do { \
+        if (!x16)           k_norm<NV, 0><<<g, t, 0, st>>>(vs, vd, nrows, eps, w, b, nullptr); \
+        else if (emit == 2) k_norm<NV, 2><<<g, t, 0, st>>>(vs, vd, nrows, eps, w, b, (half_t *) x16); \
+        else                k_norm<NV, 1><<<g, t, 0, st>>>(vs, vd, nrows, eps, w, b, (half_t *) x16); \
+    } while (0)
+    switch (nv) {
+        case 0:  k_norm<0, 0><<<g, t, 0, st>>>(vs, vd, nrows, eps, w, b, nullptr); break;
+        case 1:  NORM_LAUNCH(1); break;
+        case 2:  NORM_LAUNCH(2); break;
+        case 3:  NORM_LAUNCH(3); break;
+        case 4:  NORM_LAUNCH(4); break;
+        case 5:  NORM_LAUNCH(5); break;
+        case 6:  NORM_LAUNCH(6); break;
+        default: NORM_LAUNCH(8); break;
     }
-    if (in_regs) k_norm<true,  0><<<(unsigned) grid, ROWS_PER_BLOCK * WAVE, 0, st>>>(make_view(src), make_view(dst), nrows, eps, w, b, nullptr);
-    else         k_norm<false, 0><<<(unsigned) grid, ROWS_PER_BLOCK * WAVE, 0, st>>>(make_view(src), make_view(dst), nrows, eps, w, b, nullptr);
+#undef NORM_LAUNCH
     return launch_status();
 }
 
