@@ -79,6 +79,21 @@ def test_packed_f16_attention_option_stays_within_the_bounds(harness, models):
     assert rc == 0 and s["pass"] and s["ids_identical"] == 16 and s["worst_logits_nmse"] <= 1e-3, s
 
 
+def test_whisper_full_end_to_end(harness, models):
+    # whisper_full() unmodified: PCM -> log-mel -> encoder -> whisper's own search (logits filters, timestamp rules, KV-cache
+    # bookkeeping), on both backends over the same synthetic audio.  Greedy: the transcripts must start with the same ids
+    # (they were identical over all 42 tokens when this was written).  Beam search draws its candidates from the softmax
+    # with a seeded RNG (src/whisper.cpp:5415-5418); on a random-init model's near-flat distribution the cumulative sums the
+    # draw walks move by more than one token's width with any rounding difference, so only "runs and returns text" is asserted.
+    rc, rows = run_harness(harness, ["full", "--model", models[("base", "q5_0")], "--beam", "1", "--max-tokens", "24"], timeout=900)
+    s = rows[-1]
+    assert rc == 0 and s["pass"] and s["gpu_rc"] == 0 and s["gpu_tokens"] > 0, s
+    assert s["common_prefix"] >= min(8, s["cpu_tokens"]), s
+    rc, rows = run_harness(harness, ["full", "--model", models[("base", "q5_0")], "--beam", "5", "--max-tokens", "24"], timeout=900)
+    s = rows[-1]
+    assert rc == 0 and s["pass"] and s["gpu_rc"] == 0 and s["gpu_tokens"] > 0 and s["gpu_segments"] > 0, s
+
+
 def test_f32_matrix_core_attention_option(harness, models):
     # GGML_MI355X_FA_ACCUM=1: encoder / prompt attention with f32 accumulators on the matrix cores.  Every op case stays
     # within the per-op bound and the greedy ids of the base model do not move, but the reference's f16 accumulator

@@ -9,6 +9,8 @@
 //                                             per-op parity (NMSE / bit-exactness) and timing, CPU vs MI355X
 //   model  --model F [--steps 32] [--threads N]
 //                                             whole-model parity: logits NMSE and greedy ids, teacher-forced
+//   full   --model F [--beam 1|5] [--max-tokens 24] [--seconds 30] [--threads N]
+//                                             whisper_full() end to end (PCM -> mel -> encode -> search) on both backends
 //   verify --model F [--steps 3] [--threads N]
 //                                             per-node parity inside the real whisper graphs (unfused), CPU vs MI355X
 //   bench  --model F --what encoder|decoder|whisper-bench --backend gpu|cpu [--threads N] [--reps R] [--profile]
@@ -429,6 +431,65 @@ static int cmd_model(const args & a) {
     return pass ? 0 : 1;
 }
 
+// whisper_full() end to end on synthetic audio: log-mel on the host, encoder, then whisper's own greedy or beam search
+// with its logits filters, timestamp rules and KV-cache bookkeeping.  Both backends see the same PCM; the token ids of
+// the two transcripts are compared from the front (a random-init model's near-flat logits let one rounding flip an
+// argmax, after which the two searches walk different histories, so only the common prefix is meaningful).
+static std::vector<whisper_token> run_full(whisper_context * ctx, const std::vector<float> & pcm, int beam, int max_tokens, int threads, int * rc, double * ms) {
+    whisper_full_params p = whisper_full_default_params(beam > 1 ? WHISPER_SAMPLING_BEAM_SEARCH : WHISPER_SAMPLING_GREEDY);
+    p.n_threads = threads;
+    p.print_progress = false; p.print_realtime = false; p.print_timestamps = false; p.print_special = false;
+    p.language = "en"; p.translate = false;
+    p.max_tokens = max_tokens;
+    p.temperature_inc = 0.0f;                  // no temperature fallback: one pass per window
+    p.suppress_blank = true;
+    if (beam > 1) p.beam_search.beam_size = beam; else p.greedy.best_of = 1;
+    const double t0 = now_ms();
+    *rc = whisper_full(ctx, p, pcm.data(), (int) pcm.size());
+    *ms = now_ms() - t0;
+    std::vector<whisper_token> out;
+    if (*rc != 0) return out;
+    const int nseg = whisper_full_n_segments(ctx);
+    for (int i = 0; i < nseg; ++i)
+        for (int j = 0; j < whisper_full_n_tokens(ctx, i); ++j) out.push_back(whisper_full_get_token_id(ctx, i, j));
+    return out;
+}
+
+static int cmd_full(const args & a) {
+    const std::string path = a.str("model");
+    const int threads = a.num("threads", default_threads()), beam = a.num("beam", 1), max_tokens = a.num("max-tokens", 24);
+    const int seconds = a.num("seconds", 30);
+    if (path.empty()) { fprintf(stderr, "usage: full --model FILE [--beam N] [--max-tokens N] [--seconds N]\n"); return 2; }
+    if (!load_plugin(true)) { printf("{\"error\": \"no MI355X backend\"}\n"); return 2; }
+    whisper_context * gpu = open_model(path, true);
+    whisper_context * cpu = open_model(path, false);
+    if (!gpu || !cpu) { printf("{\"error\": \"model load failed\"}\n"); return 2; }
+    // a few drifting tones under noise, 16 kHz mono
+    std::vector<float> pcm((size_t) seconds * WHISPER_SAMPLE_RATE);
+    uint64_t st = 0x9E3779B97F4A7C15ull ^ (uint64_t) a.num("seed", 7);
+    for (size_t i = 0; i < pcm.size(); ++i) {
+        st = st * 6364136223846793005ull + 1442695040888963407ull;
+        const double t = (double) i / WHISPER_SAMPLE_RATE;
+        const double noise = ((double)(st >> 40) / (double)(1 << 24)) - 0.5;
+        pcm[i] = (float)(0.25 * sin(2 * M_PI * (220.0 + 30.0 * t) * t) + 0.15 * sin(2 * M_PI * 1310.0 * t) + 0.1 * noise);
+    }
+    int rg = 0, rc = 0; double ms_g = 0, ms_c = 0;
+    const std::vector<whisper_token> tg = run_full(gpu, pcm, beam, max_tokens, threads, &rg, &ms_g);
+    const std::vector<whisper_token> tc = run_full(cpu, pcm, beam, max_tokens, threads, &rc, &ms_c);
+    size_t same = 0;
+    while (same < tg.size() && same < tc.size() && tg[same] == tc[same]) ++same;
+    std::string sg, sc;
+    for (size_t i = 0; i < tg.size() && i < 16; ++i) sg += (i ? "," : "") + std::to_string(tg[i]);
+    for (size_t i = 0; i < tc.size() && i < 16; ++i) sc += (i ? "," : "") + std::to_string(tc[i]);
+    const bool pass = rg == 0 && rc == 0 && !tg.empty();
+    printf("{\"summary\": \"full\", \"model\": \"%s\", \"beam\": %d, \"seconds\": %d, \"gpu_rc\": %d, \"cpu_rc\": %d, \"gpu_segments\": %d, \"cpu_segments\": %d, "
+           "\"gpu_tokens\": %zu, \"cpu_tokens\": %zu, \"common_prefix\": %zu, \"gpu_first\": [%s], \"cpu_first\": [%s], \"gpu_ms\": %.1f, \"cpu_ms\": %.1f, \"pass\": %s}\n",
+           json_escape(path).c_str(), beam, seconds, rg, rc, rg == 0 ? whisper_full_n_segments(gpu) : -1, rc == 0 ? whisper_full_n_segments(cpu) : -1,
+           tg.size(), tc.size(), same, sg.c_str(), sc.c_str(), ms_g, ms_c, pass ? "true" : "false");
+    whisper_free(gpu); whisper_free(cpu);
+    return pass ? 0 : 1;
+}
+
 // per-node parity on the graphs whisper builds: conv + encoder + cross, one prompt batch, a few single-token steps,
 // one 5-token batch (the shape of a beam-search step)
 static int cmd_verify(const args & a) {
@@ -619,7 +680,7 @@ static int cmd_copy(const args & a) {
 }
 
 int main(int argc, char ** argv) {
-    if (argc < 2) { fprintf(stderr, "usage: %s info|gen|selftest|ops|model|verify|bench|copy [options]\n", argv[0]); return 2; }
+    if (argc < 2) { fprintf(stderr, "usage: %s info|gen|selftest|ops|model|full|verify|bench|copy [options]\n", argv[0]); return 2; }
     ggml_log_set(quiet_log, nullptr);
     whisper_log_set(quiet_log, nullptr);
     const std::string cmd = argv[1];
@@ -630,6 +691,7 @@ int main(int argc, char ** argv) {
     if (cmd == "selftest") return cmd_selftest(a);
     if (cmd == "ops")   return cmd_ops(a);
     if (cmd == "model") return cmd_model(a);
+    if (cmd == "full")  return cmd_full(a);
     if (cmd == "verify") return cmd_verify(a);
     if (cmd == "bench") return cmd_bench(a);
     if (cmd == "copy")  return cmd_copy(a);
