@@ -129,7 +129,9 @@ MI355X_API int    mi355x_mul_mat(const mi355x_tensor * src0, const mi355x_tensor
  * device where a single 1280-row product covers half of it.  No counterpart in the reference, whose graphs issue these
  * products one node at a time.  Only the shape this exists for: every src0 a dense 2-d F16 matrix of the same size (e.g.
  * the f16 images of quantized weights, with MI355X_MM_ACT_Q8_0 in `flags`), K a multiple of 256, more than 8 columns,
- * count <= 64; anything else returns MI355X_ERR_UNSUPPORTED and the caller issues single calls.
+ * count <= 64 — or, for at most 8 columns, every src0 a Q5_0 / Q8_0 matrix of one type and size that takes the
+ * workspace form of the few-column product (mi355x_mul_mat_workspace_size > 0), count <= 8: a decode step's Q, K and V;
+ * anything else returns MI355X_ERR_UNSUPPORTED and the caller issues single calls.
  * `flags`: MI355X_MM_* options common to all items; the items' epilogues carry MI355X_EPI_* only. */
 typedef struct mi355x_mul_mat_item {
     const mi355x_tensor *   src0;

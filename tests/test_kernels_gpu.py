@@ -265,6 +265,47 @@ def test_mul_mat_group_equals_single_calls(pkg, oracle, gpu):
     assert lib.mi355x_mul_mat_group(it, 1, pkg.tensor(xs, pkg.F32), 0, ws.data_ptr(), need, gpu.stream) == -1
 
 
+@pytest.mark.parametrize("wtype,n", [("Q8_0", 5), ("Q5_0", 1), ("Q8_0", 8)])
+def test_mul_mat_group_few_columns(pkg, oracle, gpu, wtype, n):
+    # a decode step's Q, K and V in one launch: the same results as single calls (same kernel body, same order of sums)
+    lib = pkg.kernels()
+    t = getattr(pkg, wtype)
+    k, m = 1280, 1280
+    x = rnd((n, k))
+    d_x = gpu.up(x)
+    tx = pkg.tensor(d_x, pkg.F32)
+    mats = [oracle.quantize(t, rnd((m, k), 0.02)) for _ in range(3)]
+    d_w = [gpu.up(b) for b in mats]
+    tws = [pkg.tensor(w, t, ne=[k, m]) for w in d_w]
+    bias = rnd((m,), 0.5)
+    d_b = gpu.up(bias)
+    need = lib.mi355x_mul_mat_workspace_size(tws[0], tx)
+    assert need > 0
+    ws = torch.empty(need, dtype=torch.uint8, device=gpu.dev)
+    outs = [torch.zeros((n, m), dtype=torch.float32, device=gpu.dev), torch.zeros((n, m), dtype=torch.float16, device=gpu.dev),
+            torch.zeros((n, m), dtype=torch.float32, device=gpu.dev)]
+    tds = [pkg.tensor(outs[0], pkg.F32), pkg.tensor(outs[1], pkg.F16), pkg.tensor(outs[2], pkg.F32)]
+    epis = [pkg.Epilogue() for _ in range(3)]
+    epis[0].flags, epis[0].scale, epis[0].bias = pkg.EPI_BIAS | pkg.EPI_SCALE, 0.125, d_b.data_ptr()
+    epis[1].flags, epis[1].scale = pkg.EPI_OUT_F16, 1.0
+    epis[2].flags, epis[2].scale, epis[2].bias = pkg.EPI_BIAS, 1.0, d_b.data_ptr()
+    items = (pkg.MulMatItem * 3)()
+    for i in range(3):
+        items[i].src0, items[i].dst, items[i].epi = C.pointer(tws[i]), C.pointer(tds[i]), C.pointer(epis[i])
+    pkg.check(lib.mi355x_mul_mat_group(items, 3, tx, 0, ws.data_ptr(), need, gpu.stream))
+    got = [gpu.down(o).astype(np.float32) for o in outs]
+    for i in range(3):
+        single = torch.zeros_like(outs[i])
+        pkg.check(lib.mi355x_mul_mat(tws[i], tx, pkg.tensor(single, pkg.F16 if i == 1 else pkg.F32), C.byref(epis[i]), ws.data_ptr(), need, gpu.stream))
+        assert np.array_equal(got[i], gpu.down(single).astype(np.float32))
+    base = [oracle.mul_mat(t, b, x) for b in mats]
+    assert oracle.nmse(got[0], (base[0] + bias) * np.float32(0.125)) <= 1e-10
+    assert oracle.nmse(got[1], oracle.f16_bits_to_f32(oracle.f32_to_f16_bits(base[1]))) <= 1e-10
+    assert oracle.nmse(got[2], base[2] + bias) <= 1e-10
+    # without the workspace the grouped form has nothing to read the activations from
+    assert lib.mi355x_mul_mat_group(items, 3, tx, 0, None, 0, gpu.stream) == -3
+
+
 def test_mul_mat_rejects_bad_arguments(pkg, gpu):
     lib = pkg.kernels()
     d_w = torch.zeros(22 * 4, dtype=torch.uint8, device=gpu.dev)

@@ -328,12 +328,16 @@ struct graph_runner {
     // Products that follow each other over the same activations with weights of one shape (Q, K, V of a layer; the
     // cross-attention K / V of all decoder layers) go out as one launch.  Returns the nodes consumed, 0 if no group formed.
     int run_mul_mat_group(int i, const mm_chain & first, const mm_operands & o0, int & status) {
-        if (!ctx->fuse || o0.vw.type != MI355X_TYPE_F16 || strncmp(o0.kernel_name, "mul_mat.gemm", 12) != 0) return 0;
-        if (first.mm->ne[2] != 1 || first.mm->ne[3] != 1 || first.w->ne[0] % 256 != 0) return 0;
+        // (the few-column form: a decode step's Q, K and V over quantized weights, up to 8 products)
+        const bool gemv = strncmp(o0.kernel_name, "mul_mat.gemv", 12) == 0;
+        if (!ctx->fuse || first.mm->ne[2] != 1 || first.mm->ne[3] != 1) return 0;
+        if (gemv) {
+            if (mi355x_mul_mat_workspace_size(&o0.vw, &o0.vx) == 0) return 0;
+        } else if (o0.vw.type != MI355X_TYPE_F16 || strncmp(o0.kernel_name, "mul_mat.gemm", 12) != 0 || first.w->ne[0] % 256 != 0) return 0;
         std::vector<mm_chain>    chains{ first };
         std::vector<mm_operands> ops{ o0 };
         int end = i + first.used;                       // first node after the group
-        while ((int) chains.size() < 64) {
+        while ((int) chains.size() < (gemv ? 8 : 64)) {
             int j = end;
             while (node_at(j) && (is_view_op(node_at(j)->op) || ggml_is_empty(node_at(j)))) ++j;
             ggml_tensor * n = node_at(j);
@@ -341,7 +345,7 @@ struct graph_runner {
                 !ggml_are_same_shape(n->src[0], first.w) || !ggml_are_same_shape(n, first.mm)) break;
             mm_chain c = plan_chain(j);
             mm_operands o = describe(c);
-            if (o.vw.type != MI355X_TYPE_F16 || o.mm_flags != o0.mm_flags || o.vw.nb[1] != o0.vw.nb[1]) break;
+            if (o.vw.type != o0.vw.type || o.mm_flags != o0.mm_flags || o.vw.nb[1] != o0.vw.nb[1]) break;
             // nothing in the group may read what another member writes
             bool clash = false;
             for (const mm_chain & p : chains) {
@@ -367,12 +371,12 @@ struct graph_runner {
         }
         int rc;
         {
-            launch_scope ls(ctx, "mul_mat.gemm_group", bytes, flops);
+            launch_scope ls(ctx, gemv ? "mul_mat.gemv_group" : "mul_mat.gemm_group", bytes, flops);
             rc = mi355x_mul_mat_group(items.data(), (int) items.size(), &o0.vx, o0.mm_flags | ready, ctx->ws, ctx->ws_size, ctx->stream);
         }
         if (rc == MI355X_ERR_UNSUPPORTED) return 0;     // the single-product path takes them one by one
         status = rc;
-        if (ctx->debug) GGML_LOG_INFO("ggml-mi355x: mul_mat.gemm_group of %zu starting at %s, %d nodes\n", chains.size(), first.mm->name, end - i);
+        if (ctx->debug) GGML_LOG_INFO("ggml-mi355x: %s of %zu starting at %s, %d nodes\n", gemv ? "mul_mat.gemv_group" : "mul_mat.gemm_group", chains.size(), first.mm->name, end - i);
         for (const mm_chain & c : chains) note_write(c.out);
         return end - i;
     }

@@ -752,7 +752,7 @@ __global__ void __launch_bounds__(256) k_quantize_x_q8(const char * __restrict__
 // the activations in LDS, their reads (NC x 32 bytes per 34-byte block) are what bounds the kernel, and quantizing them
 // in every workgroup costs more than the product itself once K is large.
 template <int T0, int NC, int LPR, int NB>
-__global__ void __launch_bounds__(256) k_gemv_qr(mm_args a) {
+__device__ __forceinline__ void gemv_qr_rows(const mm_args & a) {
     const int64_t K = a.K;
     const int nbk = (int)(K / QK);
     const int32_t * xq   = (const int32_t *) a.x;
@@ -882,6 +882,22 @@ __global__ void __launch_bounds__(256) k_gemv_qr(mm_args a) {
     }
 }
 
+template <int T0, int NC, int LPR, int NB>
+__global__ void __launch_bounds__(256) k_gemv_qr(mm_args a) { gemv_qr_rows<T0, NC, LPR, NB>(a); }
+
+// several products over the same activations in one launch (a decode step's Q, K and V): blockIdx.y picks the matrix
+struct gemv_group_entry { const char * w; char * d; const float * bias; const char * residual; int64_t d_nb1; int flags; float scale; };
+#define GEMV_GROUP_MAX 8
+struct gemv_group { gemv_group_entry e[GEMV_GROUP_MAX]; };
+
+template <int T0, int NC, int LPR, int NB>
+__global__ void __launch_bounds__(256) k_gemv_qr_group(mm_args a, gemv_group grp) {
+    const gemv_group_entry & ge = grp.e[blockIdx.y];
+    a.w = ge.w; a.d = ge.d; a.d_nb1 = ge.d_nb1;
+    a.e.flags = ge.flags; a.e.scale = ge.scale; a.e.bias = ge.bias; a.e.residual = ge.residual;
+    gemv_qr_rows<T0, NC, LPR, NB>(a);
+}
+
 // ------------------------------------------------------------------------------------------------------
 // generic fallback: one wavefront per (m, group of up to 8 columns, batch); element-wise dequant, f32 FMA
 // ------------------------------------------------------------------------------------------------------
@@ -969,44 +985,50 @@ static size_t gemv_ws_bytes(const mi355x_tensor * src0, const mi355x_tensor * sr
     return round256((size_t)(N * K + N * (K / QK) * 8));
 }
 
+template <int T0, int NC, int LPR, int NB>
+static int launch_gemv_r_k(const mm_args & a, unsigned grid, const gemv_group * grp, int count, hipStream_t st) {
+    if (grp) k_gemv_qr_group<T0, NC, LPR, NB><<<dim3(grid, (unsigned) count), 256, 0, st>>>(a, *grp);
+    else     k_gemv_qr<T0, NC, LPR, NB><<<grid, 256, 0, st>>>(a);
+    return launch_status();
+}
 template <int T0, int NC, int LPR>
-static int launch_gemv_r_nb(const mm_args & a, int nb, unsigned grid, hipStream_t st) {
+static int launch_gemv_r_nb(const mm_args & a, int nb, unsigned grid, const gemv_group * grp, int count, hipStream_t st) {
     switch (nb) {
-        case 1: k_gemv_qr<T0, NC, LPR, 1><<<grid, 256, 0, st>>>(a); return launch_status();
-        case 2: if constexpr (NC * 2 <= 15) { k_gemv_qr<T0, NC, LPR, 2><<<grid, 256, 0, st>>>(a); return launch_status(); } break;
-        case 3: if constexpr (NC * 3 <= 15) { k_gemv_qr<T0, NC, LPR, 3><<<grid, 256, 0, st>>>(a); return launch_status(); } break;
+        case 1: return launch_gemv_r_k<T0, NC, LPR, 1>(a, grid, grp, count, st);
+        case 2: if constexpr (NC * 2 <= 15) return launch_gemv_r_k<T0, NC, LPR, 2>(a, grid, grp, count, st); break;
+        case 3: if constexpr (NC * 3 <= 15) return launch_gemv_r_k<T0, NC, LPR, 3>(a, grid, grp, count, st); break;
     }
     return MI355X_ERR_UNSUPPORTED;
 }
 template <int T0, int NC>
-static int launch_gemv_r(const mm_args & a, hipStream_t st) {
-    const int lpr = gemv_r_lanes(a.M, NC, a.K);
+static int launch_gemv_r(const mm_args & a, hipStream_t st, const gemv_group * grp = nullptr, int count = 1) {
+    const int lpr = gemv_r_lanes(a.M * count, NC, a.K);
     if (!lpr) return MI355X_ERR_UNSUPPORTED;
     const int nb = (int)((a.K / QK + lpr - 1) / lpr);
     const int rows_per_wg = 4 * (WAVE / lpr);
     const int64_t n_groups = (a.M + rows_per_wg - 1) / rows_per_wg;
     // one resident set of workgroups (the registers allow 4 per CU with one block per lane, else 2), each walking its
     // share of the row groups: a second, partly filled set would double the time
-    const int64_t resident = 256 * (nb == 1 ? 4 : 2);
+    const int64_t resident = 256 * (nb == 1 ? 4 : 2) / count > 0 ? 256 * (nb == 1 ? 4 : 2) / count : 1;
     const int64_t rounds   = (n_groups + resident - 1) / resident;
     const unsigned grid    = (unsigned)((n_groups + rounds - 1) / rounds);
     switch (lpr) {
-        case 16: return launch_gemv_r_nb<T0, NC, 16>(a, nb, grid, st);
-        case 32: return launch_gemv_r_nb<T0, NC, 32>(a, nb, grid, st);
-        default: return launch_gemv_r_nb<T0, NC, 64>(a, nb, grid, st);
+        case 16: return launch_gemv_r_nb<T0, NC, 16>(a, nb, grid, grp, count, st);
+        case 32: return launch_gemv_r_nb<T0, NC, 32>(a, nb, grid, grp, count, st);
+        default: return launch_gemv_r_nb<T0, NC, 64>(a, nb, grid, grp, count, st);
     }
 }
 template <int T0>
-static int launch_gemv_r_n(const mm_args & a, hipStream_t st) {
+static int launch_gemv_r_n(const mm_args & a, hipStream_t st, const gemv_group * grp = nullptr, int count = 1) {
     switch (a.N) {
-        case 1: return launch_gemv_r<T0, 1>(a, st);
-        case 2: return launch_gemv_r<T0, 2>(a, st);
-        case 3: return launch_gemv_r<T0, 3>(a, st);
-        case 4: return launch_gemv_r<T0, 4>(a, st);
-        case 5: return launch_gemv_r<T0, 5>(a, st);
-        case 6: return launch_gemv_r<T0, 6>(a, st);
-        case 7: return launch_gemv_r<T0, 7>(a, st);
-        case 8: return launch_gemv_r<T0, 8>(a, st);
+        case 1: return launch_gemv_r<T0, 1>(a, st, grp, count);
+        case 2: return launch_gemv_r<T0, 2>(a, st, grp, count);
+        case 3: return launch_gemv_r<T0, 3>(a, st, grp, count);
+        case 4: return launch_gemv_r<T0, 4>(a, st, grp, count);
+        case 5: return launch_gemv_r<T0, 5>(a, st, grp, count);
+        case 6: return launch_gemv_r<T0, 6>(a, st, grp, count);
+        case 7: return launch_gemv_r<T0, 7>(a, st, grp, count);
+        case 8: return launch_gemv_r<T0, 8>(a, st, grp, count);
     }
     return MI355X_ERR_INVALID;
 }
@@ -1098,12 +1120,60 @@ extern "C" size_t mi355x_mul_mat_workspace_size(const mi355x_tensor * src0, cons
     return x16_bytes(src1) + w16_bytes(src0);
 }
 
+// the few-column form of mi355x_mul_mat_group: quantized weights of one type and shape, activations quantized once
+static int mul_mat_group_gemv(const mi355x_mul_mat_item * items, int count, const mi355x_tensor * src1, int flags,
+                              void * workspace, size_t workspace_size, void * stream) {
+    const mi355x_tensor * w0 = items[0].src0;
+    if (count > GEMV_GROUP_MAX || src1->type != MI355X_TYPE_F32 || mm_path(w0, src1) != MM_GEMV) return MI355X_ERR_UNSUPPORTED;
+    if (w0->type != MI355X_TYPE_Q8_0 && w0->type != MI355X_TYPE_Q5_0) return MI355X_ERR_UNSUPPORTED;
+    mm_args a;
+    a.K = w0->ne[0]; a.M = w0->ne[1]; a.N = src1->ne[1];
+    if (src1->ne[0] != a.K || a.K % QK != 0) return MI355X_ERR_INVALID;
+    if (a.M == 0 || a.N == 0) return MI355X_OK;
+    const size_t need = gemv_ws_bytes(w0, src1);
+    if (!need || !gemv_r_lanes(a.M * count, a.N, a.K)) return MI355X_ERR_UNSUPPORTED;
+    if (!workspace || workspace_size < need || (uintptr_t) workspace % 16 != 0) return MI355X_ERR_WORKSPACE;
+    gemv_group grp;
+    bool any_gelu = false;
+    for (int i = 0; i < count; ++i) {
+        const mi355x_tensor * w = items[i].src0, * d = items[i].dst;
+        const mi355x_epilogue * e = items[i].epi;
+        if (!w || !d) return MI355X_ERR_INVALID;
+        if (w->type != w0->type || w->ne[0] != a.K || w->ne[1] != a.M || w->ne[2] != 1 || w->ne[3] != 1 || w->nb[1] != w0->nb[1] || (uintptr_t) w->data % 2 != 0) return MI355X_ERR_UNSUPPORTED;
+        if (e && (e->flags & MI355X_EPI_EMIT_F16)) return MI355X_ERR_UNSUPPORTED;
+        const int ef = e ? (e->flags & 63) : 0;
+        const int td = (ef & MI355X_EPI_OUT_F16) ? MI355X_TYPE_F16 : MI355X_TYPE_F32;
+        if (d->type != td || d->ne[0] != a.M || d->ne[1] != a.N || d->ne[2] != 1 || d->ne[3] != 1 || d->nb[0] != type_size(td)) return MI355X_ERR_UNSUPPORTED;
+        if ((ef & (MI355X_EPI_BIAS | MI355X_EPI_BIAS_COL)) && !e->bias) return MI355X_ERR_INVALID;
+        if ((ef & MI355X_EPI_BIAS) && (ef & MI355X_EPI_BIAS_COL)) return MI355X_ERR_INVALID;
+        if ((ef & MI355X_EPI_RESIDUAL) && (!e->residual || (ef & MI355X_EPI_OUT_F16))) return MI355X_ERR_INVALID;
+        any_gelu = any_gelu || (ef & MI355X_EPI_GELU);
+        grp.e[i] = { (const char *) w->data, (char *) d->data, e ? (const float *) e->bias : nullptr, e ? (const char *) e->residual : nullptr, (int64_t) d->nb[1], ef, e ? e->scale : 1.0f };
+    }
+    a.w = (const char *) w0->data; a.x = (const char *) src1->data; a.d = (char *) items[0].dst->data;
+    a.w_nb1 = w0->nb[1]; a.w_nb2 = a.w_nb3 = 0;
+    a.x_nb1 = src1->nb[1]; a.x_nb2 = a.x_nb3 = 0;
+    a.d_nb1 = items[0].dst->nb[1]; a.d_nb2 = a.d_nb3 = 0;
+    a.ne12 = a.ne13 = a.r2 = a.r3 = 1;
+    a.e.flags = 0; a.e.scale = 1.0f; a.e.bias = nullptr; a.e.residual = nullptr; a.e.gelu = nullptr; a.e.image = nullptr;
+    if (any_gelu && !(a.e.gelu = gelu_table_device())) return MI355X_ERR_HIP;
+    hipStream_t st = (hipStream_t) stream;
+    if (!(flags & MI355X_MM_WS_READY)) {
+        k_quantize_x_q8<<<(unsigned)((a.N * (a.K / 4) + 255) / 256), 256, 0, st>>>(a.x, a.x_nb1, a.K, a.N, (char *) workspace);
+        if (const int rc = launch_status()) return rc;
+    }
+    if (flags & MI355X_MM_PREPARE_ONLY) return MI355X_OK;
+    a.x = (const char *) workspace;
+    return w0->type == MI355X_TYPE_Q8_0 ? launch_gemv_r_n<MI355X_TYPE_Q8_0>(a, st, &grp, count) : launch_gemv_r_n<MI355X_TYPE_Q5_0>(a, st, &grp, count);
+}
+
 extern "C" int mi355x_mul_mat_group(const mi355x_mul_mat_item * items, int count, const mi355x_tensor * src1, int flags,
                                     void * workspace, size_t workspace_size, void * stream) {
     if (!items || !src1 || count < 1) return MI355X_ERR_INVALID;
     if (count > MM_GROUP_MAX) return MI355X_ERR_UNSUPPORTED;
     const mi355x_tensor * w0 = items[0].src0;
     if (!w0 || !items[0].dst) return MI355X_ERR_INVALID;
+    if (blck_size(w0->type) > 1) return mul_mat_group_gemv(items, count, src1, flags, workspace, workspace_size, stream);
     // one shape of problem only: dense f16 weights (or weight images), 2-d, K a multiple of 256, the MFMA GEMM path
     if (w0->type != MI355X_TYPE_F16 || (src1->type != MI355X_TYPE_F32 && src1->type != MI355X_TYPE_F16)) return MI355X_ERR_UNSUPPORTED;
     if (src1->ne[2] != 1 || src1->ne[3] != 1 || w0->ne[2] != 1 || w0->ne[3] != 1) return MI355X_ERR_UNSUPPORTED;
