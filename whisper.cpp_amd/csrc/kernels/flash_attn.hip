@@ -154,7 +154,8 @@ __device__ __forceinline__ void seq_factors(float s, float & M, float & vs, floa
 // ------------------------------------------------------------------------------------------------------
 
 #define ROW_CHUNK 64
-#define ROW_STAGE 256     // keys staged per step = threads per workgroup
+#define ROW_STAGE 192     // keys staged per step: one per thread of the three wavefronts that do not walk the chain
+#define ROW_VT    (ROW_STAGE + 8)   // f16 pitch of a d-row of the transposed V stage
 
 __global__ void __launch_bounds__(256) k_fattn_seq_row(fa_args a, int kv_pad) {
     extern __shared__ __attribute__((aligned(16))) float sm[];
@@ -179,23 +180,32 @@ __global__ void __launch_bounds__(256) k_fattn_seq_row(fa_args a, int kv_pad) {
         const float4 t = *(const float4 *)(qp + d);
         q[d] = (float)(half_t) t.x; q[d+1] = (float)(half_t) t.y; q[d+2] = (float)(half_t) t.z; q[d+3] = (float)(half_t) t.w;
     }
-    for (int key = tid; key < kv_pad; key += 256) {
-        float s = -INFINITY;
-        if (key < KV) {
-            const float mv = mp ? (float) mp[key] : 0.0f;
-            if (mv != -INFINITY) {
-                const half8_t * kr = (const half8_t *)(kb + (int64_t) key * a.k_nb1);
-                float dot = 0.0f;
+    // keys tid, tid + 256, ...: the next key's row (and mask value) is in flight while this one's dot product is formed;
+    // the loads are unconditional (clamped) so that the wait in front of the dot product covers this key's row only
+    {
+        half8_t kcur[FA_D / 8], knext[FA_D / 8];
+        float mcur = 0.0f, mnext = 0.0f;
+        auto load_key = [&](half8_t (&kk)[FA_D / 8], float & mv, int key) __attribute__((always_inline)) {
+            const int kc = key < KV ? key : KV - 1;
+            const half8_t * kr = (const half8_t *)(kb + (int64_t) kc * a.k_nb1);
 #pragma unroll
-                for (int c = 0; c < FA_D / 8; ++c) {
-                    const half8_t kk = kr[c];
+            for (int c = 0; c < FA_D / 8; ++c) kk[c] = kr[c];
+            mv = mp ? (float) mp[kc] : 0.0f;
+        };
+        load_key(kcur, mcur, tid);
+        for (int key = tid; key < kv_pad; key += 256) {
+            load_key(knext, mnext, key + 256);
+            float dot = 0.0f;
 #pragma unroll
-                    for (int e = 0; e < 8; ++e) dot += q[8*c + e] * (float) kk[e];
-                }
-                s = __fadd_rn(__fmul_rn(dot, a.scale), mv);
+            for (int c = 0; c < FA_D / 8; ++c) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) dot += q[8*c + e] * (float) kcur[c][e];
             }
+            vs_s[key] = key < KV && mcur != -INFINITY ? __fadd_rn(__fmul_rn(dot, a.scale), mcur) : -INFINITY;
+#pragma unroll
+            for (int c = 0; c < FA_D / 8; ++c) kcur[c] = knext[c];
+            mcur = mnext;
         }
-        vs_s[key] = s;
     }
     __syncthreads();
 
@@ -240,40 +250,55 @@ __global__ void __launch_bounds__(256) k_fattn_seq_row(fa_args a, int kv_pad) {
     // dependent instructions, so the common case is straight-line code of two per key: v_fma_mix_f32 (f16 V, f32
     // factor, f16 accumulator -> f32) and v_cvt_f16_f32 — the reference's f32 fma and its f16 store.  The factors are
     // read once per 64 keys, one per lane (vs, or -ms where the key raises the maximum: then vs is 1), and reach the
-    // chain as scalar operands through v_readlane.  V is staged by the whole workgroup: 256 keys (rows of 128 B) per
-    // step into one of two LDS buffers, the next step's rows in flight meanwhile, so the walker never waits on HBM.
-    half_t * v_lds = (half_t *)(sm + 2 * kv_pad);          // [2][ROW_STAGE][FA_D]
+    // chain as scalar operands through v_readlane.  V is staged by the other three wavefronts: 192 keys (rows of 128 B) per
+    // step into one of two LDS buffers, the next step's rows in flight meanwhile, so the walker never waits on HBM and
+    // spends no issue slots on the staging itself.
+    // V sits in LDS transposed, [d][key] (pitch ROW_VT: 16-byte reads of 16 lanes cover all banks once), so that the walker's
+    // lane reads eight keys of its d with one instruction: with one 2-byte read per key, the 64 reads of a chunk could not
+    // be kept in flight under the chunk before it (the wait counter only counts to 15) and took longer than the chain.
+    half_t * v_lds = (half_t *)(sm + 2 * kv_pad);          // [2][FA_D][ROW_VT]
     u32x4 vrow[8];
+    const int stid = tid - WAVE;                           // staging thread: wavefronts 1 .. 3
     auto load_rows = [&](int key0) __attribute__((always_inline)) {
-        const int key = key0 + tid;
+        const int key = key0 + stid;
         const u32x4 * src = (const u32x4 *)(vb + (int64_t)(key < KV ? key : KV - 1) * a.v_nb1);
 #pragma unroll
         for (int i = 0; i < 8; ++i) vrow[i] = key < KV ? src[i] : (u32x4){0, 0, 0, 0};
     };
     auto store_rows = [&](int buf) __attribute__((always_inline)) {
-        u32x4 * dst = (u32x4 *)(v_lds + ((size_t) buf * ROW_STAGE + tid) * FA_D);
+        uint16_t * dst = (uint16_t *)(v_lds + (size_t) buf * FA_D * ROW_VT) + stid;      // column `stid` of the stage
 #pragma unroll
-        for (int i = 0; i < 8; ++i) dst[i] = vrow[i];
+        for (int i = 0; i < 8; ++i) {
+#pragma unroll
+            for (int w = 0; w < 4; ++w) {
+                dst[(8 * i + 2 * w    ) * ROW_VT] = (uint16_t) vrow[i][w];
+                dst[(8 * i + 2 * w + 1) * ROW_VT] = (uint16_t)(vrow[i][w] >> 16);
+            }
+        }
     };
 
     uint32_t acc = 0;                                      // f16 accumulator in the low half
-    auto mad = [&](half_t v, uint32_t vs_bits) __attribute__((always_inline)) {
+    // one key: acc = f16(fma(v, vs, acc)); v is the low or the high half of `pair`
+    auto mad = [&](uint32_t pair, bool high, uint32_t vs_bits) __attribute__((always_inline)) {
         float t;
-        asm("v_fma_mix_f32 %0, %1, %2, %3 op_sel_hi:[1,0,1]" : "=v"(t) : "v"(v), "s"(vs_bits), "v"(acc));
+        if (high) asm("v_fma_mix_f32 %0, %1, %2, %3 op_sel:[1,0,0] op_sel_hi:[1,0,1]" : "=v"(t) : "v"(pair), "s"(vs_bits), "v"(acc));
+        else      asm("v_fma_mix_f32 %0, %1, %2, %3 op_sel_hi:[1,0,1]" : "=v"(t) : "v"(pair), "s"(vs_bits), "v"(acc));
         asm("v_cvt_f16_f32 %0, %1" : "=v"(acc) : "v"(t));
     };
-    auto read_chunk = [&](half_t * dst, const half_t * vbuf, int k0) __attribute__((always_inline)) {
+    struct chunk { u32x4 c[ROW_CHUNK / 8]; };              // 64 keys of this lane's d, two per register
+    auto read_chunk = [&](chunk & ch, const half_t * vbuf, int k0) __attribute__((always_inline)) {
+        const u32x4 * src = (const u32x4 *)(vbuf + lane * ROW_VT + k0);
 #pragma unroll
-        for (int j = 0; j < ROW_CHUNK; ++j) dst[j] = vbuf[(k0 + j) * FA_D + lane];
+        for (int i = 0; i < ROW_CHUNK / 8; ++i) ch.c[i] = src[i];
     };
-    auto run_chunk = [&](const half_t * v, int key0) __attribute__((always_inline)) {
-        const float vs_f = vs_s[key0 + lane], ms_f = ms_s[key0 + lane];
+    // (vs_f, ms_f): the factors of key key0 + lane, read while the chunk before was walked
+    auto run_chunk = [&](const chunk & ch, float vs_f, float ms_f) __attribute__((always_inline)) {
         const bool  raised_l = ms_f != 1.0f;
         const uint32_t f_l = __float_as_uint(raised_l ? -ms_f : vs_f);
         const uint64_t raised = __ballot(raised_l);        // uniform: which of the 64 keys move the maximum
         if (raised == 0) {
 #pragma unroll
-            for (int j = 0; j < ROW_CHUNK; ++j) mad(v[j], __builtin_amdgcn_readlane(f_l, j));   // masked keys: vs = 0 leaves acc as it is
+            for (int j = 0; j < ROW_CHUNK; ++j) mad(ch.c[j >> 3][(j >> 1) & 3], j & 1, __builtin_amdgcn_readlane(f_l, j));   // masked keys: vs = 0 leaves acc as it is
         } else {
 #pragma unroll
             for (int j = 0; j < ROW_CHUNK; ++j) {
@@ -284,29 +309,39 @@ __global__ void __launch_bounds__(256) k_fattn_seq_row(fa_args a, int kv_pad) {
                     asm("v_cvt_f16_f32 %0, %1" : "=v"(acc) : "v"(t));
                     f = 0x3f800000u;                       // vs = 1
                 }
-                mad(v[j], f);
+                mad(ch.c[j >> 3][(j >> 1) & 3], j & 1, f);
             }
         }
     };
 
-    load_rows(0);
+    if (wave != 0) load_rows(0);
+    float fv = vs_s[lane], fm = ms_s[lane];                // factors of the chunk walked next (kv_pad >= ROW_CHUNK)
     int buf = 0;
     for (int key0 = 0; key0 < kv_pad; key0 += ROW_STAGE, buf ^= 1) {
-        store_rows(buf);
+        if (wave != 0) store_rows(buf);
         __syncthreads();       // rows visible; the buffer written next time was last read before the previous barrier
-        if (key0 + ROW_STAGE < kv_pad) load_rows(key0 + ROW_STAGE);
-        if (wave == 0) {
-            const half_t * vbuf = v_lds + (size_t) buf * ROW_STAGE * FA_D;
+        if (wave != 0) {
+            if (key0 + ROW_STAGE < kv_pad) load_rows(key0 + ROW_STAGE);
+        } else {
+            const half_t * vbuf = v_lds + (size_t) buf * FA_D * ROW_VT;
             const int nk = min(ROW_STAGE, kv_pad - key0);                   // multiple of ROW_CHUNK
-            half_t va[ROW_CHUNK], vn[ROW_CHUNK];
+            chunk va, vn;
             read_chunk(va, vbuf, 0);
             for (int k0 = 0; k0 < nk; k0 += 2 * ROW_CHUNK) {
                 const bool more = k0 + ROW_CHUNK < nk;
                 if (more) read_chunk(vn, vbuf, k0 + ROW_CHUNK);
-                run_chunk(va, key0 + k0);
+                {
+                    const float cv = fv, cm = fm;
+                    const int nxt = key0 + k0 + ROW_CHUNK < kv_pad ? key0 + k0 + ROW_CHUNK : 0;
+                    fv = vs_s[nxt + lane]; fm = ms_s[nxt + lane];
+                    run_chunk(va, cv, cm);
+                }
                 if (more) {
                     if (k0 + 2 * ROW_CHUNK < nk) read_chunk(va, vbuf, k0 + 2 * ROW_CHUNK);
-                    run_chunk(vn, key0 + k0 + ROW_CHUNK);
+                    const float cv = fv, cm = fm;
+                    const int nxt = key0 + k0 + 2 * ROW_CHUNK < kv_pad ? key0 + k0 + 2 * ROW_CHUNK : 0;
+                    fv = vs_s[nxt + lane]; fm = ms_s[nxt + lane];
+                    run_chunk(vn, cv, cm);
                 }
             }
         }
@@ -941,12 +976,12 @@ extern "C" int mi355x_flash_attn_ext(const mi355x_tensor * q, const mi355x_tenso
         case FA_K_SEQ_ROW: {
             const int kv_pad = (int)((KV + ROW_CHUNK - 1) / ROW_CHUNK * ROW_CHUNK);
             dim3 grid((unsigned) N, (unsigned) H, (unsigned) q->ne[3]);
-            const size_t lds = (size_t) kv_pad * 8 + (size_t) 2 * ROW_STAGE * FA_D * sizeof(half_t);   // factors + two V stages
+            const size_t lds = (size_t) kv_pad * 8 + (size_t) 2 * ROW_VT * FA_D * sizeof(half_t);      // factors + two V stages
             static bool configured[64];                    // per device: more than the default 64 KB of dynamic LDS
             int dev = 0;
             if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return MI355X_ERR_HIP;
             if (!configured[dev]) {
-                if (hipFuncSetAttribute((const void *) k_fattn_seq_row, hipFuncAttributeMaxDynamicSharedMemorySize, SEQ_ROW_MAX_KV * 8 + 2 * ROW_STAGE * FA_D * 2) != hipSuccess) return MI355X_ERR_HIP;
+                if (hipFuncSetAttribute((const void *) k_fattn_seq_row, hipFuncAttributeMaxDynamicSharedMemorySize, SEQ_ROW_MAX_KV * 8 + 2 * ROW_VT * FA_D * 2) != hipSuccess) return MI355X_ERR_HIP;
                 configured[dev] = true;
             }
             k_fattn_seq_row<<<grid, 256, lds, st>>>(a, kv_pad);
