@@ -92,16 +92,31 @@ __device__ __forceinline__ uint16_t f2h_bits(float f) {
     return h;
 }
 
-__device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, WAVE);
-    return v;
+// Reductions over aligned groups of W = 4 .. 64 lanes, the result in every lane of the group: DPP steps inside the rows
+// of 16 lanes (a mirror pairs the lanes as well as an exchange does, for a commutative reduction), a swizzle across two
+// rows, a permute across the halves of the wavefront.  A DPP step costs one vector instruction; the ds_bpermute behind
+// __shfl_xor costs an LDS round trip, which is what kernels over a handful of rows spend their time waiting for.
+template <typename T, int CTRL>
+__device__ __forceinline__ T dpp_move(T v) {
+    static_assert(sizeof(T) == 4, "one 32-bit register");
+    return __builtin_bit_cast(T, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
 }
-__device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, WAVE));
-    return v;
+template <int W, typename T, typename OP>
+__device__ __forceinline__ T lanes_reduce(T x, OP op) {
+    static_assert(W == 4 || W == 8 || W == 16 || W == 32 || W == 64, "aligned power-of-two groups");
+    x = op(x, dpp_move<T, 0xB1>(x));                        // quad_perm [1,0,3,2]
+    x = op(x, dpp_move<T, 0x4E>(x));                        // quad_perm [2,3,0,1]
+    if (W >= 8)  x = op(x, dpp_move<T, 0x141>(x));          // row_half_mirror
+    if (W >= 16) x = op(x, dpp_move<T, 0x140>(x));          // row_mirror
+    if (W >= 32) x = op(x, __builtin_bit_cast(T, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, x), 0x401F)));   // lane ^ 16
+    if (W >= 64) x = op(x, __shfl_xor(x, 32, WAVE));
+    return x;
 }
+template <int W> __device__ __forceinline__ float lanes_sum(float x) { return lanes_reduce<W>(x, [](float a, float b) { return a + b; }); }
+template <int W> __device__ __forceinline__ int   lanes_sum(int x)   { return lanes_reduce<W>(x, [](int a, int b) { return a + b; }); }
+template <int W> __device__ __forceinline__ float lanes_max(float x) { return lanes_reduce<W>(x, [](float a, float b) { return fmaxf(a, b); }); }
+__device__ __forceinline__ float wave_sum(float v) { return lanes_sum<WAVE>(v); }
+__device__ __forceinline__ float wave_max(float v) { return lanes_max<WAVE>(v); }
 
 // GELU as ggml_vec_gelu_f32 evaluates it (ggml/src/ggml-cpu/vec.h:443-457): outside (-10, 10) the clamps, inside a
 // lookup in a 65536-entry table indexed by the f16 bits of x that holds f16(gelu(f32(f16 x))).  `table` is the device

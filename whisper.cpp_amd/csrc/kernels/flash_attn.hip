@@ -355,13 +355,11 @@ __global__ void __launch_bounds__(256) k_fattn_seq_row(fa_args a, int kv_pad) {
         // MI355X_FA_EMIT_Q8_0: the projection that follows reads its activations as Q8_0 (rows [N][H * 64]: int8 quants |
         // f32 scales | int32 block sums); this wavefront holds two blocks of one row, one per 32 lanes
         float amax = fabsf(o);
-#pragma unroll
-        for (int s = 1; s < 32; s <<= 1) amax = fmaxf(amax, __shfl_xor(amax, s, 32));
+        amax = lanes_max<32>(amax);
         const float id = amax != 0.0f ? 127.0f / amax : 0.0f;
         const int q = (int) rintf(o * id);
         int qsum = q;
-#pragma unroll
-        for (int s = 1; s < 32; s <<= 1) qsum += __shfl_xor(qsum, s, 32);
+        qsum = lanes_sum<32>(qsum);
         char * q8 = (char *) a.x16;
         const int64_t K = a.H * FA_D, nbk = K / 32, rows = a.N * a.ne3, rowi = i3 * a.N + n;
         ((int8_t *) q8)[rowi * K + h * FA_D + lane] = (int8_t) q;

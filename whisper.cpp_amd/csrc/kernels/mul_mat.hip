@@ -45,19 +45,6 @@ __device__ __forceinline__ float apply_epilogue(float v, const epi_args & e, int
 // The same for the 16 registers of one 32x32 accumulator patch (column m, rows n[0..15]) and the stores.  All loads of
 // one kind are issued together before their first use; rows beyond N and columns beyond M are computed from clamped
 // addresses and not stored.
-// maximum over the 32 lanes of a half-wavefront, in every lane: four DPP steps inside the rows of 16 (a mirror pairs the
-// lanes as well as an exchange does, for a maximum) and one swizzle across the two rows
-__device__ __forceinline__ float half_wave_max(float x) {
-    auto dpp = [](float v, auto ctrl) __attribute__((always_inline)) {
-        return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), decltype(ctrl)::value, 0xf, 0xf, true));
-    };
-    x = fmaxf(x, dpp(x, std::integral_constant<int, 0xB1>()));    // quad_perm [1,0,3,2]
-    x = fmaxf(x, dpp(x, std::integral_constant<int, 0x4E>()));    // quad_perm [2,3,0,1]
-    x = fmaxf(x, dpp(x, std::integral_constant<int, 0x141>()));   // row_half_mirror
-    x = fmaxf(x, dpp(x, std::integral_constant<int, 0x140>()));   // row_mirror
-    return fmaxf(x, __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, x), 0x401F)));   // lane ^ 16
-}
-
 template <bool EMIT>
 __device__ __forceinline__ void patch_epilogue(float16_t v, const epi_args & e, char * db, int64_t batch_off, int64_t d_nb1,
                                                int64_t m, int64_t M, const int64_t (&n)[16], int64_t N) {
@@ -109,7 +96,7 @@ __device__ __forceinline__ void patch_epilogue(float16_t v, const epi_args & e, 
         // butterfly, and the image f16(q * d) is written here instead of by a pass of its own over dst.
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
-            const float amax = half_wave_max(fabsf(v[i]));
+            const float amax = lanes_max<32>(fabsf(v[i]));
             const float id = amax != 0.0f ? 127.0f / amax : 0.0f;
             const float dq = h2f(f2h_bits(amax / 127.0f));
             if (m_ok && n[i] < N) e.image[n[i] * M + m] = (half_t)((rintf(v[i] * id) + 0.0f) * dq);
@@ -239,9 +226,7 @@ __global__ void k_x_to_f16(const char * __restrict__ x, half_t * __restrict__ ou
     half4_t h;
     if (Q8) {
         float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
-        amax = fmaxf(amax, __shfl_xor(amax, 1, 8));
-        amax = fmaxf(amax, __shfl_xor(amax, 2, 8));
-        amax = fmaxf(amax, __shfl_xor(amax, 4, 8));
+        amax = lanes_max<8>(amax);
         const float id = amax != 0.0f ? 127.0f / amax : 0.0f;
         const float d  = h2f(f2h_bits(amax / 127.0f));                      // the scale goes through f16, like block_q8_0.d
         // (+ 0.0f: a quant that rounds to -0 is the integer 0, whose product with d is +0)
@@ -555,16 +540,12 @@ __device__ __forceinline__ void quantize_x_to_lds(const mm_args & a, int32_t * x
             for (int u = 0; u < 8; ++u) {
                 const int idx = base + u * 256 + (int) threadIdx.x;      // lanes 8i .. 8i+7 share a block
                 float amax = fmaxf(fmaxf(fabsf(v[u].x), fabsf(v[u].y)), fmaxf(fabsf(v[u].z), fabsf(v[u].w)));
-                amax = fmaxf(amax, __shfl_xor(amax, 1, 8));
-                amax = fmaxf(amax, __shfl_xor(amax, 2, 8));
-                amax = fmaxf(amax, __shfl_xor(amax, 4, 8));
+                amax = lanes_max<8>(amax);
                 const float d  = amax / 127.0f;
                 const float id = amax != 0.0f ? 127.0f / amax : 0.0f;
                 const int q0 = (int) rintf(v[u].x * id), q1 = (int) rintf(v[u].y * id), q2 = (int) rintf(v[u].z * id), q3 = (int) rintf(v[u].w * id);
                 int sum = q0 + q1 + q2 + q3;
-                sum += __shfl_xor(sum, 1, 8);
-                sum += __shfl_xor(sum, 2, 8);
-                sum += __shfl_xor(sum, 4, 8);
+                sum = lanes_sum<8>(sum);
                 if (idx < total) {
                     const int n = idx / k8, c = idx % k8;       // c: float4 piece within the row
                     xq[(int64_t) n * (K / 4) + c] = (q0 & 0xFF) | ((q1 & 0xFF) << 8) | ((q2 & 0xFF) << 16) | ((q3 & 0xFF) << 24);
@@ -700,22 +681,6 @@ __global__ void __launch_bounds__(256) k_gemv_q(mm_args a) {
     }
 }
 
-// sum over the LPR lanes of a row, in every lane: DPP steps inside the rows of 16 (a mirror pairs the lanes as well as an
-// exchange does, for a sum), a swizzle across two rows, a permute across the halves of the wavefront
-template <int LPR>
-__device__ __forceinline__ float lanes_sum(float x) {
-    auto dpp = [](float v, auto ctrl) __attribute__((always_inline)) {
-        return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), decltype(ctrl)::value, 0xf, 0xf, true));
-    };
-    x += dpp(x, std::integral_constant<int, 0xB1>());                   // quad_perm [1,0,3,2]
-    x += dpp(x, std::integral_constant<int, 0x4E>());                   // quad_perm [2,3,0,1]
-    x += dpp(x, std::integral_constant<int, 0x141>());                  // row_half_mirror
-    if (LPR >= 16) x += dpp(x, std::integral_constant<int, 0x140>());   // row_mirror
-    if (LPR >= 32) x += __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, x), 0x401F));   // lane ^ 16
-    if (LPR >= 64) x += __shfl_xor(x, 32, WAVE);
-    return x;
-}
-
 // Activations quantized ahead of the product, once for every product that reads them:
 //   int8 xq[N][K] | float xd[N][K/32] (the f16-rounded block scales) | int32 xsum[N][K/32] (sum of a block's quants)
 // One thread per four values, eight lanes per block; rounding as quantize_row_q8_0 (ggml-cpu-quants.c:808-865).
@@ -726,16 +691,12 @@ __global__ void __launch_bounds__(256) k_quantize_x_q8(const char * __restrict__
     const int64_t n = idx / k4, c = idx % k4;
     const float4 v = *(const float4 *)(x + n * x_nb1 + c * 16);
     float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
-    amax = fmaxf(amax, __shfl_xor(amax, 1, 8));
-    amax = fmaxf(amax, __shfl_xor(amax, 2, 8));
-    amax = fmaxf(amax, __shfl_xor(amax, 4, 8));
+    amax = lanes_max<8>(amax);
     const float d  = amax / 127.0f;
     const float id = amax != 0.0f ? 127.0f / amax : 0.0f;
     const int q0 = (int) rintf(v.x * id), q1 = (int) rintf(v.y * id), q2 = (int) rintf(v.z * id), q3 = (int) rintf(v.w * id);
     int sum = q0 + q1 + q2 + q3;
-    sum += __shfl_xor(sum, 1, 8);
-    sum += __shfl_xor(sum, 2, 8);
-    sum += __shfl_xor(sum, 4, 8);
+    sum = lanes_sum<8>(sum);
     int32_t * xq   = (int32_t *) ws;
     float *   xd   = (float *)(ws + N * K);
     int32_t * xsum = (int32_t *)(ws + N * K + N * nbk * 4);

@@ -62,9 +62,7 @@ __global__ void __launch_bounds__(ROWS_PER_BLOCK * WAVE) k_norm(tview s, tview d
                 ((float4 *) y)[c] = r;
                 if (EMIT) {                                // a 32-value block = 8 consecutive lanes (ne0 % 32 == 0: they are all here)
                     float amax = fmaxf(fmaxf(fabsf(r.x), fabsf(r.y)), fmaxf(fabsf(r.z), fabsf(r.w)));
-                    amax = fmaxf(amax, __shfl_xor(amax, 1, 8));
-                    amax = fmaxf(amax, __shfl_xor(amax, 2, 8));
-                    amax = fmaxf(amax, __shfl_xor(amax, 4, 8));
+                    amax = lanes_max<8>(amax);
                     const float id = amax != 0.0f ? 127.0f / amax : 0.0f;
                     const float dq = h2f(f2h_bits(amax / 127.0f));
                     if (EMIT == 1) {
@@ -73,9 +71,7 @@ __global__ void __launch_bounds__(ROWS_PER_BLOCK * WAVE) k_norm(tview s, tview d
                     } else {
                         const int q0 = (int) rintf(r.x * id), q1 = (int) rintf(r.y * id), q2 = (int) rintf(r.z * id), q3 = (int) rintf(r.w * id);
                         int qsum = q0 + q1 + q2 + q3;
-                        qsum += __shfl_xor(qsum, 1, 8);
-                        qsum += __shfl_xor(qsum, 2, 8);
-                        qsum += __shfl_xor(qsum, 4, 8);
+                        qsum = lanes_sum<8>(qsum);
                         char * q8 = (char *) x16;
                         const int64_t nbk = ne0 / 32;
                         ((int32_t *) q8)[row * (ne0 / 4) + c] = (q0 & 0xFF) | ((q1 & 0xFF) << 8) | ((q2 & 0xFF) << 16) | ((q3 & 0xFF) << 24);
