@@ -434,8 +434,13 @@ __global__ void __launch_bounds__(256) k_fattn_seq_tile(fa_args a) {
     }
     if (tid < T_Q) { m_run[tid] = -INFINITY; s_run[tid] = 0.0f; }
 
-    // chain role: lane = query, this wavefront's d slice
-    const int d0 = wave * 16;
+    // chain role: a lane owns 16 of the 64 d of one query.  A wavefront takes 16 queries x all four d slices (lane = query
+    // 16 w + l % 16, slice l / 16): a key that raises the running maximum of any query of the wavefront costs the whole
+    // wavefront a rescale of its accumulators, and with 16 queries instead of 64 that happens for 6 % of the keys instead
+    // of 18 % (records of an i.i.d. sequence: about min(1, queries / k) at key k).  The packed variant keeps lane = query,
+    // wavefront = slice, because it hands V over as wavefront-uniform scalars.
+    const int cq = PACKED ? lane : 16 * wave + (lane & 15);
+    const int d0 = PACKED ? wave * 16 : (lane >> 4) * 16;
     half2_t acc2[8];                                       // 16 f16 accumulators, two per register
 #pragma unroll
     for (int e = 0; e < 8; ++e) acc2[e] = (half2_t){ (half_t) 0.0f, (half_t) 0.0f };
@@ -545,7 +550,7 @@ __global__ void __launch_bounds__(256) k_fattn_seq_tile(fa_args a) {
         // ---- the sequential f16 chains over this tile's keys -----------------------------------------------------------------------------
         if constexpr (PACKED) {
             const int nk = (int)(a.KV - key0 < T_KV ? a.KV - key0 : T_KV);       // uniform
-            const float4 * fp = (const float4 *)(f_s + lane * T_LDF);
+            const float4 * fp = (const float4 *)(f_s + cq * T_LDF);
             uint32_t vk[8];                                                       // V[key = lane][d0 .. d0 + 15]
             {
                 const u32x4 * vr = (const u32x4 *)(v_s + lane * FA_D + d0);
@@ -589,7 +594,7 @@ __global__ void __launch_bounds__(256) k_fattn_seq_tile(fa_args a) {
             }
         } else {
             const int nk = (int)(a.KV - key0 < T_KV ? a.KV - key0 : T_KV);       // uniform
-            const float4 * fp = (const float4 *)(f_s + lane * T_LDF);
+            const float4 * fp = (const float4 *)(f_s + cq * T_LDF);
             const half8_t * vp = (const half8_t *)(v_s + d0);                    // + key * FA_D halves = 8 of these
             // one group = four keys: their factors (one b128 read) and their V values (two broadcast b128 reads per key);
             // the next group is read while this one is consumed
@@ -655,10 +660,10 @@ __global__ void __launch_bounds__(256) k_fattn_seq_tile(fa_args a) {
         }
     }
 
-    const int64_t n = n0 + lane;
+    const int64_t n = n0 + cq;
     float o[16];
     {
-        const float inv = 1.0f / s_run[lane];
+        const float inv = 1.0f / s_run[cq];
 #pragma unroll
         for (int i = 0; i < 8; ++i) { o[2*i] = (float) acc2[i][0] * inv; o[2*i + 1] = (float) acc2[i][1] * inv; }
     }
@@ -674,10 +679,14 @@ __global__ void __launch_bounds__(256) k_fattn_seq_tile(fa_args a) {
         float amax = 0.0f;
 #pragma unroll
         for (int e = 0; e < 16; ++e) amax = fmaxf(amax, fabsf(o[e]));
-        __syncthreads();                                   // every chain is done with the factor tile
-        f_s[wave * T_Q + lane] = amax;
-        __syncthreads();
-        amax = fmaxf(amax, f_s[(wave ^ 1) * T_Q + lane]);
+        if constexpr (PACKED) {                            // the other half of the block is in the neighbouring wavefront
+            __syncthreads();                               // every chain is done with the factor tile
+            f_s[wave * T_Q + lane] = amax;
+            __syncthreads();
+            amax = fmaxf(amax, f_s[(wave ^ 1) * T_Q + lane]);
+        } else {                                           // ... in lane ^ 16
+            amax = fmaxf(amax, __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, amax), 0x401F)));
+        }
         if (n < a.N) {
             const float id = amax != 0.0f ? 127.0f / amax : 0.0f;
             const float dq = h2f(f2h_bits(amax / 127.0f));
