@@ -94,6 +94,18 @@ def test_whisper_full_end_to_end(harness, models):
     assert rc == 0 and s["pass"] and s["gpu_rc"] == 0 and s["gpu_tokens"] > 0 and s["gpu_segments"] > 0, s
 
 
+def test_whisper_full_with_dtw_token_timestamps(harness, models):
+    # cparams.dtw_token_timestamps (src/whisper.cpp:2731-2747, 2833-2838): the non-flash decoder graph also gathers the
+    # cross-attention probabilities of the top alignment heads — transposed copies, an f32 x f32 MUL_MAT with the head mask,
+    # CONCAT over layers — and whisper_full runs its DTW over them.  The transcript prefix and most of its DTW times must
+    # agree with the CPU backend's (the alignment of a random-init model follows near-flat attention, so not all of them).
+    rc, rows = run_harness(harness, ["full", "--model", models[("base", "q5_0")], "--beam", "1", "--max-tokens", "24", "--dtw"], timeout=900)
+    s = rows[-1]
+    assert rc == 0 and s["pass"] and s["dtw"] and s["gpu_rc"] == 0 and s["gpu_tokens"] > 0, s
+    assert s["common_prefix"] >= min(8, s["cpu_tokens"]), s
+    assert s["gpu_t_dtw_first"] >= 0 and 2 * s["dtw_identical_in_prefix"] >= s["common_prefix"], s
+
+
 def test_f32_matrix_core_attention_option(harness, models):
     # GGML_MI355X_FA_ACCUM=1: encoder / prompt attention with f32 accumulators on the matrix cores.  Every op case stays
     # within the per-op bound and the greedy ids of the base model do not move, but the reference's f16 accumulator

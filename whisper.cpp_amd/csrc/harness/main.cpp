@@ -347,10 +347,17 @@ static int cmd_gen(const args & a) {
 
 static bool g_flash_attn = true;   // --no-flash-attn: whisper.cpp's default graphs (KQ MUL_MAT, SOFT_MAX, KQV MUL_MAT; src/whisper.cpp:3620)
 
+static bool g_dtw = false;     // --dtw: token-level timestamps from the cross-attention of the top alignment heads (needs --no-flash-attn)
+
 static whisper_context * open_model(const std::string & path, bool use_gpu) {
     whisper_context_params cp = whisper_context_default_params();
     cp.use_gpu    = use_gpu;
     cp.flash_attn = g_flash_attn;
+    if (g_dtw) {
+        cp.dtw_token_timestamps = true;
+        cp.dtw_aheads_preset    = WHISPER_AHEADS_N_TOP_MOST;
+        cp.dtw_n_top            = 2;
+    }
     return whisper_init_from_file_with_params(path.c_str(), cp);
 }
 
@@ -435,7 +442,8 @@ static int cmd_model(const args & a) {
 // with its logits filters, timestamp rules and KV-cache bookkeeping.  Both backends see the same PCM; the token ids of
 // the two transcripts are compared from the front (a random-init model's near-flat logits let one rounding flip an
 // argmax, after which the two searches walk different histories, so only the common prefix is meaningful).
-static std::vector<whisper_token> run_full(whisper_context * ctx, const std::vector<float> & pcm, int beam, int max_tokens, int threads, int * rc, double * ms) {
+static std::vector<whisper_token> run_full(whisper_context * ctx, const std::vector<float> & pcm, int beam, int max_tokens, int threads, int * rc, double * ms,
+                                           std::vector<int64_t> * t_dtw = nullptr) {
     whisper_full_params p = whisper_full_default_params(beam > 1 ? WHISPER_SAMPLING_BEAM_SEARCH : WHISPER_SAMPLING_GREEDY);
     p.n_threads = threads;
     p.print_progress = false; p.print_realtime = false; p.print_timestamps = false; p.print_special = false;
@@ -451,7 +459,10 @@ static std::vector<whisper_token> run_full(whisper_context * ctx, const std::vec
     if (*rc != 0) return out;
     const int nseg = whisper_full_n_segments(ctx);
     for (int i = 0; i < nseg; ++i)
-        for (int j = 0; j < whisper_full_n_tokens(ctx, i); ++j) out.push_back(whisper_full_get_token_id(ctx, i, j));
+        for (int j = 0; j < whisper_full_n_tokens(ctx, i); ++j) {
+            out.push_back(whisper_full_get_token_id(ctx, i, j));
+            if (t_dtw) t_dtw->push_back(whisper_full_get_token_data(ctx, i, j).t_dtw);
+        }
     return out;
 }
 
@@ -474,18 +485,23 @@ static int cmd_full(const args & a) {
         pcm[i] = (float)(0.25 * sin(2 * M_PI * (220.0 + 30.0 * t) * t) + 0.15 * sin(2 * M_PI * 1310.0 * t) + 0.1 * noise);
     }
     int rg = 0, rc = 0; double ms_g = 0, ms_c = 0;
-    const std::vector<whisper_token> tg = run_full(gpu, pcm, beam, max_tokens, threads, &rg, &ms_g);
-    const std::vector<whisper_token> tc = run_full(cpu, pcm, beam, max_tokens, threads, &rc, &ms_c);
+    std::vector<int64_t> dg, dc;
+    const std::vector<whisper_token> tg = run_full(gpu, pcm, beam, max_tokens, threads, &rg, &ms_g, &dg);
+    const std::vector<whisper_token> tc = run_full(cpu, pcm, beam, max_tokens, threads, &rc, &ms_c, &dc);
     size_t same = 0;
     while (same < tg.size() && same < tc.size() && tg[same] == tc[same]) ++same;
+    // DTW timestamps of the common prefix (only meaningful with --dtw; -1 otherwise)
+    size_t dtw_same = 0;
+    for (size_t i = 0; i < same; ++i) dtw_same += dg[i] == dc[i];
     std::string sg, sc;
     for (size_t i = 0; i < tg.size() && i < 16; ++i) sg += (i ? "," : "") + std::to_string(tg[i]);
     for (size_t i = 0; i < tc.size() && i < 16; ++i) sc += (i ? "," : "") + std::to_string(tc[i]);
     const bool pass = rg == 0 && rc == 0 && !tg.empty();
     printf("{\"summary\": \"full\", \"model\": \"%s\", \"beam\": %d, \"seconds\": %d, \"gpu_rc\": %d, \"cpu_rc\": %d, \"gpu_segments\": %d, \"cpu_segments\": %d, "
-           "\"gpu_tokens\": %zu, \"cpu_tokens\": %zu, \"common_prefix\": %zu, \"gpu_first\": [%s], \"cpu_first\": [%s], \"gpu_ms\": %.1f, \"cpu_ms\": %.1f, \"pass\": %s}\n",
+           "\"gpu_tokens\": %zu, \"cpu_tokens\": %zu, \"common_prefix\": %zu, \"dtw\": %s, \"dtw_identical_in_prefix\": %zu, \"gpu_t_dtw_first\": %lld, "
+           "\"gpu_first\": [%s], \"cpu_first\": [%s], \"gpu_ms\": %.1f, \"cpu_ms\": %.1f, \"pass\": %s}\n",
            json_escape(path).c_str(), beam, seconds, rg, rc, rg == 0 ? whisper_full_n_segments(gpu) : -1, rc == 0 ? whisper_full_n_segments(cpu) : -1,
-           tg.size(), tc.size(), same, sg.c_str(), sc.c_str(), ms_g, ms_c, pass ? "true" : "false");
+           tg.size(), tc.size(), same, g_dtw ? "true" : "false", dtw_same, dg.empty() ? -1LL : (long long) dg[0], sg.c_str(), sc.c_str(), ms_g, ms_c, pass ? "true" : "false");
     whisper_free(gpu); whisper_free(cpu);
     return pass ? 0 : 1;
 }
@@ -686,6 +702,7 @@ int main(int argc, char ** argv) {
     const std::string cmd = argv[1];
     const args a = parse_args(argc, argv, 2);
     if (a.has("no-flash-attn")) g_flash_attn = false;
+    if (a.has("dtw")) { g_dtw = true; g_flash_attn = false; }        // whisper.cpp turns DTW off under flash attention
     if (cmd == "info")  return cmd_info(a);
     if (cmd == "gen")   return cmd_gen(a);
     if (cmd == "selftest") return cmd_selftest(a);
