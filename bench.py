@@ -135,17 +135,20 @@ def main() -> int:
     dec = run_harness(["bench", "--model", dec_model, "--what", "decoder", "--backend", "gpu", "--reps", "3", "--warmup", "2",
                        "--steps", "224", "--batch", "5", "--profile", "--threads", str(a.threads)])
     dk = {k["kernel"]: k for k in dec["kernels"]}
-    gemv = dk.get("mul_mat.gemv_q8_0.vocab")     # the logits product, 70.5 MB of Q8_0 blocks: the one GEMV that bandwidth bounds
+    # the logits product, 70.5 MB of Q8_0 blocks: the one GEMV that bandwidth bounds (launched together with the final LayerNorm)
+    gemv_name = "norm_mul_mat.gemv.vocab" if "norm_mul_mat.gemv.vocab" in dk else "mul_mat.gemv_q8_0.vocab"
+    gemv = dk.get(gemv_name)
     decode = {"model": "large-v3-turbo Q8_0", "steps": dec["steps"], "beams": dec["batch"], "ms_per_step": round(dec["ms_per_step"], 4),
               "steps_per_s": round(dec["steps_per_s"], 1), "beam_tokens_per_s": round(dec["batch_tokens_per_s"], 1)}
     if gemv:
-        decode["gemv_roofline"] = kernel_roofline("mul_mat.gemv_q8_0.vocab", gemv)
+        decode["gemv_roofline"] = kernel_roofline(gemv_name, gemv)
         decode["gemv_roofline"]["traffic"] = round(70.7e6 + 1.3e6)
-    if dk.get("mul_mat.gemv_q8_0"):
-        # the 32 products per step over 1.7 ... 7 MB matrices: over in the launch-to-store latency of a small kernel
-        decode["gemv_small_roofline"] = kernel_roofline("mul_mat.gemv_q8_0", dk["mul_mat.gemv_q8_0"])
+    for small in ("mul_mat.gemv_q8_0", "norm_mul_mat.gemv"):
+        if dk.get(small):
+            # the products over 1.7 ... 7 MB matrices: over in the launch-to-store latency of a small kernel
+            decode.setdefault("gemv_small_rooflines", []).append(kernel_roofline(small, dk[small]))
     decode["kernel_breakdown"] = {n: {"launches_per_step": k["calls"] / dec["steps"], "ms_per_step": round(k["ms"] / dec["steps"], 4)}
-                                  for n, k in sorted(dk.items(), key=lambda kv: -kv[1]["ms"])[:6]}
+                                  for n, k in sorted(dk.items(), key=lambda kv: -kv[1]["ms"])[:8]}
 
     # ---- CPU baseline: the reference's ggml CPU backend, same model file, same window ------------------------------------------
     cpu_baseline = None

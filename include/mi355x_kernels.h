@@ -140,6 +140,15 @@ typedef struct mi355x_mul_mat_item {
 } mi355x_mul_mat_item;
 MI355X_API int    mi355x_mul_mat_group(const mi355x_mul_mat_item * items, int count, const mi355x_tensor * src1, int flags,
                                        void * workspace, size_t workspace_size, void * stream);
+/* LayerNorm (mi355x_norm: eps, optional affine w / b) of the rows of `src`, written to `normed`, and in the same launch the
+ * few-column products of mi355x_mul_mat_group over `normed` (count 1 .. 8; one product is the common case).  For a decode
+ * step, where a LayerNorm of five rows costs a launch of its own and nothing else: every workgroup normalizes the rows
+ * for itself while its first weight blocks travel.  Also leaves the Q8_0 form of `normed` in `workspace`, as the products'
+ * quantization pass would.  src / normed: F32 [K, N] with N <= 8, K a multiple of 32 and at most 2048, 16-byte aligned
+ * rows; items as for the few-column form of mi355x_mul_mat_group; MI355X_ERR_UNSUPPORTED otherwise (then call
+ * mi355x_norm_emit_q8_0 and the products).  No counterpart in the reference, whose graphs hold these as separate nodes. */
+MI355X_API int    mi355x_norm_mul_mat_group(const mi355x_tensor * src, const mi355x_tensor * normed, float eps, const float * w, const float * b,
+                                            const mi355x_mul_mat_item * items, int count, void * workspace, size_t workspace_size, void * stream);
 
 /* FLASH_ATTN_EXT --------------------------------------------------------------------------------------
  * ggml_compute_forward_flash_attn_ext_f16 (ggml/src/ggml-cpu/ops.cpp:6638-6851), max_bias = 0 and

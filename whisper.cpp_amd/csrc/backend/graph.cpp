@@ -325,8 +325,37 @@ struct graph_runner {
                ((c.epi.flags & MI355X_EPI_RESIDUAL) ? nbytes_of(c.mm) : 0.0);
     }
 
+    // A LayerNorm of a decode step (a handful of rows) whose result only feeds few-column products is not launched when
+    // it is met: it is held here and goes out inside the launch of those products (mi355x_norm_mul_mat_group).  If the
+    // next node to execute turns out to be something else, or the fused form does not take the shapes, it runs on its own
+    // after all (flush_norm).
+    struct held_norm {
+        bool active = false;
+        const ggml_tensor * src = nullptr, * out = nullptr, * key = nullptr;
+        float eps = 0.0f; const float * w = nullptr, * b = nullptr;
+        bool affine = false;
+    } held;
+
+    int flush_norm() {
+        if (!held.active) return MI355X_OK;
+        held.active = false;
+        mi355x_tensor vs = to_view(held.src), vd = to_view(held.out);
+        const size_t image_bytes = (size_t)(held.out->ne[0] * held.out->ne[1] + held.out->ne[0] / 32 * held.out->ne[1] * 8);
+        bool emit = ctx->reserve_workspace(image_bytes + 256);
+        int status;
+        {
+            launch_scope ls(ctx, held.affine ? (emit ? "norm_affine_emit" : "norm_affine") : "norm", nbytes_of(held.src) + nbytes_of(held.out) + (emit ? image_bytes : 0), 0.0);
+            status = emit ? mi355x_norm_emit_q8_0(&vs, &vd, held.eps, held.w, held.b, ctx->ws, ctx->stream) : mi355x_norm(&vs, &vd, held.eps, held.w, held.b, ctx->stream);
+        }
+        if (emit && status == MI355X_ERR_UNSUPPORTED) { emit = false; status = mi355x_norm(&vs, &vd, held.eps, held.w, held.b, ctx->stream); }
+        note_write(held.out);
+        if (emit && status == MI355X_OK) workspace_holds(held.key, ctx->ws_slot, 2);
+        return status;
+    }
+
     // Products that follow each other over the same activations with weights of one shape (Q, K, V of a layer; the
     // cross-attention K / V of all decoder layers) go out as one launch.  Returns the nodes consumed, 0 if no group formed.
+    // With a held LayerNorm over these activations the launch includes it, and one product is group enough.
     int run_mul_mat_group(int i, const mm_chain & first, const mm_operands & o0, int & status) {
         // (the few-column form: a decode step's Q, K and V over quantized weights, up to 8 products)
         const bool gemv = strncmp(o0.kernel_name, "mul_mat.gemv", 12) == 0;
@@ -358,17 +387,34 @@ struct graph_runner {
             chains.push_back(c); ops.push_back(o);
             end = j + c.used;
         }
-        if (chains.size() < 2) return 0;
+        const bool with_norm = held.active && gemv && held.key == first.x;
+        if (chains.size() < 2 && !with_norm) return 0;
 
         const size_t need = mi355x_mul_mat_workspace_size(&o0.vw, &o0.vx);
-        const int ready = prepare_src1(first, o0, need, status);
-        if (ready < 0) return end - i;
         std::vector<mi355x_mul_mat_item> items(chains.size());
         double flops = 0.0, bytes = 0.0;
         for (size_t k = 0; k < chains.size(); ++k) {
             items[k] = { &ops[k].vw, &ops[k].vd, &chains[k].epi };
             flops += chain_flops(chains[k]); bytes += chain_bytes(chains[k]) - (k ? nbytes_of(first.x) : 0.0);
         }
+        if (with_norm) {
+            if (!ctx->reserve_workspace(need)) { status = MI355X_ERR_WORKSPACE; return end - i; }
+            mi355x_tensor vs = to_view(held.src), vn = to_view(held.out);
+            int rc;
+            {
+                launch_scope ls(ctx, nbytes_of(first.w) >= 32e6 ? "norm_mul_mat.gemv.vocab" : "norm_mul_mat.gemv", bytes + nbytes_of(held.src) + nbytes_of(held.out), flops);
+                rc = mi355x_norm_mul_mat_group(&vs, &vn, held.eps, held.w, held.b, items.data(), (int) items.size(), ctx->ws, ctx->ws_size, ctx->stream);
+            }
+            if (rc == MI355X_ERR_UNSUPPORTED) return 0;      // the caller lets the LayerNorm run on its own and takes the usual path
+            held.active = false;
+            status = rc;
+            note_write(held.out);
+            if (rc == MI355X_OK) workspace_holds(held.key, ctx->ws_slot, 2);
+            for (const mm_chain & c : chains) note_write(c.out);
+            return end - i;
+        }
+        const int ready = prepare_src1(first, o0, need, status);
+        if (ready < 0) return end - i;
         int rc;
         {
             launch_scope ls(ctx, gemv ? "mul_mat.gemv_group" : "mul_mat.gemm_group", bytes, flops);
@@ -386,6 +432,7 @@ struct graph_runner {
         const mm_chain c = plan_chain(i);
         mm_operands o = describe(c);
         if (const int grouped = run_mul_mat_group(i, c, o, status)) return grouped;
+        if (held.active && (status = flush_norm()) != MI355X_OK) return c.used;
 
         mi355x_epilogue epi = c.epi;
         epi.flags |= o.mm_flags;
@@ -492,6 +539,10 @@ struct graph_runner {
         const ggml_tensor * key = out->ne[0] <= 2048 ? image_consumer(out, i + used) : nullptr;
         int mode = 1;
         if (!key && out->ne[0] <= 2048 && (key = image_consumer(out, i + used, true))) mode = 2;
+        if (mode == 2 && nm->src[0]->ne[2] == 1 && nm->src[0]->ne[3] == 1 && next_is_product_over(key, i + used)) {
+            held.active = true; held.src = nm->src[0]; held.out = out; held.key = key; held.eps = eps; held.w = w; held.b = b; held.affine = used == 3;
+            return used;
+        }
         const size_t image_bytes = mode == 1 ? (size_t)(out->ne[0] * out->ne[1] * 2) : (size_t)(out->ne[0] * out->ne[1] + out->ne[0] / 32 * out->ne[1] * 8);
         bool emit = key && ctx->reserve_workspace(image_bytes + 256);
         {
@@ -505,6 +556,14 @@ struct graph_runner {
         return used;
     }
 
+    // the next node that executes (views and empty nodes skipped) is a MUL_MAT with `key` as src1
+    bool next_is_product_over(const ggml_tensor * key, int from) const {
+        int j = from;
+        while (node_at(j) && (is_view_op(node_at(j)->op) || ggml_is_empty(node_at(j)))) ++j;
+        const ggml_tensor * n = node_at(j);
+        return n && n->op == GGML_OP_MUL_MAT && n->src[1] == key;
+    }
+
     // the workspace copy of the activations goes stale when something overwrites them
     const ggml_tensor * cached_x = nullptr;
     void note_write(const ggml_tensor * out) {
@@ -516,6 +575,7 @@ struct graph_runner {
         status = MI355X_OK;
         if (ggml_is_empty(n) || is_view_op(n->op)) return 1;
         const ggml_tensor * s0 = n->src[0], * s1 = n->src[1];
+        if (held.active && !(n->op == GGML_OP_MUL_MAT && s1 == held.key) && (status = flush_norm()) != MI355X_OK) return 1;
         if (n->op != GGML_OP_MUL_MAT && n->op != GGML_OP_NORM) note_write(n->op == GGML_OP_CPY ? s1 : n);
         switch (n->op) {
             case GGML_OP_MUL_MAT: return run_mul_mat(i, status);
@@ -624,6 +684,10 @@ enum ggml_status mi355x_graph_compute(mi355x_backend_ctx * ctx, struct ggml_cgra
             return GGML_STATUS_FAILED;
         }
         i += used;
+    }
+    if (const int status = run.flush_norm()) {               // a LayerNorm at the very end of a graph
+        GGML_LOG_ERROR("ggml-mi355x: trailing NORM failed: %s\n", mi355x_status_string(status));
+        return GGML_STATUS_FAILED;
     }
     return GGML_STATUS_SUCCESS;
 }

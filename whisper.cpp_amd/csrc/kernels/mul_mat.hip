@@ -712,13 +712,14 @@ __global__ void __launch_bounds__(256) k_quantize_x_q8(const char * __restrict__
 // registers while the workgroup walks its row groups: the loop is weight loads and integer dot products only.  With
 // the activations in LDS, their reads (NC x 32 bytes per 34-byte block) are what bounds the kernel, and quantizing them
 // in every workgroup costs more than the product itself once K is large.
-template <int T0, int NC, int LPR, int NB>
-__device__ __forceinline__ void gemv_qr_rows(const mm_args & a) {
+struct gemv_no_prologue { __device__ __forceinline__ const char * operator()(const char * x) const { return x; } };
+
+// `prologue` runs once the first weight blocks are requested and returns where the quantized activations are: for the
+// plain product the workspace as passed; for the fused LayerNorm it first produces them in LDS.
+template <int T0, int NC, int LPR, int NB, typename PRO = gemv_no_prologue>
+__device__ __forceinline__ void gemv_qr_rows(const mm_args & a, PRO prologue = PRO()) {
     const int64_t K = a.K;
     const int nbk = (int)(K / QK);
-    const int32_t * xq   = (const int32_t *) a.x;
-    const float *   xd   = (const float *)(a.x + (size_t) NC * K);
-    const int32_t * xsum = (const int32_t *)(a.x + (size_t) NC * K + (size_t) NC * nbk * 4);
 
     constexpr int RPW = WAVE / LPR;                 // rows per wavefront
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -743,6 +744,10 @@ __device__ __forceinline__ void gemv_qr_rows(const mm_args & a) {
     };
     load_blocks();
 
+    const char * xbase = prologue(a.x);
+    const int32_t * xq   = (const int32_t *) xbase;
+    const float *   xd   = (const float *)(xbase + (size_t) NC * K);
+    const int32_t * xsum = (const int32_t *)(xbase + (size_t) NC * K + (size_t) NC * nbk * 4);
     int32_t xr[NC][NB][8];
     float   xs[NC][NB];          // scale of the block
     int32_t xo[NC][NB];          // 16 x sum of its quants (Q5_0 weights are stored with an offset of 16)
@@ -859,6 +864,85 @@ __global__ void __launch_bounds__(256) k_gemv_qr_group(mm_args a, gemv_group grp
     gemv_qr_rows<T0, NC, LPR, NB>(a);
 }
 
+// LayerNorm in front of the products, in the same launch.  A decode step's LayerNorm has five rows to work on and is
+// over in the latency of a launch (7 us); here every workgroup normalizes the rows for itself while its first weight
+// blocks travel — wavefront w takes rows w and w + 4, the row in registers between the passes as in k_norm — and leaves
+// them quantized in LDS, where the lanes pick up their slices.  The first workgroup also writes what a separate
+// LayerNorm would have left behind: the f32 rows and the Q8_0 form in the workspace, for whatever reads them later.
+struct gemv_norm_args {
+    const char * src; int64_t src_nb1;
+    const float * w; const float * b; float eps;
+    char * dst; int64_t dst_nb1;       // f32 rows of the normalized activations
+    char * ws;                         // their Q8_0 form (layout of k_quantize_x_q8)
+};
+
+template <int NC>
+struct gemv_norm_prologue {
+    const gemv_norm_args & nm; int64_t K; char * lds;
+    __device__ __forceinline__ const char * operator()(const char *) const {
+        const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+        const int n4 = (int)(K / 4), nbk = (int)(K / QK);
+        const bool writer = blockIdx.x == 0 && blockIdx.y == 0;
+        int32_t * xq   = (int32_t *) lds;
+        float *   xd   = (float *)(lds + (size_t) NC * K);
+        int32_t * xsum = (int32_t *)(lds + (size_t) NC * K + (size_t) NC * nbk * 4);
+        for (int row = wave; row < NC; row += 4) {
+            const float4 * x = (const float4 *)(nm.src + row * nm.src_nb1);
+            float4 v[8], ww[8], bb[8];
+#pragma unroll
+            for (int jj = 0; jj < 8; ++jj) {
+                const int c = lane + jj * WAVE;
+                v[jj] = make_float4(0.f, 0.f, 0.f, 0.f); ww[jj] = make_float4(1.f, 1.f, 1.f, 1.f); bb[jj] = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (c < n4) { v[jj] = x[c]; if (nm.w) ww[jj] = ((const float4 *) nm.w)[c]; if (nm.b) bb[jj] = ((const float4 *) nm.b)[c]; }
+            }
+            float sum = 0.0f;
+#pragma unroll
+            for (int jj = 0; jj < 8; ++jj) if (lane + jj * WAVE < n4) sum += (v[jj].x + v[jj].y) + (v[jj].z + v[jj].w);
+            const float mean = wave_sum(sum) / (float) K;
+            float sum2 = 0.0f;
+#pragma unroll
+            for (int jj = 0; jj < 8; ++jj) {
+                if (lane + jj * WAVE < n4) {
+                    v[jj].x -= mean; v[jj].y -= mean; v[jj].z -= mean; v[jj].w -= mean;
+                    sum2 += (v[jj].x*v[jj].x + v[jj].y*v[jj].y) + (v[jj].z*v[jj].z + v[jj].w*v[jj].w);
+                }
+            }
+            const float scale = 1.0f / sqrtf(wave_sum(sum2) / (float) K + nm.eps);
+#pragma unroll
+            for (int jj = 0; jj < 8; ++jj) {
+                const int c = lane + jj * WAVE;
+                if (c < n4) {                               // whole 8-lane groups: K is a multiple of 32
+                    float4 r = { v[jj].x * scale, v[jj].y * scale, v[jj].z * scale, v[jj].w * scale };
+                    if (nm.w) { r.x *= ww[jj].x; r.y *= ww[jj].y; r.z *= ww[jj].z; r.w *= ww[jj].w; }
+                    if (nm.b) { r.x += bb[jj].x; r.y += bb[jj].y; r.z += bb[jj].z; r.w += bb[jj].w; }
+                    if (writer) ((float4 *)(nm.dst + row * nm.dst_nb1))[c] = r;
+                    const float amax = lanes_max<8>(fmaxf(fmaxf(fabsf(r.x), fabsf(r.y)), fmaxf(fabsf(r.z), fabsf(r.w))));
+                    const float id = amax != 0.0f ? 127.0f / amax : 0.0f;
+                    const int q0 = (int) rintf(r.x * id), q1 = (int) rintf(r.y * id), q2 = (int) rintf(r.z * id), q3 = (int) rintf(r.w * id);
+                    const int qsum = lanes_sum<8>(q0 + q1 + q2 + q3);
+                    xq[row * n4 + c] = (q0 & 0xFF) | ((q1 & 0xFF) << 8) | ((q2 & 0xFF) << 16) | ((q3 & 0xFF) << 24);
+                    if ((c & 7) == 0) { xd[row * nbk + c / 8] = h2f(f2h_bits(amax / 127.0f)); xsum[row * nbk + c / 8] = qsum; }
+                }
+            }
+        }
+        __syncthreads();
+        if (writer) {                                       // the workspace copy, 16 bytes per thread and step
+            const int pieces = (int)(((size_t) NC * K + (size_t) NC * nbk * 8) / 16);
+            for (int i = threadIdx.x; i < pieces; i += 256) ((u32x4 *) nm.ws)[i] = ((const u32x4 *) lds)[i];
+        }
+        return lds;
+    }
+};
+
+template <int T0, int NC, int LPR, int NB>
+__global__ void __launch_bounds__(256) k_gemv_qr_norm_group(mm_args a, gemv_group grp, gemv_norm_args nm) {
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    const gemv_group_entry & ge = grp.e[blockIdx.y];
+    a.w = ge.w; a.d = ge.d; a.d_nb1 = ge.d_nb1;
+    a.e.flags = ge.flags; a.e.scale = ge.scale; a.e.bias = ge.bias; a.e.residual = ge.residual;
+    gemv_qr_rows<T0, NC, LPR, NB>(a, gemv_norm_prologue<NC>{ nm, a.K, smem });
+}
+
 // ------------------------------------------------------------------------------------------------------
 // generic fallback: one wavefront per (m, group of up to 8 columns, batch); element-wise dequant, f32 FMA
 // ------------------------------------------------------------------------------------------------------
@@ -947,22 +1031,26 @@ static size_t gemv_ws_bytes(const mi355x_tensor * src0, const mi355x_tensor * sr
 }
 
 template <int T0, int NC, int LPR, int NB>
-static int launch_gemv_r_k(const mm_args & a, unsigned grid, const gemv_group * grp, int count, hipStream_t st) {
-    if (grp) k_gemv_qr_group<T0, NC, LPR, NB><<<dim3(grid, (unsigned) count), 256, 0, st>>>(a, *grp);
-    else     k_gemv_qr<T0, NC, LPR, NB><<<grid, 256, 0, st>>>(a);
+static int launch_gemv_r_k(const mm_args & a, unsigned grid, const gemv_group * grp, int count, const gemv_norm_args * nm, hipStream_t st) {
+    if (nm) {
+        const size_t lds = (size_t) NC * a.K + (size_t) NC * (a.K / QK) * 8;
+        k_gemv_qr_norm_group<T0, NC, LPR, NB><<<dim3(grid, (unsigned) count), 256, lds, st>>>(a, *grp, *nm);
+    }
+    else if (grp) k_gemv_qr_group<T0, NC, LPR, NB><<<dim3(grid, (unsigned) count), 256, 0, st>>>(a, *grp);
+    else          k_gemv_qr<T0, NC, LPR, NB><<<grid, 256, 0, st>>>(a);
     return launch_status();
 }
 template <int T0, int NC, int LPR>
-static int launch_gemv_r_nb(const mm_args & a, int nb, unsigned grid, const gemv_group * grp, int count, hipStream_t st) {
+static int launch_gemv_r_nb(const mm_args & a, int nb, unsigned grid, const gemv_group * grp, int count, const gemv_norm_args * nm, hipStream_t st) {
     switch (nb) {
-        case 1: return launch_gemv_r_k<T0, NC, LPR, 1>(a, grid, grp, count, st);
-        case 2: if constexpr (NC * 2 <= 15) return launch_gemv_r_k<T0, NC, LPR, 2>(a, grid, grp, count, st); break;
-        case 3: if constexpr (NC * 3 <= 15) return launch_gemv_r_k<T0, NC, LPR, 3>(a, grid, grp, count, st); break;
+        case 1: return launch_gemv_r_k<T0, NC, LPR, 1>(a, grid, grp, count, nm, st);
+        case 2: if constexpr (NC * 2 <= 15) return launch_gemv_r_k<T0, NC, LPR, 2>(a, grid, grp, count, nm, st); break;
+        case 3: if constexpr (NC * 3 <= 15) return launch_gemv_r_k<T0, NC, LPR, 3>(a, grid, grp, count, nm, st); break;
     }
     return MI355X_ERR_UNSUPPORTED;
 }
 template <int T0, int NC>
-static int launch_gemv_r(const mm_args & a, hipStream_t st, const gemv_group * grp = nullptr, int count = 1) {
+static int launch_gemv_r(const mm_args & a, hipStream_t st, const gemv_group * grp = nullptr, int count = 1, const gemv_norm_args * nm = nullptr) {
     const int lpr = gemv_r_lanes(a.M * count, NC, a.K);
     if (!lpr) return MI355X_ERR_UNSUPPORTED;
     const int nb = (int)((a.K / QK + lpr - 1) / lpr);
@@ -970,26 +1058,27 @@ static int launch_gemv_r(const mm_args & a, hipStream_t st, const gemv_group * g
     const int64_t n_groups = (a.M + rows_per_wg - 1) / rows_per_wg;
     // one resident set of workgroups (the registers allow 4 per CU with one block per lane, else 2), each walking its
     // share of the row groups: a second, partly filled set would double the time
-    const int64_t resident = 256 * (nb == 1 ? 4 : 2) / count > 0 ? 256 * (nb == 1 ? 4 : 2) / count : 1;
+    const int per_cu = nb > 1 ? 2 : nm ? 3 : 4;           // (the LayerNorm prologue costs the one-block kernels 50 registers)
+    const int64_t resident = 256 * per_cu / count > 0 ? 256 * per_cu / count : 1;
     const int64_t rounds   = (n_groups + resident - 1) / resident;
     const unsigned grid    = (unsigned)((n_groups + rounds - 1) / rounds);
     switch (lpr) {
-        case 16: return launch_gemv_r_nb<T0, NC, 16>(a, nb, grid, grp, count, st);
-        case 32: return launch_gemv_r_nb<T0, NC, 32>(a, nb, grid, grp, count, st);
-        default: return launch_gemv_r_nb<T0, NC, 64>(a, nb, grid, grp, count, st);
+        case 16: return launch_gemv_r_nb<T0, NC, 16>(a, nb, grid, grp, count, nm, st);
+        case 32: return launch_gemv_r_nb<T0, NC, 32>(a, nb, grid, grp, count, nm, st);
+        default: return launch_gemv_r_nb<T0, NC, 64>(a, nb, grid, grp, count, nm, st);
     }
 }
 template <int T0>
-static int launch_gemv_r_n(const mm_args & a, hipStream_t st, const gemv_group * grp = nullptr, int count = 1) {
+static int launch_gemv_r_n(const mm_args & a, hipStream_t st, const gemv_group * grp = nullptr, int count = 1, const gemv_norm_args * nm = nullptr) {
     switch (a.N) {
-        case 1: return launch_gemv_r<T0, 1>(a, st, grp, count);
-        case 2: return launch_gemv_r<T0, 2>(a, st, grp, count);
-        case 3: return launch_gemv_r<T0, 3>(a, st, grp, count);
-        case 4: return launch_gemv_r<T0, 4>(a, st, grp, count);
-        case 5: return launch_gemv_r<T0, 5>(a, st, grp, count);
-        case 6: return launch_gemv_r<T0, 6>(a, st, grp, count);
-        case 7: return launch_gemv_r<T0, 7>(a, st, grp, count);
-        case 8: return launch_gemv_r<T0, 8>(a, st, grp, count);
+        case 1: return launch_gemv_r<T0, 1>(a, st, grp, count, nm);
+        case 2: return launch_gemv_r<T0, 2>(a, st, grp, count, nm);
+        case 3: return launch_gemv_r<T0, 3>(a, st, grp, count, nm);
+        case 4: return launch_gemv_r<T0, 4>(a, st, grp, count, nm);
+        case 5: return launch_gemv_r<T0, 5>(a, st, grp, count, nm);
+        case 6: return launch_gemv_r<T0, 6>(a, st, grp, count, nm);
+        case 7: return launch_gemv_r<T0, 7>(a, st, grp, count, nm);
+        case 8: return launch_gemv_r<T0, 8>(a, st, grp, count, nm);
     }
     return MI355X_ERR_INVALID;
 }
@@ -1083,7 +1172,7 @@ extern "C" size_t mi355x_mul_mat_workspace_size(const mi355x_tensor * src0, cons
 
 // the few-column form of mi355x_mul_mat_group: quantized weights of one type and shape, activations quantized once
 static int mul_mat_group_gemv(const mi355x_mul_mat_item * items, int count, const mi355x_tensor * src1, int flags,
-                              void * workspace, size_t workspace_size, void * stream) {
+                              void * workspace, size_t workspace_size, void * stream, gemv_norm_args * nm = nullptr) {
     const mi355x_tensor * w0 = items[0].src0;
     if (count > GEMV_GROUP_MAX || src1->type != MI355X_TYPE_F32 || mm_path(w0, src1) != MM_GEMV) return MI355X_ERR_UNSUPPORTED;
     if (w0->type != MI355X_TYPE_Q8_0 && w0->type != MI355X_TYPE_Q5_0) return MI355X_ERR_UNSUPPORTED;
@@ -1119,6 +1208,10 @@ static int mul_mat_group_gemv(const mi355x_mul_mat_item * items, int count, cons
     a.e.flags = 0; a.e.scale = 1.0f; a.e.bias = nullptr; a.e.residual = nullptr; a.e.gelu = nullptr; a.e.image = nullptr;
     if (any_gelu && !(a.e.gelu = gelu_table_device())) return MI355X_ERR_HIP;
     hipStream_t st = (hipStream_t) stream;
+    if (nm) {                                               // the LayerNorm in front, in the same launch: it writes src1 and the workspace
+        nm->ws = (char *) workspace;
+        return w0->type == MI355X_TYPE_Q8_0 ? launch_gemv_r_n<MI355X_TYPE_Q8_0>(a, st, &grp, count, nm) : launch_gemv_r_n<MI355X_TYPE_Q5_0>(a, st, &grp, count, nm);
+    }
     if (!(flags & MI355X_MM_WS_READY)) {
         k_quantize_x_q8<<<(unsigned)((a.N * (a.K / 4) + 255) / 256), 256, 0, st>>>(a.x, a.x_nb1, a.K, a.N, (char *) workspace);
         if (const int rc = launch_status()) return rc;
@@ -1126,6 +1219,20 @@ static int mul_mat_group_gemv(const mi355x_mul_mat_item * items, int count, cons
     if (flags & MI355X_MM_PREPARE_ONLY) return MI355X_OK;
     a.x = (const char *) workspace;
     return w0->type == MI355X_TYPE_Q8_0 ? launch_gemv_r_n<MI355X_TYPE_Q8_0>(a, st, &grp, count) : launch_gemv_r_n<MI355X_TYPE_Q5_0>(a, st, &grp, count);
+}
+
+extern "C" int mi355x_norm_mul_mat_group(const mi355x_tensor * src, const mi355x_tensor * normed, float eps, const float * w, const float * b,
+                                         const mi355x_mul_mat_item * items, int count, void * workspace, size_t workspace_size, void * stream) {
+    if (!src || !normed || !items || count < 1 || !(eps >= 0.0f)) return MI355X_ERR_INVALID;
+    if (!items[0].src0 || !items[0].dst) return MI355X_ERR_INVALID;
+    if (src->type != MI355X_TYPE_F32 || normed->type != MI355X_TYPE_F32 || src->nb[0] != 4 || normed->nb[0] != 4) return MI355X_ERR_UNSUPPORTED;
+    for (int i = 0; i < 4; ++i) if (src->ne[i] != normed->ne[i]) return MI355X_ERR_INVALID;
+    const int64_t K = src->ne[0], N = src->ne[1];
+    if (src->ne[2] != 1 || src->ne[3] != 1 || N < 1 || N > MI355X_GEMV_MAX_COLS || K % QK != 0 || K > 2048) return MI355X_ERR_UNSUPPORTED;
+    if (!aligned16(src) || !aligned16(normed) || (uintptr_t) w % 16 != 0 || (uintptr_t) b % 16 != 0) return MI355X_ERR_UNSUPPORTED;
+    if (blck_size(items[0].src0->type) <= 1) return MI355X_ERR_UNSUPPORTED;
+    gemv_norm_args nm = { (const char *) src->data, (int64_t) src->nb[1], w, b, eps, (char *) normed->data, (int64_t) normed->nb[1], nullptr };
+    return mul_mat_group_gemv(items, count, normed, 0, workspace, workspace_size, stream, &nm);
 }
 
 extern "C" int mi355x_mul_mat_group(const mi355x_mul_mat_item * items, int count, const mi355x_tensor * src1, int flags,
