@@ -866,8 +866,8 @@ __global__ void __launch_bounds__(256) k_gemv_qr_group(mm_args a, gemv_group grp
 
 // LayerNorm in front of the products, in the same launch.  A decode step's LayerNorm has five rows to work on and is
 // over in the latency of a launch (7 us); here every workgroup normalizes the rows for itself while its first weight
-// blocks travel — wavefront w takes rows w and w + 4, the row in registers between the passes as in k_norm — and leaves
-// them quantized in LDS, where the lanes pick up their slices.  The first workgroup also writes what a separate
+// blocks travel — the rows in registers between the passes as in k_norm — and leaves them quantized in LDS, where the
+// lanes pick up their slices.  The first workgroup also writes what a separate
 // LayerNorm would have left behind: the f32 rows and the Q8_0 form in the workspace, for whatever reads them later.
 struct gemv_norm_args {
     const char * src; int64_t src_nb1;
@@ -886,25 +886,37 @@ struct gemv_norm_prologue {
         int32_t * xq   = (int32_t *) lds;
         float *   xd   = (float *)(lds + (size_t) NC * K);
         int32_t * xsum = (int32_t *)(lds + (size_t) NC * K + (size_t) NC * nbk * 4);
-        for (int row = wave; row < NC; row += 4) {
-            const float4 * x = (const float4 *)(nm.src + row * nm.src_nb1);
-            float4 v[8], ww[8], bb[8];
+        // wavefront w takes rows w and w + 4; both rows and the affine vectors are requested before anything is reduced, so
+        // the prologue is one memory round trip long
+        constexpr int RW = (NC + 3) / 4;                    // rows per wavefront
+        float4 v[RW][8], ww[8], bb[8];
 #pragma unroll
-            for (int jj = 0; jj < 8; ++jj) {
-                const int c = lane + jj * WAVE;
-                v[jj] = make_float4(0.f, 0.f, 0.f, 0.f); ww[jj] = make_float4(1.f, 1.f, 1.f, 1.f); bb[jj] = make_float4(0.f, 0.f, 0.f, 0.f);
-                if (c < n4) { v[jj] = x[c]; if (nm.w) ww[jj] = ((const float4 *) nm.w)[c]; if (nm.b) bb[jj] = ((const float4 *) nm.b)[c]; }
+        for (int jj = 0; jj < 8; ++jj) {
+            const int c = lane + jj * WAVE;
+            ww[jj] = make_float4(1.f, 1.f, 1.f, 1.f); bb[jj] = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (c < n4) { if (nm.w) ww[jj] = ((const float4 *) nm.w)[c]; if (nm.b) bb[jj] = ((const float4 *) nm.b)[c]; }
+#pragma unroll
+            for (int rr = 0; rr < RW; ++rr) {
+                const int row = wave + 4 * rr;
+                v[rr][jj] = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (c < n4 && row < NC) v[rr][jj] = ((const float4 *)(nm.src + row * nm.src_nb1))[c];
             }
+        }
+#pragma unroll
+        for (int rr = 0; rr < RW; ++rr) {
+            const int row = wave + 4 * rr;
+            if (row >= NC) break;                           // uniform
             float sum = 0.0f;
 #pragma unroll
-            for (int jj = 0; jj < 8; ++jj) if (lane + jj * WAVE < n4) sum += (v[jj].x + v[jj].y) + (v[jj].z + v[jj].w);
+            for (int jj = 0; jj < 8; ++jj) if (lane + jj * WAVE < n4) sum += (v[rr][jj].x + v[rr][jj].y) + (v[rr][jj].z + v[rr][jj].w);
             const float mean = wave_sum(sum) / (float) K;
             float sum2 = 0.0f;
 #pragma unroll
             for (int jj = 0; jj < 8; ++jj) {
                 if (lane + jj * WAVE < n4) {
-                    v[jj].x -= mean; v[jj].y -= mean; v[jj].z -= mean; v[jj].w -= mean;
-                    sum2 += (v[jj].x*v[jj].x + v[jj].y*v[jj].y) + (v[jj].z*v[jj].z + v[jj].w*v[jj].w);
+                    float4 & t = v[rr][jj];
+                    t.x -= mean; t.y -= mean; t.z -= mean; t.w -= mean;
+                    sum2 += (t.x*t.x + t.y*t.y) + (t.z*t.z + t.w*t.w);
                 }
             }
             const float scale = 1.0f / sqrtf(wave_sum(sum2) / (float) K + nm.eps);
@@ -912,7 +924,7 @@ struct gemv_norm_prologue {
             for (int jj = 0; jj < 8; ++jj) {
                 const int c = lane + jj * WAVE;
                 if (c < n4) {                               // whole 8-lane groups: K is a multiple of 32
-                    float4 r = { v[jj].x * scale, v[jj].y * scale, v[jj].z * scale, v[jj].w * scale };
+                    float4 r = { v[rr][jj].x * scale, v[rr][jj].y * scale, v[rr][jj].z * scale, v[rr][jj].w * scale };
                     if (nm.w) { r.x *= ww[jj].x; r.y *= ww[jj].y; r.z *= ww[jj].z; r.w *= ww[jj].w; }
                     if (nm.b) { r.x += bb[jj].x; r.y += bb[jj].y; r.z += bb[jj].z; r.w += bb[jj].w; }
                     if (writer) ((float4 *)(nm.dst + row * nm.dst_nb1))[c] = r;
