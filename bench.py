@@ -61,7 +61,7 @@ def model_file(arch: str, ftype: str) -> str:
 # x2 KiB and x1 KiB), for the large-v3 encoder shapes; the summary with the commands is under profiles/
 # (mul_mat.gemm_q5_0 averages its two templates: 64 launches of 86.7 + 7.7 MB and 32 of 149.0 + 48.4 MB per window)
 MEASURED_TRAFFIC_MB = {"mul_mat.gemm_q5_0": (64 * (86.7 + 7.7) + 32 * (149.0 + 48.4)) / 96, "flash_attn.seq_tile": 70.9 + 11.5,
-                       "mul_mat.gemm_group": 144.3 + 23.1, "norm_affine_emit": 9.1 + 13.8}
+                       "mul_mat.gemm_group": 143.4 + 23.1, "norm_affine_emit": 7.9 + 11.5}
 
 # kernels that live on the matrix cores (bound "mfma"); everything else streams memory (bound "hbm")
 MFMA_KERNELS = ("mul_mat.gemm_", "flash_attn.seq_tile")
