@@ -508,8 +508,8 @@ __global__ void __launch_bounds__(256) k_fattn_seq_tile(fa_args a) {
             for (int i = 0; i < 16; ++i) lmax = fmaxf(lmax, sv[i]);
             float M = m_run[qi];
             const float S0 = s_run[qi];
-            const int base = lane & ~3;
-            const float m0 = __shfl(lmax, base + 0, WAVE), m1 = __shfl(lmax, base + 1, WAVE), m2 = __shfl(lmax, base + 2, WAVE);
+            // (the four runs of a query sit in one quad of lanes: broadcasts inside it are DPP moves, not LDS permutes)
+            const float m0 = dpp_move<float, 0x00>(lmax), m1 = dpp_move<float, 0x55>(lmax), m2 = dpp_move<float, 0xAA>(lmax);
             if (sgm > 0) M = fmaxf(M, m0);
             if (sgm > 1) M = fmaxf(M, m1);
             if (sgm > 2) M = fmaxf(M, m2);
@@ -535,10 +535,10 @@ __global__ void __launch_bounds__(256) k_fattn_seq_tile(fa_args a) {
 #pragma unroll
             for (int i = 0; i < 4; ++i) fp[i] = make_float4(sv[4*i], sv[4*i+1], sv[4*i+2], sv[4*i+3]);
             // fold the four runs of this query in key order
-            const float P1 = __shfl(P, base + 1, WAVE), A1 = __shfl(A, base + 1, WAVE);
-            const float P2 = __shfl(P, base + 2, WAVE), A2 = __shfl(A, base + 2, WAVE);
-            const float P3 = __shfl(P, base + 3, WAVE), A3 = __shfl(A, base + 3, WAVE);
-            const float M3 = __shfl(M, base + 3, WAVE);
+            const float P1 = dpp_move<float, 0x55>(P), A1 = dpp_move<float, 0x55>(A);
+            const float P2 = dpp_move<float, 0xAA>(P), A2 = dpp_move<float, 0xAA>(A);
+            const float P3 = dpp_move<float, 0xFF>(P), A3 = dpp_move<float, 0xFF>(A);
+            const float M3 = dpp_move<float, 0xFF>(M);
             if (sgm == 0) {
                 float S = S0 * P + A;
                 S = S * P1 + A1; S = S * P2 + A2; S = S * P3 + A3;
