@@ -94,6 +94,17 @@ def test_whisper_full_end_to_end(harness, models):
     assert rc == 0 and s["pass"] and s["gpu_rc"] == 0 and s["gpu_tokens"] > 0 and s["gpu_segments"] > 0, s
 
 
+def test_whisper_full_parallel_states_share_one_device(harness, models):
+    # whisper_full_parallel (src/whisper.cpp:6407-6470): three states, three backend instances and streams, three host
+    # threads on one GPU, all starting at once over shared weights — the f16 weight images are made on first use and must be
+    # complete before another instance can find them.  The merged transcript must start like the CPU backend's.
+    rc, rows = run_harness(harness, ["full", "--model", models[("base", "q5_0")], "--beam", "1", "--max-tokens", "16", "--seconds", "120",
+                                     "--processors", "3"], timeout=900)
+    s = rows[-1]
+    assert rc == 0 and s["pass"] and s["gpu_rc"] == 0 and s["gpu_tokens"] > 0, s
+    assert s["common_prefix"] >= min(16, s["cpu_tokens"]), s
+
+
 def test_whisper_full_with_dtw_token_timestamps(harness, models):
     # cparams.dtw_token_timestamps (src/whisper.cpp:2731-2747, 2833-2838): the non-flash decoder graph also gathers the
     # cross-attention probabilities of the top alignment heads — transposed copies, an f32 x f32 MUL_MAT with the head mask,

@@ -108,6 +108,9 @@ const void * mi355x_buffer_ctx::weight_image(const struct ggml_tensor * w, hipSt
         return nullptr;
     }
     if (mi355x_dequantize_row_f16((int) w->type, w->data, im.f16, n, stream) != MI355X_OK) { (void) hipFree(im.f16); return nullptr; }
+    // The image is shared by every backend instance that uses these weights (whisper_full_parallel: one instance and one
+    // stream per state), so it is complete before anyone can find it: once per weight matrix.
+    if (hipStreamSynchronize(stream) != hipSuccess) { (void) hipGetLastError(); (void) hipFree(im.f16); return nullptr; }
     images.emplace(key, im);
     return im.f16;
 }

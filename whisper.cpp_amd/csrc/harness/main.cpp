@@ -9,7 +9,7 @@
 //                                             per-op parity (NMSE / bit-exactness) and timing, CPU vs MI355X
 //   model  --model F [--steps 32] [--threads N]
 //                                             whole-model parity: logits NMSE and greedy ids, teacher-forced
-//   full   --model F [--beam 1|5] [--max-tokens 24] [--seconds 30] [--threads N]
+//   full   --model F [--beam 1|5] [--max-tokens 24] [--seconds 30] [--threads N] [--dtw] [--processors N]
 //                                             whisper_full() end to end (PCM -> mel -> encode -> search) on both backends
 //   verify --model F [--steps 3] [--threads N]
 //                                             per-node parity inside the real whisper graphs (unfused), CPU vs MI355X
@@ -347,6 +347,7 @@ static int cmd_gen(const args & a) {
 
 static bool g_flash_attn = true;   // --no-flash-attn: whisper.cpp's default graphs (KQ MUL_MAT, SOFT_MAX, KQV MUL_MAT; src/whisper.cpp:3620)
 
+static int  g_processors = 1;
 static bool g_dtw = false;     // --dtw: token-level timestamps from the cross-attention of the top alignment heads (needs --no-flash-attn)
 
 static whisper_context * open_model(const std::string & path, bool use_gpu) {
@@ -453,7 +454,8 @@ static std::vector<whisper_token> run_full(whisper_context * ctx, const std::vec
     p.suppress_blank = true;
     if (beam > 1) p.beam_search.beam_size = beam; else p.greedy.best_of = 1;
     const double t0 = now_ms();
-    *rc = whisper_full(ctx, p, pcm.data(), (int) pcm.size());
+    // --processors N: whisper_full_parallel splits the audio over N states, each with its own backend instance and host thread
+    *rc = g_processors > 1 ? whisper_full_parallel(ctx, p, pcm.data(), (int) pcm.size(), g_processors) : whisper_full(ctx, p, pcm.data(), (int) pcm.size());
     *ms = now_ms() - t0;
     std::vector<whisper_token> out;
     if (*rc != 0) return out;
@@ -702,6 +704,7 @@ int main(int argc, char ** argv) {
     const std::string cmd = argv[1];
     const args a = parse_args(argc, argv, 2);
     if (a.has("no-flash-attn")) g_flash_attn = false;
+    g_processors = a.num("processors", 1);
     if (a.has("dtw")) { g_dtw = true; g_flash_attn = false; }        // whisper.cpp turns DTW off under flash attention
     if (cmd == "info")  return cmd_info(a);
     if (cmd == "gen")   return cmd_gen(a);
