@@ -387,15 +387,17 @@ __global__ void __launch_bounds__(256) k_fattn_seq_row(fa_args a, int kv_pad) {
 #define T_LDH (FA_D + 8)      // f16 pitch of the Q and K tiles (144 B rows: conflict-free b128 reads for the MFMA operands)
 #define T_LDF (T_KV + 4)      // f32 pitch of the factor tile (272 B rows: conflict-free b128 reads with lane = row)
 
-// exp(x) for x <= 0 to about 1 ulp: 2^(x log2 e) with the rounding error of the product fed back in
+// exp(x) for x <= 0 to about 1 ulp: 2^(x log2 e) with the rounding error of the product fed back in.  Without a branch:
+// below the smallest denormal, at x = -inf (first key of a row) and for NaN (-inf - -inf: a masked key before any other)
+// the result is selected to 0 afterwards.
 __device__ __forceinline__ float exp_neg(float x) {
-    if (x < -104.0f) return 0.0f;                         // below the smallest denormal; also x = -inf (first key of a row)
     const float l2e_hi = 1.44269502e+0f, l2e_lo = 1.92596299e-8f;
     const float t = x * l2e_hi;
     float e = __builtin_fmaf(x, l2e_hi, -t);
     e = __builtin_fmaf(x, l2e_lo, e);
     const float r = __builtin_amdgcn_exp2f(t);
-    return __builtin_fmaf(r, e * 0.693147182f, r);
+    const float y = __builtin_fmaf(r, e * 0.693147182f, r);
+    return x >= -104.0f ? y : 0.0f;
 }
 
 typedef const uint32_t __attribute__((address_space(4))) * const_u32_ptr;   // read-only data: uniform loads become scalar loads
@@ -521,8 +523,7 @@ __global__ void __launch_bounds__(256) k_fattn_seq_tile(fa_args a) {
                 // one (vs = exp(s - M); masked keys, s = -inf, get vs = 0, a no-op on the accumulator)
                 const float s = sv[i];
                 const bool  raised = s > M;
-                const float x = raised ? M - s : s - M;    // <= 0; -inf - -inf (masked key before any other) is NaN ...
-                const float ex = s == -INFINITY ? 0.0f : exp_neg(x);                          // ... and never used
+                const float ex = exp_neg(-fabsf(s - M));   // M - s when raised, s - M otherwise: both <= 0 (or NaN / -inf: 0)
                 const float ms = raised ? ex : 1.0f, vs = raised ? 1.0f : ex;
                 M = raised ? s : M;
                 P *= ms; A = A * ms + vs;
