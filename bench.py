@@ -121,7 +121,8 @@ def main() -> int:
     if roofline and dom_name == "flash_attn.seq_tile":
         roofline["note"] = ("priced against the dense f16 matrix-core peak as the brief asks; the matrix cores only form the scores. "
                             "The reference accumulates V key by key in f16 (f32 fma, f16 store), and reproducing that takes 1.5 vector "
-                            "instructions per (query, key, d): 110 us per launch at the vector units' issue rate, which is the bound that applies")
+                            "instructions per (query, key, d): 150 us per launch at the 2.0 ns per instruction the vector units sustain under this load, "
+                            "plus 60 us of score / factor phases that are vector work as well; that is the bound that applies")
 
     # ---- the same window with the packed f16 attention option (an optional arithmetic, reported beside the headline) -------
     packed = run_harness(["bench", "--model", enc_model, "--what", "encoder", "--backend", "gpu", "--reps", str(a.steps),
