@@ -13,8 +13,8 @@
 //       k_fattn_seq_tile   N > 8:  64 queries x 64 keys per step; QK^T on v_mfma_f32_32x32x16_f16 from LDS-staged K,
 //                                  softmax factors in LDS, then 16 queries per wavefront walk the 64 keys with
 //                                  v_fma_mixlo/hi_f16 chains against the LDS-staged V tile.
-//       k_fattn_seq_row    N <= 8: one block per (query, head): 256 threads score all keys and scan the maximum,
-//                                  one wavefront (lane = d) runs the chain with V streamed from global memory.
+//       k_fattn_seq_row    N <= 8: one block per (query, head): one wavefront (lane = d) runs the chain while the
+//                                  other three score, scan and stage the next 192 keys.
 //   MI355X_FA_F32          f32 accumulators: closer to exact arithmetic, not to the reference (whose f16 accumulator
 //                          loses about 1e-4 NMSE per attention, which whole-model logits then show as several 1e-3).
 //       k_fattn_mfma       N > 8:  both products on the matrix cores, online softmax, probabilities as f16 operands
@@ -154,129 +154,127 @@ __device__ __forceinline__ void seq_factors(float s, float & M, float & vs, floa
 // ------------------------------------------------------------------------------------------------------
 
 #define ROW_CHUNK 64
-#define ROW_STAGE 192     // keys staged per step: one per thread of the three wavefronts that do not walk the chain
+#define ROW_STAGE 192     // keys per stage: one per thread of the three wavefronts that do not walk the chain
 #define ROW_VT    (ROW_STAGE + 8)   // f16 pitch of a d-row of the transposed V stage
 
+// A pipeline of two roles with a stage of 192 keys between them.  Wavefronts 1 .. 3 (one key per thread) produce stage
+// s + 1 while wavefront 0 (lane = d) walks the chain over stage s:
+//   producer, first half   dot product of the key's row (requested a stage earlier) with q, the score, the maximum of the
+//                          wavefront's 64 scores as an inclusive scan; request the K row of the stage after
+//   -- barrier --
+//   producer, second half  exclusive prefix maximum (running maximum of the stages before, the wavefronts before, the scan),
+//                          the key's factor (vs, or -ms where it raises the maximum: then vs is exactly 1) -> LDS, the
+//                          stage's share (P, A) of the denominator S <- S * P + A, the key's V row -> LDS transposed;
+//                          request the V row of the stage after
+//   -- barrier --
+// The walker spends a stage's time (192 keys x two dependent instructions) between the barriers of its own 64-key chunks,
+// so what a query costs is the chain plus one stage of lead-in: the scores, the exponentials and the staging all run
+// beside it on the other three SIMDs, and no array grows with the number of keys.
 __global__ void __launch_bounds__(256) k_fattn_seq_row(fa_args a, int kv_pad) {
-    extern __shared__ __attribute__((aligned(16))) float sm[];
-    float * vs_s = sm;                 // [kv_pad] scores, then vs
-    float * ms_s = sm + kv_pad;        // [kv_pad]
-    __shared__ float red_m[4], red_p[4], red_a[4];
-    __shared__ float s_total;
+    __shared__ __attribute__((aligned(16))) half_t v_lds[2][FA_D * ROW_VT];   // V stage, transposed: [d][key]
+    __shared__ float f_lds[2][ROW_STAGE];
+    __shared__ float red_m[3], red_p[2][3], red_a[2][3];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int64_t n = blockIdx.x, h = blockIdx.y, i3 = blockIdx.z;
     const int KV = (int) a.KV;
+    const int n_stages = (kv_pad + ROW_STAGE - 1) / ROW_STAGE;
 
-    const float * qp = (const float *)(a.q + n * a.q_nb1 + h * a.q_nb2 + i3 * a.q_nb3);
-    const char *  kb = a.k + (h / a.hk_ratio) * a.k_nb2 + (i3 / a.k_ne3_ratio) * a.k_nb3;
-    const char *  vb = a.v + (h / a.hv_ratio) * a.v_nb2 + (i3 / a.v_ne3_ratio) * a.v_nb3;
-    const half_t * mp = a.mask ? (const half_t *)(a.mask + n * a.m_nb1) : nullptr;
+    if (wave != 0) {
+        // ---- producers ----------------------------------------------------------------------------------------------
+        const float * qp = (const float *)(a.q + n * a.q_nb1 + h * a.q_nb2 + i3 * a.q_nb3);
+        const char *  kb = a.k + (h / a.hk_ratio) * a.k_nb2 + (i3 / a.k_ne3_ratio) * a.k_nb3;
+        const char *  vb = a.v + (h / a.hv_ratio) * a.v_nb2 + (i3 / a.v_ne3_ratio) * a.v_nb3;
+        const half_t * mp = a.mask ? (const half_t *)(a.mask + n * a.m_nb1) : nullptr;
+        const int stid = tid - WAVE, pw = wave - 1;
 
-    // ---- scores -------------------------------------------------------------------------------------
-    float q[FA_D];
+        float q[FA_D];
 #pragma unroll
-    for (int d = 0; d < FA_D; d += 4) {
-        const float4 t = *(const float4 *)(qp + d);
-        q[d] = (float)(half_t) t.x; q[d+1] = (float)(half_t) t.y; q[d+2] = (float)(half_t) t.z; q[d+3] = (float)(half_t) t.w;
-    }
-    // keys tid, tid + 256, ...: the next key's row (and mask value) is in flight while this one's dot product is formed;
-    // the loads are unconditional (clamped) so that the wait in front of the dot product covers this key's row only
-    {
-        half8_t kcur[FA_D / 8], knext[FA_D / 8];
-        float mcur = 0.0f, mnext = 0.0f;
-        auto load_key = [&](half8_t (&kk)[FA_D / 8], float & mv, int key) __attribute__((always_inline)) {
+        for (int d = 0; d < FA_D; d += 4) {
+            const float4 t = *(const float4 *)(qp + d);
+            q[d] = (float)(half_t) t.x; q[d+1] = (float)(half_t) t.y; q[d+2] = (float)(half_t) t.z; q[d+3] = (float)(half_t) t.w;
+        }
+        // loads are unconditional (a key beyond the end reads the last one; its score is -inf and its V row zero)
+        half8_t krow[FA_D / 8];
+        u32x4 vrow[FA_D / 8];
+        float mval = 0.0f;
+        auto load_k = [&](int key) __attribute__((always_inline)) {
             const int kc = key < KV ? key : KV - 1;
             const half8_t * kr = (const half8_t *)(kb + (int64_t) kc * a.k_nb1);
 #pragma unroll
-            for (int c = 0; c < FA_D / 8; ++c) kk[c] = kr[c];
-            mv = mp ? (float) mp[kc] : 0.0f;
+            for (int c = 0; c < FA_D / 8; ++c) krow[c] = kr[c];
+            mval = mp ? (float) mp[kc] : 0.0f;
         };
-        load_key(kcur, mcur, tid);
-        for (int key = tid; key < kv_pad; key += 256) {
-            load_key(knext, mnext, key + 256);
-            float dot = 0.0f;
+        auto load_v = [&](int key) __attribute__((always_inline)) {
+            const u32x4 * src = (const u32x4 *)(vb + (int64_t)(key < KV ? key : KV - 1) * a.v_nb1);
 #pragma unroll
-            for (int c = 0; c < FA_D / 8; ++c) {
+            for (int i = 0; i < FA_D / 8; ++i) vrow[i] = src[i];
+        };
+        load_k(stid);
+        load_v(stid);
+
+        float M = -INFINITY;                               // running maximum over the stages produced so far
+        for (int s = 0; s <= n_stages; ++s) {
+            const bool produce = s < n_stages;             // the last round only keeps the barriers in step with the walker
+            const int key = s * ROW_STAGE + stid;
+            float score = -INFINITY, exc = -INFINITY;
+            if (produce) {
+                float dot = 0.0f;
 #pragma unroll
-                for (int e = 0; e < 8; ++e) dot += q[8*c + e] * (float) kcur[c][e];
+                for (int c = 0; c < FA_D / 8; ++c) {
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) dot += q[8*c + e] * (float) krow[c][e];
+                }
+                score = key < KV && mval != -INFINITY ? __fadd_rn(__fmul_rn(dot, a.scale), mval) : -INFINITY;
+                load_k(key + ROW_STAGE);
+                float inc = score;
+#pragma unroll
+                for (int o = 1; o < WAVE; o <<= 1) { const float t = __shfl_up(inc, o, WAVE); if (lane >= o) inc = fmaxf(inc, t); }
+                if (lane == WAVE - 1) red_m[pw] = inc;
+                exc = __shfl_up(inc, 1, WAVE);
+                if (lane == 0) exc = -INFINITY;
             }
-            vs_s[key] = key < KV && mcur != -INFINITY ? __fadd_rn(__fmul_rn(dot, a.scale), mcur) : -INFINITY;
+            __syncthreads();
+            if (produce) {
+                float Mk = fmaxf(exc, M);
+                for (int w = 0; w < pw; ++w) Mk = fmaxf(Mk, red_m[w]);
+                M = fmaxf(fmaxf(M, red_m[0]), fmaxf(red_m[1], red_m[2]));
+                float vs, ms, P = 1.0f, A = 0.0f;
+                seq_factors(score, Mk, vs, ms, P, A);
+                f_lds[s & 1][stid] = ms != 1.0f ? -ms : vs;
+                // ordered reduction of (P, A): (P1, A1) then (P2, A2) -> (P1*P2, A1*P2 + A2)
 #pragma unroll
-            for (int c = 0; c < FA_D / 8; ++c) kcur[c] = knext[c];
-            mcur = mnext;
-        }
-    }
-    __syncthreads();
-
-    // ---- prefix maximum and softmax factors: thread t owns keys [t*seg, (t+1)*seg) ---------------------------------
-    const int seg = (kv_pad + 255) / 256;
-    const int k0 = tid * seg, k1 = min(kv_pad, k0 + seg);
-    float lmax = -INFINITY;
-    for (int key = k0; key < k1; ++key) lmax = fmaxf(lmax, vs_s[key]);
-    // exclusive prefix maximum across the block: inclusive scan inside the wavefront, then the wavefront totals
-    float inc = lmax;
+                for (int o = 1; o < WAVE; o <<= 1) {
+                    const float Pn = __shfl_down(P, o, WAVE), An = __shfl_down(A, o, WAVE);
+                    if ((lane & (2 * o - 1)) == 0) { A = A * Pn + An; P = P * Pn; }
+                }
+                if (lane == 0) { red_p[s & 1][pw] = P; red_a[s & 1][pw] = A; }
+                uint16_t * dst = (uint16_t *) v_lds[s & 1] + stid;               // column `stid` of the stage
+                const bool vok = key < KV;
 #pragma unroll
-    for (int o = 1; o < WAVE; o <<= 1) { const float t = __shfl_up(inc, o, WAVE); if (lane >= o) inc = fmaxf(inc, t); }
-    if (lane == WAVE - 1) red_m[wave] = inc;
-    float exc = __shfl_up(inc, 1, WAVE);
-    if (lane == 0) exc = -INFINITY;
-    __syncthreads();
-    for (int w = 0; w < wave; ++w) exc = fmaxf(exc, red_m[w]);
-
-    float M = exc, P = 1.0f, A = 0.0f;
-    for (int key = k0; key < k1; ++key) {
-        float vs, ms;
-        seq_factors(vs_s[key], M, vs, ms, P, A);
-        vs_s[key] = vs; ms_s[key] = ms;
-    }
-    // ordered reduction of (P, A): (P1, A1) then (P2, A2) -> (P1*P2, A1*P2 + A2)
+                for (int i = 0; i < FA_D / 8; ++i) {
 #pragma unroll
-    for (int o = 1; o < WAVE; o <<= 1) {
-        const float Pn = __shfl_down(P, o, WAVE), An = __shfl_down(A, o, WAVE);
-        if ((lane & (2 * o - 1)) == 0) { A = A * Pn + An; P = P * Pn; }
-    }
-    if (lane == 0) { red_p[wave] = P; red_a[wave] = A; }
-    __syncthreads();
-    if (tid == 0) {
-        float S = 0.0f;
-        for (int w = 0; w < 4; ++w) S = S * red_p[w] + red_a[w];
-        s_total = S;
-    }
-    __syncthreads();
-
-    // ---- the sequential f16 chain: lane = d -----------------------------------------------------------------------------------
-    // One wavefront walks the keys; with nothing else running on its SIMD the time of a key is the latency of its
-    // dependent instructions, so the common case is straight-line code of two per key: v_fma_mix_f32 (f16 V, f32
-    // factor, f16 accumulator -> f32) and v_cvt_f16_f32 — the reference's f32 fma and its f16 store.  The factors are
-    // read once per 64 keys, one per lane (vs, or -ms where the key raises the maximum: then vs is 1), and reach the
-    // chain as scalar operands through v_readlane.  V is staged by the other three wavefronts: 192 keys (rows of 128 B) per
-    // step into one of two LDS buffers, the next step's rows in flight meanwhile, so the walker never waits on HBM and
-    // spends no issue slots on the staging itself.
-    // V sits in LDS transposed, [d][key] (pitch ROW_VT: 16-byte reads of 16 lanes cover all banks once), so that the walker's
-    // lane reads eight keys of its d with one instruction: with one 2-byte read per key, the 64 reads of a chunk could not
-    // be kept in flight under the chunk before it (the wait counter only counts to 15) and took longer than the chain.
-    half_t * v_lds = (half_t *)(sm + 2 * kv_pad);          // [2][FA_D][ROW_VT]
-    u32x4 vrow[8];
-    const int stid = tid - WAVE;                           // staging thread: wavefronts 1 .. 3
-    auto load_rows = [&](int key0) __attribute__((always_inline)) {
-        const int key = key0 + stid;
-        const u32x4 * src = (const u32x4 *)(vb + (int64_t)(key < KV ? key : KV - 1) * a.v_nb1);
-#pragma unroll
-        for (int i = 0; i < 8; ++i) vrow[i] = key < KV ? src[i] : (u32x4){0, 0, 0, 0};
-    };
-    auto store_rows = [&](int buf) __attribute__((always_inline)) {
-        uint16_t * dst = (uint16_t *)(v_lds + (size_t) buf * FA_D * ROW_VT) + stid;      // column `stid` of the stage
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-#pragma unroll
-            for (int w = 0; w < 4; ++w) {
-                dst[(8 * i + 2 * w    ) * ROW_VT] = (uint16_t) vrow[i][w];
-                dst[(8 * i + 2 * w + 1) * ROW_VT] = (uint16_t)(vrow[i][w] >> 16);
+                    for (int w = 0; w < 4; ++w) {
+                        const uint32_t pair = vok ? vrow[i][w] : 0u;
+                        dst[(8 * i + 2 * w    ) * ROW_VT] = (uint16_t) pair;
+                        dst[(8 * i + 2 * w + 1) * ROW_VT] = (uint16_t)(pair >> 16);
+                    }
+                }
+                load_v(key + ROW_STAGE);
             }
+            __syncthreads();
         }
-    };
+        return;
+    }
 
+    // ---- the walker: the sequential f16 chain, lane = d -------------------------------------------------------------------
+    // With nothing else running on its SIMD the time of a key is the latency of its dependent instructions, so the common
+    // case is straight-line code of two per key: v_fma_mix_f32 (f16 V, f32 factor, f16 accumulator -> f32) and
+    // v_cvt_f16_f32 — the reference's f32 fma and its f16 store.  The factors are read once per 64 keys, one per lane, and
+    // reach the chain as scalar operands through v_readlane.  V sits in LDS transposed (pitch ROW_VT: 16-byte reads of 16
+    // lanes cover all banks once), so that a lane reads eight keys of its d with one instruction: with one 2-byte read per
+    // key, the 64 reads of a chunk could not be kept in flight under the chunk before it (the wait counter only counts to
+    // 15) and took longer than the chain.
     uint32_t acc = 0;                                      // f16 accumulator in the low half
     // one key: acc = f16(fma(v, vs, acc)); v is the low or the high half of `pair`
     auto mad = [&](uint32_t pair, bool high, uint32_t vs_bits) __attribute__((always_inline)) {
@@ -291,65 +289,56 @@ __global__ void __launch_bounds__(256) k_fattn_seq_row(fa_args a, int kv_pad) {
 #pragma unroll
         for (int i = 0; i < ROW_CHUNK / 8; ++i) ch.c[i] = src[i];
     };
-    // (vs_f, ms_f): the factors of key key0 + lane, read while the chunk before was walked
-    auto run_chunk = [&](const chunk & ch, float vs_f, float ms_f) __attribute__((always_inline)) {
-        const bool  raised_l = ms_f != 1.0f;
-        const uint32_t f_l = __float_as_uint(raised_l ? -ms_f : vs_f);
-        const uint64_t raised = __ballot(raised_l);        // uniform: which of the 64 keys move the maximum
+    // f: the factor of key k0 + lane
+    auto run_chunk = [&](const chunk & ch, float f) __attribute__((always_inline)) {
+        const uint32_t f_l = __float_as_uint(f);
+        const uint64_t raised = __ballot((int32_t) f_l < 0);   // uniform: which of the 64 keys move the maximum (-ms, down to -0)
         if (raised == 0) {
 #pragma unroll
             for (int j = 0; j < ROW_CHUNK; ++j) mad(ch.c[j >> 3][(j >> 1) & 3], j & 1, __builtin_amdgcn_readlane(f_l, j));   // masked keys: vs = 0 leaves acc as it is
         } else {
 #pragma unroll
             for (int j = 0; j < ROW_CHUNK; ++j) {
-                uint32_t f = __builtin_amdgcn_readlane(f_l, j);
+                uint32_t fj = __builtin_amdgcn_readlane(f_l, j);
                 if ((raised >> j) & 1) {                   // scalar condition
                     float t;
-                    asm("v_fma_mix_f32 %0, %1, %2, 0 op_sel_hi:[1,0,0]" : "=v"(t) : "v"(acc), "s"(f ^ 0x80000000u));
+                    asm("v_fma_mix_f32 %0, %1, %2, 0 op_sel_hi:[1,0,0]" : "=v"(t) : "v"(acc), "s"(fj ^ 0x80000000u));
                     asm("v_cvt_f16_f32 %0, %1" : "=v"(acc) : "v"(t));
-                    f = 0x3f800000u;                       // vs = 1
+                    fj = 0x3f800000u;                      // vs = 1
                 }
-                mad(ch.c[j >> 3][(j >> 1) & 3], j & 1, f);
+                mad(ch.c[j >> 3][(j >> 1) & 3], j & 1, fj);
             }
         }
     };
 
-    if (wave != 0) load_rows(0);
-    float fv = vs_s[lane], fm = ms_s[lane];                // factors of the chunk walked next (kv_pad >= ROW_CHUNK)
-    int buf = 0;
-    for (int key0 = 0; key0 < kv_pad; key0 += ROW_STAGE, buf ^= 1) {
-        if (wave != 0) store_rows(buf);
-        __syncthreads();       // rows visible; the buffer written next time was last read before the previous barrier
-        if (wave != 0) {
-            if (key0 + ROW_STAGE < kv_pad) load_rows(key0 + ROW_STAGE);
-        } else {
-            const half_t * vbuf = v_lds + (size_t) buf * FA_D * ROW_VT;
-            const int nk = min(ROW_STAGE, kv_pad - key0);                   // multiple of ROW_CHUNK
-            chunk va, vn;
-            read_chunk(va, vbuf, 0);
-            for (int k0 = 0; k0 < nk; k0 += 2 * ROW_CHUNK) {
-                const bool more = k0 + ROW_CHUNK < nk;
-                if (more) read_chunk(vn, vbuf, k0 + ROW_CHUNK);
-                {
-                    const float cv = fv, cm = fm;
-                    const int nxt = key0 + k0 + ROW_CHUNK < kv_pad ? key0 + k0 + ROW_CHUNK : 0;
-                    fv = vs_s[nxt + lane]; fm = ms_s[nxt + lane];
-                    run_chunk(va, cv, cm);
-                }
-                if (more) {
-                    if (k0 + 2 * ROW_CHUNK < nk) read_chunk(va, vbuf, k0 + 2 * ROW_CHUNK);
-                    const float cv = fv, cm = fm;
-                    const int nxt = key0 + k0 + 2 * ROW_CHUNK < kv_pad ? key0 + k0 + 2 * ROW_CHUNK : 0;
-                    fv = vs_s[nxt + lane]; fm = ms_s[nxt + lane];
-                    run_chunk(vn, cv, cm);
-                }
-            }
+    float S = 0.0f;
+    __syncthreads();                                       // stage 0 is being produced
+    __syncthreads();
+    for (int s = 0; s < n_stages; ++s) {
+        const int buf = s & 1;
+        const int nk = min(ROW_STAGE, kv_pad - s * ROW_STAGE);                  // 64, 128 or 192
+        const half_t * vbuf = v_lds[buf];
+        chunk va, vn;
+        read_chunk(va, vbuf, 0);
+        const float f0 = f_lds[buf][lane];
+        const float f1 = nk > ROW_CHUNK ? f_lds[buf][ROW_CHUNK + lane] : 0.0f;
+        const float f2 = nk > 2 * ROW_CHUNK ? f_lds[buf][2 * ROW_CHUNK + lane] : 0.0f;
+#pragma unroll
+        for (int w = 0; w < 3; ++w) S = S * red_p[buf][w] + red_a[buf][w];
+        if (nk > ROW_CHUNK) read_chunk(vn, vbuf, ROW_CHUNK);
+        run_chunk(va, f0);
+        __syncthreads();
+        if (nk > ROW_CHUNK) {
+            if (nk > 2 * ROW_CHUNK) read_chunk(va, vbuf, 2 * ROW_CHUNK);
+            run_chunk(vn, f1);
+            if (nk > 2 * ROW_CHUNK) run_chunk(va, f2);
         }
+        __syncthreads();
     }
-    if (wave != 0) return;
+
     half_t acc_h; { const uint16_t t16 = (uint16_t) acc; __builtin_memcpy(&acc_h, &t16, 2); }
     float * dp = (float *) a.d + ((i3 * a.N + n) * a.H + h) * FA_D;
-    const float o = (float) acc_h * (1.0f / s_total);
+    const float o = (float) acc_h * (1.0f / S);
     dp[lane] = o;
     if (a.x16) {
         // MI355X_FA_EMIT_Q8_0: the projection that follows reads its activations as Q8_0 (rows [N][H * 64]: int8 quants |
@@ -902,13 +891,13 @@ __global__ void __launch_bounds__(256) k_fattn_mfma(fa_args a) {
 // ------------------------------------------------------------------------------------------------------
 
 #define SEQ_ROW_MAX_N   8
-#define SEQ_ROW_MAX_KV  7168      // two f32 arrays of that many keys stay under 64 KB of LDS
 
 enum { FA_K_VEC = 0, FA_K_SEQ_ROW = 1, FA_K_SEQ_TILE = 2, FA_K_MFMA = 3 };
 
 static int fa_kernel(const mi355x_tensor * q, const mi355x_tensor * k, int mode) {
     if (mode == MI355X_FA_F32) return q->ne[1] > SEQ_ROW_MAX_N ? FA_K_MFMA : FA_K_VEC;
-    if (q->ne[1] <= SEQ_ROW_MAX_N && k->ne[1] <= SEQ_ROW_MAX_KV) return FA_K_SEQ_ROW;
+    (void) k;
+    if (q->ne[1] <= SEQ_ROW_MAX_N) return FA_K_SEQ_ROW;
     return FA_K_SEQ_TILE;
 }
 
@@ -951,6 +940,7 @@ extern "C" int mi355x_flash_attn_ext(const mi355x_tensor * q, const mi355x_tenso
     };
     if (!al16(q) || !al16(k) || !al16(v) || (uintptr_t) dst->data % 16 != 0) return MI355X_ERR_UNSUPPORTED;
     if (N == 0 || H == 0 || q->ne[3] == 0) return MI355X_OK;
+    if (KV == 0 || KV > (1 << 30)) return MI355X_ERR_UNSUPPORTED;        // every kernel reads key 0 and counts keys in 32 bits
     if (H > 65535 || q->ne[3] > 65535) return MI355X_ERR_UNSUPPORTED;
 
     fa_args a;
@@ -984,15 +974,7 @@ extern "C" int mi355x_flash_attn_ext(const mi355x_tensor * q, const mi355x_tenso
         case FA_K_SEQ_ROW: {
             const int kv_pad = (int)((KV + ROW_CHUNK - 1) / ROW_CHUNK * ROW_CHUNK);
             dim3 grid((unsigned) N, (unsigned) H, (unsigned) q->ne[3]);
-            const size_t lds = (size_t) kv_pad * 8 + (size_t) 2 * ROW_VT * FA_D * sizeof(half_t);      // factors + two V stages
-            static bool configured[64];                    // per device: more than the default 64 KB of dynamic LDS
-            int dev = 0;
-            if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return MI355X_ERR_HIP;
-            if (!configured[dev]) {
-                if (hipFuncSetAttribute((const void *) k_fattn_seq_row, hipFuncAttributeMaxDynamicSharedMemorySize, SEQ_ROW_MAX_KV * 8 + 2 * ROW_VT * FA_D * 2) != hipSuccess) return MI355X_ERR_HIP;
-                configured[dev] = true;
-            }
-            k_fattn_seq_row<<<grid, 256, lds, st>>>(a, kv_pad);
+            k_fattn_seq_row<<<grid, 256, 0, st>>>(a, kv_pad);
         } break;
         case FA_K_SEQ_TILE: {
             const int64_t gx = (N + T_Q - 1) / T_Q;
