@@ -157,23 +157,37 @@ __device__ __forceinline__ void seq_factors(float s, float & M, float & vs, floa
 #define ROW_STAGE 192     // keys per stage: one per thread of the three wavefronts that do not walk the chain
 #define ROW_VT    (ROW_STAGE + 8)   // f16 pitch of a d-row of the transposed V stage
 
-// A pipeline of two roles with a stage of 192 keys between them.  Wavefronts 1 .. 3 (one key per thread) produce stage
-// s + 1 while wavefront 0 (lane = d) walks the chain over stage s:
-//   producer, first half   dot product of the key's row (requested a stage earlier) with q, the score, the maximum of the
-//                          wavefront's 64 scores as an inclusive scan; request the K row of the stage after
-//   -- barrier --
-//   producer, second half  exclusive prefix maximum (running maximum of the stages before, the wavefronts before, the scan),
-//                          the key's factor (vs, or -ms where it raises the maximum: then vs is exactly 1) -> LDS, the
-//                          stage's share (P, A) of the denominator S <- S * P + A, the key's V row -> LDS transposed;
-//                          request the V row of the stage after
-//   -- barrier --
-// The walker spends a stage's time (192 keys x two dependent instructions) between the barriers of its own 64-key chunks,
-// so what a query costs is the chain plus one stage of lead-in: the scores, the exponentials and the staging all run
-// beside it on the other three SIMDs, and no array grows with the number of keys.
+// x of lane - N of the same row of 16 lanes (FILL where there is none), and lane 15 / lane 31 handed to the rows after it:
+// the steps of a scan over the wavefront that stays out of LDS
+template <int CTRL, int ROW_MASK = 0xf>
+__device__ __forceinline__ float dpp_fill(float v, float fill) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, fill), __builtin_bit_cast(int, v), CTRL, ROW_MASK, 0xf, false));
+}
+__device__ __forceinline__ float wave_scan_max(float v) {                      // inclusive
+    v = fmaxf(v, dpp_fill<0x111>(v, -INFINITY));                               // row_shr:1
+    v = fmaxf(v, dpp_fill<0x112>(v, -INFINITY));                               // row_shr:2
+    v = fmaxf(v, dpp_fill<0x114>(v, -INFINITY));                               // row_shr:4
+    v = fmaxf(v, dpp_fill<0x118>(v, -INFINITY));                               // row_shr:8
+    v = fmaxf(v, dpp_fill<0x142, 0xa>(v, -INFINITY));                          // row_bcast:15 into rows 1 and 3
+    v = fmaxf(v, dpp_fill<0x143, 0xc>(v, -INFINITY));                          // row_bcast:31 into rows 2 and 3
+    return v;
+}
+
+// A pipeline of two roles with a stage of 192 keys between them.  Wavefront 0 (lane = d) walks the chain over stage s
+// while wavefronts 1 .. 3 (one key per thread) work on the two stages after it, one barrier per stage:
+//   factors of stage s + 1   exclusive prefix maximum (running maximum of the stages before, the wavefronts before, the
+//                            thread's own scan value from the round before), the key's factor (vs, or -ms where it raises
+//                            the maximum: then vs is exactly 1) -> LDS, the stage's share (P, A) of the denominator
+//                            S <- S * P + A, the key's V row -> LDS transposed; request the V row of the stage after
+//   scores of stage s + 2    dot product of the key's row (requested a round earlier) with q, the score, the maximum of
+//                            the wavefront's 64 scores as an inclusive scan -> LDS; request the K row of the stage after
+// so what a query costs is the chain (192 keys x two dependent instructions per stage) plus two rounds of lead-in: the
+// scores, the exponentials and the staging run beside it on the other three SIMDs, and no array grows with the number
+// of keys.
 __global__ void __launch_bounds__(256) k_fattn_seq_row(fa_args a, int kv_pad) {
     __shared__ __attribute__((aligned(16))) half_t v_lds[2][FA_D * ROW_VT];   // V stage, transposed: [d][key]
     __shared__ float f_lds[2][ROW_STAGE];
-    __shared__ float red_m[3], red_p[2][3], red_a[2][3];
+    __shared__ float red_m[2][3], red_p[2][3], red_a[2][3];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int64_t n = blockIdx.x, h = blockIdx.y, i3 = blockIdx.z;
@@ -194,62 +208,75 @@ __global__ void __launch_bounds__(256) k_fattn_seq_row(fa_args a, int kv_pad) {
             const float4 t = *(const float4 *)(qp + d);
             q[d] = (float)(half_t) t.x; q[d+1] = (float)(half_t) t.y; q[d+2] = (float)(half_t) t.z; q[d+3] = (float)(half_t) t.w;
         }
-        // loads are unconditional (a key beyond the end reads the last one; its score is -inf and its V row zero)
+        // Every load is unconditional and nothing in the loop is: a key beyond the end reads the last one (its score is
+        // -inf and its V row zero), and after the last stage one more is scored that nobody walks.  With a load behind
+        // a condition the registers it fills are copied where the paths join, and the copy waits for the load — the next
+        // stage's rows would be waited for in the round that requests them.
         half8_t krow[FA_D / 8];
         u32x4 vrow[FA_D / 8];
-        float mval = 0.0f;
+        uint16_t mbits = 0;                                // the key's mask value as loaded (f16)
+        const uint16_t * mrow = mp ? (const uint16_t *) mp : (const uint16_t *) kb;      // without a mask: any readable address
+        const int64_t m_step = mp ? 1 : 0;
         auto load_k = [&](int key) __attribute__((always_inline)) {
             const int kc = key < KV ? key : KV - 1;
             const half8_t * kr = (const half8_t *)(kb + (int64_t) kc * a.k_nb1);
 #pragma unroll
             for (int c = 0; c < FA_D / 8; ++c) krow[c] = kr[c];
-            mval = mp ? (float) mp[kc] : 0.0f;
+            mbits = mrow[kc * m_step];
         };
         auto load_v = [&](int key) __attribute__((always_inline)) {
             const u32x4 * src = (const u32x4 *)(vb + (int64_t)(key < KV ? key : KV - 1) * a.v_nb1);
 #pragma unroll
             for (int i = 0; i < FA_D / 8; ++i) vrow[i] = src[i];
         };
-        load_k(stid);
-        load_v(stid);
 
-        float M = -INFINITY;                               // running maximum over the stages produced so far
-        for (int s = 0; s <= n_stages; ++s) {
-            const bool produce = s < n_stages;             // the last round only keeps the barriers in step with the walker
+        float score, inc, exc;                             // of the stage scored last: the score, the scan and the scan of the lane before
+        auto score_phase = [&](int s) __attribute__((always_inline)) {
             const int key = s * ROW_STAGE + stid;
-            float score = -INFINITY, exc = -INFINITY;
-            if (produce) {
-                float dot = 0.0f;
+            float dot = 0.0f;
 #pragma unroll
-                for (int c = 0; c < FA_D / 8; ++c) {
+            for (int c = 0; c < FA_D / 8; ++c) {
 #pragma unroll
-                    for (int e = 0; e < 8; ++e) dot += q[8*c + e] * (float) krow[c][e];
-                }
-                score = key < KV && mval != -INFINITY ? __fadd_rn(__fmul_rn(dot, a.scale), mval) : -INFINITY;
-                load_k(key + ROW_STAGE);
-                float inc = score;
-#pragma unroll
-                for (int o = 1; o < WAVE; o <<= 1) { const float t = __shfl_up(inc, o, WAVE); if (lane >= o) inc = fmaxf(inc, t); }
-                if (lane == WAVE - 1) red_m[pw] = inc;
-                exc = __shfl_up(inc, 1, WAVE);
-                if (lane == 0) exc = -INFINITY;
+                for (int e = 0; e < 8; ++e) dot += q[8*c + e] * (float) krow[c][e];
             }
-            __syncthreads();
-            if (produce) {
+            const float mval = mp ? h2f(mbits) : 0.0f;
+            score = key < KV && mval != -INFINITY ? __fadd_rn(__fmul_rn(dot, a.scale), mval) : -INFINITY;
+            load_k(key + ROW_STAGE);
+            inc = wave_scan_max(score);
+            if (lane == WAVE - 1) red_m[s & 1][pw] = inc;
+            exc = dpp_fill<0x138>(inc, -INFINITY);         // wave_shr:1
+        };
+
+        // V rows first, then K rows, as in the loop: the wait in front of a use then leaves the younger loads in flight
+        // on every path into it
+        load_v(stid);
+        __builtin_amdgcn_sched_barrier(0);
+        load_k(stid);
+        __builtin_amdgcn_sched_barrier(0);
+        score_phase(0);
+        __syncthreads();
+
+        float M = -INFINITY;                               // running maximum over the stages whose factors are made
+        for (int s = 1; s <= n_stages; ++s) {
+            // ---- factors of stage s - 1
+            {
+                const int f = (s - 1) & 1;
+                const int key = (s - 1) * ROW_STAGE + stid;
                 float Mk = fmaxf(exc, M);
-                for (int w = 0; w < pw; ++w) Mk = fmaxf(Mk, red_m[w]);
-                M = fmaxf(fmaxf(M, red_m[0]), fmaxf(red_m[1], red_m[2]));
+                if (pw > 0) Mk = fmaxf(Mk, red_m[f][0]);
+                if (pw > 1) Mk = fmaxf(Mk, red_m[f][1]);
+                M = fmaxf(fmaxf(M, red_m[f][0]), fmaxf(red_m[f][1], red_m[f][2]));
                 float vs, ms, P = 1.0f, A = 0.0f;
                 seq_factors(score, Mk, vs, ms, P, A);
-                f_lds[s & 1][stid] = ms != 1.0f ? -ms : vs;
+                f_lds[f][stid] = ms != 1.0f ? -ms : vs;
                 // ordered reduction of (P, A): (P1, A1) then (P2, A2) -> (P1*P2, A1*P2 + A2)
 #pragma unroll
                 for (int o = 1; o < WAVE; o <<= 1) {
                     const float Pn = __shfl_down(P, o, WAVE), An = __shfl_down(A, o, WAVE);
                     if ((lane & (2 * o - 1)) == 0) { A = A * Pn + An; P = P * Pn; }
                 }
-                if (lane == 0) { red_p[s & 1][pw] = P; red_a[s & 1][pw] = A; }
-                uint16_t * dst = (uint16_t *) v_lds[s & 1] + stid;               // column `stid` of the stage
+                if (lane == 0) { red_p[f][pw] = P; red_a[f][pw] = A; }
+                uint16_t * dst = (uint16_t *) v_lds[f] + stid;                   // column `stid` of the stage
                 const bool vok = key < KV;
 #pragma unroll
                 for (int i = 0; i < FA_D / 8; ++i) {
@@ -262,6 +289,8 @@ __global__ void __launch_bounds__(256) k_fattn_seq_row(fa_args a, int kv_pad) {
                 }
                 load_v(key + ROW_STAGE);
             }
+            // ---- scores of stage s
+            score_phase(s);
             __syncthreads();
         }
         return;
@@ -312,9 +341,9 @@ __global__ void __launch_bounds__(256) k_fattn_seq_row(fa_args a, int kv_pad) {
     };
 
     float S = 0.0f;
-    __syncthreads();                                       // stage 0 is being produced
-    __syncthreads();
+    __syncthreads();                                       // stage 0 is scored
     for (int s = 0; s < n_stages; ++s) {
+        __syncthreads();                                   // stage s has its factors and its V rows; stage s - 1 is walked
         const int buf = s & 1;
         const int nk = min(ROW_STAGE, kv_pad - s * ROW_STAGE);                  // 64, 128 or 192
         const half_t * vbuf = v_lds[buf];
@@ -327,13 +356,11 @@ __global__ void __launch_bounds__(256) k_fattn_seq_row(fa_args a, int kv_pad) {
         for (int w = 0; w < 3; ++w) S = S * red_p[buf][w] + red_a[buf][w];
         if (nk > ROW_CHUNK) read_chunk(vn, vbuf, ROW_CHUNK);
         run_chunk(va, f0);
-        __syncthreads();
         if (nk > ROW_CHUNK) {
             if (nk > 2 * ROW_CHUNK) read_chunk(va, vbuf, 2 * ROW_CHUNK);
             run_chunk(vn, f1);
             if (nk > 2 * ROW_CHUNK) run_chunk(va, f2);
         }
-        __syncthreads();
     }
 
     half_t acc_h; { const uint16_t t16 = (uint16_t) acc; __builtin_memcpy(&acc_h, &t16, 2); }
