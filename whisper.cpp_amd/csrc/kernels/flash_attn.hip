@@ -163,6 +163,7 @@ template <int CTRL, int ROW_MASK = 0xf>
 __device__ __forceinline__ float dpp_fill(float v, float fill) {
     return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, fill), __builtin_bit_cast(int, v), CTRL, ROW_MASK, 0xf, false));
 }
+__device__ __forceinline__ float readlane_f(float v, int l) { return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), l)); }
 __device__ __forceinline__ float wave_scan_max(float v) {                      // inclusive
     v = fmaxf(v, dpp_fill<0x111>(v, -INFINITY));                               // row_shr:1
     v = fmaxf(v, dpp_fill<0x112>(v, -INFINITY));                               // row_shr:2
@@ -186,7 +187,7 @@ __device__ __forceinline__ float wave_scan_max(float v) {                      /
 // of keys.
 __global__ void __launch_bounds__(256) k_fattn_seq_row(fa_args a, int kv_pad) {
     __shared__ __attribute__((aligned(16))) half_t v_lds[2][FA_D * ROW_VT];   // V stage, transposed: [d][key]
-    __shared__ float f_lds[2][ROW_STAGE];
+    __shared__ __attribute__((aligned(16))) float f_lds[2][ROW_STAGE];       // one factor per key
     __shared__ float red_m[2][3], red_p[2][3], red_a[2][3];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -202,46 +203,61 @@ __global__ void __launch_bounds__(256) k_fattn_seq_row(fa_args a, int kv_pad) {
         const half_t * mp = a.mask ? (const half_t *)(a.mask + n * a.m_nb1) : nullptr;
         const int stid = tid - WAVE, pw = wave - 1;
 
-        float q[FA_D];
-#pragma unroll
-        for (int d = 0; d < FA_D; d += 4) {
-            const float4 t = *(const float4 *)(qp + d);
-            q[d] = (float)(half_t) t.x; q[d+1] = (float)(half_t) t.y; q[d+2] = (float)(half_t) t.z; q[d+3] = (float)(half_t) t.w;
+        // Rows are read eight lanes to a row (16 bytes each): lane (r = lane / 8, c = lane % 8) takes piece c of the rows
+        // 8 r + i, i = 0 .. 7, of its wavefront's 64 keys, so that every load instruction covers eight whole 128-byte
+        // rows — with a row per lane it touches 64 of them and the stage's loads alone take longer than the chain.
+        const int r8 = lane >> 3, c8 = lane & 7;
+        float q[8];                                        // this lane's piece of q
+        {
+            const float4 t0 = *(const float4 *)(qp + 8 * c8), t1 = *(const float4 *)(qp + 8 * c8 + 4);
+            q[0] = (float)(half_t) t0.x; q[1] = (float)(half_t) t0.y; q[2] = (float)(half_t) t0.z; q[3] = (float)(half_t) t0.w;
+            q[4] = (float)(half_t) t1.x; q[5] = (float)(half_t) t1.y; q[6] = (float)(half_t) t1.z; q[7] = (float)(half_t) t1.w;
         }
         // Every load is unconditional and nothing in the loop is: a key beyond the end reads the last one (its score is
         // -inf and its V row zero), and after the last stage one more is scored that nobody walks.  With a load behind
         // a condition the registers it fills are copied where the paths join, and the copy waits for the load — the next
         // stage's rows would be waited for in the round that requests them.
-        half8_t krow[FA_D / 8];
-        u32x4 vrow[FA_D / 8];
-        uint16_t mbits = 0;                                // the key's mask value as loaded (f16)
+        half8_t krow[8];
+        u32x4 vrow[8];
+        uint16_t mbits = 0;                                // the mask value of key `stid` of the stage as loaded (f16)
         const uint16_t * mrow = mp ? (const uint16_t *) mp : (const uint16_t *) kb;      // without a mask: any readable address
         const int64_t m_step = mp ? 1 : 0;
-        auto load_k = [&](int key) __attribute__((always_inline)) {
-            const int kc = key < KV ? key : KV - 1;
-            const half8_t * kr = (const half8_t *)(kb + (int64_t) kc * a.k_nb1);
+        auto load_k = [&](int s) __attribute__((always_inline)) {
+            const int key0 = s * ROW_STAGE + pw * WAVE + 8 * r8;
 #pragma unroll
-            for (int c = 0; c < FA_D / 8; ++c) krow[c] = kr[c];
-            mbits = mrow[kc * m_step];
+            for (int i = 0; i < 8; ++i) {
+                const int kc = key0 + i < KV ? key0 + i : KV - 1;
+                krow[i] = *(const half8_t *)(kb + (int64_t) kc * a.k_nb1 + 16 * c8);
+            }
+            const int key = s * ROW_STAGE + stid;
+            mbits = mrow[(key < KV ? key : KV - 1) * m_step];
         };
-        auto load_v = [&](int key) __attribute__((always_inline)) {
-            const u32x4 * src = (const u32x4 *)(vb + (int64_t)(key < KV ? key : KV - 1) * a.v_nb1);
+        auto load_v = [&](int s) __attribute__((always_inline)) {
+            const int key0 = s * ROW_STAGE + pw * WAVE + 8 * r8;
 #pragma unroll
-            for (int i = 0; i < FA_D / 8; ++i) vrow[i] = src[i];
+            for (int i = 0; i < 8; ++i) {
+                const int kc = key0 + i < KV ? key0 + i : KV - 1;
+                vrow[i] = *(const u32x4 *)(vb + (int64_t) kc * a.v_nb1 + 16 * c8);
+            }
         };
 
         float score, inc, exc;                             // of the stage scored last: the score, the scan and the scan of the lane before
         auto score_phase = [&](int s) __attribute__((always_inline)) {
             const int key = s * ROW_STAGE + stid;
+            // the piece's share of the eight rows' dot products, summed over the eight lanes of a row; lane c keeps row 8 r + c:
+            // its own key
             float dot = 0.0f;
 #pragma unroll
-            for (int c = 0; c < FA_D / 8; ++c) {
+            for (int i = 0; i < 8; ++i) {
+                float part = 0.0f;
 #pragma unroll
-                for (int e = 0; e < 8; ++e) dot += q[8*c + e] * (float) krow[c][e];
+                for (int e = 0; e < 8; ++e) part += q[e] * (float) krow[i][e];
+                part = lanes_sum<8>(part);
+                dot = c8 == i ? part : dot;
             }
             const float mval = mp ? h2f(mbits) : 0.0f;
             score = key < KV && mval != -INFINITY ? __fadd_rn(__fmul_rn(dot, a.scale), mval) : -INFINITY;
-            load_k(key + ROW_STAGE);
+            load_k(s + 1);
             inc = wave_scan_max(score);
             if (lane == WAVE - 1) red_m[s & 1][pw] = inc;
             exc = dpp_fill<0x138>(inc, -INFINITY);         // wave_shr:1
@@ -249,9 +265,9 @@ __global__ void __launch_bounds__(256) k_fattn_seq_row(fa_args a, int kv_pad) {
 
         // V rows first, then K rows, as in the loop: the wait in front of a use then leaves the younger loads in flight
         // on every path into it
-        load_v(stid);
+        load_v(0);
         __builtin_amdgcn_sched_barrier(0);
-        load_k(stid);
+        load_k(0);
         __builtin_amdgcn_sched_barrier(0);
         score_phase(0);
         __syncthreads();
@@ -269,25 +285,37 @@ __global__ void __launch_bounds__(256) k_fattn_seq_row(fa_args a, int kv_pad) {
                 float vs, ms, P = 1.0f, A = 0.0f;
                 seq_factors(score, Mk, vs, ms, P, A);
                 f_lds[f][stid] = ms != 1.0f ? -ms : vs;
-                // ordered reduction of (P, A): (P1, A1) then (P2, A2) -> (P1*P2, A1*P2 + A2)
-#pragma unroll
-                for (int o = 1; o < WAVE; o <<= 1) {
-                    const float Pn = __shfl_down(P, o, WAVE), An = __shfl_down(A, o, WAVE);
-                    if ((lane & (2 * o - 1)) == 0) { A = A * Pn + An; P = P * Pn; }
+                // ordered reduction of (P, A): (P1, A1) then (P2, A2) -> (P1*P2, A1*P2 + A2), as a binary tree over the
+                // 64 keys: inside each row of 16 lanes with the lane 1, 2, 4, 8 further on (row_shl; beyond the row the
+                // identity), then the four row totals
+#define ROW_PA_STEP(CTRL) { const float Pn = dpp_fill<CTRL>(P, 1.0f), An = dpp_fill<CTRL>(A, 0.0f); A = A * Pn + An; P = P * Pn; }
+                ROW_PA_STEP(0x101) ROW_PA_STEP(0x102) ROW_PA_STEP(0x104) ROW_PA_STEP(0x108)
+#undef ROW_PA_STEP
+                {
+                    const float P0 = readlane_f(P, 0), P1 = readlane_f(P, 16), P2 = readlane_f(P, 32), P3 = readlane_f(P, 48);
+                    const float A0 = readlane_f(A, 0), A1 = readlane_f(A, 16), A2 = readlane_f(A, 32), A3 = readlane_f(A, 48);
+                    const float A01 = A0 * P1 + A1, P01 = P0 * P1, A23 = A2 * P3 + A3, P23 = P2 * P3;
+                    if (lane == 0) { red_p[f][pw] = P01 * P23; red_a[f][pw] = A01 * P23 + A23; }
                 }
-                if (lane == 0) { red_p[f][pw] = P; red_a[f][pw] = A; }
-                uint16_t * dst = (uint16_t *) v_lds[f] + stid;                   // column `stid` of the stage
-                const bool vok = key < KV;
+                // V rows -> [d][key]: the lane holds d = 8 c .. 8 c + 7 of the keys 8 r .. 8 r + 7, which are 16 contiguous bytes
+                // of each of its eight d-rows once the 8 x 8 block of halves is transposed in registers
+                {
+                    const int key0 = (s - 1) * ROW_STAGE + pw * WAVE + 8 * r8;
+                    half_t * dst = v_lds[f] + (8 * c8) * ROW_VT + pw * WAVE + 8 * r8;
 #pragma unroll
-                for (int i = 0; i < FA_D / 8; ++i) {
+                    for (int e = 0; e < 8; ++e) {
+                        u32x4 o;
 #pragma unroll
-                    for (int w = 0; w < 4; ++w) {
-                        const uint32_t pair = vok ? vrow[i][w] : 0u;
-                        dst[(8 * i + 2 * w    ) * ROW_VT] = (uint16_t) pair;
-                        dst[(8 * i + 2 * w + 1) * ROW_VT] = (uint16_t)(pair >> 16);
+                        for (int j = 0; j < 4; ++j) {
+                            const uint32_t lo = key0 + 2 * j     < KV ? vrow[2 * j    ][e >> 1] : 0u;
+                            const uint32_t hi = key0 + 2 * j + 1 < KV ? vrow[2 * j + 1][e >> 1] : 0u;
+                            o[j] = __builtin_amdgcn_perm(hi, lo, (e & 1) ? 0x07060302u : 0x05040100u);
+                        }
+                        *(u32x4 *)(dst + e * ROW_VT) = o;
                     }
                 }
-                load_v(key + ROW_STAGE);
+                load_v(s);
+                __builtin_amdgcn_sched_barrier(0);         // requested here, a round before the rows are stored: not after the dot product
             }
             // ---- scores of stage s
             score_phase(s);
@@ -299,69 +327,96 @@ __global__ void __launch_bounds__(256) k_fattn_seq_row(fa_args a, int kv_pad) {
     // ---- the walker: the sequential f16 chain, lane = d -------------------------------------------------------------------
     // With nothing else running on its SIMD the time of a key is the latency of its dependent instructions, so the common
     // case is straight-line code of two per key: v_fma_mix_f32 (f16 V, f32 factor, f16 accumulator -> f32) and
-    // v_cvt_f16_f32 — the reference's f32 fma and its f16 store.  The factors are read once per 64 keys, one per lane, and
-    // reach the chain as scalar operands through v_readlane.  V sits in LDS transposed (pitch ROW_VT: 16-byte reads of 16
-    // lanes cover all banks once), so that a lane reads eight keys of its d with one instruction: with one 2-byte read per
-    // key, the 64 reads of a chunk could not be kept in flight under the chunk before it (the wait counter only counts to
-    // 15) and took longer than the chain.
+    // v_cvt_f16_f32 — the reference's f32 fma and its f16 store — and nothing between them: a v_readlane per key for the
+    // factor would add a quarter to the time of a key.  So a unit of 32 keys is read from LDS a unit ahead as registers
+    // only: the lane's V values, eight keys per 16-byte read (V sits in LDS transposed, pitch ROW_VT: such reads of 16
+    // lanes cover all banks once), the 32 factors as eight reads of one address for all lanes, and factor k0 + lane % 32
+    // once more for the vote on which keys raise the maximum.
     uint32_t acc = 0;                                      // f16 accumulator in the low half
     // one key: acc = f16(fma(v, vs, acc)); v is the low or the high half of `pair`
-    auto mad = [&](uint32_t pair, bool high, uint32_t vs_bits) __attribute__((always_inline)) {
+    auto mad = [&](uint32_t pair, bool high, float vs) __attribute__((always_inline)) {
         float t;
-        if (high) asm("v_fma_mix_f32 %0, %1, %2, %3 op_sel:[1,0,0] op_sel_hi:[1,0,1]" : "=v"(t) : "v"(pair), "s"(vs_bits), "v"(acc));
-        else      asm("v_fma_mix_f32 %0, %1, %2, %3 op_sel_hi:[1,0,1]" : "=v"(t) : "v"(pair), "s"(vs_bits), "v"(acc));
+        if (high) asm("v_fma_mix_f32 %0, %1, %2, %3 op_sel:[1,0,0] op_sel_hi:[1,0,1]" : "=v"(t) : "v"(pair), "v"(vs), "v"(acc));
+        else      asm("v_fma_mix_f32 %0, %1, %2, %3 op_sel_hi:[1,0,1]" : "=v"(t) : "v"(pair), "v"(vs), "v"(acc));
         asm("v_cvt_f16_f32 %0, %1" : "=v"(acc) : "v"(t));
     };
-    struct chunk { u32x4 c[ROW_CHUNK / 8]; };              // 64 keys of this lane's d, two per register
-    auto read_chunk = [&](chunk & ch, const half_t * vbuf, int k0) __attribute__((always_inline)) {
-        const u32x4 * src = (const u32x4 *)(vbuf + lane * ROW_VT + k0);
+    constexpr int UNIT = 32;
+    struct unit { u32x4 v[UNIT / 8]; float4 f[UNIT / 4]; float fl; };
+    auto read_unit = [&](unit & u, int buf, int k0) __attribute__((always_inline)) {
+        const u32x4 * src = (const u32x4 *)(v_lds[buf] + lane * ROW_VT + k0);
 #pragma unroll
-        for (int i = 0; i < ROW_CHUNK / 8; ++i) ch.c[i] = src[i];
+        for (int i = 0; i < UNIT / 8; ++i) u.v[i] = src[i];
+        const float4 * fs = (const float4 *)(f_lds[buf] + k0);
+#pragma unroll
+        for (int i = 0; i < UNIT / 4; ++i) u.f[i] = fs[i];
+        u.fl = f_lds[buf][k0 + (lane & (UNIT - 1))];
     };
-    // f: the factor of key k0 + lane
-    auto run_chunk = [&](const chunk & ch, float f) __attribute__((always_inline)) {
-        const uint32_t f_l = __float_as_uint(f);
-        const uint64_t raised = __ballot((int32_t) f_l < 0);   // uniform: which of the 64 keys move the maximum (-ms, down to -0)
+    auto factor_of = [&](const unit & u, int j) __attribute__((always_inline)) {
+        const float4 & f4 = u.f[j >> 2];
+        return (j & 3) == 0 ? f4.x : (j & 3) == 1 ? f4.y : (j & 3) == 2 ? f4.z : f4.w;
+    };
+    auto run_unit = [&](const unit & u) __attribute__((always_inline)) {
+        const uint32_t raised = (uint32_t) __ballot((int32_t) __float_as_uint(u.fl) < 0);   // uniform: keys with -ms (down to -0)
         if (raised == 0) {
 #pragma unroll
-            for (int j = 0; j < ROW_CHUNK; ++j) mad(ch.c[j >> 3][(j >> 1) & 3], j & 1, __builtin_amdgcn_readlane(f_l, j));   // masked keys: vs = 0 leaves acc as it is
+            for (int j = 0; j < UNIT; ++j) mad(u.v[j >> 3][(j >> 1) & 3], j & 1, factor_of(u, j));   // masked keys: vs = 0 leaves acc as it is
         } else {
+            // rare after the first keys of a row: eight keys at a time, key by key only where one of the eight raises
 #pragma unroll
-            for (int j = 0; j < ROW_CHUNK; ++j) {
-                uint32_t fj = __builtin_amdgcn_readlane(f_l, j);
-                if ((raised >> j) & 1) {                   // scalar condition
-                    float t;
-                    asm("v_fma_mix_f32 %0, %1, %2, 0 op_sel_hi:[1,0,0]" : "=v"(t) : "v"(acc), "s"(fj ^ 0x80000000u));
-                    asm("v_cvt_f16_f32 %0, %1" : "=v"(acc) : "v"(t));
-                    fj = 0x3f800000u;                      // vs = 1
+            for (int g = 0; g < UNIT / 8; ++g) {
+                if (((raised >> (8 * g)) & 0xff) == 0) {
+#pragma unroll
+                    for (int j = 8 * g; j < 8 * g + 8; ++j) mad(u.v[g][(j >> 1) & 3], j & 1, factor_of(u, j));
+                } else {
+#pragma unroll
+                    for (int j = 8 * g; j < 8 * g + 8; ++j) {
+                        float fj = factor_of(u, j);
+                        if ((raised >> j) & 1) {           // scalar condition
+                            float t;
+                            asm("v_fma_mix_f32 %0, %1, %2, 0 op_sel_hi:[1,0,0]" : "=v"(t) : "v"(acc), "v"(-fj));
+                            asm("v_cvt_f16_f32 %0, %1" : "=v"(acc) : "v"(t));
+                            fj = 1.0f;                     // vs = 1
+                        }
+                        mad(u.v[g][(j >> 1) & 3], j & 1, fj);
+                    }
                 }
-                mad(ch.c[j >> 3][(j >> 1) & 3], j & 1, fj);
             }
         }
     };
 
+    // Three sets of registers go round the six units of a stage.  The last unit of a stage is walked after the barrier that
+    // opens the next one, under that stage's first LDS reads: its values are in registers by then, and the producers get
+    // the buffer a unit earlier.
     float S = 0.0f;
+    unit ua, ub, uc;
+    bool pending = false;                                  // uc holds the sixth unit of the stage before
     __syncthreads();                                       // stage 0 is scored
     for (int s = 0; s < n_stages; ++s) {
-        __syncthreads();                                   // stage s has its factors and its V rows; stage s - 1 is walked
+        __syncthreads();                                   // stage s has its factors and its V rows
         const int buf = s & 1;
         const int nk = min(ROW_STAGE, kv_pad - s * ROW_STAGE);                  // 64, 128 or 192
-        const half_t * vbuf = v_lds[buf];
-        chunk va, vn;
-        read_chunk(va, vbuf, 0);
-        const float f0 = f_lds[buf][lane];
-        const float f1 = nk > ROW_CHUNK ? f_lds[buf][ROW_CHUNK + lane] : 0.0f;
-        const float f2 = nk > 2 * ROW_CHUNK ? f_lds[buf][2 * ROW_CHUNK + lane] : 0.0f;
+        read_unit(ua, buf, 0);
 #pragma unroll
         for (int w = 0; w < 3; ++w) S = S * red_p[buf][w] + red_a[buf][w];
-        if (nk > ROW_CHUNK) read_chunk(vn, vbuf, ROW_CHUNK);
-        run_chunk(va, f0);
-        if (nk > ROW_CHUNK) {
-            if (nk > 2 * ROW_CHUNK) read_chunk(va, vbuf, 2 * ROW_CHUNK);
-            run_chunk(vn, f1);
-            if (nk > 2 * ROW_CHUNK) run_chunk(va, f2);
+        if (pending) run_unit(uc);
+        read_unit(ub, buf, UNIT);
+        run_unit(ua);
+        if (nk > 2 * UNIT) read_unit(uc, buf, 2 * UNIT);
+        run_unit(ub);
+        pending = false;
+        if (nk > 2 * UNIT) {
+            read_unit(ua, buf, 3 * UNIT);
+            run_unit(uc);
+            if (nk > 4 * UNIT) read_unit(ub, buf, 4 * UNIT);
+            run_unit(ua);
+            if (nk > 4 * UNIT) {
+                read_unit(uc, buf, 5 * UNIT);
+                run_unit(ub);
+                pending = true;
+            }
         }
     }
+    if (pending) run_unit(uc);
 
     half_t acc_h; { const uint16_t t16 = (uint16_t) acc; __builtin_memcpy(&acc_h, &t16, 2); }
     float * dp = (float *) a.d + ((i3 * a.N + n) * a.H + h) * FA_D;
