@@ -186,7 +186,10 @@ __device__ __forceinline__ float wave_scan_max(float v) {                      /
 // scores, the exponentials and the staging run beside it on the other three SIMDs, and no array grows with the number
 // of keys.
 __global__ void __launch_bounds__(256) k_fattn_seq_row(fa_args a, int kv_pad) {
-    __shared__ __attribute__((aligned(16))) half_t v_lds[2][FA_D * ROW_VT];   // V stage, transposed: [d][key]
+    // V stage, transposed: [d][key], in 16-byte pieces of eight keys.  Inside each run of 64 keys, piece p of row d sits at
+    // p ^ 2 (d / 16): the producers' 16-byte writes (lanes: 8 pieces of d x 2 pieces of keys) then cover all banks once, as
+    // the walker's reads do (16 consecutive d, one piece; the pitch is an odd number of pieces).
+    __shared__ __attribute__((aligned(16))) half_t v_lds[2][FA_D * ROW_VT];
     __shared__ __attribute__((aligned(16))) float f_lds[2][ROW_STAGE];       // one factor per key
     __shared__ float red_m[2][3], red_p[2][3], red_a[2][3];
 
@@ -301,7 +304,7 @@ __global__ void __launch_bounds__(256) k_fattn_seq_row(fa_args a, int kv_pad) {
                 // of each of its eight d-rows once the 8 x 8 block of halves is transposed in registers
                 {
                     const int key0 = (s - 1) * ROW_STAGE + pw * WAVE + 8 * r8;
-                    half_t * dst = v_lds[f] + (8 * c8) * ROW_VT + pw * WAVE + 8 * r8;
+                    half_t * dst = v_lds[f] + (8 * c8) * ROW_VT + pw * WAVE + 8 * (r8 ^ (2 * (c8 >> 1)));   // (swizzled, see v_lds)
 #pragma unroll
                     for (int e = 0; e < 8; ++e) {
                         u32x4 o;
@@ -342,10 +345,11 @@ __global__ void __launch_bounds__(256) k_fattn_seq_row(fa_args a, int kv_pad) {
     };
     constexpr int UNIT = 32;
     struct unit { u32x4 v[UNIT / 8]; float4 f[UNIT / 4]; float fl; };
-    auto read_unit = [&](unit & u, int buf, int k0) __attribute__((always_inline)) {
-        const u32x4 * src = (const u32x4 *)(v_lds[buf] + lane * ROW_VT + k0);
+    const int swz = 2 * (lane >> 4);                       // of this lane's row of the V stage
+    auto read_unit = [&](unit & u, int buf, int k0) __attribute__((always_inline)) {      // k0: a multiple of 32
+        const half_t * row = v_lds[buf] + lane * ROW_VT + (k0 & ~63);
 #pragma unroll
-        for (int i = 0; i < UNIT / 8; ++i) u.v[i] = src[i];
+        for (int i = 0; i < UNIT / 8; ++i) u.v[i] = *(const u32x4 *)(row + 8 * ((((k0 & 32) >> 3) + i) ^ swz));
         const float4 * fs = (const float4 *)(f_lds[buf] + k0);
 #pragma unroll
         for (int i = 0; i < UNIT / 4; ++i) u.f[i] = fs[i];
