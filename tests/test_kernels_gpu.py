@@ -400,7 +400,9 @@ def run_fa(pkg, gpu, q, kb, vb, mask, scale, mode):
 @pytest.mark.parametrize("case", [
     dict(H=2, N=70, KV=100), dict(H=3, N=200, KV=1536, flat=True, pad_from=1500), dict(H=20, N=5, KV=1536, flat=True, pad_from=1500),
     dict(H=4, N=1, KV=1), dict(H=4, N=5, KV=37, mask="beam"), dict(H=2, N=3, KV=200, mask="causal"), dict(H=2, N=100, KV=100, mask="causal"),
-    dict(H=2, N=8, KV=448, mask="beam"), dict(H=2, N=9, KV=63)])
+    dict(H=2, N=8, KV=448, mask="beam"), dict(H=2, N=9, KV=63),
+    # the few-query kernel's stages of 192 keys: exactly one, one key into the second, and far more keys than it ever staged at once
+    dict(H=2, N=1, KV=192), dict(H=2, N=4, KV=193, mask="beam"), dict(H=1, N=2, KV=7500)])
 def test_flash_attn_reference_faithful(pkg, oracle, gpu, case):
     H, N, KV = case["H"], case["N"], case["KV"]
     q, kb, vb = _attention_inputs(oracle, H, N, KV, case.get("flat", False), case.get("pad_from"))
