@@ -150,6 +150,25 @@ MI355X_API int    mi355x_mul_mat_group(const mi355x_mul_mat_item * items, int co
 MI355X_API int    mi355x_norm_mul_mat_group(const mi355x_tensor * src, const mi355x_tensor * normed, float eps, const float * w, const float * b,
                                             const mi355x_mul_mat_item * items, int count, void * workspace, size_t workspace_size, void * stream);
 
+/* The few-column product (ggml_compute_forward_mul_mat with ggml_vec_dot_q8_0_q8_0, ggml-cpu.c:1266-1458,
+ * ggml-cpu-quants.c:3597) over a Q8_0 matrix long enough to be a stream — the vocabulary projection — with the integer
+ * dot products on the matrix cores, from a copy of the matrix in the order those want: per 16 rows and pair of blocks,
+ * 1024 bytes of quants (lane l of v_mfma_i32_16x16x64_i8's B operand: row l % 16, block (l / 16) / 2 of the pair, half
+ * (l / 16) % 2) followed by the 32 f16 scales ([block of the pair][row]); rows padded to a multiple of 16 with zero
+ * blocks.  The same bytes as the block rows (68 per row and pair), the same integer sums and scales as the reference;
+ * a row's blocks are added up as two f32 sequences (even blocks, odd blocks) that are joined at the end.  No
+ * counterpart in the reference, which keeps one layout per type.
+ *   mi355x_q8_0_tiles_size    bytes of the copy for a [K, M] matrix (0: K is not a multiple of 64)
+ *   mi355x_q8_0_tiles_pack    src0: Q8_0 [K, M], 2-d, rows at 2-byte alignment -> `tiles` (16-byte aligned)
+ *   mi355x_mul_mat_q8_0_tiles dst[m, n] over `tiles`; src1: F32 [K, N <= 8], dst: F32 [M, N] (F16 with
+ *                             MI355X_EPI_OUT_F16); K one of 384, 512, 768, 1024, 1280 (else MI355X_ERR_UNSUPPORTED).
+ *                             `workspace` (16-byte aligned, N * K * 1.25 bytes rounded up to 256) receives the Q8_0 form of
+ *                             src1 unless MI355X_MM_WS_READY says it is there; MI355X_MM_PREPARE_ONLY stops after that. */
+MI355X_API size_t mi355x_q8_0_tiles_size(int64_t K, int64_t M);
+MI355X_API int    mi355x_q8_0_tiles_pack(const mi355x_tensor * src0, void * tiles, void * stream);
+MI355X_API int    mi355x_mul_mat_q8_0_tiles(const void * tiles, int64_t K, int64_t M, const mi355x_tensor * src1, const mi355x_tensor * dst,
+                                            int flags, void * workspace, size_t workspace_size, void * stream);
+
 /* FLASH_ATTN_EXT --------------------------------------------------------------------------------------
  * ggml_compute_forward_flash_attn_ext_f16 (ggml/src/ggml-cpu/ops.cpp:6638-6851), max_bias = 0 and
  * logit_softcap = 0 (the only values whisper uses):

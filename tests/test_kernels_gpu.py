@@ -123,6 +123,49 @@ def test_mul_mat_quantized(pkg, oracle, gpu, wtype, shape):
         assert oracle.nmse(alone if n * m * k <= 2e9 else alone[:, sel], want) <= 1e-10
 
 
+@pytest.mark.parametrize("shape", [(1280, 51866, 5), (1280, 2000, 8), (384, 1000, 1), (512, 47, 3), (768, 16, 2), (1024, 333, 7)])
+def test_mul_mat_q8_0_tiles(pkg, oracle, gpu, shape):
+    # the matrix-core form of the few-column product: the block rows repacked 16 rows x 2 blocks at a time
+    lib = pkg.kernels()
+    k, m, n = shape
+    blocks = oracle.quantize(pkg.Q8_0, rnd((m, k), 0.02))
+    x = rnd((n, k))
+    d_w, d_x = gpu.up(blocks), gpu.up(x)
+    tw, tx = pkg.tensor(d_w, pkg.Q8_0, ne=[k, m]), pkg.tensor(d_x, pkg.F32)
+    size = lib.mi355x_q8_0_tiles_size(k, m)
+    assert size == -(-m // 16) * (k // 64) * 1088
+    tiles = torch.full((size,), 0xAA, dtype=torch.uint8, device=gpu.dev)
+    pkg.check(lib.mi355x_q8_0_tiles_pack(tw, tiles.data_ptr(), gpu.stream))
+    # the repacked bytes: lane l of a (tile, step) holds 16 quants of row 16 tile + l % 16, block 2 step + l / 32, half (l / 16) % 2
+    img = gpu.down(tiles).reshape(-(-m // 16), k // 64, 1088)
+    rows = np.zeros((-(-m // 16) * 16, k // 32, 34), dtype=np.uint8)
+    rows[:m] = blocks.reshape(m, k // 32, 34)
+    rows = rows.reshape(-1, 16, k // 64, 2, 34)                                   # [tile][r][step][block of the pair][34]
+    quants = rows[..., 2:].reshape(rows.shape[0], 16, k // 64, 2, 2, 16)           # ... [half][16]
+    want_q = quants.transpose(0, 2, 3, 4, 1, 5).reshape(rows.shape[0], k // 64, 1024)   # [tile][step][g = 2 block + half][r][16]
+    assert np.array_equal(img[:, :, :1024], want_q)
+    want_d = rows[..., :2].transpose(0, 2, 3, 1, 4).reshape(rows.shape[0], k // 64, 64)  # [tile][step][block][r][2]
+    assert np.array_equal(img[:, :, 1024:], want_d)
+
+    need = n * k + n * (k // 32) * 8
+    ws = torch.zeros((need + 255) // 256 * 256, dtype=torch.uint8, device=gpu.dev)
+    d_y = torch.full((n, m), 7.0, dtype=torch.float32, device=gpu.dev)
+    pkg.check(lib.mi355x_mul_mat_q8_0_tiles(tiles.data_ptr(), k, m, tx, pkg.tensor(d_y, pkg.F32), 0, ws.data_ptr(), ws.numel(), gpu.stream))
+    got = gpu.down(d_y)
+    sel = np.r_[0:min(64, m), max(m - 64, 0):m] if n * m * k > 2e9 else np.arange(m)
+    want = oracle.mul_mat(pkg.Q8_0, blocks.reshape(m, -1)[sel], x)
+    assert oracle.nmse(got[:, sel], want) <= 1e-10          # the reference's integer sums and scales; f32 order of the blocks differs
+    # f16 output, over the activations already in the workspace
+    d_h = torch.zeros((n, m), dtype=torch.float16, device=gpu.dev)
+    d_x.zero_()
+    pkg.check(lib.mi355x_mul_mat_q8_0_tiles(tiles.data_ptr(), k, m, tx, pkg.tensor(d_h, pkg.F16), pkg.EPI_OUT_F16 | pkg.MM_WS_READY, ws.data_ptr(), ws.numel(), gpu.stream))
+    assert np.array_equal(gpu.down(d_h).view(np.uint16), oracle.f32_to_f16_bits(got))
+    # shapes and arguments it does not take
+    assert lib.mi355x_q8_0_tiles_size(96, 16) == 0
+    assert lib.mi355x_mul_mat_q8_0_tiles(tiles.data_ptr(), k, m, tx, pkg.tensor(d_y, pkg.F32), 0, None, 0, gpu.stream) == -3
+    assert lib.mi355x_mul_mat_q8_0_tiles(tiles.data_ptr(), 640, m, tx, pkg.tensor(d_y, pkg.F32), 0, ws.data_ptr(), ws.numel(), gpu.stream) == -1
+
+
 def test_gemv_over_activations_quantized_ahead(pkg, oracle, gpu):
     # MI355X_MM_PREPARE_ONLY leaves the quantized activations in the workspace; products over them pass MI355X_MM_WS_READY
     lib = pkg.kernels()

@@ -34,9 +34,13 @@ struct mi355x_device_ctx {
     std::string description;   // marketing name from the driver
 };
 
-// f16 image of a quantized weight tensor (rows of f16(d * q)), operand of the MFMA GEMM
+// A second form of a quantized weight tensor, kept beside it in HBM:
+//   MI355X_IMAGE_F16     rows of f16(d * q), operand of the MFMA GEMM
+//   MI355X_IMAGE_TILES   Q8_0 blocks in the order of mi355x_q8_0_tiles_pack, operand of the few-column product over a
+//                        matrix long enough to be a stream (the vocabulary projection)
+enum { MI355X_IMAGE_F16 = 0, MI355X_IMAGE_TILES = 1 };
 struct mi355x_weight_image {
-    void * f16;        // device memory, ne0 * ne1 halves
+    void * f16;        // device memory (F16: ne0 * ne1 halves)
     size_t src_bytes;  // bytes of the tensor it mirrors
     int    type;
     int64_t ne0, ne1;
@@ -49,11 +53,12 @@ struct mi355x_buffer_ctx {
     // Weight buffers keep, next to a Q5_0 / Q8_0 matrix that is multiplied with many columns at once, its f16 image:
     // 2 bytes per weight more HBM, so that the GEMM streams matrix-core operands instead of unpacking the same blocks
     // in every workgroup and on every call.  Keyed by the tensor's data address; anything that writes into the buffer
-    // drops the images it overlaps.
+    // drops the images it overlaps.  (Key: the address with the kind of image in its lowest bit — block rows start at
+    // even addresses.)
     std::mutex                               image_mutex;
     std::map<uintptr_t, mi355x_weight_image> images;
 
-    const void * weight_image(const struct ggml_tensor * w, hipStream_t stream);   // NULL: none could be made
+    const void * weight_image(const struct ggml_tensor * w, hipStream_t stream, int kind = MI355X_IMAGE_F16);   // NULL: none could be made
     void         drop_images(const void * begin, size_t size);
     void         drop_all_images();
 };

@@ -89,9 +89,10 @@ static bool upload(int device, void * dst, const void * src, size_t size) {
 // buffer  (ggml_backend_buffer_i, ggml-backend-impl.h:41-58)
 // ------------------------------------------------------------------------------------------------------
 
-const void * mi355x_buffer_ctx::weight_image(const struct ggml_tensor * w, hipStream_t stream) {
+const void * mi355x_buffer_ctx::weight_image(const struct ggml_tensor * w, hipStream_t stream, int kind) {
     std::lock_guard<std::mutex> lock(image_mutex);
-    const uintptr_t key = (uintptr_t) w->data;
+    if ((uintptr_t) w->data & 1) return nullptr;
+    const uintptr_t key = (uintptr_t) w->data | (uintptr_t) kind;
     auto it = images.find(key);
     if (it != images.end()) {
         const mi355x_weight_image & im = it->second;
@@ -101,13 +102,24 @@ const void * mi355x_buffer_ctx::weight_image(const struct ggml_tensor * w, hipSt
     }
     mi355x_weight_image im = { nullptr, ggml_nbytes(w), (int) w->type, w->ne[0], w->ne[1] };
     const int64_t n = w->ne[0] * w->ne[1];
-    if (hipMalloc(&im.f16, (size_t) n * 2) != hipSuccess || !im.f16) {
+    const size_t bytes = kind == MI355X_IMAGE_TILES ? mi355x_q8_0_tiles_size(w->ne[0], w->ne[1]) : (size_t) n * 2;
+    if (!bytes) return nullptr;
+    if (hipMalloc(&im.f16, bytes) != hipSuccess || !im.f16) {
         (void) hipGetLastError();
         static bool warned = false;
-        if (!warned) { warned = true; GGML_LOG_WARN("ggml-mi355x: no memory for the f16 image of %s (%.1f MiB); its blocks are unpacked on every call\n", w->name, n * 2 / 1048576.0); }
+        if (!warned) { warned = true; GGML_LOG_WARN("ggml-mi355x: no memory for the %s of %s (%.1f MiB); it is multiplied from its block rows\n", kind == MI355X_IMAGE_TILES ? "tiles" : "f16 image", w->name, bytes / 1048576.0); }
         return nullptr;
     }
-    if (mi355x_dequantize_row_f16((int) w->type, w->data, im.f16, n, stream) != MI355X_OK) { (void) hipFree(im.f16); return nullptr; }
+    int rc;
+    if (kind == MI355X_IMAGE_TILES) {
+        mi355x_tensor t = {};
+        t.data = w->data; t.type = (int) w->type;
+        for (int i = 0; i < 4; ++i) { t.ne[i] = w->ne[i]; t.nb[i] = w->nb[i]; }
+        rc = mi355x_q8_0_tiles_pack(&t, im.f16, stream);
+    } else {
+        rc = mi355x_dequantize_row_f16((int) w->type, w->data, im.f16, n, stream);
+    }
+    if (rc != MI355X_OK) { (void) hipFree(im.f16); return nullptr; }
     // The image is shared by every backend instance that uses these weights (whisper_full_parallel: one instance and one
     // stream per state), so it is complete before anyone can find it: once per weight matrix.
     if (hipStreamSynchronize(stream) != hipSuccess) { (void) hipGetLastError(); (void) hipFree(im.f16); return nullptr; }

@@ -269,7 +269,7 @@ struct graph_runner {
 
     // operand descriptors of a planned chain; a quantized weight matrix that meets many columns is replaced by its f16
     // image, kept beside it in HBM (then MI355X_MM_ACT_Q8_0 goes into `mm_flags`)
-    struct mm_operands { mi355x_tensor vw, vx, vd; int mm_flags; const char * kernel_name; };
+    struct mm_operands { mi355x_tensor vw, vx, vd; int mm_flags; const char * kernel_name; const void * tiles; };
     mm_operands describe(const mm_chain & c) const {
         mm_operands o;
         o.vw = to_view(c.w); o.vx = to_view(c.x); o.vd = to_view(c.mm);
@@ -290,6 +290,15 @@ struct graph_runner {
                 o.vw.nb[0] = 2; o.vw.nb[1] = 2 * (size_t) w->ne[0]; o.vw.nb[2] = o.vw.nb[1] * (size_t) w->ne[1]; o.vw.nb[3] = o.vw.nb[2];
                 o.mm_flags |= MI355X_MM_ACT_Q8_0;
             }
+        }
+        // the few-column product over a Q8_0 matrix of tens of MB (the logits over the vocabulary) reads a copy of it in
+        // matrix-core order
+        o.tiles = nullptr;
+        if (ctx->weight_images && w->type == GGML_TYPE_Q8_0 && nbytes_of(w) >= 32e6 && w->ne[2] == 1 && w->ne[3] == 1 && ggml_is_contiguous(w) &&
+            !w->view_src && w->buffer && w->buffer->usage == GGML_BACKEND_BUFFER_USAGE_WEIGHTS && mi355x_buffer_is_ours(w->buffer) &&
+            strcmp(o.kernel_name, "mul_mat.gemv_q8_0") == 0 && !(c.epi.flags & ~MI355X_EPI_OUT_F16) && c.x->type == GGML_TYPE_F32 &&
+            c.mm->ne[2] == 1 && c.mm->ne[3] == 1 && mi355x_q8_0_tiles_size(w->ne[0], w->ne[1]) > 0) {
+            o.tiles = ((mi355x_buffer_ctx *) w->buffer->context)->weight_image(w, ctx->stream, MI355X_IMAGE_TILES);
         }
         return o;
     }
@@ -462,6 +471,12 @@ struct graph_runner {
         }
         {
             launch_scope ls(ctx, scope, chain_bytes(c), chain_flops(c));
+            status = MI355X_ERR_UNSUPPORTED;
+            if (o.tiles && !key) {
+                status = mi355x_mul_mat_q8_0_tiles(o.tiles, c.w->ne[0], c.w->ne[1], &o.vx, &o.vd,
+                                                   epi.flags & (MI355X_EPI_OUT_F16 | MI355X_MM_WS_READY), ctx->ws, ctx->ws_size, ctx->stream);
+            }
+            if (status == MI355X_ERR_UNSUPPORTED)       // (a K the tiles kernel is not built for)
             status = mi355x_mul_mat(&o.vw, &o.vx, &o.vd, epi.flags ? &epi : nullptr, ctx->ws, ctx->ws_size, ctx->stream);
             if (key && status == MI355X_ERR_UNSUPPORTED) {          // shapes the epilogue cannot emit for: plain product
                 epi.flags &= ~MI355X_EPI_EMIT_F16; key = nullptr;

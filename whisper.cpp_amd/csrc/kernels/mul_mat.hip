@@ -16,6 +16,7 @@
 //   * k_mul_mat_generic — any strides / K; one wavefront per output row, f32 FMA.
 #include "common.h"
 #include <stdlib.h>
+#include <type_traits>
 
 typedef uint32_t __attribute__((aligned(2))) u32a2;
 struct __attribute__((packed, aligned(2))) u128a2 { uint32_t x, y, z, w; };
@@ -850,6 +851,138 @@ __device__ __forceinline__ void gemv_qr_rows(const mm_args & a, PRO prologue = P
 template <int T0, int NC, int LPR, int NB>
 __global__ void __launch_bounds__(256) k_gemv_qr(mm_args a) { gemv_qr_rows<T0, NC, LPR, NB>(a); }
 
+// ------------------------------------------------------------------------------------------------------
+// Q8_0 weights as tiles for the matrix cores: the product over a matrix long enough to be a stream (the vocabulary
+// projection: 70 MB a decode step)
+// ------------------------------------------------------------------------------------------------------
+// What holds the register kernel back on that matrix is its vector work — 40 v_dot4 per block for five columns — which
+// adds to the stream instead of hiding under it.  One v_mfma_i32_16x16x64_i8 takes 16 weight rows x two blocks (the B
+// operand: lane (r, g) holds 16 quants of row r — block g / 2 of the pair, half g % 2) against the activations of up
+// to eight columns (the A operand, in registers for the whole kernel).  The two blocks of a pair have scales of their
+// own, so their sums must not mix: column n sits in A row n with the first block's quants and zeros where the second's
+// would be, and in A row 8 + n the other way round.  Result row 4 g' + i then reaches lane (r, g') for the block whose
+// scale that lane loads (g' / 2), and what is left per lane and pair of blocks is four conversions, four scale
+// products and four f32 fused multiply-adds.  A row's blocks are therefore summed as two interleaved f32 sequences
+// (even blocks, odd blocks) that are added at the end.
+// Read from the block rows as ggml lays them out, that operand costs more than it saves: every load takes 16 bytes
+// from each of 16 rows, at 2-byte alignment, plus a 2-byte load per lane for the scale.  So the matrix is repacked once
+// into the order the instruction wants — per 16 rows and pair of blocks, 1024 bytes of quants in lane order followed by
+// the 32 scales (68 bytes a row, as before) — and every load of the stream is one aligned, contiguous run of a kilobyte.
+typedef int v4i_t __attribute__((ext_vector_type(4)));
+#define Q8T_STEP 1088      // bytes of 16 rows x one pair of blocks
+
+__global__ void k_q8_0_tiles_pack(const char * __restrict__ w, int64_t w_nb1, int64_t M, int ksteps, int64_t n_tiles, char * __restrict__ tiles) {
+    const int64_t i = (int64_t) blockIdx.x * blockDim.x + threadIdx.x;     // (tile, step, lane)
+    if (i >= n_tiles * ksteps * 64) return;
+    const int lane = (int)(i & 63), r = lane & 15, g = lane >> 4;
+    const int64_t ts = i >> 6, tile = ts / ksteps;
+    const int step = (int)(ts % ksteps);
+    const int64_t row = tile * 16 + r;
+    u32x4 q = { 0, 0, 0, 0 };
+    uint16_t d = 0;
+    if (row < M) {                                     // rows beyond the matrix: zero quants, zero scale
+        const char * b = w + row * w_nb1 + (int64_t)(2 * step + (g >> 1)) * 34;
+        const u128a2 t = *(const u128a2 *)(b + 2 + 16 * (g & 1));
+        q = (u32x4){ t.x, t.y, t.z, t.w };
+        d = *(const uint16_t *) b;
+    }
+    char * o = tiles + ts * Q8T_STEP;
+    *(u32x4 *)(o + lane * 16) = q;
+    if ((g & 1) == 0) *(uint16_t *)(o + 1024 + ((g >> 1) * 16 + r) * 2) = d;
+}
+
+// a.w: the tiles; a.x: the activations quantized ahead (layout of k_quantize_x_q8); K = 64 KSTEPS
+template <int KSTEPS>
+__global__ void __launch_bounds__(256, 2) k_gemv_q8_0_tiles(mm_args a) {
+    __shared__ __attribute__((aligned(16))) float xs_lds[KSTEPS * 2 * 8];       // activation scales, [block][column 0 .. 7]
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int r = lane & 15, g = lane >> 4;
+    const int nbk = KSTEPS * 2;
+    const int64_t n_tiles = (a.M + 15) / 16;
+    const int64_t stride = (int64_t) gridDim.x * 4;
+    int64_t tile = (int64_t) blockIdx.x * 4 + wave;
+    constexpr int H = KSTEPS / 2;
+    u32x4 wq[2][H]; uint32_t wd[2][H];
+    const int q_ofs = lane * 16, d_ofs = 1024 + ((g >> 1) * 16 + r) * 2;
+    auto request = [&](int half, int64_t t) __attribute__((always_inline)) {
+        const char * p = a.w + (t * KSTEPS + half * H) * Q8T_STEP;
+#pragma unroll
+        for (int s = 0; s < H; ++s) {
+            wq[half][s] = *(const u32x4 *)(p + s * Q8T_STEP + q_ofs);
+            wd[half][s] = *(const uint16_t *)(p + s * Q8T_STEP + d_ofs);
+        }
+    };
+    const bool live = tile < n_tiles;                   // (a matrix of fewer than 64 rows)
+    request(0, live ? tile : n_tiles - 1);
+    __builtin_amdgcn_sched_barrier(0);
+    request(1, live ? tile : n_tiles - 1);
+    __builtin_amdgcn_sched_barrier(0);
+
+    // activations: quants as the A operand (lane = A row r, 16 k of group g), scales through LDS
+    const char *  xq = a.x;
+    const float * xd = (const float *)(a.x + (size_t) a.N * a.K);
+    const int col = r & 7;
+    const bool mine = ((r < 8) == (g < 2)) && col < a.N;
+    v4i_t xa[KSTEPS];
+#pragma unroll
+    for (int s = 0; s < KSTEPS; ++s) {
+        xa[s] = (v4i_t){ 0, 0, 0, 0 };
+        if (mine) xa[s] = *(const v4i_t *)(xq + (int64_t) col * a.K + 64 * s + 16 * g);
+    }
+    for (int i = threadIdx.x; i < nbk * 8; i += 256) xs_lds[i] = (i & 7) < a.N ? xd[(i & 7) * nbk + (i >> 3)] : 0.0f;
+    __syncthreads();
+    if (!live) return;
+    const float * xsl = xs_lds + (g >> 1) * 8 + (g & 1) * 4;      // + 16 per pair of blocks
+    const bool out_f16 = a.e.flags & MI355X_EPI_OUT_F16;
+
+    auto do_tile = [&](auto again) __attribute__((always_inline)) {
+        float acc[4] = { 0.0f, 0.0f, 0.0f, 0.0f };
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+#pragma unroll
+            for (int s = 0; s < H; ++s) {
+                const u32x4 w = wq[half][s];
+                const v4i_t d = __builtin_amdgcn_mfma_i32_16x16x64_i8(xa[half * H + s], (v4i_t){ (int) w.x, (int) w.y, (int) w.z, (int) w.w }, (v4i_t){ 0, 0, 0, 0 }, 0, 0, 0);
+                const float dw = h2f((uint16_t) wd[half][s]);
+                const float4 x4 = *(const float4 *)(xsl + (half * H + s) * 16);
+                acc[0] += (float) d[0] * (dw * x4.x); acc[1] += (float) d[1] * (dw * x4.y);
+                acc[2] += (float) d[2] * (dw * x4.z); acc[3] += (float) d[3] * (dw * x4.w);
+            }
+            if constexpr (decltype(again)::value) {
+                request(half, tile + stride);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[i] += __shfl_xor(acc[i], 32, WAVE);     // even blocks + odd blocks
+        const int64_t row = tile * 16 + r;
+        if (g < 2 && row < a.M) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int n = 4 * g + i;
+                if (n < a.N) {
+                    if (out_f16) *(half_t *)(a.d + n * a.d_nb1 + row * 2) = (half_t) acc[i];
+                    else         *(float  *)(a.d + n * a.d_nb1 + row * 4) = acc[i];
+                }
+            }
+        }
+    };
+    // every tile but the wavefront's last requests the next one's halves as its own are used up
+    for (; tile + stride < n_tiles; tile += stride) do_tile(std::true_type{});
+    do_tile(std::false_type{});
+}
+
+template <int KSTEPS>
+static int launch_gemv_q8_0_tiles_k(const mm_args & a, hipStream_t st) {
+    const int64_t n_tiles = (a.M + 15) / 16;
+    const int64_t resident = 256 * 2 * 4;                 // wavefronts: two workgroups of four per CU
+    const int64_t rounds = (n_tiles + resident - 1) / resident;
+    const int64_t waves = (n_tiles + rounds - 1) / rounds;
+    k_gemv_q8_0_tiles<KSTEPS><<<(unsigned)(waves / 4 > 0 ? waves / 4 : 1), 256, 0, st>>>(a);
+    return launch_status();
+}
+static bool q8_0_tiles_k_ok(int64_t K) { return K == 384 || K == 512 || K == 768 || K == 1024 || K == 1280; }
+
 // several products over the same activations in one launch (a decode step's Q, K and V): blockIdx.y picks the matrix
 struct gemv_group_entry { const char * w; char * d; const float * bias; const char * residual; int64_t d_nb1; int flags; float scale; };
 #define GEMV_GROUP_MAX 8
@@ -1301,6 +1434,56 @@ extern "C" int mi355x_mul_mat_group(const mi355x_mul_mat_item * items, int count
     if (flags & MI355X_MM_PREPARE_ONLY) return launch_status();
     const int64_t blocks22 = ((a.N + 127) / 128) * ((a.M + 127) / 128) * count;
     return blocks22 >= 300 ? launch_gemm_f16_group<2, 2>(a, grp, count, st) : launch_gemm_f16_group<2, 1>(a, grp, count, st);
+}
+
+extern "C" size_t mi355x_q8_0_tiles_size(int64_t K, int64_t M) {
+    if (K <= 0 || M <= 0 || K % 64 != 0) return 0;
+    return (size_t)((M + 15) / 16) * (size_t)(K / 64) * Q8T_STEP;
+}
+
+extern "C" int mi355x_q8_0_tiles_pack(const mi355x_tensor * src0, void * tiles, void * stream) {
+    if (!src0 || !tiles) return MI355X_ERR_INVALID;
+    if (src0->type != MI355X_TYPE_Q8_0 || src0->ne[2] != 1 || src0->ne[3] != 1 || src0->nb[0] != 34) return MI355X_ERR_UNSUPPORTED;
+    const int64_t K = src0->ne[0], M = src0->ne[1];
+    if (K <= 0 || M <= 0 || K % 64 != 0 || (uintptr_t) src0->data % 2 != 0 || src0->nb[1] % 2 != 0 || (uintptr_t) tiles % 16 != 0) return MI355X_ERR_UNSUPPORTED;
+    const int64_t n_tiles = (M + 15) / 16, threads = n_tiles * (K / 64) * 64;
+    if ((threads + 255) / 256 > 0x7fffffff) return MI355X_ERR_UNSUPPORTED;
+    k_q8_0_tiles_pack<<<(unsigned)((threads + 255) / 256), 256, 0, (hipStream_t) stream>>>((const char *) src0->data, (int64_t) src0->nb[1], M, (int)(K / 64), n_tiles, (char *) tiles);
+    return launch_status();
+}
+
+extern "C" int mi355x_mul_mat_q8_0_tiles(const void * tiles, int64_t K, int64_t M, const mi355x_tensor * src1, const mi355x_tensor * dst,
+                                         int flags, void * workspace, size_t workspace_size, void * stream) {
+    if (!tiles || !src1 || !dst) return MI355X_ERR_INVALID;
+    if (!q8_0_tiles_k_ok(K) || M <= 0 || (uintptr_t) tiles % 16 != 0) return MI355X_ERR_UNSUPPORTED;
+    if (flags & ~(MI355X_EPI_OUT_F16 | MI355X_MM_WS_READY | MI355X_MM_PREPARE_ONLY)) return MI355X_ERR_UNSUPPORTED;
+    const int td = (flags & MI355X_EPI_OUT_F16) ? MI355X_TYPE_F16 : MI355X_TYPE_F32;
+    const int64_t N = src1->ne[1];
+    if (src1->type != MI355X_TYPE_F32 || dst->type != td || src1->nb[0] != 4 || dst->nb[0] != type_size(td)) return MI355X_ERR_UNSUPPORTED;
+    if (src1->ne[0] != K || dst->ne[0] != M || dst->ne[1] != N) return MI355X_ERR_INVALID;
+    if (N < 1 || N > MI355X_GEMV_MAX_COLS || src1->ne[2] != 1 || src1->ne[3] != 1 || dst->ne[2] != 1 || dst->ne[3] != 1 || !aligned16(src1)) return MI355X_ERR_UNSUPPORTED;
+    const size_t need = round256((size_t)(N * K + N * (K / QK) * 8));
+    if (!workspace || workspace_size < need || (uintptr_t) workspace % 16 != 0) return MI355X_ERR_WORKSPACE;
+    hipStream_t st = (hipStream_t) stream;
+    if (!(flags & MI355X_MM_WS_READY)) {
+        k_quantize_x_q8<<<(unsigned)((N * (K / 4) + 255) / 256), 256, 0, st>>>((const char *) src1->data, (int64_t) src1->nb[1], K, N, (char *) workspace);
+        if (const int rc = launch_status()) return rc;
+    }
+    if (flags & MI355X_MM_PREPARE_ONLY) return MI355X_OK;
+    mm_args a;
+    a.K = K; a.M = M; a.N = N;
+    a.w = (const char *) tiles; a.x = (const char *) workspace; a.d = (char *) dst->data;
+    a.w_nb1 = a.w_nb2 = a.w_nb3 = 0; a.x_nb1 = a.x_nb2 = a.x_nb3 = 0;
+    a.d_nb1 = dst->nb[1]; a.d_nb2 = a.d_nb3 = 0;
+    a.ne12 = a.ne13 = a.r2 = a.r3 = 1;
+    a.e.flags = flags & MI355X_EPI_OUT_F16; a.e.scale = 1.0f; a.e.bias = nullptr; a.e.residual = nullptr; a.e.gelu = nullptr; a.e.image = nullptr;
+    switch (K) {
+        case 384:  return launch_gemv_q8_0_tiles_k<6>(a, st);
+        case 512:  return launch_gemv_q8_0_tiles_k<8>(a, st);
+        case 768:  return launch_gemv_q8_0_tiles_k<12>(a, st);
+        case 1024: return launch_gemv_q8_0_tiles_k<16>(a, st);
+        default:   return launch_gemv_q8_0_tiles_k<20>(a, st);
+    }
 }
 
 extern "C" int mi355x_dequantize_row_f16(int type, const void * src, void * dst, int64_t k, void * stream) {
