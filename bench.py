@@ -143,7 +143,7 @@ def main() -> int:
               "steps_per_s": round(dec["steps_per_s"], 1), "beam_tokens_per_s": round(dec["batch_tokens_per_s"], 1)}
     if gemv:
         decode["gemv_roofline"] = kernel_roofline(gemv_name, gemv)
-        decode["gemv_roofline"]["traffic"] = round(70.7e6 + 1.3e6)
+        decode["gemv_roofline"]["traffic"] = round(72.8e6 + 3.2e6)    # FETCH_SIZE + WRITE_SIZE per launch of k_gemv_q8_0_tiles (profiles/)
     for small in ("mul_mat.gemv_q8_0", "norm_mul_mat.gemv"):
         if dk.get(small):
             # the products over 1.7 ... 7 MB matrices: over in the launch-to-store latency of a small kernel
