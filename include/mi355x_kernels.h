@@ -253,6 +253,21 @@ MI355X_API int mi355x_im2col_1d(const mi355x_tensor * src, const mi355x_tensor *
 /* CONCAT along `dim` (ggml/src/ggml-cpu/ops.cpp:2575).  F32. */
 MI355X_API int mi355x_concat(const mi355x_tensor * src0, const mi355x_tensor * src1, const mi355x_tensor * dst, int dim, void * stream);
 
+/* Log-mel front end -----------------------------------------------------------------------------------
+ * log_mel_spectrogram (src/whisper.cpp:3181-3270; worker :3113-3179; tables and transform :3008-3111), the step
+ * whisper_pcm_to_mel (:3881) runs on host threads before the encoder: 16 kHz f32 samples -> mel f32 [n_mel][n_len],
+ * n_len = (n_samples + 480000) / 160, ready for whisper_set_mel.  The signal is extended by 200 reflected samples in
+ * front and 30 s + 200 samples of zeros behind; 400-sample frames every 160 samples under the periodic Hann window;
+ * power of bins 0 .. 200 of each frame's transform; filter bank `filters` [n_mel][201] (the model file's);
+ * log10(max(., 1e-10)); values below (global maximum - 8) raised to it; (x + 4) / 4.  The transform is evaluated as
+ * direct sums in f64 where the reference runs an f32 halving scheme: results agree with it to its own rounding
+ * (about 1e-5 absolute on the output's range of roughly [-1, 1.5]), not bitwise.
+ * All pointers are device memory; n_samples > 200; n_mel <= 128; workspace 16-byte aligned. */
+MI355X_API int64_t mi355x_log_mel_n_len(int64_t n_samples);
+MI355X_API size_t  mi355x_log_mel_workspace_size(int n_mel);          /* 0: n_mel out of range */
+MI355X_API int     mi355x_log_mel_spectrogram(const float * samples, int64_t n_samples, const float * filters, int n_mel, float * mel,
+                                              void * workspace, size_t workspace_size, void * stream);
+
 /* Fill `n` bytes at `dst` with `value` through a kernel (safe inside HIP graph capture). */
 MI355X_API int mi355x_fill_bytes(void * dst, uint8_t value, size_t n, void * stream);
 

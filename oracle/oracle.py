@@ -210,3 +210,35 @@ def nmse(got, want) -> float:
     den = float(np.sum(want * want))
     num = float(np.sum((got - want) ** 2))
     return num / den if den > 0 else (0.0 if num == 0 else float("inf"))
+
+
+def log_mel_spectrogram(samples, filters) -> np.ndarray:
+    """samples f32 [n] at 16 kHz, filters f32 [n_mel, 201] -> mel f32 [n_mel, (n + 480000) // 160]"""
+    s = _f32(samples).ravel()
+    f = _f32(filters)
+    assert s.size > 200 and f.ndim == 2 and f.shape[1] == 201
+    L = lib()
+    L.oracle_log_mel_n_len.restype = C.c_int64
+    L.oracle_log_mel_spectrogram.restype = C.c_int64
+    n_len = L.oracle_log_mel_n_len(C.c_int64(s.size))
+    mel = np.empty((f.shape[0], n_len), dtype=np.float32)
+    got = L.oracle_log_mel_spectrogram(_p(s), C.c_int64(s.size), _p(f), C.c_int(f.shape[0]), _p(mel))
+    assert got == n_len
+    return mel
+
+
+def mel_filter_bank(n_mel: int, n_fft: int = 400, sample_rate: int = 16000) -> np.ndarray:
+    """A triangular filter bank on the mel scale with area normalization, [n_mel, n_fft // 2 + 1] f32: synthetic test
+    input of the kind a model file carries (the checks do not depend on its exact values)."""
+    def hz_to_mel(f):
+        return 2595.0 * np.log10(1.0 + np.asarray(f, dtype=np.float64) / 700.0)
+    def mel_to_hz(m):
+        return 700.0 * (10.0 ** (np.asarray(m, dtype=np.float64) / 2595.0) - 1.0)
+    freqs = np.linspace(0.0, sample_rate / 2, n_fft // 2 + 1)
+    edges = mel_to_hz(np.linspace(hz_to_mel(0.0), hz_to_mel(sample_rate / 2), n_mel + 2))
+    bank = np.zeros((n_mel, freqs.size))
+    for j in range(n_mel):
+        lo, mid, hi = edges[j], edges[j + 1], edges[j + 2]
+        up, down = (freqs - lo) / (mid - lo), (hi - freqs) / (hi - mid)
+        bank[j] = np.maximum(0.0, np.minimum(up, down)) * 2.0 / (hi - lo)
+    return bank.astype(np.float32)

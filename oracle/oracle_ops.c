@@ -413,3 +413,104 @@ void oracle_get_rows(int type, const void * table, const int32_t * ids, float * 
         }
     }
 }
+
+/* ---------------------------------------------------------------------------------------------------------
+ * Log-mel front end (log_mel_spectrogram and its worker, src/whisper.cpp:3113-3270; tables :3008-3045; the
+ * transform :3049-3111): samples f32 [n_samples] at 16 kHz -> mel f32 [n_mel][n_len], n_len = (n_samples +
+ * 480000) / 160.  The signal is extended by 200 reflected samples in front and 30 s + 200 samples of zeros
+ * behind; frame i is 400 samples from 160 i under a periodic Hann window; its 400-point transform is taken
+ * by halving down to 25 points (25-point sums over a 400-entry f32 sine / cosine table, then four rounds of
+ * butterflies), all in f32 in the order below; power of bins 0 .. 200; filter bank [n_mel][201] with the
+ * products added in fours in f32 and the fours in f64; log10(max(., 1e-10)); finally everything below
+ * (global maximum - 8) is raised to it and the result is (x + 4) / 4.
+ * Pinned in tests/test_golden.py against vectors written by the reference's compiled function
+ * (oracle/ref_mel_shim.cpp) and in tests/test_oracle.py against numpy's float64 rfft.
+ * ------------------------------------------------------------------------------------------------------- */
+#define MEL_NFFT 400
+#define MEL_HOP  160
+
+static float mel_sin[MEL_NFFT], mel_cos[MEL_NFFT], mel_hann[MEL_NFFT];
+static int   mel_tables_ready = 0;
+
+static void mel_tables(void) {
+    if (mel_tables_ready) return;
+    for (int i = 0; i < MEL_NFFT; ++i) {
+        const double theta = (2 * M_PI * i) / MEL_NFFT;
+        mel_sin[i] = sinf((float) theta);
+        mel_cos[i] = cosf((float) theta);
+        mel_hann[i] = (float)(0.5 * (1.0 - (double) cosf((float)((2.0 * M_PI * i) / MEL_NFFT))));
+    }
+    mel_tables_ready = 1;
+}
+
+/* transform of x[0], x[stride], ..., n points, into re[0 .. n), im[0 .. n); `tmp` holds 4 n floats */
+static void mel_transform(const float * x, int stride, int n, float * re, float * im, float * tmp) {
+    const int step = MEL_NFFT / n;
+    if (n == 1) { re[0] = x[0]; im[0] = 0.0f; return; }
+    if (n % 2 == 1) {
+        for (int k = 0; k < n; ++k) {
+            float sr = 0.0f, si = 0.0f;
+            for (int j = 0; j < n; ++j) {
+                const int idx = (k * j * step) % MEL_NFFT;
+                sr += x[j * stride] * mel_cos[idx];
+                si -= x[j * stride] * mel_sin[idx];
+            }
+            re[k] = sr; im[k] = si;
+        }
+        return;
+    }
+    const int h = n / 2;
+    float * er = tmp, * ei = tmp + h, * orr = tmp + 2 * h, * oi = tmp + 3 * h;
+    mel_transform(x,          2 * stride, h, er,  ei, tmp + 4 * h);
+    mel_transform(x + stride, 2 * stride, h, orr, oi, tmp + 4 * h);
+    for (int k = 0; k < h; ++k) {
+        const float c = mel_cos[k * step], s = -mel_sin[k * step];
+        re[k]     = er[k] + c * orr[k] - s * oi[k];
+        im[k]     = ei[k] + c * oi[k]  + s * orr[k];
+        re[k + h] = er[k] - c * orr[k] + s * oi[k];
+        im[k + h] = ei[k] - c * oi[k]  - s * orr[k];
+    }
+}
+
+int64_t oracle_log_mel_n_len(int64_t n_samples) { return (n_samples + 480000) / MEL_HOP; }
+
+/* returns n_len; mel must hold n_mel * n_len floats; n_samples > 200 */
+int64_t oracle_log_mel_spectrogram(const float * samples, int64_t n_samples, const float * filters, int n_mel, float * mel) {
+    mel_tables();
+    const int     n_bins = MEL_NFFT / 2 + 1;
+    const int64_t n_pad  = n_samples + 480000 + MEL_NFFT, n_len = (n_pad - MEL_NFFT) / MEL_HOP;
+    const int64_t n_eff  = n_samples + MEL_NFFT / 2;
+    float * padded = (float *) calloc((size_t) n_pad, sizeof(float));
+    for (int q = 0; q < MEL_NFFT / 2; ++q) padded[q] = samples[MEL_NFFT / 2 - q];
+    memcpy(padded + MEL_NFFT / 2, samples, (size_t) n_samples * sizeof(float));
+    int64_t n_frames = n_eff / MEL_HOP + 1;
+    if (n_frames > n_len) n_frames = n_len;
+    float frame[MEL_NFFT], re[MEL_NFFT], im[MEL_NFFT], tmp[2 * 4 * MEL_NFFT], power[MEL_NFFT / 2 + 1];
+    for (int64_t i = 0; i < n_len; ++i) {
+        if (i >= n_frames) {
+            for (int j = 0; j < n_mel; ++j) mel[(int64_t) j * n_len + i] = (float) log10(1e-10);
+            continue;
+        }
+        const int64_t off = i * MEL_HOP;
+        for (int j = 0; j < MEL_NFFT; ++j) frame[j] = off + j < n_eff ? mel_hann[j] * padded[off + j] : 0.0f;
+        mel_transform(frame, 1, MEL_NFFT, re, im, tmp);
+        for (int k = 0; k < n_bins; ++k) power[k] = re[k] * re[k] + im[k] * im[k];
+        for (int j = 0; j < n_mel; ++j) {
+            const float * f = filters + (int64_t) j * n_bins;
+            double sum = 0.0;
+            int k = 0;
+            for (; k < n_bins - 3; k += 4) sum += power[k] * f[k] + power[k + 1] * f[k + 1] + power[k + 2] * f[k + 2] + power[k + 3] * f[k + 3];
+            for (; k < n_bins; ++k) sum += power[k] * f[k];
+            mel[(int64_t) j * n_len + i] = (float) log10(sum > 1e-10 ? sum : 1e-10);
+        }
+    }
+    free(padded);
+    double mmax = -1e20;
+    for (int64_t i = 0; i < n_mel * n_len; ++i) if (mel[i] > mmax) mmax = mel[i];
+    mmax -= 8.0;
+    for (int64_t i = 0; i < n_mel * n_len; ++i) {
+        if (mel[i] < mmax) mel[i] = (float) mmax;
+        mel[i] = (float)((mel[i] + 4.0) / 4.0);
+    }
+    return n_len;
+}

@@ -194,3 +194,26 @@ class Graph:
 
     def __exit__(self, *exc):
         self.close()
+
+
+# --- the reference's log-mel front end (oracle/ref_mel_shim.cpp -> oracle/_ref/libref_mel.so) ----------------------
+
+def log_mel_available() -> bool:
+    return (REF_DIR / "libref_mel.so").exists()
+
+
+_mel_lib = None
+
+
+def log_mel_spectrogram(samples: np.ndarray, filters: np.ndarray, n_threads: int = 4) -> np.ndarray:
+    """log_mel_spectrogram (src/whisper.cpp:3181-3270) on f32 samples and a [n_mel, 201] filter bank -> [n_mel, n_len]"""
+    global _mel_lib
+    if _mel_lib is None:
+        _mel_lib = C.CDLL(str(REF_DIR / "libref_mel.so"))
+    s = np.ascontiguousarray(samples, dtype=np.float32).ravel()
+    f = np.ascontiguousarray(filters, dtype=np.float32)
+    n_len = C.c_int()
+    assert _mel_lib.ref_log_mel_spectrogram(_ptr(s), C.c_int(s.size), _ptr(f), C.c_int(f.shape[0]), C.c_int(n_threads), None, C.c_int(0), C.byref(n_len), None) == 0
+    out = np.empty((f.shape[0], n_len.value), dtype=np.float32)
+    assert _mel_lib.ref_log_mel_spectrogram(_ptr(s), C.c_int(s.size), _ptr(f), C.c_int(f.shape[0]), C.c_int(n_threads), _ptr(out), C.c_int(out.size), None, None) == 0
+    return out

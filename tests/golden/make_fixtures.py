@@ -102,5 +102,39 @@ def main() -> None:
     print(f"wrote {len(out)} arrays, {total / 1024:.0f} KiB uncompressed")
 
 
+def mel_signal(n: int, seed: int) -> np.ndarray:
+    """tones, a chirp, a click and noise: energy in every part of the band, frames of very different level"""
+    r = np.random.default_rng(seed)
+    t = np.arange(n) / 16000.0
+    s = 0.3 * np.sin(2 * np.pi * 440.0 * t) + 0.1 * np.sin(2 * np.pi * (500.0 + 9000.0 * t) * t) + 0.01 * r.normal(size=n)
+    s[n // 3] += 0.9
+    s[: n // 8] *= 1e-3
+    return s.astype(np.float32)
+
+
+def write_log_mel() -> None:
+    """tests/golden/log_mel_vectors.npz: the reference's log-mel front end on two short signals.  Frames beyond the
+    signal all hold one value, so only the leading frames and that value are kept."""
+    assert ref.log_mel_available(), "build oracle/_ref first (make -C oracle)"
+    sys.path.insert(0, str(HERE.parent.parent / "oracle"))
+    import oracle
+    out = {}
+    for name, n, n_mel, seed in (("a", 16000 + 123, 80, 7), ("b", 8000 + 1, 128, 8)):
+        s = mel_signal(n, seed)
+        f = oracle.mel_filter_bank(n_mel)
+        mel = ref.log_mel_spectrogram(s, f)
+        keep = (n + 200) // 160 + 9
+        assert np.all(mel[:, keep:] == mel[:, keep: keep + 1])
+        out[f"mel_{name}_samples"] = s
+        out[f"mel_{name}_filters"] = f
+        out[f"mel_{name}_head"] = mel[:, :keep].copy()
+        out[f"mel_{name}_tail_value"] = mel[:, keep].copy()
+        out[f"mel_{name}_n_len"] = np.int64(mel.shape[1])
+    np.savez_compressed(HERE / "log_mel_vectors.npz", **out)
+    print(f"wrote log_mel_vectors.npz: {sum(v.nbytes for v in out.values()) / 1024:.0f} KiB uncompressed")
+
+
 if __name__ == "__main__":
-    main()
+    if "--log-mel-only" not in sys.argv:
+        main()
+    write_log_mel()

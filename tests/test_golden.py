@@ -48,3 +48,30 @@ def test_norm_gelu_soft_max(oracle, vec):
     assert oracle.nmse(oracle.norm(vec["norm_x"], 1e-5), vec["norm_y"]) <= 1e-12
     assert np.array_equal(oracle.gelu(vec["gelu_x"]), vec["gelu_y"])
     assert oracle.nmse(oracle.soft_max(vec["soft_max_x"], None, float(vec["soft_max_scale"])), vec["soft_max_y"]) <= 1e-12
+
+
+# ------------------------------------------------------------------------------------------------------------------
+# log-mel front end: tests/golden/log_mel_vectors.npz, written by the reference's compiled log_mel_spectrogram
+# ------------------------------------------------------------------------------------------------------------------
+
+MEL_GOLDEN = Path(__file__).resolve().parent / "golden" / "log_mel_vectors.npz"
+
+
+def mel_cases():
+    v = np.load(MEL_GOLDEN, allow_pickle=False)
+    for name in ("a", "b"):
+        head, tail = v[f"mel_{name}_head"], v[f"mel_{name}_tail_value"]
+        want = np.empty((head.shape[0], int(v[f"mel_{name}_n_len"])), dtype=np.float32)
+        want[:, :head.shape[1]] = head
+        want[:, head.shape[1]:] = tail[:, None]
+        yield name, v[f"mel_{name}_samples"], v[f"mel_{name}_filters"], want
+
+
+@pytest.mark.parametrize("case", list(mel_cases()), ids=lambda c: c[0])
+def test_log_mel_spectrogram(oracle, case):
+    _, samples, filters, want = case
+    got = oracle.log_mel_spectrogram(samples, filters)
+    assert got.shape == want.shape
+    # the restatement keeps the reference's f32 operation order (it was bit-equal where the vectors were written);
+    # libm's sinf / cosf / log10 are the only parts that may differ between machines
+    assert np.max(np.abs(got - want)) <= 1e-6

@@ -769,3 +769,65 @@ def test_golden_norm_gelu_soft_max(pkg, oracle, gpu, vec):
 def test_smoke_entry_point():
     import __graft_entry__ as entry
     entry.smoke()
+
+
+# ------------------------------------------------------------------------------------------------------------------
+# log-mel front end
+# ------------------------------------------------------------------------------------------------------------------
+
+def run_log_mel(pkg, gpu, samples, filters):
+    lib = pkg.kernels()
+    d_s, d_f = gpu.up(samples), gpu.up(filters)
+    n_mel, n_len = filters.shape[0], lib.mi355x_log_mel_n_len(samples.size)
+    d_mel = torch.full((n_mel, n_len), 99.0, dtype=torch.float32, device=gpu.dev)
+    ws = torch.empty(lib.mi355x_log_mel_workspace_size(n_mel), dtype=torch.uint8, device=gpu.dev)
+    pkg.check(lib.mi355x_log_mel_spectrogram(d_s.data_ptr(), samples.size, d_f.data_ptr(), n_mel, d_mel.data_ptr(), ws.data_ptr(), ws.numel(), gpu.stream), "log_mel")
+    return gpu.down(d_mel)
+
+
+def mel_test_signal(n, seed):
+    r = np.random.default_rng(seed)
+    t = np.arange(n) / 16000.0
+    s = 0.3 * np.sin(2 * np.pi * 440.0 * t) + 0.1 * np.sin(2 * np.pi * (300.0 + 2000.0 * t) * t) + 0.01 * r.normal(size=n)
+    s[: n // 5] *= 1e-2
+    return s.astype(np.float32)
+
+
+# Tolerance: the kernel evaluates the transform in f64, the reference in f32 (halving scheme); on the output's scale
+# ((log10 power + 4) / 4, values in about [-1, 1.5]) the two agree to 1e-4 absolute, NMSE <= 1e-8.
+@pytest.mark.parametrize("n,n_mel", [(201, 80), (16000 + 123, 80), (8001, 128), (160 * 16 * 7 - 200, 128), (480000, 128), (480000, 80)])
+def test_log_mel_against_the_oracle(pkg, oracle, gpu, n, n_mel):
+    s, f = mel_test_signal(n, n), oracle.mel_filter_bank(n_mel)
+    got, want = run_log_mel(pkg, gpu, s, f), oracle.log_mel_spectrogram(s, f)
+    assert got.shape == want.shape == (n_mel, (n + 480000) // 160)
+    assert np.max(np.abs(got - want)) <= 1e-4
+    assert oracle.nmse(got, want) <= 1e-8
+
+
+def test_log_mel_golden_vectors(pkg, gpu):
+    from test_golden import mel_cases
+    for _, samples, filters, want in mel_cases():
+        got = run_log_mel(pkg, gpu, samples, filters)
+        assert got.shape == want.shape
+        assert np.max(np.abs(got - want)) <= 1e-4
+
+
+def test_log_mel_properties_and_arguments(pkg, oracle, gpu):
+    lib = pkg.kernels()
+    f = oracle.mel_filter_bank(80)
+    s = mel_test_signal(48000, 3)
+    a = run_log_mel(pkg, gpu, s, f)
+    # scaling the signal shifts log10 power by a constant before the clamp: (x + 4) / 4 moves by log10(g^2) / 4 everywhere
+    b = run_log_mel(pkg, gpu, (s * 4.0).astype(np.float32), f)
+    assert np.max(np.abs((b - a) - np.log10(16.0) / 4.0)) <= 1e-5
+    # the same call twice gives the same bits (the maximum is the only value formed by atomics, and a maximum has no order)
+    assert np.array_equal(a.view(np.uint32), run_log_mel(pkg, gpu, s, f).view(np.uint32))
+    # silence: every value is the clamp floor of the reference, (log10(1e-10) + 4) / 4
+    z = run_log_mel(pkg, gpu, np.zeros(4000, dtype=np.float32), f)
+    assert np.all(z == np.float32(-1.5))
+    # arguments it does not take
+    d = torch.zeros(1024, dtype=torch.float32, device=gpu.dev)
+    assert lib.mi355x_log_mel_workspace_size(129) == 0 and lib.mi355x_log_mel_n_len(480000) == 6000
+    assert lib.mi355x_log_mel_spectrogram(d.data_ptr(), 200, d.data_ptr(), 80, d.data_ptr(), d.data_ptr(), 4096, gpu.stream) == -2
+    assert lib.mi355x_log_mel_spectrogram(d.data_ptr(), 1000, d.data_ptr(), 129, d.data_ptr(), d.data_ptr(), 4096, gpu.stream) == -1
+    assert lib.mi355x_log_mel_spectrogram(d.data_ptr(), 1000, d.data_ptr(), 80, d.data_ptr(), None, 0, gpu.stream) == -3

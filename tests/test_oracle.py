@@ -313,3 +313,49 @@ def test_scale_softmax_im2col_get_rows(oracle, ref):
         with ref.Graph() as g:
             want = g.run(g.op("ggml_get_rows", g.tensor(t, blocks, ne=[64, 20]), g.tensor(ref.I32, ids)), out_shape=(4, 64))
         assert np.array_equal(got, want)
+
+
+# ------------------------------------------------------------------------------------------------------------------
+# log-mel front end
+# ------------------------------------------------------------------------------------------------------------------
+
+def mel_closed_form(samples, filters):
+    """the same quantity from numpy's float64 rfft, with none of the reference's structure"""
+    s = np.asarray(samples, dtype=np.float64)
+    padded = np.concatenate([s[200:0:-1], s, np.zeros(480000 + 200)])
+    n_len = (s.size + 480000) // 160
+    idx = 160 * np.arange(n_len)[:, None] + np.arange(400)[None, :]
+    window = 0.5 * (1.0 - np.cos(2.0 * np.pi * np.arange(400) / 400.0))
+    power = np.abs(np.fft.rfft(padded[idx] * window, axis=1)) ** 2            # [n_len, 201]
+    mel = np.log10(np.maximum(np.asarray(filters, dtype=np.float64) @ power.T, 1e-10))
+    mel = np.maximum(mel, mel.max() - 8.0)
+    return (mel + 4.0) / 4.0
+
+
+def test_log_mel_against_float64_rfft(oracle):
+    n = 16000 + 321
+    t = np.arange(n) / 16000.0
+    s = (0.25 * np.sin(2 * np.pi * 1000.0 * t) + 0.05 * RNG.normal(size=n)).astype(np.float32)
+    f = oracle.mel_filter_bank(80)
+    got, want = oracle.log_mel_spectrogram(s, f), mel_closed_form(s, f)
+    assert got.shape == want.shape == (80, (n + 480000) // 160)
+    # f32 transform against f64: the noise floor keeps every band well above the f32 rounding of the strongest one
+    assert np.max(np.abs(got - want)) <= 2e-4
+    # frames beyond the signal hold the clamp value; the band of the tone holds the maximum
+    assert np.all(got[:, 110:] == got[0, 200])
+    band = int(np.argmax(f[:, 25]))                       # bin 25 = 1000 Hz
+    assert int(np.argmax(got[:, 50])) == band
+    assert np.isclose(got.max(), (np.log10((f.astype(np.float64) @ (np.abs(np.fft.rfft(np.concatenate([s[200:0:-1], s])[160 * 50: 160 * 50 + 400].astype(np.float64)
+                      * (0.5 - 0.5 * np.cos(2 * np.pi * np.arange(400) / 400)))) ** 2)).max()) + 4.0) / 4.0, atol=0.05)
+
+
+def test_log_mel_against_the_reference(oracle, ref):
+    if not ref.log_mel_available():
+        pytest.skip("oracle/_ref/libref_mel.so is not built")
+    for n, n_mel in ((4000 + 7, 80), (16000 * 2, 128), (201, 80)):
+        t = np.arange(n) / 16000.0
+        s = (0.5 * np.sin(2 * np.pi * (200.0 + 3000.0 * t) * t) + 0.02 * RNG.normal(size=n)).astype(np.float32)
+        f = oracle.mel_filter_bank(n_mel)
+        got, want = oracle.log_mel_spectrogram(s, f), ref.log_mel_spectrogram(s, f, n_threads=3)
+        assert got.shape == want.shape
+        assert np.array_equal(got.view(np.uint32), want.view(np.uint32))

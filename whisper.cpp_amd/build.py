@@ -32,7 +32,7 @@ ARCH = "gfx950"
 DEVICE_FLAGS = ["--offload-arch=" + ARCH, "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 COMMON = ["-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden", "-Wall", "-Wno-unused-function", "-Wno-unused-variable"]
 
-KERNEL_SOURCES = ["misc.hip", "elementwise.hip", "rowwise.hip", "mul_mat.hip", "flash_attn.hip"]
+KERNEL_SOURCES = ["misc.hip", "elementwise.hip", "rowwise.hip", "mul_mat.hip", "flash_attn.hip", "log_mel.hip"]
 BACKEND_SOURCES = ["ggml-mi355x.cpp", "graph.cpp"]
 HARNESS_SOURCES = ["main.cpp", "synth_model.cpp", "op_cases.cpp", "verify.cpp"]
 

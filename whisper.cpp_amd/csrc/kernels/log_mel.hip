@@ -1,0 +1,162 @@
+// Log-mel front end on the device: 16 kHz samples -> the [n_mel, n_len] input of the encoder's conv stem
+// (log_mel_spectrogram, src/whisper.cpp:3181-3270, and its worker :3113-3179).
+//
+// The reference extends the signal by 200 reflected samples in front and 30 s + 200 samples of zeros behind, takes
+// 400-sample frames every 160 samples under a periodic Hann window, a 400-point transform per frame (f32, halved down
+// to 25-point sums), the power of bins 0 .. 200, a [n_mel, 201] filter bank, log10(max(., 1e-10)), and finally raises
+// everything below (global maximum - 8) to it and maps x to (x + 4) / 4.
+//
+// Here a frame's transform is the direct sum over its 400 samples — 0.5 GFLOP for a 30 s window, nothing for this
+// part, where the halving scheme would be 25 x less arithmetic but a dependent chain of small passes — in f64: the
+// vector units issue v_fma_f64 at the f32 rate, and with f64 sums the result does not depend on the order of the
+// terms, so it is the mathematical value to 1e-12 where the reference's f32 transform is within about 1e-6 of it.
+// One workgroup takes 16 consecutive frames: thread k < 201 owns bin k of all 16 (32 f64 accumulators), the windowed
+// samples sit in LDS sample-major (the 16 frames' values of one sample index are one 128-byte broadcast read), the
+// twiddles cos, sin(2 pi i / 400) are a 400-entry LDS table walked by (k n) mod 400.  Then thread (band j, half of
+// the frames) applies the filter bank from a transposed copy ([201][n_mel]: lanes = bands read consecutive floats)
+// to the powers, which have replaced the samples in LDS.  Frames past the end of the signal are not computed: they
+// hold log10(1e-10) by definition, and the last pass writes that.  Three launches: filters transposed + maximum
+// cleared; frames; clamp and scale.
+#include "common.h"
+
+#define MEL_NFFT   400
+#define MEL_HOP    160
+#define MEL_BINS   201
+#define MEL_FRAMES 16           // frames per workgroup
+#define MEL_MAX_BANDS 128
+
+typedef double double2_t __attribute__((ext_vector_type(2)));
+
+// order-preserving map of f32 onto signed integers, for atomicMax
+__device__ __forceinline__ int   mel_key(float x)  { const int i = __float_as_int(x); return i ^ ((i >> 31) & 0x7fffffff); }
+__device__ __forceinline__ float mel_unkey(int k)  { return __int_as_float(k ^ ((k >> 31) & 0x7fffffff)); }
+
+__global__ void k_log_mel_setup(const float * __restrict__ filters, int n_mel, float * __restrict__ filters_t, int * __restrict__ max_key) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;          // element of the transposed copy: (k, j)
+    if (i < MEL_BINS * n_mel) { const int k = i / n_mel, j = i % n_mel; filters_t[i] = filters[j * MEL_BINS + k]; }
+    if (i == 0) *max_key = mel_key(-INFINITY);
+}
+
+__global__ void __launch_bounds__(256) k_log_mel_frames(const float * __restrict__ samples, int64_t n_samples, const float * __restrict__ filters_t,
+                                                       int n_mel, int64_t n_frames, int64_t n_len, float * __restrict__ mel, int * __restrict__ max_key) {
+    __shared__ __attribute__((aligned(16))) double    fr[MEL_NFFT * MEL_FRAMES];   // windowed samples [n][frame]; later powers [bin][frame]
+    __shared__ __attribute__((aligned(16))) double2_t cs[MEL_NFFT];                // (cos, sin)(2 pi i / 400)
+    const int tid = threadIdx.x;
+    const int64_t i0 = (int64_t) blockIdx.x * MEL_FRAMES;
+
+    for (int i = tid; i < MEL_NFFT; i += 256) {
+        double s, c;
+        sincospi(2.0 * i / MEL_NFFT, &s, &c);
+        cs[i] = (double2_t){ c, s };
+    }
+    __syncthreads();
+    // sample p of the extended signal: reflected head, the samples, zeros
+    for (int e = tid; e < MEL_NFFT * MEL_FRAMES; e += 256) {
+        const int n = e / MEL_FRAMES, f = e % MEL_FRAMES;
+        const int64_t p = (i0 + f) * MEL_HOP + n;
+        float x = 0.0f;
+        if (p < MEL_NFFT / 2) x = samples[MEL_NFFT / 2 - p];
+        else if (p < n_samples + MEL_NFFT / 2) x = samples[p - MEL_NFFT / 2];
+        fr[e] = (0.5 * (1.0 - cs[n].x)) * (double) x;
+    }
+    __syncthreads();
+
+    double pw[MEL_FRAMES];
+    if (tid < MEL_BINS) {
+        double re[MEL_FRAMES], im[MEL_FRAMES];
+#pragma unroll
+        for (int f = 0; f < MEL_FRAMES; ++f) { re[f] = 0.0; im[f] = 0.0; }
+        int idx = 0;                                                  // (tid * n) mod 400
+        for (int n = 0; n < MEL_NFFT; ++n) {
+            const double2_t w = cs[idx];
+            const double2_t * x2 = (const double2_t *)(fr + n * MEL_FRAMES);
+#pragma unroll
+            for (int f = 0; f < MEL_FRAMES / 2; ++f) {
+                const double2_t x = x2[f];
+                re[2 * f]     = __builtin_fma(x.x, w.x, re[2 * f]);     im[2 * f]     = __builtin_fma(x.x, w.y, im[2 * f]);
+                re[2 * f + 1] = __builtin_fma(x.y, w.x, re[2 * f + 1]); im[2 * f + 1] = __builtin_fma(x.y, w.y, im[2 * f + 1]);
+            }
+            idx += tid; if (idx >= MEL_NFFT) idx -= MEL_NFFT;
+        }
+#pragma unroll
+        for (int f = 0; f < MEL_FRAMES; ++f) pw[f] = re[f] * re[f] + im[f] * im[f];
+    }
+    __syncthreads();                                                  // every bin is done with the samples
+    if (tid < MEL_BINS) {
+#pragma unroll
+        for (int f = 0; f < MEL_FRAMES; ++f) fr[tid * MEL_FRAMES + f] = pw[f];
+    }
+    __syncthreads();
+
+    // filter bank: thread = (band j, half of the frames)
+    const int j = tid & (MEL_MAX_BANDS - 1), fh = tid >> 7;
+    float vmax = -INFINITY;
+    if (j < n_mel) {
+        double sum[MEL_FRAMES / 2];
+#pragma unroll
+        for (int f = 0; f < MEL_FRAMES / 2; ++f) sum[f] = 0.0;
+        for (int k = 0; k < MEL_BINS; ++k) {
+            const double w = (double) filters_t[k * n_mel + j];
+            const double2_t * p2 = (const double2_t *)(fr + k * MEL_FRAMES + fh * (MEL_FRAMES / 2));
+#pragma unroll
+            for (int f = 0; f < MEL_FRAMES / 4; ++f) {
+                const double2_t p = p2[f];
+                sum[2 * f] = __builtin_fma(p.x, w, sum[2 * f]); sum[2 * f + 1] = __builtin_fma(p.y, w, sum[2 * f + 1]);
+            }
+        }
+#pragma unroll
+        for (int f = 0; f < MEL_FRAMES / 2; ++f) {
+            const int64_t i = i0 + fh * (MEL_FRAMES / 2) + f;
+            if (i < n_frames) {
+                const float v = (float) log10(sum[f] > 1e-10 ? sum[f] : 1e-10);
+                mel[(int64_t) j * n_len + i] = v;
+                vmax = fmaxf(vmax, v);
+            }
+        }
+    }
+    vmax = wave_max(vmax);
+    if ((tid & 63) == 0 && vmax > -INFINITY) atomicMax(max_key, mel_key(vmax));
+}
+
+// frames past the signal hold log10(1e-10); everything below (maximum - 8) is raised to it; (x + 4) / 4 (in f64, as the
+// reference's expressions are)
+__global__ void k_log_mel_finish(float * __restrict__ mel, int n_mel, int64_t n_frames, int64_t n_len, const int * __restrict__ max_key) {
+    const int64_t e = (int64_t) blockIdx.x * blockDim.x + threadIdx.x;
+    if (e >= (int64_t) n_mel * n_len) return;
+    const int64_t i = e % n_len;
+    float top = mel_unkey(*max_key);
+    if (n_frames < n_len) top = fmaxf(top, -10.0f);
+    const double floor_ = (double) top - 8.0;
+    float x = i < n_frames ? mel[e] : -10.0f;
+    if ((double) x < floor_) x = (float) floor_;
+    mel[e] = (float)(((double) x + 4.0) / 4.0);
+}
+
+extern "C" int64_t mi355x_log_mel_n_len(int64_t n_samples) { return n_samples > 0 ? (n_samples + 30 * 16000) / MEL_HOP : 0; }
+
+extern "C" size_t mi355x_log_mel_workspace_size(int n_mel) {
+    if (n_mel < 1 || n_mel > MEL_MAX_BANDS) return 0;
+    return ((size_t) MEL_BINS * n_mel * 4 + 256 + 255) / 256 * 256;
+}
+
+extern "C" int mi355x_log_mel_spectrogram(const float * samples, int64_t n_samples, const float * filters, int n_mel, float * mel,
+                                          void * workspace, size_t workspace_size, void * stream) {
+    if (!samples || !filters || !mel) return MI355X_ERR_INVALID;
+    if (n_mel < 1 || n_mel > MEL_MAX_BANDS) return MI355X_ERR_UNSUPPORTED;
+    if (n_samples <= MEL_NFFT / 2 || n_samples > (int64_t) 1 << 40) return MI355X_ERR_INVALID;      // the reflected head reads samples 1 .. 200
+    if (!workspace || workspace_size < mi355x_log_mel_workspace_size(n_mel) || (uintptr_t) workspace % 16 != 0) return MI355X_ERR_WORKSPACE;
+    hipStream_t st = (hipStream_t) stream;
+    const int64_t n_len = mi355x_log_mel_n_len(n_samples);
+    int64_t n_frames = (n_samples + MEL_NFFT / 2) / MEL_HOP + 1;
+    if (n_frames > n_len) n_frames = n_len;
+    float * filters_t = (float *) workspace;
+    int *   max_key   = (int *)((char *) workspace + (size_t) MEL_BINS * n_mel * 4);
+    const int64_t groups = (n_frames + MEL_FRAMES - 1) / MEL_FRAMES, elems = (int64_t) n_mel * n_len;
+    if (groups > 0x7fffffff || (elems + 255) / 256 > 0x7fffffff) return MI355X_ERR_UNSUPPORTED;
+    k_log_mel_setup<<<(MEL_BINS * n_mel + 255) / 256, 256, 0, st>>>(filters, n_mel, filters_t, max_key);
+    if (const int rc = launch_status()) return rc;
+    k_log_mel_frames<<<(unsigned) groups, 256, 0, st>>>(samples, n_samples, filters_t, n_mel, n_frames, n_len, mel, max_key);
+    if (const int rc = launch_status()) return rc;
+    k_log_mel_finish<<<(unsigned)((elems + 255) / 256), 256, 0, st>>>(mel, n_mel, n_frames, n_len, max_key);
+    return launch_status();
+}
