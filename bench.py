@@ -151,6 +151,15 @@ def main() -> int:
     decode["kernel_breakdown"] = {n: {"launches_per_step": k["calls"] / dec["steps"], "ms_per_step": round(k["ms"] / dec["steps"], 4)}
                                   for n, k in sorted(dk.items(), key=lambda kv: -kv[1]["ms"])[:8]}
 
+    # ---- the step in front of the encoder: log-mel of the 30 s window on the device beside whisper_pcm_to_mel on the host threads -------
+    mel = run_harness(["mel", "--model", enc_model, "--seconds", "30", "--reps", "20", "--threads", str(a.threads)])
+    log_mel = {"device_us": mel["device_us"], "host_to_host_ms": mel["host_to_host_ms"], "cpu_ms": mel["cpu_ms"], "cpu_threads": mel["cpu_threads"],
+               "n_mel": mel["n_mel"], "n_len": mel["n_len"],
+               "roofline": {"kernel": "log_mel (3 launches)", "bound": "hbm", "achieved": round(mel["algorithmic_mb"] / mel["device_us"] * 1e3, 1), "peak": PEAK_HBM_GBS,
+                            "unit": "GB/s", "frac": round(mel["algorithmic_mb"] / mel["device_us"] * 1e3 / PEAK_HBM_GBS, 5),
+                            "algorithmic_mb_per_launch": mel["algorithmic_mb"], "traffic": None,
+                            "note": "samples in + mel out; 0.97 GFLOP of f64 multiply-adds over 5 MB: launch latency and f64 issue, not bandwidth"}}
+
     # ---- CPU baseline: the reference's ggml CPU backend, same model file, same window ------------------------------------------
     cpu_baseline = None
     if not a.no_cpu:
@@ -184,6 +193,7 @@ def main() -> int:
         "encoder_ms_with_f32_mfma_attention_option": round(f32att["ms_per_step"], 4),
         "decode_tok_per_s": decode["steps_per_s"],
         "decode": decode,
+        "log_mel": log_mel,
         "kernel_breakdown": breakdown,
         "roofline": roofline,
         "kernel_rooflines": [r for r in rooflines.values() if r["launches"] / enc["profile_reps"] >= 30],

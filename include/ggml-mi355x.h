@@ -47,6 +47,7 @@ GGML_BACKEND_API int                ggml_backend_score(void);
  *   "ggml_backend_get_features"        ggml_backend_get_features_t
  *   "ggml_backend_mi355x_set_option"   ggml_backend_mi355x_set_option_t
  *   "ggml_backend_mi355x_get_stats"    ggml_backend_mi355x_get_stats_t
+ *   "ggml_backend_mi355x_log_mel"      ggml_backend_mi355x_log_mel_t
  */
 
 /* Options: "fuse" (0/1: fold bias/activation/residual/LayerNorm-affine neighbours into one kernel, default 1),
@@ -72,6 +73,17 @@ typedef int (*ggml_backend_mi355x_set_option_t)(ggml_backend_t backend, const ch
  * into buf (at most size bytes, NUL-terminated), resets the counters when `reset` is non-zero and returns the
  * length needed. */
 typedef size_t (*ggml_backend_mi355x_get_stats_t)(ggml_backend_t backend, char * buf, size_t size, int reset);
+
+/* The log-mel front end (log_mel_spectrogram, src/whisper.cpp:3181-3270 — what whisper_pcm_to_mel, :3881, runs on
+ * host threads) on device `device`, for a host that holds its samples in host memory: uploads the 16 kHz f32 samples
+ * and the model's filter bank [n_mel][201], runs mi355x_log_mel_spectrogram and downloads mel [n_mel][n_len] into
+ * `mel` (capacity in floats).  Returns n_len = (n_samples + 480000) / 160, which is what whisper_set_mel takes next to
+ * `mel`, or a negative mi355x status; with mel == NULL it only returns n_len.  whisper_full(ctx, params, NULL, 0) then
+ * transcribes from that mel without computing its own (src/whisper.cpp:5492).  `device_ms`, when not NULL, receives
+ * the time of the device work alone (HIP events around the kernels; the rest of the call is the allocation and the
+ * three copies). */
+typedef int64_t (*ggml_backend_mi355x_log_mel_t)(int device, const float * samples, int64_t n_samples, const float * filters, int n_mel,
+                                                 float * mel, int64_t mel_capacity, float * device_ms);
 
 #ifdef __cplusplus
 }

@@ -94,6 +94,16 @@ def test_whisper_full_end_to_end(harness, models):
     assert rc == 0 and s["pass"] and s["gpu_rc"] == 0 and s["gpu_tokens"] > 0 and s["gpu_segments"] > 0, s
 
 
+def test_whisper_full_from_the_device_log_mel(harness, models):
+    # the plugin's "ggml_backend_mi355x_log_mel" in place of whisper_pcm_to_mel: the harness computes the mel of the same
+    # synthetic audio on the device, hands it over with whisper_set_mel and calls whisper_full without samples; the CPU run
+    # goes through whisper's own front end.  The greedy transcripts must start alike, as in the test above.
+    rc, rows = run_harness(harness, ["full", "--model", models[("base", "q5_0")], "--beam", "1", "--max-tokens", "24", "--gpu-mel"], timeout=900)
+    s = rows[-1]
+    assert rc == 0 and s["pass"] and s["gpu_mel"] and s["gpu_rc"] == 0 and s["gpu_tokens"] > 0 and s["gpu_mel_ms"] > 0, s
+    assert s["common_prefix"] >= min(8, s["cpu_tokens"]), s
+
+
 def test_whisper_full_parallel_states_share_one_device(harness, models):
     # whisper_full_parallel (src/whisper.cpp:6407-6470): three states, three backend instances and streams, three host
     # threads on one GPU, all starting at once over shared weights — the f16 weight images are made on first use and must be

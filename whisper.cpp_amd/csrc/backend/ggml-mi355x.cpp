@@ -522,11 +522,47 @@ static size_t get_stats(ggml_backend_t backend, char * buf, size_t size, int res
     return s.size() + 1;
 }
 
+// host-memory front of mi355x_log_mel_spectrogram: one allocation for samples, filter bank, result and workspace, the
+// null stream, blocking copies.  Called once per audio file, next to milliseconds of host work it replaces.
+static int64_t log_mel(int device, const float * samples, int64_t n_samples, const float * filters, int n_mel, float * mel, int64_t mel_capacity, float * device_ms) {
+    const int64_t n_len = mi355x_log_mel_n_len(n_samples);
+    const size_t ws_bytes = mi355x_log_mel_workspace_size(n_mel);
+    if (!samples || !filters || n_len <= 0) return MI355X_ERR_INVALID;
+    if (!ws_bytes) return MI355X_ERR_UNSUPPORTED;
+    if (!mel) return n_len;
+    if (mel_capacity < n_len * n_mel) return MI355X_ERR_INVALID;
+    HIP_TRY(hipSetDevice(device), return MI355X_ERR_HIP);
+    auto pad = [](size_t b) { return (b + 255) / 256 * 256; };
+    const size_t b_s = pad((size_t) n_samples * 4), b_f = pad((size_t) n_mel * 201 * 4), b_m = pad((size_t) n_len * n_mel * 4);
+    char * base = nullptr;
+    HIP_TRY(hipMalloc((void **) &base, b_s + b_f + b_m + ws_bytes), return MI355X_ERR_HIP);
+    int64_t rc = MI355X_ERR_HIP;
+    if (hipMemcpy(base, samples, (size_t) n_samples * 4, hipMemcpyHostToDevice) == hipSuccess &&
+        hipMemcpy(base + b_s, filters, (size_t) n_mel * 201 * 4, hipMemcpyHostToDevice) == hipSuccess) {
+        hipEvent_t e0 = nullptr, e1 = nullptr;
+        if (device_ms && (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess)) { (void) hipGetLastError(); device_ms = nullptr; }
+        if (device_ms) (void) hipEventRecord(e0, nullptr);
+        rc = mi355x_log_mel_spectrogram((const float *) base, n_samples, (const float *)(base + b_s), n_mel, (float *)(base + b_s + b_f),
+                                        base + b_s + b_f + b_m, ws_bytes, nullptr);
+        if (device_ms) {
+            (void) hipEventRecord(e1, nullptr);
+            if (hipEventSynchronize(e1) != hipSuccess || hipEventElapsedTime(device_ms, e0, e1) != hipSuccess) { (void) hipGetLastError(); *device_ms = -1.0f; }
+        }
+        if (e0) (void) hipEventDestroy(e0);
+        if (e1) (void) hipEventDestroy(e1);
+        if (rc == MI355X_OK) rc = hipMemcpy(mel, base + b_s + b_f, (size_t) n_len * n_mel * 4, hipMemcpyDeviceToHost) == hipSuccess ? n_len : (int64_t) MI355X_ERR_HIP;
+    }
+    if (rc == MI355X_ERR_HIP) (void) hipGetLastError();
+    (void) hipFree(base);
+    return rc;
+}
+
 static void * reg_get_proc_address(ggml_backend_reg_t, const char * name) {
     if (!name) return NULL;
     if (strcmp(name, "ggml_backend_get_features") == 0)      return (void *) get_features;
     if (strcmp(name, "ggml_backend_mi355x_set_option") == 0) return (void *) set_option;
     if (strcmp(name, "ggml_backend_mi355x_get_stats") == 0)  return (void *) get_stats;
+    if (strcmp(name, "ggml_backend_mi355x_log_mel") == 0)    return (void *) log_mel;
     return NULL;
 }
 

@@ -9,8 +9,10 @@
 //                                             per-op parity (NMSE / bit-exactness) and timing, CPU vs MI355X
 //   model  --model F [--steps 32] [--threads N]
 //                                             whole-model parity: logits NMSE and greedy ids, teacher-forced
-//   full   --model F [--beam 1|5] [--max-tokens 24] [--seconds 30] [--threads N] [--dtw] [--processors N]
+//   full   --model F [--beam 1|5] [--max-tokens 24] [--seconds 30] [--threads N] [--dtw] [--processors N] [--gpu-mel]
 //                                             whisper_full() end to end (PCM -> mel -> encode -> search) on both backends
+//   mel    --model F [--seconds 30] [--reps 20] [--threads N]
+//                                             the log-mel front end: device path through the plugin vs whisper_pcm_to_mel
 //   verify --model F [--steps 3] [--threads N]
 //                                             per-node parity inside the real whisper graphs (unfused), CPU vs MI355X
 //   bench  --model F --what encoder|decoder|whisper-bench --backend gpu|cpu [--threads N] [--reps R] [--profile]
@@ -348,6 +350,10 @@ static int cmd_gen(const args & a) {
 static bool g_flash_attn = true;   // --no-flash-attn: whisper.cpp's default graphs (KQ MUL_MAT, SOFT_MAX, KQV MUL_MAT; src/whisper.cpp:3620)
 
 static int  g_processors = 1;
+static bool g_gpu_mel = false; // --gpu-mel: the GPU run takes its log-mel from the plugin ("ggml_backend_mi355x_log_mel") instead of whisper_pcm_to_mel
+static ggml_backend_mi355x_log_mel_t g_log_mel = nullptr;
+static std::string g_model_path;
+static double g_mel_ms = -1.0;
 static bool g_dtw = false;     // --dtw: token-level timestamps from the cross-attention of the top alignment heads (needs --no-flash-attn)
 
 static whisper_context * open_model(const std::string & path, bool use_gpu) {
@@ -443,8 +449,24 @@ static int cmd_model(const args & a) {
 // with its logits filters, timestamp rules and KV-cache bookkeeping.  Both backends see the same PCM; the token ids of
 // the two transcripts are compared from the front (a random-init model's near-flat logits let one rounding flip an
 // argmax, after which the two searches walk different histories, so only the common prefix is meaningful).
+// the filter bank of a model file (the loader keeps its copy private): magic, 11 hyper-parameters, n_mel, n_fft, data
+// (src/whisper.cpp:1522-1597)
+static std::vector<float> read_filters(const std::string & path, int32_t * n_mel) {
+    std::vector<float> filters;
+    int32_t n_fft = 0;
+    *n_mel = 0;
+    if (FILE * f = fopen(path.c_str(), "rb")) {
+        if (fseek(f, 4 + 11 * 4, SEEK_SET) == 0 && fread(n_mel, 4, 1, f) == 1 && fread(&n_fft, 4, 1, f) == 1 && n_fft == 201 && *n_mel > 0 && *n_mel <= 128) {
+            filters.resize((size_t) *n_mel * n_fft);
+            if (fread(filters.data(), 4, filters.size(), f) != filters.size()) filters.clear();
+        }
+        fclose(f);
+    }
+    return filters;
+}
+
 static std::vector<whisper_token> run_full(whisper_context * ctx, const std::vector<float> & pcm, int beam, int max_tokens, int threads, int * rc, double * ms,
-                                           std::vector<int64_t> * t_dtw = nullptr) {
+                                           std::vector<int64_t> * t_dtw = nullptr, bool use_gpu_mel = false) {
     whisper_full_params p = whisper_full_default_params(beam > 1 ? WHISPER_SAMPLING_BEAM_SEARCH : WHISPER_SAMPLING_GREEDY);
     p.n_threads = threads;
     p.print_progress = false; p.print_realtime = false; p.print_timestamps = false; p.print_special = false;
@@ -454,6 +476,18 @@ static std::vector<whisper_token> run_full(whisper_context * ctx, const std::vec
     p.suppress_blank = true;
     if (beam > 1) p.beam_search.beam_size = beam; else p.greedy.best_of = 1;
     const double t0 = now_ms();
+    if (use_gpu_mel) {
+        int32_t n_mel = 0;
+        const std::vector<float> filters = read_filters(g_model_path, &n_mel);
+        if (filters.empty()) { *rc = -100; *ms = 0; return {}; }
+        const double m0 = now_ms();
+        const int64_t n_len = g_log_mel(0, pcm.data(), (int64_t) pcm.size(), filters.data(), n_mel, nullptr, 0, nullptr);
+        std::vector<float> mel(n_len > 0 ? (size_t) n_len * n_mel : 0);
+        if (n_len <= 0 || g_log_mel(0, pcm.data(), (int64_t) pcm.size(), filters.data(), n_mel, mel.data(), (int64_t) mel.size(), nullptr) != n_len) { *rc = -101; *ms = 0; return {}; }
+        g_mel_ms = now_ms() - m0;
+        if (whisper_set_mel(ctx, mel.data(), (int) n_len, n_mel) != 0) { *rc = -102; *ms = 0; return {}; }
+        *rc = whisper_full(ctx, p, nullptr, 0);          // no samples: transcribes from the mel it was given (src/whisper.cpp:5492)
+    } else
     // --processors N: whisper_full_parallel splits the audio over N states, each with its own backend instance and host thread
     *rc = g_processors > 1 ? whisper_full_parallel(ctx, p, pcm.data(), (int) pcm.size(), g_processors) : whisper_full(ctx, p, pcm.data(), (int) pcm.size());
     *ms = now_ms() - t0;
@@ -472,8 +506,14 @@ static int cmd_full(const args & a) {
     const std::string path = a.str("model");
     const int threads = a.num("threads", default_threads()), beam = a.num("beam", 1), max_tokens = a.num("max-tokens", 24);
     const int seconds = a.num("seconds", 30);
-    if (path.empty()) { fprintf(stderr, "usage: full --model FILE [--beam N] [--max-tokens N] [--seconds N]\n"); return 2; }
-    if (!load_plugin(true)) { printf("{\"error\": \"no MI355X backend\"}\n"); return 2; }
+    if (path.empty()) { fprintf(stderr, "usage: full --model FILE [--beam N] [--max-tokens N] [--seconds N] [--gpu-mel]\n"); return 2; }
+    ggml_backend_reg_t reg = load_plugin(true);
+    if (!reg) { printf("{\"error\": \"no MI355X backend\"}\n"); return 2; }
+    g_model_path = path;
+    if (g_gpu_mel) {
+        g_log_mel = (ggml_backend_mi355x_log_mel_t) ggml_backend_reg_get_proc_address(reg, "ggml_backend_mi355x_log_mel");
+        if (!g_log_mel || g_processors > 1) { printf("{\"error\": \"--gpu-mel needs the plugin's log-mel entry and one processor\"}\n"); return 2; }
+    }
     whisper_context * gpu = open_model(path, true);
     whisper_context * cpu = open_model(path, false);
     if (!gpu || !cpu) { printf("{\"error\": \"model load failed\"}\n"); return 2; }
@@ -488,7 +528,7 @@ static int cmd_full(const args & a) {
     }
     int rg = 0, rc = 0; double ms_g = 0, ms_c = 0;
     std::vector<int64_t> dg, dc;
-    const std::vector<whisper_token> tg = run_full(gpu, pcm, beam, max_tokens, threads, &rg, &ms_g, &dg);
+    const std::vector<whisper_token> tg = run_full(gpu, pcm, beam, max_tokens, threads, &rg, &ms_g, &dg, g_gpu_mel);
     const std::vector<whisper_token> tc = run_full(cpu, pcm, beam, max_tokens, threads, &rc, &ms_c, &dc);
     size_t same = 0;
     while (same < tg.size() && same < tc.size() && tg[same] == tc[same]) ++same;
@@ -501,9 +541,9 @@ static int cmd_full(const args & a) {
     const bool pass = rg == 0 && rc == 0 && !tg.empty();
     printf("{\"summary\": \"full\", \"model\": \"%s\", \"beam\": %d, \"seconds\": %d, \"gpu_rc\": %d, \"cpu_rc\": %d, \"gpu_segments\": %d, \"cpu_segments\": %d, "
            "\"gpu_tokens\": %zu, \"cpu_tokens\": %zu, \"common_prefix\": %zu, \"dtw\": %s, \"dtw_identical_in_prefix\": %zu, \"gpu_t_dtw_first\": %lld, "
-           "\"gpu_first\": [%s], \"cpu_first\": [%s], \"gpu_ms\": %.1f, \"cpu_ms\": %.1f, \"pass\": %s}\n",
+           "\"gpu_first\": [%s], \"cpu_first\": [%s], \"gpu_ms\": %.1f, \"cpu_ms\": %.1f, \"gpu_mel\": %s, \"gpu_mel_ms\": %.3f, \"pass\": %s}\n",
            json_escape(path).c_str(), beam, seconds, rg, rc, rg == 0 ? whisper_full_n_segments(gpu) : -1, rc == 0 ? whisper_full_n_segments(cpu) : -1,
-           tg.size(), tc.size(), same, g_dtw ? "true" : "false", dtw_same, dg.empty() ? -1LL : (long long) dg[0], sg.c_str(), sc.c_str(), ms_g, ms_c, pass ? "true" : "false");
+           tg.size(), tc.size(), same, g_dtw ? "true" : "false", dtw_same, dg.empty() ? -1LL : (long long) dg[0], sg.c_str(), sc.c_str(), ms_g, ms_c, g_gpu_mel ? "true" : "false", g_mel_ms, pass ? "true" : "false");
     whisper_free(gpu); whisper_free(cpu);
     return pass ? 0 : 1;
 }
@@ -669,6 +709,50 @@ static int cmd_bench(const args & a) {
 // counters of a profiler are scaled by
 // ---------------------------------------------------------------------------------------------------------------
 
+// the log-mel front end of one window: the device path through the plugin (device time from HIP events, and the whole
+// host-to-host call) beside whisper_pcm_to_mel on the host threads, same samples, same filter bank
+static int cmd_mel(const args & a) {
+    const std::string path = a.str("model");
+    const int threads = a.num("threads", default_threads()), seconds = a.num("seconds", 30), reps = a.num("reps", 20);
+    if (path.empty()) { fprintf(stderr, "usage: mel --model FILE [--seconds N] [--reps N] [--threads N]\n"); return 2; }
+    ggml_backend_reg_t reg = load_plugin(true);
+    auto fn = reg ? (ggml_backend_mi355x_log_mel_t) ggml_backend_reg_get_proc_address(reg, "ggml_backend_mi355x_log_mel") : nullptr;
+    if (!fn) { printf("{\"error\": \"no MI355X backend\"}\n"); return 2; }
+    int32_t n_mel = 0;
+    const std::vector<float> filters = read_filters(path, &n_mel);
+    whisper_context * cpu = open_model(path, false);
+    if (filters.empty() || !cpu) { printf("{\"error\": \"model load failed\"}\n"); return 2; }
+    std::vector<float> pcm((size_t) seconds * WHISPER_SAMPLE_RATE);
+    uint64_t st = 0x9E3779B97F4A7C15ull;
+    for (size_t i = 0; i < pcm.size(); ++i) {
+        st = st * 6364136223846793005ull + 1442695040888963407ull;
+        const double t = (double) i / WHISPER_SAMPLE_RATE;
+        pcm[i] = (float)(0.25 * sin(2 * M_PI * (220.0 + 30.0 * t) * t) + 0.1 * (((double)(st >> 40) / (double)(1 << 24)) - 0.5));
+    }
+    const int64_t n_len = fn(0, pcm.data(), (int64_t) pcm.size(), filters.data(), n_mel, nullptr, 0, nullptr);
+    std::vector<float> mel((size_t) n_len * n_mel);
+    std::vector<double> dev, whole, host;
+    for (int r = 0; r < reps + 2; ++r) {
+        float ms = 0.0f;
+        const double t0 = now_ms();
+        if (fn(0, pcm.data(), (int64_t) pcm.size(), filters.data(), n_mel, mel.data(), (int64_t) mel.size(), &ms) != n_len) { printf("{\"error\": \"device log-mel failed\"}\n"); return 1; }
+        if (r >= 2) { dev.push_back(ms); whole.push_back(now_ms() - t0); }
+    }
+    for (int r = 0; r < 5; ++r) {
+        const double t0 = now_ms();
+        if (whisper_pcm_to_mel(cpu, pcm.data(), (int) pcm.size(), threads) != 0) { printf("{\"error\": \"whisper_pcm_to_mel failed\"}\n"); return 1; }
+        if (r >= 1) host.push_back(now_ms() - t0);
+    }
+    auto median = [](std::vector<double> v) { std::sort(v.begin(), v.end()); return v[v.size() / 2]; };
+    // algorithmic bytes of the device work: samples in, mel out (the filter bank and the workspace stay in the caches)
+    const double bytes = (double) pcm.size() * 4 + (double) mel.size() * 4;
+    printf("{\"bench\": \"log_mel\", \"seconds\": %d, \"n_mel\": %d, \"n_len\": %lld, \"device_us\": %.2f, \"host_to_host_ms\": %.3f, "
+           "\"cpu_ms\": %.3f, \"cpu_threads\": %d, \"algorithmic_mb\": %.3f, \"model\": \"%s\"}\n",
+           seconds, n_mel, (long long) n_len, median(dev) * 1e3, median(whole), median(host), threads, bytes / 1e6, json_escape(path).c_str());
+    whisper_free(cpu);
+    return 0;
+}
+
 static int cmd_copy(const args & a) {
     const int64_t mib = a.num("mib", 256), reps = a.num("reps", 5);
     ggml_backend_reg_t reg = load_plugin(true);
@@ -698,13 +782,14 @@ static int cmd_copy(const args & a) {
 }
 
 int main(int argc, char ** argv) {
-    if (argc < 2) { fprintf(stderr, "usage: %s info|gen|selftest|ops|model|full|verify|bench|copy [options]\n", argv[0]); return 2; }
+    if (argc < 2) { fprintf(stderr, "usage: %s info|gen|selftest|ops|model|full|verify|bench|copy|mel [options]\n", argv[0]); return 2; }
     ggml_log_set(quiet_log, nullptr);
     whisper_log_set(quiet_log, nullptr);
     const std::string cmd = argv[1];
     const args a = parse_args(argc, argv, 2);
     if (a.has("no-flash-attn")) g_flash_attn = false;
     g_processors = a.num("processors", 1);
+    g_gpu_mel = a.has("gpu-mel");
     if (a.has("dtw")) { g_dtw = true; g_flash_attn = false; }        // whisper.cpp turns DTW off under flash attention
     if (cmd == "info")  return cmd_info(a);
     if (cmd == "gen")   return cmd_gen(a);
@@ -715,6 +800,7 @@ int main(int argc, char ** argv) {
     if (cmd == "verify") return cmd_verify(a);
     if (cmd == "bench") return cmd_bench(a);
     if (cmd == "copy")  return cmd_copy(a);
+    if (cmd == "mel")   return cmd_mel(a);
     fprintf(stderr, "unknown command %s\n", cmd.c_str());
     return 2;
 }

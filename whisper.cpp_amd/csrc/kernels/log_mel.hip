@@ -10,11 +10,12 @@
 // part, where the halving scheme would be 25 x less arithmetic but a dependent chain of small passes — in f64: the
 // vector units issue v_fma_f64 at the f32 rate, and with f64 sums the result does not depend on the order of the
 // terms, so it is the mathematical value to 1e-12 where the reference's f32 transform is within about 1e-6 of it.
-// One workgroup takes 16 consecutive frames: thread k < 201 owns bin k of all 16 (32 f64 accumulators), the windowed
-// samples sit in LDS sample-major (the 16 frames' values of one sample index are one 128-byte broadcast read), the
+// One workgroup takes 12 consecutive frames: thread k < 201 owns bin k of all 12 (24 f64 accumulators), the windowed
+// samples sit in LDS sample-major (the 12 frames' values of one sample index are one 96-byte broadcast read), the
 // twiddles cos, sin(2 pi i / 400) are a 400-entry LDS table walked by (k n) mod 400.  Then thread (band j, half of
-// the frames) applies the filter bank from a transposed copy ([201][n_mel]: lanes = bands read consecutive floats)
-// to the powers, which have replaced the samples in LDS.  Frames past the end of the signal are not computed: they
+// the frames) applies the filter bank from a transposed copy ([208][n_mel], zero rows past bin 200: lanes = bands read
+// consecutive floats, 16 rows per request and the next request in flight) to the powers, which have replaced the
+// samples in LDS.  Frames past the end of the signal are not computed: they
 // hold log10(1e-10) by definition, and the last pass writes that.  Three launches: filters transposed + maximum
 // cleared; frames; clamp and scale.
 #include "common.h"
@@ -22,7 +23,9 @@
 #define MEL_NFFT   400
 #define MEL_HOP    160
 #define MEL_BINS   201
-#define MEL_FRAMES 16           // frames per workgroup
+#define MEL_FRAMES 12           // frames per workgroup: the 3002 frames of a 30 s window make 251 workgroups for 256 CUs
+#define MEL_CHUNK  16           // filter-bank rows a thread requests at a time
+#define MEL_ROWS   208          // rows of the transposed filter bank: 201 bins padded with zero rows to whole chunks
 #define MEL_MAX_BANDS 128
 
 typedef double double2_t __attribute__((ext_vector_type(2)));
@@ -33,7 +36,7 @@ __device__ __forceinline__ float mel_unkey(int k)  { return __int_as_float(k ^ (
 
 __global__ void k_log_mel_setup(const float * __restrict__ filters, int n_mel, float * __restrict__ filters_t, int * __restrict__ max_key) {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;          // element of the transposed copy: (k, j)
-    if (i < MEL_BINS * n_mel) { const int k = i / n_mel, j = i % n_mel; filters_t[i] = filters[j * MEL_BINS + k]; }
+    if (i < MEL_ROWS * n_mel) { const int k = i / n_mel, j = i % n_mel; filters_t[i] = k < MEL_BINS ? filters[j * MEL_BINS + k] : 0.0f; }
     if (i == 0) *max_key = mel_key(-INFINITY);
 }
 
@@ -50,67 +53,131 @@ __global__ void __launch_bounds__(256) k_log_mel_frames(const float * __restrict
         cs[i] = (double2_t){ c, s };
     }
     __syncthreads();
-    // sample p of the extended signal: reflected head, the samples, zeros
-    for (int e = tid; e < MEL_NFFT * MEL_FRAMES; e += 256) {
-        const int n = e / MEL_FRAMES, f = e % MEL_FRAMES;
-        const int64_t p = (i0 + f) * MEL_HOP + n;
-        float x = 0.0f;
-        if (p < MEL_NFFT / 2) x = samples[MEL_NFFT / 2 - p];
-        else if (p < n_samples + MEL_NFFT / 2) x = samples[p - MEL_NFFT / 2];
-        fr[e] = (0.5 * (1.0 - cs[n].x)) * (double) x;
+    // sample p of the extended signal: reflected head, the samples, zeros.  Every load is unconditional (index clamped,
+    // value selected afterwards) and all of a thread's loads are requested before the first is used: behind a condition
+    // each of the 19 rounds would wait for its own trip to memory.
+    {
+        constexpr int ROUNDS = (MEL_NFFT * MEL_FRAMES + 255) / 256;
+        float xs[ROUNDS];
+#pragma unroll
+        for (int r = 0; r < ROUNDS; ++r) {
+            const int e = tid + r * 256, n = e / MEL_FRAMES, f = e % MEL_FRAMES;
+            const int64_t p = (i0 + f) * MEL_HOP + n;
+            int64_t at = p < MEL_NFFT / 2 ? MEL_NFFT / 2 - p : p - MEL_NFFT / 2;
+            at = at < n_samples ? at : n_samples - 1;
+            const float x = samples[at];
+            xs[r] = p < n_samples + MEL_NFFT / 2 ? x : 0.0f;
+        }
+#pragma unroll
+        for (int r = 0; r < ROUNDS; ++r) {
+            const int e = tid + r * 256;
+            if (e < MEL_NFFT * MEL_FRAMES) fr[e] = (0.5 * (1.0 - cs[e / MEL_FRAMES].x)) * (double) xs[r];
+        }
     }
     __syncthreads();
+
+    // filter bank role: thread = (band j, half of the frames).  Its filter column comes MEL_CHUNK rows per request through a
+    // ring of four chunks, so that a request has three chunks' worth of arithmetic to arrive in.
+    const int j = tid & (MEL_MAX_BANDS - 1), fh = tid >> 7;
+    const float * fcol = filters_t + (j < n_mel ? j : 0);
+    constexpr int CHUNKS = MEL_ROWS / MEL_CHUNK;
+    static_assert(CHUNKS % 4 == 1, "rounds of four plus one");
+    float wr[4][MEL_CHUNK];
+    auto request = [&](float (&w)[MEL_CHUNK], int c) __attribute__((always_inline)) {
+        c = c < CHUNKS ? c : CHUNKS - 1;
+#pragma unroll
+        for (int i = 0; i < MEL_CHUNK; ++i) w[i] = fcol[(c * MEL_CHUNK + i) * n_mel];
+    };
 
     double pw[MEL_FRAMES];
     if (tid < MEL_BINS) {
         double re[MEL_FRAMES], im[MEL_FRAMES];
 #pragma unroll
         for (int f = 0; f < MEL_FRAMES; ++f) { re[f] = 0.0; im[f] = 0.0; }
+        // one sample index per step: its twiddle and the frames' values are read from LDS a step ahead of their use
+        struct step { double2_t w; double2_t x[MEL_FRAMES / 2]; };
         int idx = 0;                                                  // (tid * n) mod 400
-        for (int n = 0; n < MEL_NFFT; ++n) {
-            const double2_t w = cs[idx];
+        auto fetch = [&](step & s, int n) __attribute__((always_inline)) {
+            s.w = cs[idx];
             const double2_t * x2 = (const double2_t *)(fr + n * MEL_FRAMES);
 #pragma unroll
-            for (int f = 0; f < MEL_FRAMES / 2; ++f) {
-                const double2_t x = x2[f];
-                re[2 * f]     = __builtin_fma(x.x, w.x, re[2 * f]);     im[2 * f]     = __builtin_fma(x.x, w.y, im[2 * f]);
-                re[2 * f + 1] = __builtin_fma(x.y, w.x, re[2 * f + 1]); im[2 * f + 1] = __builtin_fma(x.y, w.y, im[2 * f + 1]);
-            }
+            for (int f = 0; f < MEL_FRAMES / 2; ++f) s.x[f] = x2[f];
             idx += tid; if (idx >= MEL_NFFT) idx -= MEL_NFFT;
+        };
+        auto mad = [&](const step & s) __attribute__((always_inline)) {
+#pragma unroll
+            for (int f = 0; f < MEL_FRAMES / 2; ++f) {
+                re[2 * f]     = __builtin_fma(s.x[f].x, s.w.x, re[2 * f]);     im[2 * f]     = __builtin_fma(s.x[f].x, s.w.y, im[2 * f]);
+                re[2 * f + 1] = __builtin_fma(s.x[f].y, s.w.x, re[2 * f + 1]); im[2 * f + 1] = __builtin_fma(s.x[f].y, s.w.y, im[2 * f + 1]);
+            }
+        };
+        step sa, sb;
+        fetch(sa, 0);
+#pragma unroll 1
+        for (int n = 0; n < MEL_NFFT; n += 2) {
+            fetch(sb, n + 1);
+            __builtin_amdgcn_sched_barrier(0);
+            mad(sa);
+            __builtin_amdgcn_sched_barrier(0);
+            fetch(sa, n + 2 < MEL_NFFT ? n + 2 : MEL_NFFT - 1);      // (the last one is not used)
+            __builtin_amdgcn_sched_barrier(0);
+            mad(sb);
+            __builtin_amdgcn_sched_barrier(0);
         }
 #pragma unroll
         for (int f = 0; f < MEL_FRAMES; ++f) pw[f] = re[f] * re[f] + im[f] * im[f];
+    } else {
+#pragma unroll
+        for (int f = 0; f < MEL_FRAMES; ++f) pw[f] = 0.0;            // rows 201 .. 207 of the power tile meet zero filter rows
     }
+    request(wr[0], 0); request(wr[1], 1); request(wr[2], 2); request(wr[3], 3);
+    __builtin_amdgcn_sched_barrier(0);
     __syncthreads();                                                  // every bin is done with the samples
-    if (tid < MEL_BINS) {
+    if (tid < MEL_ROWS) {
 #pragma unroll
         for (int f = 0; f < MEL_FRAMES; ++f) fr[tid * MEL_FRAMES + f] = pw[f];
     }
     __syncthreads();
 
-    // filter bank: thread = (band j, half of the frames)
-    const int j = tid & (MEL_MAX_BANDS - 1), fh = tid >> 7;
     float vmax = -INFINITY;
-    if (j < n_mel) {
+    {
         double sum[MEL_FRAMES / 2];
 #pragma unroll
         for (int f = 0; f < MEL_FRAMES / 2; ++f) sum[f] = 0.0;
-        for (int k = 0; k < MEL_BINS; ++k) {
-            const double w = (double) filters_t[k * n_mel + j];
-            const double2_t * p2 = (const double2_t *)(fr + k * MEL_FRAMES + fh * (MEL_FRAMES / 2));
+        auto use = [&](const float (&w)[MEL_CHUNK], int c) __attribute__((always_inline)) {
 #pragma unroll
-            for (int f = 0; f < MEL_FRAMES / 4; ++f) {
-                const double2_t p = p2[f];
-                sum[2 * f] = __builtin_fma(p.x, w, sum[2 * f]); sum[2 * f + 1] = __builtin_fma(p.y, w, sum[2 * f + 1]);
+            for (int i = 0; i < MEL_CHUNK; ++i) {
+                const double wk = (double) w[i];
+                const double2_t * p2 = (const double2_t *)(fr + (c * MEL_CHUNK + i) * MEL_FRAMES + fh * (MEL_FRAMES / 2));
+#pragma unroll
+                for (int f = 0; f < MEL_FRAMES / 4; ++f) {
+                    const double2_t p = p2[f];
+                    sum[2 * f] = __builtin_fma(p.x, wk, sum[2 * f]); sum[2 * f + 1] = __builtin_fma(p.y, wk, sum[2 * f + 1]);
+                }
+            }
+        };
+        // rounds of four chunks in a loop that is not unrolled (unrolled, every request moves to the top and the registers
+        // run out); a chunk's buffer is requested again as soon as it is used up
+#pragma unroll 1
+        for (int c = 0; c < CHUNKS - 1; c += 4) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                use(wr[q], c + q);
+                __builtin_amdgcn_sched_barrier(0);
+                request(wr[q], c + q + 4);
+                __builtin_amdgcn_sched_barrier(0);
             }
         }
+        use(wr[0], CHUNKS - 1);
+        if (j < n_mel) {
 #pragma unroll
-        for (int f = 0; f < MEL_FRAMES / 2; ++f) {
-            const int64_t i = i0 + fh * (MEL_FRAMES / 2) + f;
-            if (i < n_frames) {
-                const float v = (float) log10(sum[f] > 1e-10 ? sum[f] : 1e-10);
-                mel[(int64_t) j * n_len + i] = v;
-                vmax = fmaxf(vmax, v);
+            for (int f = 0; f < MEL_FRAMES / 2; ++f) {
+                const int64_t i = i0 + fh * (MEL_FRAMES / 2) + f;
+                if (i < n_frames) {
+                    const float v = (float) log10(sum[f] > 1e-10 ? sum[f] : 1e-10);
+                    mel[(int64_t) j * n_len + i] = v;
+                    vmax = fmaxf(vmax, v);
+                }
             }
         }
     }
@@ -136,7 +203,7 @@ extern "C" int64_t mi355x_log_mel_n_len(int64_t n_samples) { return n_samples > 
 
 extern "C" size_t mi355x_log_mel_workspace_size(int n_mel) {
     if (n_mel < 1 || n_mel > MEL_MAX_BANDS) return 0;
-    return ((size_t) MEL_BINS * n_mel * 4 + 256 + 255) / 256 * 256;
+    return ((size_t) MEL_ROWS * n_mel * 4 + 256 + 255) / 256 * 256;
 }
 
 extern "C" int mi355x_log_mel_spectrogram(const float * samples, int64_t n_samples, const float * filters, int n_mel, float * mel,
@@ -150,10 +217,10 @@ extern "C" int mi355x_log_mel_spectrogram(const float * samples, int64_t n_sampl
     int64_t n_frames = (n_samples + MEL_NFFT / 2) / MEL_HOP + 1;
     if (n_frames > n_len) n_frames = n_len;
     float * filters_t = (float *) workspace;
-    int *   max_key   = (int *)((char *) workspace + (size_t) MEL_BINS * n_mel * 4);
+    int *   max_key   = (int *)((char *) workspace + (size_t) MEL_ROWS * n_mel * 4);
     const int64_t groups = (n_frames + MEL_FRAMES - 1) / MEL_FRAMES, elems = (int64_t) n_mel * n_len;
     if (groups > 0x7fffffff || (elems + 255) / 256 > 0x7fffffff) return MI355X_ERR_UNSUPPORTED;
-    k_log_mel_setup<<<(MEL_BINS * n_mel + 255) / 256, 256, 0, st>>>(filters, n_mel, filters_t, max_key);
+    k_log_mel_setup<<<(MEL_ROWS * n_mel + 255) / 256, 256, 0, st>>>(filters, n_mel, filters_t, max_key);
     if (const int rc = launch_status()) return rc;
     k_log_mel_frames<<<(unsigned) groups, 256, 0, st>>>(samples, n_samples, filters_t, n_mel, n_frames, n_len, mel, max_key);
     if (const int rc = launch_status()) return rc;
