@@ -245,6 +245,11 @@ MI355X_API int mi355x_cpy(const mi355x_tensor * src, const mi355x_tensor * dst, 
 /* GET_ROWS (ggml/src/ggml-cpu/ops.cpp:4146-4188, 4313): dst[:, i] = dequant(src0[:, ids[i]]).
  * src0: Q5_0 | Q8_0 | F16 | F32, ids: I32, dst: F32. */
 MI355X_API int mi355x_get_rows(const mi355x_tensor * src0, const mi355x_tensor * ids, const mi355x_tensor * dst, void * stream);
+/* dst[:, i] = dequant(src0 row ids0[i]) + src1 row ids1[i]: the token embedding plus the positional embedding of a
+ * decoder input (GET_ROWS, GET_ROWS and ADD of src/whisper.cpp:2526-2529, ops.cpp:4313 and binary-ops.cpp:49-142) in one
+ * launch; the same f32 values and the same f32 sum.  src1 F32; ids0, ids1 I32 vectors of one length; dst F32 [ne0, n]. */
+MI355X_API int mi355x_get_rows_add(const mi355x_tensor * src0, const mi355x_tensor * ids0, const mi355x_tensor * src1, const mi355x_tensor * ids1,
+                                   const mi355x_tensor * dst, void * stream);
 
 /* IM2COL, 1-D, F16 output (ggml/src/ggml-cpu/ops.cpp:5784-5855; ggml/src/ggml.c:3818-3858):
  * dst[ic*KW + kw, ow, n] = f16(src[ow*s0 + kw*d0 - p0, ic, n]) or 0 outside.  src F32 [IW, IC, N]. */

@@ -684,6 +684,15 @@ def test_cpy_get_rows_im2col_softmax_concat(pkg, oracle, gpu):
         d_o = torch.empty((5, 128), dtype=torch.float32, device=gpu.dev)
         pkg.check(lib.mi355x_get_rows(pkg.tensor(d_w, t, ne=[128, 300]), pkg.tensor(d_i, pkg.I32), pkg.tensor(d_o, pkg.F32), gpu.stream))
         assert np.array_equal(gpu.down(d_o), oracle.get_rows(t, blocks, ids, 128))
+        # the token + positional embedding of a decoder input as one launch: the same gathers and the same f32 sum
+        pos_table, pos = rnd((40, 128)), np.array([7, 8, 39, 0, 7], dtype=np.int32)
+        d_p, d_pi = gpu.up(pos_table), gpu.up(pos)
+        d_o.fill_(3.0)
+        pkg.check(lib.mi355x_get_rows_add(pkg.tensor(d_w, t, ne=[128, 300]), pkg.tensor(d_i, pkg.I32), pkg.tensor(d_p, pkg.F32), pkg.tensor(d_pi, pkg.I32),
+                                          pkg.tensor(d_o, pkg.F32), gpu.stream))
+        assert np.array_equal(gpu.down(d_o), oracle.binary(0, oracle.get_rows(t, blocks, ids, 128), pos_table[pos]))
+        assert lib.mi355x_get_rows_add(pkg.tensor(d_w, t, ne=[128, 300]), pkg.tensor(d_i, pkg.I32), pkg.tensor(d_p, pkg.F32), pkg.tensor(d_pi[:4], pkg.I32),
+                                       pkg.tensor(d_o, pkg.F32), gpu.stream) == -1
     # im2col, the two strides of the conv stem, odd sizes
     src = rnd((33, 77))
     for s0 in (1, 2):

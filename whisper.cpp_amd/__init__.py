@@ -86,6 +86,7 @@ def kernels() -> C.CDLL:
             "mi355x_soft_max": (C.c_int, [T, T, T, C.c_float, P]),
             "mi355x_cpy": (C.c_int, [T, T, P]),
             "mi355x_get_rows": (C.c_int, [T, T, T, P]),
+            "mi355x_get_rows_add": (C.c_int, [T, T, T, T, T, P]),
             "mi355x_im2col_1d": (C.c_int, [T, T, C.c_int, C.c_int, C.c_int, C.c_int, P]),
             "mi355x_concat": (C.c_int, [T, T, T, C.c_int, P]),
             "mi355x_fill_bytes": (C.c_int, [P, C.c_uint8, C.c_size_t, P]),

@@ -632,6 +632,32 @@ struct graph_runner {
                 return 1;
             }
             case GGML_OP_GET_ROWS: {
+                // token embedding + positional embedding of a decoder input (src/whisper.cpp:2526-2529): GET_ROWS, GET_ROWS, ADD
+                // as one launch when the two gathered tensors feed nothing else
+                if (ctx->fuse && only_feeds_next(n) && s1->ne[1] == 1 && s1->ne[2] == 1 && s1->ne[3] == 1) {
+                    int j = i + 1;
+                    while (node_at(j) && (is_view_op(node_at(j)->op) || ggml_is_empty(node_at(j)))) ++j;
+                    ggml_tensor * g2 = node_at(j);
+                    int k = j + 1;
+                    while (node_at(k) && (is_view_op(node_at(k)->op) || ggml_is_empty(node_at(k)))) ++k;
+                    ggml_tensor * add = node_at(k);
+                    if (g2 && add && g2->op == GGML_OP_GET_ROWS && add->op == GGML_OP_ADD && only_feeds_next(g2) && g2->src[0]->type == GGML_TYPE_F32 &&
+                        ((add->src[0] == n && add->src[1] == g2) || (add->src[0] == g2 && add->src[1] == n)) &&
+                        ggml_are_same_shape(n, g2) && ggml_are_same_shape(n, add) && add->type == GGML_TYPE_F32 && ggml_is_contiguous(add) &&
+                        g2->src[1]->ne[0] == s1->ne[0] && g2->src[1]->ne[1] == 1 && g2->src[1]->ne[2] == 1 && g2->src[1]->ne[3] == 1) {
+                        bool plain = true;                  // nothing between the three nodes may be a view of the gathered tensors
+                        for (int v = i + 1; v < k; ++v) plain = plain && (v == j || (node_at(v)->src[0] != n && node_at(v)->view_src != n && node_at(v)->src[0] != g2 && node_at(v)->view_src != g2));
+                        if (plain) {
+                            mi355x_tensor a = to_view(s0), ia = to_view(s1), b = to_view(g2->src[0]), ib = to_view(g2->src[1]), d = to_view(add);
+                            int rc;
+                            {
+                                launch_scope ls(ctx, "get_rows_add", 3.0 * nbytes_of(add), 0.0);
+                                rc = mi355x_get_rows_add(&a, &ia, &b, &ib, &d, ctx->stream);
+                            }
+                            if (rc != MI355X_ERR_UNSUPPORTED) { status = rc; note_write(add); return k - i + 1; }
+                        }
+                    }
+                }
                 mi355x_tensor a = to_view(s0), b = to_view(s1), d = to_view(n);
                 launch_scope ls(ctx, "get_rows", 2.0 * nbytes_of(n), 0.0);
                 status = mi355x_get_rows(&a, &b, &d, ctx->stream);

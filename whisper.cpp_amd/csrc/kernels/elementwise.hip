@@ -311,6 +311,44 @@ extern "C" int mi355x_get_rows(const mi355x_tensor * src0, const mi355x_tensor *
     return launch_status();
 }
 
+// dst[:, i] = dequant(src0 row ids0[i]) + src1 row ids1[i]: a decode step's token embedding plus positional embedding
+// (GET_ROWS, GET_ROWS, ADD of src/whisper.cpp:2526-2529) as one launch; the same f32 values and the same f32 sum
+template <int TYPE>
+__global__ void k_get_rows_add(tview s0, tview ids0, tview s1, tview ids1, tview d) {
+    const int64_t i = blockIdx.y;
+    const int32_t r0 = *(const int32_t *)(ids0.p + i * ids0.nb0), r1 = *(const int32_t *)(ids1.p + i * ids1.nb0);
+    const uint8_t * sp = (const uint8_t *) s0.p + (int64_t) r0 * s0.nb1;
+    const float *   pp = (const float *)(s1.p + (int64_t) r1 * s1.nb1);
+    float * dp = (float *)(d.p + i * d.nb1);
+    for (int64_t k = (int64_t) blockIdx.x * blockDim.x + threadIdx.x; k < d.ne0; k += (int64_t) gridDim.x * blockDim.x) {
+        dp[k] = dq_elem<TYPE>(sp, k) + pp[k];
+    }
+}
+
+extern "C" int mi355x_get_rows_add(const mi355x_tensor * src0, const mi355x_tensor * ids0, const mi355x_tensor * src1, const mi355x_tensor * ids1,
+                                   const mi355x_tensor * dst, void * stream) {
+    if (!src0 || !ids0 || !src1 || !ids1 || !dst) return MI355X_ERR_INVALID;
+    if (ids0->type != MI355X_TYPE_I32 || ids1->type != MI355X_TYPE_I32 || dst->type != MI355X_TYPE_F32 || src1->type != MI355X_TYPE_F32) return MI355X_ERR_UNSUPPORTED;
+    const int64_t nr = ids0->ne[0];
+    if (ids0->ne[1] != 1 || ids0->ne[2] != 1 || ids0->ne[3] != 1 || ids1->ne[0] != nr || ids1->ne[1] != 1 || ids1->ne[2] != 1 || ids1->ne[3] != 1 ||
+        dst->ne[1] != nr || dst->ne[2] != 1 || dst->ne[3] != 1 || src0->ne[2] != 1 || src0->ne[3] != 1 || src1->ne[2] != 1 || src1->ne[3] != 1) return MI355X_ERR_UNSUPPORTED;
+    if (dst->ne[0] != src0->ne[0] || dst->ne[0] != src1->ne[0] || dst->nb[0] != 4 || src1->nb[0] != 4 || src0->nb[0] != type_size(src0->type)) return MI355X_ERR_INVALID;
+    if (nr == 0 || dst->ne[0] == 0) return MI355X_OK;
+    if (nr > 65535) return MI355X_ERR_UNSUPPORTED;
+    hipStream_t st = (hipStream_t) stream;
+    int gx = (int) ((dst->ne[0] + EW_BLOCK - 1) / EW_BLOCK); if (gx > 64) gx = 64;
+    dim3 grid(gx, (unsigned) nr);
+    tview a = make_view(src0), ia = make_view(ids0), b = make_view(src1), ib = make_view(ids1), d = make_view(dst);
+    switch (src0->type) {
+        case MI355X_TYPE_Q5_0: k_get_rows_add<MI355X_TYPE_Q5_0><<<grid, EW_BLOCK, 0, st>>>(a, ia, b, ib, d); break;
+        case MI355X_TYPE_Q8_0: k_get_rows_add<MI355X_TYPE_Q8_0><<<grid, EW_BLOCK, 0, st>>>(a, ia, b, ib, d); break;
+        case MI355X_TYPE_F16:  k_get_rows_add<MI355X_TYPE_F16 ><<<grid, EW_BLOCK, 0, st>>>(a, ia, b, ib, d); break;
+        case MI355X_TYPE_F32:  k_get_rows_add<MI355X_TYPE_F32 ><<<grid, EW_BLOCK, 0, st>>>(a, ia, b, ib, d); break;
+        default: return MI355X_ERR_UNSUPPORTED;
+    }
+    return launch_status();
+}
+
 // ------------------------------------------------------------------------------------------------------
 // quantize_row_q8_0, AVX2 flavour (ggml/src/ggml-cpu/ggml-cpu-quants.c:808-865): one 32-lane half-wave per block
 // ------------------------------------------------------------------------------------------------------
