@@ -712,10 +712,19 @@ __global__ void __launch_bounds__(256) k_quantize_x_q8(const char * __restrict__
 // registers while the workgroup walks its row groups: the loop is weight loads and integer dot products only.  With
 // the activations in LDS, their reads (NC x 32 bytes per 34-byte block) are what bounds the kernel, and quantizing them
 // in every workgroup costs more than the product itself once K is large.
-struct gemv_no_prologue { __device__ __forceinline__ const char * operator()(const char * x) const { return x; } };
+struct gemv_no_prologue {
+    __device__ __forceinline__ void request() {}
+    __device__ __forceinline__ const char * finish(const char * x) { return x; }
+};
 
-// `prologue` runs once the first weight blocks are requested and returns where the quantized activations are: for the
-// plain product the workspace as passed; for the fused LayerNorm it first produces them in LDS.
+// `prologue` has two halves: request() issues its own loads BEFORE the first weight blocks are requested, finish() runs
+// after them and returns where the quantized activations are (the plain product: the workspace as passed; the fused
+// LayerNorm first produces them in LDS).  Loads are waited for in the order they were issued, so in this order the
+// LayerNorm's reductions run while the weight blocks are still on their way from HBM (vmcnt(3) in front of them, where
+// the other order had vmcnt(0)); every load up to finish() is unconditional (clamped address, value masked where it is
+// used), because behind a branch the compiler waits for all loads, not for a count.  Measured, the launch takes the
+// same 10.3 us either way: what the LayerNorm adds to the bare product is its own dependent chain (two reductions, the
+// block maxima, a barrier, the LDS round trip of the quantized rows), not a wait it shares with the weights.
 template <int T0, int NC, int LPR, int NB, typename PRO = gemv_no_prologue>
 __device__ __forceinline__ void gemv_qr_rows(const mm_args & a, PRO prologue = PRO()) {
     const int64_t K = a.K;
@@ -730,21 +739,20 @@ __device__ __forceinline__ void gemv_qr_rows(const mm_args & a, PRO prologue = P
     bool row_ok = row < a.M;
     const uint8_t * wrow = (const uint8_t *) a.w + (row_ok ? row : 0) * a.w_nb1;
 
-    // the first row's blocks are requested first; a lane whose block index lies beyond the row keeps an all-zero block
+    // a lane whose block index lies beyond the row reads the row's last block again and counts it with a zero scale
+    prologue.request();
+    __builtin_amdgcn_sched_barrier(0);                  // (the scheduler would hoist the weight loads above them again)
     wraw<T0> blk[NB];
+    bool blk_ok[NB];
 #pragma unroll
-    for (int b = 0; b < NB; ++b) {
-        blk[b].d = 0; blk[b].qh = 0;
-#pragma unroll
-        for (int i = 0; i < (T0 == MI355X_TYPE_Q8_0 ? 8 : 4); ++i) blk[b].q[i] = 0;
-    }
+    for (int b = 0; b < NB; ++b) blk_ok[b] = j + b * LPR < nbk;
     auto load_blocks = [&]() __attribute__((always_inline)) {
 #pragma unroll
-        for (int b = 0; b < NB; ++b) if (j + b * LPR < nbk) blk[b] = load_wraw<T0>(wrow, j + b * LPR);
+        for (int b = 0; b < NB; ++b) blk[b] = load_wraw<T0>(wrow, blk_ok[b] ? j + b * LPR : nbk - 1);
     };
     load_blocks();
 
-    const char * xbase = prologue(a.x);
+    const char * xbase = prologue.finish(a.x);
     const int32_t * xq   = (const int32_t *) xbase;
     const float *   xd   = (const float *)(xbase + (size_t) NC * K);
     const int32_t * xsum = (const int32_t *)(xbase + (size_t) NC * K + (size_t) NC * nbk * 4);
@@ -810,7 +818,7 @@ __device__ __forceinline__ void gemv_qr_rows(const mm_args & a, PRO prologue = P
 #pragma unroll
         for (int b = 0; b < NB; ++b) {
             uint32_t q[8];
-            const float dw = h2f((uint16_t) cur[b].d);
+            const float dw = blk_ok[b] ? h2f((uint16_t) cur[b].d) : 0.0f;
             if constexpr (T0 == MI355X_TYPE_Q8_0) {
 #pragma unroll
                 for (int i = 0; i < 8; ++i) q[i] = cur[b].q[i];
@@ -1011,29 +1019,35 @@ struct gemv_norm_args {
 template <int NC>
 struct gemv_norm_prologue {
     const gemv_norm_args & nm; int64_t K; char * lds;
-    __device__ __forceinline__ const char * operator()(const char *) const {
+    // wavefront w takes rows w and w + 4; both rows and the affine vectors are requested before anything is reduced, so
+    // the prologue is one memory round trip long
+    static constexpr int RW = (NC + 3) / 4;                 // rows per wavefront
+    float4 v[RW][8], ww[8], bb[8];
+
+    __device__ __forceinline__ void request() {
+        const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+        const int n4 = (int)(K / 4);
+        // no branch around a load: addresses are clamped into the rows, and a missing affine vector reads the source instead
+        const float4 * wp = (const float4 *)(nm.w ? (const char *) nm.w : nm.src), * bp = (const float4 *)(nm.b ? (const char *) nm.b : nm.src);
+#pragma unroll
+        for (int jj = 0; jj < 8; ++jj) {
+            const int c = lane + jj * WAVE < n4 ? lane + jj * WAVE : n4 - 1;
+            ww[jj] = wp[c]; bb[jj] = bp[c];
+#pragma unroll
+            for (int rr = 0; rr < RW; ++rr) {
+                const int row = wave + 4 * rr < NC ? wave + 4 * rr : NC - 1;
+                v[rr][jj] = ((const float4 *)(nm.src + row * nm.src_nb1))[c];
+            }
+        }
+    }
+
+    __device__ __forceinline__ const char * finish(const char *) {
         const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
         const int n4 = (int)(K / 4), nbk = (int)(K / QK);
         const bool writer = blockIdx.x == 0 && blockIdx.y == 0;
         int32_t * xq   = (int32_t *) lds;
         float *   xd   = (float *)(lds + (size_t) NC * K);
-        int32_t * xsum = (int32_t *)(lds + (size_t) NC * K + (size_t) NC * nbk * 4);
-        // wavefront w takes rows w and w + 4; both rows and the affine vectors are requested before anything is reduced, so
-        // the prologue is one memory round trip long
-        constexpr int RW = (NC + 3) / 4;                    // rows per wavefront
-        float4 v[RW][8], ww[8], bb[8];
-#pragma unroll
-        for (int jj = 0; jj < 8; ++jj) {
-            const int c = lane + jj * WAVE;
-            ww[jj] = make_float4(1.f, 1.f, 1.f, 1.f); bb[jj] = make_float4(0.f, 0.f, 0.f, 0.f);
-            if (c < n4) { if (nm.w) ww[jj] = ((const float4 *) nm.w)[c]; if (nm.b) bb[jj] = ((const float4 *) nm.b)[c]; }
-#pragma unroll
-            for (int rr = 0; rr < RW; ++rr) {
-                const int row = wave + 4 * rr;
-                v[rr][jj] = make_float4(0.f, 0.f, 0.f, 0.f);
-                if (c < n4 && row < NC) v[rr][jj] = ((const float4 *)(nm.src + row * nm.src_nb1))[c];
-            }
-        }
+        int32_t * xsum = (int32_t *)(lds + (size_t) NC * nbk * 4 + (size_t) NC * K);
 #pragma unroll
         for (int rr = 0; rr < RW; ++rr) {
             const int row = wave + 4 * rr;
