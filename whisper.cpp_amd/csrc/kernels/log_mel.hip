@@ -7,9 +7,10 @@
 // everything below (global maximum - 8) to it and maps x to (x + 4) / 4.
 //
 // Here a frame's transform is the direct sum over its 400 samples — 0.5 GFLOP for a 30 s window, nothing for this
-// part, where the halving scheme would be 25 x less arithmetic but a dependent chain of small passes — in f64: the
-// vector units issue v_fma_f64 at the f32 rate, and with f64 sums the result does not depend on the order of the
-// terms, so it is the mathematical value to 1e-12 where the reference's f32 transform is within about 1e-6 of it.
+// part, where the halving scheme would be 25 x less arithmetic but a dependent chain of small passes — in f64: with
+// f64 sums the result does not depend on the order of the terms, so it is the mathematical value to 1e-12 where the
+// reference's f32 transform is within about 1e-6 of it (v_fma_f64 issues at half the f32 rate, 4.2 ns per wavefront,
+// which is what the kernel's time comes to).
 // One workgroup takes 12 consecutive frames: thread k < 201 owns bin k of all 12 (24 f64 accumulators), the windowed
 // samples sit in LDS sample-major (the 12 frames' values of one sample index are one 96-byte broadcast read), the
 // twiddles cos, sin(2 pi i / 400) are a 400-entry LDS table walked by (k n) mod 400.  Then thread (band j, half of
