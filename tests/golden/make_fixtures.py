@@ -2,7 +2,9 @@
 reference's own compiled code (oracle/_ref: libggml-base quantizers, one-op graphs on the ggml CPU backend).
 
 Run in a container that has the reference built (python oracle/... make, see oracle/Makefile):
-    python tests/golden/make_fixtures.py
+    python tests/golden/make_fixtures.py                    # cpu_backend_vectors.npz and log_mel_vectors.npz
+    python tests/golden/make_fixtures.py --log-mel-only     # only log_mel_vectors.npz (the reference's log-mel front end,
+                                                            # reached through oracle/ref_mel_shim.cpp)
 The fixtures are data only; tests/test_golden.py checks the oracle restatement against them on the CPU, and
 tests/test_kernels_gpu.py checks the HIP kernels against them on the GPU box, where the reference does not exist.
 """
