@@ -131,7 +131,8 @@ void mi355x_buffer_ctx::drop_images(const void * begin, size_t nbytes) {
     std::lock_guard<std::mutex> lock(image_mutex);
     const uintptr_t b = (uintptr_t) begin, e = b + nbytes;
     for (auto it = images.begin(); it != images.end();) {
-        if (it->first < e && b < it->first + it->second.src_bytes) { (void) hipFree(it->second.f16); it = images.erase(it); }   // hipFree waits for the device
+        const uintptr_t at = it->first & ~(uintptr_t) 1;                // (the lowest bit of the key is the kind of image)
+        if (at < e && b < at + it->second.src_bytes) { (void) hipFree(it->second.f16); it = images.erase(it); }   // hipFree waits for the device
         else ++it;
     }
 }
