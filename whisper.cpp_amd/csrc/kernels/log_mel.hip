@@ -6,7 +6,7 @@
 // to 25-point sums), the power of bins 0 .. 200, a [n_mel, 201] filter bank, log10(max(., 1e-10)), and finally raises
 // everything below (global maximum - 8) to it and maps x to (x + 4) / 4.
 //
-// Here a frame's transform is the direct sum over its 400 samples — 0.5 GFLOP for a 30 s window, nothing for this
+// Here a frame's transform is the direct sum over its 400 samples — 0.48 G multiply-adds for a 30 s window, little for this
 // part, where the halving scheme would be 25 x less arithmetic but a dependent chain of small passes — in f64: with
 // f64 sums the result does not depend on the order of the terms, so it is the mathematical value to 1e-12 where the
 // reference's f32 transform is within about 1e-6 of it (v_fma_f64 issues at half the f32 rate, 4.2 ns per wavefront,
@@ -16,9 +16,8 @@
 // twiddles cos, sin(2 pi i / 400) are a 400-entry LDS table walked by (k n) mod 400.  Then thread (band j, half of
 // the frames) applies the filter bank from a transposed copy ([208][n_mel], zero rows past bin 200: lanes = bands read
 // consecutive floats, 16 rows per request and the next request in flight) to the powers, which have replaced the
-// samples in LDS.  Frames past the end of the signal are not computed: they
-// hold log10(1e-10) by definition, and the last pass writes that.  Three launches: filters transposed + maximum
-// cleared; frames; clamp and scale.
+// samples in LDS.  Frames past the end of the signal are not computed: they hold log10(1e-10) by definition, and the
+// last pass writes that.  Three launches: filters transposed + maximum cleared; frames; clamp and scale.
 #include "common.h"
 
 #define MEL_NFFT   400
