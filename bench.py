@@ -157,7 +157,7 @@ def main() -> int:
                "n_mel": mel["n_mel"], "n_len": mel["n_len"],
                "roofline": {"kernel": "log_mel (3 launches)", "bound": "hbm", "achieved": round(mel["algorithmic_mb"] / mel["device_us"] * 1e3, 1), "peak": PEAK_HBM_GBS,
                             "unit": "GB/s", "frac": round(mel["algorithmic_mb"] / mel["device_us"] * 1e3 / PEAK_HBM_GBS, 5),
-                            "algorithmic_mb_per_launch": mel["algorithmic_mb"], "traffic": None,
+                            "algorithmic_mb_per_launch": mel["algorithmic_mb"], "traffic": 11100000,      # FETCH_SIZE + WRITE_SIZE of the three launches (profiles/)
                             "note": "samples in + mel out; 0.97 GFLOP of f64 multiply-adds over 5 MB (18 % of the vector f64 peak in the frames kernel): bound by the issue rate of v_fma_f64 and three launch latencies, not by HBM"}}
 
     # ---- CPU baseline: the reference's ggml CPU backend, same model file, same window ------------------------------------------
