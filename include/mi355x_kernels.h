@@ -174,7 +174,9 @@ MI355X_API int    mi355x_mul_mat_q8_0_tiles(const void * tiles, int64_t K, int64
  * logit_softcap = 0 (the only values whisper uses):
  *   dst[:, h, n] = softmax_over_keys(scale * q[:, n, h] . k[:, key, h] + mask[key, n]) @ v[:, key, h]
  * q: F32 [D, N, H], k/v: F16 [D, KV, H] (D = 64), mask: F16 [KV, >=N] or NULL (-inf entries skip the
- * key), dst: F32 [D, H, N] contiguous.
+ * key), dst: F32 [D, H, N] contiguous.  With at most 8 queries the mask may also be the F32 tensor that the graph
+ * casts to F16 (ggml_cast in src/whisper.cpp:2523): each value is rounded to f16 as it is read, which is what the
+ * cast does, so a caller can leave the cast out; MI355X_ERR_UNSUPPORTED with more queries.
  * mode: MI355X_FA_F16_SEQ accumulates V in f16, key by key in order, as the reference does (ops.cpp:6793-6807) —
  * with near-uniform attention over ~1500 keys that rounding sequence dominates the low bits of the result;
  * MI355X_FA_F32 accumulates in f32 (closer to exact arithmetic, further from the reference); with more than 8 queries
@@ -197,6 +199,13 @@ MI355X_API size_t mi355x_flash_attn_ext_workspace_size(const mi355x_tensor * q, 
 MI355X_API int    mi355x_flash_attn_ext(const mi355x_tensor * q, const mi355x_tensor * k, const mi355x_tensor * v,
                                         const mi355x_tensor * mask, const mi355x_tensor * dst, float scale, int mode,
                                         void * workspace, size_t workspace_size, void * stream);
+
+/* The same with an F32 mask (at most 8 queries, see above) whose f16 form — the result of the ggml_cast that precedes the
+ * first attention node of a decode step, src/whisper.cpp:2523 — is also written to `mask_f16` (F16 [KV, >=N]; rows < N),
+ * for the attention nodes of the later layers: the cast needs no launch of its own. */
+MI355X_API int    mi355x_flash_attn_ext_cast_mask(const mi355x_tensor * q, const mi355x_tensor * k, const mi355x_tensor * v,
+                                                  const mi355x_tensor * mask_f32, const mi355x_tensor * mask_f16, const mi355x_tensor * dst,
+                                                  float scale, int mode, void * workspace, size_t workspace_size, void * stream);
 
 /* elementwise / row ops ------------------------------------------------------------------------------ */
 

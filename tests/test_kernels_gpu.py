@@ -465,6 +465,37 @@ def test_flash_attn_reference_faithful(pkg, oracle, gpu, case):
     assert oracle.nmse(got, want) <= 1e-6      # same key order, same f16 accumulator: only exp() and dot-product ulps differ
 
 
+def test_flash_attn_few_queries_take_the_f32_mask(pkg, oracle, gpu):
+    # the few-query kernel reads the f32 tensor a graph would cast to f16 and rounds each value as the cast does: the same bits
+    # as with the f16 copy, also for values that are not representable in f16; with more than 8 queries it says no
+    lib = pkg.kernels()
+    for H, N, KV in ((4, 5, 300), (2, 1, 193), (3, 8, 64)):
+        q, kb, vb = _attention_inputs(oracle, H, N, KV, False, None)
+        m = (RNG.normal(size=(64, KV)) * 0.37).astype(np.float32)
+        m[:, KV // 2:][RNG.random((64, KV - KV // 2)) < 0.4] = -np.inf
+        m[:, 0] = 0.0
+        want, name = run_fa(pkg, gpu, q, kb, vb, oracle.f32_to_f16_bits(m), 0.125, pkg.FA_F16_SEQ)
+        assert name == "flash_attn.seq_row"
+        d_q, d_k, d_v, d_m = gpu.up(q), gpu.up(kb), gpu.up(vb), gpu.up(m)
+        d_o = torch.zeros((N, H, 64), dtype=torch.float32, device=gpu.dev)
+        pkg.check(lib.mi355x_flash_attn_ext(pkg.tensor(d_q, pkg.F32), pkg.tensor(d_k, pkg.F16), pkg.tensor(d_v, pkg.F16), pkg.tensor(d_m, pkg.F32),
+                                            pkg.tensor(d_o, pkg.F32), 0.125, pkg.FA_F16_SEQ, None, 0, gpu.stream))
+        assert np.array_equal(gpu.down(d_o).view(np.uint32), want.view(np.uint32))
+        # ... and leaves the f16 copy behind for later readers (rows of the queries; the rest is not touched)
+        d_c = torch.full((64, KV), 7, dtype=torch.int16, device=gpu.dev)
+        d_o.zero_()
+        pkg.check(lib.mi355x_flash_attn_ext_cast_mask(pkg.tensor(d_q, pkg.F32), pkg.tensor(d_k, pkg.F16), pkg.tensor(d_v, pkg.F16), pkg.tensor(d_m, pkg.F32),
+                                                      pkg.tensor(d_c, pkg.F16), pkg.tensor(d_o, pkg.F32), 0.125, pkg.FA_F16_SEQ, None, 0, gpu.stream))
+        assert np.array_equal(gpu.down(d_o).view(np.uint32), want.view(np.uint32))
+        copy = gpu.down(d_c).view(np.uint16)
+        assert np.array_equal(copy[:N], oracle.f32_to_f16_bits(m)[:N]) and np.all(copy[N:] == 7)
+    q, kb, vb = _attention_inputs(oracle, 2, 9, 64, False, None)
+    d_m = gpu.up(np.zeros((64, 64), dtype=np.float32))
+    d_o = torch.zeros((9, 2, 64), dtype=torch.float32, device=gpu.dev)
+    assert lib.mi355x_flash_attn_ext(pkg.tensor(gpu.up(q), pkg.F32), pkg.tensor(gpu.up(kb), pkg.F16), pkg.tensor(gpu.up(vb), pkg.F16), pkg.tensor(d_m, pkg.F32),
+                                     pkg.tensor(d_o, pkg.F32), 0.125, pkg.FA_F16_SEQ, None, 0, gpu.stream) == -1
+
+
 @pytest.mark.parametrize("case", [dict(H=2, N=70, KV=100), dict(H=3, N=200, KV=1536, flat=True, pad_from=1500), dict(H=2, N=100, KV=100, mask="causal")])
 def test_flash_attn_f16_fma_mode(pkg, oracle, gpu, case):
     H, N, KV = case["H"], case["N"], case["KV"]

@@ -77,6 +77,7 @@ def kernels() -> C.CDLL:
             "mi355x_flash_attn_ext_kernel_name": (C.c_char_p, [T, T, C.c_int]),
             "mi355x_flash_attn_ext_workspace_size": (C.c_size_t, [T, T]),
             "mi355x_flash_attn_ext": (C.c_int, [T, T, T, T, T, C.c_float, C.c_int, P, C.c_size_t, P]),
+            "mi355x_flash_attn_ext_cast_mask": (C.c_int, [T, T, T, T, T, T, C.c_float, C.c_int, P, C.c_size_t, P]),
             "mi355x_binary": (C.c_int, [C.c_int, T, T, T, P]),
             "mi355x_scale": (C.c_int, [T, T, C.c_float, P]),
             "mi355x_gelu": (C.c_int, [T, T, P]),

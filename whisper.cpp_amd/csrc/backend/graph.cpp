@@ -580,6 +580,28 @@ struct graph_runner {
         return n && n->op == GGML_OP_MUL_MAT && n->src[1] == key;
     }
 
+    // A decode step casts its f32 mask to f16 (src/whisper.cpp:2523) right in front of its first FLASH_ATTN_EXT node.  When
+    // that node runs on the few-query kernel, the cast is not launched — it is a launch on the step's critical path — and
+    // the attention launch rounds the f32 values itself and leaves the f16 copy behind for the later layers' nodes
+    // (mi355x_flash_attn_ext_cast_mask).  The f32 tensor is read in the launch that takes the cast's place, so the
+    // allocator's reuse of its memory after the cast (ggml/src/ggml-alloc.c:640-667) is not a concern.
+    const ggml_tensor * cast_dst = nullptr, * cast_src = nullptr;          // a cast that the next attention node carries out
+    bool next_attention_casts(int i) const {
+        const ggml_tensor * n = g->nodes[i], * s0 = n->src[0];
+        if (!ctx->fuse || ctx->exact || n->src[1] != n || s0->type != GGML_TYPE_F32 || n->type != GGML_TYPE_F16 ||
+            (n->flags & GGML_TENSOR_FLAG_OUTPUT) || !ggml_is_contiguous(s0) || !ggml_is_contiguous(n) || !ggml_are_same_shape(s0, n) ||
+            n->ne[2] != 1 || n->ne[3] != 1 || n->view_src) return false;
+        int j = i + 1;
+        while (node_at(j) && (is_view_op(node_at(j)->op) || ggml_is_empty(node_at(j)))) {
+            if (node_at(j)->src[0] == n || node_at(j)->view_src == n) return false;       // a view of the copy: someone else reads it
+            ++j;
+        }
+        const ggml_tensor * r = node_at(j);
+        if (!r || r->op != GGML_OP_FLASH_ATTN_EXT || r->src[3] != n || r->src[0]->ne[1] > n->ne[1]) return false;
+        mi355x_tensor vq = to_view(r->src[0]), vk = to_view(r->src[1]);
+        return strcmp(mi355x_flash_attn_ext_kernel_name(&vq, &vk, MI355X_FA_F16_SEQ), "flash_attn.seq_row") == 0;
+    }
+
     // the workspace copy of the activations goes stale when something overwrites them
     const ggml_tensor * cached_x = nullptr;
     void note_write(const ggml_tensor * out) {
@@ -625,6 +647,7 @@ struct graph_runner {
                 return 1;
             }
             case GGML_OP_CPY: case GGML_OP_CONT: case GGML_OP_DUP: {
+                if (n->op == GGML_OP_CPY && next_attention_casts(i)) { cast_dst = n; cast_src = s0; return 1; }
                 const ggml_tensor * dt = n->op == GGML_OP_CPY ? s1 : n;
                 mi355x_tensor a = to_view(s0), d = to_view(dt);
                 launch_scope ls(ctx, "cpy", nbytes_of(s0) + nbytes_of(dt), 0.0);
@@ -672,6 +695,8 @@ struct graph_runner {
             }
             case GGML_OP_FLASH_ATTN_EXT: {
                 const ggml_tensor * k = n->src[1], * v = n->src[2], * m = n->src[3];
+                const ggml_tensor * m16 = nullptr;          // the f16 copy this launch leaves behind
+                if (m && m == cast_dst) { m16 = m; m = cast_src; cast_dst = cast_src = nullptr; }
                 float scale; memcpy(&scale, n->op_params, sizeof(float));
                 mi355x_tensor vq = to_view(s0), vk = to_view(k), vv = to_view(v), vm, vd = to_view(n);
                 if (m) vm = to_view(m);
@@ -691,8 +716,12 @@ struct graph_runner {
                 if (key && !ctx->reserve_workspace(image_bytes + 256)) key = nullptr;
                 {
                     launch_scope ls(ctx, name, bytes + (key ? image_bytes : 0), flops);
-                    status = mi355x_flash_attn_ext(&vq, &vk, &vv, m ? &vm : nullptr, &vd, scale,
-                                                   mode | (!key ? 0 : form == 1 ? MI355X_FA_EMIT_F16 : MI355X_FA_EMIT_Q8_0),
+                    const int flags = mode | (!key ? 0 : form == 1 ? MI355X_FA_EMIT_F16 : MI355X_FA_EMIT_Q8_0);
+                    if (m16) {
+                        mi355x_tensor vm16 = to_view(m16);
+                        status = mi355x_flash_attn_ext_cast_mask(&vq, &vk, &vv, &vm, &vm16, &vd, scale, flags, key ? ctx->ws : nullptr, key ? ctx->ws_size : 0, ctx->stream);
+                    } else
+                    status = mi355x_flash_attn_ext(&vq, &vk, &vv, m ? &vm : nullptr, &vd, scale, flags,
                                                    key ? ctx->ws : nullptr, key ? ctx->ws_size : 0, ctx->stream);
                 }
                 if (key && status == MI355X_OK) workspace_holds(key, ctx->ws_slot, form);

@@ -32,6 +32,9 @@ struct fa_args {
     int64_t k_nb1, k_nb2, k_nb3;
     int64_t v_nb1, v_nb2, v_nb3;
     int64_t m_nb1;
+    int     mask_f32;                // the mask is F32 and is rounded to f16 as it is read (k_fattn_seq_row only)
+    half_t * mask_copy;              // when set (with mask_f32): head 0 also stores the rounded values here, rows of mc_nb1 bytes
+    int64_t mc_nb1;
     int64_t hk_ratio, hv_ratio;      // q heads per k head / v head (broadcast)
     int64_t ne3, k_ne3_ratio, v_ne3_ratio;
     float scale;
@@ -203,7 +206,7 @@ __global__ void __launch_bounds__(256) k_fattn_seq_row(fa_args a, int kv_pad) {
         const float * qp = (const float *)(a.q + n * a.q_nb1 + h * a.q_nb2 + i3 * a.q_nb3);
         const char *  kb = a.k + (h / a.hk_ratio) * a.k_nb2 + (i3 / a.k_ne3_ratio) * a.k_nb3;
         const char *  vb = a.v + (h / a.hv_ratio) * a.v_nb2 + (i3 / a.v_ne3_ratio) * a.v_nb3;
-        const half_t * mp = a.mask ? (const half_t *)(a.mask + n * a.m_nb1) : nullptr;
+        const char * mp = a.mask ? a.mask + n * a.m_nb1 : nullptr;
         const int stid = tid - WAVE, pw = wave - 1;
 
         // Rows are read eight lanes to a row (16 bytes each): lane (r = lane / 8, c = lane % 8) takes piece c of the rows
@@ -223,8 +226,11 @@ __global__ void __launch_bounds__(256) k_fattn_seq_row(fa_args a, int kv_pad) {
         half8_t krow[8];
         u32x4 vrow[8];
         uint16_t mbits = 0;                                // the mask value of key `stid` of the stage as loaded (f16)
-        const uint16_t * mrow = mp ? (const uint16_t *) mp : (const uint16_t *) kb;      // without a mask: any readable address
-        const int64_t m_step = mp ? 1 : 0;
+        // The mask comes as f16, or as the f32 tensor an f16 copy would have been made of (then each value is rounded here
+        // as that copy rounds it).  Both forms are read, from an address that is readable either way, and one is kept.
+        const uint16_t * mrow  = mp && !a.mask_f32 ? (const uint16_t *) mp : (const uint16_t *) kb;   // without such a mask: any readable address
+        const float *    mrowf = mp && a.mask_f32 ? (const float *) mp : (const float *) kb;
+        const int64_t m_step = mp && !a.mask_f32 ? 1 : 0, m_stepf = mp && a.mask_f32 ? 1 : 0;
         auto load_k = [&](int s) __attribute__((always_inline)) {
             const int key0 = s * ROW_STAGE + pw * WAVE + 8 * r8;
 #pragma unroll
@@ -233,7 +239,10 @@ __global__ void __launch_bounds__(256) k_fattn_seq_row(fa_args a, int kv_pad) {
                 krow[i] = *(const half8_t *)(kb + (int64_t) kc * a.k_nb1 + 16 * c8);
             }
             const int key = s * ROW_STAGE + stid;
-            mbits = mrow[(key < KV ? key : KV - 1) * m_step];
+            const uint16_t m16 = mrow[(key < KV ? key : KV - 1) * m_step];
+            const float    m32 = mrowf[(key < KV ? key : KV - 1) * m_stepf];
+            mbits = a.mask_f32 ? f2h_bits(m32) : m16;
+            if (a.mask_copy && h == 0 && key < KV) *(uint16_t *)((char *) a.mask_copy + n * a.mc_nb1 + (int64_t) key * 2) = mbits;
         };
         auto load_v = [&](int s) __attribute__((always_inline)) {
             const int key0 = s * ROW_STAGE + pw * WAVE + 8 * r8;
@@ -1002,9 +1011,9 @@ extern "C" size_t mi355x_flash_attn_ext_workspace_size(const mi355x_tensor * q, 
     return 0;
 }
 
-extern "C" int mi355x_flash_attn_ext(const mi355x_tensor * q, const mi355x_tensor * k, const mi355x_tensor * v,
-                                     const mi355x_tensor * mask, const mi355x_tensor * dst, float scale, int mode,
-                                     void * workspace, size_t workspace_size, void * stream) {
+static int flash_attn_ext(const mi355x_tensor * q, const mi355x_tensor * k, const mi355x_tensor * v,
+                          const mi355x_tensor * mask, const mi355x_tensor * mask_f16, const mi355x_tensor * dst, float scale, int mode,
+                          void * workspace, size_t workspace_size, void * stream) {
     if (!q || !k || !v || !dst) return MI355X_ERR_INVALID;
     const bool emit = mode & MI355X_FA_EMIT_F16, emit_q8 = mode & MI355X_FA_EMIT_Q8_0;
     mode &= ~(MI355X_FA_EMIT_F16 | MI355X_FA_EMIT_Q8_0);
@@ -1018,8 +1027,14 @@ extern "C" int mi355x_flash_attn_ext(const mi355x_tensor * q, const mi355x_tenso
     if (k->ne[3] <= 0 || v->ne[3] <= 0 || q->ne[3] % k->ne[3] != 0 || q->ne[3] % v->ne[3] != 0) return MI355X_ERR_INVALID;
     if (dst->ne[0] != FA_D || dst->ne[1] != H || dst->ne[2] != N || dst->ne[3] != q->ne[3] || !is_contiguous(dst)) return MI355X_ERR_INVALID;
     if (mask) {
-        if (mask->type != MI355X_TYPE_F16) return MI355X_ERR_UNSUPPORTED;
-        if (mask->ne[0] != KV || mask->ne[1] < N || mask->nb[0] != 2) return MI355X_ERR_INVALID;
+        // an F32 mask is what the few-query kernel takes in place of its f16 copy (same values after its own rounding)
+        if (mask->type == MI355X_TYPE_F32) { if (fa_kernel(q, k, mode) != FA_K_SEQ_ROW) return MI355X_ERR_UNSUPPORTED; }
+        else if (mask->type != MI355X_TYPE_F16) return MI355X_ERR_UNSUPPORTED;
+        if (mask->ne[0] != KV || mask->ne[1] < N || mask->nb[0] != type_size(mask->type)) return MI355X_ERR_INVALID;
+    }
+    if (mask_f16) {                                        // the f16 copy of an F32 mask, written on the way
+        if (!mask || mask->type != MI355X_TYPE_F32 || mask_f16->type != MI355X_TYPE_F16) return MI355X_ERR_UNSUPPORTED;
+        if (mask_f16->ne[0] != KV || mask_f16->ne[1] < N || mask_f16->nb[0] != 2 || !mask_f16->data) return MI355X_ERR_INVALID;
     }
     auto al16 = [](const mi355x_tensor * t) {
         return (uintptr_t) t->data % 16 == 0 && t->nb[1] % 16 == 0 && t->nb[2] % 16 == 0 && t->nb[3] % 16 == 0;
@@ -1037,6 +1052,8 @@ extern "C" int mi355x_flash_attn_ext(const mi355x_tensor * q, const mi355x_tenso
     a.k_nb1 = k->nb[1]; a.k_nb2 = k->nb[2]; a.k_nb3 = k->nb[3];
     a.v_nb1 = v->nb[1]; a.v_nb2 = v->nb[2]; a.v_nb3 = v->nb[3];
     a.m_nb1 = mask ? mask->nb[1] : 0;
+    a.mask_f32 = mask && mask->type == MI355X_TYPE_F32;
+    a.mask_copy = mask_f16 ? (half_t *) mask_f16->data : nullptr; a.mc_nb1 = mask_f16 ? (int64_t) mask_f16->nb[1] : 0;
     a.hk_ratio = H / k->ne[2]; a.hv_ratio = H / v->ne[2];
     a.ne3 = q->ne[3]; a.k_ne3_ratio = q->ne[3] / k->ne[3]; a.v_ne3_ratio = q->ne[3] / v->ne[3];
     a.scale = scale;
@@ -1082,4 +1099,17 @@ extern "C" int mi355x_flash_attn_ext(const mi355x_tensor * q, const mi355x_tenso
         }
     }
     return launch_status();
+}
+
+extern "C" int mi355x_flash_attn_ext(const mi355x_tensor * q, const mi355x_tensor * k, const mi355x_tensor * v,
+                                     const mi355x_tensor * mask, const mi355x_tensor * dst, float scale, int mode,
+                                     void * workspace, size_t workspace_size, void * stream) {
+    return flash_attn_ext(q, k, v, mask, nullptr, dst, scale, mode, workspace, workspace_size, stream);
+}
+
+extern "C" int mi355x_flash_attn_ext_cast_mask(const mi355x_tensor * q, const mi355x_tensor * k, const mi355x_tensor * v,
+                                               const mi355x_tensor * mask_f32, const mi355x_tensor * mask_f16, const mi355x_tensor * dst, float scale, int mode,
+                                               void * workspace, size_t workspace_size, void * stream) {
+    if (!mask_f32 || !mask_f16) return MI355X_ERR_INVALID;
+    return flash_attn_ext(q, k, v, mask_f32, mask_f16, dst, scale, mode, workspace, workspace_size, stream);
 }
