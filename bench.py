@@ -124,23 +124,24 @@ def main() -> int:
                             "instructions per (query, key, d): 150 us per launch at the 2.0 ns per instruction the vector units sustain under this load, "
                             "plus 60 us of score / factor phases that are vector work as well; that is the bound that applies")
 
-    # ---- the same window with the packed f16 attention option (an optional arithmetic, reported beside the headline) -------
-    packed = run_harness(["bench", "--model", enc_model, "--what", "encoder", "--backend", "gpu", "--reps", str(a.steps),
-                          "--warmup", str(a.warmup), "--threads", str(a.threads)], env={"GGML_MI355X_FA_PACKED": "1"})
-
     # ---- and with f32 matrix-core attention (faster, but outside the whole-model parity bound: reported, never the headline) ----
     f32att = run_harness(["bench", "--model", enc_model, "--what", "encoder", "--backend", "gpu", "--reps", str(a.steps),
                           "--warmup", str(a.warmup), "--threads", str(a.threads)], env={"GGML_MI355X_FA_ACCUM": "1"})
 
-    # ---- decode: 224 five-token steps (the shape of a 5-beam search step) on large-v3-turbo Q8_0 ----------------------------
-    dec = run_harness(["bench", "--model", dec_model, "--what", "decoder", "--backend", "gpu", "--reps", "3", "--warmup", "2",
-                       "--steps", "224", "--batch", "5", "--profile", "--threads", str(a.threads)])
+    # ---- decode: 224 five-token steps (the shape of a 5-beam search step) on large-v3-turbo Q8_0; step i writes positions
+    # 2 i .. 2 i + 4 of the self-attention cache, so that it grows to its 448 positions over the run --------------------------
+    dec_args = ["bench", "--model", dec_model, "--what", "decoder", "--reps", "3", "--warmup", "2", "--steps", "224", "--batch", "5", "--kv-stride", "2"]
+    dec = run_harness(dec_args + ["--backend", "gpu", "--profile", "--threads", str(a.threads)])
+    # the same with every logits download a blocking copy (the pinned host mirror of the logits switched off)
+    dec_nomirror = run_harness(dec_args + ["--backend", "gpu", "--threads", str(a.threads)], env={"GGML_MI355X_NO_MIRROR": "1"})
     dk = {k["kernel"]: k for k in dec["kernels"]}
     # the logits product, 70.5 MB of Q8_0 blocks: the one GEMV that bandwidth bounds
     gemv_name = "mul_mat.gemv_q8_0.vocab"
     gemv = dk.get(gemv_name)
-    decode = {"model": "large-v3-turbo Q8_0", "steps": dec["steps"], "beams": dec["batch"], "ms_per_step": round(dec["ms_per_step"], 4),
-              "steps_per_s": round(dec["steps_per_s"], 1), "beam_tokens_per_s": round(dec["batch_tokens_per_s"], 1)}
+    decode = {"model": "large-v3-turbo Q8_0", "steps": dec["steps"], "beams": dec["batch"], "max_kv_positions": dec["max_kv_positions"],
+              "ms_per_step": round(dec["ms_per_step"], 4), "steps_per_s": round(dec["steps_per_s"], 1), "beam_tokens_per_s": round(dec["batch_tokens_per_s"], 1),
+              "launches_per_step": dec["launches_per_step"], "logits_reads_from_pinned_mirror_per_step": dec["downloads_from_mirror_per_step"],
+              "ms_per_step_with_blocking_logits_downloads": round(dec_nomirror["ms_per_step"], 4)}
     if gemv:
         decode["gemv_roofline"] = kernel_roofline(gemv_name, gemv)
         decode["gemv_roofline"]["traffic"] = round(72.8e6 + 3.2e6)    # FETCH_SIZE + WRITE_SIZE per launch of k_gemv_q8_0_tiles (profiles/)
@@ -160,14 +161,24 @@ def main() -> int:
                             "algorithmic_mb_per_launch": mel["algorithmic_mb"], "traffic": 11100000,      # FETCH_SIZE + WRITE_SIZE of the three launches (profiles/)
                             "note": "samples in + mel out; 0.97 GFLOP of f64 multiply-adds over 5 MB (18 % of the vector f64 peak in the frames kernel): bound by the issue rate of v_fma_f64 and three launch latencies, not by HBM"}}
 
-    # ---- CPU baseline: the reference's ggml CPU backend, same model file, same window ------------------------------------------
+    # ---- CPU baseline: the reference's ggml CPU backend, same model files, same inputs ----------------------------------------
     cpu_baseline = None
     if not a.no_cpu:
-        cpu = run_harness(["bench", "--model", enc_model, "--what", "encoder", "--backend", "cpu", "--reps", "2", "--warmup", "1",
+        cpu = run_harness(["bench", "--model", enc_model, "--what", "encoder", "--backend", "cpu", "--reps", "5", "--warmup", "1",
                            "--threads", str(a.threads)], timeout=1500)
-        cpu_baseline = {"value": round(cpu["ms_per_step"], 2), "unit": "ms", "cores": a.threads, "kind": "reference",
-                        "sample": "1 warm-up + 2 timed whisper_encode() calls of the same large-v3 Q5_0 model file and mel window on the ggml CPU "
-                                  "backend (AVX2/FMA/F16C build of the reference, OpenMP)"}
+        cpu1 = run_harness(["bench", "--model", enc_model, "--what", "encoder", "--backend", "cpu", "--reps", "1", "--warmup", "0",
+                            "--threads", "1"], timeout=1500)
+        cpu_baseline = {"value": round(cpu["encode_ms_median"], 2), "unit": "ms", "cores": a.threads, "kind": "reference",
+                        "sample": "median of 5 timed whisper_encode() calls after 1 warm-up, same large-v3 Q5_0 model file and mel window, on the ggml CPU "
+                                  "backend (AVX2/FMA/F16C build of the reference, OpenMP), timed by whisper_get_timings as whisper-bench does",
+                        "one_thread": {"value": round(cpu1["encode_ms_median"], 1), "unit": "ms", "cores": 1, "sample": "one whisper_encode() call of the same window, no warm-up"}}
+        dcpu = run_harness(dec_args + ["--backend", "cpu", "--threads", str(a.threads)], timeout=1500)
+        dcpu1 = run_harness(["bench", "--model", dec_model, "--what", "decoder", "--reps", "1", "--warmup", "1", "--steps", "56", "--batch", "5", "--kv-stride", "8",
+                             "--backend", "cpu", "--threads", "1"], timeout=1500)
+        decode["cpu_baseline"] = {"value": round(dcpu["ms_per_step"], 3), "unit": "ms per 5-token step", "cores": a.threads, "kind": "reference",
+                                  "sample": "the same 224 steps (median of 3 passes) through whisper_decode() on the ggml CPU backend",
+                                  "one_thread": {"value": round(dcpu1["ms_per_step"], 3), "unit": "ms per 5-token step", "cores": 1,
+                                                 "sample": "56 steps, every fourth of the walk over the cache (stride 8), one pass"}}
 
     out = {
         "metric": "encoder_ms_per_30s_window",
@@ -189,9 +200,9 @@ def main() -> int:
                    "flash_attn": True, "algorithmic_gflop": 2597.2},
         "encode_ms_median": round(enc["encode_ms_median"], 4),
         "encode_tflops": round(2597.2 / ms_per_step, 2),
-        "encoder_ms_with_fa_packed_option": round(packed["ms_per_step"], 4),
         "encoder_ms_with_f32_mfma_attention_option": round(f32att["ms_per_step"], 4),
-        "decode_tok_per_s": decode["steps_per_s"],
+        "decode_steps_per_s": decode["steps_per_s"],
+        "decode_beam_tokens_per_s": decode["beam_tokens_per_s"],
         "decode": decode,
         "log_mel": log_mel,
         "kernel_breakdown": breakdown,

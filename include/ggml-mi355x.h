@@ -47,6 +47,7 @@ GGML_BACKEND_API int                ggml_backend_score(void);
  *   "ggml_backend_get_features"        ggml_backend_get_features_t
  *   "ggml_backend_mi355x_set_option"   ggml_backend_mi355x_set_option_t
  *   "ggml_backend_mi355x_get_stats"    ggml_backend_mi355x_get_stats_t
+ *   "ggml_backend_mi355x_get_counters" ggml_backend_mi355x_get_counters_t
  *   "ggml_backend_mi355x_log_mel"      ggml_backend_mi355x_log_mel_t
  */
 
@@ -55,15 +56,13 @@ GGML_BACKEND_API int                ggml_backend_score(void);
  * "exact" (0/1, default 0: 0 reproduces the two roundings that the reference's CPU backend applies — Q8_0-rounded
  * activations in front of quantized MUL_MAT, f16 key-by-key V accumulation in FLASH_ATTN_EXT; 1 keeps f16 activations
  * and f32 accumulators, which is closer to exact arithmetic and further from the reference),
- * "fa_accum" (0/1/2, default 0: how FLASH_ATTN_EXT over more than 8 queries accumulates V.  0: key by key with an f16
- * accumulator, f32 fma + f16 store — the reference's x86 build, and the only setting that keeps whole-model logits within
- * 1e-3 NMSE of the CPU backend.  1: f32 accumulators with both products on the matrix cores — six times faster, within
- * the per-op bound, but the reference's f16 rounding is then missing and whole-model logits sit several 1e-3 away.
- * 2: key by key with f16 fused multiply-adds, the arithmetic of the reference's Arm fp16 build, simd-mappings.h:67-78 —
- * a third of the accumulation work, about 1e-7 NMSE per op away from the x86 build),
- * "fa_packed" (0/1: the same as "fa_accum" 2/0).
- * The environment variables GGML_MI355X_FUSE, GGML_MI355X_PROFILE, GGML_MI355X_EXACT, GGML_MI355X_FA_ACCUM and
- * GGML_MI355X_FA_PACKED give the initial values.
+ * "fa_accum" (0/1, default 0: how FLASH_ATTN_EXT over more than 8 queries accumulates V.  0: key by key with an f16
+ * accumulator, f32 fma + f16 store — the reference's sequence (ops.cpp:6793-6807), and the only setting that keeps
+ * whole-model logits within 1e-3 NMSE of the CPU backend.  1: f32 accumulators with both products on the matrix cores —
+ * six times faster, within the per-op bound, but the reference's f16 rounding is then missing and whole-model logits sit
+ * several 1e-3 away).
+ * The environment variables GGML_MI355X_FUSE, GGML_MI355X_PROFILE, GGML_MI355X_EXACT and GGML_MI355X_FA_ACCUM give the
+ * initial values.
  * backend == NULL addresses every live MI355X backend of the process (a host such as whisper.cpp keeps its
  * backends private). */
 typedef int (*ggml_backend_mi355x_set_option_t)(ggml_backend_t backend, const char * name, int value);
@@ -73,6 +72,16 @@ typedef int (*ggml_backend_mi355x_set_option_t)(ggml_backend_t backend, const ch
  * into buf (at most size bytes, NUL-terminated), resets the counters when `reset` is non-zero and returns the
  * length needed. */
 typedef size_t (*ggml_backend_mi355x_get_stats_t)(ggml_backend_t backend, char * buf, size_t size, int reset);
+
+/* What graph_compute was handed and did since the last reset (always counted, whatever "profile" says):
+ * out[0] graph_compute calls, out[1] nodes of the graphs as received, out[2] those of them that are not view ops or empty
+ * tensors (every one of them is carried out by a launch of this backend: there is no other path), out[3] kernel
+ * launches, out[4] get_tensor calls served from the pinned host mirror of a graph output, out[5] get_tensor calls that
+ * were a blocking device-to-host copy, out[6..7] zero.  A host that sees one call per graph it computes, with the graph's
+ * full node count, knows that the scheduler (ggml_backend_sched_split_graph, ggml/src/ggml-backend.cpp:863-1317) left
+ * no node to another backend. */
+#define GGML_MI355X_N_COUNTERS 8
+typedef void (*ggml_backend_mi355x_get_counters_t)(ggml_backend_t backend, int64_t out[GGML_MI355X_N_COUNTERS], int reset);
 
 /* The log-mel front end (log_mel_spectrogram, src/whisper.cpp:3181-3270 — what whisper_pcm_to_mel, :3881, runs on
  * host threads) on device `device`, for a host that holds its samples in host memory: uploads the 16 kHz f32 samples

@@ -180,12 +180,8 @@ MI355X_API int    mi355x_mul_mat_q8_0_tiles(const void * tiles, int64_t K, int64
  * mode: MI355X_FA_F16_SEQ accumulates V in f16, key by key in order, as the reference does (ops.cpp:6793-6807) —
  * with near-uniform attention over ~1500 keys that rounding sequence dominates the low bits of the result;
  * MI355X_FA_F32 accumulates in f32 (closer to exact arithmetic, further from the reference); with more than 8 queries
- * both products run on the matrix cores with the softmax probabilities as f16 operands.
- * MI355X_FA_F16_PACKED keeps the key order and the f16 accumulator but forms each step as one f16 fused multiply-add
- * with the softmax factor converted to f16 — the arithmetic of the reference's Arm fp16 build (GGML_F16_VEC_FMA =
- * vfmaq_f16, ggml/src/ggml-cpu/simd-mappings.h:67-78) rather than of its x86 build; about 1e-7 NMSE from the latter,
- * a third of the accumulation work.  It applies to more than 8 queries (fewer run as MI355X_FA_F16_SEQ). */
-enum mi355x_fa_mode { MI355X_FA_F16_SEQ = 0, MI355X_FA_F32 = 1, MI355X_FA_F16_PACKED = 2,
+ * both products run on the matrix cores with the softmax probabilities as f16 operands. */
+enum mi355x_fa_mode { MI355X_FA_F16_SEQ = 0, MI355X_FA_F32 = 1,
     /* or-ed into the mode: also write into `workspace` (16-byte aligned, N * H * ne3 * 64 halves) the image of dst that
      * a following MUL_MAT with quantized weights wants — rows [N][H * 64] rounded to Q8_0 as quantize_row_q8_0 does and
      * stored as f16(q * d) (then pass MI355X_MM_WS_READY there).  More than 8 queries; MI355X_ERR_UNSUPPORTED otherwise. */
@@ -252,7 +248,8 @@ MI355X_API int mi355x_soft_max(const mi355x_tensor * src, const mi355x_tensor * 
 MI355X_API int mi355x_cpy(const mi355x_tensor * src, const mi355x_tensor * dst, void * stream);
 
 /* GET_ROWS (ggml/src/ggml-cpu/ops.cpp:4146-4188, 4313): dst[:, i] = dequant(src0[:, ids[i]]).
- * src0: Q5_0 | Q8_0 | F16 | F32, ids: I32, dst: F32. */
+ * src0: Q5_0 | Q8_0 | F16 | F32, ids: I32, dst: F32.  An index outside [0, src0 ne1) — on which the reference aborts the
+ * process (GGML_ASSERT, ops.cpp:4174) — reads nothing and yields a row of NaN. */
 MI355X_API int mi355x_get_rows(const mi355x_tensor * src0, const mi355x_tensor * ids, const mi355x_tensor * dst, void * stream);
 /* dst[:, i] = dequant(src0 row ids0[i]) + src1 row ids1[i]: the token embedding plus the positional embedding of a
  * decoder input (GET_ROWS, GET_ROWS and ADD of src/whisper.cpp:2526-2529, ops.cpp:4313 and binary-ops.cpp:49-142) in one

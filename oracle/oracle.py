@@ -116,11 +116,8 @@ def mul_mat_f16_f16(a_bits, b_bits) -> np.ndarray:
     return dst
 
 
-def flash_attn_ext(q, k_bits, v_bits, mask_bits, scale: float, f16_fma: bool = False) -> np.ndarray:
-    """q f32 [H, N, D], k/v f16 bits [H, KV, D], mask f16 bits [N, KV] or None -> f32 [N, H, D]
-
-    f16_fma: accumulate V as the reference's Arm fp16 build does (f16 factor, f16 fused multiply-add) instead of as its
-    x86 build does (f32 fma, result stored as f16)."""
+def flash_attn_ext(q, k_bits, v_bits, mask_bits, scale: float) -> np.ndarray:
+    """q f32 [H, N, D], k/v f16 bits [H, KV, D], mask f16 bits [N, KV] or None -> f32 [N, H, D]"""
     q = _f32(q)
     k = np.ascontiguousarray(k_bits, dtype=np.uint16)
     v = np.ascontiguousarray(v_bits, dtype=np.uint16)
@@ -128,19 +125,9 @@ def flash_attn_ext(q, k_bits, v_bits, mask_bits, scale: float, f16_fma: bool = F
     kv = k.shape[1]
     m = None if mask_bits is None else np.ascontiguousarray(mask_bits, dtype=np.uint16)
     dst = np.empty((n, h, d), dtype=np.float32)
-    fn = lib().oracle_flash_attn_ext_f16fma if f16_fma else lib().oracle_flash_attn_ext
-    fn(_p(q), _p(k), _p(v), _p(m) if m is not None else None, _p(dst),
+    lib().oracle_flash_attn_ext(_p(q), _p(k), _p(v), _p(m) if m is not None else None, _p(dst),
        C.c_int64(n), C.c_int64(kv), C.c_int64(h), C.c_int64(d), C.c_float(scale))
     return dst
-
-
-def f64_to_f16_bits(x) -> np.ndarray:
-    """round-to-nearest-even of doubles straight to f16 (the single rounding of an f16 fused multiply-add)"""
-    x = np.ascontiguousarray(x, dtype=np.float64)
-    fn = lib().oracle_f64_to_f16
-    fn.restype = C.c_uint16
-    fn.argtypes = [C.c_double]
-    return np.array([fn(float(v)) for v in x.reshape(-1)], dtype=np.uint16).reshape(x.shape)
 
 
 def norm(x, eps: float) -> np.ndarray:

@@ -16,8 +16,7 @@
  * (oracle/_ref: libggml-base.so for the quantizers, the ggml CPU backend for the graph ops) and against
  * closed forms that do not share its structure (numpy float64 GEMM / softmax / layer-norm, brute force over
  * all 65536 f16 bit patterns for the conversions, all nibble/high-bit patterns for dequantization).
- * One exception, PARITY UNPINNED: oracle_flash_attn_ext_f16fma restates the accumulation of the reference's Arm fp16
- * build, which cannot be built or run here; only its rounding primitive (oracle_f64_to_f16) is pinned, against numpy.
+ * No function here is left without such a check.
  */
 #include <math.h>
 #include <stdint.h>
@@ -240,46 +239,8 @@ void oracle_mul_mat_f16_f16(const uint16_t * a, const uint16_t * b, float * dst,
  * after every key (ops.cpp:6793-6807; the F16C build's ggml_vec_mad_f16 / ggml_vec_scale_f16 compute in f32 and
  * store f16), the softmax sum S and maximum M are f32.
  * ------------------------------------------------------------------------------------------------------- */
-static void flash_attn_ext_impl(const float * q, const uint16_t * k, const uint16_t * v, const uint16_t * mask, float * dst,
-                                int64_t N, int64_t KV, int64_t H, int64_t D, float scale, int f16_fma);
-
 void oracle_flash_attn_ext(const float * q, const uint16_t * k, const uint16_t * v, const uint16_t * mask, float * dst,
                            int64_t N, int64_t KV, int64_t H, int64_t D, float scale) {
-    flash_attn_ext_impl(q, k, v, mask, dst, N, KV, H, D, scale, 0);
-}
-
-/* The V accumulation as the reference's Arm fp16 build performs it (__ARM_FEATURE_FP16_VECTOR_ARITHMETIC:
- * ggml_vec_mad_f16 / ggml_vec_scale_f16 with GGML_F16_VEC_SET1 = vdupq_n_f16, GGML_F16_VEC_FMA = vfmaq_f16,
- * GGML_F16_VEC_MUL = vmulq_f16; ggml/src/ggml-cpu/simd-mappings.h:67-78, vec.h:180-197, 295-310): the factor is
- * converted to f16 and every step is one f16 fused multiply-add (a single rounding of the exact result).  Scores,
- * maximum and the softmax sum stay as in the x86 path above.  PARITY UNPINNED: no Arm build of the reference can run
- * here; the arithmetic is restated from the intrinsics' definitions (exact product and sum in double, one rounding). */
-void oracle_flash_attn_ext_f16fma(const float * q, const uint16_t * k, const uint16_t * v, const uint16_t * mask, float * dst,
-                                  int64_t N, int64_t KV, int64_t H, int64_t D, float scale) {
-    flash_attn_ext_impl(q, k, v, mask, dst, N, KV, H, D, scale, 1);
-}
-
-/* one rounding of a double that holds an exact f16 x f16 (+ f16) result: via f32 is safe only if no double rounding can
- * occur, so round directly */
-uint16_t oracle_f64_to_f16(double x) {
-    const float f = (float) x;                      /* candidate; fix the ties-and-near-ties the f32 step may have moved */
-    uint16_t h = oracle_f32_to_f16(f);
-    const double back = (double) oracle_f16_to_f32(h);
-    if (back == x || isinf(back) || isnan(x)) return h;
-    /* neighbours of h in the direction of x */
-    const uint16_t up = (uint16_t)(h + 1), dn = (uint16_t)(h - 1);
-    uint16_t cand[3] = { h, up, dn };
-    double best = fabs(back - x); uint16_t bh = h;
-    for (int i = 1; i < 3; ++i) {
-        if ((cand[i] & 0x7C00) == 0x7C00 && (h & 0x7C00) != 0x7C00) continue;
-        const double d = fabs((double) oracle_f16_to_f32(cand[i]) - x);
-        if (d < best || (d == best && !(cand[i] & 1))) { best = d; bh = cand[i]; }
-    }
-    return bh;
-}
-
-static void flash_attn_ext_impl(const float * q, const uint16_t * k, const uint16_t * v, const uint16_t * mask, float * dst,
-                                int64_t N, int64_t KV, int64_t H, int64_t D, float scale, int f16_fma) {
     uint16_t * vkq = (uint16_t *) malloc((size_t) D * sizeof(uint16_t));
     float * qh = (float *) malloc((size_t) D * sizeof(float));
     for (int64_t h = 0; h < H; ++h) for (int64_t n = 0; n < N; ++n) {
@@ -296,20 +257,10 @@ static void flash_attn_ext_impl(const float * q, const uint16_t * k, const uint1
             float ms = 1.0f, vs = 1.0f;
             if (s > M) {
                 M = s; ms = expf(Mold - M);
-                if (f16_fma) {
-                    const double m16 = (double) rnd16(ms);
-                    for (int64_t e = 0; e < D; ++e) vkq[e] = oracle_f64_to_f16((double) oracle_f16_to_f32(vkq[e]) * m16);
-                } else {
-                    for (int64_t e = 0; e < D; ++e) vkq[e] = oracle_f32_to_f16(oracle_f16_to_f32(vkq[e]) * ms);
-                }
+                for (int64_t e = 0; e < D; ++e) vkq[e] = oracle_f32_to_f16(oracle_f16_to_f32(vkq[e]) * ms);
             } else {
                 vs = expf(s - M);
             }
-            if (f16_fma) {                     /* VKQ16 = fma_f16(v, f16(vs), VKQ16) */
-                const double v16 = (double) rnd16(vs);
-                for (int64_t e = 0; e < D; ++e)
-                    vkq[e] = oracle_f64_to_f16((double) oracle_f16_to_f32(v[(h * KV + ic) * D + e]) * v16 + (double) oracle_f16_to_f32(vkq[e]));
-            } else
             for (int64_t e = 0; e < D; ++e)    /* VKQ16 += v * vs: fma in f32, stored as f16 */
                 vkq[e] = oracle_f32_to_f16(fmaf(oracle_f16_to_f32(v[(h * KV + ic) * D + e]), vs, oracle_f16_to_f32(vkq[e])));
             S = S * ms + vs;

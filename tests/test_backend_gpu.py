@@ -31,6 +31,20 @@ def test_plugin_registers_one_gpu_device(harness):
     assert info["features"]["GFX950"] == "1"
 
 
+def test_results_the_host_reads_back_are_mirrored_in_pinned_memory(harness):
+    # whisper_decode fetches the logits with one blocking ggml_backend_tensor_get per row (src/whisper.cpp:2960-2966).  After
+    # the first fetch of a graph's result the backend copies it into pinned memory at the end of every graph and serves the
+    # reads from there: the bytes must equal a plain download, and a write into the tensor must retire the mirror.  Also the
+    # device's pinned host buffer type (get_host_buffer_type): host-visible, and a source / target of device copies.
+    rc, rows = run_harness(harness, ["download"])
+    s = rows[-1]
+    assert rc == 0 and s["summary"] == "download" and s["failed"] == 0, rows
+    assert s["host_buffer_ok"] and s["caps_host_buffer"] and s["host_buffer_type"] == "MI355X_Host", s
+    steps = [r for r in rows if "download" in r]
+    assert len(steps) >= 6 and all(r["ok"] and r["bytes_equal"] for r in steps), steps
+    assert steps[0]["from_mirror"] == 0 and steps[1]["from_mirror"] == 5 and steps[3]["by_copy"] == 5, steps
+
+
 def test_every_op_case_against_the_cpu_backend(harness):
     rc, rows = run_harness(harness, ["ops", "--reps", "1"], timeout=1500)
     cases = [r for r in rows if "case" in r]
@@ -65,18 +79,6 @@ def test_every_node_of_the_whisper_graphs(harness, models, key):
     assert summary["summary"] == "verify" and summary["pass"], [r for r in rows if "bad_node" in r]
     ops = {r["op"] for r in rows if "phase" in r}
     assert {"FLASH_ATTN_EXT", "NORM", "GET_ROWS", "IM2COL"} <= ops
-
-
-def test_packed_f16_attention_option_stays_within_the_bounds(harness, models):
-    # GGML_MI355X_FA_PACKED=1: encoder / prompt attention accumulates with f16 fused multiply-adds (the reference's Arm
-    # arithmetic); against the x86 CPU backend it must still meet the per-op and whole-model bounds
-    env = {"GGML_MI355X_FA_PACKED": "1"}
-    rc, rows = run_harness(harness, ["ops", "--quick", "--reps", "0", "--filter", "flash_attn"], env=env, timeout=900)
-    cases = [r for r in rows if "case" in r]
-    assert rc == 0 and cases and all(r["pass"] for r in cases), [r for r in cases if not r["pass"]]
-    rc, rows = run_harness(harness, ["model", "--model", models[("base", "q5_0")], "--steps", "16"], env=env, timeout=900)
-    s = rows[-1]
-    assert rc == 0 and s["pass"] and s["ids_identical"] == 16 and s["worst_logits_nmse"] <= 1e-3, s
 
 
 def test_whisper_full_end_to_end(harness, models):
@@ -154,17 +156,55 @@ def test_default_attention_graphs_without_flash_attn(harness, models):
     assert "SOFT_MAX" in {r["op"] for r in rows if "phase" in r}
 
 
-@pytest.mark.parametrize("key,steps", [(("base", "q5_0"), 32), (("base", "q8_0"), 32), (("base", "f16"), 32),
-                                       (("large-v3", "q5_0"), 32), (("large-v3-turbo", "q8_0"), 32)])
-def test_whole_model_logits_and_greedy_ids(harness, models, key, steps):
-    rc, rows = run_harness(harness, ["model", "--model", models[key], "--steps", str(steps)], timeout=1500)
-    s = rows[-1]
+def check_model_summary(s, strict_ids):
     assert s["summary"] == "model"
-    assert s["worst_logits_nmse"] <= 1e-3, s                 # north-star bound on the final logits
-    # Greedy ids: identical at every step where the reference's top-1 / top-2 margin stands clear (> 6x) of the RMS
+    assert s["worst_logits_nmse"] <= 1e-3, s                 # north-star bound on the final logits, every row of every step
+    # Greedy ids: identical on every row where the reference's top-1 / top-2 margin stands clear (> 6x) of the RMS
     # difference between the two logit vectors.  The reference accumulates attention in f16; one differently-rounded
     # f16 value cascades, so beyond bit-identical arithmetic the two runs are two draws of the same rounding noise and
     # a random-init model with near-flat logits can flip an argmax whose margin is inside that noise.
     assert s["clear_ids_identical"] == s["clear_steps"], s
-    assert s["ids_identical"] >= (steps if key[0] == "base" else int(0.75 * steps)), s
-    assert rc == 0 and s["pass"]
+    assert s["ids_identical"] >= (s["rows"] if strict_ids else int(0.75 * s["rows"])), s
+    # nothing left the device: the scheduler reported one split per graph, all on the MI355X device, and the plugin was
+    # handed exactly one graph per graph whisper computed
+    assert s["one_split_per_graph"] and s["sched_splits"] == s["graphs"] == s["plugin_graph_computes"] and s["sched_splits_not_on_device"] == 0, s
+    assert s["pass"]
+
+
+@pytest.mark.parametrize("key,steps", [(("base", "q5_0"), 32), (("base", "q8_0"), 32), (("base", "f16"), 32),
+                                       (("large-v3", "q5_0"), 32), (("large-v3-turbo", "q8_0"), 32)])
+def test_whole_model_logits_and_greedy_ids(harness, models, key, steps):
+    rc, rows = run_harness(harness, ["model", "--model", models[key], "--steps", str(steps)], timeout=1500)
+    check_model_summary(rows[-1], strict_ids=key[0] == "base")
+    assert rc == 0
+    if key == ("large-v3", "q5_0"):
+        # the encoder graph of large-v3 arrives whole: 3 graphs per window, and far more nodes than launches
+        assert rows[-1]["encode_nodes"] > 1200 and rows[-1]["encode_launches"] < 300, rows[-1]
+
+
+@pytest.mark.parametrize("arch,ftype", [("large-v3", "q5_0"), ("large-v3-turbo", "q8_0")])
+def test_whole_model_parity_on_other_seeds(harness, tmp_path, arch, ftype):
+    # the criterion above on two more random-init models and mel windows each (the parametrized test above runs seeds 1234 / 7)
+    for model_seed, mel_seed in ((2024, 11), (77, 3)):
+        path = tmp_path / f"{arch}-{ftype}-{model_seed}.bin"
+        rc, rows = run_harness(harness, ["gen", "--arch", arch, "--ftype", ftype, "--out", str(path), "--seed", str(model_seed)], timeout=300)
+        assert rc == 0 and rows[-1]["ok"]
+        rc, rows = run_harness(harness, ["model", "--model", str(path), "--steps", "32", "--seed", str(mel_seed)], timeout=1500)
+        s = rows[-1]
+        print(f"{arch} {ftype} model seed {model_seed} mel seed {mel_seed}: ids {s['ids_identical']}/{s['rows']}, clear {s['clear_ids_identical']}/{s['clear_steps']}, "
+              f"worst NMSE {s['worst_logits_nmse']:.2e}", flush=True)
+        check_model_summary(s, strict_ids=False)
+        path.unlink()
+
+
+@pytest.mark.parametrize("key,env", [(("large-v3-turbo", "q8_0"), {}), (("large-v3-turbo", "q8_0"), {"GGML_MI355X_FUSE": "0"}), (("base", "q5_0"), {})])
+def test_five_row_decode_steps_until_the_cache_is_full(harness, models, key, env):
+    # the shape of a 5-beam search step (BASELINE configs[4]): after the 4-token prompt every step feeds 5 tokens — the 5
+    # greedy ids of the CPU backend's previous step — until the self-attention cache holds all 448 positions; all 5 rows
+    # of every step are compared.  Five rows take other planner branches than one (LayerNorm held for the product group,
+    # grouped Q / K / V, fused embeddings, the mask cast inside the first attention launch, the tile-ordered logits product).
+    rc, rows = run_harness(harness, ["model", "--model", models[key], "--batch", "5", "--kv-to", "448"], env=env, timeout=1500)
+    s = rows[-1]
+    assert s["kv_positions"] == 448 and s["batch"] == 5 and s["rows"] >= 440, s
+    check_model_summary(s, strict_ids=False)
+    assert rc == 0

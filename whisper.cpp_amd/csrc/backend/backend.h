@@ -17,6 +17,8 @@
 #include "mi355x_kernels.h"
 
 #define MI355X_BUFFER_ALIGN 256
+#define MI355X_N_COUNTERS   8
+#define MI355X_MIRROR_MAX   (4u << 20)       // outputs larger than this are never mirrored (an encoder's states stay on the device)
 
 #define HIP_TRY(expr, on_fail)                                                                            \
     do {                                                                                                  \
@@ -85,9 +87,8 @@ struct mi355x_backend_ctx {
     bool        fuse    = true;
     bool        profile = false;
     bool        debug   = false;   // log what every MUL_MAT launch folds in (GGML_MI355X_DEBUG=1)
-    int         fa_accum = 0;           // V accumulation of attention over more than 8 queries: 0 the reference's x86 sequence (f32 fma,
-                                        // f16 store, key by key), 1 f32 accumulators on the matrix cores, 2 f16 fused multiply-adds
-                                        // key by key (the reference's Arm fp16 build)
+    int         fa_accum = 0;           // V accumulation of attention over more than 8 queries: 0 the reference's sequence (f32 fma,
+                                        // f16 store, key by key), 1 f32 accumulators on the matrix cores
     bool        weight_images = true;   // keep f16 images of quantized GEMM weights (GGML_MI355X_WEIGHT_IMAGES=0 turns it off)
     bool        exact   = false;   // true: f32 attention accumulators and un-rounded GEMM activations instead of the
                                    // reference's f16-sequential / Q8_0-rounded arithmetic
@@ -103,6 +104,22 @@ struct mi355x_backend_ctx {
     size_t       ws_x_nb[4] = {0, 0, 0, 0};
     bool         reserve_workspace(size_t size);
 
+    // what graph_compute was handed and did, always counted: calls, nodes of the graphs as received, nodes that are not
+    // views or empty (each of them is carried out by some launch), kernel launches
+    int64_t      counters[MI355X_N_COUNTERS] = {};
+
+    // Host mirror of graph outputs (the logits of a decode step): tensors flagged GGML_TENSOR_FLAG_OUTPUT that the host has
+    // downloaded before are copied into pinned memory at the end of graph_compute, on the stream, in one transfer each;
+    // get_tensor then serves any slice of them from there until something writes the tensor or the next graph runs.
+    struct mirror_entry { const char * dev; size_t size, off; };
+    std::mutex                mirror_mutex;
+    char *                    mirror_host = nullptr;      // pinned
+    size_t                    mirror_cap  = 0;
+    std::vector<mirror_entry> mirror;                     // what the pinned block holds of the last graph's outputs
+    hipEvent_t                mirror_done = nullptr;      // recorded behind the transfers
+    void mirror_outputs(struct ggml_cgraph * cgraph);     // end of graph_compute
+    void mirror_drop(const void * begin, size_t size);    // a write into [begin, begin + size)
+
     // profiling
     std::vector<mi355x_pending_event>         pending;
     std::vector<hipEvent_t>                   event_pool;
@@ -111,6 +128,9 @@ struct mi355x_backend_ctx {
     hipEvent_t take_event();
     void       drain_events();           // call after the stream has been synchronized
 };
+
+// ggml-mi355x.cpp: has the host downloaded the tensor at this address before (so that mirroring it pays)?
+bool mi355x_download_is_wanted(int device, const void * data, size_t size);
 
 // graph.cpp
 enum ggml_status mi355x_graph_compute(mi355x_backend_ctx * ctx, struct ggml_cgraph * cgraph);

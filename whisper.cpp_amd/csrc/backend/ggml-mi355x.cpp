@@ -31,6 +31,13 @@ static bool env_flag(const char * name, bool dflt) {
     return atoi(v) != 0;
 }
 
+// live backend contexts, so that options and statistics can address all of them at once (backend == NULL) and the
+// buffer-level transfers can find the host mirrors of graph outputs
+static std::mutex                        g_live_mutex;
+static std::vector<mi355x_backend_ctx *> g_live;
+static std::map<std::string, mi355x_kernel_stat> g_retired_stats;   // statistics of backends that were freed
+static int64_t g_retired_counters[MI355X_N_COUNTERS] = {};
+
 // ------------------------------------------------------------------------------------------------------
 // host <-> device transfers of the buffer interface
 //
@@ -40,9 +47,64 @@ static bool env_flag(const char * name, bool dflt) {
 // The ordering ggml relies on is kept by the streams: every backend instance's stream is a blocking stream, so work
 // queued on it later starts after the transfer, and the transfer starts after the kernels queued before it; reads
 // back go through the same null stream.  The caller's memory is free for reuse on return, as set_tensor promises.
-// (Downloads stay with hipMemcpy: staging 1 MB of logits through the ring, whole or in overlapped pieces, measured
-// within 10 % of it — the copy out of the ring costs what the runtime's own staging costs.)
+//
+// Downloads: a graph's result that the host has fetched once (a decode step's logits, which whisper_decode reads row by row
+// with one blocking ggml_backend_tensor_get per beam, src/whisper.cpp:2960-2966) is from then on copied into pinned
+// memory at the end of every graph_compute that produces it — as its last node or as a flagged output, the two kinds of
+// tensor whose memory still holds their value when the graph is over — in one transfer on the backend's stream
+// (mi355x_backend_ctx::mirror_outputs); get_tensor serves slices of it from there — a memcpy — until something writes
+// the tensor or the next graph runs.  Compute-buffer addresses are stable from step to step (ggml/src/ggml-alloc.c:816-914),
+// which is what makes "the tensor at this address" a usable key.  Everything else is a plain hipMemcpy.
 // ------------------------------------------------------------------------------------------------------
+
+struct wanted_download { int device; const void * data; size_t size; };
+static std::mutex                   g_wanted_mutex;
+static std::vector<wanted_download> g_wanted;            // a handful of entries: the outputs the host reads back
+
+bool mi355x_download_is_wanted(int device, const void * data, size_t size) {
+    std::lock_guard<std::mutex> lock(g_wanted_mutex);
+    for (const wanted_download & w : g_wanted) if (w.device == device && w.data == data && w.size == size) return true;
+    return false;
+}
+
+static void want_download(int device, const void * data, size_t size) {
+    std::lock_guard<std::mutex> lock(g_wanted_mutex);
+    for (const wanted_download & w : g_wanted) if (w.device == device && w.data == data && w.size == size) return;
+    if (g_wanted.size() >= 64) g_wanted.erase(g_wanted.begin());
+    g_wanted.push_back({ device, data, size });
+}
+
+// a buffer is going away: nothing at its addresses is wanted any more
+static void forget_downloads(int device, const void * begin, size_t size) {
+    std::lock_guard<std::mutex> lock(g_wanted_mutex);
+    const char * b = (const char *) begin;
+    for (size_t i = 0; i < g_wanted.size();) {
+        if (g_wanted[i].device == device && (const char *) g_wanted[i].data >= b && (const char *) g_wanted[i].data < b + size) g_wanted.erase(g_wanted.begin() + (long) i); else ++i;
+    }
+}
+
+// [data + offset, + size) of a tensor from the host mirror of a backend instance on this device; false: not mirrored
+static bool download_from_mirror(int device, const struct ggml_tensor * tensor, void * data, size_t offset, size_t size) {
+    std::lock_guard<std::mutex> live(g_live_mutex);
+    for (mi355x_backend_ctx * ctx : g_live) {
+        if (ctx->device != device) continue;
+        std::lock_guard<std::mutex> lock(ctx->mirror_mutex);
+        for (const mi355x_backend_ctx::mirror_entry & e : ctx->mirror) {
+            if (e.dev != (const char *) tensor->data || offset + size > e.size) continue;
+            if (hipEventSynchronize(ctx->mirror_done) != hipSuccess) { (void) hipGetLastError(); return false; }
+            memcpy(data, ctx->mirror_host + e.off + offset, size);
+            ctx->counters[4] += 1;
+            return true;
+        }
+    }
+    return false;
+}
+
+// something writes [begin, begin + size) on this device: mirrors of that range are stale
+static void drop_mirrors(int device, const void * begin, size_t size) {
+    std::lock_guard<std::mutex> live(g_live_mutex);
+    for (mi355x_backend_ctx * ctx : g_live) if (ctx->device == device) ctx->mirror_drop(begin, size);
+}
 
 #define STAGE_RING_BYTES   (8u << 20)
 #define STAGE_UPLOAD_MAX   (512u << 10)      // larger uploads (model weights) take the runtime's own path
@@ -58,6 +120,7 @@ static staging_ring g_rings[64];             // per device, pinned for the life 
 static staging_ring * ring_of(int device) {
     if (device < 0 || device >= 64) return nullptr;
     staging_ring & r = g_rings[device];
+    std::lock_guard<std::mutex> lock(r.m);             // two states of one context may make their first upload at once
     if (!r.base && !r.failed) {
         void * p = nullptr;
         const bool ok = hipHostMalloc(&p, STAGE_RING_BYTES, hipHostMallocDefault) == hipSuccess && p;
@@ -148,6 +211,8 @@ static void buffer_free(ggml_backend_buffer_t buffer) {
     HIP_TRY(hipSetDevice(ctx->device), (void) 0);
     HIP_TRY(hipDeviceSynchronize(), (void) 0);
     ctx->drop_all_images();
+    drop_mirrors(ctx->device, ctx->base, ctx->size);
+    forget_downloads(ctx->device, ctx->base, ctx->size);
     HIP_TRY(hipFree(ctx->base), (void) 0);
     delete ctx;
 }
@@ -166,7 +231,8 @@ static enum ggml_status buffer_init_tensor(ggml_backend_buffer_t, struct ggml_te
 static void buffer_memset_tensor(ggml_backend_buffer_t buffer, struct ggml_tensor * tensor, uint8_t value, size_t offset, size_t size) {
     mi355x_buffer_ctx * ctx = (mi355x_buffer_ctx *) buffer->context;
     HIP_TRY(hipSetDevice(ctx->device), return);
-    if (!ctx->images.empty()) ctx->drop_images((char *) tensor->data + offset, size);
+    ctx->drop_images((char *) tensor->data + offset, size);
+    drop_mirrors(ctx->device, (char *) tensor->data + offset, size);
     HIP_TRY(hipMemset((char *) tensor->data + offset, value, size), return);
     HIP_TRY(hipStreamSynchronize(nullptr), return);
 }
@@ -174,7 +240,8 @@ static void buffer_memset_tensor(ggml_backend_buffer_t buffer, struct ggml_tenso
 static void buffer_set_tensor(ggml_backend_buffer_t buffer, struct ggml_tensor * tensor, const void * data, size_t offset, size_t size) {
     mi355x_buffer_ctx * ctx = (mi355x_buffer_ctx *) buffer->context;
     HIP_TRY(hipSetDevice(ctx->device), return);
-    if (!ctx->images.empty()) ctx->drop_images((char *) tensor->data + offset, size);
+    ctx->drop_images((char *) tensor->data + offset, size);
+    drop_mirrors(ctx->device, (char *) tensor->data + offset, size);
     if (!upload(ctx->device, (char *) tensor->data + offset, data, size)) {
         GGML_LOG_ERROR("ggml-mi355x: upload of %zu bytes into %s failed: %s\n", size, tensor->name, hipGetErrorString(hipGetLastError()));
     }
@@ -182,8 +249,16 @@ static void buffer_set_tensor(ggml_backend_buffer_t buffer, struct ggml_tensor *
 
 static void buffer_get_tensor(ggml_backend_buffer_t buffer, const struct ggml_tensor * tensor, void * data, size_t offset, size_t size) {
     mi355x_buffer_ctx * ctx = (mi355x_buffer_ctx *) buffer->context;
+    if (download_from_mirror(ctx->device, tensor, data, offset, size)) return;
     HIP_TRY(hipSetDevice(ctx->device), return);
     HIP_TRY(hipMemcpy(data, (const char *) tensor->data + offset, size, hipMemcpyDeviceToHost), return);
+    // a result that the host reads back (whisper.cpp does not flag its logits as an output: they are the graph's last node,
+    // src/whisper.cpp:2953): from the next graph on it is mirrored in pinned memory
+    static const bool no_mirror = env_flag("GGML_MI355X_NO_MIRROR", false);
+    if (!no_mirror && buffer->usage != GGML_BACKEND_BUFFER_USAGE_WEIGHTS && !tensor->view_src && ggml_is_contiguous(tensor) &&
+        ggml_nbytes(tensor) <= MI355X_MIRROR_MAX) want_download(ctx->device, tensor->data, ggml_nbytes(tensor));
+    std::lock_guard<std::mutex> live(g_live_mutex);
+    for (mi355x_backend_ctx * b : g_live) if (b->device == ctx->device) { b->counters[5] += 1; break; }
 }
 
 static bool buffer_is_mi355x(ggml_backend_buffer_t buffer) { return buffer && buffer->iface.get_base == buffer_get_base; }
@@ -194,7 +269,8 @@ static bool buffer_cpy_tensor(ggml_backend_buffer_t buffer, const struct ggml_te
     ggml_backend_buffer_t sbuf = src->view_src ? src->view_src->buffer : src->buffer;
     if (!ggml_is_contiguous(src) || !ggml_is_contiguous(dst) || ggml_nbytes(src) != ggml_nbytes(dst)) return false;
     HIP_TRY(hipSetDevice(ctx->device), return false);
-    if (!ctx->images.empty()) ctx->drop_images(dst->data, ggml_nbytes(dst));
+    ctx->drop_images(dst->data, ggml_nbytes(dst));
+    drop_mirrors(ctx->device, dst->data, ggml_nbytes(dst));
     if (buffer_is_mi355x(sbuf)) {
         const int sdev = ((mi355x_buffer_ctx *) sbuf->context)->device;
         if (sdev != ctx->device) {                          // uploads queued on the other device's null stream come first
@@ -214,6 +290,7 @@ static void buffer_clear(ggml_backend_buffer_t buffer, uint8_t value) {
     mi355x_buffer_ctx * ctx = (mi355x_buffer_ctx *) buffer->context;
     HIP_TRY(hipSetDevice(ctx->device), return);
     ctx->drop_all_images();
+    drop_mirrors(ctx->device, ctx->base, ctx->size);
     HIP_TRY(hipMemset(ctx->base, value, ctx->size), return);
     HIP_TRY(hipDeviceSynchronize(), return);
 }
@@ -280,13 +357,47 @@ static const struct ggml_backend_buffer_type_i mi355x_buft_iface = {
 };
 
 // ------------------------------------------------------------------------------------------------------
+// host buffer type  (ggml_backend_device_i::get_host_buffer_type, ggml-backend-impl.h:160): host memory that the device
+// reads and writes at full PCIe speed — pinned with hipHostMalloc — behind ggml's own host-buffer interface, so that every
+// CPU-side user (ggml_backend_tensor_set / _get are memcpy, the CPU backend computes on it) sees an ordinary host buffer.
+// A host that stages its graph inputs or results there spares the runtime its own staging copy on every transfer.
+// ------------------------------------------------------------------------------------------------------
+
+static const char * host_buft_get_name(ggml_backend_buffer_type_t) { return GGML_MI355X_NAME "_Host"; }
+
+static void host_buffer_free(ggml_backend_buffer_t buffer) {
+    if (hipHostFree(buffer->context) != hipSuccess) (void) hipGetLastError();
+}
+
+static ggml_backend_buffer_t host_buft_alloc_buffer(ggml_backend_buffer_type_t buft, size_t size) {
+    void * p = nullptr;
+    if (hipHostMalloc(&p, size ? size : 1, hipHostMallocDefault) != hipSuccess || !p) {
+        (void) hipGetLastError();
+        GGML_LOG_WARN("ggml-mi355x: could not pin %.2f MiB of host memory; the buffer is ordinary host memory\n", size / 1048576.0);
+        return ggml_backend_buft_alloc_buffer(ggml_backend_cpu_buffer_type(), size);
+    }
+    ggml_backend_buffer_t buffer = ggml_backend_cpu_buffer_from_ptr(p, size);     // host-buffer vtable over memory of ours
+    buffer->buft = buft;
+    buffer->iface.free_buffer = host_buffer_free;                                 // its context is the pointer
+    return buffer;
+}
+
+static size_t host_buft_get_alignment(ggml_backend_buffer_type_t) { return ggml_backend_buft_get_alignment(ggml_backend_cpu_buffer_type()); }
+static bool   host_buft_is_host(ggml_backend_buffer_type_t) { return true; }
+
+static const struct ggml_backend_buffer_type_i mi355x_host_buft_iface = {
+    /* .get_name       = */ host_buft_get_name,
+    /* .alloc_buffer   = */ host_buft_alloc_buffer,
+    /* .get_alignment  = */ host_buft_get_alignment,
+    /* .get_max_size   = */ NULL,
+    /* .get_alloc_size = */ NULL,
+    /* .is_host        = */ host_buft_is_host,
+};
+
+// ------------------------------------------------------------------------------------------------------
 // backend / stream  (ggml_backend_i, ggml-backend-impl.h:87-117)
 // ------------------------------------------------------------------------------------------------------
 
-// live backend contexts, so that options and statistics can address all of them at once (backend == NULL)
-static std::mutex                        g_live_mutex;
-static std::vector<mi355x_backend_ctx *> g_live;
-static std::map<std::string, mi355x_kernel_stat> g_retired_stats;   // statistics of backends that were freed
 
 static ggml_guid_t backend_guid() {
     static ggml_guid guid = { 0x4d, 0x49, 0x33, 0x35, 0x35, 0x58, 0x2d, 0x67, 0x66, 0x78, 0x39, 0x35, 0x30, 0x2d, 0x76, 0x31 };
@@ -314,9 +425,12 @@ static void backend_free(ggml_backend_t backend) {
             auto & s = g_retired_stats[kv.first];
             s.calls += kv.second.calls; s.ms += kv.second.ms; s.bytes += kv.second.bytes; s.flops += kv.second.flops;
         }
+        for (int i = 0; i < MI355X_N_COUNTERS; ++i) g_retired_counters[i] += ctx->counters[i];
     }
     for (hipEvent_t e : ctx->event_pool) (void) hipEventDestroy(e);
     if (ctx->ws_base) (void) hipFree(ctx->ws_base);
+    if (ctx->mirror_host) (void) hipHostFree(ctx->mirror_host);
+    if (ctx->mirror_done) (void) hipEventDestroy(ctx->mirror_done);
     if (ctx->stream) (void) hipStreamDestroy(ctx->stream);
     delete ctx;
     delete backend;
@@ -328,8 +442,9 @@ static void backend_set_tensor_async(ggml_backend_t backend, struct ggml_tensor 
     ggml_backend_buffer_t buf = tensor->view_src ? tensor->view_src->buffer : tensor->buffer;
     if (buffer_is_mi355x(buf)) {
         mi355x_buffer_ctx * bctx = (mi355x_buffer_ctx *) buf->context;
-        if (!bctx->images.empty()) bctx->drop_images((char *) tensor->data + offset, size);
+        bctx->drop_images((char *) tensor->data + offset, size);
     }
+    ctx->mirror_drop((char *) tensor->data + offset, size);
     HIP_TRY(hipMemcpyAsync((char *) tensor->data + offset, data, size, hipMemcpyHostToDevice, ctx->stream), return);
 }
 
@@ -380,7 +495,7 @@ static void device_get_props(ggml_backend_dev_t dev, struct ggml_backend_dev_pro
     props->description = device_get_description(dev);
     props->type        = device_get_type(dev);
     device_get_memory(dev, &props->memory_free, &props->memory_total);
-    props->caps = { /* async */ false, /* host_buffer */ false, /* buffer_from_host_ptr */ false, /* events */ false };
+    props->caps = { /* async */ false, /* host_buffer */ true, /* buffer_from_host_ptr */ false, /* events */ false };
 }
 
 static ggml_backend_t device_init_backend(ggml_backend_dev_t dev, const char *) {
@@ -392,8 +507,7 @@ static ggml_backend_t device_init_backend(ggml_backend_dev_t dev, const char *) 
     ctx->fuse    = env_flag("GGML_MI355X_FUSE", true);
     ctx->profile = env_flag("GGML_MI355X_PROFILE", false);
     ctx->exact   = env_flag("GGML_MI355X_EXACT", false);
-    ctx->fa_accum = env_flag("GGML_MI355X_FA_PACKED", false) ? 2 : 0;
-    if (const char * e = getenv("GGML_MI355X_FA_ACCUM")) { const int v = atoi(e); if (v >= 0 && v <= 2) ctx->fa_accum = v; }
+    if (const char * e = getenv("GGML_MI355X_FA_ACCUM")) { const int v = atoi(e); if (v >= 0 && v <= 1) ctx->fa_accum = v; }
     ctx->weight_images = env_flag("GGML_MI355X_WEIGHT_IMAGES", true);
     ctx->debug   = env_flag("GGML_MI355X_DEBUG", false);
     // default priority, blocking with respect to the null stream used by the buffer-level copies
@@ -412,6 +526,7 @@ static ggml_backend_t device_init_backend(ggml_backend_dev_t dev, const char *) 
 }
 
 static ggml_backend_buffer_type_t device_get_buffer_type(ggml_backend_dev_t dev);
+static ggml_backend_buffer_type_t device_get_host_buffer_type(ggml_backend_dev_t dev);
 
 static bool device_supports_op(ggml_backend_dev_t, const struct ggml_tensor * op) { return mi355x_supports_op(op); }
 
@@ -429,7 +544,7 @@ static const struct ggml_backend_device_i mi355x_device_iface = {
     /* .get_props            = */ device_get_props,
     /* .init_backend         = */ device_init_backend,
     /* .get_buffer_type      = */ device_get_buffer_type,
-    /* .get_host_buffer_type = */ NULL,
+    /* .get_host_buffer_type = */ device_get_host_buffer_type,
     /* .buffer_from_host_ptr = */ NULL,
     /* .supports_op          = */ device_supports_op,
     /* .supports_buft        = */ device_supports_buft,
@@ -446,6 +561,7 @@ static const struct ggml_backend_device_i mi355x_device_iface = {
 struct mi355x_reg_ctx {
     std::vector<ggml_backend_device>      devices;
     std::vector<ggml_backend_buffer_type> bufts;
+    std::vector<ggml_backend_buffer_type> host_bufts;
 };
 
 static const char * reg_get_name(ggml_backend_reg_t) { return GGML_MI355X_NAME; }
@@ -476,15 +592,14 @@ static void ctx_synchronize(mi355x_backend_ctx * ctx) {
 static int set_option(ggml_backend_t backend, const char * name, int value) {
     if (!name || (backend && !ggml_backend_is_mi355x(backend))) return -1;
     const bool is_fuse = strcmp(name, "fuse") == 0, is_profile = strcmp(name, "profile") == 0, is_exact = strcmp(name, "exact") == 0;
-    const bool is_packed = strcmp(name, "fa_packed") == 0, is_accum = strcmp(name, "fa_accum") == 0;
-    if (!is_fuse && !is_profile && !is_exact && !is_packed && !is_accum) return -1;
-    if (is_accum && (value < 0 || value > 2)) return -1;
+    const bool is_accum = strcmp(name, "fa_accum") == 0;
+    if (!is_fuse && !is_profile && !is_exact && !is_accum) return -1;
+    if (is_accum && (value < 0 || value > 1)) return -1;
     std::lock_guard<std::mutex> lock(g_live_mutex);
     for (mi355x_backend_ctx * ctx : g_live) {
         if (backend && ctx != (mi355x_backend_ctx *) backend->context) continue;
         if (is_fuse) ctx->fuse = value != 0;
         else if (is_exact) ctx->exact = value != 0;
-        else if (is_packed) ctx->fa_accum = value != 0 ? 2 : 0;
         else if (is_accum) ctx->fa_accum = value;
         else { ctx_synchronize(ctx); ctx->profile = value != 0; }
     }
@@ -521,6 +636,19 @@ static size_t get_stats(ggml_backend_t backend, char * buf, size_t size, int res
     s += "]";
     if (buf && size) { const size_t n = s.size() < size - 1 ? s.size() : size - 1; memcpy(buf, s.data(), n); buf[n] = 0; }
     return s.size() + 1;
+}
+
+// graph_compute calls, graph nodes received, nodes that are not views or empty, kernel launches, downloads served from the
+// host mirror, downloads by hipMemcpy — since the last reset
+static void get_counters(ggml_backend_t backend, int64_t out[MI355X_N_COUNTERS], int reset) {
+    for (int i = 0; i < MI355X_N_COUNTERS; ++i) out[i] = 0;
+    if (backend && !ggml_backend_is_mi355x(backend)) return;
+    std::lock_guard<std::mutex> lock(g_live_mutex);
+    for (mi355x_backend_ctx * ctx : g_live) {
+        if (backend && ctx != (mi355x_backend_ctx *) backend->context) continue;
+        for (int i = 0; i < MI355X_N_COUNTERS; ++i) { out[i] += ctx->counters[i]; if (reset) ctx->counters[i] = 0; }
+    }
+    if (!backend) for (int i = 0; i < MI355X_N_COUNTERS; ++i) { out[i] += g_retired_counters[i]; if (reset) g_retired_counters[i] = 0; }
 }
 
 // host-memory front of mi355x_log_mel_spectrogram: one allocation for samples, filter bank, result and workspace, the
@@ -563,6 +691,7 @@ static void * reg_get_proc_address(ggml_backend_reg_t, const char * name) {
     if (strcmp(name, "ggml_backend_get_features") == 0)      return (void *) get_features;
     if (strcmp(name, "ggml_backend_mi355x_set_option") == 0) return (void *) set_option;
     if (strcmp(name, "ggml_backend_mi355x_get_stats") == 0)  return (void *) get_stats;
+    if (strcmp(name, "ggml_backend_mi355x_get_counters") == 0) return (void *) get_counters;
     if (strcmp(name, "ggml_backend_mi355x_log_mel") == 0)    return (void *) log_mel;
     return NULL;
 }
@@ -580,6 +709,12 @@ static ggml_backend_buffer_type_t device_get_buffer_type(ggml_backend_dev_t dev)
     return NULL;
 }
 
+static ggml_backend_buffer_type_t device_get_host_buffer_type(ggml_backend_dev_t dev) {
+    mi355x_reg_ctx * rctx = (mi355x_reg_ctx *) dev->reg->context;
+    for (size_t i = 0; i < rctx->devices.size(); ++i) if (&rctx->devices[i] == dev) return &rctx->host_bufts[i];
+    return NULL;
+}
+
 // ------------------------------------------------------------------------------------------------------
 // public entry points
 // ------------------------------------------------------------------------------------------------------
@@ -594,6 +729,7 @@ ggml_backend_reg_t ggml_backend_mi355x_reg(void) {
         const std::vector<int> & devs = gfx950_devices();
         ctx->devices.reserve(devs.size());
         ctx->bufts.reserve(devs.size());
+        ctx->host_bufts.reserve(devs.size());
         reg = { GGML_BACKEND_API_VERSION, mi355x_reg_iface, ctx };
         for (size_t i = 0; i < devs.size(); ++i) {
             mi355x_device_ctx * d = new mi355x_device_ctx;
@@ -604,6 +740,7 @@ ggml_backend_reg_t ggml_backend_mi355x_reg(void) {
             else { (void) hipGetLastError(); d->description = "AMD Instinct MI355X"; }
             ctx->devices.push_back({ mi355x_device_iface, &reg, d });
             ctx->bufts.push_back({ mi355x_buft_iface, &ctx->devices.back(), NULL });
+            ctx->host_bufts.push_back({ mi355x_host_buft_iface, &ctx->devices.back(), NULL });
         }
     });
     return &reg;

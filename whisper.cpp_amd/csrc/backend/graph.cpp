@@ -11,6 +11,7 @@
 #include "backend.h"
 
 #include <string.h>
+#include <algorithm>
 #include <unordered_map>
 
 static mi355x_tensor to_view(const ggml_tensor * t) {
@@ -132,6 +133,46 @@ bool mi355x_backend_ctx::reserve_workspace(size_t size) {
     return true;
 }
 
+// Queue the download of those results of this graph that the host is known to read (whisper_decode reads the logits row by row
+// with blocking ggml_backend_tensor_get calls, src/whisper.cpp:2960-2966): one transfer per tensor into pinned memory,
+// behind the graph on the same stream, so that it is over when the host's synchronize returns.
+void mi355x_backend_ctx::mirror_outputs(struct ggml_cgraph * cgraph) {
+    std::lock_guard<std::mutex> lock(mirror_mutex);
+    size_t used = 0;
+    for (int i = 0; i < cgraph->n_nodes; ++i) {
+        const ggml_tensor * n = cgraph->nodes[i];
+        // only tensors whose memory the allocator cannot have handed on by the end of the graph
+        if (!((n->flags & GGML_TENSOR_FLAG_OUTPUT) || i == cgraph->n_nodes - 1) || !n->data || n->view_src || ggml_is_empty(n) || !ggml_is_contiguous(n)) continue;
+        const size_t size = ggml_nbytes(n);
+        if (size > MI355X_MIRROR_MAX || !mi355x_download_is_wanted(device, n->data, size)) continue;
+        const size_t off = (used + 255) & ~(size_t) 255;
+        if (off + size > mirror_cap) {
+            if (!mirror.empty()) continue;                 // transfers into the block are queued: it cannot move now
+            if (hipStreamSynchronize(stream) != hipSuccess) { (void) hipGetLastError(); return; }
+            if (mirror_host) (void) hipHostFree(mirror_host);
+            mirror_host = nullptr; mirror_cap = 0;
+            const size_t want = std::max<size_t>(2 * (off + size), 2u << 20);
+            void * p = nullptr;
+            if (hipHostMalloc(&p, want, hipHostMallocDefault) != hipSuccess || !p) { (void) hipGetLastError(); return; }
+            mirror_host = (char *) p; mirror_cap = want;
+        }
+        if (hipMemcpyAsync(mirror_host + off, n->data, size, hipMemcpyDeviceToHost, stream) != hipSuccess) { (void) hipGetLastError(); continue; }
+        mirror.push_back({ (const char *) n->data, size, off });
+        used = off + size;
+    }
+    if (mirror.empty()) return;
+    if (!mirror_done && hipEventCreateWithFlags(&mirror_done, hipEventDisableTiming) != hipSuccess) { (void) hipGetLastError(); mirror_done = nullptr; }
+    if (!mirror_done || hipEventRecord(mirror_done, stream) != hipSuccess) { (void) hipGetLastError(); mirror.clear(); }
+}
+
+void mi355x_backend_ctx::mirror_drop(const void * begin, size_t size) {
+    std::lock_guard<std::mutex> lock(mirror_mutex);
+    const char * b = (const char *) begin;
+    for (size_t i = 0; i < mirror.size();) {
+        if (mirror[i].dev < b + size && b < mirror[i].dev + mirror[i].size) mirror.erase(mirror.begin() + (long) i); else ++i;
+    }
+}
+
 namespace {
 
 struct launch_scope {   // brackets one kernel launch with events when profiling
@@ -139,6 +180,7 @@ struct launch_scope {   // brackets one kernel launch with events when profiling
     mi355x_pending_event ev;
     bool on;
     launch_scope(mi355x_backend_ctx * c, const char * name, double bytes, double flops) : ctx(c), on(c->profile) {
+        ctx->counters[3] += 1;
         if (!on) return;
         ev.name = name; ev.bytes = bytes; ev.flops = flops;
         ev.start = ctx->take_event(); ev.stop = ctx->take_event();
@@ -598,6 +640,10 @@ struct graph_runner {
         }
         const ggml_tensor * r = node_at(j);
         if (!r || r->op != GGML_OP_FLASH_ATTN_EXT || r->src[3] != n || r->src[0]->ne[1] > n->ne[1]) return false;
+        // The allocator frees the f32 mask after the cast (ggml/src/ggml-alloc.c:612-667) and may place the attention node's
+        // own output there: its workgroups would then overwrite mask rows that others are still reading.  (The f16 copy
+        // is a source of the attention node, so the allocator keeps that apart from the output by itself.)
+        if (ranges_overlap(r, s0) || ranges_overlap(r, n)) return false;
         mi355x_tensor vq = to_view(r->src[0]), vk = to_view(r->src[1]);
         return strcmp(mi355x_flash_attn_ext_kernel_name(&vq, &vk, MI355X_FA_F16_SEQ), "flash_attn.seq_row") == 0;
     }
@@ -704,7 +750,7 @@ struct graph_runner {
                 const double bytes = (double) ggml_nelements(s0) * 4 + 2.0 * (double) k->ne[0] * k->ne[1] * k->ne[2] * k->ne[3] * 2 + nbytes_of(n);
                 // the accumulation option is for the many-query kernels; a decode step keeps the reference's sequence
                 const int accum = s0->ne[1] > 8 ? ctx->fa_accum : 0;
-                const int mode = ctx->exact || accum == 1 ? MI355X_FA_F32 : accum == 2 ? MI355X_FA_F16_PACKED : MI355X_FA_F16_SEQ;
+                const int mode = ctx->exact || accum == 1 ? MI355X_FA_F32 : MI355X_FA_F16_SEQ;
                 const char * name = mi355x_flash_attn_ext_kernel_name(&vq, &vk, mode);
                 // the output projection that follows takes its Q8_0-rounded activations from the attention kernel itself
                 const bool emits = !ctx->exact && (strncmp(name, "flash_attn.seq_tile", 19) == 0 || strcmp(name, "flash_attn.mfma_f32") == 0);
@@ -745,6 +791,10 @@ struct graph_runner {
 enum ggml_status mi355x_graph_compute(mi355x_backend_ctx * ctx, struct ggml_cgraph * cgraph) {
     HIP_TRY(hipSetDevice(ctx->device), return GGML_STATUS_FAILED);
     ctx->ws_x = nullptr;   // tensors may have been rewritten between graphs
+    { std::lock_guard<std::mutex> lock(ctx->mirror_mutex); ctx->mirror.clear(); }      // this graph may write anywhere in the compute buffer
+    ctx->counters[0] += 1;
+    ctx->counters[1] += cgraph->n_nodes;
+    for (int i = 0; i < cgraph->n_nodes; ++i) ctx->counters[2] += !(ggml_is_empty(cgraph->nodes[i]) || is_view_op(cgraph->nodes[i]->op));
     graph_runner run(ctx, cgraph);
     for (int i = 0; i < cgraph->n_nodes;) {
         int status = MI355X_OK;
@@ -760,5 +810,6 @@ enum ggml_status mi355x_graph_compute(mi355x_backend_ctx * ctx, struct ggml_cgra
         GGML_LOG_ERROR("ggml-mi355x: trailing NORM failed: %s\n", mi355x_status_string(status));
         return GGML_STATUS_FAILED;
     }
+    ctx->mirror_outputs(cgraph);
     return GGML_STATUS_SUCCESS;
 }

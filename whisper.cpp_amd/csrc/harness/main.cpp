@@ -7,14 +7,15 @@
 //   selftest                                  the writer's quantizers / f16 conversion vs the reference's, byte for byte
 //   ops    [--filter S] [--quick] [--threads N] [--reps R] [--cpu-only]
 //                                             per-op parity (NMSE / bit-exactness) and timing, CPU vs MI355X
-//   model  --model F [--steps 32] [--threads N]
-//                                             whole-model parity: logits NMSE and greedy ids, teacher-forced
+//   model  --model F [--steps 32] [--batch B] [--kv-to N] [--seed S] [--threads N]
+//                                             whole-model parity: logits NMSE and greedy ids, teacher-forced; one split per graph
 //   full   --model F [--beam 1|5] [--max-tokens 24] [--seconds 30] [--threads N] [--dtw] [--processors N] [--gpu-mel]
 //                                             whisper_full() end to end (PCM -> mel -> encode -> search) on both backends
 //   mel    --model F [--seconds 30] [--reps 20] [--threads N]
 //                                             the log-mel front end: device path through the plugin vs whisper_pcm_to_mel
 //   verify --model F [--steps 3] [--threads N]
 //                                             per-node parity inside the real whisper graphs (unfused), CPU vs MI355X
+//   download                                  the pinned host mirror of results the host reads back, and the pinned host buffer type
 //   bench  --model F --what encoder|decoder|whisper-bench --backend gpu|cpu [--threads N] [--reps R] [--profile]
 //                                             timings with the whisper-bench protocol (examples/bench/bench.cpp:108-138)
 #include <math.h>
@@ -68,8 +69,20 @@ static args parse_args(int argc, char ** argv, int first) {
     return a;
 }
 
+// The scheduler's own account of how it split a graph (GGML_SCHED_DEBUG=1: ggml_backend_sched_print_assignments,
+// ggml/src/ggml-backend.cpp:791-802, one "## SPLIT #i: <backend> # n inputs" line per split), counted while enabled.
+static bool g_count_splits = false;
+static int  g_splits_total = 0, g_splits_not_on_device = 0;
+
 static void quiet_log(enum ggml_log_level level, const char * text, void *) {
     static const bool verbose = getenv("GGML_MI355X_DEBUG") != nullptr;
+    if (g_count_splits) {
+        if (const char * p = strstr(text, "## SPLIT #")) {
+            ++g_splits_total;
+            const char * colon = strchr(p, ':');
+            if (!colon || strncmp(colon + 2, GGML_MI355X_NAME, strlen(GGML_MI355X_NAME)) != 0) ++g_splits_not_on_device;
+        }
+    }
     if (level == GGML_LOG_LEVEL_ERROR || level == GGML_LOG_LEVEL_WARN || (verbose && strncmp(text, "ggml-mi355x", 11) == 0)) fputs(text, stderr);
 }
 
@@ -378,69 +391,113 @@ static int argmax(const float * v, int n, float * margin) {
 }
 
 // whole-model parity: both contexts encode the same synthetic mel, then decode the same token history step by step
-// (teacher-forced with the CPU's greedy choice so that one flipped argmax cannot cascade); per step compares the
-// logits of the newest token.
+// (teacher-forced with the CPU's greedy choices so that one flipped argmax cannot cascade); per step compares the
+// logits of every row.  --batch B feeds B tokens per step after the prompt (the shape of a B-beam search step: B rows
+// through every product, B queries per attention node) — the B greedy ids of the step before — and --kv-to N keeps
+// stepping until the self-attention cache holds N positions (448 = n_text_ctx fills it).
+//
+// Also checks that nothing left the device: the scheduler reports its splits (GGML_SCHED_DEBUG=1) and the plugin counts
+// the graphs and nodes it was handed; every graph whisper computes must be one split on the MI355X device.
 static int cmd_model(const args & a) {
     const std::string path = a.str("model");
-    const int steps = a.num("steps", 32), threads = a.num("threads", default_threads());
-    if (path.empty()) { fprintf(stderr, "usage: model --model FILE [--steps N]\n"); return 2; }
-    if (!load_plugin(true)) { printf("{\"error\": \"no MI355X backend\"}\n"); return 2; }
+    const int threads = a.num("threads", default_threads()), batch = std::max(1, a.num("batch", 1));
+    if (path.empty()) { fprintf(stderr, "usage: model --model FILE [--steps N] [--batch B] [--kv-to N] [--seed S]\n"); return 2; }
+    ggml_backend_reg_t reg = load_plugin(true);
+    if (!reg) { printf("{\"error\": \"no MI355X backend\"}\n"); return 2; }
+    auto get_counters = (ggml_backend_mi355x_get_counters_t) ggml_backend_reg_get_proc_address(reg, "ggml_backend_mi355x_get_counters");
+    setenv("GGML_SCHED_DEBUG", "1", 1);                 // read when a scheduler is created (ggml/src/ggml-backend.cpp:1462)
     whisper_context * gpu = open_model(path, true);
+    unsetenv("GGML_SCHED_DEBUG");
     whisper_context * cpu = open_model(path, false);
-    if (!gpu || !cpu) { printf("{\"error\": \"model load failed\"}\n"); return 2; }
-    const int n_mels = whisper_model_n_mels(cpu), n_vocab = whisper_n_vocab(cpu);
+    if (!gpu || !cpu || !get_counters) { printf("{\"error\": \"model load failed\"}\n"); return 2; }
+    const int n_mels = whisper_model_n_mels(cpu), n_vocab = whisper_n_vocab(cpu), n_text_ctx = whisper_n_text_ctx(cpu);
+    const int kv_to = std::min(a.num("kv-to", 0), n_text_ctx);
+    const int steps = a.num("steps", 32);
     const std::vector<float> mel = synth::synthetic_mel(n_mels, 3000, (uint64_t) a.num("seed", 7));
     whisper_set_mel(gpu, mel.data(), 3000, n_mels);
     whisper_set_mel(cpu, mel.data(), 3000, n_mels);
+
+    // graphs whisper computes vs what the scheduler and the plugin saw, over the GPU context's calls
+    int64_t graphs_expected = 0, cnt[GGML_MI355X_N_COUNTERS];
+    get_counters(nullptr, cnt, 1);
+    g_splits_total = g_splits_not_on_device = 0;
+
     double t0 = now_ms();
+    g_count_splits = true;
     const int eg = whisper_encode(gpu, 0, threads);
+    g_count_splits = false;
+    graphs_expected += 3;                                // conv stem, encoder, cross-attention K / V (src/whisper.cpp:2362-2466)
     const double enc_gpu_ms = now_ms() - t0; t0 = now_ms();
     const int ec = whisper_encode(cpu, 0, threads);
     const double enc_cpu_ms = now_ms() - t0;
     if (eg != 0 || ec != 0) { printf("{\"error\": \"encode failed\", \"gpu\": %d, \"cpu\": %d}\n", eg, ec); return 1; }
+    get_counters(nullptr, cnt, 0);
+    const int64_t encode_nodes = cnt[1], encode_launches = cnt[3];
 
     // prompt: <|sot|> <|en|> <|transcribe|> <|notimestamps|>  (4-token batch: exercises the n_tokens > 1 path)
-    std::vector<whisper_token> hist = { whisper_token_sot(cpu), whisper_token_lang(cpu, whisper_lang_id("en")),
+    std::vector<whisper_token> feed = { whisper_token_sot(cpu), whisper_token_lang(cpu, whisper_lang_id("en")),
                                         whisper_token_transcribe(cpu), whisper_token_not(cpu) };
-    int n_past = 0, n_same = 0, n_total = 0, n_clear = 0, n_clear_same = 0;
+    int n_past = 0, n_same = 0, n_total = 0, n_clear = 0, n_clear_same = 0, n_steps = 0;
     double worst_nmse = 0, min_margin = 1e30, sum_nmse = 0;
-    std::vector<whisper_token> feed = hist;
     bool all_ok = true;
-    for (int s = 0; s < steps; ++s) {
+    for (int s = 0; kv_to > 0 ? n_past < kv_to : s < steps; ++s) {
+        if (n_past + (int) feed.size() > n_text_ctx) feed.resize((size_t)(n_text_ctx - n_past));
+        if (kv_to > 0 && n_past + (int) feed.size() > kv_to) feed.resize((size_t)(kv_to - n_past));
+        g_count_splits = true;
         const int rg = whisper_decode(gpu, feed.data(), (int) feed.size(), n_past, threads);
+        g_count_splits = false;
+        graphs_expected += 1;
         const int rc = whisper_decode(cpu, feed.data(), (int) feed.size(), n_past, threads);
         if (rg != 0 || rc != 0) { printf("{\"error\": \"decode failed\", \"step\": %d, \"gpu\": %d, \"cpu\": %d}\n", s, rg, rc); return 1; }
-        // logits of every fed token are returned; compare all rows, sample from the last
+        // logits of every fed token are returned: every row is compared on its own
         const int rows = (int) feed.size();
         const float * lg = whisper_get_logits(gpu), * lc = whisper_get_logits(cpu);
-        double num = 0, den = 0;
-        for (int64_t i = 0; i < (int64_t) rows * n_vocab; ++i) { const double d = (double) lg[i] - lc[i]; num += d * d; den += (double) lc[i] * lc[i]; }
-        const double nmse = den > 0 ? num / den : 0;
-        float margin = 0;
-        const int tok_c = argmax(lc + (size_t)(rows - 1) * n_vocab, n_vocab, &margin);
-        const int tok_g = argmax(lg + (size_t)(rows - 1) * n_vocab, n_vocab, nullptr);
-        double d2 = 0;
-        for (int i = 0; i < n_vocab; ++i) { const double d = (double) lg[(size_t)(rows - 1) * n_vocab + i] - lc[(size_t)(rows - 1) * n_vocab + i]; d2 += d * d; }
-        const double rms_diff = sqrt(d2 / n_vocab);
-        // a step is "clear" when the reference's own top-1 / top-2 margin is more than six times the RMS difference between
-        // the two logit vectors: then the two argmaxes can only differ through an error, not through rounding noise
-        const bool clear = margin > 6.0 * rms_diff;
-        worst_nmse = std::max(worst_nmse, nmse); sum_nmse += nmse; min_margin = std::min(min_margin, (double) margin);
-        n_same += tok_c == tok_g; ++n_total;
-        n_clear += clear; n_clear_same += clear && tok_c == tok_g;
-        printf("{\"step\": %d, \"n_tokens\": %d, \"n_past\": %d, \"logits_nmse\": %.3e, \"cpu_token\": %d, \"gpu_token\": %d, \"top1_top2_margin\": %.4e, "
-               "\"logits_rms_diff\": %.4e, \"clear\": %s}\n", s, rows, n_past, nmse, tok_c, tok_g, margin, rms_diff, clear ? "true" : "false");
-        if (!(nmse <= 1e-3)) all_ok = false;
-        n_past += rows;
-        feed.assign(1, tok_c);
+        std::vector<whisper_token> next;
+        double step_worst = 0, step_min_margin = 1e30, step_rms = 0;
+        int step_same = 0, step_clear = 0, step_clear_same = 0;
+        for (int r = 0; r < rows; ++r) {
+            const float * g = lg + (size_t) r * n_vocab, * c = lc + (size_t) r * n_vocab;
+            double num = 0, den = 0;
+            for (int i = 0; i < n_vocab; ++i) { const double d = (double) g[i] - c[i]; num += d * d; den += (double) c[i] * c[i]; }
+            const double nmse = den > 0 ? num / den : 0, rms_diff = sqrt(num / n_vocab);
+            float margin = 0;
+            const int tok_c = argmax(c, n_vocab, &margin), tok_g = argmax(g, n_vocab, nullptr);
+            next.push_back(tok_c);
+            // a row is "clear" when the reference's own top-1 / top-2 margin is more than six times the RMS difference between
+            // the two logit vectors: then the two argmaxes can only differ through an error, not through rounding noise
+            const bool clear = margin > 6.0 * rms_diff;
+            const bool counted = batch > 1 || r == rows - 1;      // one-row mode: the prompt's earlier rows are compared, not sampled
+            if (!(nmse <= 1e-3)) all_ok = false;
+            step_worst = std::max(step_worst, nmse); step_rms = std::max(step_rms, rms_diff);
+            if (counted) {
+                step_min_margin = std::min(step_min_margin, (double) margin);
+                step_same += tok_c == tok_g; step_clear += clear; step_clear_same += clear && tok_c == tok_g;
+                n_same += tok_c == tok_g; ++n_total; n_clear += clear; n_clear_same += clear && tok_c == tok_g;
+                sum_nmse += nmse;
+            }
+        }
+        worst_nmse = std::max(worst_nmse, step_worst); min_margin = std::min(min_margin, step_min_margin);
+        printf("{\"step\": %d, \"n_tokens\": %d, \"n_past\": %d, \"worst_row_logits_nmse\": %.3e, \"rows_ids_identical\": %d, \"rows_clear\": %d, "
+               "\"rows_clear_identical\": %d, \"min_top1_top2_margin\": %.4e, \"max_logits_rms_diff\": %.4e}\n",
+               s, rows, n_past, step_worst, step_same, step_clear, step_clear_same, step_min_margin, step_rms);
+        n_past += rows; ++n_steps;
+        if (batch > 1) { next.resize((size_t) std::min<int>(batch, (int) next.size())); while ((int) next.size() < batch) next.push_back(next.back()); feed = next; }
+        else feed.assign(1, next.back());
     }
-    // pass: logits within the bound at every step, and identical greedy ids at every step whose margin is clear of the noise
-    const bool pass = all_ok && n_clear_same == n_clear;
-    printf("{\"summary\": \"model\", \"model\": \"%s\", \"steps\": %d, \"ids_identical\": %d, \"clear_steps\": %d, \"clear_ids_identical\": %d, "
-           "\"worst_logits_nmse\": %.3e, \"mean_logits_nmse\": %.3e, "
-           "\"min_top1_top2_margin\": %.4e, \"encode_gpu_ms_first_call\": %.2f, \"encode_cpu_ms\": %.2f, \"cpu_threads\": %d, \"pass\": %s}\n",
-           json_escape(path).c_str(), n_total, n_same, n_clear, n_clear_same, worst_nmse, sum_nmse / std::max(1, n_total), min_margin, enc_gpu_ms, enc_cpu_ms, threads,
-           pass ? "true" : "false");
+    get_counters(nullptr, cnt, 0);
+    // one split per graph, all on the device, and the plugin was called exactly once per graph
+    const bool one_split = g_splits_total == graphs_expected && g_splits_not_on_device == 0 && cnt[0] == graphs_expected;
+    // pass: logits within the bound on every row, identical greedy ids on every row whose margin is clear of the noise
+    const bool pass = all_ok && n_clear_same == n_clear && one_split;
+    printf("{\"summary\": \"model\", \"model\": \"%s\", \"batch\": %d, \"steps\": %d, \"kv_positions\": %d, \"rows\": %d, \"ids_identical\": %d, \"clear_steps\": %d, "
+           "\"clear_ids_identical\": %d, \"worst_logits_nmse\": %.3e, \"mean_logits_nmse\": %.3e, \"min_top1_top2_margin\": %.4e, "
+           "\"graphs\": %lld, \"sched_splits\": %d, \"sched_splits_not_on_device\": %d, \"plugin_graph_computes\": %lld, \"plugin_nodes\": %lld, "
+           "\"plugin_launches\": %lld, \"encode_nodes\": %lld, \"encode_launches\": %lld, \"one_split_per_graph\": %s, "
+           "\"encode_gpu_ms_first_call\": %.2f, \"encode_cpu_ms\": %.2f, \"cpu_threads\": %d, \"seed\": %d, \"pass\": %s}\n",
+           json_escape(path).c_str(), batch, n_steps, n_past, n_total, n_same, n_clear, n_clear_same, worst_nmse, sum_nmse / std::max(1, n_total), min_margin,
+           (long long) graphs_expected, g_splits_total, g_splits_not_on_device, (long long) cnt[0], (long long) cnt[1], (long long) cnt[3],
+           (long long) encode_nodes, (long long) encode_launches, one_split ? "true" : "false",
+           enc_gpu_ms, enc_cpu_ms, threads, a.num("seed", 7), pass ? "true" : "false");
     whisper_free(gpu); whisper_free(cpu);
     return pass ? 0 : 1;
 }
@@ -659,7 +716,11 @@ static int cmd_bench(const args & a) {
     } else if (what == "decoder") {
         // 5-token batches with a growing self-attention cache: the per-step work of a 5-beam search
         // (src/whisper.cpp:6089-6117), driven through whisper_decode like the batch-5 leg of whisper-bench.
-        const int n_steps = a.num("steps", 224), batch = a.num("batch", 5);
+        // Step i places its tokens at positions kv_stride * i .. + batch - 1 (capped so that they fit the cache): with
+        // --kv-stride 2 the 224 steps walk the self-attention cache up to its 448 positions.
+        const int n_steps = a.num("steps", 224), batch = a.num("batch", 5), kv_stride = a.num("kv-stride", 1);
+        const int n_text_ctx = whisper_n_text_ctx(ctx);
+        auto past_of = [&](int i) { return std::min(kv_stride * i, n_text_ctx - batch); };
         if (whisper_encode(ctx, 0, threads) != 0) return 1;
         std::vector<whisper_token> tok((size_t) batch, 0);
         for (int i = 0; i < warmup; ++i) if (whisper_decode(ctx, tok.data(), batch, i, threads) != 0) return 1;
@@ -668,21 +729,32 @@ static int cmd_bench(const args & a) {
             const double t0 = now_ms();
             for (int i = 0; i < n_steps; ++i) {
                 for (int j = 0; j < batch; ++j) tok[(size_t) j] = (whisper_token)((i * 131 + j * 17) % 50000);
-                if (whisper_decode(ctx, tok.data(), batch, i, threads) != 0) return 1;
+                if (whisper_decode(ctx, tok.data(), batch, past_of(i), threads) != 0) return 1;
             }
             per_rep.push_back(now_ms() - t0);
         }
         const double ms = median(per_rep);
         std::string kernels = "[]";
+        int64_t cnt[GGML_MI355X_N_COUNTERS] = {};
+        if (use_gpu) {
+            auto get_counters = (ggml_backend_mi355x_get_counters_t) ggml_backend_reg_get_proc_address(reg, "ggml_backend_mi355x_get_counters");
+            if (get_counters) {                           // launches and downloads of one more pass, unprofiled
+                get_counters(nullptr, cnt, 1);
+                for (int i = 0; i < n_steps; ++i) if (whisper_decode(ctx, tok.data(), batch, past_of(i), threads) != 0) return 1;
+                get_counters(nullptr, cnt, 1);
+            }
+        }
         if (profile) {
             plugin_set_option(reg, "profile", 1); plugin_stats(reg, true);
-            for (int i = 0; i < n_steps; ++i) if (whisper_decode(ctx, tok.data(), batch, i, threads) != 0) return 1;
+            for (int i = 0; i < n_steps; ++i) if (whisper_decode(ctx, tok.data(), batch, past_of(i), threads) != 0) return 1;
             kernels = plugin_stats(reg, true);
             plugin_set_option(reg, "profile", 0);
         }
-        printf("{\"bench\": \"decoder\", \"backend\": \"%s\", \"threads\": %d, \"reps\": %d, \"steps\": %d, \"batch\": %d, \"total_ms_median\": %.3f, "
-               "\"ms_per_step\": %.5f, \"steps_per_s\": %.2f, \"batch_tokens_per_s\": %.2f, \"profiled\": %s, \"kernels\": %s, \"model\": \"%s\"}\n",
-               be.c_str(), threads, reps, n_steps, batch, ms, ms / n_steps, 1000.0 * n_steps / ms, 1000.0 * n_steps * batch / ms,
+        printf("{\"bench\": \"decoder\", \"backend\": \"%s\", \"threads\": %d, \"reps\": %d, \"steps\": %d, \"batch\": %d, \"kv_stride\": %d, \"max_kv_positions\": %d, "
+               "\"total_ms_median\": %.3f, \"ms_per_step\": %.5f, \"ms_per_step_min\": %.5f, \"steps_per_s\": %.2f, \"batch_tokens_per_s\": %.2f, \"launches_per_step\": %.2f, "
+               "\"downloads_from_mirror_per_step\": %.2f, \"downloads_by_copy_per_step\": %.2f, \"profiled\": %s, \"kernels\": %s, \"model\": \"%s\"}\n",
+               be.c_str(), threads, reps, n_steps, batch, kv_stride, past_of(n_steps - 1) + batch, ms, ms / n_steps, *std::min_element(per_rep.begin(), per_rep.end()) / n_steps,
+               1000.0 * n_steps / ms, 1000.0 * n_steps * batch / ms, (double) cnt[3] / n_steps, (double) cnt[4] / n_steps, (double) cnt[5] / n_steps,
                profile ? "true" : "false", kernels.c_str(), json_escape(path).c_str());
     } else {   // whisper-bench protocol, verbatim counts (examples/bench/bench.cpp:86-138)
         whisper_token tokens[512]; memset(tokens, 0, sizeof(tokens));
@@ -781,8 +853,101 @@ static int cmd_copy(const args & a) {
     return 0;
 }
 
+// the host side of a step's boundary: results that the host reads back are mirrored in pinned memory after the first
+// download and served from there until something writes them; and the device's pinned host buffer type
+static int cmd_download(const args & a) {
+    ggml_backend_reg_t reg = load_plugin(true);
+    if (!reg) { printf("{\"error\": \"no MI355X backend\"}\n"); return 2; }
+    ggml_backend_dev_t dev = ggml_backend_reg_dev_get(reg, 0);
+    ggml_backend_t be = ggml_backend_dev_init(dev, nullptr);
+    auto get_counters = (ggml_backend_mi355x_get_counters_t) ggml_backend_reg_get_proc_address(reg, "ggml_backend_mi355x_get_counters");
+    if (!be || !get_counters) return 1;
+    const int64_t n = a.num("n", 51866 * 5);            // the logits of a 5-beam step
+    const int rows = 5;
+    ggml_init_params ip = { ggml_tensor_overhead() * 8 + ggml_graph_overhead(), nullptr, true };
+    ggml_context * ctx = ggml_init(ip);
+    ggml_tensor * x = ggml_new_tensor_1d(ctx, GGML_TYPE_F32, n);
+    ggml_tensor * y = ggml_scale(ctx, x, 2.0f);         // the graph's last node: what whisper's logits are (src/whisper.cpp:2953)
+    ggml_cgraph * gf = ggml_new_graph(ctx);
+    ggml_build_forward_expand(gf, y);
+    ggml_backend_buffer_t buf = ggml_backend_alloc_ctx_tensors(ctx, be);
+    if (!buf) return 1;
+    std::vector<float> in1((size_t) n), in2((size_t) n), got((size_t) n), other((size_t) n);
+    for (int64_t i = 0; i < n; ++i) { in1[(size_t) i] = synth::normal_at(5, (uint64_t) i); in2[(size_t) i] = synth::normal_at(6, (uint64_t) i); other[(size_t) i] = (float) i; }
+    int64_t c[GGML_MI355X_N_COUNTERS];
+    int bad = 0;
+    auto fetch_rows = [&]() {                              // row by row, as whisper_decode does (src/whisper.cpp:2960-2966)
+        std::fill(got.begin(), got.end(), -1.0f);
+        const int64_t per = n / rows;
+        for (int r = 0; r < rows; ++r) {
+            const int64_t cnt = r == rows - 1 ? n - per * (rows - 1) : per;
+            ggml_backend_tensor_get(y, got.data() + per * r, sizeof(float) * (size_t)(per * r), sizeof(float) * (size_t) cnt);
+        }
+    };
+    auto expect = [&](const std::vector<float> & in, float f, const char * what, int64_t want_mirror, int64_t want_copy) {
+        bool same = true;
+        for (int64_t i = 0; i < n && same; ++i) same = got[(size_t) i] == in[(size_t) i] * f;
+        get_counters(be, c, 1);
+        const bool ok = same && c[4] == want_mirror && c[5] == want_copy;
+        bad += !ok;
+        printf("{\"download\": \"%s\", \"bytes_equal\": %s, \"from_mirror\": %lld, \"by_copy\": %lld, \"ok\": %s}\n", what, same ? "true" : "false", (long long) c[4], (long long) c[5], ok ? "true" : "false");
+    };
+    get_counters(be, c, 1);
+    ggml_backend_tensor_set(x, in1.data(), 0, ggml_nbytes(x));
+    if (ggml_backend_graph_compute(be, gf) != GGML_STATUS_SUCCESS) return 1;
+    fetch_rows(); expect(in1, 2.0f, "first graph: blocking copies (the tensor is not known yet)", 0, rows);
+    ggml_backend_tensor_set(x, in2.data(), 0, ggml_nbytes(x));
+    if (ggml_backend_graph_compute(be, gf) != GGML_STATUS_SUCCESS) return 1;
+    fetch_rows(); expect(in2, 2.0f, "second graph: served from the pinned mirror", rows, 0);
+    fetch_rows(); expect(in2, 2.0f, "read again: still the mirror", rows, 0);
+    ggml_backend_tensor_set(y, other.data(), 0, ggml_nbytes(y));               // the host overwrites the result
+    fetch_rows(); expect(other, 1.0f, "after a write into the tensor: the mirror is stale, blocking copies", 0, rows);
+    ggml_backend_tensor_set(y, in1.data(), sizeof(float) * 100, sizeof(float) * 50);   // (and a partial write, after a new graph)
+    if (ggml_backend_graph_compute(be, gf) != GGML_STATUS_SUCCESS) return 1;
+    ggml_backend_tensor_set(y, other.data(), sizeof(float) * 100, sizeof(float) * 50);
+    fetch_rows();
+    { std::vector<float> want((size_t) n); for (int64_t i = 0; i < n; ++i) want[(size_t) i] = (i >= 100 && i < 150) ? other[(size_t)(i - 100)] : 2.0f * in2[(size_t) i];
+      expect(want, 1.0f, "after a partial write behind a new graph: blocking copies", 0, rows); }
+    if (ggml_backend_graph_compute(be, gf) != GGML_STATUS_SUCCESS) return 1;
+    double t0 = now_ms();
+    for (int i = 0; i < 50; ++i) { if (ggml_backend_graph_compute(be, gf) != GGML_STATUS_SUCCESS) return 1; fetch_rows(); }
+    const double ms_mirror = (now_ms() - t0) / 50;
+    expect(in2, 2.0f, "timed loop with the mirror", 50 * rows, 0);
+
+    // the pinned host buffer type: an ordinary host buffer for every CPU-side user, a source of device copies
+    ggml_backend_buffer_type_t hbt = ggml_backend_dev_host_buffer_type(dev);
+    bool host_ok = hbt && ggml_backend_buft_is_host(hbt);
+    if (host_ok) {
+        ggml_init_params ip2 = { ggml_tensor_overhead() * 4, nullptr, true };
+        ggml_context * hctx = ggml_init(ip2);
+        ggml_tensor * hx = ggml_new_tensor_1d(hctx, GGML_TYPE_F32, n);
+        ggml_backend_buffer_t hbuf = ggml_backend_alloc_ctx_tensors_from_buft(hctx, hbt);
+        host_ok = hbuf && ggml_backend_buffer_is_host(hbuf) && hx->data;
+        if (host_ok) {
+            memcpy(hx->data, in1.data(), ggml_nbytes(hx));            // host code writes it directly
+            ggml_backend_tensor_copy(hx, x);                          // pinned host -> device
+            if (ggml_backend_graph_compute(be, gf) != GGML_STATUS_SUCCESS) return 1;
+            fetch_rows();
+            for (int64_t i = 0; i < n && host_ok; ++i) host_ok = got[(size_t) i] == 2.0f * in1[(size_t) i];
+            ggml_backend_tensor_copy(y, hx);                          // device -> pinned host
+            ggml_backend_synchronize(be);
+            for (int64_t i = 0; i < n && host_ok; ++i) host_ok = ((const float *) hx->data)[i] == 2.0f * in1[(size_t) i];
+        }
+        if (hbuf) ggml_backend_buffer_free(hbuf);
+        ggml_free(hctx);
+    }
+    bad += !host_ok;
+    ggml_backend_dev_props props; ggml_backend_dev_get_props(dev, &props);
+    printf("{\"summary\": \"download\", \"failed\": %d, \"host_buffer_type\": \"%s\", \"host_buffer_ok\": %s, \"caps_host_buffer\": %s, \"ms_per_graph_and_5_reads_mirror\": %.4f, \"bytes\": %lld}\n",
+           bad, hbt ? ggml_backend_buft_name(hbt) : "", host_ok ? "true" : "false", props.caps.host_buffer ? "true" : "false", ms_mirror, (long long)(n * 4));
+    ggml_backend_buffer_free(buf);
+    ggml_free(ctx);
+    ggml_backend_free(be);
+    return bad ? 1 : 0;
+}
+
 int main(int argc, char ** argv) {
-    if (argc < 2) { fprintf(stderr, "usage: %s info|gen|selftest|ops|model|full|verify|bench|copy|mel [options]\n", argv[0]); return 2; }
+    if (argc < 2) { fprintf(stderr, "usage: %s info|gen|selftest|ops|model|full|verify|bench|copy|mel|download [options]\n", argv[0]); return 2; }
     ggml_log_set(quiet_log, nullptr);
     whisper_log_set(quiet_log, nullptr);
     const std::string cmd = argv[1];
@@ -801,6 +966,7 @@ int main(int argc, char ** argv) {
     if (cmd == "bench") return cmd_bench(a);
     if (cmd == "copy")  return cmd_copy(a);
     if (cmd == "mel")   return cmd_mel(a);
+    if (cmd == "download") return cmd_download(a);
     fprintf(stderr, "unknown command %s\n", cmd.c_str());
     return 2;
 }

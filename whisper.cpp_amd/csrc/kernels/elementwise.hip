@@ -283,10 +283,14 @@ __global__ void k_get_rows(tview s, tview ids, tview d) {
     const int64_t r   = blockIdx.y;
     const int64_t i10 = r % ids.ne0, i11 = (r / ids.ne0) % ids.ne1, i12 = r / (ids.ne0 * ids.ne1);
     const int32_t row = *(const int32_t *)(ids.p + i10*ids.nb0 + i11*ids.nb1 + i12*ids.nb2);
-    const uint8_t * sp = (const uint8_t *) s.p + (int64_t) row*s.nb1 + i11*s.nb2 + i12*s.nb3;
+    // The reference stops the process on an index outside the matrix (GGML_ASSERT(i01 >= 0 && i01 < ne01), ops.cpp:4174).
+    // Here such a row is not read — the address would be outside the tensor — and the gathered row is NaN throughout, so
+    // that the mistake shows in everything computed from it.
+    const bool ok = row >= 0 && row < s.ne1;
+    const uint8_t * sp = (const uint8_t *) s.p + (int64_t)(ok ? row : 0)*s.nb1 + i11*s.nb2 + i12*s.nb3;
     float * dp = (float *)(d.p + i10*d.nb1 + i11*d.nb2 + i12*d.nb3);
     for (int64_t k = (int64_t) blockIdx.x * blockDim.x + threadIdx.x; k < d.ne0; k += (int64_t) gridDim.x * blockDim.x) {
-        dp[k] = dq_elem<TYPE>(sp, k);
+        dp[k] = ok ? dq_elem<TYPE>(sp, k) : __builtin_nanf("");
     }
 }
 
@@ -317,11 +321,12 @@ template <int TYPE>
 __global__ void k_get_rows_add(tview s0, tview ids0, tview s1, tview ids1, tview d) {
     const int64_t i = blockIdx.y;
     const int32_t r0 = *(const int32_t *)(ids0.p + i * ids0.nb0), r1 = *(const int32_t *)(ids1.p + i * ids1.nb0);
-    const uint8_t * sp = (const uint8_t *) s0.p + (int64_t) r0 * s0.nb1;
-    const float *   pp = (const float *)(s1.p + (int64_t) r1 * s1.nb1);
+    const bool ok = r0 >= 0 && r0 < s0.ne1 && r1 >= 0 && r1 < s1.ne1;      // as in k_get_rows: an index outside either matrix gives a NaN row
+    const uint8_t * sp = (const uint8_t *) s0.p + (int64_t)(ok ? r0 : 0) * s0.nb1;
+    const float *   pp = (const float *)(s1.p + (int64_t)(ok ? r1 : 0) * s1.nb1);
     float * dp = (float *)(d.p + i * d.nb1);
     for (int64_t k = (int64_t) blockIdx.x * blockDim.x + threadIdx.x; k < d.ne0; k += (int64_t) gridDim.x * blockDim.x) {
-        dp[k] = dq_elem<TYPE>(sp, k) + pp[k];
+        dp[k] = ok ? dq_elem<TYPE>(sp, k) + pp[k] : __builtin_nanf("");
     }
 }
 

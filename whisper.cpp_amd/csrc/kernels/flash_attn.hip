@@ -12,7 +12,7 @@
 //                                parallel up front and only the one-instruction f16 fma chain stays sequential.
 //       k_fattn_seq_tile   N > 8:  64 queries x 64 keys per step; QK^T on v_mfma_f32_32x32x16_f16 from LDS-staged K,
 //                                  softmax factors in LDS, then 16 queries per wavefront walk the 64 keys with
-//                                  v_fma_mixlo/hi_f16 chains against the LDS-staged V tile.
+//                                  v_fma_mix_f32 + v_cvt_pk_f16_f32 chains against the LDS-staged V tile.
 //       k_fattn_seq_row    N <= 8: one block per (query, head): one wavefront (lane = d) runs the chain while the
 //                                  other three score, scan and stage the next 192 keys.
 //   MI355X_FA_F32          f32 accumulators: closer to exact arithmetic, not to the reference (whose f16 accumulator
@@ -486,12 +486,6 @@ __device__ __forceinline__ float exp_neg(float x) {
 
 typedef const uint32_t __attribute__((address_space(4))) * const_u32_ptr;   // read-only data: uniform loads become scalar loads
 
-// PACKED (MI355X_FA_F16_PACKED): the accumulation is the f16 fused multiply-add of the reference's Arm fp16 build instead
-// (GGML_F16_VEC_FMA = vfmaq_f16 on the factor converted to f16, GGML_F16_VEC_MUL for the rescale; simd-mappings.h:67-78,
-// vec.h:180-197, 295-310): one v_pk_fma_f16 per two accumulators.  A third of the arithmetic; LDS could not deliver the
-// V operands that fast as broadcast reads, so a wavefront holds the tile's V slice distributed over its lanes (lane =
-// key) and hands each key's eight registers to the packed fma as scalar operands through v_readlane.
-template <bool PACKED>
 __global__ void __launch_bounds__(256) k_fattn_seq_tile(fa_args a) {
     __shared__ __attribute__((aligned(16))) half_t q_s[T_Q * T_LDH];
     __shared__ __attribute__((aligned(16))) half_t k_s[T_KV * T_LDH];
@@ -523,10 +517,9 @@ __global__ void __launch_bounds__(256) k_fattn_seq_tile(fa_args a) {
     // chain role: a lane owns 16 of the 64 d of one query.  A wavefront takes 16 queries x all four d slices (lane = query
     // 16 w + l % 16, slice l / 16): a key that raises the running maximum of any query of the wavefront costs the whole
     // wavefront a rescale of its accumulators, and with 16 queries instead of 64 that happens for 6 % of the keys instead
-    // of 18 % (records of an i.i.d. sequence: about min(1, queries / k) at key k).  The packed variant keeps lane = query,
-    // wavefront = slice, because it hands V over as wavefront-uniform scalars.
-    const int cq = PACKED ? lane : 16 * wave + (lane & 15);
-    const int d0 = PACKED ? wave * 16 : (lane >> 4) * 16;
+    // of 18 % (records of an i.i.d. sequence: about min(1, queries / k) at key k).
+    const int cq = 16 * wave + (lane & 15);
+    const int d0 = (lane >> 4) * 16;
     half2_t acc2[8];                                       // 16 f16 accumulators, two per register
 #pragma unroll
     for (int e = 0; e < 8; ++e) acc2[e] = (half2_t){ (half_t) 0.0f, (half_t) 0.0f };
@@ -612,10 +605,6 @@ __global__ void __launch_bounds__(256) k_fattn_seq_tile(fa_args a) {
                 M = raised ? s : M;
                 P *= ms; A = A * ms + vs;
                 sv[i] = raised ? -ex : ex;                 // -0.0 keeps the sign
-                if (PACKED) {                              // the factor as the f16 pair the packed fma takes
-                    const uint32_t hb = f2h_bits(sv[i]);
-                    sv[i] = __uint_as_float(hb | (hb << 16));
-                }
             }
 #pragma unroll
             for (int i = 0; i < 4; ++i) fp[i] = make_float4(sv[4*i], sv[4*i+1], sv[4*i+2], sv[4*i+3]);
@@ -633,51 +622,7 @@ __global__ void __launch_bounds__(256) k_fattn_seq_tile(fa_args a) {
         __syncthreads();
 
         // ---- the sequential f16 chains over this tile's keys -----------------------------------------------------------------------------
-        if constexpr (PACKED) {
-            const int nk = (int)(a.KV - key0 < T_KV ? a.KV - key0 : T_KV);       // uniform
-            const float4 * fp = (const float4 *)(f_s + cq * T_LDF);
-            uint32_t vk[8];                                                       // V[key = lane][d0 .. d0 + 15]
-            {
-                const u32x4 * vr = (const u32x4 *)(v_s + lane * FA_D + d0);
-                const u32x4 lo = vr[0], hi = vr[1];
-                vk[0] = lo.x; vk[1] = lo.y; vk[2] = lo.z; vk[3] = lo.w; vk[4] = hi.x; vk[5] = hi.y; vk[6] = hi.z; vk[7] = hi.w;
-            }
-            float4 fnext = fp[0];
-            for (int k4 = 0; k4 < nk; k4 += 4) {
-                const float4 f4 = fnext;
-                if (k4 + 4 < nk) fnext = fp[(k4 >> 2) + 1];
-                const uint32_t fk[4] = { __float_as_uint(f4.x), __float_as_uint(f4.y), __float_as_uint(f4.z), __float_as_uint(f4.w) };
-                const bool any_raised = __any((fk[0] | fk[1] | fk[2] | fk[3]) >> 31);
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    if (k4 + j < nk) {
-                        half2_t f2; __builtin_memcpy(&f2, &fk[j], 4);
-                        if (any_raised) {
-                            const bool raised = fk[j] >> 31;
-                            if (__any(raised)) {
-                                const half2_t one = { (half_t) 1.0f, (half_t) 1.0f };
-                                const half2_t ms2 = raised ? -f2 : one;
-#pragma unroll
-                                for (int e = 0; e < 8; ++e) acc2[e] = acc2[e] * ms2;
-                                f2 = raised ? one : f2;
-                            }
-                        }
-                        // all eight scalar reads first, then the eight fmas: a scalar register written by the vector unit
-                        // needs two idle cycles before the vector unit may read it, paid once per key instead of per fma
-                        uint32_t vs8[8];
-#pragma unroll
-                        for (int e = 0; e < 8; ++e) vs8[e] = (uint32_t) __builtin_amdgcn_readlane((int) vk[e], k4 + j);
-                        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-                        for (int e = 0; e < 8; ++e) {
-                            half2_t v2; __builtin_memcpy(&v2, &vs8[e], 4);
-                            acc2[e] = __builtin_elementwise_fma(v2, f2, acc2[e]);
-                        }
-                        __builtin_amdgcn_sched_barrier(0);
-                    }
-                }
-            }
-        } else {
+        {
             const int nk = (int)(a.KV - key0 < T_KV ? a.KV - key0 : T_KV);       // uniform
             const float4 * fp = (const float4 *)(f_s + cq * T_LDF);
             const half8_t * vp = (const half8_t *)(v_s + d0);                    // + key * FA_D halves = 8 of these
@@ -764,14 +709,8 @@ __global__ void __launch_bounds__(256) k_fattn_seq_tile(fa_args a) {
         float amax = 0.0f;
 #pragma unroll
         for (int e = 0; e < 16; ++e) amax = fmaxf(amax, fabsf(o[e]));
-        if constexpr (PACKED) {                            // the other half of the block is in the neighbouring wavefront
-            __syncthreads();                               // every chain is done with the factor tile
-            f_s[wave * T_Q + lane] = amax;
-            __syncthreads();
-            amax = fmaxf(amax, f_s[(wave ^ 1) * T_Q + lane]);
-        } else {                                           // ... in lane ^ 16
-            amax = fmaxf(amax, __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, amax), 0x401F)));
-        }
+        // (the other half of the block is in lane ^ 16)
+        amax = fmaxf(amax, __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, amax), 0x401F)));
         if (n < a.N) {
             const float id = amax != 0.0f ? 127.0f / amax : 0.0f;
             const float dq = h2f(f2h_bits(amax / 127.0f));
@@ -1000,7 +939,7 @@ extern "C" const char * mi355x_flash_attn_ext_kernel_name(const mi355x_tensor * 
     if (!q || !k) return "flash_attn.invalid";
     switch (fa_kernel(q, k, mode)) {
         case FA_K_SEQ_ROW:  return "flash_attn.seq_row";
-        case FA_K_SEQ_TILE: return mode == MI355X_FA_F16_PACKED ? "flash_attn.seq_tile_packed" : "flash_attn.seq_tile";
+        case FA_K_SEQ_TILE: return "flash_attn.seq_tile";
         case FA_K_MFMA:     return "flash_attn.mfma_f32";
         default:            return "flash_attn.vec_f32";
     }
@@ -1018,7 +957,7 @@ static int flash_attn_ext(const mi355x_tensor * q, const mi355x_tensor * k, cons
     const bool emit = mode & MI355X_FA_EMIT_F16, emit_q8 = mode & MI355X_FA_EMIT_Q8_0;
     mode &= ~(MI355X_FA_EMIT_F16 | MI355X_FA_EMIT_Q8_0);
     if (emit && emit_q8) return MI355X_ERR_INVALID;
-    if (mode != MI355X_FA_F16_SEQ && mode != MI355X_FA_F32 && mode != MI355X_FA_F16_PACKED) return MI355X_ERR_INVALID;
+    if (mode != MI355X_FA_F16_SEQ && mode != MI355X_FA_F32) return MI355X_ERR_INVALID;
     if (q->type != MI355X_TYPE_F32 || k->type != MI355X_TYPE_F16 || v->type != MI355X_TYPE_F16 || dst->type != MI355X_TYPE_F32) return MI355X_ERR_UNSUPPORTED;
     if (q->ne[0] != FA_D || k->ne[0] != FA_D || v->ne[0] != FA_D) return MI355X_ERR_UNSUPPORTED;
     if (q->nb[0] != 4 || k->nb[0] != 2 || v->nb[0] != 2) return MI355X_ERR_UNSUPPORTED;
@@ -1035,6 +974,12 @@ static int flash_attn_ext(const mi355x_tensor * q, const mi355x_tensor * k, cons
     if (mask_f16) {                                        // the f16 copy of an F32 mask, written on the way
         if (!mask || mask->type != MI355X_TYPE_F32 || mask_f16->type != MI355X_TYPE_F16) return MI355X_ERR_UNSUPPORTED;
         if (mask_f16->ne[0] != KV || mask_f16->ne[1] < N || mask_f16->nb[0] != 2 || !mask_f16->data) return MI355X_ERR_INVALID;
+        // dst is written by workgroups that finish while others still read the mask, and the copy is written while the f32
+        // form is read: the three may not share memory
+        auto overlap = [](const void * a, size_t an, const void * b, size_t bn) { return (const char *) a < (const char *) b + bn && (const char *) b < (const char *) a + an; };
+        const size_t dst_bytes = (size_t)(N * H * q->ne[3]) * FA_D * 4, m32_bytes = (size_t) mask->nb[1] * (size_t) N, m16_bytes = (size_t) mask_f16->nb[1] * (size_t) N;
+        if (overlap(dst->data, dst_bytes, mask->data, m32_bytes) || overlap(dst->data, dst_bytes, mask_f16->data, m16_bytes) ||
+            overlap(mask->data, m32_bytes, mask_f16->data, m16_bytes)) return MI355X_ERR_INVALID;
     }
     auto al16 = [](const mi355x_tensor * t) {
         return (uintptr_t) t->data % 16 == 0 && t->nb[1] % 16 == 0 && t->nb[2] % 16 == 0 && t->nb[3] % 16 == 0;
@@ -1083,8 +1028,7 @@ static int flash_attn_ext(const mi355x_tensor * q, const mi355x_tensor * k, cons
             const int64_t gx = (N + T_Q - 1) / T_Q;
             if (gx > 0x7fffffff) return MI355X_ERR_UNSUPPORTED;
             dim3 grid((unsigned) gx, (unsigned) H, (unsigned) q->ne[3]);
-            if (mode == MI355X_FA_F16_PACKED) k_fattn_seq_tile<true ><<<grid, 256, 0, st>>>(a);
-            else                              k_fattn_seq_tile<false><<<grid, 256, 0, st>>>(a);
+            k_fattn_seq_tile<<<grid, 256, 0, st>>>(a);
         } break;
         case FA_K_MFMA: {
             const int64_t gx = (N + M_Q - 1) / M_Q;
