@@ -124,6 +124,20 @@ MI355X_API size_t mi355x_mul_mat_workspace_size(const mi355x_tensor * src0, cons
 MI355X_API int    mi355x_mul_mat(const mi355x_tensor * src0, const mi355x_tensor * src1, const mi355x_tensor * dst,
                                  const mi355x_epilogue * epi, void * workspace, size_t workspace_size, void * stream);
 
+/* mi355x_mul_mat without a workspace argument and without any allocation: the scratch memory (the f16 / Q8_0 forms of the
+ * operands that mi355x_mul_mat keeps in `workspace`) is a fixed array of MI355X_MUL_MAT_NOALLOC_MAX bytes in device
+ * memory that the library owns, one copy per GPU, held until the process ends.  No counterpart in the reference; it is
+ * for callers that cannot allocate device memory: code under HIP graph capture, tight serving loops, harnesses that
+ * forbid hipMalloc.  Same arguments, kernels and results as mi355x_mul_mat.  MI355X_ERR_WORKSPACE when the operands need
+ * more scratch than the array holds (mi355x_mul_mat_workspace_size > MI355X_MUL_MAT_NOALLOC_MAX);
+ * MI355X_ERR_INVALID with MI355X_MM_WS_READY or MI355X_MM_PREPARE_ONLY (the array is shared by every call on a GPU and keeps
+ * the last call's contents, so no call may rely on them).  Calls that overlap on one GPU (two streams, two threads) race
+ * on the array: serialize them.  The first call on a device looks up the array's address, and the first call with
+ * MI355X_EPI_GELU fills the GELU table with a synchronous copy: make those calls before a capture starts. */
+#define MI355X_MUL_MAT_NOALLOC_MAX ((size_t) 32 << 20)
+MI355X_API int    mi355x_mul_mat_noalloc(const mi355x_tensor * src0, const mi355x_tensor * src1, const mi355x_tensor * dst,
+                                         const mi355x_epilogue * epi, void * stream);
+
 /* Several MUL_MATs over the same src1 in one launch (a layer's Q, K and V projections; the cross-attention K and V of all
  * decoder layers): the same arithmetic as `count` calls of mi355x_mul_mat, item by item, but one grid that fills the
  * device where a single 1280-row product covers half of it.  No counterpart in the reference, whose graphs issue these

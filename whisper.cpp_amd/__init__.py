@@ -25,6 +25,7 @@ BLOCK_BYTES = {Q5_0: 22, Q8_0: 34}
 # enum mi355x_epilogue_flags
 EPI_BIAS, EPI_GELU, EPI_SCALE, EPI_RESIDUAL, EPI_BIAS_COL, EPI_OUT_F16 = 1, 2, 4, 8, 16, 32
 MM_EXACT_ACT, MM_WS_READY, MM_ACT_Q8_0, MM_PREPARE_ONLY, EPI_EMIT_F16 = 64, 128, 256, 512, 1024
+MUL_MAT_NOALLOC_MAX = 32 << 20
 # enum mi355x_fa_mode
 FA_F16_SEQ, FA_F32, FA_EMIT_F16, FA_EMIT_Q8_0 = 0, 1, 0x100, 0x200
 
@@ -69,6 +70,7 @@ def kernels() -> C.CDLL:
             "mi355x_mul_mat_kernel_name": (C.c_char_p, [T, T]),
             "mi355x_mul_mat_workspace_size": (C.c_size_t, [T, T]),
             "mi355x_mul_mat": (C.c_int, [T, T, T, C.POINTER(Epilogue), P, C.c_size_t, P]),
+            "mi355x_mul_mat_noalloc": (C.c_int, [T, T, T, C.POINTER(Epilogue), P]),
             "mi355x_mul_mat_group": (C.c_int, [C.POINTER(MulMatItem), C.c_int, T, C.c_int, P, C.c_size_t, P]),
             "mi355x_q8_0_tiles_size": (C.c_size_t, [C.c_int64, C.c_int64]),
             "mi355x_q8_0_tiles_pack": (C.c_int, [T, P, P]),

@@ -15,6 +15,8 @@
 //                     ggml_vec_dot_q8_0_q8_0 / ggml_vec_dot_q5_0_q8_0 (ggml-cpu-quants.c:3597, 2930).
 //   * k_mul_mat_generic — any strides / K; one wavefront per output row, f32 FMA.
 #include "common.h"
+
+#include <mutex>
 #include <stdlib.h>
 #include <type_traits>
 
@@ -1611,3 +1613,44 @@ extern "C" int mi355x_mul_mat(const mi355x_tensor * src0, const mi355x_tensor * 
     k_mul_mat_generic<<<grid, WAVE, 0, st>>>(a, t0, t1);
     return launch_status();
 }
+
+// ------------------------------------------------------------------------------------------------------
+// mi355x_mul_mat for callers that cannot allocate (code under HIP graph capture, serving loops, harnesses that forbid
+// hipMalloc): the workspace is a fixed array in device memory that belongs to the library, one copy per GPU.
+// ------------------------------------------------------------------------------------------------------
+
+#define MM_SCRATCH_BYTES (32u << 20)
+
+static __device__ __align__(256) unsigned char scratch[MM_SCRATCH_BYTES];
+
+// The array's device address on the current device (each GPU holds its own copy at its own address), looked up once per
+// device with that device current.  `scratch` itself is only a host-side handle: host code never passes it to a kernel
+// or a copy, always this pointer.
+static void * scratch_on_current_device() {
+    static std::mutex mu;
+    static void * ptr[64] = {};
+    static bool   failed[64] = {};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) { (void) hipGetLastError(); return nullptr; }
+    std::lock_guard<std::mutex> lock(mu);
+    if (ptr[dev] || failed[dev]) return ptr[dev];
+    void * p = nullptr;
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || !p) { (void) hipGetLastError(); failed[dev] = true; return nullptr; }
+    ptr[dev] = p;
+    return p;
+}
+
+extern "C" int mi355x_mul_mat_noalloc(const mi355x_tensor * src0, const mi355x_tensor * src1, const mi355x_tensor * dst,
+                                      const mi355x_epilogue * epi, void * stream) {
+    if (!src0 || !src1 || !dst) return MI355X_ERR_INVALID;
+    // the array keeps whatever the call before left in it: nothing may claim that it already holds this call's activations
+    if (epi && (epi->flags & (MI355X_MM_WS_READY | MI355X_MM_PREPARE_ONLY))) return MI355X_ERR_INVALID;
+    const size_t need = mi355x_mul_mat_workspace_size(src0, src1);
+    if (need > MM_SCRATCH_BYTES) return MI355X_ERR_WORKSPACE;         // beyond the array: use mi355x_mul_mat with a workspace of the caller's
+    void * ws = scratch_on_current_device();
+    if (!ws) return MI355X_ERR_HIP;
+    // every byte a kernel of this call reads from the array is written by this call's own conversion pass first, so
+    // nothing needs clearing
+    return mi355x_mul_mat(src0, src1, dst, epi, ws, MM_SCRATCH_BYTES, stream);
+}
+
