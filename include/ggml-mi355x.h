@@ -77,7 +77,8 @@ typedef size_t (*ggml_backend_mi355x_get_stats_t)(ggml_backend_t backend, char *
  * out[0] graph_compute calls, out[1] nodes of the graphs as received, out[2] those of them that are not view ops or empty
  * tensors (every one of them is carried out by a launch of this backend: there is no other path), out[3] kernel
  * launches, out[4] get_tensor calls served from the pinned host mirror of a graph output, out[5] get_tensor calls that
- * were a blocking device-to-host copy, out[6..7] zero.  A host that sees one call per graph it computes, with the graph's
+ * were a blocking device-to-host copy, out[6] nanoseconds of host time inside graph_compute (planning and queueing the
+ * launches), out[7] nanoseconds the host waited inside synchronize.  A host that sees one call per graph it computes, with the graph's
  * full node count, knows that the scheduler (ggml_backend_sched_split_graph, ggml/src/ggml-backend.cpp:863-1317) left
  * no node to another backend. */
 #define GGML_MI355X_N_COUNTERS 8

@@ -111,7 +111,7 @@ struct mi355x_backend_ctx {
     // Host mirror of graph outputs (the logits of a decode step): tensors flagged GGML_TENSOR_FLAG_OUTPUT that the host has
     // downloaded before are copied into pinned memory at the end of graph_compute, on the stream, in one transfer each;
     // get_tensor then serves any slice of them from there until something writes the tensor or the next graph runs.
-    struct mirror_entry { const char * dev; size_t size, off; };
+    struct mirror_entry { const char * dev; size_t lo, size, off; };    // bytes [lo, lo + size) of the tensor at `dev`, at `off` in the block
     std::mutex                mirror_mutex;
     char *                    mirror_host = nullptr;      // pinned
     size_t                    mirror_cap  = 0;
@@ -130,7 +130,7 @@ struct mi355x_backend_ctx {
 };
 
 // ggml-mi355x.cpp: has the host downloaded the tensor at this address before (so that mirroring it pays)?
-bool mi355x_download_is_wanted(int device, const void * data, size_t size);
+bool mi355x_download_is_wanted(int device, const void * data, size_t size, size_t * lo, size_t * hi);
 
 // graph.cpp
 enum ggml_status mi355x_graph_compute(mi355x_backend_ctx * ctx, struct ggml_cgraph * cgraph);

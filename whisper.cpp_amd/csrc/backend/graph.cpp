@@ -12,6 +12,7 @@
 
 #include <string.h>
 #include <algorithm>
+#include <chrono>
 #include <unordered_map>
 
 static mi355x_tensor to_view(const ggml_tensor * t) {
@@ -143,8 +144,9 @@ void mi355x_backend_ctx::mirror_outputs(struct ggml_cgraph * cgraph) {
         const ggml_tensor * n = cgraph->nodes[i];
         // only tensors whose memory the allocator cannot have handed on by the end of the graph
         if (!((n->flags & GGML_TENSOR_FLAG_OUTPUT) || i == cgraph->n_nodes - 1) || !n->data || n->view_src || ggml_is_empty(n) || !ggml_is_contiguous(n)) continue;
-        const size_t size = ggml_nbytes(n);
-        if (size > MI355X_MIRROR_MAX || !mi355x_download_is_wanted(device, n->data, size)) continue;
+        size_t lo = 0, hi = 0;                            // the part of it the host has asked for (one row of five, or all)
+        if (ggml_nbytes(n) > MI355X_MIRROR_MAX || !mi355x_download_is_wanted(device, n->data, ggml_nbytes(n), &lo, &hi) || hi <= lo) continue;
+        const size_t size = hi - lo;
         const size_t off = (used + 255) & ~(size_t) 255;
         if (off + size > mirror_cap) {
             if (!mirror.empty()) continue;                 // transfers into the block are queued: it cannot move now
@@ -156,8 +158,8 @@ void mi355x_backend_ctx::mirror_outputs(struct ggml_cgraph * cgraph) {
             if (hipHostMalloc(&p, want, hipHostMallocDefault) != hipSuccess || !p) { (void) hipGetLastError(); return; }
             mirror_host = (char *) p; mirror_cap = want;
         }
-        if (hipMemcpyAsync(mirror_host + off, n->data, size, hipMemcpyDeviceToHost, stream) != hipSuccess) { (void) hipGetLastError(); continue; }
-        mirror.push_back({ (const char *) n->data, size, off });
+        if (hipMemcpyAsync(mirror_host + off, (const char *) n->data + lo, size, hipMemcpyDeviceToHost, stream) != hipSuccess) { (void) hipGetLastError(); continue; }
+        mirror.push_back({ (const char *) n->data, lo, size, off });
         used = off + size;
     }
     if (mirror.empty()) return;
@@ -169,7 +171,7 @@ void mi355x_backend_ctx::mirror_drop(const void * begin, size_t size) {
     std::lock_guard<std::mutex> lock(mirror_mutex);
     const char * b = (const char *) begin;
     for (size_t i = 0; i < mirror.size();) {
-        if (mirror[i].dev < b + size && b < mirror[i].dev + mirror[i].size) mirror.erase(mirror.begin() + (long) i); else ++i;
+        if (mirror[i].dev + mirror[i].lo < b + size && b < mirror[i].dev + mirror[i].lo + mirror[i].size) mirror.erase(mirror.begin() + (long) i); else ++i;
     }
 }
 
@@ -788,7 +790,15 @@ struct graph_runner {
 
 } // namespace
 
+static int64_t host_now_ns() {
+    return std::chrono::duration_cast<std::chrono::nanoseconds>(std::chrono::steady_clock::now().time_since_epoch()).count();
+}
+
 enum ggml_status mi355x_graph_compute(mi355x_backend_ctx * ctx, struct ggml_cgraph * cgraph) {
+    struct host_timer {                                    // host time spent planning and queueing, into counters[6]
+        mi355x_backend_ctx * c; int64_t t0;
+        ~host_timer() { c->counters[6] += host_now_ns() - t0; }
+    } timer{ ctx, host_now_ns() };
     HIP_TRY(hipSetDevice(ctx->device), return GGML_STATUS_FAILED);
     ctx->ws_x = nullptr;   // tensors may have been rewritten between graphs
     { std::lock_guard<std::mutex> lock(ctx->mirror_mutex); ctx->mirror.clear(); }      // this graph may write anywhere in the compute buffer

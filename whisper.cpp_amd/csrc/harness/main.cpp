@@ -752,9 +752,9 @@ static int cmd_bench(const args & a) {
         }
         printf("{\"bench\": \"decoder\", \"backend\": \"%s\", \"threads\": %d, \"reps\": %d, \"steps\": %d, \"batch\": %d, \"kv_stride\": %d, \"max_kv_positions\": %d, "
                "\"total_ms_median\": %.3f, \"ms_per_step\": %.5f, \"ms_per_step_min\": %.5f, \"steps_per_s\": %.2f, \"batch_tokens_per_s\": %.2f, \"launches_per_step\": %.2f, "
-               "\"downloads_from_mirror_per_step\": %.2f, \"downloads_by_copy_per_step\": %.2f, \"profiled\": %s, \"kernels\": %s, \"model\": \"%s\"}\n",
+               "\"downloads_from_mirror_per_step\": %.2f, \"downloads_by_copy_per_step\": %.2f, \"host_us_in_graph_compute_per_step\": %.2f, \"host_us_waiting_in_synchronize_per_step\": %.2f, \"profiled\": %s, \"kernels\": %s, \"model\": \"%s\"}\n",
                be.c_str(), threads, reps, n_steps, batch, kv_stride, past_of(n_steps - 1) + batch, ms, ms / n_steps, *std::min_element(per_rep.begin(), per_rep.end()) / n_steps,
-               1000.0 * n_steps / ms, 1000.0 * n_steps * batch / ms, (double) cnt[3] / n_steps, (double) cnt[4] / n_steps, (double) cnt[5] / n_steps,
+               1000.0 * n_steps / ms, 1000.0 * n_steps * batch / ms, (double) cnt[3] / n_steps, (double) cnt[4] / n_steps, (double) cnt[5] / n_steps, cnt[6] / 1e3 / n_steps, cnt[7] / 1e3 / n_steps,
                profile ? "true" : "false", kernels.c_str(), json_escape(path).c_str());
     } else {   // whisper-bench protocol, verbatim counts (examples/bench/bench.cpp:86-138)
         whisper_token tokens[512]; memset(tokens, 0, sizeof(tokens));

@@ -25,6 +25,37 @@ extern "C" const char * mi355x_status_string(int status) {
 }
 
 // ------------------------------------------------------------------------------------------------------
+// Read yardstick: what a kernel that does nothing but stream `n` bytes out of HBM takes on this device — the figure the
+// bandwidth-bound kernels (the product over the vocabulary matrix above all) are to be judged against, next to the
+// data-sheet peak.  Every lane has eight 16-byte loads in flight; the words are folded so that the loads stay.
+// ------------------------------------------------------------------------------------------------------
+
+typedef uint32_t probe_u32x4 __attribute__((ext_vector_type(4)));
+
+__global__ void __launch_bounds__(256) k_read_probe(const probe_u32x4 * __restrict__ p, int64_t n16, uint32_t * __restrict__ out) {
+    const int64_t stride = (int64_t) gridDim.x * 256;
+    int64_t i = (int64_t) blockIdx.x * 256 + threadIdx.x;
+    probe_u32x4 acc = { 0, 0, 0, 0 };
+    for (; i + 7 * stride < n16; i += 8 * stride) {
+        probe_u32x4 v[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[j] = p[i + j * stride];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) acc ^= v[j];
+    }
+    for (; i < n16; i += stride) acc ^= p[i];
+    const uint32_t f = acc.x ^ acc.y ^ acc.z ^ acc.w;
+    if (f == 0x9E3779B9u) out[0] = f;                      // (practically never: the loads are kept without a store per thread)
+}
+
+extern "C" int mi355x_read_probe(const void * src, size_t n, void * out, int workgroups, void * stream) {
+    if (!src || !out || (uintptr_t) src % 16 != 0 || (uintptr_t) out % 4 != 0 || workgroups < 1 || workgroups > 65535) return MI355X_ERR_INVALID;
+    if (n < 16) return MI355X_OK;
+    k_read_probe<<<(unsigned) workgroups, 256, 0, (hipStream_t) stream>>>((const probe_u32x4 *) src, (int64_t)(n / 16), (uint32_t *) out);
+    return launch_status();
+}
+
+// ------------------------------------------------------------------------------------------------------
 // GELU table
 // ------------------------------------------------------------------------------------------------------
 

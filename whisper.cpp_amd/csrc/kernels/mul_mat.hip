@@ -16,6 +16,7 @@
 //   * k_mul_mat_generic — any strides / K; one wavefront per output row, f32 FMA.
 #include "common.h"
 
+#include <algorithm>
 #include <mutex>
 #include <stdlib.h>
 #include <type_traits>
@@ -257,7 +258,7 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 // KTAIL: K is not a multiple of 64 (but of 8); FULL: K / 64 is a multiple of S; EMIT: MI355X_EPI_EMIT_F16 (a kernel of its
 // own, because its epilogue needs more registers than two workgroups per CU leave)
 template <int TI, int TJ, int S, bool KTAIL, bool FULL, bool EMIT = false>
-__device__ __forceinline__ void gemm_f16_tile(const mm_args & a, int tiles_m, int tiles_n, const char * wb, const char * xb, char * db,
+__device__ __forceinline__ void gemm_f16_tile(const mm_args & a, int tiles_m, int tiles_n, int sw, int tile, const char * wb, const char * xb, char * db,
                                               const epi_args & epi, int64_t batch_off, int64_t d_nb1) {
     constexpr int BN = 64 * TI, BM = 64 * TJ;
     constexpr int XR = BN / 32, WR = BM / 32;          // 16-byte pieces per thread and step
@@ -265,13 +266,13 @@ __device__ __forceinline__ void gemm_f16_tile(const mm_args & a, int tiles_m, in
     half_t * xs_base = (half_t *) smem;                // [2][BN * GB_LD]
     half_t * ws_base = xs_base + 2 * BN * GB_LD;       // [2][BM * GB_LD]
 
-    // Workgroups are dealt round-robin to the 8 XCDs, each with its own L2.  Give every XCD one contiguous run of
-    // tiles (m fastest), so that the X rows and the W rows it touches are shared inside that L2.
-    const int nblk = tiles_m * tiles_n;
-    const int xcd = blockIdx.x % 8, q = nblk / 8, r = nblk % 8;
-    const int tile = xcd * q + (xcd < r ? xcd : r) + blockIdx.x / 8;
-    const int64_t m0 = (int64_t)(tile % tiles_m) * BM;
-    const int64_t n0 = (int64_t)(tile / tiles_m) * BN;
+    // `tile` counts along a path over the tile grid that walks columns of `sw` m-tiles, each from the first n-panel to the
+    // last (m fastest inside the column): a run of consecutive tiles — what one XCD gets, see xcd_run_index — then covers
+    // about sqrt(run) tiles in each direction, the shape that touches the fewest X and W rows.
+    const int per_col = sw * tiles_n, col = tile / per_col, rem = tile - col * per_col;
+    const int cw = min(sw, tiles_m - col * sw);        // (the last column is narrower when sw does not divide tiles_m)
+    const int64_t m0 = (int64_t)(col * sw + rem % cw) * BM;
+    const int64_t n0 = (int64_t)(rem / cw) * BN;
 
     const int tid = threadIdx.x;
     const int lc = tid & 7, lr = tid >> 3;             // piece column (8 halves) and first row of this thread
@@ -418,10 +419,31 @@ __device__ __forceinline__ void gemm_f16_tile(const mm_args & a, int tiles_m, in
     }
 }
 
+// Workgroups are dealt round-robin to the 8 XCDs, each with its own L2: workgroup `lin` of `total` runs on XCD lin % 8.
+// Give every XCD one run of consecutive work items, so that what its workgroups read is shared inside that L2: the index
+// of this workgroup's item when XCD x takes items [x q + min(x, r), ...) with q = total / 8, r = total % 8.
+__device__ __forceinline__ int xcd_run_index(int lin, int total) {
+    const int xcd = lin % 8, q = total / 8, r = total % 8;
+    return xcd * q + (xcd < r ? xcd : r) + lin / 8;
+}
+
+// width (in m-tiles) of the columns of the tile path: a run of `run` tiles should be as square as the tiles allow
+static int tile_path_width(int64_t tiles_m, int64_t tiles_n, int64_t run, int bn, int bm) {
+    if (run >= tiles_m * tiles_n || tiles_n == 1) return (int) tiles_m;
+    int best = (int) tiles_m; int64_t best_cost = INT64_MAX;
+    for (int64_t sw = 1; sw <= tiles_m; ++sw) {
+        // rows of X and of W that a run touches (one more panel for a run that starts mid-way), more when the columns are uneven
+        const int64_t cost = (std::min(tiles_n, (run + sw - 1) / sw + 1)) * bn + sw * bm + (tiles_m % sw ? bm : 0);
+        if (cost < best_cost) { best_cost = cost; best = (int) sw; }
+    }
+    return best;
+}
+
 template <int TI, int TJ, int S, bool KTAIL, bool FULL, bool EMIT>
-__global__ void __launch_bounds__(256, 2) k_gemm_f16(mm_args a, int tiles_m, int tiles_n) {
+__global__ void __launch_bounds__(256, 2) k_gemm_f16(mm_args a, int tiles_m, int tiles_n, int sw) {
     const int64_t b2 = blockIdx.y % a.ne12, b3 = blockIdx.y / a.ne12;
-    gemm_f16_tile<TI, TJ, S, KTAIL, FULL, EMIT>(a, tiles_m, tiles_n, a.w + (b2 / a.r2) * a.w_nb2 + (b3 / a.r3) * a.w_nb3, a.x + b2 * a.x_nb2 + b3 * a.x_nb3,
+    gemm_f16_tile<TI, TJ, S, KTAIL, FULL, EMIT>(a, tiles_m, tiles_n, sw, xcd_run_index(blockIdx.x, tiles_m * tiles_n),
+                                          a.w + (b2 / a.r2) * a.w_nb2 + (b3 / a.r3) * a.w_nb3, a.x + b2 * a.x_nb2 + b3 * a.x_nb3,
                                           a.d + b2 * a.d_nb2 + b3 * a.d_nb3, a.e, b2 * a.d_nb2 + b3 * a.d_nb3, a.d_nb1);
 }
 
@@ -433,11 +455,14 @@ struct mm_group_entry { const char * w; char * d; const float * bias; const char
 struct mm_group { mm_group_entry e[MM_GROUP_MAX]; };
 
 template <int TI, int TJ, int S>
-__global__ void __launch_bounds__(256) k_gemm_f16_group(mm_args a, int tiles_m, int tiles_n, mm_group grp) {
-    const mm_group_entry & ge = grp.e[blockIdx.y];
+__global__ void __launch_bounds__(256) k_gemm_f16_group(mm_args a, int tiles_m, int tiles_n, int sw, mm_group grp) {
+    // the products' tiles form one pool, product after product, and an XCD's run may cross from one product into the next
+    const int nblk = tiles_m * tiles_n;
+    const int item = xcd_run_index((int)(blockIdx.x + gridDim.x * blockIdx.y), nblk * (int) gridDim.y);
+    const mm_group_entry & ge = grp.e[item / nblk];
     epi_args e;
     e.flags = ge.flags; e.scale = ge.scale; e.bias = ge.bias; e.residual = ge.residual; e.gelu = a.e.gelu; e.image = nullptr;
-    gemm_f16_tile<TI, TJ, S, false, true>(a, tiles_m, tiles_n, ge.w, a.x, ge.d, e, 0, ge.d_nb1);
+    gemm_f16_tile<TI, TJ, S, false, true>(a, tiles_m, tiles_n, sw, item % nblk, ge.w, a.x, ge.d, e, 0, ge.d_nb1);
 }
 
 template <int TI, int TJ, int S, bool KTAIL, bool FULL, bool EMIT = false>
@@ -455,7 +480,8 @@ static int launch_gemm_f16_k(const mm_args & a, hipStream_t st) {
     const int64_t tm = (a.M + BM - 1) / BM, tn = (a.N + BN - 1) / BN;
     if (tm * tn > 0x7fffffff) return MI355X_ERR_UNSUPPORTED;
     dim3 grid((unsigned)(tm * tn), (unsigned)(a.ne12 * a.ne13));
-    k_gemm_f16<TI, TJ, S, KTAIL, FULL, EMIT><<<grid, 256, lds, st>>>(a, (int) tm, (int) tn);
+    const int sw = tile_path_width(tm, tn, (tm * tn + 7) / 8, BN, BM);
+    k_gemm_f16<TI, TJ, S, KTAIL, FULL, EMIT><<<grid, 256, lds, st>>>(a, (int) tm, (int) tn, sw);
     return launch_status();
 }
 template <int TI, int TJ>
@@ -485,7 +511,8 @@ static int launch_gemm_f16_group(const mm_args & a, const mm_group & grp, int co
     const int64_t tm = (a.M + BM - 1) / BM, tn = (a.N + BN - 1) / BN;
     if (tm * tn > 0x7fffffff) return MI355X_ERR_UNSUPPORTED;
     dim3 grid((unsigned)(tm * tn), (unsigned) count);
-    k_gemm_f16_group<TI, TJ, 4><<<grid, 256, lds, st>>>(a, (int) tm, (int) tn, grp);
+    const int sw = tile_path_width(tm, tn, (tm * tn * count + 7) / 8, BN, BM);
+    k_gemm_f16_group<TI, TJ, 4><<<grid, 256, lds, st>>>(a, (int) tm, (int) tn, sw, grp);
     return launch_status();
 }
 
