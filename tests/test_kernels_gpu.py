@@ -241,6 +241,29 @@ def test_mul_mat_epilogues(pkg, oracle, gpu):
         assert oracle.nmse(got, base + colbias[:, None]) <= 1e-6
 
 
+def test_mul_mat_gelu_epilogue_from_the_lds_table_slice(pkg, oracle, gpu):
+    # On 128 x 128 tiles (the FFN-up shape) the GELU epilogue looks its values up in the part of the f16 table kept in LDS
+    # (|x| < 8) and goes to the table in global memory for anything larger: both routes, against the standalone GELU kernel
+    # on the product without the epilogue — the same table, so the same bits.
+    lib = pkg.kernels()
+    k, m, n = 256, 2560, 1500
+    blocks = oracle.quantize(pkg.Q8_0, rnd((m, k), 0.02))
+    x = rnd((n, k))
+    bias = rnd((m,), 2.0)
+    bias[::97] = 40.0 * np.sign(bias[::97])                 # a few columns far outside the slice (|x| >= 8, and beyond the clamps at 10)
+    bias[5::89] = 8.5
+    plain, name = run_mul_mat(pkg, gpu, pkg.Q8_0, blocks, x, k, m, flags=pkg.EPI_BIAS, bias=bias)
+    got, _ = run_mul_mat(pkg, gpu, pkg.Q8_0, blocks, x, k, m, flags=pkg.EPI_BIAS | pkg.EPI_GELU, bias=bias)
+    assert "gemm" in name
+    d_p = gpu.up(plain)
+    d_g = torch.empty_like(d_p)
+    pkg.check(lib.mi355x_gelu(pkg.tensor(d_p, pkg.F32), pkg.tensor(d_g, pkg.F32), gpu.stream))
+    want = gpu.down(d_g)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    assert (np.abs(plain) >= 8).sum() > 1000 and (np.abs(plain) < 8).sum() > 1000
+    assert oracle.nmse(got[:64], oracle.gelu(plain[:64])) <= 1e-7
+
+
 def test_mul_mat_epilogue_emits_the_next_products_activation_image(pkg, oracle, gpu):
     # MI355X_EPI_EMIT_F16: besides dst (here with bias and GELU, the FFN's first matrix), its rows rounded to Q8_0 as f16(q * d)
     lib = pkg.kernels()

@@ -49,9 +49,14 @@ __device__ __forceinline__ float apply_epilogue(float v, const epi_args & e, int
 // The same for the 16 registers of one 32x32 accumulator patch (column m, rows n[0..15]) and the stores.  All loads of
 // one kind are issued together before their first use; rows beyond N and columns beyond M are computed from clamped
 // addresses and not stored.
+// The part of the GELU table that the values in front of a GELU fall into, as a workgroup keeps it in LDS: the f16 patterns
+// of |x| < 8 — 0x0000 .. 0x47ff and 0x8000 .. 0xc7ff, 2 x 18432 entries, 73728 bytes — positive half first.
+#define GELU_LDS_HALF  0x4800
+#define GELU_LDS_BYTES (2 * GELU_LDS_HALF * 2)
+
 template <bool EMIT>
 __device__ __forceinline__ void patch_epilogue(float16_t v, const epi_args & e, char * db, int64_t batch_off, int64_t d_nb1,
-                                               int64_t m, int64_t M, const int64_t (&n)[16], int64_t N) {
+                                               int64_t m, int64_t M, const int64_t (&n)[16], int64_t N, const uint16_t * gelu_lds = nullptr) {
     const bool    m_ok = m < M;
     const int64_t mc   = m_ok ? m : M - 1;
     int64_t nc[16];
@@ -71,8 +76,26 @@ __device__ __forceinline__ void patch_epilogue(float16_t v, const epi_args & e, 
     }
     if (e.flags & MI355X_EPI_GELU) {
         uint16_t t[16];
+        if (gelu_lds) {
+            // 64 gathers per lane out of the 128 KB table in global memory cost the FFN-up product 10 us of its 45; out of
+            // LDS, 8.  A value of 8 or more in magnitude (none in a whisper model's activations) sends the wavefront to the
+            // table in global memory for that register.
+            uint32_t hb[16]; bool far = false;
 #pragma unroll
-        for (int i = 0; i < 16; ++i) t[i] = e.gelu[f2h_bits(v[i])];
+            for (int i = 0; i < 16; ++i) { hb[i] = f2h_bits(v[i]); far = far || (hb[i] & 0x7FFFu) >= GELU_LDS_HALF; }
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const uint32_t a = hb[i] & 0x7FFFu;
+                t[i] = gelu_lds[(a < GELU_LDS_HALF ? a : 0u) + (hb[i] >> 15) * GELU_LDS_HALF];
+            }
+            if (__any(far)) {
+#pragma unroll
+                for (int i = 0; i < 16; ++i) if ((hb[i] & 0x7FFFu) >= GELU_LDS_HALF) t[i] = e.gelu[hb[i]];
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) t[i] = e.gelu[f2h_bits(v[i])];
+        }
 #pragma unroll
         for (int i = 0; i < 16; ++i) v[i] = v[i] <= -10.0f ? 0.0f : v[i] >= 10.0f ? v[i] : h2f(t[i]);
     }
@@ -407,6 +430,20 @@ __device__ __forceinline__ void gemm_f16_tile(const mm_args & a, int tiles_m, in
         }
     }
 
+    // GELU reads its table from LDS when the operand buffers, free now (the loop's last barrier is behind every wavefront),
+    // are large enough to hold the part that matters
+    const uint16_t * gelu_lds = nullptr;
+    if constexpr ((size_t) 2 * (BN + BM) * GB_LD * sizeof(half_t) >= GELU_LDS_BYTES) {
+        if (epi.flags & MI355X_EPI_GELU) {
+            const u32x4 * pos = (const u32x4 *) epi.gelu, * neg = (const u32x4 *)(epi.gelu + 0x8000);
+            u32x4 * dst = (u32x4 *) smem;
+            constexpr int pieces = GELU_LDS_HALF * 2 / 16;
+            for (int p = tid; p < pieces; p += 256) { dst[p] = pos[p]; dst[pieces + p] = neg[p]; }
+            __syncthreads();
+            gelu_lds = (const uint16_t *) smem;
+        }
+    }
+
     // accumulator register e of a 32x32 patch: row (= n) 8*(e/4) + 4*g + e%4, column (= m) lane%32
 #pragma unroll
     for (int i = 0; i < TI; ++i) {
@@ -415,7 +452,7 @@ __device__ __forceinline__ void gemm_f16_tile(const mm_args & a, int tiles_m, in
         for (int e = 0; e < 16; ++e) n[e] = n0 + wn + 32 * i + 8 * (e >> 2) + 4 * g + (e & 3);
 #pragma unroll
         for (int j = 0; j < TJ; ++j)
-            patch_epilogue<EMIT>(acc[i][j], epi, db, batch_off, d_nb1, m0 + wmo + 32 * j + l32, a.M, n, a.N);
+            patch_epilogue<EMIT>(acc[i][j], epi, db, batch_off, d_nb1, m0 + wmo + 32 * j + l32, a.M, n, a.N, gelu_lds);
     }
 }
 
