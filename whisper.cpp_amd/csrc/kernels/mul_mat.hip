@@ -121,11 +121,23 @@ __device__ __forceinline__ void patch_epilogue(float16_t v, const epi_args & e, 
         // The product that reads dst next rounds its rows to Q8_0 first.  The 32 lanes of a half-wavefront hold 32
         // consecutive m of one dst row — exactly one Q8_0 block (M % 32 == 0) — so the block maximum is a 5-step
         // butterfly, and the image f16(q * d) is written here instead of by a pass of its own over dst.
+        // The two divisions of a block (127 / amax and amax / 127) would be repeated by all 32 lanes that hold it, for each
+        // of the 16 registers: 32 IEEE divisions per lane and patch, most of this epilogue's time.  Instead lane l divides
+        // for register l % 16 of its half-wavefront, and the 16 results travel back by lane permutes.
+        float amax[16];
+#pragma unroll
+        for (int i = 0; i < 16; ++i) amax[i] = lanes_max<32>(fabsf(v[i]));
+        const int lane = threadIdx.x & 63;
+        float mine = amax[0];
+#pragma unroll
+        for (int i = 1; i < 16; ++i) mine = (lane & 15) == i ? amax[i] : mine;
+        const float id_m = mine != 0.0f ? 127.0f / mine : 0.0f;
+        const float dq_m = h2f(f2h_bits(mine / 127.0f));
+        const int src = ((lane & 32) << 2);                 // byte address of lane 0 of this half-wavefront for ds_bpermute
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
-            const float amax = lanes_max<32>(fabsf(v[i]));
-            const float id = amax != 0.0f ? 127.0f / amax : 0.0f;
-            const float dq = h2f(f2h_bits(amax / 127.0f));
+            const float id = __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(src + 4 * i, __builtin_bit_cast(int, id_m)));
+            const float dq = __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(src + 4 * i, __builtin_bit_cast(int, dq_m)));
             if (m_ok && n[i] < N) e.image[n[i] * M + m] = (half_t)((rintf(v[i] * id) + 0.0f) * dq);
         }
     }
