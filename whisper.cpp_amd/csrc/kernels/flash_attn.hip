@@ -130,6 +130,78 @@ __device__ __forceinline__ half2_t seq_mad2(half2_t acc, half2_t v, float vs) {
     asm("v_cvt_pk_f16_f32 %0, %1, %2" : "=v"(r) : "v"(lo), "v"(hi));
     return r;
 }
+// One key for the 16 accumulators of a lane (eight pairs): the 16 fma first, then the 8 packs — in that order no
+// instruction reads what the one or two before it wrote.  Written pair by pair (fma, fma, pack) every pack waited for the
+// fma in front of it, and the compiler, which does not move instructions out of asm statements, also had to put a wait state
+// between them: the chains ran at three quarters of the vector issue rate.
+// va / vb: the key's V values d0 .. d0 + 7 and d0 + 8 .. d0 + 15 (two f16 per register).
+__device__ __forceinline__ void seq_mad16(half2_t (&acc)[8], const u32x4 va, const u32x4 vb, float vs) {
+    float t0, t1, t2, t3, t4, t5, t6, t7, t8, t9, t10, t11, t12, t13, t14, t15;
+    asm("v_fma_mix_f32 %0, %8, %12, %13 op_sel_hi:[1,0,1]\n\t"
+        "v_fma_mix_f32 %1, %8, %12, %13 op_sel:[1,0,1] op_sel_hi:[1,0,1]\n\t"
+        "v_fma_mix_f32 %2, %9, %12, %14 op_sel_hi:[1,0,1]\n\t"
+        "v_fma_mix_f32 %3, %9, %12, %14 op_sel:[1,0,1] op_sel_hi:[1,0,1]\n\t"
+        "v_fma_mix_f32 %4, %10, %12, %15 op_sel_hi:[1,0,1]\n\t"
+        "v_fma_mix_f32 %5, %10, %12, %15 op_sel:[1,0,1] op_sel_hi:[1,0,1]\n\t"
+        "v_fma_mix_f32 %6, %11, %12, %16 op_sel_hi:[1,0,1]\n\t"
+        "v_fma_mix_f32 %7, %11, %12, %16 op_sel:[1,0,1] op_sel_hi:[1,0,1]"
+        : "=&v"(t0), "=&v"(t1), "=&v"(t2), "=&v"(t3), "=&v"(t4), "=&v"(t5), "=&v"(t6), "=&v"(t7)
+        : "v"(va.x), "v"(va.y), "v"(va.z), "v"(va.w), "v"(vs), "v"(acc[0]), "v"(acc[1]), "v"(acc[2]), "v"(acc[3]));
+    asm("v_fma_mix_f32 %0, %8, %12, %13 op_sel_hi:[1,0,1]\n\t"
+        "v_fma_mix_f32 %1, %8, %12, %13 op_sel:[1,0,1] op_sel_hi:[1,0,1]\n\t"
+        "v_fma_mix_f32 %2, %9, %12, %14 op_sel_hi:[1,0,1]\n\t"
+        "v_fma_mix_f32 %3, %9, %12, %14 op_sel:[1,0,1] op_sel_hi:[1,0,1]\n\t"
+        "v_fma_mix_f32 %4, %10, %12, %15 op_sel_hi:[1,0,1]\n\t"
+        "v_fma_mix_f32 %5, %10, %12, %15 op_sel:[1,0,1] op_sel_hi:[1,0,1]\n\t"
+        "v_fma_mix_f32 %6, %11, %12, %16 op_sel_hi:[1,0,1]\n\t"
+        "v_fma_mix_f32 %7, %11, %12, %16 op_sel:[1,0,1] op_sel_hi:[1,0,1]"
+        : "=&v"(t8), "=&v"(t9), "=&v"(t10), "=&v"(t11), "=&v"(t12), "=&v"(t13), "=&v"(t14), "=&v"(t15)
+        : "v"(vb.x), "v"(vb.y), "v"(vb.z), "v"(vb.w), "v"(vs), "v"(acc[4]), "v"(acc[5]), "v"(acc[6]), "v"(acc[7]));
+    asm("v_cvt_pk_f16_f32 %0, %8, %9\n\t"
+        "v_cvt_pk_f16_f32 %1, %10, %11\n\t"
+        "v_cvt_pk_f16_f32 %2, %12, %13\n\t"
+        "v_cvt_pk_f16_f32 %3, %14, %15\n\t"
+        "v_cvt_pk_f16_f32 %4, %16, %17\n\t"
+        "v_cvt_pk_f16_f32 %5, %18, %19\n\t"
+        "v_cvt_pk_f16_f32 %6, %20, %21\n\t"
+        "v_cvt_pk_f16_f32 %7, %22, %23"
+        : "=&v"(acc[0]), "=&v"(acc[1]), "=&v"(acc[2]), "=&v"(acc[3]), "=&v"(acc[4]), "=&v"(acc[5]), "=&v"(acc[6]), "=&v"(acc[7])
+        : "v"(t0), "v"(t1), "v"(t2), "v"(t3), "v"(t4), "v"(t5), "v"(t6), "v"(t7), "v"(t8), "v"(t9), "v"(t10), "v"(t11), "v"(t12), "v"(t13), "v"(t14), "v"(t15));
+}
+// the rescale of the 16 accumulators by ms (f32 product, rounded to f16), instructions ordered like seq_mad16
+__device__ __forceinline__ void seq_scale16(half2_t (&acc)[8], float ms) {
+    float t0, t1, t2, t3, t4, t5, t6, t7, t8, t9, t10, t11, t12, t13, t14, t15;
+    asm("v_fma_mix_f32 %0, %8, %12, 0 op_sel_hi:[1,0,0]\n\t"
+        "v_fma_mix_f32 %1, %8, %12, 0 op_sel:[1,0,0] op_sel_hi:[1,0,0]\n\t"
+        "v_fma_mix_f32 %2, %9, %12, 0 op_sel_hi:[1,0,0]\n\t"
+        "v_fma_mix_f32 %3, %9, %12, 0 op_sel:[1,0,0] op_sel_hi:[1,0,0]\n\t"
+        "v_fma_mix_f32 %4, %10, %12, 0 op_sel_hi:[1,0,0]\n\t"
+        "v_fma_mix_f32 %5, %10, %12, 0 op_sel:[1,0,0] op_sel_hi:[1,0,0]\n\t"
+        "v_fma_mix_f32 %6, %11, %12, 0 op_sel_hi:[1,0,0]\n\t"
+        "v_fma_mix_f32 %7, %11, %12, 0 op_sel:[1,0,0] op_sel_hi:[1,0,0]"
+        : "=&v"(t0), "=&v"(t1), "=&v"(t2), "=&v"(t3), "=&v"(t4), "=&v"(t5), "=&v"(t6), "=&v"(t7)
+        : "v"(acc[0]), "v"(acc[1]), "v"(acc[2]), "v"(acc[3]), "v"(ms));
+    asm("v_fma_mix_f32 %0, %8, %12, 0 op_sel_hi:[1,0,0]\n\t"
+        "v_fma_mix_f32 %1, %8, %12, 0 op_sel:[1,0,0] op_sel_hi:[1,0,0]\n\t"
+        "v_fma_mix_f32 %2, %9, %12, 0 op_sel_hi:[1,0,0]\n\t"
+        "v_fma_mix_f32 %3, %9, %12, 0 op_sel:[1,0,0] op_sel_hi:[1,0,0]\n\t"
+        "v_fma_mix_f32 %4, %10, %12, 0 op_sel_hi:[1,0,0]\n\t"
+        "v_fma_mix_f32 %5, %10, %12, 0 op_sel:[1,0,0] op_sel_hi:[1,0,0]\n\t"
+        "v_fma_mix_f32 %6, %11, %12, 0 op_sel_hi:[1,0,0]\n\t"
+        "v_fma_mix_f32 %7, %11, %12, 0 op_sel:[1,0,0] op_sel_hi:[1,0,0]"
+        : "=&v"(t8), "=&v"(t9), "=&v"(t10), "=&v"(t11), "=&v"(t12), "=&v"(t13), "=&v"(t14), "=&v"(t15)
+        : "v"(acc[4]), "v"(acc[5]), "v"(acc[6]), "v"(acc[7]), "v"(ms));
+    asm("v_cvt_pk_f16_f32 %0, %8, %9\n\t"
+        "v_cvt_pk_f16_f32 %1, %10, %11\n\t"
+        "v_cvt_pk_f16_f32 %2, %12, %13\n\t"
+        "v_cvt_pk_f16_f32 %3, %14, %15\n\t"
+        "v_cvt_pk_f16_f32 %4, %16, %17\n\t"
+        "v_cvt_pk_f16_f32 %5, %18, %19\n\t"
+        "v_cvt_pk_f16_f32 %6, %20, %21\n\t"
+        "v_cvt_pk_f16_f32 %7, %22, %23"
+        : "=&v"(acc[0]), "=&v"(acc[1]), "=&v"(acc[2]), "=&v"(acc[3]), "=&v"(acc[4]), "=&v"(acc[5]), "=&v"(acc[6]), "=&v"(acc[7])
+        : "v"(t0), "v"(t1), "v"(t2), "v"(t3), "v"(t4), "v"(t5), "v"(t6), "v"(t7), "v"(t8), "v"(t9), "v"(t10), "v"(t11), "v"(t12), "v"(t13), "v"(t14), "v"(t15));
+}
 __device__ __forceinline__ half2_t seq_scale2(half2_t acc, float ms) {
     float lo, hi;
     half2_t r;
@@ -486,185 +558,198 @@ __device__ __forceinline__ float exp_neg(float x) {
 
 typedef const uint32_t __attribute__((address_space(4))) * const_u32_ptr;   // read-only data: uniform loads become scalar loads
 
-__global__ void __launch_bounds__(256) k_fattn_seq_tile(fa_args a) {
-    __shared__ __attribute__((aligned(16))) half_t q_s[T_Q * T_LDH];
-    __shared__ __attribute__((aligned(16))) half_t k_s[T_KV * T_LDH];
-    __shared__ __attribute__((aligned(16))) half_t v_s[T_KV * FA_D];
-    __shared__ __attribute__((aligned(16))) float  f_s[T_Q * T_LDF];
-    __shared__ float m_run[T_Q], s_run[T_Q];
+// Eight wavefronts in two roles, a tile of 64 keys between them:
+//   wavefronts 4 .. 7 (producers) prepare tile t + 1: K / V rows -> LDS, S = Q K^T on the matrix cores, the factors;
+//   wavefronts 0 .. 3 (chains) walk tile t: 16 queries x all 64 d each (lane = query 16 w + l % 16, d slice l / 16).
+// The factor tile and the V tile are double buffered, so the two roles meet at two barriers per tile — the tile boundary
+// and the point inside a tile where the producers' factor step needs all of their score writes — and otherwise run side
+// by side: a SIMD holds one chain and one producer wavefront of each workgroup,
+// and the chains' vector work, which is what bounds the kernel, no longer waits for the score and factor steps.
+#define T_LDS_BYTES ((T_Q * T_LDH + T_KV * T_LDH + 2 * T_KV * FA_D) * 2 + (2 * T_Q * T_LDF + 2 * T_Q) * 4)     // 70144: beyond the 64 KB a launch gets unasked
 
-    const int tid = threadIdx.x, lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+__global__ void __launch_bounds__(512, 2) k_fattn_seq_tile(fa_args a) {
+    extern __shared__ __attribute__((aligned(16))) char t_smem[];
+    half_t * q_s = (half_t *) t_smem;                      // [T_Q * T_LDH]
+    half_t * k_s = q_s + T_Q * T_LDH;                      // [T_KV * T_LDH]
+    half_t * v_s2 = k_s + T_KV * T_LDH;                    // [2][T_KV * FA_D]
+    float *  f_s2 = (float *)(v_s2 + 2 * T_KV * FA_D);     // [2][T_Q * T_LDF]
+    float *  m_run = f_s2 + 2 * T_Q * T_LDF, * s_run = m_run + T_Q;
+
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int64_t n0 = (int64_t) blockIdx.x * T_Q, h = blockIdx.y, i3 = blockIdx.z;
-    const char * qb = a.q + h * a.q_nb2 + i3 * a.q_nb3;
-    const char * kb = a.k + (h / a.hk_ratio) * a.k_nb2 + (i3 / a.k_ne3_ratio) * a.k_nb3;
-    const char * vb = a.v + (h / a.hv_ratio) * a.v_nb2 + (i3 / a.v_ne3_ratio) * a.v_nb3;
+    const int n_tiles = (int)((a.KV + T_KV - 1) / T_KV);
 
-    // Q tile -> f16 in LDS; thread t: row t/4, 16 values
-    {
-        const int r = tid >> 2, c = (tid & 3) * 16;
-        const int64_t n = n0 + r;
+    if (wave >= 4) {
+        // ---- producers ---------------------------------------------------------------------------------------------------------------
+        const int tid = threadIdx.x - 256, pw = wave - 4;
+        const char * qb = a.q + h * a.q_nb2 + i3 * a.q_nb3;
+        const char * kb = a.k + (h / a.hk_ratio) * a.k_nb2 + (i3 / a.k_ne3_ratio) * a.k_nb3;
+        const char * vb = a.v + (h / a.hv_ratio) * a.v_nb2 + (i3 / a.v_ne3_ratio) * a.v_nb3;
+
+        // Q tile -> f16 in LDS; thread t: row t/4, 16 values
+        {
+            const int r = tid >> 2, c = (tid & 3) * 16;
+            const int64_t n = n0 + r;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            float4 t = make_float4(0.f, 0.f, 0.f, 0.f);
-            if (n < a.N) t = *(const float4 *)(qb + n * a.q_nb1 + (c + 4 * i) * 4);
-            half4_t hq = { (half_t) t.x, (half_t) t.y, (half_t) t.z, (half_t) t.w };
-            *(half4_t *)(q_s + r * T_LDH + c + 4 * i) = hq;
+            for (int i = 0; i < 4; ++i) {
+                float4 t = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (n < a.N) t = *(const float4 *)(qb + n * a.q_nb1 + (c + 4 * i) * 4);
+                half4_t hq = { (half_t) t.x, (half_t) t.y, (half_t) t.z, (half_t) t.w };
+                *(half4_t *)(q_s + r * T_LDH + c + 4 * i) = hq;
+            }
         }
-    }
-    if (tid < T_Q) { m_run[tid] = -INFINITY; s_run[tid] = 0.0f; }
+        if (tid < T_Q) { m_run[tid] = -INFINITY; s_run[tid] = 0.0f; }
 
-    // chain role: a lane owns 16 of the 64 d of one query.  A wavefront takes 16 queries x all four d slices (lane = query
-    // 16 w + l % 16, slice l / 16): a key that raises the running maximum of any query of the wavefront costs the whole
-    // wavefront a rescale of its accumulators, and with 16 queries instead of 64 that happens for 6 % of the keys instead
-    // of 18 % (records of an i.i.d. sequence: about min(1, queries / k) at key k).
+        // score role: wavefront w computes the 32x32 patch (queries 32*(w/2).., keys 32*(w%2)..)
+        const int sq = (pw >> 1) * 32, sk = (pw & 1) * 32, l32 = lane & 31, g = lane >> 5;
+        // K / V tile staging: thread t: row t/4, 32 bytes of each; the tile after the next is in flight while one is worked on
+        const int kr = tid >> 2, kc = (tid & 3) * 16;
+        u32x4 kreg0, kreg1, vreg0, vreg1;
+        auto load_kv = [&](int64_t key0) __attribute__((always_inline)) {
+            const int64_t key = key0 + kr < a.KV ? key0 + kr : a.KV - 1;      // rows past the end repeat the last key; their scores are masked
+            const u32x4 * kp = (const u32x4 *)(kb + key * a.k_nb1 + kc * 2);
+            const u32x4 * vp = (const u32x4 *)(vb + key * a.v_nb1 + kc * 2);
+            kreg0 = kp[0]; kreg1 = kp[1]; vreg0 = vp[0]; vreg1 = vp[1];
+        };
+        load_kv(0);
+        *(u32x4 *)(k_s + kr * T_LDH + kc) = kreg0; *(u32x4 *)(k_s + kr * T_LDH + kc + 8) = kreg1;
+
+        for (int it = 0; it <= n_tiles; ++it) {
+            // tile boundary: buffer it & 1 is free (its chains ended with the previous iteration); the K tile staged at the end
+            // of that iteration (and, first time, the Q tile) is visible
+            __syncthreads();
+            if (it == n_tiles) { __syncthreads(); break; }
+            const int64_t key0 = (int64_t) it * T_KV;
+            half_t * vs_buf = v_s2 + (it & 1) * T_KV * FA_D;
+            float *  fs_buf = f_s2 + (it & 1) * T_Q * T_LDF;
+            *(u32x4 *)(vs_buf + kr * FA_D + kc) = vreg0; *(u32x4 *)(vs_buf + kr * FA_D + kc + 8) = vreg1;
+            if (it + 1 < n_tiles) load_kv(key0 + T_KV);    // a whole iteration ahead of its use
+
+            // ---- scores: S = Q K^T on the matrix cores
+            {
+                float16_t c16;
+#pragma unroll
+                for (int r = 0; r < 16; ++r) c16[r] = 0.0f;
+#pragma unroll
+                for (int kk = 0; kk < FA_D / 16; ++kk) {
+                    const half8_t av = *(const half8_t *)(q_s + (sq + l32) * T_LDH + kk * 16 + 8 * g);
+                    const half8_t bv = *(const half8_t *)(k_s + (sk + l32) * T_LDH + kk * 16 + 8 * g);
+                    c16 = __builtin_amdgcn_mfma_f32_32x32x16_f16(av, bv, c16, 0, 0, 0);
+                }
+                const int64_t key = key0 + sk + l32;                  // accumulator column = key, rows = queries
+                const bool key_ok = key < a.KV;
+                float mv[16];
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int qi = sq + 8 * (r >> 2) + 4 * g + (r & 3);
+                    mv[r] = 0.0f;
+                    if (a.mask) {
+                        const int64_t n = n0 + qi < a.N ? n0 + qi : a.N - 1;
+                        mv[r] = (float) *(const half_t *)(a.mask + n * a.m_nb1 + (key_ok ? key : a.KV - 1) * 2);
+                    }
+                }
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int qi = sq + 8 * (r >> 2) + 4 * g + (r & 3);
+                    fs_buf[qi * T_LDF + sk + l32] = key_ok ? __fadd_rn(__fmul_rn(c16[r], a.scale), mv[r]) : -INFINITY;
+                }
+            }
+            __syncthreads();                               // scores visible
+
+            // ---- factors: thread t: query t/4, keys 16*(t%4) .. +15
+            {
+                const int qi = tid >> 2, sgm = tid & 3;
+                float4 * fp = (float4 *)(fs_buf + qi * T_LDF + sgm * 16);
+                float sv[16], lmax = -INFINITY;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) { const float4 t = fp[i]; sv[4*i] = t.x; sv[4*i+1] = t.y; sv[4*i+2] = t.z; sv[4*i+3] = t.w; }
+#pragma unroll
+                for (int i = 0; i < 16; ++i) lmax = fmaxf(lmax, sv[i]);
+                float M = m_run[qi];
+                const float S0 = s_run[qi];
+                // (the four runs of a query sit in one quad of lanes: broadcasts inside it are DPP moves, not LDS permutes)
+                const float m0 = dpp_move<float, 0x00>(lmax), m1 = dpp_move<float, 0x55>(lmax), m2 = dpp_move<float, 0xAA>(lmax);
+                if (sgm > 0) M = fmaxf(M, m0);
+                if (sgm > 1) M = fmaxf(M, m1);
+                if (sgm > 2) M = fmaxf(M, m2);
+                // this run's effect on the softmax denominator: S_after = S_before * P + A
+                float P = 1.0f, A = 0.0f;
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    // one exp serves both cases: a new maximum (ms = exp(M - s), 0 for the first key; vs = 1) and a standing
+                    // one (vs = exp(s - M); masked keys, s = -inf, get vs = 0, a no-op on the accumulator)
+                    const float s = sv[i];
+                    const bool  raised = s > M;
+                    const float ex = exp_neg(-fabsf(s - M));   // M - s when raised, s - M otherwise: both <= 0 (or NaN / -inf: 0)
+                    const float ms = raised ? ex : 1.0f, vs = raised ? 1.0f : ex;
+                    M = raised ? s : M;
+                    P *= ms; A = A * ms + vs;
+                    sv[i] = raised ? -ex : ex;                 // -0.0 keeps the sign
+                }
+#pragma unroll
+                for (int i = 0; i < 4; ++i) fp[i] = make_float4(sv[4*i], sv[4*i+1], sv[4*i+2], sv[4*i+3]);
+                // fold the four runs of this query in key order
+                const float P1 = dpp_move<float, 0x55>(P), A1 = dpp_move<float, 0x55>(A);
+                const float P2 = dpp_move<float, 0xAA>(P), A2 = dpp_move<float, 0xAA>(A);
+                const float P3 = dpp_move<float, 0xFF>(P), A3 = dpp_move<float, 0xFF>(A);
+                const float M3 = dpp_move<float, 0xFF>(M);
+                if (sgm == 0) {
+                    float S = S0 * P + A;
+                    S = S * P1 + A1; S = S * P2 + A2; S = S * P3 + A3;
+                    s_run[qi] = S; m_run[qi] = M3;
+                }
+            }
+            // the next tile's K rows: every wavefront's matrix instructions over this tile's are behind the barrier above
+            if (it + 1 < n_tiles) { *(u32x4 *)(k_s + kr * T_LDH + kc) = kreg0; *(u32x4 *)(k_s + kr * T_LDH + kc + 8) = kreg1; }
+        }
+        return;
+    }
+
+    // ---- chains: the sequential f16 accumulation, tile by tile ------------------------------------------------------------------------
+    // A lane owns 16 of the 64 d of one query.  A wavefront takes 16 queries x all four d slices: a key that raises the running
+    // maximum of any query of the wavefront costs the whole wavefront a rescale of its accumulators, and with 16 queries
+    // instead of 64 that happens for 6 % of the keys instead of 18 % (records of an i.i.d. sequence: about
+    // min(1, queries / k) at key k).
     const int cq = 16 * wave + (lane & 15);
     const int d0 = (lane >> 4) * 16;
     half2_t acc2[8];                                       // 16 f16 accumulators, two per register
 #pragma unroll
     for (int e = 0; e < 8; ++e) acc2[e] = (half2_t){ (half_t) 0.0f, (half_t) 0.0f };
 
-    // score role: wavefront w computes the 32x32 patch (queries 32*(w/2).., keys 32*(w%2)..)
-    const int sq = (wave >> 1) * 32, sk = (wave & 1) * 32, l32 = lane & 31, g = lane >> 5;
-
-    // K / V tile staging: thread t: row t/4, 32 bytes of each; the next tile is in flight while this one is worked on
-    const int kr = tid >> 2, kc = (tid & 3) * 16;
-    u32x4 kreg0, kreg1, vreg0, vreg1;
-    auto load_kv = [&](int64_t key0) __attribute__((always_inline)) {
-        const int64_t key = key0 + kr < a.KV ? key0 + kr : a.KV - 1;      // rows past the end repeat the last key; their scores are masked
-        const u32x4 * kp = (const u32x4 *)(kb + key * a.k_nb1 + kc * 2);
-        const u32x4 * vp = (const u32x4 *)(vb + key * a.v_nb1 + kc * 2);
-        kreg0 = kp[0]; kreg1 = kp[1]; vreg0 = vp[0]; vreg1 = vp[1];
-    };
-    load_kv(0);
-
-    for (int64_t key0 = 0; key0 < a.KV; key0 += T_KV) {
-        __syncthreads();                                   // the previous step's chains are done with v_s and f_s
-        *(u32x4 *)(k_s + kr * T_LDH + kc) = kreg0; *(u32x4 *)(k_s + kr * T_LDH + kc + 8) = kreg1;
-        *(u32x4 *)(v_s + kr * FA_D  + kc) = vreg0; *(u32x4 *)(v_s + kr * FA_D  + kc + 8) = vreg1;
-        __syncthreads();                                   // K / V tile (and, first time, Q tile) visible
-        if (key0 + T_KV < a.KV) load_kv(key0 + T_KV);
-
-        // ---- scores: S = Q K^T on the matrix cores ------------------------------------------------------------------------------
-        {
-            float16_t c16;
-#pragma unroll
-            for (int r = 0; r < 16; ++r) c16[r] = 0.0f;
-#pragma unroll
-            for (int kk = 0; kk < FA_D / 16; ++kk) {
-                const half8_t av = *(const half8_t *)(q_s + (sq + l32) * T_LDH + kk * 16 + 8 * g);
-                const half8_t bv = *(const half8_t *)(k_s + (sk + l32) * T_LDH + kk * 16 + 8 * g);
-                c16 = __builtin_amdgcn_mfma_f32_32x32x16_f16(av, bv, c16, 0, 0, 0);
-            }
-            const int64_t key = key0 + sk + l32;                  // accumulator column = key, rows = queries
-            const bool key_ok = key < a.KV;
-            float mv[16];
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int qi = sq + 8 * (r >> 2) + 4 * g + (r & 3);
-                mv[r] = 0.0f;
-                if (a.mask) {
-                    const int64_t n = n0 + qi < a.N ? n0 + qi : a.N - 1;
-                    mv[r] = (float) *(const half_t *)(a.mask + n * a.m_nb1 + (key_ok ? key : a.KV - 1) * 2);
-                }
-            }
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int qi = sq + 8 * (r >> 2) + 4 * g + (r & 3);
-                f_s[qi * T_LDF + sk + l32] = key_ok ? __fadd_rn(__fmul_rn(c16[r], a.scale), mv[r]) : -INFINITY;
-            }
-        }
-        __syncthreads();
-
-        // ---- factors: thread t: query t/4, keys 16*(t%4) .. +15 ---------------------------------------------------------------------
-        {
-            const int qi = tid >> 2, sgm = tid & 3;
-            float4 * fp = (float4 *)(f_s + qi * T_LDF + sgm * 16);
-            float sv[16], lmax = -INFINITY;
-#pragma unroll
-            for (int i = 0; i < 4; ++i) { const float4 t = fp[i]; sv[4*i] = t.x; sv[4*i+1] = t.y; sv[4*i+2] = t.z; sv[4*i+3] = t.w; }
-#pragma unroll
-            for (int i = 0; i < 16; ++i) lmax = fmaxf(lmax, sv[i]);
-            float M = m_run[qi];
-            const float S0 = s_run[qi];
-            // (the four runs of a query sit in one quad of lanes: broadcasts inside it are DPP moves, not LDS permutes)
-            const float m0 = dpp_move<float, 0x00>(lmax), m1 = dpp_move<float, 0x55>(lmax), m2 = dpp_move<float, 0xAA>(lmax);
-            if (sgm > 0) M = fmaxf(M, m0);
-            if (sgm > 1) M = fmaxf(M, m1);
-            if (sgm > 2) M = fmaxf(M, m2);
-            // this run's effect on the softmax denominator: S_after = S_before * P + A
-            float P = 1.0f, A = 0.0f;
-#pragma unroll
-            for (int i = 0; i < 16; ++i) {
-                // one exp serves both cases: a new maximum (ms = exp(M - s), 0 for the first key; vs = 1) and a standing
-                // one (vs = exp(s - M); masked keys, s = -inf, get vs = 0, a no-op on the accumulator)
-                const float s = sv[i];
-                const bool  raised = s > M;
-                const float ex = exp_neg(-fabsf(s - M));   // M - s when raised, s - M otherwise: both <= 0 (or NaN / -inf: 0)
-                const float ms = raised ? ex : 1.0f, vs = raised ? 1.0f : ex;
-                M = raised ? s : M;
-                P *= ms; A = A * ms + vs;
-                sv[i] = raised ? -ex : ex;                 // -0.0 keeps the sign
-            }
-#pragma unroll
-            for (int i = 0; i < 4; ++i) fp[i] = make_float4(sv[4*i], sv[4*i+1], sv[4*i+2], sv[4*i+3]);
-            // fold the four runs of this query in key order
-            const float P1 = dpp_move<float, 0x55>(P), A1 = dpp_move<float, 0x55>(A);
-            const float P2 = dpp_move<float, 0xAA>(P), A2 = dpp_move<float, 0xAA>(A);
-            const float P3 = dpp_move<float, 0xFF>(P), A3 = dpp_move<float, 0xFF>(A);
-            const float M3 = dpp_move<float, 0xFF>(M);
-            if (sgm == 0) {
-                float S = S0 * P + A;
-                S = S * P1 + A1; S = S * P2 + A2; S = S * P3 + A3;
-                s_run[qi] = S; m_run[qi] = M3;
-            }
-        }
-        __syncthreads();
-
-        // ---- the sequential f16 chains over this tile's keys -----------------------------------------------------------------------------
-        {
+    for (int it = 0; it <= n_tiles; ++it) {
+        __syncthreads();                                   // tile boundary: tile it - 1 has its factors and its V rows
+        int barriers = 0;                                  // the meeting point inside an iteration, wherever the keys end
+        if (it > 0) {
+            const int64_t key0 = (int64_t)(it - 1) * T_KV;
             const int nk = (int)(a.KV - key0 < T_KV ? a.KV - key0 : T_KV);       // uniform
-            const float4 * fp = (const float4 *)(f_s + cq * T_LDF);
-            const half8_t * vp = (const half8_t *)(v_s + d0);                    // + key * FA_D halves = 8 of these
+            const float4 * fp = (const float4 *)(f_s2 + ((it - 1) & 1) * T_Q * T_LDF + cq * T_LDF);
+            const u32x4 * vp = (const u32x4 *)(v_s2 + ((it - 1) & 1) * T_KV * FA_D + d0);      // + key * FA_D halves = 8 of these
             // one group = four keys: their factors (one b128 read) and their V values (two broadcast b128 reads per key);
             // the next group is read while this one is consumed
-            struct group { float4 f; half8_t v[4][2]; };
+            // (Keys of the tile past the last one carry a factor of exactly 0 — their scores are -inf — and finite V values,
+            // the last key's: walking them leaves every accumulator as it is, so groups are walked whole and the code has no
+            // per-key bounds.)
+            struct group { float4 f; u32x4 v[4][2]; };
             auto gload = [&](group & gr, int k4) __attribute__((always_inline)) {
                 gr.f = fp[k4 >> 2];
 #pragma unroll
                 for (int j = 0; j < 4; ++j) { gr.v[j][0] = vp[(k4 + j) * 8]; gr.v[j][1] = vp[(k4 + j) * 8 + 1]; }
             };
-            auto chain4 = [&](const group & gr, int k4) __attribute__((always_inline)) {
+            auto chain4 = [&](const group & gr) __attribute__((always_inline)) {
                 const float fk[4] = { gr.f.x, gr.f.y, gr.f.z, gr.f.w };
                 const uint32_t sign = (__float_as_uint(fk[0]) | __float_as_uint(fk[1]) | __float_as_uint(fk[2]) | __float_as_uint(fk[3])) >> 31;
                 if (__any(sign)) {                         // some query's maximum moved within these keys: rescale its accumulators
 #pragma unroll
                     for (int j = 0; j < 4; ++j) {
-                        if (k4 + j < nk) {
-                            const bool raised = __float_as_uint(fk[j]) >> 31;
-                            const float ms = raised ? -fk[j] : 1.0f, vs = raised ? 1.0f : fk[j];
-                            if (__any(raised)) {
-#pragma unroll
-                                for (int e = 0; e < 8; ++e) acc2[e] = seq_scale2(acc2[e], ms);   // ms == 1 leaves the value as it is
-                            }
-#pragma unroll
-                            for (int e = 0; e < 8; ++e) {
-                                const half8_t v8 = gr.v[j][e >> 2];
-                                acc2[e] = seq_mad2(acc2[e], (half2_t){ v8[2 * (e & 3)], v8[2 * (e & 3) + 1] }, vs);
-                            }
-                        }
+                        const bool raised = __float_as_uint(fk[j]) >> 31;
+                        const float ms = raised ? -fk[j] : 1.0f, vs = raised ? 1.0f : fk[j];
+                        if (__any(raised)) seq_scale16(acc2, ms);          // ms == 1 leaves the value as it is
+                        seq_mad16(acc2, gr.v[j][0], gr.v[j][1], vs);
                     }
                 } else {
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) {
-                        if (k4 + j < nk) {
-#pragma unroll
-                            for (int e = 0; e < 8; ++e) {
-                                const half8_t v8 = gr.v[j][e >> 2];
-                                acc2[e] = seq_mad2(acc2[e], (half2_t){ v8[2 * (e & 3)], v8[2 * (e & 3) + 1] }, fk[j]);
-                            }
-                        }
-                    }
+                    for (int j = 0; j < 4; ++j) seq_mad16(acc2, gr.v[j][0], gr.v[j][1], fk[j]);
                 }
             };
             // arrived(): first use of a group, placed before the next group's reads are issued, so that the wait it
@@ -675,19 +760,22 @@ __global__ void __launch_bounds__(256) k_fattn_seq_tile(fa_args a) {
             };
             group ga, gb;
             gload(ga, 0);
-            for (int k4 = 0; k4 < nk; k4 += 8) {
+            const int nk8 = (nk + 7) & ~7;                 // whole pairs of groups (a tile holds 64 keys' worth of factors and rows)
+            for (int k4 = 0; k4 < nk8; k4 += 8) {
                 arrived(ga);
-                if (k4 + 4 < nk) gload(gb, k4 + 4);
+                gload(gb, k4 + 4);
                 __builtin_amdgcn_sched_barrier(0);
-                chain4(ga, k4);
-                if (k4 + 4 < nk) {
-                    arrived(gb);
-                    if (k4 + 8 < nk) gload(ga, k4 + 8);
-                    __builtin_amdgcn_sched_barrier(0);
-                    chain4(gb, k4 + 4);
-                }
+                chain4(ga);
+                arrived(gb);
+                gload(ga, k4 + 8 < T_KV ? k4 + 8 : 0);     // (behind the last group: any readable group, nobody walks it)
+                __builtin_amdgcn_sched_barrier(0);
+                chain4(gb);
+                // the producers' meeting point: after 16 keys their scores are written; the other 48 keys are the time their
+                // factor step has
+                if (k4 == 8) { __syncthreads(); ++barriers; }
             }
         }
+        for (; barriers < 1; ++barriers) __syncthreads();
     }
 
     const int64_t n = n0 + cq;
@@ -1028,7 +1116,14 @@ static int flash_attn_ext(const mi355x_tensor * q, const mi355x_tensor * k, cons
             const int64_t gx = (N + T_Q - 1) / T_Q;
             if (gx > 0x7fffffff) return MI355X_ERR_UNSUPPORTED;
             dim3 grid((unsigned) gx, (unsigned) H, (unsigned) q->ne[3]);
-            k_fattn_seq_tile<<<grid, 256, 0, st>>>(a);
+            static bool configured[64];                    // per device: the kernel asks for more LDS than a launch gets by default
+            int dev = 0;
+            if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) { (void) hipGetLastError(); return MI355X_ERR_HIP; }
+            if (!configured[dev]) {
+                if (hipFuncSetAttribute((const void *) k_fattn_seq_tile, hipFuncAttributeMaxDynamicSharedMemorySize, (int) T_LDS_BYTES) != hipSuccess) { (void) hipGetLastError(); return MI355X_ERR_HIP; }
+                configured[dev] = true;
+            }
+            k_fattn_seq_tile<<<grid, 512, T_LDS_BYTES, st>>>(a);
         } break;
         case FA_K_MFMA: {
             const int64_t gx = (N + M_Q - 1) / M_Q;
