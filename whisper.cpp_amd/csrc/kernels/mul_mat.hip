@@ -504,7 +504,7 @@ struct mm_group_entry { const char * w; char * d; const float * bias; const char
 struct mm_group { mm_group_entry e[MM_GROUP_MAX]; };
 
 template <int TI, int TJ, int S>
-__global__ void __launch_bounds__(256) k_gemm_f16_group(mm_args a, int tiles_m, int tiles_n, int sw, mm_group grp) {
+__global__ void __launch_bounds__(256, 2) k_gemm_f16_group(mm_args a, int tiles_m, int tiles_n, int sw, mm_group grp) {
     // the products' tiles form one pool, product after product, and an XCD's run may cross from one product into the next
     const int nblk = tiles_m * tiles_n;
     const int item = xcd_run_index((int)(blockIdx.x + gridDim.x * blockIdx.y), nblk * (int) gridDim.y);
