@@ -56,11 +56,12 @@ GGML_BACKEND_API int                ggml_backend_score(void);
  * "exact" (0/1, default 0: 0 reproduces the two roundings that the reference's CPU backend applies — Q8_0-rounded
  * activations in front of quantized MUL_MAT, f16 key-by-key V accumulation in FLASH_ATTN_EXT; 1 keeps f16 activations
  * and f32 accumulators, which is closer to exact arithmetic and further from the reference),
- * "fa_accum" (0/1, default 0: how FLASH_ATTN_EXT over more than 8 queries accumulates V.  0: key by key with an f16
- * accumulator, f32 fma + f16 store — the reference's sequence (ops.cpp:6793-6807), and the only setting that keeps
- * whole-model logits within 1e-3 NMSE of the CPU backend.  1: f32 accumulators with both products on the matrix cores —
- * six times faster, within the per-op bound, but the reference's f16 rounding is then missing and whole-model logits sit
- * several 1e-3 away).
+ * "fa_accum" (0..3, default 0: how FLASH_ATTN_EXT accumulates V.  0: key by key with an f16 accumulator, f32 fma + f16
+ * store — the reference's sequence (ops.cpp:6793-6807), and the only setting that keeps whole-model logits within 1e-3
+ * NMSE of the CPU backend.  Bit 0: f32 accumulators with both products on the matrix cores for more than 8 queries —
+ * five times faster, within the per-op bound, but the reference's f16 rounding is then missing and whole-model logits sit
+ * several 1e-3 away.  Bit 1: f32 accumulators for a decode step's few queries; the decoder's layers alone move the
+ * logits to 6e-3 … 8e-3 NMSE).
  * The environment variables GGML_MI355X_FUSE, GGML_MI355X_PROFILE, GGML_MI355X_EXACT and GGML_MI355X_FA_ACCUM give the
  * initial values.
  * backend == NULL addresses every live MI355X backend of the process (a host such as whisper.cpp keeps its

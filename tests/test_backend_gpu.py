@@ -142,7 +142,13 @@ def test_f32_matrix_core_attention_option(harness, models):
     s = rows[-1]
     assert s["summary"] == "model" and s["ids_identical"] == 16 and s["worst_logits_nmse"] <= 2e-2, s
     rc, rows = run_harness(harness, ["model", "--model", models[("base", "q5_0")], "--steps", "16"], timeout=900)
-    assert rows[-1]["worst_logits_nmse"] < s["worst_logits_nmse"], (rows[-1], s)
+    default = rows[-1]
+    assert default["worst_logits_nmse"] < s["worst_logits_nmse"], (default, s)
+    # bit 1 of the option: f32 accumulators for a decode step's few queries only (the encoder keeps the reference's sequence).
+    # The four or six decoder layers alone already move the logits past the bound: the decode step keeps the sequence too.
+    rc, rows = run_harness(harness, ["model", "--model", models[("base", "q5_0")], "--steps", "16"], env={"GGML_MI355X_FA_ACCUM": "2"}, timeout=900)
+    d = rows[-1]
+    assert d["summary"] == "model" and d["ids_identical"] == 16 and 1e-3 < d["worst_logits_nmse"] <= 2e-2, d
 
 
 def test_default_attention_graphs_without_flash_attn(harness, models):

@@ -87,8 +87,9 @@ struct mi355x_backend_ctx {
     bool        fuse    = true;
     bool        profile = false;
     bool        debug   = false;   // log what every MUL_MAT launch folds in (GGML_MI355X_DEBUG=1)
-    int         fa_accum = 0;           // V accumulation of attention over more than 8 queries: 0 the reference's sequence (f32 fma,
-                                        // f16 store, key by key), 1 f32 accumulators on the matrix cores
+    int         fa_accum = 0;           // V accumulation of attention: 0 the reference's sequence (f32 fma, f16 store, key by key);
+                                        // bit 0: f32 accumulators (matrix cores) for more than 8 queries, bit 1: f32
+                                        // accumulators for a decode step's few queries
     bool        weight_images = true;   // keep f16 images of quantized GEMM weights (GGML_MI355X_WEIGHT_IMAGES=0 turns it off)
     bool        exact   = false;   // true: f32 attention accumulators and un-rounded GEMM activations instead of the
                                    // reference's f16-sequential / Q8_0-rounded arithmetic

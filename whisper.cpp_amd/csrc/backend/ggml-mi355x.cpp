@@ -528,7 +528,7 @@ static ggml_backend_t device_init_backend(ggml_backend_dev_t dev, const char *) 
     ctx->fuse    = env_flag("GGML_MI355X_FUSE", true);
     ctx->profile = env_flag("GGML_MI355X_PROFILE", false);
     ctx->exact   = env_flag("GGML_MI355X_EXACT", false);
-    if (const char * e = getenv("GGML_MI355X_FA_ACCUM")) { const int v = atoi(e); if (v >= 0 && v <= 1) ctx->fa_accum = v; }
+    if (const char * e = getenv("GGML_MI355X_FA_ACCUM")) { const int v = atoi(e); if (v >= 0 && v <= 3) ctx->fa_accum = v; }
     ctx->weight_images = env_flag("GGML_MI355X_WEIGHT_IMAGES", true);
     ctx->debug   = env_flag("GGML_MI355X_DEBUG", false);
     // default priority, blocking with respect to the null stream used by the buffer-level copies
@@ -615,7 +615,7 @@ static int set_option(ggml_backend_t backend, const char * name, int value) {
     const bool is_fuse = strcmp(name, "fuse") == 0, is_profile = strcmp(name, "profile") == 0, is_exact = strcmp(name, "exact") == 0;
     const bool is_accum = strcmp(name, "fa_accum") == 0;
     if (!is_fuse && !is_profile && !is_exact && !is_accum) return -1;
-    if (is_accum && (value < 0 || value > 1)) return -1;
+    if (is_accum && (value < 0 || value > 3)) return -1;
     std::lock_guard<std::mutex> lock(g_live_mutex);
     for (mi355x_backend_ctx * ctx : g_live) {
         if (backend && ctx != (mi355x_backend_ctx *) backend->context) continue;

@@ -632,7 +632,7 @@ struct graph_runner {
     const ggml_tensor * cast_dst = nullptr, * cast_src = nullptr;          // a cast that the next attention node carries out
     bool next_attention_casts(int i) const {
         const ggml_tensor * n = g->nodes[i], * s0 = n->src[0];
-        if (!ctx->fuse || ctx->exact || n->src[1] != n || s0->type != GGML_TYPE_F32 || n->type != GGML_TYPE_F16 ||
+        if (!ctx->fuse || ctx->exact || (ctx->fa_accum & 2) || n->src[1] != n || s0->type != GGML_TYPE_F32 || n->type != GGML_TYPE_F16 ||
             (n->flags & GGML_TENSOR_FLAG_OUTPUT) || !ggml_is_contiguous(s0) || !ggml_is_contiguous(n) || !ggml_are_same_shape(s0, n) ||
             n->ne[2] != 1 || n->ne[3] != 1 || n->view_src) return false;
         int j = i + 1;
@@ -750,9 +750,9 @@ struct graph_runner {
                 if (m) vm = to_view(m);
                 const double flops = 4.0 * s0->ne[1] * k->ne[1] * 64.0 * s0->ne[2] * s0->ne[3];
                 const double bytes = (double) ggml_nelements(s0) * 4 + 2.0 * (double) k->ne[0] * k->ne[1] * k->ne[2] * k->ne[3] * 2 + nbytes_of(n);
-                // the accumulation option is for the many-query kernels; a decode step keeps the reference's sequence
-                const int accum = s0->ne[1] > 8 ? ctx->fa_accum : 0;
-                const int mode = ctx->exact || accum == 1 ? MI355X_FA_F32 : MI355X_FA_F16_SEQ;
+                // the accumulation option, bit 0: more than 8 queries, bit 1: a decode step's few queries
+                const bool f32_accum = s0->ne[1] > 8 ? (ctx->fa_accum & 1) != 0 : (ctx->fa_accum & 2) != 0;
+                const int mode = ctx->exact || f32_accum ? MI355X_FA_F32 : MI355X_FA_F16_SEQ;
                 const char * name = mi355x_flash_attn_ext_kernel_name(&vq, &vk, mode);
                 // the output projection that follows takes its Q8_0-rounded activations from the attention kernel itself
                 const bool emits = !ctx->exact && (strncmp(name, "flash_attn.seq_tile", 19) == 0 || strcmp(name, "flash_attn.mfma_f32") == 0);
