@@ -10,9 +10,10 @@
 //                                the reference's sequence.  The running maximum is turned into a prefix maximum, so
 //                                all exp() factors (vs = exp(s - M_k), ms = exp(M_{k-1} - M_k)) are computed in
 //                                parallel up front and only the one-instruction f16 fma chain stays sequential.
-//       k_fattn_seq_tile   N > 8:  64 queries x 64 keys per step; QK^T on v_mfma_f32_32x32x16_f16 from LDS-staged K,
-//                                  softmax factors in LDS, then 16 queries per wavefront walk the 64 keys with
-//                                  v_fma_mix_f32 + v_cvt_pk_f16_f32 chains against the LDS-staged V tile.
+//       k_fattn_seq_tile   N > 8:  64 queries x 64 keys per tile, two roles: four wavefronts make the next tile's
+//                                  factors (QK^T on v_mfma_f32_32x32x16_f16 from LDS-staged K) while four walk this
+//                                  tile's 64 keys, 16 queries each, with v_fma_mix_f32 + v_cvt_pk_f16_f32 chains
+//                                  against the LDS-staged V tile.
 //       k_fattn_seq_row    N <= 8: one block per (query, head): one wavefront (lane = d) runs the chain while the
 //                                  other three score, scan and stage the next 192 keys.
 //   MI355X_FA_F32          f32 accumulators: closer to exact arithmetic, not to the reference (whose f16 accumulator
