@@ -290,6 +290,35 @@ __global__ void k_x_to_f16(const char * __restrict__ x, half_t * __restrict__ ou
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
+// What follows the K loop of a tile: GELU reads its table from LDS when the operand buffers, free now (the loop's last barrier
+// is behind every wavefront), are large enough to hold the part that matters (TABLE_FITS); then the 32x32 patches.
+template <int TI, int TJ, bool EMIT, bool TABLE_FITS>
+__device__ __forceinline__ void gemm_tile_epilogue(float16_t (&acc)[TI][TJ], const mm_args & a, const epi_args & epi, char * db, int64_t batch_off, int64_t d_nb1,
+                                                   int64_t n0, int64_t m0, int wn, int wmo, char * smem) {
+    const int tid = threadIdx.x, lane = tid & 63, l32 = lane & 31, g = lane >> 5;
+    const uint16_t * gelu_lds = nullptr;
+    if constexpr (TABLE_FITS) {
+        if (epi.flags & MI355X_EPI_GELU) {
+            const u32x4 * pos = (const u32x4 *) epi.gelu, * neg = (const u32x4 *)(epi.gelu + 0x8000);
+            u32x4 * dst = (u32x4 *) smem;
+            constexpr int pieces = GELU_LDS_HALF * 2 / 16;
+            for (int p = tid; p < pieces; p += 256) { dst[p] = pos[p]; dst[pieces + p] = neg[p]; }
+            __syncthreads();
+            gelu_lds = (const uint16_t *) smem;
+        }
+    }
+    // accumulator register e of a 32x32 patch: row (= n) 8*(e/4) + 4*g + e%4, column (= m) lane%32
+#pragma unroll
+    for (int i = 0; i < TI; ++i) {
+        int64_t n[16];
+#pragma unroll
+        for (int e = 0; e < 16; ++e) n[e] = n0 + wn + 32 * i + 8 * (e >> 2) + 4 * g + (e & 3);
+#pragma unroll
+        for (int j = 0; j < TJ; ++j)
+            patch_epilogue<EMIT>(acc[i][j], epi, db, batch_off, d_nb1, m0 + wmo + 32 * j + l32, a.M, n, a.N, gelu_lds);
+    }
+}
+
 // KTAIL: K is not a multiple of 64 (but of 8); FULL: K / 64 is a multiple of S; EMIT: MI355X_EPI_EMIT_F16 (a kernel of its
 // own, because its epilogue needs more registers than two workgroups per CU leave)
 template <int TI, int TJ, int S, bool KTAIL, bool FULL, bool EMIT = false>
@@ -442,30 +471,115 @@ __device__ __forceinline__ void gemm_f16_tile(const mm_args & a, int tiles_m, in
         }
     }
 
-    // GELU reads its table from LDS when the operand buffers, free now (the loop's last barrier is behind every wavefront),
-    // are large enough to hold the part that matters
-    const uint16_t * gelu_lds = nullptr;
-    if constexpr ((size_t) 2 * (BN + BM) * GB_LD * sizeof(half_t) >= GELU_LDS_BYTES) {
-        if (epi.flags & MI355X_EPI_GELU) {
-            const u32x4 * pos = (const u32x4 *) epi.gelu, * neg = (const u32x4 *)(epi.gelu + 0x8000);
-            u32x4 * dst = (u32x4 *) smem;
-            constexpr int pieces = GELU_LDS_HALF * 2 / 16;
-            for (int p = tid; p < pieces; p += 256) { dst[p] = pos[p]; dst[pieces + p] = neg[p]; }
-            __syncthreads();
-            gelu_lds = (const uint16_t *) smem;
-        }
-    }
+    gemm_tile_epilogue<TI, TJ, EMIT, ((size_t) 2 * (BN + BM) * GB_LD * sizeof(half_t) >= GELU_LDS_BYTES)>(acc, a, epi, db, batch_off, d_nb1, n0, m0, wn, wmo, smem);
+}
 
-    // accumulator register e of a 32x32 patch: row (= n) 8*(e/4) + 4*g + e%4, column (= m) lane%32
+// The same tile with the operands going from global memory straight into LDS (global_load_lds_dwordx4: lane l's 16 bytes
+// land at the wave's LDS base + 16 l, no register and no LDS store instruction in between).  Measured on the register-staged
+// loop above, a wavefront spends two thirds of a K step outside its matrix phase — issuing the global loads, whose return
+// path into the registers is busy, and the LDS stores — and here both phases are gone: a step is a wait, a barrier,
+// the issue of the loads NBUF - 1 steps ahead and the matrix phase.
+// LDS tile of an operand: row pairs form 256-byte lines, the 16-byte chunk c of row r sits in slot (r & 1) * 8 +
+// (c ^ ((r >> 1) & 7)) of line r >> 1 — the 16 lanes of a b128 fragment read (16 consecutive rows, one chunk) then cover 256
+// consecutive bytes' worth of banks, and a wave's load (1 KB: 8 rows) writes whole lines from whole 128-byte row pieces.
+// K a multiple of 64; operands as f16 rows (16-byte aligned).
+#define DL_STEP_ROW 128     // bytes of a row in one K step
+
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {                // s_waitcnt vmcnt(N) only (gfx9 encoding: expcnt and lgkmcnt at their maxima)
+    static_assert(N >= 0 && N < 64, "vmcnt has six bits");
+    __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
+}
+
+template <int TI, int TJ, int NBUF, bool EMIT>
+__device__ __forceinline__ void gemm_f16_tile_dl(const mm_args & a, int tiles_m, int tiles_n, int sw, int tile, const char * wb, const char * xb, char * db,
+                                                 const epi_args & epi, int64_t batch_off, int64_t d_nb1) {
+    constexpr int BN = 64 * TI, BM = 64 * TJ;
+    constexpr int XL = BN / 32, WL = BM / 32;          // 1 KB loads per wavefront and step (8 rows each)
+    constexpr int STEP_BYTES = (BN + BM) * DL_STEP_ROW;
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+
+    const int per_col = sw * tiles_n, col = tile / per_col, rem = tile - col * per_col;
+    const int cw = min(sw, tiles_m - col * sw);
+    const int64_t m0 = (int64_t)(col * sw + rem % cw) * BM;
+    const int64_t n0 = (int64_t)(rem / cw) * BN;
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    // load i of this wavefront covers rows 32 i + 8 wave .. + 7 of the tile; this lane: row lrow of the 8, chunk lchunk
+    const int lrow = 2 * (lane >> 4) + ((lane & 15) >> 3);
+    const int lchunk = (lane & 7) ^ ((4 * (wave & 1) + (lane >> 4)) & 7);
+    const char * xp[XL]; const char * wp[WL];
 #pragma unroll
-    for (int i = 0; i < TI; ++i) {
-        int64_t n[16];
+    for (int i = 0; i < XL; ++i) { const int64_t n = n0 + 32 * i + 8 * wave + lrow; xp[i] = xb + (n < a.N ? n : a.N - 1) * a.x_nb1 + lchunk * 16; }
 #pragma unroll
-        for (int e = 0; e < 16; ++e) n[e] = n0 + wn + 32 * i + 8 * (e >> 2) + 4 * g + (e & 3);
+    for (int i = 0; i < WL; ++i) { const int64_t m = m0 + 32 * i + 8 * wave + lrow; wp[i] = wb + (m < a.M ? m : a.M - 1) * a.w_nb1 + lchunk * 16; }
+    auto load = [&](int step, int buf) __attribute__((always_inline)) {
+        const int64_t ko = (int64_t) step * DL_STEP_ROW;
+        char * xs = smem + buf * STEP_BYTES + wave * 1024, * ws = xs + BN * DL_STEP_ROW;
+#pragma unroll
+        for (int i = 0; i < XL; ++i)
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(xp[i] + ko), (__attribute__((address_space(3))) void *)(xs + i * 4096), 16, 0, 0);
+#pragma unroll
+        for (int i = 0; i < WL; ++i)
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(wp[i] + ko), (__attribute__((address_space(3))) void *)(ws + i * 4096), 16, 0, 0);
+    };
+
+    const int wn = (wave >> 1) * 32 * TI, wmo = (wave & 1) * 32 * TJ;   // wave patch origin inside the tile
+    const int l32 = lane & 31, g = lane >> 5;
+    // fragment reads: row wn + 32 i + l32 (its line and half of the line), chunk 2 kk + g swizzled by the row
+    const int rsw = (l32 >> 1) & 7;
+    const int xrow = ((wn + l32) >> 1) * 256 + (l32 & 1) * 128, wrow = BN * DL_STEP_ROW + ((wmo + l32) >> 1) * 256 + (l32 & 1) * 128;
+    int koff[GB_K / 16];
+#pragma unroll
+    for (int kk = 0; kk < GB_K / 16; ++kk) koff[kk] = ((2 * kk + g) ^ rsw) * 16;
+
+    float16_t acc[TI][TJ];
+#pragma unroll
+    for (int i = 0; i < TI; ++i)
 #pragma unroll
         for (int j = 0; j < TJ; ++j)
-            patch_epilogue<EMIT>(acc[i][j], epi, db, batch_off, d_nb1, m0 + wmo + 32 * j + l32, a.M, n, a.N, gelu_lds);
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
+
+    // one K step: all fragment reads of the step go out first (they return in order, so the matrix instructions start when
+    // the first sub-step's have arrived and never wait for a read issued behind them), then the 4 TI TJ matrix instructions
+    auto mma = [&](int buf) __attribute__((always_inline)) {
+        const char * xs = smem + buf * STEP_BYTES + xrow, * ws = smem + buf * STEP_BYTES + wrow;
+        half8_t av[GB_K / 16][TI], bv[GB_K / 16][TJ];
+#pragma unroll
+        for (int kk = 0; kk < GB_K / 16; ++kk) {
+#pragma unroll
+            for (int i = 0; i < TI; ++i) av[kk][i] = *(const half8_t *)(xs + i * 4096 + koff[kk]);
+#pragma unroll
+            for (int j = 0; j < TJ; ++j) bv[kk][j] = *(const half8_t *)(ws + j * 4096 + koff[kk]);
+        }
+#pragma unroll
+        for (int kk = 0; kk < GB_K / 16; ++kk)
+#pragma unroll
+            for (int i = 0; i < TI; ++i)
+#pragma unroll
+                for (int j = 0; j < TJ; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(av[kk][i], bv[kk][j], acc[i][j], 0, 0, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, (GB_K / 16) * (TI + TJ), 0);     // the DS reads
+        __builtin_amdgcn_sched_group_barrier(0x008, (GB_K / 16) * TI * TJ, 0);       // the MFMAs
+    };
+
+    const int KT = (int)(a.K / GB_K), last = KT - 1;
+    // Every step issues its XL + WL loads unconditionally (beyond the end it re-reads the last step into a buffer nobody reads
+    // again), so "all but the (NBUF - 2) (XL + WL) youngest have landed" is a constant wait.
+#pragma unroll
+    for (int st = 0; st < NBUF - 1; ++st) load(min(st, last), st);
+    int buf = 0, fill = NBUF - 1;                      // buffer of step kt; buffer that step kt + NBUF - 1 goes into
+    for (int kt = 0; kt < KT; ++kt) {
+        wait_vmcnt<(NBUF - 2) * (XL + WL)>();             // this wavefront's pieces of step kt are in LDS
+        __syncthreads();                                // ... everybody's are, and everybody is done reading step kt - 1
+        load(min(kt + NBUF - 1, last), fill);           // into the buffer of step kt - 1
+        mma(buf);
+        buf = buf + 1 == NBUF ? 0 : buf + 1; fill = fill + 1 == NBUF ? 0 : fill + 1;
     }
+    wait_vmcnt<0>();                                    // the surplus loads still write LDS, which the epilogue reuses
+    __syncthreads();
+    gemm_tile_epilogue<TI, TJ, EMIT, true>(acc, a, epi, db, batch_off, d_nb1, n0, m0, wn, wmo, smem);
 }
 
 // Workgroups are dealt round-robin to the 8 XCDs, each with its own L2: workgroup `lin` of `total` runs on XCD lin % 8.
@@ -514,6 +628,49 @@ __global__ void __launch_bounds__(256, 2) k_gemm_f16_group(mm_args a, int tiles_
     gemm_f16_tile<TI, TJ, S, false, true>(a, tiles_m, tiles_n, sw, item % nblk, ge.w, a.x, ge.d, e, 0, ge.d_nb1);
 }
 
+// the direct-to-LDS form of the two kernels above (K a multiple of 64)
+template <int TI, int TJ, int NBUF, bool EMIT>
+__global__ void __launch_bounds__(256, 2) k_gemm_f16_dl(mm_args a, int tiles_m, int tiles_n, int sw) {
+    const int64_t b2 = blockIdx.y % a.ne12, b3 = blockIdx.y / a.ne12;
+    gemm_f16_tile_dl<TI, TJ, NBUF, EMIT>(a, tiles_m, tiles_n, sw, xcd_run_index(blockIdx.x, tiles_m * tiles_n),
+                                         a.w + (b2 / a.r2) * a.w_nb2 + (b3 / a.r3) * a.w_nb3, a.x + b2 * a.x_nb2 + b3 * a.x_nb3,
+                                         a.d + b2 * a.d_nb2 + b3 * a.d_nb3, a.e, b2 * a.d_nb2 + b3 * a.d_nb3, a.d_nb1);
+}
+template <int TI, int TJ, int NBUF>
+__global__ void __launch_bounds__(256, 2) k_gemm_f16_dl_group(mm_args a, int tiles_m, int tiles_n, int sw, mm_group grp) {
+    const int nblk = tiles_m * tiles_n;
+    const int item = xcd_run_index((int)(blockIdx.x + gridDim.x * blockIdx.y), nblk * (int) gridDim.y);
+    const mm_group_entry & ge = grp.e[item / nblk];
+    epi_args e;
+    e.flags = ge.flags; e.scale = ge.scale; e.bias = ge.bias; e.residual = ge.residual; e.gelu = a.e.gelu; e.image = nullptr;
+    gemm_f16_tile_dl<TI, TJ, NBUF, false>(a, tiles_m, tiles_n, sw, item % nblk, ge.w, a.x, ge.d, e, 0, ge.d_nb1);
+}
+// LDS buffers of K steps in flight by tile shape: 128 x 128 tiles keep two workgroups per CU (2 x 32 KB each)
+template <int TI, int TJ> constexpr int dl_buffers() { return TI * TJ == 4 ? 2 : 3; }
+template <int TI, int TJ> constexpr size_t dl_lds_bytes() {
+    constexpr size_t ring = (size_t) dl_buffers<TI, TJ>() * 64 * (TI + TJ) * DL_STEP_ROW;
+    return ring > GELU_LDS_BYTES ? ring : GELU_LDS_BYTES;        // the epilogue keeps the GELU table slice there
+}
+
+template <int TI, int TJ, bool EMIT>
+static int launch_gemm_f16_dl(const mm_args & a, hipStream_t st) {
+    constexpr int BN = 64 * TI, BM = 64 * TJ, NBUF = dl_buffers<TI, TJ>();
+    constexpr size_t lds = dl_lds_bytes<TI, TJ>();
+    static bool configured[64];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return MI355X_ERR_HIP;
+    if (!configured[dev]) {
+        if (hipFuncSetAttribute((const void *) k_gemm_f16_dl<TI, TJ, NBUF, EMIT>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds) != hipSuccess) return MI355X_ERR_HIP;
+        configured[dev] = true;
+    }
+    const int64_t tm = (a.M + BM - 1) / BM, tn = (a.N + BN - 1) / BN;
+    if (tm * tn > 0x7fffffff) return MI355X_ERR_UNSUPPORTED;
+    dim3 grid((unsigned)(tm * tn), (unsigned)(a.ne12 * a.ne13));
+    const int sw = tile_path_width(tm, tn, (tm * tn + 7) / 8, BN, BM);
+    k_gemm_f16_dl<TI, TJ, NBUF, EMIT><<<grid, 256, lds, st>>>(a, (int) tm, (int) tn, sw);
+    return launch_status();
+}
+
 template <int TI, int TJ, int S, bool KTAIL, bool FULL, bool EMIT = false>
 static int launch_gemm_f16_k(const mm_args & a, hipStream_t st) {
     static_assert(S % 2 == 0, "the LDS buffer index is the parity of the register slot");
@@ -535,6 +692,12 @@ static int launch_gemm_f16_k(const mm_args & a, hipStream_t st) {
 }
 template <int TI, int TJ>
 static int launch_gemm_f16(const mm_args & a, hipStream_t st) {
+    static const bool staged = getenv("MI355X_GEMM_STAGED") != nullptr;        // the register-staged loop, for comparison
+    // 128 x 128 tiles only: the direct loads move about half the bytes per clock of the register path, which pays where two
+    // workgroups share a CU (10 - 13 % faster) and loses on the 128 x 64 tiles that run one to a CU
+    if constexpr (TI * TJ == 4) {
+        if (a.K % GB_K == 0 && !staged) return (a.e.flags & MI355X_EPI_EMIT_F16) ? launch_gemm_f16_dl<TI, TJ, true>(a, st) : launch_gemm_f16_dl<TI, TJ, false>(a, st);
+    }
     if (a.e.flags & MI355X_EPI_EMIT_F16) {
         if (a.K % (2 * GB_K)) return MI355X_ERR_UNSUPPORTED;
         return a.K % (4 * GB_K) == 0 ? launch_gemm_f16_k<TI, TJ, 4, false, true, true>(a, st) : launch_gemm_f16_k<TI, TJ, 2, false, true, true>(a, st);
@@ -561,6 +724,19 @@ static int launch_gemm_f16_group(const mm_args & a, const mm_group & grp, int co
     if (tm * tn > 0x7fffffff) return MI355X_ERR_UNSUPPORTED;
     dim3 grid((unsigned)(tm * tn), (unsigned) count);
     const int sw = tile_path_width(tm, tn, (tm * tn * count + 7) / 8, BN, BM);
+    static const bool staged = getenv("MI355X_GEMM_STAGED") != nullptr;
+    if constexpr (TI * TJ == 4) {
+    if (!staged) {
+        static bool dl_configured[64];
+        constexpr size_t dl_lds = dl_lds_bytes<TI, TJ>();
+        if (!dl_configured[dev]) {
+            if (hipFuncSetAttribute((const void *) k_gemm_f16_dl_group<TI, TJ, dl_buffers<TI, TJ>()>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) dl_lds) != hipSuccess) return MI355X_ERR_HIP;
+            dl_configured[dev] = true;
+        }
+        k_gemm_f16_dl_group<TI, TJ, dl_buffers<TI, TJ>()><<<grid, 256, dl_lds, st>>>(a, (int) tm, (int) tn, sw, grp);
+        return launch_status();
+    }
+    }
     k_gemm_f16_group<TI, TJ, 4><<<grid, 256, lds, st>>>(a, (int) tm, (int) tn, sw, grp);
     return launch_status();
 }
