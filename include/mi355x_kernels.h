@@ -69,6 +69,8 @@ enum mi355x_epilogue_flags {
     MI355X_EPI_EMIT_F16 = 1024, /* GEMM path, f32 dst with ne0 a multiple of 32: also write to `image` the rows of dst
                                   rounded to Q8_0 like quantize_row_q8_0 and stored as f16(q * d), dense [N][M] — what
                                   the src1 conversion pass of the MUL_MAT that reads dst next would produce            */
+    MI355X_EPI_IMAGE_ONLY = 2048, /* with MI355X_EPI_EMIT_F16: write the image only, not dst (whose data pointer may then be
+                                  NULL) — for a result whose only readers are products that take the image              */
     MI355X_MM_PREPARE_ONLY = 512, /* GEMM path: run only the src1 conversion pass into `workspace` and return; the
                                   product itself then follows in a second call with MI355X_MM_WS_READY (lets a
                                   caller time or overlap the two separately); a no-op on the other paths       */
@@ -240,7 +242,8 @@ MI355X_API int mi355x_norm(const mi355x_tensor * src, const mi355x_tensor * dst,
 /* The same, and in the same pass the result's image for the MFMA GEMM: rounded to Q8_0 as quantize_row_q8_0 does
  * (ggml-cpu-quants.c:808-865) and stored as f16(q * d), dense [rows][ne0], at `x16` — what mi355x_mul_mat's src1
  * conversion pass would write into its workspace (then pass MI355X_MM_WS_READY).  ne0 multiple of 32 and at most 2048,
- * 16-byte aligned rows; MI355X_ERR_UNSUPPORTED otherwise. */
+ * 16-byte aligned rows; MI355X_ERR_UNSUPPORTED otherwise.  With dst->data == NULL (shape and strides still describe the
+ * result) only the image is written: for a result whose only readers are products that take the image. */
 MI355X_API int mi355x_norm_emit_f16(const mi355x_tensor * src, const mi355x_tensor * dst, float eps, const float * w, const float * b,
                                     void * x16, void * stream);
 /* The same for the few-column product (N <= 8) over quantized weights: the result quantized to Q8_0 itself, in the layout

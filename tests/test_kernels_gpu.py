@@ -283,6 +283,19 @@ def test_mul_mat_epilogue_emits_the_next_products_activation_image(pkg, oracle, 
     assert oracle.nmse(y, oracle.gelu(oracle.mul_mat(pkg.Q5_0, blocks, x) + bias)) <= 1e-5
     image = oracle.dequantize(oracle.Q8_0, oracle.quantize(oracle.Q8_0, y, act=True), m).reshape(n, m)
     assert np.array_equal(gpu.down(d_h, np.uint16), oracle.f32_to_f16_bits(image))
+    # MI355X_EPI_IMAGE_ONLY: the same image, dst untouched (its data pointer may be NULL); not without the image
+    d_h2 = torch.zeros((n, m), dtype=torch.float16, device=gpu.dev)
+    epi.flags, epi.image = pkg.EPI_BIAS | pkg.EPI_GELU | pkg.EPI_EMIT_F16 | pkg.EPI_IMAGE_ONLY, d_h2.data_ptr()
+    d_y.fill_(7.0)
+    pkg.check(lib.mi355x_mul_mat(tw, tx, ty, C.byref(epi), ws.data_ptr(), need, gpu.stream))
+    assert np.array_equal(gpu.down(d_h2, np.uint16), gpu.down(d_h, np.uint16)) and np.all(gpu.down(d_y) == 7.0)
+    t_null = pkg.tensor(d_y, pkg.F32); t_null.data = None
+    d_h2.zero_()
+    pkg.check(lib.mi355x_mul_mat(tw, tx, t_null, C.byref(epi), ws.data_ptr(), need, gpu.stream))
+    assert np.array_equal(gpu.down(d_h2, np.uint16), gpu.down(d_h, np.uint16))
+    epi.flags = pkg.EPI_BIAS | pkg.EPI_IMAGE_ONLY
+    assert lib.mi355x_mul_mat(tw, tx, ty, C.byref(epi), ws.data_ptr(), need, gpu.stream) == -2
+    epi.flags, epi.image = pkg.EPI_BIAS | pkg.EPI_GELU | pkg.EPI_EMIT_F16, d_h.data_ptr()
     # the GEMV path has no such epilogue
     d_x5 = gpu.up(x[:5])
     d_y5 = torch.zeros((5, m), dtype=torch.float32, device=gpu.dev)
@@ -656,6 +669,12 @@ def test_norm_and_affine(pkg, oracle, gpu):
             assert oracle.nmse(y, want * w + b) <= 1e-10
             image = oracle.dequantize(oracle.Q8_0, oracle.quantize(oracle.Q8_0, y, act=True), shape[1]).reshape(shape)
             assert np.array_equal(gpu.down(d_h, np.uint16), oracle.f32_to_f16_bits(image))
+            # without a destination (data pointer NULL): the same image and no other store
+            t_null = pkg.tensor(d_y, pkg.F32); t_null.data = None
+            d_h2 = torch.zeros(shape, dtype=torch.float16, device=gpu.dev)
+            d_y.fill_(7.0)
+            pkg.check(lib.mi355x_norm_emit_f16(pkg.tensor(d_x, pkg.F32), t_null, 1e-5, d_w.data_ptr(), d_b.data_ptr(), d_h2.data_ptr(), gpu.stream))
+            assert np.array_equal(gpu.down(d_h2, np.uint16), gpu.down(d_h, np.uint16)) and np.all(gpu.down(d_y) == 7.0)
         else:
             assert rc == -1                      # unsupported shapes say so; the caller falls back to the plain kernel
         # and the variant for the few-column product: Q8_0 itself, quants | scales | block sums

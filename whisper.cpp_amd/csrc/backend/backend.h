@@ -90,6 +90,8 @@ struct mi355x_backend_ctx {
     int         fa_accum = 0;           // V accumulation of attention: 0 the reference's sequence (f32 fma, f16 store, key by key);
                                         // bit 0: f32 accumulators (matrix cores) for more than 8 queries, bit 1: f32
                                         // accumulators for a decode step's few queries
+    bool        dead_f32 = true;        // a result whose only reader is the next launch's activation image is not also written as f32
+                                        // (GGML_MI355X_DEAD_F32=0: always write it)
     bool        weight_images = true;   // keep f16 images of quantized GEMM weights (GGML_MI355X_WEIGHT_IMAGES=0 turns it off)
     bool        exact   = false;   // true: f32 attention accumulators and un-rounded GEMM activations instead of the
                                    // reference's f16-sequential / Q8_0-rounded arithmetic
@@ -99,6 +101,7 @@ struct mi355x_backend_ctx {
     void *       ws       = nullptr;   // the current slot (where the cached activation image lives)
     size_t       ws_size  = 0;         // bytes per slot
     int          ws_slot  = 0;
+    const void * image_only = nullptr; // activations whose producer wrote their image into the workspace and nothing else (this graph)
     const void * ws_x     = nullptr;
     int          ws_x_mode = 0;
     int64_t      ws_x_ne[4] = {0, 0, 0, 0};

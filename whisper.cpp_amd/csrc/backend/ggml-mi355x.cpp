@@ -530,6 +530,7 @@ static ggml_backend_t device_init_backend(ggml_backend_dev_t dev, const char *) 
     ctx->exact   = env_flag("GGML_MI355X_EXACT", false);
     if (const char * e = getenv("GGML_MI355X_FA_ACCUM")) { const int v = atoi(e); if (v >= 0 && v <= 3) ctx->fa_accum = v; }
     ctx->weight_images = env_flag("GGML_MI355X_WEIGHT_IMAGES", true);
+    ctx->dead_f32 = env_flag("GGML_MI355X_DEAD_F32", true);
     ctx->debug   = env_flag("GGML_MI355X_DEBUG", false);
     // default priority, blocking with respect to the null stream used by the buffer-level copies
     HIP_TRY(hipStreamCreate(&ctx->stream), { delete ctx; return NULL; });

@@ -123,14 +123,23 @@ void mi355x_backend_ctx::drain_events() {
 // next product's image into the other.
 bool mi355x_backend_ctx::reserve_workspace(size_t size) {
     if (size <= ws_size) return true;
-    // the stream may still be reading the old block
-    if (hipStreamSynchronize(stream) != hipSuccess) { (void) hipGetLastError(); return false; }
-    if (ws_base) (void) hipFree(ws_base);
-    ws_base = nullptr; ws = nullptr; ws_size = 0; ws_x = nullptr; ws_slot = 0;
+    // Grow: the slots keep their contents (an activation image that a producer left there may be the only copy of its values,
+    // see image_only), so the old block is copied over before it goes.
     const size_t want = (size + size / 2 + 255) / 256 * 256;
-    if (hipMalloc(&ws_base, 2 * want) != hipSuccess) { (void) hipGetLastError(); ws_base = nullptr; return false; }
+    void * fresh = nullptr;
+    if (hipMalloc(&fresh, 2 * want) != hipSuccess) { (void) hipGetLastError(); return false; }
+    bool ok = true;
+    if (ws_base) {
+        ok = hipMemcpyAsync(fresh, ws_base, ws_size, hipMemcpyDeviceToDevice, stream) == hipSuccess &&
+             hipMemcpyAsync((char *) fresh + want, (char *) ws_base + ws_size, ws_size, hipMemcpyDeviceToDevice, stream) == hipSuccess;
+    }
+    // the stream may still be reading the old block
+    ok = hipStreamSynchronize(stream) == hipSuccess && ok;
+    if (!ok) { (void) hipGetLastError(); (void) hipFree(fresh); return false; }
+    if (ws_base) (void) hipFree(ws_base);
+    ws_base = fresh;
     ws_size = want;
-    ws = ws_base;
+    ws = (char *) ws_base + (size_t) ws_slot * ws_size;
     return true;
 }
 
@@ -362,6 +371,13 @@ struct graph_runner {
                          memcmp(ctx->ws_x_nb, x->nb, sizeof(x->nb)) == 0;
         ctx->ws_x = x->data; ctx->ws_x_mode = mode; memcpy(ctx->ws_x_ne, x->ne, sizeof(x->ne)); memcpy(ctx->ws_x_nb, x->nb, sizeof(x->nb));
         cached_x = x;
+        if (!hit && ctx->image_only == x->data) {
+            // the producer of these activations wrote nothing but their image, and the image is gone: a planner error, not
+            // something to paper over with a conversion of memory that was never written
+            GGML_LOG_ERROR("ggml-mi355x: the activation image of %s was dropped before %s read it\n", x->name, c.mm->name);
+            status = MI355X_ERR_INVALID;
+            return -1;
+        }
         if (!hit) {
             mi355x_epilogue prep = c.epi;                 // same call as the product itself, stopped after the conversion
             prep.flags |= o.mm_flags | MI355X_MM_PREPARE_ONLY;
@@ -502,6 +518,9 @@ struct graph_runner {
         if (ready < 0) return c.used;
         epi.flags |= ready;
         if (key && ctx->ws_base) { epi.flags |= MI355X_EPI_EMIT_F16; epi.image = slot_ptr(ctx->ws_slot ^ 1); } else key = nullptr;
+        // ... and nothing else when the product that takes the image is the very next launch: the f32 values would have no reader
+        const bool image_only = key && ctx->dead_f32 && next_is_product_over(key, i + c.used);
+        if (image_only) epi.flags |= MI355X_EPI_IMAGE_ONLY;
         if (ctx->debug) {
             GGML_LOG_INFO("ggml-mi355x: %s %s [%lld x %lld x %lld] folds %d nodes, flags 0x%x\n", o.kernel_name, c.mm->name,
                           (long long) c.mm->ne[0], (long long) c.mm->ne[1], (long long) c.w->ne[0], c.used, epi.flags);
@@ -523,12 +542,12 @@ struct graph_runner {
             if (status == MI355X_ERR_UNSUPPORTED)       // (a K the tiles kernel is not built for)
             status = mi355x_mul_mat(&o.vw, &o.vx, &o.vd, epi.flags ? &epi : nullptr, ctx->ws, ctx->ws_size, ctx->stream);
             if (key && status == MI355X_ERR_UNSUPPORTED) {          // shapes the epilogue cannot emit for: plain product
-                epi.flags &= ~MI355X_EPI_EMIT_F16; key = nullptr;
+                epi.flags &= ~(MI355X_EPI_EMIT_F16 | MI355X_EPI_IMAGE_ONLY); key = nullptr;
                 status = mi355x_mul_mat(&o.vw, &o.vx, &o.vd, epi.flags ? &epi : nullptr, ctx->ws, ctx->ws_size, ctx->stream);
             }
         }
         note_write(c.out);
-        if (key && status == MI355X_OK) workspace_holds(key, ctx->ws_slot ^ 1);
+        if (key && status == MI355X_OK) { workspace_holds(key, ctx->ws_slot ^ 1); if (image_only) ctx->image_only = key->data; }
         return c.used;
     }
 
@@ -605,14 +624,18 @@ struct graph_runner {
         }
         const size_t image_bytes = mode == 1 ? (size_t)(out->ne[0] * out->ne[1] * 2) : (size_t)(out->ne[0] * out->ne[1] + out->ne[0] / 32 * out->ne[1] * 8);
         bool emit = key && ctx->reserve_workspace(image_bytes + 256);
+        // the image and nothing else when the product that takes it is the very next launch: the f32 rows would have no reader
+        const bool image_only = emit && mode == 1 && ctx->dead_f32 && next_is_product_over(key, i + used);
         {
-            launch_scope ls(ctx, used == 3 ? (emit ? "norm_affine_emit" : "norm_affine") : "norm", nbytes_of(nm->src[0]) + nbytes_of(out) + (emit ? image_bytes : 0), 0.0);
+            launch_scope ls(ctx, used == 3 ? (emit ? "norm_affine_emit" : "norm_affine") : "norm", nbytes_of(nm->src[0]) + (image_only ? 0 : nbytes_of(out)) + (emit ? image_bytes : 0), 0.0);
+            mi355x_tensor vo = vd;
+            if (image_only) vo.data = nullptr;
             status = !emit ? mi355x_norm(&vs, &vd, eps, w, b, ctx->stream)
-                   : mode == 1 ? mi355x_norm_emit_f16(&vs, &vd, eps, w, b, ctx->ws, ctx->stream) : mi355x_norm_emit_q8_0(&vs, &vd, eps, w, b, ctx->ws, ctx->stream);
+                   : mode == 1 ? mi355x_norm_emit_f16(&vs, &vo, eps, w, b, ctx->ws, ctx->stream) : mi355x_norm_emit_q8_0(&vs, &vd, eps, w, b, ctx->ws, ctx->stream);
         }
         if (emit && status == MI355X_ERR_UNSUPPORTED) { emit = false; status = mi355x_norm(&vs, &vd, eps, w, b, ctx->stream); }
         note_write(out);
-        if (emit && status == MI355X_OK) workspace_holds(key, ctx->ws_slot, mode);
+        if (emit && status == MI355X_OK) { workspace_holds(key, ctx->ws_slot, mode); if (image_only) ctx->image_only = key->data; }
         return used;
     }
 
@@ -630,6 +653,7 @@ struct graph_runner {
     // (mi355x_flash_attn_ext_cast_mask).  The f32 tensor is read in the launch that takes the cast's place, so the
     // allocator's reuse of its memory after the cast (ggml/src/ggml-alloc.c:640-667) is not a concern.
     const ggml_tensor * cast_dst = nullptr, * cast_src = nullptr;          // a cast that the next attention node carries out
+
     bool next_attention_casts(int i) const {
         const ggml_tensor * n = g->nodes[i], * s0 = n->src[0];
         if (!ctx->fuse || ctx->exact || (ctx->fa_accum & 2) || n->src[1] != n || s0->type != GGML_TYPE_F32 || n->type != GGML_TYPE_F16 ||
@@ -801,6 +825,7 @@ enum ggml_status mi355x_graph_compute(mi355x_backend_ctx * ctx, struct ggml_cgra
     } timer{ ctx, host_now_ns() };
     HIP_TRY(hipSetDevice(ctx->device), return GGML_STATUS_FAILED);
     ctx->ws_x = nullptr;   // tensors may have been rewritten between graphs
+    ctx->image_only = nullptr;
     { std::lock_guard<std::mutex> lock(ctx->mirror_mutex); ctx->mirror.clear(); }      // this graph may write anywhere in the compute buffer
     ctx->counters[0] += 1;
     ctx->counters[1] += cgraph->n_nodes;

@@ -113,7 +113,7 @@ __device__ __forceinline__ void patch_epilogue(float16_t v, const epi_args & e, 
     if (e.flags & MI355X_EPI_OUT_F16) {
 #pragma unroll
         for (int i = 0; i < 16; ++i) if (m_ok && n[i] < N) *(half_t *)(db + n[i] * d_nb1 + m * 2) = (half_t) v[i];
-    } else {
+    } else if (!EMIT || !(e.flags & MI355X_EPI_IMAGE_ONLY)) {
 #pragma unroll
         for (int i = 0; i < 16; ++i) if (m_ok && n[i] < N) *(float *)(db + n[i] * d_nb1 + m * 4) = v[i];
     }
@@ -1804,6 +1804,9 @@ extern "C" int mi355x_mul_mat(const mi355x_tensor * src0, const mi355x_tensor * 
     a.e.image = epi ? (half_t *) epi->image : nullptr;
     if (flags & MI355X_EPI_EMIT_F16) {
         if (!a.e.image || (flags & MI355X_EPI_OUT_F16)) return MI355X_ERR_INVALID;
+    }
+    if ((flags & MI355X_EPI_IMAGE_ONLY) && !(flags & MI355X_EPI_EMIT_F16)) return MI355X_ERR_INVALID;
+    if (flags & MI355X_EPI_EMIT_F16) {
         if (a.M % QK != 0 || dst->ne[2] * dst->ne[3] != 1 || mm_path(src0, src1) != MM_GEMM) return MI355X_ERR_UNSUPPORTED;
     }
 

@@ -59,7 +59,7 @@ __global__ void __launch_bounds__(ROWS_PER_BLOCK * WAVE) k_norm(tview s, tview d
                 float4 r = { v[j].x * scale, v[j].y * scale, v[j].z * scale, v[j].w * scale };
                 if (w) { r.x *= ww[j].x; r.y *= ww[j].y; r.z *= ww[j].z; r.w *= ww[j].w; }
                 if (b) { r.x += bb[j].x; r.y += bb[j].y; r.z += bb[j].z; r.w += bb[j].w; }
-                ((float4 *) y)[c] = r;
+                if (EMIT != 1 || d.p) ((float4 *) y)[c] = r;     // (EMIT == 1 without a destination: the image is all the caller wants)
                 if (EMIT) {                                // a 32-value block = 8 consecutive lanes (ne0 % 32 == 0: they are all here)
                     float amax = fmaxf(fmaxf(fabsf(r.x), fabsf(r.y)), fmaxf(fabsf(r.z), fabsf(r.w)));
                     amax = lanes_max<8>(amax);
