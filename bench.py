@@ -59,9 +59,9 @@ def model_file(arch: str, ftype: str) -> str:
 
 # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled by the same counters over a 256 MiB copy:
 # x2 KiB and x1 KiB), for the large-v3 encoder shapes; the summary with the commands is under profiles/
-# (mul_mat.gemm_q5_0 averages its two templates: 64 launches of 86.7 + 7.7 MB and 32 of 149.0 + 48.4 MB per window)
-MEASURED_TRAFFIC_MB = {"mul_mat.gemm_q5_0": (64 * (86.7 + 7.7) + 32 * (149.0 + 48.4)) / 96, "flash_attn.seq_tile": 70.9 + 11.5,
-                       "mul_mat.gemm_group": 143.4 + 23.1, "norm_affine_emit": 7.9 + 11.5}
+# (mul_mat.gemm_q5_0 averages its two templates: 64 launches of 59.9 + 7.7 MB and 32 of 45.1 + 15.4 MB per window)
+MEASURED_TRAFFIC_MB = {"mul_mat.gemm_q5_0": (64 * (59.9 + 7.7) + 32 * (45.1 + 15.4)) / 96, "flash_attn.seq_tile": 71.0 + 11.5,
+                       "mul_mat.gemm_group": 68.4 + 22.5, "norm_affine_emit": 7.9 + 3.8}
 
 # kernels that live on the matrix cores (bound "mfma"); everything else streams memory (bound "hbm")
 MFMA_KERNELS = ("mul_mat.gemm_", "flash_attn.seq_tile")
@@ -157,8 +157,9 @@ def main() -> int:
     if roofline and dom_name == "flash_attn.seq_tile":
         roofline["note"] = ("priced against the dense f16 matrix-core peak as the brief asks; the matrix cores only form the scores. "
                             "The reference accumulates V key by key in f16 (f32 fma, f16 store), and reproducing that takes 1.5 vector "
-                            "instructions per (query, key, d): 150 us per launch at the 2.0 ns per instruction the vector units sustain under this load, "
-                            "plus 60 us of score / factor phases that are vector work as well; that is the bound that applies")
+                            "instructions per (query, key, d): 135 us of issue per launch at the 2.05 GHz the part runs this kernel at, plus 27 us of "
+                            "factor computation and the rescales on the same vector units; that is the bound that applies, and the kernel runs at about "
+                            "70 % of it")
 
     # ---- and with f32 matrix-core attention (faster, but outside the whole-model parity bound: reported, never the headline) ----
     f32att = run_harness(["bench", "--model", enc_model, "--what", "encoder", "--backend", "gpu", "--reps", str(a.steps),
