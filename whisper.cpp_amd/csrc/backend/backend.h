@@ -101,7 +101,7 @@ struct mi355x_backend_ctx {
     void *       ws       = nullptr;   // the current slot (where the cached activation image lives)
     size_t       ws_size  = 0;         // bytes per slot
     int          ws_slot  = 0;
-    const void * image_only = nullptr; // activations whose producer wrote their image into the workspace and nothing else (this graph)
+    const void * image_only = nullptr; // the tensor (of this graph) whose producer wrote its image into the workspace and nothing else
     const void * ws_x     = nullptr;
     int          ws_x_mode = 0;
     int64_t      ws_x_ne[4] = {0, 0, 0, 0};

@@ -371,7 +371,7 @@ struct graph_runner {
                          memcmp(ctx->ws_x_nb, x->nb, sizeof(x->nb)) == 0;
         ctx->ws_x = x->data; ctx->ws_x_mode = mode; memcpy(ctx->ws_x_ne, x->ne, sizeof(x->ne)); memcpy(ctx->ws_x_nb, x->nb, sizeof(x->nb));
         cached_x = x;
-        if (!hit && ctx->image_only == x->data) {
+        if (!hit && ctx->image_only == (const void *) x) {
             // the producer of these activations wrote nothing but their image, and the image is gone: a planner error, not
             // something to paper over with a conversion of memory that was never written
             GGML_LOG_ERROR("ggml-mi355x: the activation image of %s was dropped before %s read it\n", x->name, c.mm->name);
@@ -547,7 +547,7 @@ struct graph_runner {
             }
         }
         note_write(c.out);
-        if (key && status == MI355X_OK) { workspace_holds(key, ctx->ws_slot ^ 1); if (image_only) ctx->image_only = key->data; }
+        if (key && status == MI355X_OK) { workspace_holds(key, ctx->ws_slot ^ 1); if (image_only) ctx->image_only = key; }
         return c.used;
     }
 
@@ -635,7 +635,7 @@ struct graph_runner {
         }
         if (emit && status == MI355X_ERR_UNSUPPORTED) { emit = false; status = mi355x_norm(&vs, &vd, eps, w, b, ctx->stream); }
         note_write(out);
-        if (emit && status == MI355X_OK) { workspace_holds(key, ctx->ws_slot, mode); if (image_only) ctx->image_only = key->data; }
+        if (emit && status == MI355X_OK) { workspace_holds(key, ctx->ws_slot, mode); if (image_only) ctx->image_only = key; }
         return used;
     }
 
