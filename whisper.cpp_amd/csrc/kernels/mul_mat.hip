@@ -292,7 +292,8 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 // What follows the K loop of a tile: GELU reads its table from LDS when the operand buffers, free now (the loop's last barrier
 // is behind every wavefront), are large enough to hold the part that matters (TABLE_FITS); then the 32x32 patches.
-template <int TI, int TJ, bool EMIT, bool TABLE_FITS>
+// (NT: threads of the workgroup; the patches belong to the first 256)
+template <int TI, int TJ, bool EMIT, bool TABLE_FITS, int NT = 256>
 __device__ __forceinline__ void gemm_tile_epilogue(float16_t (&acc)[TI][TJ], const mm_args & a, const epi_args & epi, char * db, int64_t batch_off, int64_t d_nb1,
                                                    int64_t n0, int64_t m0, int wn, int wmo, char * smem) {
     const int tid = threadIdx.x, lane = tid & 63, l32 = lane & 31, g = lane >> 5;
@@ -302,11 +303,12 @@ __device__ __forceinline__ void gemm_tile_epilogue(float16_t (&acc)[TI][TJ], con
             const u32x4 * pos = (const u32x4 *) epi.gelu, * neg = (const u32x4 *)(epi.gelu + 0x8000);
             u32x4 * dst = (u32x4 *) smem;
             constexpr int pieces = GELU_LDS_HALF * 2 / 16;
-            for (int p = tid; p < pieces; p += 256) { dst[p] = pos[p]; dst[pieces + p] = neg[p]; }
+            for (int p = tid; p < pieces; p += NT) { dst[p] = pos[p]; dst[pieces + p] = neg[p]; }
             __syncthreads();
             gelu_lds = (const uint16_t *) smem;
         }
     }
+    if (NT > 256 && tid >= 256) return;
     // accumulator register e of a 32x32 patch: row (= n) 8*(e/4) + 4*g + e%4, column (= m) lane%32
 #pragma unroll
     for (int i = 0; i < TI; ++i) {
@@ -472,6 +474,125 @@ __device__ __forceinline__ void gemm_f16_tile(const mm_args & a, int tiles_m, in
     }
 
     gemm_tile_epilogue<TI, TJ, EMIT, ((size_t) 2 * (BN + BM) * GB_LD * sizeof(half_t) >= GELU_LDS_BYTES)>(acc, a, epi, db, batch_off, d_nb1, n0, m0, wn, wmo, smem);
+}
+
+// The same tile by a workgroup of eight wavefronts in two roles: wavefronts 4 .. 7 move the operands (global loads into a
+// register ring, LDS stores of the step after next), wavefronts 0 .. 3 issue the matrix instructions of the current step,
+// one barrier per step between them.  In the one-role loop above a wavefront spends two thirds of a step issuing loads and
+// stores, during which it issues no matrix instruction; here the matrix wavefronts do nothing else, and a SIMD holds
+// one of each role per workgroup.  K a multiple of 64 S.
+// NP: threads that move operands (256 or 512), behind the 256 that multiply
+template <int TI, int TJ, int S, bool EMIT, int NP>
+__device__ __forceinline__ void gemm_f16_tile_rs(const mm_args & a, int tiles_m, int tiles_n, int sw, int tile, const char * wb, const char * xb, char * db,
+                                                 const epi_args & epi, int64_t batch_off, int64_t d_nb1) {
+    constexpr int BN = 64 * TI, BM = 64 * TJ;
+    constexpr int RP = NP / 8;                         // rows that the operand threads cover in one pass (8 threads to a row)
+    constexpr int XR = BN / RP, WR = BM / RP;          // 16-byte pieces per operand thread and step
+    static_assert(BN % RP == 0 && BM % RP == 0, "");
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    half_t * xs_base = (half_t *) smem;                // [2][BN * GB_LD]
+    half_t * ws_base = xs_base + 2 * BN * GB_LD;       // [2][BM * GB_LD]
+
+    const int per_col = sw * tiles_n, col = tile / per_col, rem = tile - col * per_col;
+    const int cw = min(sw, tiles_m - col * sw);
+    const int64_t m0 = (int64_t)(col * sw + rem % cw) * BM;
+    const int64_t n0 = (int64_t)(rem / cw) * BN;
+
+    const int tid = threadIdx.x;
+    const int KT = (int)(a.K / GB_K), last = KT - 1;
+    const int lane = tid & 63, wave = (tid >> 6) & 3;
+    const int wn = (wave >> 1) * 32 * TI, wmo = (wave & 1) * 32 * TJ;   // (matrix wavefronts) patch origin inside the tile
+
+    float16_t acc[TI][TJ];
+#pragma unroll
+    for (int i = 0; i < TI; ++i)
+#pragma unroll
+        for (int j = 0; j < TJ; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.0f;
+
+    if (tid >= 256) {
+        // ---- operand wavefronts
+        const int pt = tid - 256, lc = pt & 7, lr = pt >> 3;
+        const char * xp[XR]; const char * wp[WR];
+#pragma unroll
+        for (int i = 0; i < XR; ++i) { const int64_t n = n0 + lr + RP * i; xp[i] = xb + (n < a.N ? n : a.N - 1) * a.x_nb1 + lc * 16; }
+#pragma unroll
+        for (int i = 0; i < WR; ++i) { const int64_t m = m0 + lr + RP * i; wp[i] = wb + (m < a.M ? m : a.M - 1) * a.w_nb1 + lc * 16; }
+        u32x4 xrs[S][XR], wrs[S][WR];
+        auto load = [&](u32x4 (&xr)[XR], u32x4 (&wr)[WR], int64_t k0) __attribute__((always_inline)) {
+#pragma unroll
+            for (int i = 0; i < XR; ++i) xr[i] = *(const u32x4 *)(xp[i] + k0 * 2);
+#pragma unroll
+            for (int i = 0; i < WR; ++i) wr[i] = *(const u32x4 *)(wp[i] + k0 * 2);
+        };
+        auto store = [&](const u32x4 (&xr)[XR], const u32x4 (&wr)[WR], int buf) __attribute__((always_inline)) {
+            half_t * xs = xs_base + buf * BN * GB_LD, * ws = ws_base + buf * BM * GB_LD;
+#pragma unroll
+            for (int i = 0; i < XR; ++i) *(u32x4 *)(xs + (lr + RP * i) * GB_LD + 8 * lc) = xr[i];
+#pragma unroll
+            for (int i = 0; i < WR; ++i) *(u32x4 *)(ws + (lr + RP * i) * GB_LD + 8 * lc) = wr[i];
+        };
+        // every step loads unconditionally (beyond the end: the last step again), so the waits are counts, not vmcnt(0)
+#pragma unroll
+        for (int st = 0; st < S; ++st) load(xrs[st], wrs[st], (int64_t) min(st, last) * GB_K);
+        store(xrs[0], wrs[0], 0);
+        load(xrs[0], wrs[0], (int64_t) min(S, last) * GB_K);
+        __syncthreads();                               // step 0 is in LDS
+        auto step = [&](int kt, int buf, u32x4 (&xr)[XR], u32x4 (&wr)[WR]) __attribute__((always_inline)) {   // xr / wr: slot of step kt + 1
+            store(xr, wr, buf ^ 1);                     // the matrix wavefronts read `buf`; the readers of buf ^ 1 passed the last barrier
+            load(xr, wr, (int64_t) min(kt + 1 + S, last) * GB_K);
+            __syncthreads();
+        };
+        for (int kt0 = 0; kt0 < KT; kt0 += S) {
+            step(kt0 + 0, 0, xrs[1 % S], wrs[1 % S]);
+            step(kt0 + 1, 1, xrs[2 % S], wrs[2 % S]);
+            if (S > 2) { step(kt0 + 2, 0, xrs[3 % S], wrs[3 % S]); step(kt0 + 3, 1, xrs[4 % S], wrs[4 % S]); }
+        }
+    } else {
+        // ---- matrix wavefronts
+        const int l32 = lane & 31, g = lane >> 5;
+        auto mma = [&](int buf) __attribute__((always_inline)) {
+            const half_t * xs = xs_base + buf * BN * GB_LD + (wn  + l32) * GB_LD + 8 * g;
+            const half_t * ws = ws_base + buf * BM * GB_LD + (wmo + l32) * GB_LD + 8 * g;
+            // fragments of sub-step kk + 1 are read while the matrix cores work on kk (two sets of registers: with two
+            // workgroups to a CU a wavefront has 128)
+            half8_t av[2][TI], bv[2][TJ];
+#pragma unroll
+            for (int i = 0; i < TI; ++i) av[0][i] = *(const half8_t *)(xs + 32 * i * GB_LD);
+#pragma unroll
+            for (int j = 0; j < TJ; ++j) bv[0][j] = *(const half8_t *)(ws + 32 * j * GB_LD);
+#pragma unroll
+            for (int kk = 0; kk < GB_K / 16; ++kk) {
+                const int c = kk & 1, nx = c ^ 1;
+                if (kk + 1 < GB_K / 16) {
+#pragma unroll
+                    for (int i = 0; i < TI; ++i) av[nx][i] = *(const half8_t *)(xs + 32 * i * GB_LD + (kk + 1) * 16);
+#pragma unroll
+                    for (int j = 0; j < TJ; ++j) bv[nx][j] = *(const half8_t *)(ws + 32 * j * GB_LD + (kk + 1) * 16);
+                }
+#pragma unroll
+                for (int i = 0; i < TI; ++i)
+#pragma unroll
+                    for (int j = 0; j < TJ; ++j)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(av[c][i], bv[c][j], acc[i][j], 0, 0, 0);
+                if (kk + 1 < GB_K / 16) {
+#pragma unroll
+                    for (int r = 0; r < TI + TJ; ++r) {
+                        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // 1 MFMA
+                        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);   // 1 DS read
+                    }
+                }
+            }
+        };
+        __syncthreads();                               // step 0 is in LDS
+        for (int kt = 0; kt < KT; kt += 2) {            // (KT is even)
+            mma(0); __syncthreads();
+            mma(1); __syncthreads();
+        }
+    }
+    // all eight wavefronts are behind the last barrier: the operand buffers are free
+    gemm_tile_epilogue<TI, TJ, EMIT, ((size_t) 2 * (BN + BM) * GB_LD * sizeof(half_t) >= GELU_LDS_BYTES), 256 + NP>(acc, a, epi, db, batch_off, d_nb1, n0, m0, wn, wmo, smem);
 }
 
 // The same tile with the operands going from global memory straight into LDS (global_load_lds_dwordx4: lane l's 16 bytes
@@ -671,6 +792,36 @@ static int launch_gemm_f16_dl(const mm_args & a, hipStream_t st) {
     return launch_status();
 }
 
+// the two-role form (K a multiple of 64 S)
+template <int TI, int TJ, int S, bool EMIT, int NP>
+__global__ void __launch_bounds__(256 + NP) k_gemm_f16_rs(mm_args a, int tiles_m, int tiles_n, int sw) {
+    const int64_t b2 = blockIdx.y % a.ne12, b3 = blockIdx.y / a.ne12;
+    gemm_f16_tile_rs<TI, TJ, S, EMIT, NP>(a, tiles_m, tiles_n, sw, xcd_run_index(blockIdx.x, tiles_m * tiles_n),
+                                      a.w + (b2 / a.r2) * a.w_nb2 + (b3 / a.r3) * a.w_nb3, a.x + b2 * a.x_nb2 + b3 * a.x_nb3,
+                                      a.d + b2 * a.d_nb2 + b3 * a.d_nb3, a.e, b2 * a.d_nb2 + b3 * a.d_nb3, a.d_nb1);
+}
+template <int TI, int TJ> constexpr int rs_ring() { return 4; }
+#define RS_NP 512       // operand threads: 512 (three 16-byte pieces each per step of a 128 x 64 tile) beat 256 by 7 %
+
+template <int TI, int TJ, bool EMIT>
+static int launch_gemm_f16_rs(const mm_args & a, hipStream_t st) {
+    constexpr int BN = 64 * TI, BM = 64 * TJ, S = rs_ring<TI, TJ>();
+    constexpr size_t lds = (size_t) 2 * (BN + BM) * GB_LD * sizeof(half_t);
+    static bool configured[64];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return MI355X_ERR_HIP;
+    if (!configured[dev]) {
+        if (hipFuncSetAttribute((const void *) k_gemm_f16_rs<TI, TJ, S, EMIT, RS_NP>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds) != hipSuccess) return MI355X_ERR_HIP;
+        configured[dev] = true;
+    }
+    const int64_t tm = (a.M + BM - 1) / BM, tn = (a.N + BN - 1) / BN;
+    if (tm * tn > 0x7fffffff) return MI355X_ERR_UNSUPPORTED;
+    dim3 grid((unsigned)(tm * tn), (unsigned)(a.ne12 * a.ne13));
+    const int sw = tile_path_width(tm, tn, (tm * tn + 7) / 8, BN, BM);
+    k_gemm_f16_rs<TI, TJ, S, EMIT, RS_NP><<<grid, 256 + RS_NP, lds, st>>>(a, (int) tm, (int) tn, sw);
+    return launch_status();
+}
+
 template <int TI, int TJ, int S, bool KTAIL, bool FULL, bool EMIT = false>
 static int launch_gemm_f16_k(const mm_args & a, hipStream_t st) {
     static_assert(S % 2 == 0, "the LDS buffer index is the parity of the register slot");
@@ -693,6 +844,11 @@ static int launch_gemm_f16_k(const mm_args & a, hipStream_t st) {
 template <int TI, int TJ>
 static int launch_gemm_f16(const mm_args & a, hipStream_t st) {
     static const bool staged = getenv("MI355X_GEMM_STAGED") != nullptr;        // the register-staged loop, for comparison
+    // 128 x 64 tiles (one workgroup to a CU when M = 1280): two roles, 13.0 vs 14.9 us at K = 1280, 33.5 vs 39.9 us at K = 5120
+    if constexpr (TI * TJ == 2) {
+        if (!staged && a.K % (GB_K * rs_ring<TI, TJ>()) == 0)
+            return (a.e.flags & MI355X_EPI_EMIT_F16) ? launch_gemm_f16_rs<TI, TJ, true>(a, st) : launch_gemm_f16_rs<TI, TJ, false>(a, st);
+    }
     // 128 x 128 tiles only: the direct loads move about half the bytes per clock of the register path, which pays where two
     // workgroups share a CU (10 - 13 % faster) and loses on the 128 x 64 tiles that run one to a CU
     if constexpr (TI * TJ == 4) {
