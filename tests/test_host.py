@@ -29,6 +29,35 @@ def test_kernel_library_exports_every_declared_symbol(pkg):
     assert lib.mi355x_status_string(-1).decode().startswith("unsupported")
 
 
+def test_attention_refuses_a_mask_cast_that_shares_memory_with_its_output(pkg):
+    # mi355x_flash_attn_ext_cast_mask reads the f32 mask while workgroups that finish early already store dst, and writes the
+    # f16 copy on the way: the three may not overlap (ggml's allocator frees the f32 mask after the cast it replaces,
+    # ggml/src/ggml-alloc.c:612-667, and could hand its memory to the attention node's output).  The argument checks come
+    # before any HIP call, so plain addresses stand in for device memory here.
+    import ctypes as C
+    if not pkg.KERNELS_LIB.exists():
+        pytest.skip("kernel library not built")
+    lib = pkg.kernels()
+    n, h, kv = 5, 20, 64
+    class Mem:
+        def __init__(self, addr): self.addr = addr
+        def data_ptr(self): return self.addr
+    def tensors(mask32_at, mask16_at, dst_at):
+        q = pkg.tensor(Mem(0x10000000), pkg.F32, ne=[64, n, h], nb=[4, 256, 256 * n])
+        k = pkg.tensor(Mem(0x20000000), pkg.F16, ne=[64, kv, h], nb=[2, 128, 128 * kv])
+        v = pkg.tensor(Mem(0x30000000), pkg.F16, ne=[64, kv, h], nb=[2, 128, 128 * kv])
+        m32 = pkg.tensor(Mem(mask32_at), pkg.F32, ne=[kv, 8], nb=[4, 4 * kv])
+        m16 = pkg.tensor(Mem(mask16_at), pkg.F16, ne=[kv, 8], nb=[2, 2 * kv])
+        d = pkg.tensor(Mem(dst_at), pkg.F32, ne=[64, h, n], nb=[4, 256, 256 * h])
+        return q, k, v, m32, m16, d
+    def call(*at):
+        q, k, v, m32, m16, d = tensors(*at)
+        return lib.mi355x_flash_attn_ext_cast_mask(C.byref(q), C.byref(k), C.byref(v), C.byref(m32), C.byref(m16), C.byref(d), 0.125, pkg.FA_F16_SEQ, None, 0, None)
+    assert call(0x40000000, 0x40000000 + 512, 0x50000000) == -2        # the copy inside the f32 rows
+    assert call(0x40000000, 0x60000000, 0x40000000 + 256) == -2        # dst over the f32 mask
+    assert call(0x40000000, 0x60000000, 0x60000000) == -2              # dst over the f16 copy
+
+
 def test_plugin_exports_the_ggml_entry_points_and_does_not_link_the_checker(pkg):
     if not pkg.PLUGIN_LIB.exists():
         pytest.skip("plugin not built")
