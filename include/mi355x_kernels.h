@@ -71,6 +71,10 @@ enum mi355x_epilogue_flags {
                                   the src1 conversion pass of the MUL_MAT that reads dst next would produce            */
     MI355X_EPI_IMAGE_ONLY = 2048, /* with MI355X_EPI_EMIT_F16: write the image only, not dst (whose data pointer may then be
                                   NULL) — for a result whose only readers are products that take the image              */
+    MI355X_EPI_EMIT_Q8_0 = 4096, /* few-column path with a workspace, f32 dst with ne0 a multiple of 32, one product per call: also
+                                  write to `image` (16-byte aligned) dst quantized to Q8_0 as quantize_row_q8_0 does, in the
+                                  layout of mi355x_norm_emit_q8_0 for N rows of ne0 values — what the quantization pass of the
+                                  few-column MUL_MAT that reads dst next would write into its workspace                    */
     MI355X_MM_PREPARE_ONLY = 512, /* GEMM path: run only the src1 conversion pass into `workspace` and return; the
                                   product itself then follows in a second call with MI355X_MM_WS_READY (lets a
                                   caller time or overlap the two separately); a no-op on the other paths       */

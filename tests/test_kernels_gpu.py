@@ -437,6 +437,71 @@ def test_norm_mul_mat_group(pkg, oracle, gpu, wtype, n, k, m, count):
         assert lib.mi355x_norm_mul_mat_group(tl, tl, 1e-5, None, None, (pkg.MulMatItem * 1)(), 1, None, 0, gpu.stream) in (-1, -2)
 
 
+@pytest.mark.parametrize("wtype,n,k,m", [("Q8_0", 5, 1280, 5120), ("Q5_0", 3, 512, 384), ("Q8_0", 8, 384, 1536), ("Q8_0", 1, 1280, 5120)])
+def test_few_column_product_emits_its_result_as_q8_0(pkg, oracle, gpu, wtype, n, k, m):
+    # MI355X_EPI_EMIT_Q8_0: a decode step's FFN-up product (bias + GELU) leaves its rows quantized for FFN-down, in the layout
+    # the quantization pass of that product would write (quants | f16-rounded scales as f32 | block sums): through
+    # mi355x_mul_mat, mi355x_mul_mat_group with one product and mi355x_norm_mul_mat_group — the same bytes from all three
+    lib = pkg.kernels()
+    t = getattr(pkg, wtype)
+    x = rnd((n, k), 1.0)
+    blocks = oracle.quantize(t, rnd((m, k), 0.05))
+    bias = rnd((m,), 0.5)
+    d_x, d_w, d_b = gpu.up(x), gpu.up(blocks), gpu.up(bias)
+    tw, tx = pkg.tensor(d_w, t, ne=[k, m]), pkg.tensor(d_x, pkg.F32)
+    need = lib.mi355x_mul_mat_workspace_size(tw, tx)
+    img_bytes = n * m + n * (m // 32) * 8
+
+    def layout(image, y):
+        q = oracle.quantize(oracle.Q8_0, y, act=True).reshape(n, m // 32, 34)
+        assert np.array_equal(image[: n * m].reshape(n, m // 32, 32), q[:, :, 2:])
+        d = image[n * m: n * m + n * (m // 32) * 4].view(np.float32).reshape(n, m // 32)
+        assert np.array_equal(oracle.f32_to_f16_bits(d), q[:, :, :2].copy().view(np.uint16).reshape(n, m // 32))
+        sums = image[n * m + n * (m // 32) * 4: img_bytes].view(np.int32).reshape(n, m // 32)
+        assert np.array_equal(sums, q[:, :, 2:].view(np.int8).astype(np.int32).sum(axis=2))
+
+    def run(how):
+        d_y = torch.zeros((n, m), dtype=torch.float32, device=gpu.dev)
+        d_i = torch.zeros(img_bytes, dtype=torch.uint8, device=gpu.dev)
+        ws = torch.zeros(need, dtype=torch.uint8, device=gpu.dev)
+        epi = pkg.Epilogue()
+        epi.flags, epi.scale, epi.bias, epi.image = pkg.EPI_BIAS | pkg.EPI_GELU | pkg.EPI_EMIT_Q8_0, 1.0, d_b.data_ptr(), d_i.data_ptr()
+        ty = pkg.tensor(d_y, pkg.F32)
+        if how == "single":
+            pkg.check(lib.mi355x_mul_mat(tw, tx, ty, C.byref(epi), ws.data_ptr(), need, gpu.stream))
+        else:
+            items = (pkg.MulMatItem * 1)()
+            items[0].src0, items[0].dst, items[0].epi = C.pointer(tw), C.pointer(ty), C.pointer(epi)
+            if how == "group":
+                pkg.check(lib.mi355x_mul_mat_group(items, 1, tx, 0, ws.data_ptr(), need, gpu.stream))
+            else:                                      # behind a LayerNorm without affine vectors, normalized rows written in place of x
+                d_n = torch.zeros_like(d_x)
+                pkg.check(lib.mi355x_norm_mul_mat_group(tx, pkg.tensor(d_n, pkg.F32), 1e-5, None, None, items, 1, ws.data_ptr(), need, gpu.stream))
+                return gpu.down(d_y), gpu.down(d_i), gpu.down(d_n)
+        return gpu.down(d_y), gpu.down(d_i)
+
+    y, image = run("single")
+    assert oracle.nmse(y, oracle.gelu(oracle.mul_mat(t, blocks, x) + bias)) <= 1e-9
+    layout(image, y)
+    y2, image2 = run("group")
+    assert np.array_equal(y2, y) and np.array_equal(image2, image)
+    y3, image3, rows = run("norm")
+    assert oracle.nmse(rows, oracle.norm(x, 1e-5)) <= 1e-10
+    # (a sum that lands on the other side of an f16 boundary moves its GELU table entry by one f16 step: 1e-9, not 1e-10)
+    assert oracle.nmse(y3, oracle.gelu(oracle.mul_mat(t, blocks, rows) + bias)) <= 1e-9
+    layout(image3, y3)
+    # not for more than one product per launch, not for many columns, not without a workspace
+    epi = pkg.Epilogue(); epi.flags, epi.image = pkg.EPI_EMIT_Q8_0, d_x.data_ptr()
+    d_y = torch.zeros((n, m), dtype=torch.float32, device=gpu.dev)
+    ty = pkg.tensor(d_y, pkg.F32)
+    assert lib.mi355x_mul_mat(tw, tx, ty, C.byref(epi), None, 0, gpu.stream) == -1
+    items = (pkg.MulMatItem * 2)()
+    for i in range(2):
+        items[i].src0, items[i].dst, items[i].epi = C.pointer(tw), C.pointer(ty), C.pointer(epi)
+    ws = torch.zeros(need, dtype=torch.uint8, device=gpu.dev)
+    assert lib.mi355x_mul_mat_group(items, 2, tx, 0, ws.data_ptr(), need, gpu.stream) == -1
+
+
 def test_mul_mat_rejects_bad_arguments(pkg, gpu):
     lib = pkg.kernels()
     d_w = torch.zeros(22 * 4, dtype=torch.uint8, device=gpu.dev)

@@ -24,7 +24,7 @@ BLOCK_BYTES = {Q5_0: 22, Q8_0: 34}
 
 # enum mi355x_epilogue_flags
 EPI_BIAS, EPI_GELU, EPI_SCALE, EPI_RESIDUAL, EPI_BIAS_COL, EPI_OUT_F16 = 1, 2, 4, 8, 16, 32
-MM_EXACT_ACT, MM_WS_READY, MM_ACT_Q8_0, MM_PREPARE_ONLY, EPI_EMIT_F16, EPI_IMAGE_ONLY = 64, 128, 256, 512, 1024, 2048
+MM_EXACT_ACT, MM_WS_READY, MM_ACT_Q8_0, MM_PREPARE_ONLY, EPI_EMIT_F16, EPI_IMAGE_ONLY, EPI_EMIT_Q8_0 = 64, 128, 256, 512, 1024, 2048, 4096
 MUL_MAT_NOALLOC_MAX = 32 << 20
 # enum mi355x_fa_mode
 FA_F16_SEQ, FA_F32, FA_EMIT_F16, FA_EMIT_Q8_0 = 0, 1, 0x100, 0x200

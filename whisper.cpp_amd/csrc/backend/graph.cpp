@@ -468,12 +468,27 @@ struct graph_runner {
             flops += chain_flops(chains[k]); bytes += chain_bytes(chains[k]) - (k ? nbytes_of(first.x) : 0.0);
         }
         if (with_norm) {
-            if (!ctx->reserve_workspace(need)) { status = MI355X_ERR_WORKSPACE; return end - i; }
+            // A single product whose result (the FFN's first matrix with its GELU) feeds nothing but the few-column product that
+            // is launched next also leaves it quantized to Q8_0, in the other workspace slot: that product's quantization pass —
+            // a launch on the step's critical path — is not needed then.
+            const ggml_tensor * q8_key = nullptr;
+            size_t need_all = need;
+            if (chains.size() == 1 && !(chains[0].epi.flags & MI355X_EPI_OUT_F16) && chains[0].out->ne[0] % 32 == 0) {
+                q8_key = image_consumer(chains[0].out, end, true);
+                if (q8_key && !next_is_product_over(q8_key, end)) q8_key = nullptr;
+                if (q8_key) need_all = std::max(need, (size_t)(chains[0].out->ne[0] * chains[0].out->ne[1] + chains[0].out->ne[0] / 32 * chains[0].out->ne[1] * 8) + 256);
+            }
+            if (!ctx->reserve_workspace(need_all)) { status = MI355X_ERR_WORKSPACE; return end - i; }
             mi355x_tensor vs = to_view(held.src), vn = to_view(held.out);
             int rc;
             {
                 launch_scope ls(ctx, "norm_mul_mat.gemv", bytes + nbytes_of(held.src) + nbytes_of(held.out), flops);
+                if (q8_key) { chains[0].epi.flags |= MI355X_EPI_EMIT_Q8_0; chains[0].epi.image = slot_ptr(ctx->ws_slot ^ 1); }
                 rc = mi355x_norm_mul_mat_group(&vs, &vn, held.eps, held.w, held.b, items.data(), (int) items.size(), ctx->ws, ctx->ws_size, ctx->stream);
+                if (rc == MI355X_ERR_UNSUPPORTED && q8_key) {
+                    chains[0].epi.flags &= ~MI355X_EPI_EMIT_Q8_0; chains[0].epi.image = nullptr; q8_key = nullptr;
+                    rc = mi355x_norm_mul_mat_group(&vs, &vn, held.eps, held.w, held.b, items.data(), (int) items.size(), ctx->ws, ctx->ws_size, ctx->stream);
+                }
             }
             if (rc == MI355X_ERR_UNSUPPORTED) return 0;      // the caller lets the LayerNorm run on its own and takes the usual path
             held.active = false;
@@ -481,6 +496,7 @@ struct graph_runner {
             note_write(held.out);
             if (rc == MI355X_OK) workspace_holds(held.key, ctx->ws_slot, 2);
             for (const mm_chain & c : chains) note_write(c.out);
+            if (rc == MI355X_OK && q8_key) workspace_holds(q8_key, ctx->ws_slot ^ 1, 2);       // (after note_write: the image is of what was just written)
             return end - i;
         }
         const int ready = prepare_src1(first, o0, need, status);

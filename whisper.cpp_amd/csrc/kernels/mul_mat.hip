@@ -1144,9 +1144,19 @@ __device__ __forceinline__ void gemv_qr_rows(const mm_args & a, PRO prologue = P
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int j = lane % LPR, r = lane / LPR;
     const int64_t n_groups = (a.M + 4 * RPW - 1) / (4 * RPW);
-    int64_t group = blockIdx.x;
+    // MI355X_EPI_EMIT_Q8_0: the results are also left quantized to Q8_0 for the product that reads them next.  A Q8_0 block is
+    // 32 consecutive rows, GPB groups of this kernel, so the groups are then dealt in runs (workgroup b: groups b T .. b T + T - 1,
+    // T a multiple of GPB) instead of round-robin, the results of a block meet in LDS and the workgroup rounds them.
+    constexpr int GPB = QK / (4 * RPW);
+    const bool emit_q8 = (a.e.flags & MI355X_EPI_EMIT_Q8_0) != 0;                          // uniform
+    const int64_t run = emit_q8 ? GPB * ((n_groups + (int64_t) GPB * gridDim.x - 1) / ((int64_t) GPB * gridDim.x)) : 0;
+    const int64_t group_end = emit_q8 ? (n_groups < (blockIdx.x + 1) * run ? n_groups : (blockIdx.x + 1) * run) : n_groups;
+    const int64_t group_step = emit_q8 ? 1 : gridDim.x;
+    __shared__ float q8_rows[MI355X_GEMV_MAX_COLS][QK];
+    int64_t group = emit_q8 ? blockIdx.x * run : blockIdx.x;
+    const bool idle = emit_q8 && group >= group_end;    // (a grid larger than the runs need: such a workgroup walks one group without storing)
     int64_t row = group * (4 * RPW) + wave * RPW + r;
-    bool row_ok = row < a.M;
+    bool row_ok = row < a.M && !idle;
     const uint8_t * wrow = (const uint8_t *) a.w + (row_ok ? row : 0) * a.w_nb1;
 
     // a lane whose block index lies beyond the row reads the row's last block again and counts it with a zero scale
@@ -1212,8 +1222,9 @@ __device__ __forceinline__ void gemv_qr_rows(const mm_args & a, PRO prologue = P
 #pragma unroll
         for (int n = 0; n < NC; ++n) { o_bcol[n] = e_bcol[n]; o_res[n] = e_res[n]; }
         // the next row's blocks and epilogue operands travel while this row is worked on
-        group += gridDim.x;
-        const bool more = group < n_groups;                 // uniform
+        const int64_t done_group = group;
+        group += group_step;
+        const bool more = group < group_end;                // uniform
         if (more) {
             row = group * (4 * RPW) + wave * RPW + r;
             row_ok = row < a.M;
@@ -1260,7 +1271,29 @@ __device__ __forceinline__ void gemv_qr_rows(const mm_args & a, PRO prologue = P
                 if (a.e.flags & MI355X_EPI_RESIDUAL) v += o_res[n];
                 if (out_f16) *(half_t *)(a.d + n * a.d_nb1 + done_row * 2) = (half_t) v;
                 else         *(float  *)(a.d + n * a.d_nb1 + done_row * 4) = v;
+                if (emit_q8) q8_rows[n][(int)(done_group % GPB) * (4 * RPW) + wave * RPW + r] = v;
             }
+        }
+        if (emit_q8 && ((done_group % GPB) == GPB - 1 || !more)) {          // uniform: a block of 32 rows is complete (M % 32 == 0)
+            // thread (column n, row rr of the block): rounding as quantize_row_q8_0 (ggml-cpu-quants.c:808-865), into the layout of
+            // k_quantize_x_q8 for NC rows of M values
+            __syncthreads();
+            const int n = threadIdx.x >> 5, rr = threadIdx.x & 31;
+            const float v = n < NC ? q8_rows[n][rr] : 0.0f;
+            const float amax = lanes_max<32>(fabsf(v));
+            const float id = amax != 0.0f ? 127.0f / amax : 0.0f;
+            const int q = (int) rintf(v * id);
+            const int qsum = lanes_sum<32>(q);
+            if (n < NC && !idle) {
+                char * img = (char *) a.e.image;
+                const int64_t bi = done_group / GPB, nb2 = a.M / QK;
+                ((int8_t *) img)[n * a.M + bi * QK + rr] = (int8_t) q;
+                if (rr == 0) {
+                    ((float *)(img + (size_t) NC * a.M))[n * nb2 + bi] = h2f(f2h_bits(amax / 127.0f));
+                    ((int32_t *)(img + (size_t) NC * a.M + (size_t) NC * nb2 * 4))[n * nb2 + bi] = qsum;
+                }
+            }
+            __syncthreads();
         }
         if (!more) break;
     }
@@ -1619,8 +1652,12 @@ static int launch_gemv_r_nb(const mm_args & a, int nb, unsigned grid, const gemv
 }
 template <int T0, int NC>
 static int launch_gemv_r(const mm_args & a, hipStream_t st, const gemv_group * grp = nullptr, int count = 1, const gemv_norm_args * nm = nullptr) {
-    const int lpr = gemv_r_lanes(a.M * count, NC, a.K);
+    int lpr = gemv_r_lanes(a.M * count, NC, a.K);
     if (!lpr) return MI355X_ERR_UNSUPPORTED;
+    // with the Q8_0 emission a workgroup owns whole blocks of 32 rows, so there are M / 32 workgroups at most: the fewer lanes a
+    // row takes, the fewer groups each of them walks one after the other
+    const bool emit_q8 = ((grp ? grp->e[0].flags : a.e.flags) & MI355X_EPI_EMIT_Q8_0) != 0;
+    if (emit_q8 && (a.K / QK + 15) / 16 <= 3 && (a.K / QK + 15) / 16 * NC <= 15) lpr = 16;
     const int nb = (int)((a.K / QK + lpr - 1) / lpr);
     const int rows_per_wg = 4 * (WAVE / lpr);
     const int64_t n_groups = (a.M + rows_per_wg - 1) / rows_per_wg;
@@ -1759,12 +1796,17 @@ static int mul_mat_group_gemv(const mi355x_mul_mat_item * items, int count, cons
         if (!w || !d) return MI355X_ERR_INVALID;
         if (w->type != w0->type || w->ne[0] != a.K || w->ne[1] != a.M || w->ne[2] != 1 || w->ne[3] != 1 || w->nb[1] != w0->nb[1] || (uintptr_t) w->data % 2 != 0) return MI355X_ERR_UNSUPPORTED;
         if (e && (e->flags & MI355X_EPI_EMIT_F16)) return MI355X_ERR_UNSUPPORTED;
-        const int ef = e ? (e->flags & 63) : 0;
+        int ef = e ? (e->flags & 63) : 0;
         const int td = (ef & MI355X_EPI_OUT_F16) ? MI355X_TYPE_F16 : MI355X_TYPE_F32;
         if (d->type != td || d->ne[0] != a.M || d->ne[1] != a.N || d->ne[2] != 1 || d->ne[3] != 1 || d->nb[0] != type_size(td)) return MI355X_ERR_UNSUPPORTED;
         if ((ef & (MI355X_EPI_BIAS | MI355X_EPI_BIAS_COL)) && !e->bias) return MI355X_ERR_INVALID;
         if ((ef & MI355X_EPI_BIAS) && (ef & MI355X_EPI_BIAS_COL)) return MI355X_ERR_INVALID;
         if ((ef & MI355X_EPI_RESIDUAL) && (!e->residual || (ef & MI355X_EPI_OUT_F16))) return MI355X_ERR_INVALID;
+        if (e && (e->flags & MI355X_EPI_EMIT_Q8_0)) {           // the result also as Q8_0: one product per launch, whole blocks
+            if (count != 1 || (ef & MI355X_EPI_OUT_F16) || a.M % QK != 0) return MI355X_ERR_UNSUPPORTED;
+            if (!e->image || (uintptr_t) e->image % 16 != 0) return MI355X_ERR_INVALID;
+            ef |= MI355X_EPI_EMIT_Q8_0;
+        }
         any_gelu = any_gelu || (ef & MI355X_EPI_GELU);
         grp.e[i] = { (const char *) w->data, (char *) d->data, e ? (const float *) e->bias : nullptr, e ? (const char *) e->residual : nullptr, (int64_t) d->nb[1], ef, e ? e->scale : 1.0f };
     }
@@ -1773,7 +1815,8 @@ static int mul_mat_group_gemv(const mi355x_mul_mat_item * items, int count, cons
     a.x_nb1 = src1->nb[1]; a.x_nb2 = a.x_nb3 = 0;
     a.d_nb1 = items[0].dst->nb[1]; a.d_nb2 = a.d_nb3 = 0;
     a.ne12 = a.ne13 = a.r2 = a.r3 = 1;
-    a.e.flags = 0; a.e.scale = 1.0f; a.e.bias = nullptr; a.e.residual = nullptr; a.e.gelu = nullptr; a.e.image = nullptr;
+    a.e.flags = 0; a.e.scale = 1.0f; a.e.bias = nullptr; a.e.residual = nullptr; a.e.gelu = nullptr;
+    a.e.image = (grp.e[0].flags & MI355X_EPI_EMIT_Q8_0) ? (half_t *) items[0].epi->image : nullptr;
     if (any_gelu && !(a.e.gelu = gelu_table_device())) return MI355X_ERR_HIP;
     hipStream_t st = (hipStream_t) stream;
     if (nm) {                                               // the LayerNorm in front, in the same launch: it writes src1 and the workspace
@@ -1962,6 +2005,11 @@ extern "C" int mi355x_mul_mat(const mi355x_tensor * src0, const mi355x_tensor * 
         if (!a.e.image || (flags & MI355X_EPI_OUT_F16)) return MI355X_ERR_INVALID;
     }
     if ((flags & MI355X_EPI_IMAGE_ONLY) && !(flags & MI355X_EPI_EMIT_F16)) return MI355X_ERR_INVALID;
+    if (flags & MI355X_EPI_EMIT_Q8_0) {                       // the register kernel of the few-column path only
+        if (!a.e.image || (uintptr_t) a.e.image % 16 != 0 || (flags & (MI355X_EPI_OUT_F16 | MI355X_EPI_EMIT_F16))) return MI355X_ERR_INVALID;
+        const size_t ws_need = gemv_ws_bytes(src0, src1);
+        if (a.M % QK != 0 || mm_path(src0, src1) != MM_GEMV || !ws_need || !workspace || workspace_size < ws_need || (uintptr_t) workspace % 16 != 0) return MI355X_ERR_UNSUPPORTED;
+    }
     if (flags & MI355X_EPI_EMIT_F16) {
         if (a.M % QK != 0 || dst->ne[2] * dst->ne[3] != 1 || mm_path(src0, src1) != MM_GEMM) return MI355X_ERR_UNSUPPORTED;
     }
