@@ -84,13 +84,13 @@ def test_every_node_of_the_whisper_graphs(harness, models, key):
 def test_whisper_full_end_to_end(harness, models):
     # whisper_full() unmodified: PCM -> log-mel -> encoder -> whisper's own search (logits filters, timestamp rules, KV-cache
     # bookkeeping), on both backends over the same synthetic audio.  Greedy: the transcripts must start with the same ids
-    # (they were identical over all 42 tokens when this was written).  Beam search draws its candidates from the softmax
+    # (they were identical over all 42 tokens when this was written, and 32 are asked for).  Beam search draws its candidates from the softmax
     # with a seeded RNG (src/whisper.cpp:5415-5418); on a random-init model's near-flat distribution the cumulative sums the
     # draw walks move by more than one token's width with any rounding difference, so only "runs and returns text" is asserted.
     rc, rows = run_harness(harness, ["full", "--model", models[("base", "q5_0")], "--beam", "1", "--max-tokens", "24"], timeout=900)
     s = rows[-1]
     assert rc == 0 and s["pass"] and s["gpu_rc"] == 0 and s["gpu_tokens"] > 0, s
-    assert s["common_prefix"] >= min(8, s["cpu_tokens"]), s
+    assert s["common_prefix"] >= min(32, s["cpu_tokens"]), s          # (42 of 42 on every tree so far)
     rc, rows = run_harness(harness, ["full", "--model", models[("base", "q5_0")], "--beam", "5", "--max-tokens", "24"], timeout=900)
     s = rows[-1]
     assert rc == 0 and s["pass"] and s["gpu_rc"] == 0 and s["gpu_tokens"] > 0 and s["gpu_segments"] > 0, s
@@ -103,7 +103,7 @@ def test_whisper_full_from_the_device_log_mel(harness, models):
     rc, rows = run_harness(harness, ["full", "--model", models[("base", "q5_0")], "--beam", "1", "--max-tokens", "24", "--gpu-mel"], timeout=900)
     s = rows[-1]
     assert rc == 0 and s["pass"] and s["gpu_mel"] and s["gpu_rc"] == 0 and s["gpu_tokens"] > 0 and s["gpu_mel_ms"] > 0, s
-    assert s["common_prefix"] >= min(8, s["cpu_tokens"]), s
+    assert s["common_prefix"] >= min(24, s["cpu_tokens"]), s
 
 
 def test_whisper_full_parallel_states_share_one_device(harness, models):
