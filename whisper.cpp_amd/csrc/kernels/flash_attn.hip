@@ -683,10 +683,17 @@ __global__ void __launch_bounds__(512, 2) k_fattn_seq_tile(fa_args a) {
                     const float s = sv[i];
                     const bool  raised = s > M;
                     const float ex = exp_neg(-fabsf(s - M));   // M - s when raised, s - M otherwise: both <= 0 (or NaN / -inf: 0)
-                    const float ms = raised ? ex : 1.0f, vs = raised ? 1.0f : ex;
-                    M = raised ? s : M;
-                    P *= ms; A = A * ms + vs;
-                    sv[i] = raised ? -ex : ex;                 // -0.0 keeps the sign
+                    if (__any(raised)) {
+                        const float ms = raised ? ex : 1.0f, vs = raised ? 1.0f : ex;
+                        M = raised ? s : M;
+                        P *= ms; A = A * ms + vs;
+                        sv[i] = raised ? -ex : ex;             // -0.0 keeps the sign
+                    } else {
+                        // no query of this wavefront has a new maximum at this key (nine keys in ten, past the first tiles):
+                        // ms = 1 leaves M and P as they are and A * 1 + vs is A + vs, bit for bit
+                        A = A + ex;
+                        sv[i] = ex;
+                    }
                 }
 #pragma unroll
                 for (int i = 0; i < 4; ++i) fp[i] = make_float4(sv[4*i], sv[4*i+1], sv[4*i+2], sv[4*i+3]);
