@@ -66,6 +66,14 @@ def test_op_cases_in_exact_mode_still_meet_the_per_op_bound(harness):
     assert cases and all(r["pass"] for r in cases)
 
 
+def test_register_staged_gemm_loop_still_passes_every_mul_mat_case(harness):
+    # MI355X_GEMM_STAGED=1 puts the many-column products back on the register-staged K loop (the default is direct-to-LDS loads
+    # on 128 x 128 tiles and the two-role workgroup on 128 x 64 tiles): kept for comparison, so kept correct
+    rc, rows = run_harness(harness, ["ops", "--reps", "0", "--filter", "mul_mat"], env={"MI355X_GEMM_STAGED": "1"}, timeout=900)
+    cases = [r for r in rows if "case" in r]
+    assert rc == 0 and len(cases) >= 20 and all(r["pass"] for r in cases), [r for r in cases if not r["pass"]]
+
+
 def test_unfused_graphs_match_fused_ones(harness, models):
     for env in ({"GGML_MI355X_FUSE": "0"}, {}):
         rc, rows = run_harness(harness, ["model", "--model", models[("base", "q5_0")], "--steps", "4"], env=env, timeout=900)
