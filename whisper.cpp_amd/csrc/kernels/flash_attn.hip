@@ -578,7 +578,13 @@ __global__ void __launch_bounds__(512, 2) k_fattn_seq_tile(fa_args a) {
 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int64_t n0 = (int64_t) blockIdx.x * T_Q, h = blockIdx.y, i3 = blockIdx.z;
+    // Workgroups go round-robin to the 8 XCDs, each with an L2 of its own.  The query tiles of one head all read that head's K
+    // and V (384 KB for 1500 keys), so every XCD gets one run of consecutive (head, query tile) pairs, head-major: a head's
+    // K and V are then fetched into one or two L2s instead of all eight.
+    const uint32_t lin = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z), total = gridDim.x * gridDim.y * gridDim.z;
+    const uint32_t xcd = lin % 8, per = total / 8, extra = total % 8;
+    const uint32_t item = xcd * per + (xcd < extra ? xcd : extra) + lin / 8;
+    const int64_t n0 = (int64_t)(item % gridDim.x) * T_Q, h = (item / gridDim.x) % gridDim.y, i3 = item / (gridDim.x * gridDim.y);
     const int n_tiles = (int)((a.KV + T_KV - 1) / T_KV);
 
     if (wave >= 4) {
