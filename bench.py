@@ -122,6 +122,51 @@ def read_yardstick(nbytes: int) -> dict:
     return best
 
 
+def gemm_library_yardstick() -> list | None:
+    """the encoder's four product shapes (1500 activation rows) as plain f16 x f16 products, 50 launches back to back between
+    one pair of HIP events: this library (f32 result) beside torch.mm (the vendor BLAS behind it, f16 result) on the same
+    operands.  A yardstick for what the part does on these shapes, not part of any timed leg; no product path uses it."""
+    try:
+        sys.path.insert(0, str(ROOT))
+        import ctypes as C
+        import torch
+        import __graft_entry__ as entry
+        pkg = entry.package()
+        lib = pkg.kernels()
+        dev = torch.device("cuda:0")
+
+        def timed(fn, reps=50):
+            for _ in range(5):
+                fn()
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(reps):
+                fn()
+            e1.record()
+            torch.cuda.synchronize()
+            return e0.elapsed_time(e1) / reps * 1e3
+
+        rows = []
+        for what, m, k in (("ffn up", 5120, 1280), ("ffn down", 1280, 5120), ("attention out", 1280, 1280), ("q, k, v as one matrix", 3840, 1280)):
+            n = 1500
+            w = (torch.randn(m, k, device=dev) * 0.05).half()
+            x = torch.randn(n, k, device=dev).half()
+            d = torch.empty(n, m, device=dev)
+            tw, tx, td = pkg.tensor(w, pkg.F16), pkg.tensor(x, pkg.F16), pkg.tensor(d, pkg.F32)
+            ours = timed(lambda: pkg.check(lib.mi355x_mul_mat(C.byref(tw), C.byref(tx), C.byref(td), None, None, 0, None)))
+            out16, wt = torch.empty(n, m, device=dev, dtype=torch.half), w.t()
+            blas = timed(lambda: torch.mm(x, wt, out=out16))
+            gflop = 2.0 * m * n * k / 1e9
+            rows.append({"shape": what, "m": m, "n": n, "k": k, "this_library_us": round(ours, 2), "vendor_blas_us": round(blas, 2),
+                         "this_library_tflops": round(gflop / ours * 1e3, 1), "vendor_blas_tflops": round(gflop / blas * 1e3, 1),
+                         "vendor_blas_frac_of_peak": round(gflop / blas * 1e3 / PEAK_MFMA_F16_TFLOPS, 4)})
+        return rows
+    except Exception as e:                                 # a yardstick: its absence must not fail the bench
+        print(f"bench.py: gemm_library_yardstick skipped: {e}", file=sys.stderr)
+        return None
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -249,6 +294,7 @@ def main() -> int:
         "kernel_breakdown": breakdown,
         "roofline": roofline,
         "kernel_rooflines": [r for r in rooflines.values() if r["launches"] / enc["profile_reps"] >= 30],
+        "gemm_library_yardstick": gemm_library_yardstick(),
         "cpu_baseline": cpu_baseline,
     }
     print(json.dumps(out))

@@ -302,11 +302,12 @@ def test_mul_mat_epilogue_emits_the_next_products_activation_image(pkg, oracle, 
     assert lib.mi355x_mul_mat(tw, pkg.tensor(d_x5, pkg.F32), pkg.tensor(d_y5, pkg.F32), C.byref(epi), ws.data_ptr(), need, gpu.stream) == -1
 
 
-def test_mul_mat_group_equals_single_calls(pkg, oracle, gpu):
+@pytest.mark.parametrize("k,m,n", [(512, 384, 200), (1280, 1280, 1500)])
+def test_mul_mat_group_equals_single_calls(pkg, oracle, gpu, k, m, n):
     # three products over the same activations (the shape of a layer's Q, K, V projections) as one launch: same bits as
-    # three calls, each with its own epilogue and destination type
+    # three calls, each with its own epilogue and destination type.  The second case is a large-v3 encoder layer's, which
+    # the grouped form runs on 128 x 192 tiles (one workgroup to a CU) with a partial last tile column.
     lib = pkg.kernels()
-    k, m, n = 512, 384, 200
     x = rnd((n, k))
     d_x = gpu.up(x)
     tx = pkg.tensor(d_x, pkg.F32)
