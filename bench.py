@@ -175,6 +175,14 @@ def gemm_library_yardstick() -> list | None:
             rows.append({"shape": what, "m": m, "n": n, "k": k, "this_library_us": round(ours, 2), "vendor_blas_us": round(blas, 2),
                          "this_library_tflops": round(gflop / ours * 1e3, 1), "vendor_blas_tflops": round(gflop / blas * 1e3, 1),
                          "vendor_blas_frac_of_peak": round(gflop / blas * 1e3 / PEAK_MFMA_F16_TFLOPS, 4)})
+        # the matrix instruction by itself: v_mfma_f32_32x32x16_f16 from registers, one and four wavefronts per SIMD
+        sink = torch.zeros(1, device=dev)
+        for wgs in (256, 1024):
+            iters = 20000
+            us = timed(lambda: pkg.check(lib.mi355x_mfma_probe(iters, wgs, sink.data_ptr(), None)), reps=5)
+            tf = wgs * 4 * 4 * iters * 32768.0 / us / 1e6
+            rows.append({"shape": f"matrix instruction from registers, {wgs // 256} wavefront(s) per SIMD", "us": round(us, 1),
+                         "tflops": round(tf, 1), "frac_of_peak": round(tf / PEAK_MFMA_F16_TFLOPS, 4)})
         return rows
     except Exception as e:                                 # a yardstick: its absence must not fail the bench
         print(f"bench.py: gemm_library_yardstick skipped: {e}", file=sys.stderr)

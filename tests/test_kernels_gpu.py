@@ -972,3 +972,19 @@ def test_log_mel_properties_and_arguments(pkg, oracle, gpu):
     assert lib.mi355x_log_mel_spectrogram(d.data_ptr(), 200, d.data_ptr(), 80, d.data_ptr(), d.data_ptr(), 4096, gpu.stream) == -2
     assert lib.mi355x_log_mel_spectrogram(d.data_ptr(), 1000, d.data_ptr(), 129, d.data_ptr(), d.data_ptr(), 4096, gpu.stream) == -1
     assert lib.mi355x_log_mel_spectrogram(d.data_ptr(), 1000, d.data_ptr(), 80, d.data_ptr(), None, 0, gpu.stream) == -3
+
+
+def test_measurement_probes_run_and_reject_bad_arguments(pkg, gpu):
+    # the two yardstick kernels of the benchmark: a bare read stream and the matrix instruction from registers
+    lib = pkg.kernels()
+    out = torch.zeros(4, dtype=torch.int32, device=gpu.dev)
+    buf = torch.zeros(1 << 20, dtype=torch.uint8, device=gpu.dev)
+    pkg.check(lib.mi355x_read_probe(buf.data_ptr(), buf.numel(), out.data_ptr(), 64, gpu.stream))
+    pkg.check(lib.mi355x_mfma_probe(100, 256, out.data_ptr(), gpu.stream))
+    torch.cuda.synchronize()
+    assert int(out.abs().sum()) == 0                       # neither writes its sink
+    assert lib.mi355x_mfma_probe(0, 256, out.data_ptr(), gpu.stream) == -2
+    assert lib.mi355x_mfma_probe(100, 0, out.data_ptr(), gpu.stream) == -2
+    assert lib.mi355x_mfma_probe(100, 256, None, gpu.stream) == -2
+    assert lib.mi355x_read_probe(None, 16, out.data_ptr(), 64, gpu.stream) == -2
+

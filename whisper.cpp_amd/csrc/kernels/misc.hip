@@ -56,6 +56,34 @@ extern "C" int mi355x_read_probe(const void * src, size_t n, void * out, int wor
 }
 
 // ------------------------------------------------------------------------------------------------------
+// Matrix-pipe yardstick: v_mfma_f32_32x32x16_f16 from registers, four independent accumulators per wavefront, no memory
+// in the loop — the rate the matrix cores reach on this device at the clock they run at under that load, next to the
+// data-sheet peak.  2 * 32 * 32 * 16 flops per instruction, 4 * iters instructions per wavefront, 4 wavefronts per workgroup.
+// ------------------------------------------------------------------------------------------------------
+
+typedef _Float16 probe_half8 __attribute__((ext_vector_type(8)));
+typedef float    probe_f32x16 __attribute__((ext_vector_type(16)));
+
+__global__ void __launch_bounds__(256) k_mfma_probe(int iters, float * __restrict__ out) {
+    const probe_half8 a = { (_Float16)(threadIdx.x & 7), 1, 2, 3, 4, 5, 6, 7 }, b = { 1, 1, 1, 1, 1, 1, 1, (_Float16)(blockIdx.x & 3) };
+    probe_f32x16 c0 = {}, c1 = {}, c2 = {}, c3 = {};
+    for (int i = 0; i < iters; ++i) {
+        c0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c0, 0, 0, 0);
+        c1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c1, 0, 0, 0);
+        c2 = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c2, 0, 0, 0);
+        c3 = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c3, 0, 0, 0);
+    }
+    const float f = c0[0] + c1[1] + c2[2] + c3[3];
+    if (f == -1.0f) out[0] = f;                            // (never: the sums are >= 0; keeps the instructions)
+}
+
+extern "C" int mi355x_mfma_probe(int iters, int workgroups, void * out, void * stream) {
+    if (!out || (uintptr_t) out % 4 != 0 || iters < 1 || iters > (1 << 20) || workgroups < 1 || workgroups > 65535) return MI355X_ERR_INVALID;
+    k_mfma_probe<<<(unsigned) workgroups, 256, 0, (hipStream_t) stream>>>(iters, (float *) out);
+    return launch_status();
+}
+
+// ------------------------------------------------------------------------------------------------------
 // GELU table
 // ------------------------------------------------------------------------------------------------------
 
