@@ -264,10 +264,11 @@ def test_mul_mat_gelu_epilogue_from_the_lds_table_slice(pkg, oracle, gpu):
     assert oracle.nmse(got[:64], oracle.gelu(plain[:64])) <= 1e-7
 
 
-def test_mul_mat_epilogue_emits_the_next_products_activation_image(pkg, oracle, gpu):
-    # MI355X_EPI_EMIT_F16: besides dst (here with bias and GELU, the FFN's first matrix), its rows rounded to Q8_0 as f16(q * d)
+@pytest.mark.parametrize("k,m,n", [(256, 320, 150), (256, 5120, 1500)])
+def test_mul_mat_epilogue_emits_the_next_products_activation_image(pkg, oracle, gpu, k, m, n):
+    # MI355X_EPI_EMIT_F16: besides dst (here with bias and GELU, the FFN's first matrix), its rows rounded to Q8_0 as f16(q * d).
+    # The second case has the large-v3 FFN's width and rows: the 128 x 128 tiles whose operands go straight into LDS.
     lib = pkg.kernels()
-    k, m, n = 256, 320, 150
     blocks = oracle.quantize(pkg.Q5_0, rnd((m, k), 0.05))
     x, bias = rnd((n, k)), rnd((m,), 0.5)
     d_w, d_x, d_b = gpu.up(blocks), gpu.up(x), gpu.up(bias)

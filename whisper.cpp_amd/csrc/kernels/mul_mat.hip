@@ -75,29 +75,39 @@ __device__ __forceinline__ void patch_epilogue(float16_t v, const epi_args & e, 
         for (int i = 0; i < 16; ++i) v[i] += b[i];
     }
     if (e.flags & MI355X_EPI_GELU) {
-        uint16_t t[16];
         if (gelu_lds) {
             // 64 gathers per lane out of the 128 KB table in global memory cost the FFN-up product 10 us of its 45; out of
-            // LDS, 8.  A value of 8 or more in magnitude (none in a whisper model's activations) sends the wavefront to the
-            // table in global memory for that register.
-            uint32_t hb[16]; bool far = false;
+            // LDS, 8.  A value near 8 or more in magnitude (none in a whisper model's activations) sends the wavefront through
+            // the general form: the clamps at +-10 and the table in global memory for what the slice does not hold.
+            bool far = false;
 #pragma unroll
-            for (int i = 0; i < 16; ++i) { hb[i] = f2h_bits(v[i]); far = far || (hb[i] & 0x7FFFu) >= GELU_LDS_HALF; }
+            for (int i = 0; i < 16; ++i) far = far || !(fabsf(v[i]) < 7.99f);   // (f16 rounds up to 8 from 7.998; NaN is far)
+            if (!__any(far)) {
 #pragma unroll
-            for (int i = 0; i < 16; ++i) {
-                const uint32_t a = hb[i] & 0x7FFFu;
-                t[i] = gelu_lds[(a < GELU_LDS_HALF ? a : 0u) + (hb[i] >> 15) * GELU_LDS_HALF];
-            }
-            if (__any(far)) {
+                for (int i = 0; i < 16; ++i) {
+                    const uint32_t hb = f2h_bits(v[i]);
+                    v[i] = h2f(gelu_lds[(hb & 0x7FFFu) + (hb >> 15) * GELU_LDS_HALF]);
+                }
+            } else {
+                uint32_t hb[16]; uint16_t t[16];
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    hb[i] = f2h_bits(v[i]);
+                    const uint32_t a = hb[i] & 0x7FFFu;
+                    t[i] = gelu_lds[(a < GELU_LDS_HALF ? a : 0u) + (hb[i] >> 15) * GELU_LDS_HALF];
+                }
 #pragma unroll
                 for (int i = 0; i < 16; ++i) if ((hb[i] & 0x7FFFu) >= GELU_LDS_HALF) t[i] = e.gelu[hb[i]];
+#pragma unroll
+                for (int i = 0; i < 16; ++i) v[i] = v[i] <= -10.0f ? 0.0f : v[i] >= 10.0f ? v[i] : h2f(t[i]);
             }
         } else {
+            uint16_t t[16];
 #pragma unroll
             for (int i = 0; i < 16; ++i) t[i] = e.gelu[f2h_bits(v[i])];
-        }
 #pragma unroll
-        for (int i = 0; i < 16; ++i) v[i] = v[i] <= -10.0f ? 0.0f : v[i] >= 10.0f ? v[i] : h2f(t[i]);
+            for (int i = 0; i < 16; ++i) v[i] = v[i] <= -10.0f ? 0.0f : v[i] >= 10.0f ? v[i] : h2f(t[i]);
+        }
     }
     if (e.flags & MI355X_EPI_SCALE) {
 #pragma unroll
@@ -124,20 +134,27 @@ __device__ __forceinline__ void patch_epilogue(float16_t v, const epi_args & e, 
         // The two divisions of a block (127 / amax and amax / 127) would be repeated by all 32 lanes that hold it, for each
         // of the 16 registers: 32 IEEE divisions per lane and patch, most of this epilogue's time.  Instead lane l divides
         // for register l % 16 of its half-wavefront, and the 16 results travel back by lane permutes.
-        float amax[16];
+        // Block maxima: v_permlane16_swap of registers i and i + 8 leaves, in the even rows of 16 lanes, both halves of
+        // register i's block and, in the odd rows, both halves of register i + 8's — one swap and one maximum take the
+        // first butterfly step for two registers and halve what the other four steps (inside a row) have to carry.
+        float rmax[8];
 #pragma unroll
-        for (int i = 0; i < 16; ++i) amax[i] = lanes_max<32>(fabsf(v[i]));
+        for (int i = 0; i < 8; ++i) {
+            const auto sw = __builtin_amdgcn_permlane16_swap(__float_as_uint(v[i]), __float_as_uint(v[i + 8]), false, false);
+            rmax[i] = lanes_max<16>(fmaxf(fabsf(__uint_as_float(sw[0])), fabsf(__uint_as_float(sw[1]))));
+        }
         const int lane = threadIdx.x & 63;
-        float mine = amax[0];
+        float mine = rmax[0];                               // lane (row, c) of a half-wavefront: register c % 8 + 8 (row % 2)
 #pragma unroll
-        for (int i = 1; i < 16; ++i) mine = (lane & 15) == i ? amax[i] : mine;
+        for (int i = 1; i < 8; ++i) mine = (lane & 7) == i ? rmax[i] : mine;
         const float id_m = mine != 0.0f ? 127.0f / mine : 0.0f;
         const float dq_m = h2f(f2h_bits(mine / 127.0f));
         const int src = ((lane & 32) << 2);                 // byte address of lane 0 of this half-wavefront for ds_bpermute
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
-            const float id = __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(src + 4 * i, __builtin_bit_cast(int, id_m)));
-            const float dq = __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(src + 4 * i, __builtin_bit_cast(int, dq_m)));
+            const int from = src + 4 * ((i & 7) + (i >= 8 ? 16 : 0));
+            const float id = __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(from, __builtin_bit_cast(int, id_m)));
+            const float dq = __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(from, __builtin_bit_cast(int, dq_m)));
             if (m_ok && n[i] < N) e.image[n[i] * M + m] = (half_t)((rintf(v[i] * id) + 0.0f) * dq);
         }
     }
