@@ -54,14 +54,15 @@ __device__ __forceinline__ float apply_epilogue(float v, const epi_args & e, int
 #define GELU_LDS_HALF  0x4800
 #define GELU_LDS_BYTES (2 * GELU_LDS_HALF * 2)
 
-template <bool EMIT>
+// FULL: the whole tile lies inside dst (no row or column of the patch is clamped or masked)
+template <bool EMIT, bool FULL = false>
 __device__ __forceinline__ void patch_epilogue(float16_t v, const epi_args & e, char * db, int64_t batch_off, int64_t d_nb1,
                                                int64_t m, int64_t M, const int64_t (&n)[16], int64_t N, const uint16_t * gelu_lds = nullptr) {
-    const bool    m_ok = m < M;
+    const bool    m_ok = FULL || m < M;
     const int64_t mc   = m_ok ? m : M - 1;
     int64_t nc[16];
 #pragma unroll
-    for (int i = 0; i < 16; ++i) nc[i] = n[i] < N ? n[i] : N - 1;
+    for (int i = 0; i < 16; ++i) nc[i] = FULL || n[i] < N ? n[i] : N - 1;
     if (e.flags & MI355X_EPI_BIAS) {
         const float b = e.bias[mc];
 #pragma unroll
@@ -122,10 +123,10 @@ __device__ __forceinline__ void patch_epilogue(float16_t v, const epi_args & e, 
     }
     if (e.flags & MI355X_EPI_OUT_F16) {
 #pragma unroll
-        for (int i = 0; i < 16; ++i) if (m_ok && n[i] < N) *(half_t *)(db + n[i] * d_nb1 + m * 2) = (half_t) v[i];
+        for (int i = 0; i < 16; ++i) if (m_ok && (FULL || n[i] < N)) *(half_t *)(db + n[i] * d_nb1 + m * 2) = (half_t) v[i];
     } else if (!EMIT || !(e.flags & MI355X_EPI_IMAGE_ONLY)) {
 #pragma unroll
-        for (int i = 0; i < 16; ++i) if (m_ok && n[i] < N) *(float *)(db + n[i] * d_nb1 + m * 4) = v[i];
+        for (int i = 0; i < 16; ++i) if (m_ok && (FULL || n[i] < N)) *(float *)(db + n[i] * d_nb1 + m * 4) = v[i];
     }
     if (EMIT) {
         // The product that reads dst next rounds its rows to Q8_0 first.  The 32 lanes of a half-wavefront hold 32
@@ -141,7 +142,10 @@ __device__ __forceinline__ void patch_epilogue(float16_t v, const epi_args & e, 
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
             const auto sw = __builtin_amdgcn_permlane16_swap(__float_as_uint(v[i]), __float_as_uint(v[i + 8]), false, false);
-            rmax[i] = lanes_max<16>(fmaxf(fabsf(__uint_as_float(sw[0])), fabsf(__uint_as_float(sw[1]))));
+            // (the row steps on the bit patterns: non-negative floats order like unsigned integers, and an integer maximum
+            // takes its DPP operand in the same instruction)
+            rmax[i] = __uint_as_float(lanes_reduce<16>(__float_as_uint(fmaxf(fabsf(__uint_as_float(sw[0])), fabsf(__uint_as_float(sw[1])))),
+                                                        [](uint32_t a, uint32_t b) { return a > b ? a : b; }));
         }
         const int lane = threadIdx.x & 63;
         float mine = rmax[0];                               // lane (row, c) of a half-wavefront: register c % 8 + 8 (row % 2)
@@ -155,7 +159,7 @@ __device__ __forceinline__ void patch_epilogue(float16_t v, const epi_args & e, 
             const int from = src + 4 * ((i & 7) + (i >= 8 ? 16 : 0));
             const float id = __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(from, __builtin_bit_cast(int, id_m)));
             const float dq = __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(from, __builtin_bit_cast(int, dq_m)));
-            if (m_ok && n[i] < N) e.image[n[i] * M + m] = (half_t)((rintf(v[i] * id) + 0.0f) * dq);
+            if (m_ok && (FULL || n[i] < N)) e.image[n[i] * M + m] = (half_t)((rintf(v[i] * id) + 0.0f) * dq);
         }
     }
 }
@@ -327,15 +331,19 @@ __device__ __forceinline__ void gemm_tile_epilogue(float16_t (&acc)[TI][TJ], con
     }
     if (NT > 256 && tid >= 256) return;
     // accumulator register e of a 32x32 patch: row (= n) 8*(e/4) + 4*g + e%4, column (= m) lane%32
+    auto patches = [&](auto full) __attribute__((always_inline)) {
 #pragma unroll
-    for (int i = 0; i < TI; ++i) {
-        int64_t n[16];
+        for (int i = 0; i < TI; ++i) {
+            int64_t n[16];
 #pragma unroll
-        for (int e = 0; e < 16; ++e) n[e] = n0 + wn + 32 * i + 8 * (e >> 2) + 4 * g + (e & 3);
+            for (int e = 0; e < 16; ++e) n[e] = n0 + wn + 32 * i + 8 * (e >> 2) + 4 * g + (e & 3);
 #pragma unroll
-        for (int j = 0; j < TJ; ++j)
-            patch_epilogue<EMIT>(acc[i][j], epi, db, batch_off, d_nb1, m0 + wmo + 32 * j + l32, a.M, n, a.N, gelu_lds);
-    }
+            for (int j = 0; j < TJ; ++j)
+                patch_epilogue<EMIT, decltype(full)::value>(acc[i][j], epi, db, batch_off, d_nb1, m0 + wmo + 32 * j + l32, a.M, n, a.N, gelu_lds);
+        }
+    };
+    // tiles inside dst (all but the last row of tiles when N = 1500) store without per-element bounds
+    if (n0 + 64 * TI <= a.N && m0 + 64 * TJ <= a.M) patches(std::true_type{}); else patches(std::false_type{});
 }
 
 // KTAIL: K is not a multiple of 64 (but of 8); FULL: K / 64 is a multiple of S; EMIT: MI355X_EPI_EMIT_F16 (a kernel of its
