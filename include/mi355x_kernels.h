@@ -204,7 +204,9 @@ MI355X_API int    mi355x_mul_mat_q8_0_tiles(const void * tiles, int64_t K, int64
 enum mi355x_fa_mode { MI355X_FA_F16_SEQ = 0, MI355X_FA_F32 = 1,
     /* or-ed into the mode: also write into `workspace` (16-byte aligned, N * H * ne3 * 64 halves) the image of dst that
      * a following MUL_MAT with quantized weights wants — rows [N][H * 64] rounded to Q8_0 as quantize_row_q8_0 does and
-     * stored as f16(q * d) (then pass MI355X_MM_WS_READY there).  More than 8 queries; MI355X_ERR_UNSUPPORTED otherwise. */
+     * stored as f16(q * d) (then pass MI355X_MM_WS_READY there).  More than 8 queries; MI355X_ERR_UNSUPPORTED otherwise.
+     * With MI355X_FA_F16_SEQ, dst->data may then be NULL: only the image is written (a caller whose only reader of dst is
+     * that product); MI355X_ERR_INVALID for a NULL dst->data in any other case. */
     MI355X_FA_EMIT_F16 = 0x100,
     /* or-ed into the mode, at most 8 queries (the f16-sequential kernel of a decode step): also write into `workspace`
      * (16-byte aligned) the rows [N * ne3][H * 64] of dst quantized to Q8_0, in the layout the few-column mi355x_mul_mat

@@ -618,6 +618,14 @@ def test_flash_attn_emits_the_next_products_activation_image(pkg, oracle, gpu):
     d_o5 = torch.empty((5, H, 64), dtype=torch.float32, device=gpu.dev)
     assert lib.mi355x_flash_attn_ext(pkg.tensor(d_q5, pkg.F32), tk, tv, None, pkg.tensor(d_o5, pkg.F32), 0.125, pkg.FA_EMIT_F16, d_h.data_ptr(), d_h.numel() * 2, gpu.stream) == -1
     assert lib.mi355x_flash_attn_ext(tq, tk, tv, None, to, 0.125, pkg.FA_EMIT_F16, d_h.data_ptr(), 64, gpu.stream) == -3
+    # a dst without memory: the same image and nothing else; without the image, or in f32 mode, that is an error
+    d_h2 = torch.zeros_like(d_h)
+    t_null = pkg.tensor(d_o, pkg.F32); t_null.data = None
+    d_o.fill_(7.0)
+    pkg.check(lib.mi355x_flash_attn_ext(tq, tk, tv, None, t_null, 0.125, pkg.FA_F16_SEQ | pkg.FA_EMIT_F16, d_h2.data_ptr(), d_h2.numel() * 2, gpu.stream))
+    assert np.array_equal(gpu.down(d_h2, np.uint16), gpu.down(d_h, np.uint16)) and np.all(gpu.down(d_o) == 7.0)
+    assert lib.mi355x_flash_attn_ext(tq, tk, tv, None, t_null, 0.125, pkg.FA_F16_SEQ, None, 0, gpu.stream) == -2
+    assert lib.mi355x_flash_attn_ext(tq, tk, tv, None, t_null, 0.125, pkg.FA_F32 | pkg.FA_EMIT_F16, d_h2.data_ptr(), d_h2.numel() * 2, gpu.stream) == -2
 
 
 def test_flash_attn_few_queries_emit_q8_0(pkg, oracle, gpu):

@@ -802,8 +802,11 @@ struct graph_runner {
                 if (!key && !ctx->exact && strcmp(name, "flash_attn.seq_row") == 0 && (key = image_consumer(n, i + 1, true))) form = 2;
                 const size_t image_bytes = form == 1 ? (size_t) ggml_nelements(n) * 2 : (size_t) ggml_nelements(n) / 32 * 40;
                 if (key && !ctx->reserve_workspace(image_bytes + 256)) key = nullptr;
+                // ... and only the image when the projection is the very next launch: the f32 rows would have no reader
+                const bool image_only = key && form == 1 && ctx->dead_f32 && strncmp(name, "flash_attn.seq_tile", 19) == 0 && next_is_product_over(key, i + 1);
+                if (image_only) vd.data = nullptr;
                 {
-                    launch_scope ls(ctx, name, bytes + (key ? image_bytes : 0), flops);
+                    launch_scope ls(ctx, name, bytes - (image_only ? nbytes_of(n) : 0) + (key ? image_bytes : 0), flops);
                     const int flags = mode | (!key ? 0 : form == 1 ? MI355X_FA_EMIT_F16 : MI355X_FA_EMIT_Q8_0);
                     if (m16) {
                         mi355x_tensor vm16 = to_view(m16);
@@ -812,7 +815,7 @@ struct graph_runner {
                     status = mi355x_flash_attn_ext(&vq, &vk, &vv, m ? &vm : nullptr, &vd, scale, flags,
                                                    key ? ctx->ws : nullptr, key ? ctx->ws_size : 0, ctx->stream);
                 }
-                if (key && status == MI355X_OK) workspace_holds(key, ctx->ws_slot, form);
+                if (key && status == MI355X_OK) { workspace_holds(key, ctx->ws_slot, form); if (image_only) ctx->image_only = key; }
                 return 1;
             }
             case GGML_OP_CONCAT: {

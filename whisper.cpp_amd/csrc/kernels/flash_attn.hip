@@ -799,7 +799,7 @@ __global__ void __launch_bounds__(512, 2) k_fattn_seq_tile(fa_args a) {
 #pragma unroll
         for (int i = 0; i < 8; ++i) { o[2*i] = (float) acc2[i][0] * inv; o[2*i + 1] = (float) acc2[i][1] * inv; }
     }
-    if (n < a.N) {
+    if (a.d && n < a.N) {                                  // (no dst: the caller reads the image below and nothing else)
         float * dp = (float *) a.d + ((i3 * a.N + n) * a.H + h) * FA_D + d0;
 #pragma unroll
         for (int i = 0; i < 4; ++i) *(float4 *)(dp + 4 * i) = make_float4(o[4*i], o[4*i + 1], o[4*i + 2], o[4*i + 3]);
@@ -1060,6 +1060,8 @@ static int flash_attn_ext(const mi355x_tensor * q, const mi355x_tensor * k, cons
     mode &= ~(MI355X_FA_EMIT_F16 | MI355X_FA_EMIT_Q8_0);
     if (emit && emit_q8) return MI355X_ERR_INVALID;
     if (mode != MI355X_FA_F16_SEQ && mode != MI355X_FA_F32) return MI355X_ERR_INVALID;
+    // dst without memory: only the image is wanted (the key-by-key tile kernel with MI355X_FA_EMIT_F16)
+    if (!dst->data && !(emit && fa_kernel(q, k, mode) == FA_K_SEQ_TILE)) return MI355X_ERR_INVALID;
     if (q->type != MI355X_TYPE_F32 || k->type != MI355X_TYPE_F16 || v->type != MI355X_TYPE_F16 || dst->type != MI355X_TYPE_F32) return MI355X_ERR_UNSUPPORTED;
     if (q->ne[0] != FA_D || k->ne[0] != FA_D || v->ne[0] != FA_D) return MI355X_ERR_UNSUPPORTED;
     if (q->nb[0] != 4 || k->nb[0] != 2 || v->nb[0] != 2) return MI355X_ERR_UNSUPPORTED;
