@@ -225,8 +225,8 @@ def main() -> int:
         roofline["note"] = ("priced against the dense f16 matrix-core peak as the brief asks; the matrix cores only form the scores. "
                             "The reference accumulates V key by key in f16 (f32 fma, f16 store), and reproducing that takes 1.5 vector "
                             "instructions per (query, key, d). SQ_INSTS_VALU counts 93.5 M vector instructions per launch (70.8 M of them that sequence): "
-                            "178 us of issue per SIMD at the 2.05 GHz the part runs this kernel at; that is the bound that applies, and the kernel "
-                            "runs at about 91 % of it")
+                            "178 us of issue per SIMD at the 2.05 GHz the part runs this kernel at; that is the bound that applies, and with its chain "
+                            "wavefronts issuing ahead of its producers the kernel runs within a few per cent of it")
 
     # ---- and with f32 matrix-core attention (faster, but outside the whole-model parity bound: reported, never the headline) ----
     f32att = run_harness(["bench", "--model", enc_model, "--what", "encoder", "--backend", "gpu", "--reps", str(a.steps),
