@@ -213,7 +213,7 @@ def test_whole_model_parity_on_other_seeds(harness, tmp_path, arch, ftype):
 
 @pytest.mark.parametrize("key,env", [(("large-v3-turbo", "q8_0"), {}), (("large-v3-turbo", "q8_0"), {"GGML_MI355X_FUSE": "0"}), (("base", "q5_0"), {})])
 def test_five_row_decode_steps_until_the_cache_is_full(harness, models, key, env):
-    # the shape of a 5-beam search step (BASELINE configs[4]): after the 4-token prompt every step feeds 5 tokens — the 5
+    # the shape of a 5-beam search step (large-v3-turbo, 5 beams, 224 tokens): after the 4-token prompt every step feeds 5 tokens — the 5
     # greedy ids of the CPU backend's previous step — until the self-attention cache holds all 448 positions; all 5 rows
     # of every step are compared.  Five rows take other planner branches than one (LayerNorm held for the product group,
     # grouped Q / K / V, fused embeddings, the mask cast inside the first attention launch, the tile-ordered logits product).

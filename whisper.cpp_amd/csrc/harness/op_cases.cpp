@@ -195,7 +195,7 @@ ggml_tensor * in2(ggml_context * ctx, built & b, const char * name, ggml_type t,
 std::vector<op_case> all_cases() {
     std::vector<op_case> v;
 
-    // BASELINE config 0 and the encoder GEMMs of Whisper-base and large-v3
+    // the Whisper-base FFN-up product over a 30 s window (the smallest benchmarked case) and the encoder GEMMs of Whisper-base and large-v3
     v.push_back(mm("mul_mat.q8_0.cfg0_512x2048_n1500",  GGML_TYPE_Q8_0, 512, 2048, 1500));
     v.push_back(mm("mul_mat.q5_0.base_512x512_n1500",   GGML_TYPE_Q5_0, 512, 512, 1500));
     v.push_back(mm("mul_mat.q5_0.base_2048x512_n1500",  GGML_TYPE_Q5_0, 2048, 512, 1500));
@@ -211,7 +211,7 @@ std::vector<op_case> all_cases() {
     v.push_back(mm("mul_mat.q5_0.ragged_n129_m130",     GGML_TYPE_Q5_0, 512, 130, 129));
     v.push_back(mm("mul_mat.q8_0.prompt_n448",          GGML_TYPE_Q8_0, 1280, 1280, 448));
     v.push_back(mm("mul_mat.q5_0.k32_single_block",     GGML_TYPE_Q5_0, 32, 64, 200));
-    // decoder GEMV (1..8 columns), incl. the 1280x51866 logits projection of BASELINE config 4
+    // decoder GEMV (1..8 columns), incl. the 1280x51866 logits projection of a large-v3-turbo decode step
     v.push_back(mm("mul_mat.q8_0.logits_51866_n5",      GGML_TYPE_Q8_0, 1280, 51866, 5));
     v.push_back(mm("mul_mat.q8_0.logits_51866_n1",      GGML_TYPE_Q8_0, 1280, 51866, 1));
     v.push_back(mm("mul_mat.q5_0.logits_51866_n5",      GGML_TYPE_Q5_0, 1280, 51866, 5));
@@ -244,7 +244,7 @@ std::vector<op_case> all_cases() {
     v.push_back(conv_stem("conv_stem.l3_conv1_128x3000",   3000, 128, 1280, 1, false));
     v.push_back(conv_stem("conv_stem.l3_conv2_1280x3000",  3000, 1280, 1280, 2, true));
 
-    // BASELINE config 2 and whisper's three attention kinds
+    // the large-v3 encoder's self-attention (1500 x 1500, 20 heads) and whisper's three attention kinds
     v.push_back(fa("flash_attn.cfg2_enc_n1500_kv1500_h20", 1500, 1500, 1500, 20, 0, 0.125f, true));
     v.push_back(fa("flash_attn.enc_base_n1500_kv1536pad_h8", 1500, 1536, 1500, 8, 0, 0.125f, true));
     v.push_back(fa("flash_attn.cfg2_cross_n5_kv1500_h20",  5, 1500, 1500, 20, 0, 0.125f));
