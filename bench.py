@@ -60,7 +60,7 @@ def model_file(arch: str, ftype: str) -> str:
 # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled by the same counters over a 256 MiB copy:
 # x2 KiB and x1 KiB), for the large-v3 encoder shapes; the summary with the commands is under profiles/
 # (mul_mat.gemm_q5_0 averages its two templates: 64 launches of 59.9 + 7.7 MB and 32 of 45.4 + 15.4 MB per window)
-MEASURED_TRAFFIC_MB = {"mul_mat.gemm_q5_0": (64 * (59.9 + 7.7) + 32 * (45.4 + 15.4)) / 96, "flash_attn.seq_tile": 17.4 + 11.5,
+MEASURED_TRAFFIC_MB = {"mul_mat.gemm_q5_0": (64 * (59.9 + 7.7) + 32 * (45.4 + 15.4)) / 96, "flash_attn.seq_tile": 17.4 + 3.8,
                        "mul_mat.gemm_group": 68.6 + 22.5, "norm_affine_emit": 7.9 + 3.8}
 
 # kernels that live on the matrix cores (bound "mfma"); everything else streams memory (bound "hbm")
