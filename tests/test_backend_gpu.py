@@ -80,6 +80,20 @@ def test_unfused_graphs_match_fused_ones(harness, models):
         assert rc == 0 and rows[-1]["pass"], rows[-1]
 
 
+def test_results_without_a_reader_are_not_stored_and_the_logits_do_not_change(harness, models):
+    # A LayerNorm, an FFN-up product or an attention node whose only reader is the product that takes its activation image
+    # writes the image and nothing else.  GGML_MI355X_DEAD_F32=0 stores the f32 values as well: the same logits to the
+    # last bit, so the same worst NMSE against the CPU backend and the same greedy ids.
+    summaries = []
+    for env in ({}, {"GGML_MI355X_DEAD_F32": "0"}):
+        rc, rows = run_harness(harness, ["model", "--model", models[("base", "q5_0")], "--steps", "8"], env=env, timeout=900)
+        assert rc == 0 and rows[-1]["pass"], rows[-1]
+        summaries.append(rows[-1])
+    a, b = summaries
+    assert a["worst_logits_nmse"] == b["worst_logits_nmse"] and a["ids_identical"] == b["ids_identical"], (a, b)
+    assert a["encode_launches"] == b["encode_launches"]
+
+
 @pytest.mark.parametrize("key", [("base", "q5_0"), ("base", "q8_0"), ("base", "f16")])
 def test_every_node_of_the_whisper_graphs(harness, models, key):
     rc, rows = run_harness(harness, ["verify", "--model", models[key], "--steps", "2"], timeout=1200)
