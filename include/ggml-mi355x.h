@@ -56,14 +56,20 @@ GGML_BACKEND_API int                ggml_backend_score(void);
  * "exact" (0/1, default 0: 0 reproduces the two roundings that the reference's CPU backend applies — Q8_0-rounded
  * activations in front of quantized MUL_MAT, f16 key-by-key V accumulation in FLASH_ATTN_EXT; 1 keeps f16 activations
  * and f32 accumulators, which is closer to exact arithmetic and further from the reference),
- * "fa_accum" (0..3, default 0: how FLASH_ATTN_EXT accumulates V.  0: key by key with an f16 accumulator, f32 fma + f16
- * store — the reference's sequence (ops.cpp:6793-6807), and the only setting that keeps whole-model logits within 1e-3
- * NMSE of the CPU backend.  Bit 0: f32 accumulators with both products on the matrix cores for more than 8 queries —
+ * "fa_accum" (0..3, default 0: how FLASH_ATTN_EXT accumulates V.  0: key by key with an f16 accumulator that is rounded
+ * after every key — the reference's sequence (ops.cpp:6793-6807), and the only setting that keeps whole-model logits
+ * within 1e-3 NMSE of the CPU backend.  Bit 0: f32 accumulators with both products on the matrix cores for more than 8 queries —
  * five times faster, within the per-op bound, but the reference's f16 rounding is then missing and whole-model logits sit
  * several 1e-3 away.  Bit 1: f32 accumulators for a decode step's few queries; the decoder's layers alone move the
  * logits to 6e-3 … 8e-3 NMSE).
- * The environment variables GGML_MI355X_FUSE, GGML_MI355X_PROFILE, GGML_MI355X_EXACT and GGML_MI355X_FA_ACCUM give the
- * initial values.
+ * "fa_chain" (0/1, default 1: the arithmetic of one step of that key-by-key sequence where a launch has more than 8
+ * queries.  1: the factor rounded to f16 and one fused f16 multiply-add per element, the reference's ggml_vec_mad_f16 on
+ * hardware with f16 vector arithmetic (vec.h:180-203 with GGML_F16_VEC_FMA = vfmaq_f16, simd-mappings.h:68-105) — a third
+ * of the vector instructions.  0: f32 fma followed by an f16 store, the same function in the reference's x86 build, which
+ * the few-query kernel of a decode step always uses.  Whole-model logits stay within the same 1e-3 of the x86 CPU
+ * backend with either.)
+ * The environment variables GGML_MI355X_FUSE, GGML_MI355X_PROFILE, GGML_MI355X_EXACT, GGML_MI355X_FA_ACCUM and
+ * GGML_MI355X_FA_CHAIN give the initial values.
  * backend == NULL addresses every live MI355X backend of the process (a host such as whisper.cpp keeps its
  * backends private). */
 typedef int (*ggml_backend_mi355x_set_option_t)(ggml_backend_t backend, const char * name, int value);

@@ -200,8 +200,13 @@ MI355X_API int    mi355x_mul_mat_q8_0_tiles(const void * tiles, int64_t K, int64
  * mode: MI355X_FA_F16_SEQ accumulates V in f16, key by key in order, as the reference does (ops.cpp:6793-6807) —
  * with near-uniform attention over ~1500 keys that rounding sequence dominates the low bits of the result;
  * MI355X_FA_F32 accumulates in f32 (closer to exact arithmetic, further from the reference); with more than 8 queries
- * both products run on the matrix cores with the softmax probabilities as f16 operands. */
-enum mi355x_fa_mode { MI355X_FA_F16_SEQ = 0, MI355X_FA_F32 = 1,
+ * both products run on the matrix cores with the softmax probabilities as f16 operands.
+ * MI355X_FA_F16_PK keeps the f16 accumulator and the key order and does the step in f16 arithmetic — the factor rounded
+ * to f16, one fused f16 multiply-add per element, a rescale as one f16 multiply — which is the arithmetic of the
+ * reference's builds with f16 vector units (GGML_F16_VEC_FMA = vfmaq_f16, ggml/src/ggml-cpu/simd-mappings.h:68-105, under
+ * ggml_vec_mad_f16 / ggml_vec_scale_f16, vec.h:180-203, 295-311), a third of the vector instructions of the x86 form;
+ * with at most 8 queries it is MI355X_FA_F16_SEQ. */
+enum mi355x_fa_mode { MI355X_FA_F16_SEQ = 0, MI355X_FA_F32 = 1, MI355X_FA_F16_PK = 2,
     /* or-ed into the mode: also write into `workspace` (16-byte aligned, N * H * ne3 * 64 halves) the image of dst that
      * a following MUL_MAT with quantized weights wants — rows [N][H * 64] rounded to Q8_0 as quantize_row_q8_0 does and
      * stored as f16(q * d) (then pass MI355X_MM_WS_READY there).  More than 8 queries; MI355X_ERR_UNSUPPORTED otherwise.

@@ -131,12 +131,16 @@ def test_whisper_full_from_the_device_log_mel(harness, models):
 def test_whisper_full_parallel_states_share_one_device(harness, models):
     # whisper_full_parallel (src/whisper.cpp:6407-6470): three states, three backend instances and streams, three host
     # threads on one GPU, all starting at once over shared weights — the f16 weight images are made on first use and must be
-    # complete before another instance can find them.  The merged transcript must start like the CPU backend's.
+    # complete before another instance can find them.  The run is repeated on the same context (images made by then): the two
+    # greedy transcripts must be the same tokens.  Against the CPU backend only the start is compared: a free-running greedy
+    # transcript of a random-init model follows the CPU's until the first argmax inside the rounding noise, which over six audio
+    # seeds came after 11 to 96 tokens (either form of the attention step; 90 with this seed), so a short prefix is what a
+    # correct backend guarantees here — the teacher-forced tests above are the ones that bound the logits.
     rc, rows = run_harness(harness, ["full", "--model", models[("base", "q5_0")], "--beam", "1", "--max-tokens", "16", "--seconds", "120",
-                                     "--processors", "3"], timeout=900)
+                                     "--processors", "3", "--seed", "8", "--repeat"], timeout=900)
     s = rows[-1]
-    assert rc == 0 and s["pass"] and s["gpu_rc"] == 0 and s["gpu_tokens"] > 0, s
-    assert s["common_prefix"] >= min(16, s["cpu_tokens"]), s
+    assert rc == 0 and s["pass"] and s["gpu_rc"] == 0 and s["gpu_tokens"] > 0 and s["gpu_repeat_identical"], s
+    assert s["common_prefix"] >= min(8, s["cpu_tokens"]), s
 
 
 def test_whisper_full_with_dtw_token_timestamps(harness, models):
@@ -182,6 +186,27 @@ def test_default_attention_graphs_without_flash_attn(harness, models):
     rc, rows = run_harness(harness, ["verify", "--model", models[("base", "q5_0")], "--steps", "2", "--no-flash-attn"], timeout=1200)
     assert rc == 0 and rows[-1]["pass"], [r for r in rows if "bad_node" in r]
     assert "SOFT_MAX" in {r["op"] for r in rows if "phase" in r}
+
+
+def test_graphs_that_arrive_in_pieces(harness, models):
+    # GGML_MI355X_DECLINE=GELU makes supports_op turn GELU down: the scheduler puts those nodes on the CPU backend, and the conv
+    # stem, the encoder and the decoder reach the plugin as ggml_graph_view slices with downloads and uploads in between
+    # (ggml/src/ggml-backend.cpp:1013-1034, 1196-1215, 1252).  The usual logits / ids criterion must hold.
+    rc, rows = run_harness(harness, ["model", "--model", models[("base", "q5_0")], "--steps", "8", "--pieces"], env={"GGML_MI355X_DECLINE": "GELU"}, timeout=900)
+    s = rows[-1]
+    assert rc == 0 and s["pass"] and s["worst_logits_nmse"] <= 1e-3 and s["ids_identical"] == s["rows"], s
+    assert s["sched_splits"] > s["graphs"] and s["sched_splits_not_on_device"] > 0 and s["plugin_graph_computes"] > s["graphs"], s
+    # A slice shows only the readers inside it.  A result that the walker folded away because it saw one reader, and that a
+    # later slice reads after all, is refused (failed graph, NaN download) instead of read as garbage; the instance then stores
+    # everything and the repeat is correct (first_try: GGML_STATUS_SUCCESS, GGML_STATUS_FAILED).  Also the late reader inside one graph (a product over the LayerNorm's rows after
+    # another product's image has taken their place in the workspace).
+    rc, rows = run_harness(harness, ["pieces"], timeout=300)
+    assert rc == 0 and rows[-1] == {"summary": "pieces", "failed": 0}, rows
+    cases = {(r["pieces"], r["cols"]): r for r in rows if "pieces" in r}
+    assert cases[("late_reader_in_the_next_piece", 64)]["first_try"] == [0, -1] and cases[("late_reader_in_the_next_piece", 64)]["download_poisoned"]
+    rc, rows = run_harness(harness, ["pieces"], env={"GGML_MI355X_DEAD_F32": "0"}, timeout=300, check=False)
+    late = [r for r in rows if r.get("pieces") == "late_reader_in_one_graph"]
+    assert late and all(r["pass"] for r in late), rows
 
 
 def check_model_summary(s, strict_ids):

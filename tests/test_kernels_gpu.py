@@ -568,6 +568,37 @@ def test_flash_attn_reference_faithful(pkg, oracle, gpu, case):
     assert oracle.nmse(got, want) <= 1e-6      # same key order, same f16 accumulator: only exp() and dot-product ulps differ
 
 
+@pytest.mark.parametrize("case", [
+    dict(H=2, N=70, KV=100), dict(H=3, N=200, KV=1536, flat=True, pad_from=1500), dict(H=2, N=100, KV=100, mask="causal"),
+    dict(H=2, N=9, KV=63), dict(H=2, N=130, KV=448, mask="causal"), dict(H=2, N=64, KV=1500, flat=True)])
+def test_flash_attn_packed_f16_chain(pkg, oracle, gpu, case):
+    # MI355X_FA_F16_PK: the same key order and f16 accumulator, the step as one fused f16 multiply-add on the factor rounded
+    # to f16 (the reference's arithmetic where it has f16 vector units).  Checked against the pinned restatement of the x86
+    # sequence: a step of the two forms differs by the factor's rounding and by one rounding in place of two, which leaves
+    # the results within 1e-5 NMSE of each other, and both equally far (several 1e-3 on flat attention) from an f64 evaluation.
+    H, N, KV = case["H"], case["N"], case["KV"]
+    q, kb, vb = _attention_inputs(oracle, H, N, KV, case.get("flat", False), case.get("pad_from"))
+    mask = None
+    if "mask" in case:
+        m = np.full((-(-N // 64) * 64, KV), -np.inf, dtype=np.float32)
+        for r in range(N):
+            m[r, : KV - N + r + 1] = 0.0
+        mask = oracle.f32_to_f16_bits(m)
+    got, name = run_fa(pkg, gpu, q, kb, vb, mask, 0.125, pkg.FA_F16_PK)
+    assert name == "flash_attn.seq_tile_pk"
+    want = oracle.flash_attn_ext(q, kb, vb, None if mask is None else mask[:N], 0.125)
+    seq, _ = run_fa(pkg, gpu, q, kb, vb, mask, 0.125, pkg.FA_F16_SEQ)
+    exact = _attention_float64(oracle, q, kb, vb, None if mask is None else mask, 0.125)
+    print(f"packed chain {case}: vs oracle {oracle.nmse(got, want):.3e}, x86 form vs oracle {oracle.nmse(seq, want):.3e}, "
+          f"packed vs f64 {oracle.nmse(got, exact):.3e}, oracle vs f64 {oracle.nmse(want, exact):.3e}", flush=True)
+    assert oracle.nmse(got, want) <= 1e-5
+    # with at most 8 queries the mode is the f32-fma sequence of the few-query kernel, bit for bit
+    if N == 70:
+        a, name = run_fa(pkg, gpu, q[:, :5], kb, vb, None, 0.125, pkg.FA_F16_PK)
+        b, _ = run_fa(pkg, gpu, q[:, :5], kb, vb, None, 0.125, pkg.FA_F16_SEQ)
+        assert name == "flash_attn.seq_row" and np.array_equal(a.view(np.uint32), b.view(np.uint32))
+
+
 def test_flash_attn_few_queries_take_the_f32_mask(pkg, oracle, gpu):
     # the few-query kernel reads the f32 tensor a graph would cast to f16 and rounds each value as the cast does: the same bits
     # as with the f16 copy, also for values that are not representable in f16; with more than 8 queries it says no

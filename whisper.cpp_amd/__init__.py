@@ -27,7 +27,7 @@ EPI_BIAS, EPI_GELU, EPI_SCALE, EPI_RESIDUAL, EPI_BIAS_COL, EPI_OUT_F16 = 1, 2, 4
 MM_EXACT_ACT, MM_WS_READY, MM_ACT_Q8_0, MM_PREPARE_ONLY, EPI_EMIT_F16, EPI_IMAGE_ONLY, EPI_EMIT_Q8_0 = 64, 128, 256, 512, 1024, 2048, 4096
 MUL_MAT_NOALLOC_MAX = 32 << 20
 # enum mi355x_fa_mode
-FA_F16_SEQ, FA_F32, FA_EMIT_F16, FA_EMIT_Q8_0 = 0, 1, 0x100, 0x200
+FA_F16_SEQ, FA_F32, FA_F16_PK, FA_EMIT_F16, FA_EMIT_Q8_0 = 0, 1, 2, 0x100, 0x200
 
 
 class Tensor(C.Structure):

@@ -15,6 +15,7 @@
 
 #include "ggml-mi355x.h"
 #include "mi355x_kernels.h"
+#include "range_set.h"
 
 #define MI355X_BUFFER_ALIGN 256
 #define MI355X_N_COUNTERS   8
@@ -60,6 +61,10 @@ struct mi355x_buffer_ctx {
     std::mutex                               image_mutex;
     std::map<uintptr_t, mi355x_weight_image> images;
 
+    // Results of graph nodes in this buffer that no launch stored (folded into their consumer, or kept only as the next
+    // product's activation image): a later read of such memory is refused, see range_set.h.
+    mi355x_range_set unwritten;
+
     const void * weight_image(const struct ggml_tensor * w, hipStream_t stream, int kind = MI355X_IMAGE_F16);   // NULL: none could be made
     void         drop_images(const void * begin, size_t size);
     void         drop_all_images();
@@ -90,8 +95,14 @@ struct mi355x_backend_ctx {
     int         fa_accum = 0;           // V accumulation of attention: 0 the reference's sequence (f32 fma, f16 store, key by key);
                                         // bit 0: f32 accumulators (matrix cores) for more than 8 queries, bit 1: f32
                                         // accumulators for a decode step's few queries
+    int         fa_chain = 1;           // the f16 key-by-key step for more than 8 queries: 1 fused f16 multiply-add on the factor rounded to
+                                        // f16 (the reference's builds with f16 vector units), 0 f32 fma then f16 store (its x86 build)
     bool        dead_f32 = true;        // a result whose only reader is the next launch's activation image is not also written as f32
                                         // (GGML_MI355X_DEAD_F32=0: always write it)
+    bool        check_reads = true;     // refuse to read memory whose value a launch folded away (GGML_MI355X_CHECK_READS=0 turns the
+                                        // bookkeeping off)
+    bool        pieces = false;         // a graph turned out to arrive in pieces (a later piece read a result that an earlier one had
+                                        // folded away): from then on every result is stored, whatever the visible readers say
     bool        weight_images = true;   // keep f16 images of quantized GEMM weights (GGML_MI355X_WEIGHT_IMAGES=0 turns it off)
     bool        exact   = false;   // true: f32 attention accumulators and un-rounded GEMM activations instead of the
                                    // reference's f16-sequential / Q8_0-rounded arithmetic

@@ -252,6 +252,7 @@ static void buffer_memset_tensor(ggml_backend_buffer_t buffer, struct ggml_tenso
     HIP_TRY(hipSetDevice(ctx->device), return);
     ctx->drop_images((char *) tensor->data + offset, size);
     drop_mirrors(ctx->device, (char *) tensor->data + offset, size);
+    ctx->unwritten.written((char *) tensor->data + offset, size);
     HIP_TRY(hipMemset((char *) tensor->data + offset, value, size), return);
     HIP_TRY(hipStreamSynchronize(nullptr), return);
 }
@@ -261,13 +262,25 @@ static void buffer_set_tensor(ggml_backend_buffer_t buffer, struct ggml_tensor *
     HIP_TRY(hipSetDevice(ctx->device), return);
     ctx->drop_images((char *) tensor->data + offset, size);
     drop_mirrors(ctx->device, (char *) tensor->data + offset, size);
+    ctx->unwritten.written((char *) tensor->data + offset, size);
     if (!upload(ctx->device, (char *) tensor->data + offset, data, size)) {
         GGML_LOG_ERROR("ggml-mi355x: upload of %zu bytes into %s failed: %s\n", size, tensor->name, hipGetErrorString(hipGetLastError()));
     }
 }
 
+// A download or copy of memory whose value a launch folded away (the graph came in pieces and the walker saw no reader):
+// say so, and hand over NaN patterns instead of whatever the memory held.
+static bool refuse_stale_read(mi355x_buffer_ctx * ctx, const struct ggml_tensor * tensor, size_t offset, size_t size, const char * what) {
+    char name[48];
+    if (!ctx->unwritten.stale((const char *) tensor->data + offset, size, name)) return false;
+    GGML_LOG_ERROR("ggml-mi355x: %s of %s reads memory of %s, which an earlier launch folded into its consumer and never stored "
+                   "(a graph handed over in pieces?); the data is replaced by NaN. GGML_MI355X_FUSE=0 stores every result\n", what, tensor->name, name);
+    return true;
+}
+
 static void buffer_get_tensor(ggml_backend_buffer_t buffer, const struct ggml_tensor * tensor, void * data, size_t offset, size_t size) {
     mi355x_buffer_ctx * ctx = (mi355x_buffer_ctx *) buffer->context;
+    if (refuse_stale_read(ctx, tensor, offset, size, "a download")) { memset(data, 0xff, size); return; }
     if (download_from_mirror(ctx->device, tensor, data, offset, size)) { count_download(ctx->device, tensor->data); return; }
     HIP_TRY(hipSetDevice(ctx->device), return);
     HIP_TRY(hipMemcpy(data, (const char *) tensor->data + offset, size, hipMemcpyDeviceToHost), return);
@@ -290,7 +303,13 @@ static bool buffer_cpy_tensor(ggml_backend_buffer_t buffer, const struct ggml_te
     HIP_TRY(hipSetDevice(ctx->device), return false);
     ctx->drop_images(dst->data, ggml_nbytes(dst));
     drop_mirrors(ctx->device, dst->data, ggml_nbytes(dst));
+    ctx->unwritten.written(dst->data, ggml_nbytes(dst));
     if (buffer_is_mi355x(sbuf)) {
+        if (refuse_stale_read((mi355x_buffer_ctx *) sbuf->context, src, 0, ggml_nbytes(src), "a copy")) {
+            HIP_TRY(hipMemset(dst->data, 0xff, ggml_nbytes(dst)), return false);
+            HIP_TRY(hipStreamSynchronize(nullptr), return false);
+            return true;
+        }
         const int sdev = ((mi355x_buffer_ctx *) sbuf->context)->device;
         if (sdev != ctx->device) {                          // uploads queued on the other device's null stream come first
             HIP_TRY(hipSetDevice(sdev), return false);
@@ -310,6 +329,7 @@ static void buffer_clear(ggml_backend_buffer_t buffer, uint8_t value) {
     HIP_TRY(hipSetDevice(ctx->device), return);
     ctx->drop_all_images();
     drop_mirrors(ctx->device, ctx->base, ctx->size);
+    ctx->unwritten.clear();
     HIP_TRY(hipMemset(ctx->base, value, ctx->size), return);
     HIP_TRY(hipDeviceSynchronize(), return);
 }
@@ -464,14 +484,17 @@ static void backend_set_tensor_async(ggml_backend_t backend, struct ggml_tensor 
     if (buffer_is_mi355x(buf)) {
         mi355x_buffer_ctx * bctx = (mi355x_buffer_ctx *) buf->context;
         bctx->drop_images((char *) tensor->data + offset, size);
+        bctx->unwritten.written((char *) tensor->data + offset, size);
     }
-    ctx->mirror_drop((char *) tensor->data + offset, size);
+    drop_mirrors(ctx->device, (char *) tensor->data + offset, size);          // (of every instance on the device, like the buffer-level writers)
     HIP_TRY(hipMemcpyAsync((char *) tensor->data + offset, data, size, hipMemcpyHostToDevice, ctx->stream), return);
 }
 
 static void backend_get_tensor_async(ggml_backend_t backend, const struct ggml_tensor * tensor, void * data, size_t offset, size_t size) {
     mi355x_backend_ctx * ctx = (mi355x_backend_ctx *) backend->context;
     HIP_TRY(hipSetDevice(ctx->device), return);
+    ggml_backend_buffer_t buf = tensor->view_src ? tensor->view_src->buffer : tensor->buffer;
+    if (buffer_is_mi355x(buf) && refuse_stale_read((mi355x_buffer_ctx *) buf->context, tensor, offset, size, "a download")) { memset(data, 0xff, size); return; }
     HIP_TRY(hipMemcpyAsync(data, (const char *) tensor->data + offset, size, hipMemcpyDeviceToHost, ctx->stream), return);
 }
 
@@ -529,8 +552,10 @@ static ggml_backend_t device_init_backend(ggml_backend_dev_t dev, const char *) 
     ctx->profile = env_flag("GGML_MI355X_PROFILE", false);
     ctx->exact   = env_flag("GGML_MI355X_EXACT", false);
     if (const char * e = getenv("GGML_MI355X_FA_ACCUM")) { const int v = atoi(e); if (v >= 0 && v <= 3) ctx->fa_accum = v; }
+    if (const char * e = getenv("GGML_MI355X_FA_CHAIN")) { const int v = atoi(e); if (v >= 0 && v <= 1) ctx->fa_chain = v; }
     ctx->weight_images = env_flag("GGML_MI355X_WEIGHT_IMAGES", true);
     ctx->dead_f32 = env_flag("GGML_MI355X_DEAD_F32", true);
+    ctx->check_reads = env_flag("GGML_MI355X_CHECK_READS", true);
     ctx->debug   = env_flag("GGML_MI355X_DEBUG", false);
     // default priority, blocking with respect to the null stream used by the buffer-level copies
     HIP_TRY(hipStreamCreate(&ctx->stream), { delete ctx; return NULL; });
@@ -614,15 +639,17 @@ static void ctx_synchronize(mi355x_backend_ctx * ctx) {
 static int set_option(ggml_backend_t backend, const char * name, int value) {
     if (!name || (backend && !ggml_backend_is_mi355x(backend))) return -1;
     const bool is_fuse = strcmp(name, "fuse") == 0, is_profile = strcmp(name, "profile") == 0, is_exact = strcmp(name, "exact") == 0;
-    const bool is_accum = strcmp(name, "fa_accum") == 0;
-    if (!is_fuse && !is_profile && !is_exact && !is_accum) return -1;
+    const bool is_accum = strcmp(name, "fa_accum") == 0, is_chain = strcmp(name, "fa_chain") == 0;
+    if (!is_fuse && !is_profile && !is_exact && !is_accum && !is_chain) return -1;
     if (is_accum && (value < 0 || value > 3)) return -1;
+    if (is_chain && (value < 0 || value > 1)) return -1;
     std::lock_guard<std::mutex> lock(g_live_mutex);
     for (mi355x_backend_ctx * ctx : g_live) {
         if (backend && ctx != (mi355x_backend_ctx *) backend->context) continue;
         if (is_fuse) ctx->fuse = value != 0;
         else if (is_exact) ctx->exact = value != 0;
         else if (is_accum) ctx->fa_accum = value;
+        else if (is_chain) ctx->fa_chain = value;
         else { ctx_synchronize(ctx); ctx->profile = value != 0; }
     }
     return 0;

@@ -10,8 +10,10 @@
 //     MUL_MAT [-> ADD | -> SCALE] -> CPY(f32 -> f16, dense)        (src/whisper.cpp:2316-2351, 2564-2601)
 #include "backend.h"
 
+#include <stdlib.h>
 #include <string.h>
 #include <algorithm>
+#include <string>
 #include <chrono>
 #include <unordered_map>
 
@@ -38,9 +40,28 @@ static bool is_view_op(enum ggml_op op) {
 // scheduler's CPU fallback (ggml/src/ggml-backend.cpp:1013-1034).
 // ------------------------------------------------------------------------------------------------------
 
+// GGML_MI355X_DECLINE=GELU,SCALE: ops (ggml_op_name, or ggml_unary_op_name for unary ops) that supports_op turns down although
+// a kernel exists.  The scheduler then places them on the CPU backend and every graph reaches this backend as several
+// ggml_graph_view pieces with copies in between (ggml/src/ggml-backend.cpp:1013-1034, 1196-1215) — the way to exercise that
+// contract with whisper's own graphs.
+static bool declined(const struct ggml_tensor * op) {
+    static const std::string list = [] { const char * e = getenv("GGML_MI355X_DECLINE"); return std::string(e ? e : ""); }();
+    if (list.empty() || is_view_op(op->op)) return false;
+    const char * name = op->op == GGML_OP_UNARY ? ggml_unary_op_name(ggml_get_unary_op(op)) : ggml_op_name(op->op);
+    const size_t len = strlen(name);
+    for (size_t at = 0; at < list.size();) {
+        size_t end = list.find(',', at);
+        if (end == std::string::npos) end = list.size();
+        if (end - at == len && list.compare(at, len, name) == 0) return true;
+        at = end + 1;
+    }
+    return false;
+}
+
 bool mi355x_supports_op(const struct ggml_tensor * op) {
     const ggml_tensor * s0 = op->src[0];
     const ggml_tensor * s1 = op->src[1];
+    if (declined(op)) return false;
     switch (op->op) {
         case GGML_OP_NONE: case GGML_OP_RESHAPE: case GGML_OP_VIEW: case GGML_OP_PERMUTE: case GGML_OP_TRANSPOSE:
             return true;
@@ -240,12 +261,48 @@ struct graph_runner {
 
     // `t` is read by exactly one node of the graph and is not a graph output
     bool only_feeds_next(const ggml_tensor * t) const {
-        if (t->flags & GGML_TENSOR_FLAG_OUTPUT) return false;
+        if ((t->flags & GGML_TENSOR_FLAG_OUTPUT) || ctx->pieces) return false;
         auto it = readers.find(t);
         return it != readers.end() && it->second == 1;
     }
 
     ggml_tensor * node_at(int i) const { return i < g->n_nodes ? g->nodes[i] : nullptr; }
+
+    // Results of the launch in progress that it does not store: intermediate values folded into the launch, and results
+    // kept only as the next product's activation image.  graph_compute books them as holding no value (range_set.h).
+    std::vector<const ggml_tensor *> not_stored;
+    // activations that the launch in progress took from their image in the workspace: it does not read their memory
+    std::vector<const ggml_tensor *> from_image;
+    // the nodes [i, i + used) folded into one launch whose result lands in `out`
+    void fold_nodes(int i, int used, const ggml_tensor * out) {
+        for (int k = i; k < i + used; ++k) {
+            const ggml_tensor * n = g->nodes[k];
+            if (n != out && !is_view_op(n->op) && !ggml_is_empty(n)) not_stored.push_back(n);
+        }
+    }
+
+    // every reader of `key` is a product over it (src1), and they are the next launches, one after the other, each with
+    // whatever it folds in; none but the last of them replaces the workspace image by one of its own result.  Only then
+    // can the producer of `key` write the image and nothing else: the image is there for each of them.
+    bool readers_are_the_next_products(const ggml_tensor * key, int from) const {
+        if (ctx->pieces) return false;
+        auto it = readers.find(key);
+        const int want = it == readers.end() ? 0 : it->second;
+        int served = 0, j = from;
+        while (served < want) {
+            while (node_at(j) && (is_view_op(node_at(j)->op) || ggml_is_empty(node_at(j)))) {
+                if (node_at(j)->src[0] == key || node_at(j)->view_src == key) return false;     // a view of it: another way to read it
+                ++j;
+            }
+            const ggml_tensor * n = node_at(j);
+            if (!n || n->op != GGML_OP_MUL_MAT || n->src[1] != key || n->src[0] == key) return false;
+            const mm_chain c = plan_chain(j);
+            ++served;
+            j += c.used;
+            if (served < want && image_consumer(c.out, j) != nullptr) return false;            // its epilogue would put another image in place
+        }
+        return want > 0;
+    }
 
     // ---- MUL_MAT and what can be folded behind it --------------------------------------------------------
     struct mm_chain {
@@ -378,6 +435,7 @@ struct graph_runner {
             status = MI355X_ERR_INVALID;
             return -1;
         }
+        if (hit) from_image.push_back(x);
         if (!hit) {
             mi355x_epilogue prep = c.epi;                 // same call as the product itself, stopped after the conversion
             prep.flags |= o.mm_flags | MI355X_MM_PREPARE_ONLY;
@@ -495,7 +553,7 @@ struct graph_runner {
             status = rc;
             note_write(held.out);
             if (rc == MI355X_OK) workspace_holds(held.key, ctx->ws_slot, 2);
-            for (const mm_chain & c : chains) note_write(c.out);
+            for (const mm_chain & c : chains) { note_write(c.out); fold_nodes((int)(std::find(g->nodes + i, g->nodes + end, c.mm) - g->nodes), c.used, c.out); }
             if (rc == MI355X_OK && q8_key) workspace_holds(q8_key, ctx->ws_slot ^ 1, 2);       // (after note_write: the image is of what was just written)
             return end - i;
         }
@@ -509,7 +567,7 @@ struct graph_runner {
         if (rc == MI355X_ERR_UNSUPPORTED) return 0;     // the single-product path takes them one by one
         status = rc;
         if (ctx->debug) GGML_LOG_INFO("ggml-mi355x: %s of %zu starting at %s, %d nodes\n", gemv ? "mul_mat.gemv_group" : "mul_mat.gemm_group", chains.size(), first.mm->name, end - i);
-        for (const mm_chain & c : chains) note_write(c.out);
+        for (const mm_chain & c : chains) { note_write(c.out); fold_nodes((int)(std::find(g->nodes + i, g->nodes + end, c.mm) - g->nodes), c.used, c.out); }
         return end - i;
     }
 
@@ -535,7 +593,7 @@ struct graph_runner {
         epi.flags |= ready;
         if (key && ctx->ws_base) { epi.flags |= MI355X_EPI_EMIT_F16; epi.image = slot_ptr(ctx->ws_slot ^ 1); } else key = nullptr;
         // ... and nothing else when the product that takes the image is the very next launch: the f32 values would have no reader
-        const bool image_only = key && ctx->dead_f32 && next_is_product_over(key, i + c.used);
+        const bool image_only = key && ctx->dead_f32 && readers_are_the_next_products(key, i + c.used);
         if (image_only) epi.flags |= MI355X_EPI_IMAGE_ONLY;
         if (ctx->debug) {
             GGML_LOG_INFO("ggml-mi355x: %s %s [%lld x %lld x %lld] folds %d nodes, flags 0x%x\n", o.kernel_name, c.mm->name,
@@ -563,7 +621,8 @@ struct graph_runner {
             }
         }
         note_write(c.out);
-        if (key && status == MI355X_OK) { workspace_holds(key, ctx->ws_slot ^ 1); if (image_only) ctx->image_only = key; }
+        fold_nodes(i, c.used, c.out);
+        if (key && status == MI355X_OK) { workspace_holds(key, ctx->ws_slot ^ 1); if (image_only && (epi.flags & MI355X_EPI_IMAGE_ONLY)) { ctx->image_only = key; not_stored.push_back(c.out); } }
         return c.used;
     }
 
@@ -636,12 +695,13 @@ struct graph_runner {
         if (!key && out->ne[0] <= 2048 && (key = image_consumer(out, i + used, true))) mode = 2;
         if (mode == 2 && nm->src[0]->ne[2] == 1 && nm->src[0]->ne[3] == 1 && next_is_product_over(key, i + used)) {
             held.active = true; held.src = nm->src[0]; held.out = out; held.key = key; held.eps = eps; held.w = w; held.b = b; held.affine = used == 3;
+            fold_nodes(i, used, out);
             return used;
         }
         const size_t image_bytes = mode == 1 ? (size_t)(out->ne[0] * out->ne[1] * 2) : (size_t)(out->ne[0] * out->ne[1] + out->ne[0] / 32 * out->ne[1] * 8);
         bool emit = key && ctx->reserve_workspace(image_bytes + 256);
         // the image and nothing else when the product that takes it is the very next launch: the f32 rows would have no reader
-        const bool image_only = emit && mode == 1 && ctx->dead_f32 && next_is_product_over(key, i + used);
+        const bool image_only = emit && mode == 1 && ctx->dead_f32 && readers_are_the_next_products(key, i + used);
         {
             launch_scope ls(ctx, used == 3 ? (emit ? "norm_affine_emit" : "norm_affine") : "norm", nbytes_of(nm->src[0]) + (image_only ? 0 : nbytes_of(out)) + (emit ? image_bytes : 0), 0.0);
             mi355x_tensor vo = vd;
@@ -651,7 +711,8 @@ struct graph_runner {
         }
         if (emit && status == MI355X_ERR_UNSUPPORTED) { emit = false; status = mi355x_norm(&vs, &vd, eps, w, b, ctx->stream); }
         note_write(out);
-        if (emit && status == MI355X_OK) { workspace_holds(key, ctx->ws_slot, mode); if (image_only) ctx->image_only = key; }
+        fold_nodes(i, used, out);
+        if (emit && status == MI355X_OK) { workspace_holds(key, ctx->ws_slot, mode); if (image_only) { ctx->image_only = key; not_stored.push_back(out); } }
         return used;
     }
 
@@ -765,7 +826,7 @@ struct graph_runner {
                                 launch_scope ls(ctx, "get_rows_add", 3.0 * nbytes_of(add), 0.0);
                                 rc = mi355x_get_rows_add(&a, &ia, &b, &ib, &d, ctx->stream);
                             }
-                            if (rc != MI355X_ERR_UNSUPPORTED) { status = rc; note_write(add); return k - i + 1; }
+                            if (rc != MI355X_ERR_UNSUPPORTED) { status = rc; note_write(add); fold_nodes(i, k - i + 1, add); return k - i + 1; }
                         }
                     }
                 }
@@ -792,7 +853,7 @@ struct graph_runner {
                 const double bytes = (double) ggml_nelements(s0) * 4 + 2.0 * (double) k->ne[0] * k->ne[1] * k->ne[2] * k->ne[3] * 2 + nbytes_of(n);
                 // the accumulation option, bit 0: more than 8 queries, bit 1: a decode step's few queries
                 const bool f32_accum = s0->ne[1] > 8 ? (ctx->fa_accum & 1) != 0 : (ctx->fa_accum & 2) != 0;
-                const int mode = ctx->exact || f32_accum ? MI355X_FA_F32 : MI355X_FA_F16_SEQ;
+                const int mode = ctx->exact || f32_accum ? MI355X_FA_F32 : ctx->fa_chain == 1 && s0->ne[1] > 8 ? MI355X_FA_F16_PK : MI355X_FA_F16_SEQ;
                 const char * name = mi355x_flash_attn_ext_kernel_name(&vq, &vk, mode);
                 // the output projection that follows takes its Q8_0-rounded activations from the attention kernel itself
                 const bool emits = !ctx->exact && (strncmp(name, "flash_attn.seq_tile", 19) == 0 || strcmp(name, "flash_attn.mfma_f32") == 0);
@@ -803,7 +864,7 @@ struct graph_runner {
                 const size_t image_bytes = form == 1 ? (size_t) ggml_nelements(n) * 2 : (size_t) ggml_nelements(n) / 32 * 40;
                 if (key && !ctx->reserve_workspace(image_bytes + 256)) key = nullptr;
                 // ... and only the image when the projection is the very next launch: the f32 rows would have no reader
-                const bool image_only = key && form == 1 && ctx->dead_f32 && strncmp(name, "flash_attn.seq_tile", 19) == 0 && next_is_product_over(key, i + 1);
+                const bool image_only = key && form == 1 && ctx->dead_f32 && strncmp(name, "flash_attn.seq_tile", 19) == 0 && readers_are_the_next_products(key, i + 1);
                 if (image_only) vd.data = nullptr;
                 {
                     launch_scope ls(ctx, name, bytes - (image_only ? nbytes_of(n) : 0) + (key ? image_bytes : 0), flops);
@@ -815,7 +876,7 @@ struct graph_runner {
                     status = mi355x_flash_attn_ext(&vq, &vk, &vv, m ? &vm : nullptr, &vd, scale, flags,
                                                    key ? ctx->ws : nullptr, key ? ctx->ws_size : 0, ctx->stream);
                 }
-                if (key && status == MI355X_OK) { workspace_holds(key, ctx->ws_slot, form); if (image_only) ctx->image_only = key; }
+                if (key && status == MI355X_OK) { workspace_holds(key, ctx->ws_slot, form); if (image_only) { ctx->image_only = key; not_stored.push_back(n); } }
                 return 1;
             }
             case GGML_OP_CONCAT: {
@@ -832,6 +893,49 @@ struct graph_runner {
 };
 
 } // namespace
+
+static mi355x_buffer_ctx * buffer_ctx_of(const ggml_tensor * t) {
+    ggml_backend_buffer_t b = t->buffer ? t->buffer : t->view_src ? t->view_src->buffer : nullptr;
+    return mi355x_buffer_is_ours(b) ? (mi355x_buffer_ctx *) b->context : nullptr;
+}
+
+// The nodes [i, i + used) went out as one launch.  What they read from outside the launch must hold a value; what they
+// did not store holds none from now on; everything else they produced does.  False: a source was memory that an earlier
+// launch had left unwritten — the graph reaches this backend in pieces, and the piece before had no sight of this reader.
+static bool book_reads_and_writes(mi355x_backend_ctx * ctx, const ggml_cgraph * g, int i, int used, const std::vector<const ggml_tensor *> & not_stored,
+                                  const std::vector<const ggml_tensor *> & from_image) {
+    for (int k = i; k < i + used; ++k) {
+        const ggml_tensor * n = g->nodes[k];
+        if (is_view_op(n->op) || ggml_is_empty(n)) continue;
+        for (int s = 0; s < GGML_MAX_SRC; ++s) {
+            const ggml_tensor * src = n->src[s];
+            if (!src || !src->data) continue;
+            const ggml_tensor * root = src;
+            while (root->view_src) root = root->view_src;
+            bool inside = false;                          // produced by this very launch
+            for (int j = i; j < k && !inside; ++j) inside = g->nodes[j] == src || g->nodes[j] == root;
+            if (inside || (n->op == GGML_OP_CPY && s == 1)) continue;       // (a CPY's second source is its destination)
+            if (n->op == GGML_OP_MUL_MAT && s == 1 && std::find(from_image.begin(), from_image.end(), src) != from_image.end()) continue;
+            mi355x_buffer_ctx * b = buffer_ctx_of(src);
+            char name[48];
+            if (b && b->unwritten.stale(src->data, ggml_nbytes(src), name)) {
+                GGML_LOG_ERROR("ggml-mi355x: %s (%s) reads %s, which lies in memory of %s: an earlier launch folded that result into its consumer "
+                               "and never stored it. The graph reaches this backend in pieces; from now on this instance stores every result "
+                               "(run the graph again)\n", ggml_op_desc(n), n->name, src->name, name);
+                ctx->pieces = true;
+                return false;
+            }
+        }
+    }
+    for (const ggml_tensor * t : not_stored) if (mi355x_buffer_ctx * b = buffer_ctx_of(t)) b->unwritten.add(t->data, ggml_nbytes(t), t->name);
+    for (int k = i; k < i + used; ++k) {
+        const ggml_tensor * n = g->nodes[k];
+        if (is_view_op(n->op) || ggml_is_empty(n) || std::find(not_stored.begin(), not_stored.end(), n) != not_stored.end()) continue;
+        const ggml_tensor * w = n->op == GGML_OP_CPY ? n->src[1] : n;
+        if (mi355x_buffer_ctx * b = buffer_ctx_of(w)) b->unwritten.written(w->data, ggml_nbytes(w));
+    }
+    return true;
+}
 
 static int64_t host_now_ns() {
     return std::chrono::duration_cast<std::chrono::nanoseconds>(std::chrono::steady_clock::now().time_since_epoch()).count();
@@ -852,12 +956,14 @@ enum ggml_status mi355x_graph_compute(mi355x_backend_ctx * ctx, struct ggml_cgra
     graph_runner run(ctx, cgraph);
     for (int i = 0; i < cgraph->n_nodes;) {
         int status = MI355X_OK;
+        run.not_stored.clear(); run.from_image.clear();
         const int used = run.run_node(i, status);
         if (status != MI355X_OK) {
             const ggml_tensor * n = cgraph->nodes[i];
             GGML_LOG_ERROR("ggml-mi355x: %s (%s) failed: %s\n", ggml_op_desc(n), n->name, mi355x_status_string(status));
             return GGML_STATUS_FAILED;
         }
+        if (ctx->check_reads && !book_reads_and_writes(ctx, cgraph, i, used, run.not_stored, run.from_image)) return GGML_STATUS_FAILED;
         i += used;
     }
     if (const int status = run.flush_norm()) {               // a LayerNorm at the very end of a graph

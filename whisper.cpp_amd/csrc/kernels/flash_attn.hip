@@ -21,6 +21,7 @@
 //       k_fattn_mfma       N > 8:  both products on the matrix cores, online softmax, probabilities as f16 operands
 //       k_fattn_vec        N <= 8: one wavefront per (query, head), keys split across lanes
 #include "common.h"
+#include <atomic>
 
 #define FA_D 64
 
@@ -209,6 +210,91 @@ __device__ __forceinline__ half2_t seq_scale2(half2_t acc, float ms) {
     asm("v_fma_mix_f32 %0, %2, %3, 0 op_sel_hi:[1,0,0]\n\t"
         "v_fma_mix_f32 %1, %2, %3, 0 op_sel:[1,0,0] op_sel_hi:[1,0,0]" : "=&v"(lo), "=&v"(hi) : "v"(acc), "v"(ms));
     asm("v_cvt_pk_f16_f32 %0, %1, %2" : "=v"(r) : "v"(lo), "v"(hi));
+    return r;
+}
+
+// ---- the packed-f16 form of the same chain (MI355X_FA_F16_PK) ----
+// The reference's builds with f16 vector arithmetic (Arm: GGML_F16_VEC_FMA = vfmaq_f16, GGML_F16_VEC_SET1 = vdupq_n_f16,
+// ggml/src/ggml-cpu/simd-mappings.h:68-105 under vec.h:180-203 and :295-311) round the factor to f16 once per key and do
+// the step as one fused f16 multiply-add per element: acc = f16(acc + v * f16(vs)), a rescale as acc = f16(acc * f16(ms)).
+// The accumulator is rounded to f16 after every key as in the f32-fma form; a step differs from that form by the factor's
+// rounding (2^-12 of an increment that is itself a small part of the sum) and by one rounding instead of two.  On gfx950
+// that is v_pk_fma_f16, two elements per instruction.
+//
+// One key for a lane that owns 4 queries x 4 d: acc[2 q + j] holds d pair j of query q, v the key's two d pairs, f[q] the
+// factors of two consecutive keys for query q as two f16; SEL picks the first or the second of them for both elements.
+template <int SEL>
+__device__ __forceinline__ void pk_mad8(half2_t (&acc)[8], const uint32_t v0, const uint32_t v1, const u32x4 f) {
+    if (SEL == 0) {
+        asm("v_pk_fma_f16 %0, %8, %10, %0 op_sel_hi:[1,0,1]\n\t"
+            "v_pk_fma_f16 %2, %8, %11, %2 op_sel_hi:[1,0,1]\n\t"
+            "v_pk_fma_f16 %4, %8, %12, %4 op_sel_hi:[1,0,1]\n\t"
+            "v_pk_fma_f16 %6, %8, %13, %6 op_sel_hi:[1,0,1]\n\t"
+            "v_pk_fma_f16 %1, %9, %10, %1 op_sel_hi:[1,0,1]\n\t"
+            "v_pk_fma_f16 %3, %9, %11, %3 op_sel_hi:[1,0,1]\n\t"
+            "v_pk_fma_f16 %5, %9, %12, %5 op_sel_hi:[1,0,1]\n\t"
+            "v_pk_fma_f16 %7, %9, %13, %7 op_sel_hi:[1,0,1]"
+            : "+v"(acc[0]), "+v"(acc[1]), "+v"(acc[2]), "+v"(acc[3]), "+v"(acc[4]), "+v"(acc[5]), "+v"(acc[6]), "+v"(acc[7])
+            : "v"(v0), "v"(v1), "v"(f.x), "v"(f.y), "v"(f.z), "v"(f.w));
+    } else {
+        asm("v_pk_fma_f16 %0, %8, %10, %0 op_sel:[0,1,0] op_sel_hi:[1,1,1]\n\t"
+            "v_pk_fma_f16 %2, %8, %11, %2 op_sel:[0,1,0] op_sel_hi:[1,1,1]\n\t"
+            "v_pk_fma_f16 %4, %8, %12, %4 op_sel:[0,1,0] op_sel_hi:[1,1,1]\n\t"
+            "v_pk_fma_f16 %6, %8, %13, %6 op_sel:[0,1,0] op_sel_hi:[1,1,1]\n\t"
+            "v_pk_fma_f16 %1, %9, %10, %1 op_sel:[0,1,0] op_sel_hi:[1,1,1]\n\t"
+            "v_pk_fma_f16 %3, %9, %11, %3 op_sel:[0,1,0] op_sel_hi:[1,1,1]\n\t"
+            "v_pk_fma_f16 %5, %9, %12, %5 op_sel:[0,1,0] op_sel_hi:[1,1,1]\n\t"
+            "v_pk_fma_f16 %7, %9, %13, %7 op_sel:[0,1,0] op_sel_hi:[1,1,1]"
+            : "+v"(acc[0]), "+v"(acc[1]), "+v"(acc[2]), "+v"(acc[3]), "+v"(acc[4]), "+v"(acc[5]), "+v"(acc[6]), "+v"(acc[7])
+            : "v"(v0), "v"(v1), "v"(f.x), "v"(f.y), "v"(f.z), "v"(f.w));
+    }
+}
+// acc = f16(acc * ms): m[q] holds -ms of query q in the half SEL picks (the sign is taken off by the instruction)
+template <int SEL>
+__device__ __forceinline__ void pk_scale8(half2_t (&acc)[8], const u32x4 m) {
+    if (SEL == 0) {
+        asm("v_pk_mul_f16 %0, %0, %8 op_sel_hi:[1,0] neg_lo:[0,1] neg_hi:[0,1]\n\t"
+            "v_pk_mul_f16 %2, %2, %9 op_sel_hi:[1,0] neg_lo:[0,1] neg_hi:[0,1]\n\t"
+            "v_pk_mul_f16 %4, %4, %10 op_sel_hi:[1,0] neg_lo:[0,1] neg_hi:[0,1]\n\t"
+            "v_pk_mul_f16 %6, %6, %11 op_sel_hi:[1,0] neg_lo:[0,1] neg_hi:[0,1]\n\t"
+            "v_pk_mul_f16 %1, %1, %8 op_sel_hi:[1,0] neg_lo:[0,1] neg_hi:[0,1]\n\t"
+            "v_pk_mul_f16 %3, %3, %9 op_sel_hi:[1,0] neg_lo:[0,1] neg_hi:[0,1]\n\t"
+            "v_pk_mul_f16 %5, %5, %10 op_sel_hi:[1,0] neg_lo:[0,1] neg_hi:[0,1]\n\t"
+            "v_pk_mul_f16 %7, %7, %11 op_sel_hi:[1,0] neg_lo:[0,1] neg_hi:[0,1]"
+            : "+v"(acc[0]), "+v"(acc[1]), "+v"(acc[2]), "+v"(acc[3]), "+v"(acc[4]), "+v"(acc[5]), "+v"(acc[6]), "+v"(acc[7])
+            : "v"(m.x), "v"(m.y), "v"(m.z), "v"(m.w));
+    } else {
+        asm("v_pk_mul_f16 %0, %0, %8 op_sel:[0,1] op_sel_hi:[1,1] neg_lo:[0,1] neg_hi:[0,1]\n\t"
+            "v_pk_mul_f16 %2, %2, %9 op_sel:[0,1] op_sel_hi:[1,1] neg_lo:[0,1] neg_hi:[0,1]\n\t"
+            "v_pk_mul_f16 %4, %4, %10 op_sel:[0,1] op_sel_hi:[1,1] neg_lo:[0,1] neg_hi:[0,1]\n\t"
+            "v_pk_mul_f16 %6, %6, %11 op_sel:[0,1] op_sel_hi:[1,1] neg_lo:[0,1] neg_hi:[0,1]\n\t"
+            "v_pk_mul_f16 %1, %1, %8 op_sel:[0,1] op_sel_hi:[1,1] neg_lo:[0,1] neg_hi:[0,1]\n\t"
+            "v_pk_mul_f16 %3, %3, %9 op_sel:[0,1] op_sel_hi:[1,1] neg_lo:[0,1] neg_hi:[0,1]\n\t"
+            "v_pk_mul_f16 %5, %5, %10 op_sel:[0,1] op_sel_hi:[1,1] neg_lo:[0,1] neg_hi:[0,1]\n\t"
+            "v_pk_mul_f16 %7, %7, %11 op_sel:[0,1] op_sel_hi:[1,1] neg_lo:[0,1] neg_hi:[0,1]"
+            : "+v"(acc[0]), "+v"(acc[1]), "+v"(acc[2]), "+v"(acc[3]), "+v"(acc[4]), "+v"(acc[5]), "+v"(acc[6]), "+v"(acc[7])
+            : "v"(m.x), "v"(m.y), "v"(m.z), "v"(m.w));
+    }
+}
+// A key at which some query of the wavefront has a new maximum.  The factor tile marks such a (query, key) by its sign:
+// -ms in place of vs (then vs is exactly 1).  The queries that stay as they are multiply by 1, which leaves the value.
+template <int SEL>
+__device__ __forceinline__ void pk_key_with_rescale(half2_t (&acc)[8], const uint32_t v0, const uint32_t v1, const u32x4 f) {
+    u32x4 vs, msn;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        const uint32_t w = f[q];
+        const bool raised = SEL ? (int32_t) w < 0 : (w & 0x8000u) != 0;
+        vs[q]  = raised ? 0x3c003c00u : w;                 // 1.0
+        msn[q] = raised ? w : 0xbc00bc00u;                 // -1.0
+    }
+    pk_scale8<SEL>(acc, msn);
+    pk_mad8<SEL>(acc, v0, v1, vs);
+}
+// two f32 factors -> one register of two f16 (round to nearest even, as the conversion in front of vdupq_n_f16)
+__device__ __forceinline__ uint32_t pk_factors(float f0, float f1) {
+    uint32_t r;
+    asm("v_cvt_pk_f16_f32 %0, %1, %2" : "=v"(r) : "v"(f0), "v"(f1));
     return r;
 }
 
@@ -839,6 +925,282 @@ __global__ void __launch_bounds__(512, 2) k_fattn_seq_tile(fa_args a) {
 }
 
 // ------------------------------------------------------------------------------------------------------
+// k_fattn_pk_tile: the tile kernel for the packed-f16 form of the step (MI355X_FA_F16_PK).
+//
+// Same roles, tiles and barriers as k_fattn_seq_tile.  With 8 instead of 24 vector instructions per key the chains of
+// that kernel's layout (a lane = one query x 16 d, every lane reading the key's 32 bytes of V) are bound by the LDS
+// reads, not by the vector units: a V register that arrives serves one instruction.  Here a lane owns 4 queries x 4 d
+// (lane = query quad l / 16 of the wavefront's 16 queries, d slice l % 16), so a key costs it one 8-byte read of V for
+// 8 instructions, and the factors arrive as f16, two keys to a register and the four queries of the quad side by side:
+// one 16-byte read per pair of keys.  Per key and lane 12 bytes from LDS instead of 36.
+//   factor tile  fp[key pair][query ^ swizzle]: 32 rows of 64 registers, each register the factors of keys 2 p, 2 p + 1
+//                for one query (vs, or -ms where the key raises that query's maximum); the producers' thread (query,
+//                16-key run) writes a column piece of 8, and the swizzle (bit 4 of the query index flipped in the rows
+//                of odd runs) spreads a wavefront's 64 writes over all banks twice instead of 16 banks four times
+//   raise masks  per chain wavefront and tile 64 bits: does key k raise the maximum of any of its 16 queries?  Built
+//                by the producer wavefront that has the same 16 queries; the chain tests them with scalar
+//                instructions, so a pair of keys without a raise costs its 16 multiply-adds and nothing else.
+// ------------------------------------------------------------------------------------------------------
+
+#define P_FP_ROW   T_Q                                    // registers per key-pair row of the factor tile
+#define P_FP_TILE  ((T_KV / 2) * P_FP_ROW)
+#define P_LDS_BYTES ((T_Q * T_LDH + T_KV * T_LDH + 2 * T_KV * FA_D) * 2 + T_Q * T_LDF * 4 + 2 * P_FP_TILE * 4 + 2 * 4 * 2 * 4 + 2 * T_Q * 4)   // 69184
+
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+__global__ void __launch_bounds__(512, 2) k_fattn_pk_tile(fa_args a) {
+    extern __shared__ __attribute__((aligned(16))) char t_smem[];
+    half_t *   q_s  = (half_t *) t_smem;                      // [T_Q * T_LDH]
+    half_t *   k_s  = q_s + T_Q * T_LDH;                      // [T_KV * T_LDH]
+    half_t *   v_s2 = k_s + T_KV * T_LDH;                     // [2][T_KV * FA_D]
+    float *    sc_s = (float *)(v_s2 + 2 * T_KV * FA_D);      // [T_Q * T_LDF]   scores of the tile in work (producers only)
+    uint32_t * fp_s = (uint32_t *)(sc_s + T_Q * T_LDF);       // [2][P_FP_TILE]
+    uint32_t * rm_s = fp_s + 2 * P_FP_TILE;                   // [2][4][2]
+    float *    m_run = (float *)(rm_s + 16), * s_run = m_run + T_Q;
+
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    // an XCD gets one run of consecutive (head, query tile) pairs, head-major, so that a head's K and V stay in one or two L2s
+    const uint32_t lin = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z), total = gridDim.x * gridDim.y * gridDim.z;
+    const uint32_t xcd = lin % 8, per = total / 8, extra = total % 8;
+    const uint32_t item = xcd * per + (xcd < extra ? xcd : extra) + lin / 8;
+    const int64_t n0 = (int64_t)(item % gridDim.x) * T_Q, h = (item / gridDim.x) % gridDim.y, i3 = item / (gridDim.x * gridDim.y);
+    const int n_tiles = (int)((a.KV + T_KV - 1) / T_KV);
+
+    if (wave >= 4) {
+        // ---- producers ---------------------------------------------------------------------------------------------------------------
+        const int tid = threadIdx.x - 256, pw = wave - 4;
+        const char * qb = a.q + h * a.q_nb2 + i3 * a.q_nb3;
+        const char * kb = a.k + (h / a.hk_ratio) * a.k_nb2 + (i3 / a.k_ne3_ratio) * a.k_nb3;
+        const char * vb = a.v + (h / a.hv_ratio) * a.v_nb2 + (i3 / a.v_ne3_ratio) * a.v_nb3;
+        {   // Q tile -> f16 in LDS; thread t: row t/4, 16 values
+            const int r = tid >> 2, c = (tid & 3) * 16;
+            const int64_t n = n0 + r;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                float4 t = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (n < a.N) t = *(const float4 *)(qb + n * a.q_nb1 + (c + 4 * i) * 4);
+                half4_t hq = { (half_t) t.x, (half_t) t.y, (half_t) t.z, (half_t) t.w };
+                *(half4_t *)(q_s + r * T_LDH + c + 4 * i) = hq;
+            }
+        }
+        if (tid < T_Q) { m_run[tid] = -INFINITY; s_run[tid] = 0.0f; }
+
+        const int sq = (pw >> 1) * 32, sk = (pw & 1) * 32, l32 = lane & 31, g = lane >> 5;
+        const int kr = tid >> 2, kc = (tid & 3) * 16;
+        u32x4 kreg0, kreg1, vreg0, vreg1;
+        auto load_kv = [&](int64_t key0) __attribute__((always_inline)) {
+            const int64_t key = key0 + kr < a.KV ? key0 + kr : a.KV - 1;      // rows past the end repeat the last key; their scores are masked
+            const u32x4 * kp = (const u32x4 *)(kb + key * a.k_nb1 + kc * 2);
+            const u32x4 * vp = (const u32x4 *)(vb + key * a.v_nb1 + kc * 2);
+            kreg0 = kp[0]; kreg1 = kp[1]; vreg0 = vp[0]; vreg1 = vp[1];
+        };
+        load_kv(0);
+        *(u32x4 *)(k_s + kr * T_LDH + kc) = kreg0; *(u32x4 *)(k_s + kr * T_LDH + kc + 8) = kreg1;
+
+        for (int it = 0; it <= n_tiles; ++it) {
+            __syncthreads();                               // tile boundary
+            if (it == n_tiles) { __syncthreads(); break; }
+            const int64_t key0 = (int64_t) it * T_KV;
+            half_t * vs_buf = v_s2 + (it & 1) * T_KV * FA_D;
+            *(u32x4 *)(vs_buf + kr * FA_D + kc) = vreg0; *(u32x4 *)(vs_buf + kr * FA_D + kc + 8) = vreg1;
+            if (it + 1 < n_tiles) load_kv(key0 + T_KV);
+
+            {   // ---- scores: S = Q K^T on the matrix cores
+                float16_t c16;
+#pragma unroll
+                for (int r = 0; r < 16; ++r) c16[r] = 0.0f;
+#pragma unroll
+                for (int kk = 0; kk < FA_D / 16; ++kk) {
+                    const half8_t av = *(const half8_t *)(q_s + (sq + l32) * T_LDH + kk * 16 + 8 * g);
+                    const half8_t bv = *(const half8_t *)(k_s + (sk + l32) * T_LDH + kk * 16 + 8 * g);
+                    c16 = __builtin_amdgcn_mfma_f32_32x32x16_f16(av, bv, c16, 0, 0, 0);
+                }
+                const int64_t key = key0 + sk + l32;
+                const bool key_ok = key < a.KV;
+                if (!a.mask && key0 + T_KV <= a.KV) {
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) {
+                        const int qi = sq + 8 * (r >> 2) + 4 * g + (r & 3);
+                        sc_s[qi * T_LDF + sk + l32] = __fmul_rn(c16[r], a.scale);
+                    }
+                } else {
+                    float mv[16];
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) {
+                        const int qi = sq + 8 * (r >> 2) + 4 * g + (r & 3);
+                        mv[r] = 0.0f;
+                        if (a.mask) {
+                            const int64_t n = n0 + qi < a.N ? n0 + qi : a.N - 1;
+                            mv[r] = (float) *(const half_t *)(a.mask + n * a.m_nb1 + (key_ok ? key : a.KV - 1) * 2);
+                        }
+                    }
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) {
+                        const int qi = sq + 8 * (r >> 2) + 4 * g + (r & 3);
+                        sc_s[qi * T_LDF + sk + l32] = key_ok ? __fadd_rn(__fmul_rn(c16[r], a.scale), mv[r]) : -INFINITY;
+                    }
+                }
+            }
+            __syncthreads();                               // scores visible
+
+            {   // ---- factors: thread t: query t/4, keys 16*(t%4) .. +15
+                const int qi = tid >> 2, sgm = tid & 3;
+                const float4 * sp = (const float4 *)(sc_s + qi * T_LDF + sgm * 16);
+                float sv[16], lmax = -INFINITY;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) { const float4 t = sp[i]; sv[4*i] = t.x; sv[4*i+1] = t.y; sv[4*i+2] = t.z; sv[4*i+3] = t.w; }
+#pragma unroll
+                for (int i = 0; i < 16; ++i) lmax = fmaxf(lmax, sv[i]);
+                float M = m_run[qi];
+                const float S0 = s_run[qi];
+                const float m0 = dpp_move<float, 0x00>(lmax), m1 = dpp_move<float, 0x55>(lmax), m2 = dpp_move<float, 0xAA>(lmax);
+                if (sgm > 0) M = fmaxf(M, m0);
+                if (sgm > 1) M = fmaxf(M, m1);
+                if (sgm > 2) M = fmaxf(M, m2);
+                float P = 1.0f, A = 0.0f;
+                uint32_t rbits = 0;                        // bit i: key i of this run raises this query's maximum
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    const float s = sv[i];
+                    const bool  raised = s > M;
+                    const float ex = exp_neg(-fabsf(s - M));   // M - s when raised, s - M otherwise: both <= 0 (or NaN / -inf: 0)
+                    if (__any(raised)) {
+                        const float ms = raised ? ex : 1.0f, vs = raised ? 1.0f : ex;
+                        M = raised ? s : M;
+                        P *= ms; A = A * ms + vs;
+                        sv[i] = raised ? -ex : ex;             // -0.0 keeps the sign
+                        rbits |= raised ? 1u << i : 0u;
+                    } else {
+                        A = A + ex;
+                        sv[i] = ex;
+                    }
+                }
+                // f16 factors, two keys to a register, into column (query ^ swizzle) of this run's eight key-pair rows
+                uint32_t * fpw = fp_s + (it & 1) * P_FP_TILE + (8 * sgm) * P_FP_ROW + (qi ^ ((sgm & 1) << 4));
+#pragma unroll
+                for (int j = 0; j < 8; ++j) fpw[j * P_FP_ROW] = pk_factors(sv[2*j], sv[2*j + 1]);
+                // the raise mask of the wavefront's 16 queries: OR over the lanes of a run (lane = 4 * query + run)
+                rbits |= dpp_move<uint32_t, 0x124>(rbits);     // row_ror:4
+                rbits |= dpp_move<uint32_t, 0x128>(rbits);     // row_ror:8
+                rbits |= (uint32_t) __builtin_amdgcn_ds_swizzle((int) rbits, 0x401F);       // lane ^ 16
+                rbits |= (uint32_t) __shfl_xor((int) rbits, 32, WAVE);
+                const uint32_t r1 = dpp_move<uint32_t, 0x55>(rbits), r2 = dpp_move<uint32_t, 0xAA>(rbits), r3 = dpp_move<uint32_t, 0xFF>(rbits);
+                if (lane == 0) *(u32x2 *)(rm_s + ((it & 1) * 4 + pw) * 2) = (u32x2){ rbits | (r1 << 16), r2 | (r3 << 16) };
+                // fold the four runs of this query in key order
+                const float P1 = dpp_move<float, 0x55>(P), A1 = dpp_move<float, 0x55>(A);
+                const float P2 = dpp_move<float, 0xAA>(P), A2 = dpp_move<float, 0xAA>(A);
+                const float P3 = dpp_move<float, 0xFF>(P), A3 = dpp_move<float, 0xFF>(A);
+                const float M3 = dpp_move<float, 0xFF>(M);
+                if (sgm == 0) {
+                    float S = S0 * P + A;
+                    S = S * P1 + A1; S = S * P2 + A2; S = S * P3 + A3;
+                    s_run[qi] = S; m_run[qi] = M3;
+                }
+            }
+            if (it + 1 < n_tiles) { *(u32x4 *)(k_s + kr * T_LDH + kc) = kreg0; *(u32x4 *)(k_s + kr * T_LDH + kc + 8) = kreg1; }
+        }
+        return;
+    }
+
+    // ---- chains: lane = (query quad qd, d slice ds) of the wavefront's 16 queries ----------------------------------------------------
+    __builtin_amdgcn_s_setprio(1);
+    const int qd = lane >> 4, ds = lane & 15;
+    half2_t acc[8];                                        // acc[2 q + j]: d pair j of the quad's query q
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] = (half2_t){ (half_t) 0.0f, (half_t) 0.0f };
+    const int fcol = 16 * wave + 4 * qd;
+
+    for (int it = 0; it <= n_tiles; ++it) {
+        __syncthreads();                                   // tile boundary: tile it - 1 has its factors, its masks and its V rows
+        int barriers = 0;
+        if (it > 0) {
+            const int64_t key0 = (int64_t)(it - 1) * T_KV;
+            const int nk = (int)(a.KV - key0 < T_KV ? a.KV - key0 : T_KV);       // uniform
+            const int buf = (it - 1) & 1;
+            const uint32_t * fpb = fp_s + buf * P_FP_TILE;
+            const char * vbase = (const char *)(v_s2 + buf * T_KV * FA_D) + 8 * ds;     // + key * 128
+            const u32x2 mv = *(const u32x2 *)(rm_s + (buf * 4 + wave) * 2);
+            const uint32_t mlo = __builtin_amdgcn_readfirstlane(mv.x), mhi = __builtin_amdgcn_readfirstlane(mv.y);
+            // one group = four pairs of keys: their factors (a 16-byte read per pair) and their V values (an 8-byte read per key);
+            // the next group is read while this one is walked.  (Keys past the end carry factors of exactly 0 and the last
+            // key's finite V values: walking them changes nothing, so groups are walked whole.)
+            struct pgroup { u32x4 f[4]; u32x2 v[8]; };
+            auto gload = [&](pgroup & gr, int kp0, int swz) __attribute__((always_inline)) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) gr.f[j] = *(const u32x4 *)(fpb + (kp0 + j) * P_FP_ROW + (fcol ^ swz));
+#pragma unroll
+                for (int j = 0; j < 8; ++j) gr.v[j] = *(const u32x2 *)(vbase + (2 * kp0 + j) * (FA_D * 2));
+            };
+            // bits: two per pair of keys, lowest first: does the first / the second key of the pair raise a maximum in this wavefront
+            auto walk = [&](const pgroup & gr, uint32_t bits) __attribute__((always_inline)) {
+                if (bits == 0) {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        pk_mad8<0>(acc, gr.v[2*j].x, gr.v[2*j].y, gr.f[j]);
+                        pk_mad8<1>(acc, gr.v[2*j + 1].x, gr.v[2*j + 1].y, gr.f[j]);
+                    }
+                } else {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        if (bits & (1u << (2*j))) pk_key_with_rescale<0>(acc, gr.v[2*j].x, gr.v[2*j].y, gr.f[j]);
+                        else                      pk_mad8<0>(acc, gr.v[2*j].x, gr.v[2*j].y, gr.f[j]);
+                        if (bits & (2u << (2*j))) pk_key_with_rescale<1>(acc, gr.v[2*j + 1].x, gr.v[2*j + 1].y, gr.f[j]);
+                        else                      pk_mad8<1>(acc, gr.v[2*j + 1].x, gr.v[2*j + 1].y, gr.f[j]);
+                    }
+                }
+            };
+            auto arrived = [&](const pgroup & gr) __attribute__((always_inline)) {
+                asm volatile("" :: "v"(gr.f[3].w), "v"(gr.v[7].y));
+                __builtin_amdgcn_sched_barrier(0);
+            };
+            pgroup ga, gb;
+            gload(ga, 0, 0);
+            const int n_runs = (nk + 15) >> 4;             // runs of 16 keys = 8 pairs = two groups
+            for (int u = 0; u < n_runs; ++u) {
+                const uint32_t fld = ((u & 2) ? mhi : mlo) >> (16 * (u & 1));
+                const int swz = (u & 1) << 4;
+                arrived(ga);
+                gload(gb, 8 * u + 4, swz);
+                __builtin_amdgcn_sched_barrier(0);
+                walk(ga, fld & 0xffu);
+                arrived(gb);
+                gload(ga, u < 3 ? 8 * u + 8 : 0, u < 3 ? swz ^ 16 : 0);     // (behind the last group: any readable group, nobody walks it)
+                __builtin_amdgcn_sched_barrier(0);
+                walk(gb, (fld >> 8) & 0xffu);
+                // the producers' meeting point: after 16 keys their scores are written; the other 48 keys are the time their
+                // factor step has
+                if (u == 0) { __syncthreads(); ++barriers; }
+            }
+        }
+        for (; barriers < 1; ++barriers) __syncthreads();
+    }
+
+    // ---- results: a lane holds 4 d of 4 queries
+    const int64_t nq0 = n0 + 16 * wave + 4 * qd;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        const int64_t n = nq0 + q;
+        const float inv = 1.0f / s_run[16 * wave + 4 * qd + q];
+        const float o[4] = { (float) acc[2*q][0] * inv, (float) acc[2*q][1] * inv, (float) acc[2*q + 1][0] * inv, (float) acc[2*q + 1][1] * inv };
+        if (a.d && n < a.N) *(float4 *)((float *) a.d + ((i3 * a.N + n) * a.H + h) * FA_D + 4 * ds) = make_float4(o[0], o[1], o[2], o[3]);
+        if (a.x16) {
+            // the Q8_0-rounded f16 image of the row for the projection that follows: a block is 32 d, eight lanes of a row
+            float amax = fmaxf(fmaxf(fabsf(o[0]), fabsf(o[1])), fmaxf(fabsf(o[2]), fabsf(o[3])));
+            amax = lanes_max<8>(amax);
+            if (n < a.N) {
+                const float id = amax != 0.0f ? 127.0f / amax : 0.0f;
+                const float dq = h2f(f2h_bits(amax / 127.0f));
+                half4_t hx;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) hx[e] = (half_t)((rintf(o[e] * id) + 0.0f) * dq);
+                *(half4_t *)(a.x16 + ((i3 * a.N + n) * a.H + h) * FA_D + 4 * ds) = hx;
+            }
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------------------
 // N > 8, f32 accumulators on the matrix cores (MI355X_FA_F32).
 //
 // Both products run on v_mfma_f32_32x32x16_f16, transposed so that a lane owns one query throughout:
@@ -1054,7 +1416,7 @@ extern "C" const char * mi355x_flash_attn_ext_kernel_name(const mi355x_tensor * 
     if (!q || !k) return "flash_attn.invalid";
     switch (fa_kernel(q, k, mode)) {
         case FA_K_SEQ_ROW:  return "flash_attn.seq_row";
-        case FA_K_SEQ_TILE: return "flash_attn.seq_tile";
+        case FA_K_SEQ_TILE: return mode == MI355X_FA_F16_PK ? "flash_attn.seq_tile_pk" : "flash_attn.seq_tile";
         case FA_K_MFMA:     return "flash_attn.mfma_f32";
         default:            return "flash_attn.vec_f32";
     }
@@ -1072,7 +1434,7 @@ static int flash_attn_ext(const mi355x_tensor * q, const mi355x_tensor * k, cons
     const bool emit = mode & MI355X_FA_EMIT_F16, emit_q8 = mode & MI355X_FA_EMIT_Q8_0;
     mode &= ~(MI355X_FA_EMIT_F16 | MI355X_FA_EMIT_Q8_0);
     if (emit && emit_q8) return MI355X_ERR_INVALID;
-    if (mode != MI355X_FA_F16_SEQ && mode != MI355X_FA_F32) return MI355X_ERR_INVALID;
+    if (mode != MI355X_FA_F16_SEQ && mode != MI355X_FA_F32 && mode != MI355X_FA_F16_PK) return MI355X_ERR_INVALID;
     // dst without memory: only the image is wanted (the key-by-key tile kernel with MI355X_FA_EMIT_F16)
     if (!dst->data && !(emit && fa_kernel(q, k, mode) == FA_K_SEQ_TILE)) return MI355X_ERR_INVALID;
     if (q->type != MI355X_TYPE_F32 || k->type != MI355X_TYPE_F16 || v->type != MI355X_TYPE_F16 || dst->type != MI355X_TYPE_F32) return MI355X_ERR_UNSUPPORTED;
@@ -1145,14 +1507,18 @@ static int flash_attn_ext(const mi355x_tensor * q, const mi355x_tensor * k, cons
             const int64_t gx = (N + T_Q - 1) / T_Q;
             if (gx > 0x7fffffff) return MI355X_ERR_UNSUPPORTED;
             dim3 grid((unsigned) gx, (unsigned) H, (unsigned) q->ne[3]);
-            static bool configured[64];                    // per device: the kernel asks for more LDS than a launch gets by default
+            // per device and kernel: they ask for more LDS than a launch gets by default
+            static std::atomic<bool> configured[64][2];
             int dev = 0;
             if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) { (void) hipGetLastError(); return MI355X_ERR_HIP; }
-            if (!configured[dev]) {
-                if (hipFuncSetAttribute((const void *) k_fattn_seq_tile, hipFuncAttributeMaxDynamicSharedMemorySize, (int) T_LDS_BYTES) != hipSuccess) { (void) hipGetLastError(); return MI355X_ERR_HIP; }
-                configured[dev] = true;
+            const int pk = mode == MI355X_FA_F16_PK;
+            if (!configured[dev][pk].load(std::memory_order_acquire)) {
+                const void * fn = pk ? (const void *) k_fattn_pk_tile : (const void *) k_fattn_seq_tile;
+                if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, pk ? (int) P_LDS_BYTES : (int) T_LDS_BYTES) != hipSuccess) { (void) hipGetLastError(); return MI355X_ERR_HIP; }
+                configured[dev][pk].store(true, std::memory_order_release);
             }
-            k_fattn_seq_tile<<<grid, 512, T_LDS_BYTES, st>>>(a);
+            if (pk) k_fattn_pk_tile<<<grid, 512, P_LDS_BYTES, st>>>(a);
+            else    k_fattn_seq_tile<<<grid, 512, T_LDS_BYTES, st>>>(a);
         } break;
         case FA_K_MFMA: {
             const int64_t gx = (N + M_Q - 1) / M_Q;
