@@ -138,8 +138,11 @@ MI355X_API int    mi355x_mul_mat(const mi355x_tensor * src0, const mi355x_tensor
  * more scratch than the array holds (mi355x_mul_mat_workspace_size > MI355X_MUL_MAT_NOALLOC_MAX);
  * MI355X_ERR_INVALID with MI355X_MM_WS_READY or MI355X_MM_PREPARE_ONLY (the array is shared by every call on a GPU and keeps
  * the last call's contents, so no call may rely on them).  Calls that overlap on one GPU (two streams, two threads) race
- * on the array: serialize them.  The first call on a device looks up the array's address, and the first call with
- * MI355X_EPI_GELU fills the GELU table with a synchronous copy: make those calls before a capture starts. */
+ * on the array: serialize them.  The first call on a device looks up the array's address, the first call with
+ * MI355X_EPI_GELU fills the GELU table with a synchronous copy, and the first launch of each kernel instance on a device
+ * sets its LDS size attribute (the instance follows from the operand types, the size class of M, N and K, and the epilogue
+ * flags): before a capture starts, make one call with the same types, shapes and flags as every call that will be
+ * captured. */
 #define MI355X_MUL_MAT_NOALLOC_MAX ((size_t) 32 << 20)
 MI355X_API int    mi355x_mul_mat_noalloc(const mi355x_tensor * src0, const mi355x_tensor * src1, const mi355x_tensor * dst,
                                          const mi355x_epilogue * epi, void * stream);

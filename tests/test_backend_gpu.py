@@ -216,7 +216,7 @@ def check_model_summary(s, strict_ids):
     # difference between the two logit vectors.  The reference accumulates attention in f16; one differently-rounded
     # f16 value cascades, so beyond bit-identical arithmetic the two runs are two draws of the same rounding noise and
     # a random-init model with near-flat logits can flip an argmax whose margin is inside that noise.
-    assert s["clear_ids_identical"] == s["clear_steps"], s
+    assert s["clear_steps"] >= 1 and s["clear_ids_identical"] == s["clear_steps"], s      # (never vacuous: some step stands clear of the noise)
     assert s["ids_identical"] >= (s["rows"] if strict_ids else int(0.75 * s["rows"])), s
     # nothing left the device: the scheduler reported one split per graph, all on the MI355X device, and the plugin was
     # handed exactly one graph per graph whisper computed
@@ -228,7 +228,10 @@ def check_model_summary(s, strict_ids):
                                        (("large-v3", "q5_0"), 32), (("large-v3-turbo", "q8_0"), 32)])
 def test_whole_model_logits_and_greedy_ids(harness, models, key, steps):
     rc, rows = run_harness(harness, ["model", "--model", models[key], "--steps", str(steps)], timeout=1500)
-    check_model_summary(rows[-1], strict_ids=key[0] == "base")
+    s = rows[-1]
+    print(f"{key[0]} {key[1]} model seed 1234 mel seed 7: ids {s.get('ids_identical')}/{s.get('rows')}, clear {s.get('clear_ids_identical')}/{s.get('clear_steps')}, "
+          f"worst NMSE {s.get('worst_logits_nmse', float('nan')):.2e}", flush=True)
+    check_model_summary(s, strict_ids=key[0] == "base")
     assert rc == 0
     if key == ("large-v3", "q5_0"):
         # the encoder graph of large-v3 arrives whole: 3 graphs per window, and far more nodes than launches

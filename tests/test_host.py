@@ -58,6 +58,26 @@ def test_attention_refuses_a_mask_cast_that_shares_memory_with_its_output(pkg):
     assert call(0x40000000, 0x60000000, 0x60000000) == -2              # dst over the f16 copy
 
 
+def test_norm_refuses_missing_memory(pkg):
+    # mi355x_norm_emit_f16 takes a destination without memory (image only); the plain and the Q8_0-emitting forms store
+    # through it and must say no on the host, before any launch
+    import ctypes as C
+    if not pkg.KERNELS_LIB.exists():
+        pytest.skip("kernel library not built")
+    lib = pkg.kernels()
+    class Mem:
+        def __init__(self, addr): self.addr = addr
+        def data_ptr(self): return self.addr
+    src = pkg.tensor(Mem(0x10000000), pkg.F32, ne=[1280, 5], nb=[4, 5120])
+    dst = pkg.tensor(Mem(0x20000000), pkg.F32, ne=[1280, 5], nb=[4, 5120])
+    no_dst = pkg.tensor(Mem(0x20000000), pkg.F32, ne=[1280, 5], nb=[4, 5120]); no_dst.data = None
+    no_src = pkg.tensor(Mem(0x10000000), pkg.F32, ne=[1280, 5], nb=[4, 5120]); no_src.data = None
+    assert lib.mi355x_norm(C.byref(src), C.byref(no_dst), 1e-5, None, None, None) == -2
+    assert lib.mi355x_norm(C.byref(no_src), C.byref(dst), 1e-5, None, None, None) == -2
+    assert lib.mi355x_norm_emit_q8_0(C.byref(src), C.byref(no_dst), 1e-5, None, None, 0x30000000, None) == -2
+    assert lib.mi355x_norm_emit_f16(C.byref(no_src), C.byref(no_dst), 1e-5, None, None, 0x30000000, None) == -2
+
+
 def test_plugin_exports_the_ggml_entry_points_and_does_not_link_the_checker(pkg):
     if not pkg.PLUGIN_LIB.exists():
         pytest.skip("plugin not built")

@@ -18,7 +18,7 @@
 #include "range_set.h"
 
 #define MI355X_BUFFER_ALIGN 256
-#define MI355X_N_COUNTERS   8
+#define MI355X_N_COUNTERS   10
 #define MI355X_MIRROR_MAX   (4u << 20)       // outputs larger than this are never mirrored (an encoder's states stay on the device)
 
 #define HIP_TRY(expr, on_fail)                                                                            \

@@ -104,17 +104,31 @@ static void forget_downloads(int device, const void * begin, size_t size) {
 
 // [data + offset, + size) of a tensor from the host mirror of a backend instance on this device; false: not mirrored
 static bool download_from_mirror(int device, const struct ggml_tensor * tensor, void * data, size_t offset, size_t size) {
-    std::lock_guard<std::mutex> live(g_live_mutex);
-    for (mi355x_backend_ctx * ctx : g_live) {
-        if (ctx->device != device) continue;
-        std::lock_guard<std::mutex> lock(ctx->mirror_mutex);
-        for (const mi355x_backend_ctx::mirror_entry & e : ctx->mirror) {
-            if (e.dev != (const char *) tensor->data || offset < e.lo || offset + size > e.lo + e.size) continue;
-            if (hipEventSynchronize(ctx->mirror_done) != hipSuccess) { (void) hipGetLastError(); return false; }
-            memcpy(data, ctx->mirror_host + e.off + (offset - e.lo), size);
-            ctx->counters[4] += 1;
-            return true;
+    // Find the entry under the locks, wait for its transfer without them (a host thread that reads one state's logits must
+    // not hold up the options, statistics and buffer writes of every other state for a whole graph), then look again: a
+    // write may have retired the mirror meanwhile.
+    for (int attempt = 0; attempt < 2; ++attempt) {
+        hipEvent_t done = nullptr;
+        {
+            std::lock_guard<std::mutex> live(g_live_mutex);
+            for (mi355x_backend_ctx * ctx : g_live) {
+                if (ctx->device != device) continue;
+                std::lock_guard<std::mutex> lock(ctx->mirror_mutex);
+                for (const mi355x_backend_ctx::mirror_entry & e : ctx->mirror) {
+                    if (e.dev != (const char *) tensor->data || offset < e.lo || offset + size > e.lo + e.size) continue;
+                    if (attempt == 0 && hipEventQuery(ctx->mirror_done) != hipSuccess) { (void) hipGetLastError(); done = ctx->mirror_done; break; }
+                    if (attempt == 1 && hipEventQuery(ctx->mirror_done) != hipSuccess) { (void) hipGetLastError(); return false; }
+                    memcpy(data, ctx->mirror_host + e.off + (offset - e.lo), size);
+                    ctx->counters[4] += 1;
+                    return true;
+                }
+                if (done) break;
+            }
         }
+        if (!done) return false;
+        // (the event belongs to a live instance; an instance is freed only after its host thread stopped calling into it, and a
+        // destroyed event makes the wait fail, which sends the read down the plain copy path)
+        if (hipEventSynchronize(done) != hipSuccess) { (void) hipGetLastError(); return false; }
     }
     return false;
 }
@@ -466,7 +480,9 @@ static void backend_free(ggml_backend_t backend) {
             auto & s = g_retired_stats[kv.first];
             s.calls += kv.second.calls; s.ms += kv.second.ms; s.bytes += kv.second.bytes; s.flops += kv.second.flops;
         }
-        for (int i = 0; i < MI355X_N_COUNTERS; ++i) g_retired_counters[i] += ctx->counters[i];
+        for (int i = 0; i < MI355X_N_COUNTERS; ++i) {
+            if (i == 9) g_retired_counters[i] = std::max(g_retired_counters[i], ctx->counters[i]); else g_retired_counters[i] += ctx->counters[i];
+        }
     }
     for (hipEvent_t e : ctx->event_pool) (void) hipEventDestroy(e);
     if (ctx->ws_base) (void) hipFree(ctx->ws_base);
@@ -695,9 +711,15 @@ static void get_counters(ggml_backend_t backend, int64_t out[MI355X_N_COUNTERS],
     std::lock_guard<std::mutex> lock(g_live_mutex);
     for (mi355x_backend_ctx * ctx : g_live) {
         if (backend && ctx != (mi355x_backend_ctx *) backend->context) continue;
-        for (int i = 0; i < MI355X_N_COUNTERS; ++i) { out[i] += ctx->counters[i]; if (reset) ctx->counters[i] = 0; }
+        for (int i = 0; i < MI355X_N_COUNTERS; ++i) {
+            if (i == 9) out[i] = std::max(out[i], ctx->counters[i]); else out[i] += ctx->counters[i];      // (9 is a maximum)
+            if (reset) ctx->counters[i] = 0;
+        }
     }
-    if (!backend) for (int i = 0; i < MI355X_N_COUNTERS; ++i) { out[i] += g_retired_counters[i]; if (reset) g_retired_counters[i] = 0; }
+    if (!backend) for (int i = 0; i < MI355X_N_COUNTERS; ++i) {
+        if (i == 9) out[i] = std::max(out[i], g_retired_counters[i]); else out[i] += g_retired_counters[i];
+        if (reset) g_retired_counters[i] = 0;
+    }
 }
 
 // host-memory front of mi355x_log_mel_spectrogram: one allocation for samples, filter bank, result and workspace, the

@@ -270,6 +270,7 @@ struct graph_runner {
 
     // Results of the launch in progress that it does not store: intermediate values folded into the launch, and results
     // kept only as the next product's activation image.  graph_compute books them as holding no value (range_set.h).
+    bool few_query_attention = false;   // the graph holds an attention node with at most 8 queries: a decode step
     std::vector<const ggml_tensor *> not_stored;
     // activations that the launch in progress took from their image in the workspace: it does not read their memory
     std::vector<const ggml_tensor *> from_image;
@@ -849,6 +850,7 @@ struct graph_runner {
                 float scale; memcpy(&scale, n->op_params, sizeof(float));
                 mi355x_tensor vq = to_view(s0), vk = to_view(k), vv = to_view(v), vm, vd = to_view(n);
                 if (m) vm = to_view(m);
+                if (s0->ne[1] <= 8) { few_query_attention = true; ctx->counters[9] = std::max<int64_t>(ctx->counters[9], k->ne[1]); }
                 const double flops = 4.0 * s0->ne[1] * k->ne[1] * 64.0 * s0->ne[2] * s0->ne[3];
                 const double bytes = (double) ggml_nelements(s0) * 4 + 2.0 * (double) k->ne[0] * k->ne[1] * k->ne[2] * k->ne[3] * 2 + nbytes_of(n);
                 // the accumulation option, bit 0: more than 8 queries, bit 1: a decode step's few queries
@@ -970,6 +972,7 @@ enum ggml_status mi355x_graph_compute(mi355x_backend_ctx * ctx, struct ggml_cgra
         GGML_LOG_ERROR("ggml-mi355x: trailing NORM failed: %s\n", mi355x_status_string(status));
         return GGML_STATUS_FAILED;
     }
+    ctx->counters[8] += run.few_query_attention;
     ctx->mirror_outputs(cgraph);
     return GGML_STATUS_SUCCESS;
 }

@@ -24,6 +24,7 @@
 #include <atomic>
 
 #define FA_D 64
+#define LOG2E_F 1.44269504088896340736f
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
@@ -277,19 +278,36 @@ __device__ __forceinline__ void pk_scale8(half2_t (&acc)[8], const u32x4 m) {
     }
 }
 // A key at which some query of the wavefront has a new maximum.  The factor tile marks such a (query, key) by its sign:
-// -ms in place of vs (then vs is exactly 1).  The queries that stay as they are multiply by 1, which leaves the value.
+// -ms in place of vs (then vs is exactly 1).  Rescales the accumulators — the queries that stay as they are multiply by 1,
+// which leaves the value — and puts 1 in place of -ms in the factor registers, so that the multiply-add that follows is the
+// same instruction sequence with or without a rescale.  Everything happens in the registers it finds (tied asm operands):
+// written as C++ selects, the compiler gives the changed factors or accumulators new registers and copies them back on the
+// path without a rescale, eight or four v_mov per key on the path that matters.
 template <int SEL>
-__device__ __forceinline__ void pk_key_with_rescale(half2_t (&acc)[8], const uint32_t v0, const uint32_t v1, const u32x4 f) {
-    u32x4 vs, msn;
+__device__ __forceinline__ void pk_rescale(half2_t (&acc)[8], u32x4 & f) {
+    const uint32_t keep = SEL ? 0x0000ffffu : 0xffff0000u, one = SEL ? 0x3c000000u : 0x00003c00u, neg_one = 0xbc00bc00u;
+    u32x4 msn;
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
-        const uint32_t w = f[q];
-        const bool raised = SEL ? (int32_t) w < 0 : (w & 0x8000u) != 0;
-        vs[q]  = raised ? 0x3c003c00u : w;                 // 1.0
-        msn[q] = raised ? w : 0xbc00bc00u;                 // -1.0
+        uint32_t fq = f[q], m, t;
+        if (SEL == 0)
+            asm("v_and_b32 %1, 0x8000, %0\n\t"
+                "v_cmp_ne_u32 vcc, 0, %1\n\t"
+                "v_and_or_b32 %2, %0, %3, %5\n\t"
+                "s_nop 0\n\t"
+                "v_cndmask_b32 %1, %4, %0, vcc\n\t"           // -ms, or -1
+                "v_cndmask_b32 %0, %0, %2, vcc"                 // 1 in place of -ms
+                : "+v"(fq), "=&v"(m), "=&v"(t) : "v"(keep), "v"(neg_one), "v"(one) : "vcc");
+        else
+            asm("v_cmp_gt_i32 vcc, 0, %0\n\t"
+                "v_and_or_b32 %2, %0, %3, %5\n\t"
+                "s_nop 0\n\t"
+                "v_cndmask_b32 %1, %4, %0, vcc\n\t"
+                "v_cndmask_b32 %0, %0, %2, vcc"
+                : "+v"(fq), "=&v"(m), "=&v"(t) : "v"(keep), "v"(neg_one), "v"(one) : "vcc");
+        f[q] = fq; msn[q] = m;
     }
     pk_scale8<SEL>(acc, msn);
-    pk_mad8<SEL>(acc, v0, v1, vs);
 }
 // two f32 factors -> one register of two f16 (round to nearest even, as the conversion in front of vdupq_n_f16)
 __device__ __forceinline__ uint32_t pk_factors(float f0, float f1) {
@@ -988,6 +1006,7 @@ __global__ void __launch_bounds__(512, 2) k_fattn_pk_tile(fa_args a) {
 
         const int sq = (pw >> 1) * 32, sk = (pw & 1) * 32, l32 = lane & 31, g = lane >> 5;
         const int kr = tid >> 2, kc = (tid & 3) * 16;
+        const float scale2 = a.scale * LOG2E_F;
         u32x4 kreg0, kreg1, vreg0, vreg1;
         auto load_kv = [&](int64_t key0) __attribute__((always_inline)) {
             const int64_t key = key0 + kr < a.KV ? key0 + kr : a.KV - 1;      // rows past the end repeat the last key; their scores are masked
@@ -1018,11 +1037,12 @@ __global__ void __launch_bounds__(512, 2) k_fattn_pk_tile(fa_args a) {
                 }
                 const int64_t key = key0 + sk + l32;
                 const bool key_ok = key < a.KV;
+                // (scores are kept in units of log2 e: the factors are then one v_exp_f32 each)
                 if (!a.mask && key0 + T_KV <= a.KV) {
 #pragma unroll
                     for (int r = 0; r < 16; ++r) {
                         const int qi = sq + 8 * (r >> 2) + 4 * g + (r & 3);
-                        sc_s[qi * T_LDF + sk + l32] = __fmul_rn(c16[r], a.scale);
+                        sc_s[qi * T_LDF + sk + l32] = __fmul_rn(c16[r], scale2);
                     }
                 } else {
                     float mv[16];
@@ -1038,7 +1058,7 @@ __global__ void __launch_bounds__(512, 2) k_fattn_pk_tile(fa_args a) {
 #pragma unroll
                     for (int r = 0; r < 16; ++r) {
                         const int qi = sq + 8 * (r >> 2) + 4 * g + (r & 3);
-                        sc_s[qi * T_LDF + sk + l32] = key_ok ? __fadd_rn(__fmul_rn(c16[r], a.scale), mv[r]) : -INFINITY;
+                        sc_s[qi * T_LDF + sk + l32] = key_ok ? __builtin_fmaf(c16[r], scale2, mv[r] * LOG2E_F) : -INFINITY;
                     }
                 }
             }
@@ -1064,7 +1084,9 @@ __global__ void __launch_bounds__(512, 2) k_fattn_pk_tile(fa_args a) {
                 for (int i = 0; i < 16; ++i) {
                     const float s = sv[i];
                     const bool  raised = s > M;
-                    const float ex = exp_neg(-fabsf(s - M));   // M - s when raised, s - M otherwise: both <= 0 (or NaN / -inf: 0)
+                    // 2^(M - s) when raised, 2^(s - M) otherwise: the exponent is <= 0, -inf for the first key of a row (0), and
+                    // NaN for a masked key in front of every other (-inf - -inf), which the maximum with 0 turns into 0
+                    const float ex = fmaxf(__builtin_amdgcn_exp2f(-fabsf(s - M)), 0.0f);
                     if (__any(raised)) {
                         const float ms = raised ? ex : 1.0f, vs = raised ? 1.0f : ex;
                         M = raised ? s : M;
@@ -1132,22 +1154,15 @@ __global__ void __launch_bounds__(512, 2) k_fattn_pk_tile(fa_args a) {
 #pragma unroll
                 for (int j = 0; j < 8; ++j) gr.v[j] = *(const u32x2 *)(vbase + (2 * kp0 + j) * (FA_D * 2));
             };
-            // bits: two per pair of keys, lowest first: does the first / the second key of the pair raise a maximum in this wavefront
-            auto walk = [&](const pgroup & gr, uint32_t bits) __attribute__((always_inline)) {
-                if (bits == 0) {
+            // bits: two per pair of keys, lowest first: does the first / the second key of the pair raise a maximum in this wavefront.
+            // Only the rescale sits behind the (scalar) test; the multiply-adds are the same instructions on either path.
+            auto walk = [&](pgroup & gr, uint32_t bits) __attribute__((always_inline)) {
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) {
-                        pk_mad8<0>(acc, gr.v[2*j].x, gr.v[2*j].y, gr.f[j]);
-                        pk_mad8<1>(acc, gr.v[2*j + 1].x, gr.v[2*j + 1].y, gr.f[j]);
-                    }
-                } else {
-#pragma unroll
-                    for (int j = 0; j < 4; ++j) {
-                        if (bits & (1u << (2*j))) pk_key_with_rescale<0>(acc, gr.v[2*j].x, gr.v[2*j].y, gr.f[j]);
-                        else                      pk_mad8<0>(acc, gr.v[2*j].x, gr.v[2*j].y, gr.f[j]);
-                        if (bits & (2u << (2*j))) pk_key_with_rescale<1>(acc, gr.v[2*j + 1].x, gr.v[2*j + 1].y, gr.f[j]);
-                        else                      pk_mad8<1>(acc, gr.v[2*j + 1].x, gr.v[2*j + 1].y, gr.f[j]);
-                    }
+                for (int j = 0; j < 4; ++j) {
+                    if (bits & (1u << (2*j))) pk_rescale<0>(acc, gr.f[j]);
+                    pk_mad8<0>(acc, gr.v[2*j].x, gr.v[2*j].y, gr.f[j]);
+                    if (bits & (2u << (2*j))) pk_rescale<1>(acc, gr.f[j]);
+                    pk_mad8<1>(acc, gr.v[2*j + 1].x, gr.v[2*j + 1].y, gr.f[j]);
                 }
             };
             auto arrived = [&](const pgroup & gr) __attribute__((always_inline)) {

@@ -17,6 +17,7 @@
 #include "common.h"
 
 #include <algorithm>
+#include <atomic>
 #include <mutex>
 #include <stdlib.h>
 #include <type_traits>
@@ -802,12 +803,12 @@ template <int TI, int TJ, bool EMIT>
 static int launch_gemm_f16_dl(const mm_args & a, hipStream_t st) {
     constexpr int BN = 64 * TI, BM = 64 * TJ, NBUF = dl_buffers<TI, TJ>();
     constexpr size_t lds = dl_lds_bytes<TI, TJ>();
-    static bool configured[64];
+    static std::atomic<bool> configured[64];
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return MI355X_ERR_HIP;
-    if (!configured[dev]) {
+    if (!configured[dev].load(std::memory_order_acquire)) {
         if (hipFuncSetAttribute((const void *) k_gemm_f16_dl<TI, TJ, NBUF, EMIT>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds) != hipSuccess) return MI355X_ERR_HIP;
-        configured[dev] = true;
+        configured[dev].store(true, std::memory_order_release);
     }
     const int64_t tm = (a.M + BM - 1) / BM, tn = (a.N + BN - 1) / BN;
     if (tm * tn > 0x7fffffff) return MI355X_ERR_UNSUPPORTED;
@@ -832,12 +833,12 @@ template <int TI, int TJ, bool EMIT>
 static int launch_gemm_f16_rs(const mm_args & a, hipStream_t st) {
     constexpr int BN = 64 * TI, BM = 64 * TJ, S = rs_ring<TI, TJ>();
     constexpr size_t lds = (size_t) 2 * (BN + BM) * GB_LD * sizeof(half_t);
-    static bool configured[64];
+    static std::atomic<bool> configured[64];
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return MI355X_ERR_HIP;
-    if (!configured[dev]) {
+    if (!configured[dev].load(std::memory_order_acquire)) {
         if (hipFuncSetAttribute((const void *) k_gemm_f16_rs<TI, TJ, S, EMIT, RS_NP>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds) != hipSuccess) return MI355X_ERR_HIP;
-        configured[dev] = true;
+        configured[dev].store(true, std::memory_order_release);
     }
     const int64_t tm = (a.M + BM - 1) / BM, tn = (a.N + BN - 1) / BN;
     if (tm * tn > 0x7fffffff) return MI355X_ERR_UNSUPPORTED;
@@ -852,12 +853,12 @@ static int launch_gemm_f16_k(const mm_args & a, hipStream_t st) {
     static_assert(S % 2 == 0, "the LDS buffer index is the parity of the register slot");
     constexpr int BN = 64 * TI, BM = 64 * TJ;
     constexpr size_t lds = (size_t) 2 * (BN + BM) * GB_LD * sizeof(half_t);
-    static bool configured[64];                         // per device: kernels may use more than the default 64 KB of LDS
+    static std::atomic<bool> configured[64];                         // per device: kernels may use more than the default 64 KB of LDS
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return MI355X_ERR_HIP;
-    if (!configured[dev]) {
+    if (!configured[dev].load(std::memory_order_acquire)) {
         if (hipFuncSetAttribute((const void *) k_gemm_f16<TI, TJ, S, KTAIL, FULL, EMIT>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds) != hipSuccess) return MI355X_ERR_HIP;
-        configured[dev] = true;
+        configured[dev].store(true, std::memory_order_release);
     }
     const int64_t tm = (a.M + BM - 1) / BM, tn = (a.N + BN - 1) / BN;
     if (tm * tn > 0x7fffffff) return MI355X_ERR_UNSUPPORTED;
@@ -894,12 +895,12 @@ template <int TI, int TJ>
 static int launch_gemm_f16_group(const mm_args & a, const mm_group & grp, int count, hipStream_t st) {
     constexpr int BN = 64 * TI, BM = 64 * TJ;
     constexpr size_t lds = (size_t) 2 * (BN + BM) * GB_LD * sizeof(half_t);
-    static bool configured[64];
+    static std::atomic<bool> configured[64];
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return MI355X_ERR_HIP;
-    if (!configured[dev]) {
+    if (!configured[dev].load(std::memory_order_acquire)) {
         if (hipFuncSetAttribute((const void *) k_gemm_f16_group<TI, TJ, 4>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) lds) != hipSuccess) return MI355X_ERR_HIP;
-        configured[dev] = true;
+        configured[dev].store(true, std::memory_order_release);
     }
     const int64_t tm = (a.M + BM - 1) / BM, tn = (a.N + BN - 1) / BN;
     if (tm * tn > 0x7fffffff) return MI355X_ERR_UNSUPPORTED;
@@ -912,7 +913,7 @@ static int launch_gemm_f16_group(const mm_args & a, const mm_group & grp, int co
         constexpr size_t dl_lds = dl_lds_bytes<TI, TJ>();
         if (!dl_configured[dev]) {
             if (hipFuncSetAttribute((const void *) k_gemm_f16_dl_group<TI, TJ, dl_buffers<TI, TJ>()>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) dl_lds) != hipSuccess) return MI355X_ERR_HIP;
-            dl_configured[dev] = true;
+            dl_configured[dev].store(true, std::memory_order_release);
         }
         k_gemm_f16_dl_group<TI, TJ, dl_buffers<TI, TJ>()><<<grid, 256, dl_lds, st>>>(a, (int) tm, (int) tn, sw, grp);
         return launch_status();

@@ -121,6 +121,8 @@ static int norm_impl(const mi355x_tensor * src, const mi355x_tensor * dst, float
     if (!same_shape(src, dst) || src->nb[0] != 4 || dst->nb[0] != 4) return MI355X_ERR_INVALID;
     const int64_t nrows = src->ne[1] * src->ne[2] * src->ne[3];
     if (nrows == 0 || src->ne[0] == 0) return MI355X_OK;
+    // a destination without memory is an argument of the f16-image form alone (the caller wants the image and nothing else)
+    if (!src->data || (!dst->data && emit != 1)) return MI355X_ERR_INVALID;
     const int64_t grid = (nrows + ROWS_PER_BLOCK - 1) / ROWS_PER_BLOCK;
     if (grid > 0x7fffffff) return MI355X_ERR_UNSUPPORTED;
     hipStream_t st = (hipStream_t) stream;
