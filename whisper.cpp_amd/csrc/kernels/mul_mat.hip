@@ -909,9 +909,9 @@ static int launch_gemm_f16_group(const mm_args & a, const mm_group & grp, int co
     static const bool staged = getenv("MI355X_GEMM_STAGED") != nullptr;
     if constexpr (TI * TJ == 4) {
     if (!staged) {
-        static bool dl_configured[64];
+        static std::atomic<bool> dl_configured[64];
         constexpr size_t dl_lds = dl_lds_bytes<TI, TJ>();
-        if (!dl_configured[dev]) {
+        if (!dl_configured[dev].load(std::memory_order_acquire)) {
             if (hipFuncSetAttribute((const void *) k_gemm_f16_dl_group<TI, TJ, dl_buffers<TI, TJ>()>, hipFuncAttributeMaxDynamicSharedMemorySize, (int) dl_lds) != hipSuccess) return MI355X_ERR_HIP;
             dl_configured[dev].store(true, std::memory_order_release);
         }
