@@ -57,14 +57,21 @@ def model_file(arch: str, ftype: str) -> str:
     return str(path)
 
 
-# HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled by the same counters over a 256 MiB copy:
-# x2 KiB and x1 KiB), for the large-v3 encoder shapes; the summary with the commands is under profiles/
-# (mul_mat.gemm_q5_0 averages its two templates: 64 launches of 59.9 + 7.7 MB and 32 of 45.4 + 15.4 MB per window)
-MEASURED_TRAFFIC_MB = {"mul_mat.gemm_q5_0": (64 * (59.9 + 7.7) + 32 * (45.4 + 15.4)) / 96, "flash_attn.seq_tile": 17.4 + 3.8,
-                       "mul_mat.gemm_group": 68.6 + 22.5, "norm_affine_emit": 7.9 + 3.8}
+# HBM bytes per launch, counted: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE per dispatch, scaled by what the same counters read
+# for a 256 MiB copy.  The profile step (`python whisper.cpp_amd/profile.py`, run on the GPU box) writes them into
+# profiles/traffic.json together with the commit they were taken at; nothing is typed in here.
+def measured_traffic() -> dict:
+    try:
+        doc = json.loads((ROOT / "profiles" / "traffic.json").read_text())
+        return {k: v for k, v in doc.get("bytes_per_launch", {}).items()}
+    except (OSError, ValueError):
+        return {}
+
+
+MEASURED_TRAFFIC = measured_traffic()
 
 # kernels that live on the matrix cores (bound "mfma"); everything else streams memory (bound "hbm")
-MFMA_KERNELS = ("mul_mat.gemm_", "flash_attn.seq_tile")
+MFMA_KERNELS = ("mul_mat.gemm_", "flash_attn.seq_tile")      # (also flash_attn.seq_tile_pk)
 
 
 def kernel_roofline(name: str, k: dict) -> dict:
@@ -81,20 +88,139 @@ def kernel_roofline(name: str, k: dict) -> dict:
         out.update({"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
                     "frac": round(achieved / PEAK_HBM_GBS, 5),
                     "algorithmic_mb_per_launch": round(k["bytes"] / k["calls"] / 1e6, 4)})
-    t = MEASURED_TRAFFIC_MB.get(name)
-    out["traffic"] = round(t * 1e6) if t else None
+    t = MEASURED_TRAFFIC.get(name)
+    out["traffic"] = round(t) if t else None
     return out
 
 
+def probes():
+    """the harness-only yardstick library (csrc/harness/probes.hip): nothing but this benchmark loads it"""
+    import ctypes as C
+    lib = C.CDLL(str(ROOT / "whisper.cpp_amd" / "lib" / "libmi355x_probes.so"))
+    P = C.c_void_p
+    lib.mi355x_probe_read.restype, lib.mi355x_probe_read.argtypes = C.c_int, [P, C.c_size_t, P, C.c_int, P]
+    lib.mi355x_probe_read_stamped.restype, lib.mi355x_probe_read_stamped.argtypes = C.c_int64, [P, C.c_size_t, P, C.c_int, P, P]
+    lib.mi355x_probe_mfma.restype, lib.mi355x_probe_mfma.argtypes = C.c_int, [C.c_int, C.c_int, P, P]
+    lib.mi355x_probe_gemv_tiles_stamped.restype = C.c_int
+    lib.mi355x_probe_gemv_tiles_stamped.argtypes = [P, C.c_int64, C.c_int64, P, C.c_int64, P, P, C.POINTER(C.c_int64), C.POINTER(C.c_int64), P]
+    return lib
+
+
+def plateau_of(completions_ticks, bytes_per_unit: float) -> dict:
+    """rate of a stream between the 10th and the 90th percentile of its completions (ticks of the device's 100 MHz clock, one per
+    finished unit of `bytes_per_unit`): what it sustains between ramp and tail"""
+    t = sorted(completions_ticks)
+    n = len(t)
+    i10, i90 = n // 10, n * 9 // 10
+    dt_us = (t[i90] - t[i10]) / 100.0
+    return {"units": n, "span_us": round((t[-1] - t[0]) / 100.0, 2), "p10_to_p90_us": round(dt_us, 2),
+            "gb_per_s": round((i90 - i10) * bytes_per_unit / dt_us / 1e3, 1) if dt_us > 0 else None}
+
+
+def stream_plateaus() -> dict | None:
+    """What the logits kernel and a bare read stream sustain between ramp and tail.  A stamped instance of the product's own
+    kernel (same source, built into the probes library) writes the device clock after every tile of 16 rows, the read probe
+    after every 32 KB chunk.  The vocabulary matrix itself (51866 rows, 70 MB) is two tiles per wavefront: its launch is little
+    more than a ramp and a tail, and the completions of each round arrive bunched, so the percentile rate of that launch says
+    little (it can exceed the HBM peak: the bytes were already on their way while nothing had completed).  The same kernel
+    over eight times the rows (564 MB, 16 tiles per wavefront, more than the memory-side cache holds) has a plateau to measure:
+    that is the figure reported as plateau_frac.  Median of 5 launches each, 512 MB walked in between."""
+    try:
+        sys.path.insert(0, str(ROOT))
+        import ctypes as C
+        import torch
+        import __graft_entry__ as entry
+        pkg = entry.package()
+        lib, pr = pkg.kernels(), probes()
+        dev = torch.device("cuda:0")
+        K, N = 1280, 5
+        other = torch.zeros(512 << 20, dtype=torch.uint8, device=dev)
+        sink = torch.zeros(16, dtype=torch.int32, device=dev)
+        tile_bytes = 16 * (K // 32) * 34
+        out = {"what": "bytes finished between the 10th and the 90th percentile of unit completions / the time between them, and bytes of the "
+                       "launch / (last completion - first start); s_memrealtime stamps (100 MHz)"}
+        for label, M in (("vocabulary_matrix", 51866), ("eight_times_the_rows", 8 * 51866)):
+            g = torch.Generator(device="cpu").manual_seed(5)
+            blocks = torch.randint(0, 255, (M, K // 32, 34), dtype=torch.uint8, generator=g)
+            blocks[:, :, 0] = 0x00
+            blocks[:, :, 1] = 0x1c                                                   # every scale 2^-8 as f16
+            w = blocks.to(dev)
+            del blocks
+            tw = pkg.tensor(w, pkg.Q8_0, ne=[K, M], nb=[34, (K // 32) * 34])
+            tiles = torch.empty(lib.mi355x_q8_0_tiles_size(K, M), dtype=torch.uint8, device=dev)
+            pkg.check(lib.mi355x_q8_0_tiles_pack(C.byref(tw), tiles.data_ptr(), None), "tiles_pack")
+            torch.cuda.synchronize()
+            del w
+            x = torch.randn(N, K, device=dev)
+            d0, d1 = torch.empty(N, M, device=dev), torch.zeros(N, M, device=dev)
+            need = (N * K + N * (K // 32) * 8 + 255) // 256 * 256
+            ws = torch.empty(need, dtype=torch.uint8, device=dev)
+            tx, td0 = pkg.tensor(x, pkg.F32), pkg.tensor(d0, pkg.F32)
+            pkg.check(lib.mi355x_mul_mat_q8_0_tiles(tiles.data_ptr(), K, M, C.byref(tx), C.byref(td0), 0, ws.data_ptr(), need, None), "mul_mat_q8_0_tiles")
+            waves, per = C.c_int64(0), C.c_int64(0)
+            pkg.check(pr.mi355x_probe_gemv_tiles_stamped(tiles.data_ptr(), K, M, ws.data_ptr(), N, d1.data_ptr(), None, C.byref(waves), C.byref(per), None), "probe sizes")
+            stamps = torch.zeros(waves.value * (1 + per.value), dtype=torch.int64, device=dev)
+            runs = []
+            for _ in range(7):
+                stamps.zero_()
+                pkg.check(pr.mi355x_probe_read(other.data_ptr(), other.numel(), sink.data_ptr(), 2048, None))     # cold caches, as in the loop
+                pkg.check(pr.mi355x_probe_gemv_tiles_stamped(tiles.data_ptr(), K, M, ws.data_ptr(), N, d1.data_ptr(), stamps.data_ptr(), C.byref(waves), C.byref(per), None), "stamped gemv")
+                torch.cuda.synchronize()
+                st = stamps.cpu().numpy().reshape(waves.value, 1 + per.value)
+                done = st[:, 1:][st[:, 1:] != 0]
+                r = plateau_of(done.tolist(), tile_bytes)
+                whole_us = (done.max() - st[:, 0].min()) / 100.0
+                r.update({"first_completion_after_us": round((done.min() - st[:, 0].min()) / 100.0, 2), "whole_launch_us": round(whole_us, 2),
+                          "whole_launch_gb_per_s": round(len(done) * tile_bytes / whole_us / 1e3, 1)})
+                runs.append(r)
+            same = bool(torch.equal(d0, d1))
+            runs = sorted(runs[2:], key=lambda r: r["gb_per_s"])
+            gemv = runs[len(runs) // 2]
+            gemv.update({"kernel": "k_gemv_q8_0_tiles<20> with stamps", "rows": M, "tiles_per_wavefront": per.value, "bytes_per_unit": tile_bytes,
+                         "p10_to_p90_frac_of_hbm_peak": round(gemv["gb_per_s"] / PEAK_HBM_GBS, 4),
+                         "whole_launch_frac_of_hbm_peak": round(gemv["whole_launch_gb_per_s"] / PEAK_HBM_GBS, 4), "result_equals_the_products": same})
+            # the bare read stream over the same number of bytes
+            nbytes = M * (K // 32) * 34 // 32768 * 32768
+            del d0, d1
+            buf = tiles[:nbytes]
+            best = None
+            for wgs in (1024, 2048, 4096):
+                rstamps = torch.zeros(nbytes // 32768 + wgs, dtype=torch.int64, device=dev)
+                rr = []
+                for _ in range(5):
+                    rstamps.zero_()
+                    pkg.check(pr.mi355x_probe_read(other.data_ptr(), other.numel(), sink.data_ptr(), 2048, None))
+                    n_chunks = pr.mi355x_probe_read_stamped(buf.data_ptr(), nbytes, sink.data_ptr(), wgs, rstamps.data_ptr(), None)
+                    torch.cuda.synchronize()
+                    st = rstamps.cpu().numpy()
+                    r = plateau_of(st[:n_chunks].tolist(), 32768.0)
+                    whole_us = (st[:n_chunks].max() - st[n_chunks:n_chunks + wgs].min()) / 100.0
+                    r.update({"whole_launch_us": round(whole_us, 2), "whole_launch_gb_per_s": round(nbytes / whole_us / 1e3, 1)})
+                    rr.append(r)
+                rr = sorted(rr[1:], key=lambda r: r["gb_per_s"])
+                r = rr[len(rr) // 2]
+                r["workgroups"] = wgs
+                if best is None or r["whole_launch_gb_per_s"] > best["whole_launch_gb_per_s"]:
+                    best = r
+            best.update({"kernel": "read probe with stamps, 32 KB chunks", "p10_to_p90_frac_of_hbm_peak": round(best["gb_per_s"] / PEAK_HBM_GBS, 4),
+                         "whole_launch_frac_of_hbm_peak": round(best["whole_launch_gb_per_s"] / PEAK_HBM_GBS, 4)})
+            out[label] = {"gemv": gemv, "read": best}
+            del tiles, buf
+        return out
+    except Exception as e:                                 # a yardstick: its absence must not fail the bench
+        print(f"bench.py: stream_plateaus skipped: {e}", file=sys.stderr)
+        return None
+
+
 def read_yardstick(nbytes: int) -> dict:
-    """time of a kernel that only streams `nbytes` out of HBM (mi355x_read_probe), the way the per-kernel figures of the
+    """time of a kernel that only streams `nbytes` out of HBM (mi355x_probe_read), the way the per-kernel figures of the
     decode loop are taken: one pair of HIP events around every launch, on the stream of the launch"""
     sys.path.insert(0, str(ROOT))
     import ctypes as C
     import torch
     import __graft_entry__ as entry
     pkg = entry.package()
-    lib = pkg.kernels()
+    lib = probes()
     dev = torch.device("cuda:0")
     buf = torch.empty(nbytes // 16 * 16, dtype=torch.uint8, device=dev).random_(0, 255)
     other = torch.empty(256 << 20, dtype=torch.uint8, device=dev).zero_()          # walked between launches: the caches start cold, as in the loop
@@ -102,14 +228,14 @@ def read_yardstick(nbytes: int) -> dict:
     best = None
     for wgs in (1024, 2048, 4096, 8192, 16384):
         for _ in range(3):
-            pkg.check(lib.mi355x_read_probe(buf.data_ptr(), buf.numel(), out.data_ptr(), wgs, None))
+            pkg.check(lib.mi355x_probe_read(buf.data_ptr(), buf.numel(), out.data_ptr(), wgs, None))
         torch.cuda.synchronize()
         times = []
         for _ in range(20):
-            pkg.check(lib.mi355x_read_probe(other.data_ptr(), other.numel(), out.data_ptr(), 2048, None))
+            pkg.check(lib.mi355x_probe_read(other.data_ptr(), other.numel(), out.data_ptr(), 2048, None))
             e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             e0.record()
-            pkg.check(lib.mi355x_read_probe(buf.data_ptr(), buf.numel(), out.data_ptr(), wgs, None))
+            pkg.check(lib.mi355x_probe_read(buf.data_ptr(), buf.numel(), out.data_ptr(), wgs, None))
             e1.record()
             torch.cuda.synchronize()
             times.append(e0.elapsed_time(e1) * 1e3)
@@ -177,9 +303,10 @@ def gemm_library_yardstick() -> list | None:
                          "vendor_blas_frac_of_peak": round(gflop / blas * 1e3 / PEAK_MFMA_F16_TFLOPS, 4)})
         # the matrix instruction by itself: v_mfma_f32_32x32x16_f16 from registers, one and four wavefronts per SIMD
         sink = torch.zeros(1, device=dev)
+        pr = probes()
         for wgs in (256, 1024):
             iters = 20000
-            us = timed(lambda: pkg.check(lib.mi355x_mfma_probe(iters, wgs, sink.data_ptr(), None)), reps=5)
+            us = timed(lambda: pkg.check(pr.mi355x_probe_mfma(iters, wgs, sink.data_ptr(), None)), reps=5)
             tf = wgs * 4 * 4 * iters * 32768.0 / us / 1e6
             rows.append({"shape": f"matrix instruction from registers, {wgs // 256} wavefront(s) per SIMD", "us": round(us, 1),
                          "tflops": round(tf, 1), "frac_of_peak": round(tf / PEAK_MFMA_F16_TFLOPS, 4)})
@@ -221,16 +348,21 @@ def main() -> int:
         rooflines[n] = kernel_roofline(n, k)
     dom_name = max(kernels, key=lambda n: kernels[n]["ms"]) if kernels else None
     roofline = rooflines.get(dom_name)
-    if roofline and dom_name == "flash_attn.seq_tile":
+    if roofline and dom_name.startswith("flash_attn.seq_tile"):
         roofline["note"] = ("priced against the dense f16 matrix-core peak as the brief asks; the matrix cores only form the scores. "
-                            "The reference accumulates V key by key in f16 (f32 fma, f16 store), and reproducing that takes 1.5 vector "
-                            "instructions per (query, key, d). SQ_INSTS_VALU counts 93.5 M vector instructions per launch (70.8 M of them that sequence): "
-                            "178 us of issue per SIMD at the 2.05 GHz the part runs this kernel at; that is the bound that applies, and with its chain "
-                            "wavefronts issuing ahead of its producers the kernel runs within a few per cent of it")
+                            "The reference accumulates V key by key in f16, rounding the sum after every key; that is one packed f16 "
+                            "multiply-add per (query, key, d pair) on the vector units — 2.95 G element steps, 23.6 M instructions per launch "
+                            "at the least — and the vector issue rate is the bound that applies (profiles/)")
+    if roofline is None and rooflines:
+        roofline = next(iter(rooflines.values()))
 
     # ---- and with f32 matrix-core attention (faster, but outside the whole-model parity bound: reported, never the headline) ----
     f32att = run_harness(["bench", "--model", enc_model, "--what", "encoder", "--backend", "gpu", "--reps", str(a.steps),
                           "--warmup", str(a.warmup), "--threads", str(a.threads)], env={"GGML_MI355X_FA_ACCUM": "1"})
+
+    # ---- and with the f32-fma-then-f16-store form of the attention step (the reference's x86 sequence, option fa_chain = 0) ----
+    x86att = run_harness(["bench", "--model", enc_model, "--what", "encoder", "--backend", "gpu", "--reps", str(a.steps),
+                          "--warmup", str(a.warmup), "--threads", str(a.threads)], env={"GGML_MI355X_FA_CHAIN": "0"})
 
     # ---- decode: 224 five-token steps (the shape of a 5-beam search step) on large-v3-turbo Q8_0; step i writes positions
     # 2 i .. 2 i + 4 of the self-attention cache, so that it grows to its 448 positions over the run --------------------------
@@ -248,17 +380,30 @@ def main() -> int:
               "ms_per_step_with_blocking_logits_downloads": round(dec_nomirror["ms_per_step"], 4)}
     if gemv:
         decode["gemv_roofline"] = kernel_roofline(gemv_name, gemv)
-        decode["gemv_roofline"]["traffic"] = round(72.8e6 + 3.2e6)    # FETCH_SIZE + WRITE_SIZE per launch of k_gemv_q8_0_tiles (profiles/)
         # what a bare stream of the same bytes takes here, measured the same way: the ceiling that applies to a single launch
         y = read_yardstick(int(gemv["bytes"] / gemv["calls"]))
         decode["gemv_roofline"]["read_yardstick"] = y
         decode["gemv_roofline"]["frac_of_read_yardstick"] = round(y["us_per_launch"] / (1e3 * gemv["ms"] / gemv["calls"]), 4)
+        pl = stream_plateaus()
+        if pl:
+            decode["gemv_roofline"]["plateau"] = pl
+            decode["gemv_roofline"]["plateau_frac"] = pl["eight_times_the_rows"]["gemv"]["p10_to_p90_frac_of_hbm_peak"]
     for small in sorted(dk):
         if small != gemv_name and (small.startswith("mul_mat.gemv") or small.startswith("norm_mul_mat")):
             # the products over 1.7 ... 7 MB matrices: over in the launch-to-store latency of a small kernel
             decode.setdefault("gemv_small_rooflines", []).append(kernel_roofline(small, dk[small]))
     decode["kernel_breakdown"] = {n: {"launches_per_step": k["calls"] / dec["steps"], "ms_per_step": round(k["ms"] / dec["steps"], 4)}
                                   for n, k in sorted(dk.items(), key=lambda kv: -kv[1]["ms"])[:10]}
+
+    # ---- configs[4] as a user runs it: whisper_full() with 5 beams over 30 s of synthetic audio on the turbo model --------
+    beam_args = ["bench", "--model", dec_model, "--what", "full", "--beam", "5", "--seconds", "30", "--threads", str(a.threads)]
+    fb = run_harness(beam_args + ["--backend", "gpu", "--reps", "3", "--warmup", "1"])
+    decode["whisper_full_beam5"] = {
+        "what": "whisper_full(), beam_size 5, no temperature fallback, 30 s of synthetic audio, large-v3-turbo Q8_0; last of 3 timed passes",
+        "wall_ms": fb["wall_ms_median"], "encode_ms": fb["encode_ms"], "decode_ms_total": round(fb["batchd_ms"] + fb["decode_ms"] + fb["prompt_ms"], 3),
+        "sample_ms_on_the_host": fb["sample_ms"], "decode_steps": fb["decode_step_graphs"], "ms_per_decode_step": fb["ms_per_decode_step"],
+        "decode_ms_per_beam_token": round(fb["batchd_ms"] / max(1, fb["batchd_token_runs"]), 5), "largest_n_kv": fb["largest_n_kv"],
+        "tokens_in_result": fb["tokens_in_result"], "launches": fb["launches"]}
 
     # ---- the step in front of the encoder: log-mel of the 30 s window on the device beside whisper_pcm_to_mel on the host threads -------
     mel = run_harness(["mel", "--model", enc_model, "--seconds", "30", "--reps", "20", "--threads", str(a.threads)])
@@ -283,6 +428,12 @@ def main() -> int:
         dcpu = run_harness(dec_args + ["--backend", "cpu", "--threads", str(a.threads)], timeout=1500)
         dcpu1 = run_harness(["bench", "--model", dec_model, "--what", "decoder", "--reps", "1", "--warmup", "1", "--steps", "56", "--batch", "5", "--kv-stride", "8",
                              "--backend", "cpu", "--threads", "1"], timeout=1500)
+        fbc = run_harness(beam_args + ["--backend", "cpu", "--reps", "1", "--warmup", "0"], timeout=1500)
+        decode["whisper_full_beam5"]["cpu_baseline"] = {
+            "wall_ms": fbc["wall_ms_median"], "encode_ms": fbc["encode_ms"], "decode_ms_total": round(fbc["batchd_ms"] + fbc["decode_ms"] + fbc["prompt_ms"], 3),
+            "sample_ms_on_the_host": fbc["sample_ms"], "decode_ms_per_beam_token": round(fbc["batchd_ms"] / max(1, fbc["batchd_token_runs"]), 5),
+            "tokens_in_result": fbc["tokens_in_result"], "cores": a.threads, "kind": "reference",
+            "sample": "one whisper_full() call on the ggml CPU backend, same audio, same parameters (its search draws other candidates: the step counts differ)"}
         decode["cpu_baseline"] = {"value": round(dcpu["ms_per_step"], 3), "unit": "ms per 5-token step", "cores": a.threads, "kind": "reference",
                                   "sample": "the same 224 steps (median of 3 passes) through whisper_decode() on the ggml CPU backend",
                                   "one_thread": {"value": round(dcpu1["ms_per_step"], 3), "unit": "ms per 5-token step", "cores": 1,
@@ -304,11 +455,12 @@ def main() -> int:
         "config": {"workload": "whisper large-v3 encoder forward, Q5_0 weights, batch 1, one 30 s window (128x3000 log-mel): conv stem, 32 layers "
                                "d=1280 h=20 ffn=5120, n_ctx 1500, plus cross-attention K/V of 32 decoder layers (BASELINE configs[3])",
                    "host": "unmodified whisper.cpp whisper_encode() with the MI355X backend loaded through ggml_backend_load()",
-                   "numerics": "reference-faithful (Q8_0-rounded GEMM activations, f16 sequential attention accumulator)",
+                   "numerics": "reference-faithful (Q8_0-rounded GEMM activations, f16 key-by-key attention accumulator, the step in f16 arithmetic as in the reference's builds with f16 vector units)",
                    "flash_attn": True, "algorithmic_gflop": 2597.2},
         "encode_ms_median": round(enc["encode_ms_median"], 4),
         "encode_tflops": round(2597.2 / ms_per_step, 2),
         "encoder_ms_with_f32_mfma_attention_option": round(f32att["ms_per_step"], 4),
+        "encoder_ms_with_the_x86_form_of_the_attention_step": round(x86att["ms_per_step"], 4),
         "decode_steps_per_s": decode["steps_per_s"],
         "decode_beam_tokens_per_s": decode["beam_tokens_per_s"],
         "decode": decode,

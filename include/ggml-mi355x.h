@@ -86,8 +86,8 @@ typedef size_t (*ggml_backend_mi355x_get_stats_t)(ggml_backend_t backend, char *
  * launches, out[4] get_tensor calls served from the pinned host mirror of a graph output, out[5] get_tensor calls that
  * were a blocking device-to-host copy, out[6] nanoseconds of host time inside graph_compute (planning and queueing the
  * launches), out[7] nanoseconds the host waited inside synchronize, out[8] graphs that held a FLASH_ATTN_EXT node with at
- * most 8 queries (decode steps), out[9] the largest number of keys such a node saw (the extent of the self- or
- * cross-attention cache a step walked; a maximum, not a sum).  A host that sees one call per graph it computes, with the graph's
+ * most 8 queries (decode steps), out[9] the largest number of keys such a node with a mask saw (n_kv: the extent of the
+ * self-attention cache a step walked; a maximum, not a sum).  A host that sees one call per graph it computes, with the graph's
  * full node count, knows that the scheduler (ggml_backend_sched_split_graph, ggml/src/ggml-backend.cpp:863-1317) left
  * no node to another backend. */
 #define GGML_MI355X_N_COUNTERS 10

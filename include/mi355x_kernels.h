@@ -310,16 +310,6 @@ MI355X_API size_t  mi355x_log_mel_workspace_size(int n_mel);          /* 0: n_me
 MI355X_API int     mi355x_log_mel_spectrogram(const float * samples, int64_t n_samples, const float * filters, int n_mel, float * mel,
                                               void * workspace, size_t workspace_size, void * stream);
 
-/* Measurement aid, no counterpart in the reference: a kernel that only reads the first n / 16 * 16 bytes at `src` (16-byte
- * aligned) with `workgroups` workgroups of 256 threads, eight 16-byte loads in flight per lane — the time of a bare stream
- * out of HBM, against which the bandwidth-bound kernels are read.  `out`: 4 bytes of device memory (practically never written). */
-MI355X_API int mi355x_read_probe(const void * src, size_t n, void * out, int workgroups, void * stream);
-
-/* Measurement aid, no counterpart in the reference: `workgroups` workgroups of 256 threads, each wavefront issuing
- * 4 * iters v_mfma_f32_32x32x16_f16 (32768 flops each) from registers, no memory traffic — the rate the matrix cores reach
- * on this device under their own load, against which the GEMM kernels are read.  iters <= 2^20.
- * `out`: 4 bytes of device memory (never written). */
-MI355X_API int mi355x_mfma_probe(int iters, int workgroups, void * out, void * stream);
 
 /* Fill `n` bytes at `dst` with `value` through a kernel (safe inside HIP graph capture). */
 MI355X_API int mi355x_fill_bytes(void * dst, uint8_t value, size_t n, void * stream);

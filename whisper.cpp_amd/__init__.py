@@ -93,8 +93,6 @@ def kernels() -> C.CDLL:
             "mi355x_im2col_1d": (C.c_int, [T, T, C.c_int, C.c_int, C.c_int, C.c_int, P]),
             "mi355x_concat": (C.c_int, [T, T, T, C.c_int, P]),
             "mi355x_fill_bytes": (C.c_int, [P, C.c_uint8, C.c_size_t, P]),
-            "mi355x_read_probe": (C.c_int, [P, C.c_size_t, P, C.c_int, P]),
-            "mi355x_mfma_probe": (C.c_int, [C.c_int, C.c_int, P, P]),
             "mi355x_log_mel_n_len": (C.c_int64, [C.c_int64]),
             "mi355x_log_mel_workspace_size": (C.c_size_t, [C.c_int]),
             "mi355x_log_mel_spectrogram": (C.c_int, [P, C.c_int64, P, C.c_int, P, P, C.c_size_t, P]),

@@ -1,12 +1,14 @@
 """Build recipes for the MI355X backend.
 
-Three artefacts, all written under ``whisper.cpp_amd/lib`` (git-ignored, shipped to the GPU box as built):
+Four artefacts, all written under ``whisper.cpp_amd/lib`` (git-ignored, shipped to the GPU box as built):
 
 * ``libmi355x_kernels.so`` — the HIP kernels and their C ABI (``include/mi355x_kernels.h``).  Needs only
   hipcc; builds anywhere.
 * ``libggml-mi355x.so``    — the ggml backend plugin (``include/ggml-mi355x.h``).  Compiled against the ggml
   headers of a whisper.cpp tree (``--ref`` / ``$WHISPER_CPP_ROOT``, default ``/root/reference``); its
   references to the ggml-base API stay undefined and are resolved by the host process that loads it.
+* ``libmi355x_probes.so``  — measurement yardsticks that ``bench.py`` loads (``csrc/harness/probes.hip``); not part of
+  the product.
 * ``mi355x-harness``       — test / bench driver that links the unmodified whisper.cpp host libraries
   (built by ``oracle/Makefile``) and loads the plugin with ``ggml_backend_load``.
 """
@@ -66,6 +68,14 @@ def build_kernels() -> Path:
     return out
 
 
+def build_probes() -> Path:
+    """the measurement yardsticks of bench.py (read stream, matrix instruction, stamped instance of the logits kernel): a
+    library of their own, which no product path links"""
+    out = LIB / "libmi355x_probes.so"
+    _run([HIPCC, *DEVICE_FLAGS, *COMMON, "-I", INCLUDE, "-shared", "-o", out, CSRC / "harness" / "probes.hip"])
+    return out
+
+
 def have_reference(ref: Path = REF_DEFAULT) -> bool:
     return (ref / "ggml" / "src" / "ggml-backend-impl.h").is_file()
 
@@ -118,6 +128,7 @@ def build_harness(ref: Path = REF_DEFAULT) -> Path:
 def build_all(ref: Path = REF_DEFAULT) -> None:
     LIB.mkdir(parents=True, exist_ok=True)
     build_kernels()
+    build_probes()
     build_oracle()
     if have_reference(ref):
         build_reference(ref)
@@ -130,4 +141,4 @@ def build_all(ref: Path = REF_DEFAULT) -> None:
 if __name__ == "__main__":
     target = sys.argv[1] if len(sys.argv) > 1 else "all"
     {"all": build_all, "kernels": build_kernels, "backend": build_backend, "reference": build_reference,
-     "oracle": build_oracle, "harness": build_harness}[target]()
+     "oracle": build_oracle, "harness": build_harness, "probes": build_probes}[target]()

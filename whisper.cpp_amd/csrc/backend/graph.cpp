@@ -850,7 +850,7 @@ struct graph_runner {
                 float scale; memcpy(&scale, n->op_params, sizeof(float));
                 mi355x_tensor vq = to_view(s0), vk = to_view(k), vv = to_view(v), vm, vd = to_view(n);
                 if (m) vm = to_view(m);
-                if (s0->ne[1] <= 8) { few_query_attention = true; ctx->counters[9] = std::max<int64_t>(ctx->counters[9], k->ne[1]); }
+                if (s0->ne[1] <= 8) { few_query_attention = true; if (m) ctx->counters[9] = std::max<int64_t>(ctx->counters[9], k->ne[1]); }
                 const double flops = 4.0 * s0->ne[1] * k->ne[1] * 64.0 * s0->ne[2] * s0->ne[3];
                 const double bytes = (double) ggml_nelements(s0) * 4 + 2.0 * (double) k->ne[0] * k->ne[1] * k->ne[2] * k->ne[3] * 2 + nbytes_of(n);
                 // the accumulation option, bit 0: more than 8 queries, bit 1: a decode step's few queries

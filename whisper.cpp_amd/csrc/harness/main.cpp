@@ -899,6 +899,69 @@ static int cmd_bench(const args & a) {
                be.c_str(), threads, reps, n_steps, batch, kv_stride, past_of(n_steps - 1) + batch, ms, ms / n_steps, *std::min_element(per_rep.begin(), per_rep.end()) / n_steps,
                1000.0 * n_steps / ms, 1000.0 * n_steps * batch / ms, (double) cnt[3] / n_steps, (double) cnt[4] / n_steps, (double) cnt[5] / n_steps, cnt[6] / 1e3 / n_steps, cnt[7] / 1e3 / n_steps,
                profile ? "true" : "false", kernels.c_str(), json_escape(path).c_str());
+    } else if (what == "full") {
+        // whisper_full() as a user calls it: beam search with --beam beams (src/whisper.cpp:5781-5798: one KV cache for all beams,
+        // per-row masks), up to n_text_ctx / 2 - 4 tokens per window, no temperature fallback, over synthetic audio.  Per pass:
+        // wall time, whisper's own timings and its run counts (read from whisper_print_timings through the log callback: the
+        // counts are not in whisper_timings), and from the plugin the number of decode-step graphs and the largest number of
+        // keys a step's attention walked.
+        const int beam = a.num("beam", 5), seconds = a.num("seconds", 30);
+        std::vector<float> pcm((size_t) seconds * WHISPER_SAMPLE_RATE);
+        uint64_t st = 0x9E3779B97F4A7C15ull ^ 7ull;
+        for (size_t i = 0; i < pcm.size(); ++i) {
+            st = st * 6364136223846793005ull + 1442695040888963407ull;
+            const double t = (double) i / WHISPER_SAMPLE_RATE;
+            const double noise = ((double)(st >> 40) / (double)(1 << 24)) - 0.5;
+            pcm[i] = (float)(0.25 * sin(2 * M_PI * (220.0 + 30.0 * t) * t) + 0.15 * sin(2 * M_PI * 1310.0 * t) + 0.1 * noise);
+        }
+        whisper_full_params p = whisper_full_default_params(beam > 1 ? WHISPER_SAMPLING_BEAM_SEARCH : WHISPER_SAMPLING_GREEDY);
+        p.n_threads = threads;
+        p.print_progress = false; p.print_realtime = false; p.print_timestamps = false; p.print_special = false;
+        p.language = "en"; p.translate = false;
+        p.temperature_inc = 0.0f;
+        if (beam > 1) p.beam_search.beam_size = beam; else p.greedy.best_of = 1;
+        auto get_counters = use_gpu ? (ggml_backend_mi355x_get_counters_t) ggml_backend_reg_get_proc_address(reg, "ggml_backend_mi355x_get_counters") : nullptr;
+        static std::string timing_log;
+        auto collect = [](ggml_log_level, const char * text, void *) { timing_log += text; };
+        auto run_count = [](const char * label) {          // "...   batchd time =   123.45 ms /   678 runs ..."
+            const size_t at = timing_log.find(label);
+            if (at == std::string::npos) return std::pair<double, long>(0.0, 0L);
+            double ms = 0; long runs = 0;
+            const size_t eq = timing_log.find('=', at);
+            if (eq != std::string::npos) sscanf(timing_log.c_str() + eq + 1, " %lf ms / %ld", &ms, &runs);
+            return std::pair<double, long>(ms, runs);
+        };
+        std::vector<double> wall;
+        std::string last;
+        for (int r = 0; r < warmup + reps; ++r) {
+            int64_t cnt[GGML_MI355X_N_COUNTERS] = {};
+            if (get_counters) get_counters(nullptr, cnt, 1);
+            whisper_reset_timings(ctx);
+            const double t0 = now_ms();
+            if (whisper_full(ctx, p, pcm.data(), (int) pcm.size()) != 0) return 1;
+            const double ms = now_ms() - t0;
+            if (r < warmup) continue;
+            wall.push_back(ms);
+            if (get_counters) get_counters(nullptr, cnt, 0);
+            timing_log.clear();
+            whisper_log_set(collect, nullptr);
+            whisper_print_timings(ctx);
+            whisper_log_set(nullptr, nullptr);
+            const auto enc = run_count("encode time"), dec = run_count("decode time"), bat = run_count("batchd time"), prm = run_count("prompt time"), smp = run_count("sample time");
+            int tokens = 0;
+            for (int i = 0; i < whisper_full_n_segments(ctx); ++i) tokens += whisper_full_n_tokens(ctx, i);
+            // whisper counts a batched call's tokens as its runs (src/whisper.cpp: n_batchd += n_tokens); a step is one call
+            const long steps = get_counters ? (long) cnt[8] : 0;
+            char buf[1024];
+            snprintf(buf, sizeof(buf), "\"wall_ms\": %.2f, \"encode_ms\": %.2f, \"encode_runs\": %ld, \"batchd_ms\": %.2f, \"batchd_token_runs\": %ld, \"decode_ms\": %.2f, "
+                     "\"decode_runs\": %ld, \"prompt_ms\": %.2f, \"prompt_token_runs\": %ld, \"sample_ms\": %.2f, \"tokens_in_result\": %d, \"segments\": %d, "
+                     "\"decode_step_graphs\": %ld, \"largest_n_kv\": %lld, \"ms_per_decode_step\": %.4f, \"launches\": %lld",
+                     ms, enc.first, enc.second, bat.first, bat.second, dec.first, dec.second, prm.first, prm.second, smp.first, tokens, whisper_full_n_segments(ctx),
+                     steps, (long long) cnt[9], steps > 0 ? (bat.first + dec.first) / steps : 0.0, (long long) cnt[3]);
+            last = buf;
+        }
+        printf("{\"bench\": \"full\", \"backend\": \"%s\", \"threads\": %d, \"beam\": %d, \"seconds\": %d, \"reps\": %d, \"wall_ms_median\": %.2f, %s, \"model\": \"%s\"}\n",
+               be.c_str(), threads, beam, seconds, reps, median(wall), last.c_str(), json_escape(path).c_str());
     } else {   // whisper-bench protocol, verbatim counts (examples/bench/bench.cpp:86-138)
         whisper_token tokens[512]; memset(tokens, 0, sizeof(tokens));
         if (whisper_encode(ctx, 0, threads) != 0) return 1;

@@ -1,0 +1,115 @@
+// Measurement yardsticks for bench.py — a library of its own (libmi355x_probes.so), loaded by the benchmark and by nothing
+// else: no product path links or calls it.
+//
+//   mi355x_probe_read              a kernel that only streams bytes out of HBM
+//   mi355x_probe_mfma              v_mfma_f32_32x32x16_f16 from registers, no memory in the loop
+//   mi355x_probe_read_stamped      the read stream with a time stamp per workgroup and chunk
+//   mi355x_probe_gemv_tiles_stamped  an instance of the product's own logits kernel (k_gemv_q8_0_tiles, same source) that
+//                                  also leaves a time stamp per wavefront and tile
+// The stamped forms answer what a stream sustains between its ramp and its tail: the stamps are the device's 100 MHz
+// clock (s_memrealtime), one after each unit of work; the caller sorts the completions and divides the bytes finished
+// between the 10th and the 90th percentile by the time between them.
+#include "../kernels/gemv_q8_0_tiles.h"
+
+#include <stdint.h>
+
+#define PROBE_API extern "C" __attribute__((visibility("default")))
+
+// every lane has eight 16-byte loads in flight; the words are folded so that the loads stay
+__global__ void __launch_bounds__(256) k_probe_read(const u32x4 * __restrict__ p, int64_t n16, uint32_t * __restrict__ out) {
+    const int64_t stride = (int64_t) gridDim.x * 256;
+    int64_t i = (int64_t) blockIdx.x * 256 + threadIdx.x;
+    u32x4 acc = { 0, 0, 0, 0 };
+    for (; i + 7 * stride < n16; i += 8 * stride) {
+        u32x4 v[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[j] = p[i + j * stride];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) acc ^= v[j];
+    }
+    for (; i < n16; i += stride) acc ^= p[i];
+    const uint32_t f = acc.x ^ acc.y ^ acc.z ^ acc.w;
+    if (f == 0x9E3779B9u) out[0] = f;                      // (practically never: the loads are kept without a store per thread)
+}
+
+// n: bytes at src (16-byte aligned); out: 4 bytes of device memory
+PROBE_API int mi355x_probe_read(const void * src, size_t n, void * out, int workgroups, void * stream) {
+    if (!src || !out || (uintptr_t) src % 16 != 0 || (uintptr_t) out % 4 != 0 || workgroups < 1 || workgroups > 65535) return MI355X_ERR_INVALID;
+    if (n < 16) return MI355X_OK;
+    k_probe_read<<<(unsigned) workgroups, 256, 0, (hipStream_t) stream>>>((const u32x4 *) src, (int64_t)(n / 16), (uint32_t *) out);
+    return launch_status();
+}
+
+// The same stream in chunks of 32 KB per workgroup (eight 16-byte loads per lane), workgroup w taking chunks w, w + grid, ...:
+// after each chunk the workgroup's first lane writes the clock into stamps[chunk]; stamps[n_chunks + w] is the workgroup's start.
+__global__ void __launch_bounds__(256) k_probe_read_stamped(const u32x4 * __restrict__ p, int64_t n_chunks, uint32_t * __restrict__ out, uint64_t * __restrict__ stamps) {
+    if (threadIdx.x == 0) stamps[n_chunks + blockIdx.x] = __builtin_amdgcn_s_memrealtime();
+    u32x4 acc = { 0, 0, 0, 0 };
+    for (int64_t c = blockIdx.x; c < n_chunks; c += gridDim.x) {
+        const u32x4 * q = p + c * 2048 + threadIdx.x;
+        u32x4 v[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[j] = q[j * 256];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) acc ^= v[j];
+        __syncthreads();                                   // all of the chunk's loads have arrived
+        if (threadIdx.x == 0) stamps[c] = __builtin_amdgcn_s_memrealtime();
+    }
+    const uint32_t f = acc.x ^ acc.y ^ acc.z ^ acc.w;
+    if (f == 0x9E3779B9u) out[0] = f;
+}
+
+// stamps: (n / 32768 + workgroups) x 8 bytes of device memory; returns the number of 32 KB chunks, or a negative status
+PROBE_API int64_t mi355x_probe_read_stamped(const void * src, size_t n, void * out, int workgroups, void * stamps, void * stream) {
+    if (!src || !out || !stamps || (uintptr_t) src % 16 != 0 || (uintptr_t) stamps % 8 != 0 || workgroups < 1 || workgroups > 65535) return MI355X_ERR_INVALID;
+    const int64_t n_chunks = (int64_t)(n / 32768);
+    if (n_chunks < 1) return MI355X_ERR_INVALID;
+    k_probe_read_stamped<<<(unsigned) workgroups, 256, 0, (hipStream_t) stream>>>((const u32x4 *) src, n_chunks, (uint32_t *) out, (uint64_t *) stamps);
+    const int rc = launch_status();
+    return rc ? rc : n_chunks;
+}
+
+// four independent accumulators per wavefront: 2 * 32 * 32 * 16 flops per instruction, 4 * iters instructions per wavefront
+__global__ void __launch_bounds__(256) k_probe_mfma(int iters, float * __restrict__ out) {
+    const half8_t a = { (_Float16)(threadIdx.x & 7), 1, 2, 3, 4, 5, 6, 7 }, b = { 1, 1, 1, 1, 1, 1, 1, (_Float16)(blockIdx.x & 3) };
+    float16_t c0 = {}, c1 = {}, c2 = {}, c3 = {};
+    for (int i = 0; i < iters; ++i) {
+        c0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c0, 0, 0, 0);
+        c1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c1, 0, 0, 0);
+        c2 = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c2, 0, 0, 0);
+        c3 = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c3, 0, 0, 0);
+    }
+    const float f = c0[0] + c1[1] + c2[2] + c3[3];
+    if (f == -1.0f) out[0] = f;                            // (never: the sums are >= 0; keeps the instructions)
+}
+
+PROBE_API int mi355x_probe_mfma(int iters, int workgroups, void * out, void * stream) {
+    if (!out || (uintptr_t) out % 4 != 0 || iters < 1 || iters > (1 << 20) || workgroups < 1 || workgroups > 65535) return MI355X_ERR_INVALID;
+    k_probe_mfma<<<(unsigned) workgroups, 256, 0, (hipStream_t) stream>>>(iters, (float *) out);
+    return launch_status();
+}
+
+// The logits product with stamps: `tiles` as mi355x_q8_0_tiles_pack wrote them (K = 1280), `x_q8` the quantized activations as
+// mi355x_mul_mat_q8_0_tiles leaves them in its workspace (call it with MI355X_MM_PREPARE_ONLY first), dst f32 [M, N] dense.
+// stamps: wavefronts x (1 + tiles per wavefront) x 8 bytes, zeroed by the caller; *wavefronts and *tiles_per_wavefront describe
+// the launch, which is the one mi355x_mul_mat_q8_0_tiles makes.  A tile is 16 rows: 16 * K / 32 * 34 bytes of the stream.
+PROBE_API int mi355x_probe_gemv_tiles_stamped(const void * tiles, int64_t K, int64_t M, const void * x_q8, int64_t N, void * dst, void * stamps,
+                                              int64_t * wavefronts, int64_t * tiles_per_wavefront, void * stream) {
+    if (!tiles || !x_q8 || !dst || !wavefronts || !tiles_per_wavefront || K != 1280 || M < 1 || N < 1 || N > 8) return MI355X_ERR_INVALID;
+    mm_args a;
+    a.K = K; a.M = M; a.N = N;
+    a.w = (const char *) tiles; a.x = (const char *) x_q8; a.d = (char *) dst;
+    a.w_nb1 = a.w_nb2 = a.w_nb3 = 0; a.x_nb1 = a.x_nb2 = a.x_nb3 = 0;
+    a.d_nb1 = M * 4; a.d_nb2 = a.d_nb3 = 0;
+    a.ne12 = a.ne13 = a.r2 = a.r3 = 1;
+    a.e.flags = 0; a.e.scale = 1.0f; a.e.bias = nullptr; a.e.residual = nullptr; a.e.gelu = nullptr; a.e.image = nullptr;
+    const int64_t n_tiles = (M + 15) / 16, resident = 256 * 2 * 4;
+    const int64_t rounds = (n_tiles + resident - 1) / resident;
+    const int64_t waves = (n_tiles + rounds - 1) / rounds;
+    const unsigned grid = (unsigned)(waves / 4 > 0 ? waves / 4 : 1);
+    *wavefronts = (int64_t) grid * 4;
+    *tiles_per_wavefront = (n_tiles + *wavefronts - 1) / *wavefronts;
+    if (!stamps) return MI355X_OK;                         // (sizes only)
+    k_gemv_q8_0_tiles<20, true><<<grid, 256, 0, (hipStream_t) stream>>>(a, (uint64_t *) stamps);
+    return launch_status();
+}

@@ -25,65 +25,6 @@ extern "C" const char * mi355x_status_string(int status) {
 }
 
 // ------------------------------------------------------------------------------------------------------
-// Read yardstick: what a kernel that does nothing but stream `n` bytes out of HBM takes on this device — the figure the
-// bandwidth-bound kernels (the product over the vocabulary matrix above all) are to be judged against, next to the
-// data-sheet peak.  Every lane has eight 16-byte loads in flight; the words are folded so that the loads stay.
-// ------------------------------------------------------------------------------------------------------
-
-typedef uint32_t probe_u32x4 __attribute__((ext_vector_type(4)));
-
-__global__ void __launch_bounds__(256) k_read_probe(const probe_u32x4 * __restrict__ p, int64_t n16, uint32_t * __restrict__ out) {
-    const int64_t stride = (int64_t) gridDim.x * 256;
-    int64_t i = (int64_t) blockIdx.x * 256 + threadIdx.x;
-    probe_u32x4 acc = { 0, 0, 0, 0 };
-    for (; i + 7 * stride < n16; i += 8 * stride) {
-        probe_u32x4 v[8];
-#pragma unroll
-        for (int j = 0; j < 8; ++j) v[j] = p[i + j * stride];
-#pragma unroll
-        for (int j = 0; j < 8; ++j) acc ^= v[j];
-    }
-    for (; i < n16; i += stride) acc ^= p[i];
-    const uint32_t f = acc.x ^ acc.y ^ acc.z ^ acc.w;
-    if (f == 0x9E3779B9u) out[0] = f;                      // (practically never: the loads are kept without a store per thread)
-}
-
-extern "C" int mi355x_read_probe(const void * src, size_t n, void * out, int workgroups, void * stream) {
-    if (!src || !out || (uintptr_t) src % 16 != 0 || (uintptr_t) out % 4 != 0 || workgroups < 1 || workgroups > 65535) return MI355X_ERR_INVALID;
-    if (n < 16) return MI355X_OK;
-    k_read_probe<<<(unsigned) workgroups, 256, 0, (hipStream_t) stream>>>((const probe_u32x4 *) src, (int64_t)(n / 16), (uint32_t *) out);
-    return launch_status();
-}
-
-// ------------------------------------------------------------------------------------------------------
-// Matrix-pipe yardstick: v_mfma_f32_32x32x16_f16 from registers, four independent accumulators per wavefront, no memory
-// in the loop — the rate the matrix cores reach on this device at the clock they run at under that load, next to the
-// data-sheet peak.  2 * 32 * 32 * 16 flops per instruction, 4 * iters instructions per wavefront, 4 wavefronts per workgroup.
-// ------------------------------------------------------------------------------------------------------
-
-typedef _Float16 probe_half8 __attribute__((ext_vector_type(8)));
-typedef float    probe_f32x16 __attribute__((ext_vector_type(16)));
-
-__global__ void __launch_bounds__(256) k_mfma_probe(int iters, float * __restrict__ out) {
-    const probe_half8 a = { (_Float16)(threadIdx.x & 7), 1, 2, 3, 4, 5, 6, 7 }, b = { 1, 1, 1, 1, 1, 1, 1, (_Float16)(blockIdx.x & 3) };
-    probe_f32x16 c0 = {}, c1 = {}, c2 = {}, c3 = {};
-    for (int i = 0; i < iters; ++i) {
-        c0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c0, 0, 0, 0);
-        c1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c1, 0, 0, 0);
-        c2 = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c2, 0, 0, 0);
-        c3 = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c3, 0, 0, 0);
-    }
-    const float f = c0[0] + c1[1] + c2[2] + c3[3];
-    if (f == -1.0f) out[0] = f;                            // (never: the sums are >= 0; keeps the instructions)
-}
-
-extern "C" int mi355x_mfma_probe(int iters, int workgroups, void * out, void * stream) {
-    if (!out || (uintptr_t) out % 4 != 0 || iters < 1 || iters > (1 << 20) || workgroups < 1 || workgroups > 65535) return MI355X_ERR_INVALID;
-    k_mfma_probe<<<(unsigned) workgroups, 256, 0, (hipStream_t) stream>>>(iters, (float *) out);
-    return launch_status();
-}
-
-// ------------------------------------------------------------------------------------------------------
 // GELU table
 // ------------------------------------------------------------------------------------------------------
 

@@ -29,14 +29,8 @@ struct __attribute__((packed, aligned(2))) u128a2 { uint32_t x, y, z, w; };
 // shared: epilogue
 // ------------------------------------------------------------------------------------------------------
 
-struct epi_args {
-    int          flags;
-    float        scale;
-    const float *bias;
-    const char * residual;   // same strides as dst, f32
-    const uint16_t * gelu;   // GELU table (device), set when MI355X_EPI_GELU is
-    half_t * image;          // MI355X_EPI_EMIT_F16: where the Q8_0-rounded f16 image of dst goes ([N][M] dense)
-};
+#include "mul_mat_args.h"
+#include "gemv_q8_0_tiles.h"
 
 __device__ __forceinline__ float apply_epilogue(float v, const epi_args & e, int64_t m, int64_t n, int64_t res_off) {
     if (e.flags & MI355X_EPI_BIAS)     v += e.bias[m];
@@ -165,15 +159,6 @@ __device__ __forceinline__ void patch_epilogue(float16_t v, const epi_args & e, 
     }
 }
 
-struct mm_args {
-    const char * w; const char * x; char * d;
-    int64_t M, N, K;
-    int64_t w_nb1, w_nb2, w_nb3;
-    int64_t x_nb1, x_nb2, x_nb3;
-    int64_t d_nb1, d_nb2, d_nb3;
-    int64_t ne12, ne13, r2, r3;      // batch dims of src1/dst and broadcast ratios of src0
-    epi_args e;
-};
 
 // ------------------------------------------------------------------------------------------------------
 // block -> 32 f16 weights
@@ -310,7 +295,6 @@ __global__ void k_x_to_f16(const char * __restrict__ x, half_t * __restrict__ ou
 #define GB_K  64
 #define GB_LD (GB_K + 8)
 
-typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 // What follows the K loop of a tile: GELU reads its table from LDS when the operand buffers, free now (the loop's last barrier
 // is behind every wavefront), are large enough to hold the part that matters (TABLE_FITS); then the 32x32 patches.
@@ -1345,8 +1329,6 @@ __global__ void __launch_bounds__(256) k_gemv_qr(mm_args a) { gemv_qr_rows<T0, N
 // from each of 16 rows, at 2-byte alignment, plus a 2-byte load per lane for the scale.  So the matrix is repacked once
 // into the order the instruction wants — per 16 rows and pair of blocks, 1024 bytes of quants in lane order followed by
 // the 32 scales (68 bytes a row, as before) — and every load of the stream is one aligned, contiguous run of a kilobyte.
-typedef int v4i_t __attribute__((ext_vector_type(4)));
-#define Q8T_STEP 1088      // bytes of 16 rows x one pair of blocks
 
 __global__ void k_q8_0_tiles_pack(const char * __restrict__ w, int64_t w_nb1, int64_t M, int ksteps, int64_t n_tiles, char * __restrict__ tiles) {
     const int64_t i = (int64_t) blockIdx.x * blockDim.x + threadIdx.x;     // (tile, step, lane)
@@ -1368,94 +1350,13 @@ __global__ void k_q8_0_tiles_pack(const char * __restrict__ w, int64_t w_nb1, in
     if ((g & 1) == 0) *(uint16_t *)(o + 1024 + ((g >> 1) * 16 + r) * 2) = d;
 }
 
-// a.w: the tiles; a.x: the activations quantized ahead (layout of k_quantize_x_q8); K = 64 KSTEPS
-template <int KSTEPS>
-__global__ void __launch_bounds__(256, 2) k_gemv_q8_0_tiles(mm_args a) {
-    __shared__ __attribute__((aligned(16))) float xs_lds[KSTEPS * 2 * 8];       // activation scales, [block][column 0 .. 7]
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int r = lane & 15, g = lane >> 4;
-    const int nbk = KSTEPS * 2;
-    const int64_t n_tiles = (a.M + 15) / 16;
-    const int64_t stride = (int64_t) gridDim.x * 4;
-    int64_t tile = (int64_t) blockIdx.x * 4 + wave;
-    constexpr int H = KSTEPS / 2;
-    u32x4 wq[2][H]; uint32_t wd[2][H];
-    const int q_ofs = lane * 16, d_ofs = 1024 + ((g >> 1) * 16 + r) * 2;
-    auto request = [&](int half, int64_t t) __attribute__((always_inline)) {
-        const char * p = a.w + (t * KSTEPS + half * H) * Q8T_STEP;
-#pragma unroll
-        for (int s = 0; s < H; ++s) {
-            wq[half][s] = *(const u32x4 *)(p + s * Q8T_STEP + q_ofs);
-            wd[half][s] = *(const uint16_t *)(p + s * Q8T_STEP + d_ofs);
-        }
-    };
-    const bool live = tile < n_tiles;                   // (a matrix of fewer than 64 rows)
-    request(0, live ? tile : n_tiles - 1);
-    __builtin_amdgcn_sched_barrier(0);
-    request(1, live ? tile : n_tiles - 1);
-    __builtin_amdgcn_sched_barrier(0);
-
-    // activations: quants as the A operand (lane = A row r, 16 k of group g), scales through LDS
-    const char *  xq = a.x;
-    const float * xd = (const float *)(a.x + (size_t) a.N * a.K);
-    const int col = r & 7;
-    const bool mine = ((r < 8) == (g < 2)) && col < a.N;
-    v4i_t xa[KSTEPS];
-#pragma unroll
-    for (int s = 0; s < KSTEPS; ++s) {
-        xa[s] = (v4i_t){ 0, 0, 0, 0 };
-        if (mine) xa[s] = *(const v4i_t *)(xq + (int64_t) col * a.K + 64 * s + 16 * g);
-    }
-    for (int i = threadIdx.x; i < nbk * 8; i += 256) xs_lds[i] = (i & 7) < a.N ? xd[(i & 7) * nbk + (i >> 3)] : 0.0f;
-    __syncthreads();
-    if (!live) return;
-    const float * xsl = xs_lds + (g >> 1) * 8 + (g & 1) * 4;      // + 16 per pair of blocks
-    const bool out_f16 = a.e.flags & MI355X_EPI_OUT_F16;
-
-    auto do_tile = [&](auto again) __attribute__((always_inline)) {
-        float acc[4] = { 0.0f, 0.0f, 0.0f, 0.0f };
-#pragma unroll
-        for (int half = 0; half < 2; ++half) {
-#pragma unroll
-            for (int s = 0; s < H; ++s) {
-                const u32x4 w = wq[half][s];
-                const v4i_t d = __builtin_amdgcn_mfma_i32_16x16x64_i8(xa[half * H + s], (v4i_t){ (int) w.x, (int) w.y, (int) w.z, (int) w.w }, (v4i_t){ 0, 0, 0, 0 }, 0, 0, 0);
-                const float dw = h2f((uint16_t) wd[half][s]);
-                const float4 x4 = *(const float4 *)(xsl + (half * H + s) * 16);
-                acc[0] += (float) d[0] * (dw * x4.x); acc[1] += (float) d[1] * (dw * x4.y);
-                acc[2] += (float) d[2] * (dw * x4.z); acc[3] += (float) d[3] * (dw * x4.w);
-            }
-            if constexpr (decltype(again)::value) {
-                request(half, tile + stride);
-                __builtin_amdgcn_sched_barrier(0);
-            }
-        }
-#pragma unroll
-        for (int i = 0; i < 4; ++i) acc[i] += __shfl_xor(acc[i], 32, WAVE);     // even blocks + odd blocks
-        const int64_t row = tile * 16 + r;
-        if (g < 2 && row < a.M) {
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const int n = 4 * g + i;
-                if (n < a.N) {
-                    if (out_f16) *(half_t *)(a.d + n * a.d_nb1 + row * 2) = (half_t) acc[i];
-                    else         *(float  *)(a.d + n * a.d_nb1 + row * 4) = acc[i];
-                }
-            }
-        }
-    };
-    // every tile but the wavefront's last requests the next one's halves as its own are used up
-    for (; tile + stride < n_tiles; tile += stride) do_tile(std::true_type{});
-    do_tile(std::false_type{});
-}
-
 template <int KSTEPS>
 static int launch_gemv_q8_0_tiles_k(const mm_args & a, hipStream_t st) {
     const int64_t n_tiles = (a.M + 15) / 16;
     const int64_t resident = 256 * 2 * 4;                 // wavefronts: two workgroups of four per CU
     const int64_t rounds = (n_tiles + resident - 1) / resident;
     const int64_t waves = (n_tiles + rounds - 1) / rounds;
-    k_gemv_q8_0_tiles<KSTEPS><<<(unsigned)(waves / 4 > 0 ? waves / 4 : 1), 256, 0, st>>>(a);
+    k_gemv_q8_0_tiles<KSTEPS, false><<<(unsigned)(waves / 4 > 0 ? waves / 4 : 1), 256, 0, st>>>(a, nullptr);
     return launch_status();
 }
 static bool q8_0_tiles_k_ok(int64_t K) { return K == 384 || K == 512 || K == 768 || K == 1024 || K == 1280; }
