@@ -92,6 +92,20 @@ def test_plugin_exports_the_ggml_entry_points_and_does_not_link_the_checker(pkg)
     assert not any("ggml-cpu" in l or "oracle" in l or "whisper" in l for l in libs), libs
 
 
+def test_yardstick_kernels_live_in_a_library_of_their_own(pkg):
+    # the benchmark's probes are not operators: neither product library exports or needs them
+    probes = pkg.KERNELS_LIB.parent / "libmi355x_probes.so"
+    if not pkg.KERNELS_LIB.exists() or not probes.exists():
+        pytest.skip("libraries not built")
+    assert {"mi355x_probe_read", "mi355x_probe_read_stamped", "mi355x_probe_mfma", "mi355x_probe_gemv_tiles_stamped"} <= exported(probes)
+    assert not any("probe" in name for name in exported(pkg.KERNELS_LIB)), [n for n in exported(pkg.KERNELS_LIB) if "probe" in n]
+    assert "probe" not in (ROOT / "include" / "mi355x_kernels.h").read_text()
+    for lib in (pkg.KERNELS_LIB, pkg.PLUGIN_LIB):
+        if lib.exists():
+            needed = subprocess.run(["readelf", "-d", str(lib)], stdout=subprocess.PIPE, text=True, check=True).stdout
+            assert "probes" not in needed
+
+
 def test_missing_extension_fails_loudly(pkg, monkeypatch, tmp_path):
     monkeypatch.setattr(pkg, "_lib", None)
     monkeypatch.setattr(pkg, "KERNELS_LIB", tmp_path / "libmi355x_kernels.so")

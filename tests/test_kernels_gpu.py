@@ -1015,16 +1015,31 @@ def test_log_mel_properties_and_arguments(pkg, oracle, gpu):
 
 
 def test_measurement_probes_run_and_reject_bad_arguments(pkg, gpu):
-    # the two yardstick kernels of the benchmark: a bare read stream and the matrix instruction from registers
-    lib = pkg.kernels()
+    # the yardstick kernels of the benchmark live in a library of their own (csrc/harness/probes.hip), not in the product's:
+    # a bare read stream, the matrix instruction from registers, and the stamped read
+    import ctypes as C
+    from pathlib import Path
+    assert not hasattr(pkg.kernels(), "mi355x_read_probe") and not hasattr(pkg.kernels(), "mi355x_probe_read")
+    lib = C.CDLL(str(Path(pkg.__file__).resolve().parent / "lib" / "libmi355x_probes.so"))
+    P = C.c_void_p
+    lib.mi355x_probe_read.restype, lib.mi355x_probe_read.argtypes = C.c_int, [P, C.c_size_t, P, C.c_int, P]
+    lib.mi355x_probe_read_stamped.restype, lib.mi355x_probe_read_stamped.argtypes = C.c_int64, [P, C.c_size_t, P, C.c_int, P, P]
+    lib.mi355x_probe_mfma.restype, lib.mi355x_probe_mfma.argtypes = C.c_int, [C.c_int, C.c_int, P, P]
     out = torch.zeros(4, dtype=torch.int32, device=gpu.dev)
     buf = torch.zeros(1 << 20, dtype=torch.uint8, device=gpu.dev)
-    pkg.check(lib.mi355x_read_probe(buf.data_ptr(), buf.numel(), out.data_ptr(), 64, gpu.stream))
-    pkg.check(lib.mi355x_mfma_probe(100, 256, out.data_ptr(), gpu.stream))
+    pkg.check(lib.mi355x_probe_read(buf.data_ptr(), buf.numel(), out.data_ptr(), 64, gpu.stream))
+    pkg.check(lib.mi355x_probe_mfma(100, 256, out.data_ptr(), gpu.stream))
     torch.cuda.synchronize()
     assert int(out.abs().sum()) == 0                       # neither writes its sink
-    assert lib.mi355x_mfma_probe(0, 256, out.data_ptr(), gpu.stream) == -2
-    assert lib.mi355x_mfma_probe(100, 0, out.data_ptr(), gpu.stream) == -2
-    assert lib.mi355x_mfma_probe(100, 256, None, gpu.stream) == -2
-    assert lib.mi355x_read_probe(None, 16, out.data_ptr(), 64, gpu.stream) == -2
-
+    assert lib.mi355x_probe_mfma(0, 256, out.data_ptr(), gpu.stream) == -2
+    assert lib.mi355x_probe_mfma(100, 0, out.data_ptr(), gpu.stream) == -2
+    assert lib.mi355x_probe_mfma(100, 256, None, gpu.stream) == -2
+    assert lib.mi355x_probe_read(None, 16, out.data_ptr(), 64, gpu.stream) == -2
+    # the stamped read: one (start, end) pair of device-clock ticks per 32 KB chunk, ends after starts
+    stamps = torch.zeros(2 * (buf.numel() // 32768) + 64, dtype=torch.int64, device=gpu.dev)
+    n = lib.mi355x_probe_read_stamped(buf.data_ptr(), buf.numel(), out.data_ptr(), 16, stamps.data_ptr(), gpu.stream)
+    torch.cuda.synchronize()
+    assert n == buf.numel() // 32768, n
+    st = stamps.cpu()
+    assert int(st[:n].min()) >= int(st[n:n + 16].min()) > 0        # every chunk finished after the first workgroup started
+    assert lib.mi355x_probe_read_stamped(buf.data_ptr(), buf.numel(), out.data_ptr(), 16, None, gpu.stream) == -2
