@@ -370,6 +370,8 @@ def main() -> int:
     dec = run_harness(dec_args + ["--backend", "gpu", "--profile", "--threads", str(a.threads)])
     # the same with every logits download a blocking copy (the pinned host mirror of the logits switched off)
     dec_nomirror = run_harness(dec_args + ["--backend", "gpu", "--threads", str(a.threads)], env={"GGML_MI355X_NO_MIRROR": "1"})
+    # ... and with the x86 form of the attention step in the decode kernels as well (option fa_chain = 0)
+    dec_x86 = run_harness(dec_args + ["--backend", "gpu", "--threads", str(a.threads)], env={"GGML_MI355X_FA_CHAIN": "0"})
     dk = {k["kernel"]: k for k in dec["kernels"]}
     # the logits product, 70.5 MB of Q8_0 blocks: the one GEMV that bandwidth bounds
     gemv_name = "mul_mat.gemv_q8_0.vocab"
@@ -377,7 +379,8 @@ def main() -> int:
     decode = {"model": "large-v3-turbo Q8_0", "steps": dec["steps"], "beams": dec["batch"], "max_kv_positions": dec["max_kv_positions"],
               "ms_per_step": round(dec["ms_per_step"], 4), "steps_per_s": round(dec["steps_per_s"], 1), "beam_tokens_per_s": round(dec["batch_tokens_per_s"], 1),
               "launches_per_step": dec["launches_per_step"], "logits_reads_from_pinned_mirror_per_step": dec["downloads_from_mirror_per_step"],
-              "ms_per_step_with_blocking_logits_downloads": round(dec_nomirror["ms_per_step"], 4)}
+              "ms_per_step_with_blocking_logits_downloads": round(dec_nomirror["ms_per_step"], 4),
+              "ms_per_step_with_the_x86_form_of_the_attention_step": round(dec_x86["ms_per_step"], 4)}
     if gemv:
         decode["gemv_roofline"] = kernel_roofline(gemv_name, gemv)
         # what a bare stream of the same bytes takes here, measured the same way: the ceiling that applies to a single launch

@@ -62,12 +62,12 @@ GGML_BACKEND_API int                ggml_backend_score(void);
  * five times faster, within the per-op bound, but the reference's f16 rounding is then missing and whole-model logits sit
  * several 1e-3 away.  Bit 1: f32 accumulators for a decode step's few queries; the decoder's layers alone move the
  * logits to 6e-3 … 8e-3 NMSE).
- * "fa_chain" (0/1, default 1: the arithmetic of one step of that key-by-key sequence where a launch has more than 8
- * queries.  1: the factor rounded to f16 and one fused f16 multiply-add per element, the reference's ggml_vec_mad_f16 on
- * hardware with f16 vector arithmetic (vec.h:180-203 with GGML_F16_VEC_FMA = vfmaq_f16, simd-mappings.h:68-105) — a third
- * of the vector instructions.  0: f32 fma followed by an f16 store, the same function in the reference's x86 build, which
- * the few-query kernel of a decode step always uses.  Whole-model logits stay within the same 1e-3 of the x86 CPU
- * backend with either.)
+ * "fa_chain" (0..2, default 2: the arithmetic of one step of that key-by-key sequence.  2: the factor rounded to f16 and
+ * one fused f16 multiply-add per element, the reference's ggml_vec_mad_f16 on hardware with f16 vector arithmetic
+ * (vec.h:180-203 with GGML_F16_VEC_FMA = vfmaq_f16, simd-mappings.h:68-105) — a third of the vector instructions where a
+ * launch has more than 8 queries, one dependent instruction per key instead of two in a decode step.  1: that form only
+ * where a launch has more than 8 queries.  0: f32 fma followed by an f16 store everywhere, the same function in the
+ * reference's x86 build.  Whole-model logits stay within the same 1e-3 of the x86 CPU backend with all three.)
  * The environment variables GGML_MI355X_FUSE, GGML_MI355X_PROFILE, GGML_MI355X_EXACT, GGML_MI355X_FA_ACCUM and
  * GGML_MI355X_FA_CHAIN give the initial values.
  * backend == NULL addresses every live MI355X backend of the process (a host such as whisper.cpp keeps its

@@ -207,8 +207,9 @@ MI355X_API int    mi355x_mul_mat_q8_0_tiles(const void * tiles, int64_t K, int64
  * MI355X_FA_F16_PK keeps the f16 accumulator and the key order and does the step in f16 arithmetic — the factor rounded
  * to f16, one fused f16 multiply-add per element, a rescale as one f16 multiply — which is the arithmetic of the
  * reference's builds with f16 vector units (GGML_F16_VEC_FMA = vfmaq_f16, ggml/src/ggml-cpu/simd-mappings.h:68-105, under
- * ggml_vec_mad_f16 / ggml_vec_scale_f16, vec.h:180-203, 295-311), a third of the vector instructions of the x86 form;
- * with at most 8 queries it is MI355X_FA_F16_SEQ. */
+ * ggml_vec_mad_f16 / ggml_vec_scale_f16, vec.h:180-203, 295-311), a third of the vector instructions of the x86 form
+ * and, for the at most 8 queries of a decode step, one dependent instruction per key instead of two (that kernel
+ * addresses the rows of a head's K and V with 32-bit offsets; a head slice of 2 GiB or more takes the x86 form). */
 enum mi355x_fa_mode { MI355X_FA_F16_SEQ = 0, MI355X_FA_F32 = 1, MI355X_FA_F16_PK = 2,
     /* or-ed into the mode: also write into `workspace` (16-byte aligned, N * H * ne3 * 64 halves) the image of dst that
      * a following MUL_MAT with quantized weights wants — rows [N][H * 64] rounded to Q8_0 as quantize_row_q8_0 does and
@@ -216,7 +217,7 @@ enum mi355x_fa_mode { MI355X_FA_F16_SEQ = 0, MI355X_FA_F32 = 1, MI355X_FA_F16_PK
      * With MI355X_FA_F16_SEQ, dst->data may then be NULL: only the image is written (a caller whose only reader of dst is
      * that product); MI355X_ERR_INVALID for a NULL dst->data in any other case. */
     MI355X_FA_EMIT_F16 = 0x100,
-    /* or-ed into the mode, at most 8 queries (the f16-sequential kernel of a decode step): also write into `workspace`
+    /* or-ed into the mode, at most 8 queries (the f16-sequential kernels of a decode step, either form): also write into `workspace`
      * (16-byte aligned) the rows [N * ne3][H * 64] of dst quantized to Q8_0, in the layout the few-column mi355x_mul_mat
      * reads its activations from (see mi355x_norm_emit_q8_0); MI355X_ERR_UNSUPPORTED for other kernels. */
     MI355X_FA_EMIT_Q8_0 = 0x200 };

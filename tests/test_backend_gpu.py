@@ -253,6 +253,18 @@ def test_whole_model_parity_on_other_seeds(harness, tmp_path, arch, ftype):
         path.unlink()
 
 
+def test_the_x86_form_of_the_attention_step_stays_an_option(harness, models):
+    # fa_chain = 0: f32 fma then f16 store in every attention launch (the sequence of the reference's x86 build, which the
+    # kernel tests hold to 1e-6 of the pinned oracle); fa_chain = 1: that form in the decode step's launches only
+    rc, rows = run_harness(harness, ["model", "--model", models[("base", "q5_0")], "--steps", "32"], env={"GGML_MI355X_FA_CHAIN": "0"}, timeout=900)
+    check_model_summary(rows[-1], strict_ids=True)
+    assert rc == 0
+    rc, rows = run_harness(harness, ["model", "--model", models[("large-v3-turbo", "q8_0")], "--batch", "5", "--kv-to", "448"], env={"GGML_MI355X_FA_CHAIN": "1"}, timeout=1500)
+    assert rows[-1]["kv_positions"] == 448
+    check_model_summary(rows[-1], strict_ids=False)
+    assert rc == 0
+
+
 @pytest.mark.parametrize("key,env", [(("large-v3-turbo", "q8_0"), {}), (("large-v3-turbo", "q8_0"), {"GGML_MI355X_FUSE": "0"}), (("base", "q5_0"), {})])
 def test_five_row_decode_steps_until_the_cache_is_full(harness, models, key, env):
     # the shape of a 5-beam search step (large-v3-turbo, 5 beams, 224 tokens): after the 4-token prompt every step feeds 5 tokens — the 5

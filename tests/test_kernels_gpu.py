@@ -570,7 +570,10 @@ def test_flash_attn_reference_faithful(pkg, oracle, gpu, case):
 
 @pytest.mark.parametrize("case", [
     dict(H=2, N=70, KV=100), dict(H=3, N=200, KV=1536, flat=True, pad_from=1500), dict(H=2, N=100, KV=100, mask="causal"),
-    dict(H=2, N=9, KV=63), dict(H=2, N=130, KV=448, mask="causal"), dict(H=2, N=64, KV=1500, flat=True)])
+    dict(H=2, N=9, KV=63), dict(H=2, N=130, KV=448, mask="causal"), dict(H=2, N=64, KV=1500, flat=True),
+    # at most 8 queries: the few-query kernel of the packed form (stages of 192 keys: one, one key into the second, many)
+    dict(H=20, N=5, KV=1536, flat=True, pad_from=1500), dict(H=4, N=1, KV=1), dict(H=4, N=5, KV=37, mask="beam"), dict(H=2, N=3, KV=200, mask="causal"),
+    dict(H=2, N=8, KV=448, mask="beam"), dict(H=2, N=1, KV=192), dict(H=2, N=4, KV=193, mask="beam"), dict(H=1, N=2, KV=7500), dict(H=3, N=5, KV=583, mask="beam")])
 def test_flash_attn_packed_f16_chain(pkg, oracle, gpu, case):
     # MI355X_FA_F16_PK: the same key order and f16 accumulator, the step as one fused f16 multiply-add on the factor rounded
     # to f16 (the reference's arithmetic where it has f16 vector units).  Checked against the pinned restatement of the x86
@@ -582,44 +585,45 @@ def test_flash_attn_packed_f16_chain(pkg, oracle, gpu, case):
     if "mask" in case:
         m = np.full((-(-N // 64) * 64, KV), -np.inf, dtype=np.float32)
         for r in range(N):
-            m[r, : KV - N + r + 1] = 0.0
+            if case["mask"] == "causal":
+                m[r, : KV - N + r + 1] = 0.0
+            else:
+                m[r, : (KV + 1) // 2] = 0.0
+                m[r, [c for c in range(KV) if c % N == r]] = 0.0
         mask = oracle.f32_to_f16_bits(m)
     got, name = run_fa(pkg, gpu, q, kb, vb, mask, 0.125, pkg.FA_F16_PK)
-    assert name == "flash_attn.seq_tile_pk"
+    assert name == ("flash_attn.seq_row_pk" if N <= 8 else "flash_attn.seq_tile_pk")
     want = oracle.flash_attn_ext(q, kb, vb, None if mask is None else mask[:N], 0.125)
     seq, _ = run_fa(pkg, gpu, q, kb, vb, mask, 0.125, pkg.FA_F16_SEQ)
     exact = _attention_float64(oracle, q, kb, vb, None if mask is None else mask, 0.125)
     print(f"packed chain {case}: vs oracle {oracle.nmse(got, want):.3e}, x86 form vs oracle {oracle.nmse(seq, want):.3e}, "
           f"packed vs f64 {oracle.nmse(got, exact):.3e}, oracle vs f64 {oracle.nmse(want, exact):.3e}", flush=True)
     assert oracle.nmse(got, want) <= 1e-5
-    # with at most 8 queries the mode is the f32-fma sequence of the few-query kernel, bit for bit
-    if N == 70:
-        a, name = run_fa(pkg, gpu, q[:, :5], kb, vb, None, 0.125, pkg.FA_F16_PK)
-        b, _ = run_fa(pkg, gpu, q[:, :5], kb, vb, None, 0.125, pkg.FA_F16_SEQ)
-        assert name == "flash_attn.seq_row" and np.array_equal(a.view(np.uint32), b.view(np.uint32))
+    again, _ = run_fa(pkg, gpu, q, kb, vb, mask, 0.125, pkg.FA_F16_PK)
+    assert np.array_equal(again.view(np.uint32), got.view(np.uint32))          # the same bits on every run
 
 
 def test_flash_attn_few_queries_take_the_f32_mask(pkg, oracle, gpu):
     # the few-query kernel reads the f32 tensor a graph would cast to f16 and rounds each value as the cast does: the same bits
     # as with the f16 copy, also for values that are not representable in f16; with more than 8 queries it says no
     lib = pkg.kernels()
-    for H, N, KV in ((4, 5, 300), (2, 1, 193), (3, 8, 64)):
+    for mode, H, N, KV in [(md, *shape) for md in (pkg.FA_F16_SEQ, pkg.FA_F16_PK) for shape in ((4, 5, 300), (2, 1, 193), (3, 8, 64))]:
         q, kb, vb = _attention_inputs(oracle, H, N, KV, False, None)
         m = (RNG.normal(size=(64, KV)) * 0.37).astype(np.float32)
         m[:, KV // 2:][RNG.random((64, KV - KV // 2)) < 0.4] = -np.inf
         m[:, 0] = 0.0
-        want, name = run_fa(pkg, gpu, q, kb, vb, oracle.f32_to_f16_bits(m), 0.125, pkg.FA_F16_SEQ)
-        assert name == "flash_attn.seq_row"
+        want, name = run_fa(pkg, gpu, q, kb, vb, oracle.f32_to_f16_bits(m), 0.125, mode)
+        assert name == ("flash_attn.seq_row" if mode == pkg.FA_F16_SEQ else "flash_attn.seq_row_pk")
         d_q, d_k, d_v, d_m = gpu.up(q), gpu.up(kb), gpu.up(vb), gpu.up(m)
         d_o = torch.zeros((N, H, 64), dtype=torch.float32, device=gpu.dev)
         pkg.check(lib.mi355x_flash_attn_ext(pkg.tensor(d_q, pkg.F32), pkg.tensor(d_k, pkg.F16), pkg.tensor(d_v, pkg.F16), pkg.tensor(d_m, pkg.F32),
-                                            pkg.tensor(d_o, pkg.F32), 0.125, pkg.FA_F16_SEQ, None, 0, gpu.stream))
+                                            pkg.tensor(d_o, pkg.F32), 0.125, mode, None, 0, gpu.stream))
         assert np.array_equal(gpu.down(d_o).view(np.uint32), want.view(np.uint32))
         # ... and leaves the f16 copy behind for later readers (rows of the queries; the rest is not touched)
         d_c = torch.full((64, KV), 7, dtype=torch.int16, device=gpu.dev)
         d_o.zero_()
         pkg.check(lib.mi355x_flash_attn_ext_cast_mask(pkg.tensor(d_q, pkg.F32), pkg.tensor(d_k, pkg.F16), pkg.tensor(d_v, pkg.F16), pkg.tensor(d_m, pkg.F32),
-                                                      pkg.tensor(d_c, pkg.F16), pkg.tensor(d_o, pkg.F32), 0.125, pkg.FA_F16_SEQ, None, 0, gpu.stream))
+                                                      pkg.tensor(d_c, pkg.F16), pkg.tensor(d_o, pkg.F32), 0.125, mode, None, 0, gpu.stream))
         assert np.array_equal(gpu.down(d_o).view(np.uint32), want.view(np.uint32))
         copy = gpu.down(d_c).view(np.uint16)
         assert np.array_equal(copy[:N], oracle.f32_to_f16_bits(m)[:N]) and np.all(copy[N:] == 7)
@@ -669,14 +673,16 @@ def test_flash_attn_few_queries_emit_q8_0(pkg, oracle, gpu):
     d_w = torch.zeros(N * k + N * (k // 32) * 8, dtype=torch.uint8, device=gpu.dev)
     tq, tk, tv, to = pkg.tensor(d_q, pkg.F32), pkg.tensor(d_k, pkg.F16), pkg.tensor(d_v, pkg.F16), pkg.tensor(d_o, pkg.F32)
     lib = pkg.kernels()
-    pkg.check(lib.mi355x_flash_attn_ext(tq, tk, tv, None, to, 0.125, pkg.FA_F16_SEQ | pkg.FA_EMIT_Q8_0, d_w.data_ptr(), d_w.numel(), gpu.stream))
-    y, image = gpu.down(d_o).reshape(N, k), gpu.down(d_w)
-    assert oracle.nmse(y, oracle.flash_attn_ext(q, kb, vb, None, 0.125).reshape(N, k)) <= 1e-6
-    want = oracle.quantize(oracle.Q8_0, y, act=True).reshape(N, k // 32, 34)
-    assert np.array_equal(image[: N * k].reshape(N, k // 32, 32), want[:, :, 2:])
-    assert np.array_equal(image[N * k : N * k + N * (k // 32) * 4].view(np.float32).reshape(N, k // 32),
-                          oracle.f16_bits_to_f32(want[:, :, :2].copy().view(np.uint16)[..., 0]))
-    assert np.array_equal(image[N * k + N * (k // 32) * 4 :].view(np.int32).reshape(N, k // 32), want[:, :, 2:].view(np.int8).astype(np.int32).sum(-1))
+    for mode, bound in ((pkg.FA_F16_SEQ, 1e-6), (pkg.FA_F16_PK, 1e-5)):
+        d_w.zero_()
+        pkg.check(lib.mi355x_flash_attn_ext(tq, tk, tv, None, to, 0.125, mode | pkg.FA_EMIT_Q8_0, d_w.data_ptr(), d_w.numel(), gpu.stream))
+        y, image = gpu.down(d_o).reshape(N, k), gpu.down(d_w)
+        assert oracle.nmse(y, oracle.flash_attn_ext(q, kb, vb, None, 0.125).reshape(N, k)) <= bound
+        want = oracle.quantize(oracle.Q8_0, y, act=True).reshape(N, k // 32, 34)
+        assert np.array_equal(image[: N * k].reshape(N, k // 32, 32), want[:, :, 2:])
+        assert np.array_equal(image[N * k : N * k + N * (k // 32) * 4].view(np.float32).reshape(N, k // 32),
+                              oracle.f16_bits_to_f32(want[:, :, :2].copy().view(np.uint16)[..., 0]))
+        assert np.array_equal(image[N * k + N * (k // 32) * 4 :].view(np.int32).reshape(N, k // 32), want[:, :, 2:].view(np.int8).astype(np.int32).sum(-1))
     # the many-query kernels do not write this form
     d_q9 = gpu.up(rnd((H, 9, 64)))
     d_o9 = torch.empty((9, H, 64), dtype=torch.float32, device=gpu.dev)

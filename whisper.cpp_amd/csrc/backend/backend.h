@@ -95,8 +95,9 @@ struct mi355x_backend_ctx {
     int         fa_accum = 0;           // V accumulation of attention: 0 the reference's sequence (f32 fma, f16 store, key by key);
                                         // bit 0: f32 accumulators (matrix cores) for more than 8 queries, bit 1: f32
                                         // accumulators for a decode step's few queries
-    int         fa_chain = 1;           // the f16 key-by-key step for more than 8 queries: 1 fused f16 multiply-add on the factor rounded to
-                                        // f16 (the reference's builds with f16 vector units), 0 f32 fma then f16 store (its x86 build)
+    int         fa_chain = 2;           // the f16 key-by-key step: 2 one fused f16 multiply-add on the factor rounded to f16 (the reference's
+                                        // builds with f16 vector units) in every launch, 1 only where a launch has more than 8 queries,
+                                        // 0 f32 fma then f16 store (its x86 build) everywhere
     bool        dead_f32 = true;        // a result whose only reader is the next launch's activation image is not also written as f32
                                         // (GGML_MI355X_DEAD_F32=0: always write it)
     bool        check_reads = true;     // refuse to read memory whose value a launch folded away (GGML_MI355X_CHECK_READS=0 turns the

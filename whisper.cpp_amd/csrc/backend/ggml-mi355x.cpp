@@ -568,7 +568,7 @@ static ggml_backend_t device_init_backend(ggml_backend_dev_t dev, const char *) 
     ctx->profile = env_flag("GGML_MI355X_PROFILE", false);
     ctx->exact   = env_flag("GGML_MI355X_EXACT", false);
     if (const char * e = getenv("GGML_MI355X_FA_ACCUM")) { const int v = atoi(e); if (v >= 0 && v <= 3) ctx->fa_accum = v; }
-    if (const char * e = getenv("GGML_MI355X_FA_CHAIN")) { const int v = atoi(e); if (v >= 0 && v <= 1) ctx->fa_chain = v; }
+    if (const char * e = getenv("GGML_MI355X_FA_CHAIN")) { const int v = atoi(e); if (v >= 0 && v <= 2) ctx->fa_chain = v; }
     ctx->weight_images = env_flag("GGML_MI355X_WEIGHT_IMAGES", true);
     ctx->dead_f32 = env_flag("GGML_MI355X_DEAD_F32", true);
     ctx->check_reads = env_flag("GGML_MI355X_CHECK_READS", true);
@@ -658,7 +658,7 @@ static int set_option(ggml_backend_t backend, const char * name, int value) {
     const bool is_accum = strcmp(name, "fa_accum") == 0, is_chain = strcmp(name, "fa_chain") == 0;
     if (!is_fuse && !is_profile && !is_exact && !is_accum && !is_chain) return -1;
     if (is_accum && (value < 0 || value > 3)) return -1;
-    if (is_chain && (value < 0 || value > 1)) return -1;
+    if (is_chain && (value < 0 || value > 2)) return -1;
     std::lock_guard<std::mutex> lock(g_live_mutex);
     for (mi355x_backend_ctx * ctx : g_live) {
         if (backend && ctx != (mi355x_backend_ctx *) backend->context) continue;

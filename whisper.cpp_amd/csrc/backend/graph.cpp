@@ -855,14 +855,14 @@ struct graph_runner {
                 const double bytes = (double) ggml_nelements(s0) * 4 + 2.0 * (double) k->ne[0] * k->ne[1] * k->ne[2] * k->ne[3] * 2 + nbytes_of(n);
                 // the accumulation option, bit 0: more than 8 queries, bit 1: a decode step's few queries
                 const bool f32_accum = s0->ne[1] > 8 ? (ctx->fa_accum & 1) != 0 : (ctx->fa_accum & 2) != 0;
-                const int mode = ctx->exact || f32_accum ? MI355X_FA_F32 : ctx->fa_chain == 1 && s0->ne[1] > 8 ? MI355X_FA_F16_PK : MI355X_FA_F16_SEQ;
+                const int mode = ctx->exact || f32_accum ? MI355X_FA_F32 : ctx->fa_chain == 2 || (ctx->fa_chain == 1 && s0->ne[1] > 8) ? MI355X_FA_F16_PK : MI355X_FA_F16_SEQ;
                 const char * name = mi355x_flash_attn_ext_kernel_name(&vq, &vk, mode);
                 // the output projection that follows takes its Q8_0-rounded activations from the attention kernel itself
                 const bool emits = !ctx->exact && (strncmp(name, "flash_attn.seq_tile", 19) == 0 || strcmp(name, "flash_attn.mfma_f32") == 0);
                 const ggml_tensor * key = emits ? image_consumer(n, i + 1) : nullptr;
                 // (a decode step's projection reads Q8_0 itself, written by the few-query kernel)
                 int form = 1;
-                if (!key && !ctx->exact && strcmp(name, "flash_attn.seq_row") == 0 && (key = image_consumer(n, i + 1, true))) form = 2;
+                if (!key && !ctx->exact && strncmp(name, "flash_attn.seq_row", 18) == 0 && (key = image_consumer(n, i + 1, true))) form = 2;
                 const size_t image_bytes = form == 1 ? (size_t) ggml_nelements(n) * 2 : (size_t) ggml_nelements(n) / 32 * 40;
                 if (key && !ctx->reserve_workspace(image_bytes + 256)) key = nullptr;
                 // ... and only the image when the projection is the very next launch: the f32 rows would have no reader

@@ -16,6 +16,9 @@
 //                                  against the LDS-staged V tile.
 //       k_fattn_seq_row    N <= 8: one block per (query, head): one wavefront (lane = d) runs the chain while the
 //                                  other three score, scan and stage the next 192 keys.
+//   MI355X_FA_F16_PK             the same sequence with the step of the reference's builds that have f16 vector units: the
+//                                factor rounded to f16, one fused f16 multiply-add per element (k_fattn_pk_tile for N > 8,
+//                                k_fattn_pk_row for N <= 8).
 //   MI355X_FA_F32          f32 accumulators: closer to exact arithmetic, not to the reference (whose f16 accumulator
 //                          loses about 1e-4 NMSE per attention, which whole-model logits then show as several 1e-3).
 //       k_fattn_mfma       N > 8:  both products on the matrix cores, online softmax, probabilities as f16 operands
@@ -374,7 +377,11 @@ __global__ void __launch_bounds__(256) k_fattn_seq_row(fa_args a, int kv_pad) {
     __shared__ float red_m[2][3], red_p[2][3], red_a[2][3];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int64_t n = blockIdx.x, h = blockIdx.y, i3 = blockIdx.z;
+    // Workgroup w runs on XCD w % 8, and each XCD has an L2 of its own: the queries of a head are dealt to one XCD (head h to
+    // XCD h % 8), so that a head's K and V rows are fetched into one L2, once, instead of into as many as it has queries.
+    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+    const int64_t n = slot % (int) a.N, h = xcd + 8 * (slot / (int) a.N), i3 = blockIdx.z;
+    if (h >= a.H) return;                                  // (the grid is 8 x ceil(H / 8) x N wide)
     const int KV = (int) a.KV;
     const int n_stages = (kv_pad + ROW_STAGE - 1) / ROW_STAGE;
 
@@ -628,6 +635,312 @@ __global__ void __launch_bounds__(256) k_fattn_seq_row(fa_args a, int kv_pad) {
             const int64_t blk = rowi * nbk + h * 2 + (lane >> 5);
             ((float *)(q8 + rows * K))[blk] = h2f(f2h_bits(amax / 127.0f));
             ((int32_t *)(q8 + rows * K + rows * nbk * 4))[blk] = qsum;
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------------------
+// k_fattn_pk_row: one block per (query, head), the packed-f16 form of the step (MI355X_FA_F16_PK with at most 8 queries)
+//
+// The same pipeline as k_fattn_seq_row — wavefront 0 walks the chain over stage s while wavefronts 1 .. 3 make the factors
+// of stage s + 1 and the scores of stage s + 2, one barrier per stage — with the step the reference's Arm build takes
+// (vec.h:180-203, 295-311: the factor rounded to f16, one f16 fused multiply-add per element).  A key is then ONE dependent
+// instruction for the walker, v_pk_fma_f16 on a lane's pair of d (3.7 ns against the 5.3 ns of v_fma_mix_f32 +
+// v_cvt_f16_f32), and what stood beside the chain had to shrink with it (a stage of 192 keys: 1.9 us -> 1.05 us):
+//   walker     lane l holds d = 2 (l % 32), 2 (l % 32) + 1 (the upper half of the wavefront mirrors the lower).  Per unit of
+//              32 keys: eight 16-byte reads of V (the stage holds V as [d pair][key], a dword per key), four 16-byte reads
+//              of factors (f16, eight keys each, one address for all lanes), and the unit's raise bits as a scalar: no
+//              vote, no selects.  A unit without a raise is 32 instructions in a row; a unit with one multiplies the
+//              accumulator by a second factor in front of every key (1 where the key raises nothing) — no branch per key
+//              and no copy of the code per raise pattern, which for a lone wavefront cost more than the arithmetic.
+//   producers  the factors of a key come from one v_exp_f32: with scores in log2 units, exp2(-|s - M|) against the
+//              exclusive prefix maximum M is vs where the maximum stands and ms where the key raises it (then vs is
+//              exactly 1).  The denominator's share of a stage is a plain sum of exp2(s - M_end) over its keys and
+//              P = exp2(M_before - M_end): S <- S P + A (f32, as the reference keeps it).  V rows go to the stage as
+//              they are loaded, dword by dword — pairs of d stay together, so there is nothing to transpose inside a
+//              register.  Rows come through buffer descriptors with the stage's offset as a scalar operand: no address
+//              arithmetic in the loop (it was a quarter of a round's instructions, the slow integer multiplies among them).
+//   placement  the queries of a head run on one XCD, so a head's K and V reach one L2, once (with a query per XCD, as
+//              the plain grid deals them, every XCD fetches every head: more than its L2 holds).
+// ------------------------------------------------------------------------------------------------------
+
+#define PROW_PITCH (ROW_STAGE + 4)     // dwords per d-pair row of the V stage: 784 bytes, 16 mod 256
+
+__global__ void __launch_bounds__(256) k_fattn_pk_row(fa_args a, int kv_pad) {
+    // V stage: [d pair][key], a dword per key.  The 16-byte piece g (keys 4 g .. 4 g + 3) of row p sits at piece g ^ (p / 16):
+    // 16 lanes of a producer's write (eight rows four apart, pieces 2 r and 2 r + 1) and 16 lanes of the walker's read (16
+    // consecutive rows, one piece: the pitch is 16 bytes past a multiple of 256) each cover all 64 banks once.
+    __shared__ __attribute__((aligned(16))) uint32_t v_lds[2][32 * PROW_PITCH];
+    // two f16 factors per key: the accumulator is multiplied by fm (ms where the key raises the maximum, else 1) and takes
+    // v * fv (1 where it raises, else vs); a unit of 32 keys without a raise — almost all of them — needs fv only
+    __shared__ __attribute__((aligned(16))) uint16_t fv_lds[2][ROW_STAGE], fm_lds[2][ROW_STAGE];
+    __shared__ uint32_t raise_lds[2][8];                                      // does the key raise the maximum?  32 keys to a dword
+    __shared__ float red_m[2][3], red_a[2][3], red_p[2];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    // Workgroup w runs on XCD w % 8, and each XCD has an L2 of its own: the queries of a head are dealt to one XCD (head h to
+    // XCD h % 8), so that a head's K and V rows are fetched into one L2, once, instead of into as many as it has queries.
+    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+    const int64_t n = slot % (int) a.N, h = xcd + 8 * (slot / (int) a.N), i3 = blockIdx.z;
+    if (h >= a.H) return;                                  // (the grid is 8 x ceil(H / 8) x N wide)
+    const int KV = (int) a.KV;
+    const int n_stages = (kv_pad + ROW_STAGE - 1) / ROW_STAGE;
+
+    if (wave != 0) {
+        // ---- producers ----------------------------------------------------------------------------------------------
+        const float * qp = (const float *)(a.q + n * a.q_nb1 + h * a.q_nb2 + i3 * a.q_nb3);
+        const char *  kb = a.k + (h / a.hk_ratio) * a.k_nb2 + (i3 / a.k_ne3_ratio) * a.k_nb3;
+        const char *  vb = a.v + (h / a.hv_ratio) * a.v_nb2 + (i3 / a.v_ne3_ratio) * a.v_nb3;
+        const char * mp = a.mask ? a.mask + n * a.m_nb1 : nullptr;
+        const int stid = tid - WAVE, pw = wave - 1;
+        const float scale2 = a.scale * LOG2E_F;
+
+        // Rows are read eight lanes to a row (16 bytes each), as in k_fattn_seq_row, through buffer descriptors: the offset of a
+        // lane's eight rows inside a stage is computed once, the stage's own offset is a scalar operand of the load, and a key
+        // beyond the end reads zeros (its score is -inf, its factor 0) — no address arithmetic and no clamps inside the loop.
+        const int r8 = lane >> 3, c8 = lane & 7;
+        float q[8];                                        // this lane's piece of q
+        {
+            const float4 t0 = *(const float4 *)(qp + 8 * c8), t1 = *(const float4 *)(qp + 8 * c8 + 4);
+            q[0] = (float)(half_t) t0.x; q[1] = (float)(half_t) t0.y; q[2] = (float)(half_t) t0.z; q[3] = (float)(half_t) t0.w;
+            q[4] = (float)(half_t) t1.x; q[5] = (float)(half_t) t1.y; q[6] = (float)(half_t) t1.z; q[7] = (float)(half_t) t1.w;
+        }
+        const uint32_t k_nb1 = (uint32_t) a.k_nb1, v_nb1 = (uint32_t) a.v_nb1;
+        const __amdgpu_buffer_rsrc_t k_rs = __builtin_amdgcn_make_buffer_rsrc((void *) kb, 0, (uint32_t)(KV - 1) * k_nb1 + FA_D * 2, 0x00020000);
+        const __amdgpu_buffer_rsrc_t v_rs = __builtin_amdgcn_make_buffer_rsrc((void *) vb, 0, (uint32_t)(KV - 1) * v_nb1 + FA_D * 2, 0x00020000);
+        // the mask as f16, or as the f32 tensor an f16 copy would have been made of (then each value is rounded here as that copy
+        // rounds it): both forms are read, one of them from a descriptor without records (zeros)
+        const __amdgpu_buffer_rsrc_t m16_rs = __builtin_amdgcn_make_buffer_rsrc((void *)(mp ? mp : a.k), 0, mp && !a.mask_f32 ? (uint32_t) KV * 2 : 0u, 0x00020000);
+        const __amdgpu_buffer_rsrc_t m32_rs = __builtin_amdgcn_make_buffer_rsrc((void *)(mp ? mp : a.k), 0, mp && a.mask_f32 ? (uint32_t) KV * 4 : 0u, 0x00020000);
+        uint32_t k_off[8], v_off[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) { k_off[i] = (uint32_t)(pw * WAVE + 8 * r8 + i) * k_nb1 + 16 * c8; v_off[i] = (uint32_t)(pw * WAVE + 8 * r8 + i) * v_nb1 + 16 * c8; }
+        u32x4 krow[8];
+        u32x4 vrow[8];
+        uint16_t mbits = 0;                                // the mask value of key `stid` of the stage as loaded (f16)
+        auto load_k = [&](int s) __attribute__((always_inline)) {
+            const uint32_t so = (uint32_t) __builtin_amdgcn_readfirstlane(s * ROW_STAGE) * k_nb1;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) krow[i] = __builtin_amdgcn_raw_buffer_load_b128(k_rs, k_off[i], so, 0);
+            const uint32_t ko = (uint32_t) __builtin_amdgcn_readfirstlane(s * ROW_STAGE);
+            const uint16_t m16 = __builtin_amdgcn_raw_buffer_load_b16(m16_rs, stid * 2, ko * 2, 0);
+            const float    m32 = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(m32_rs, stid * 4, ko * 4, 0));
+            mbits = a.mask_f32 ? f2h_bits(m32) : m16;
+            const int key = s * ROW_STAGE + stid;
+            if (a.mask_copy && h == 0 && key < KV) *(uint16_t *)((char *) a.mask_copy + n * a.mc_nb1 + (int64_t) key * 2) = mbits;
+        };
+        auto load_v = [&](int s) __attribute__((always_inline)) {
+            const uint32_t so = (uint32_t) __builtin_amdgcn_readfirstlane(s * ROW_STAGE) * v_nb1;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) vrow[i] = __builtin_amdgcn_raw_buffer_load_b128(v_rs, v_off[i], so, 0);
+        };
+
+        float score, inc, exc;                             // of the stage scored last, in log2 units: the score, its scan, the scan of the lane before
+        auto score_phase = [&](int s) __attribute__((always_inline)) {
+            const int key = s * ROW_STAGE + stid;
+            // the piece's share of the eight rows' dot products (f32 multiply-adds on the converted halves: v_dot2_f32_f16 would
+            // halve them, and moves flat attention over 1500 keys from 2e-7 to 2e-5 of the pinned sequence), summed over the
+            // eight lanes of a row; lane c keeps row 8 r + c: its own key
+            // (the eight rows side by side, element by element and step by step: a lone wavefront pays the full latency of
+            // every instruction that depends on the one before it)
+            float part[8] = { 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f };
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) part[i] = __builtin_fmaf(q[e], (float) __builtin_bit_cast(half8_t, krow[i])[e], part[i]);
+            }
+#pragma unroll
+            for (int i = 0; i < 8; ++i) part[i] += dpp_move<float, 0xB1>(part[i]);      // quad_perm [1,0,3,2]
+#pragma unroll
+            for (int i = 0; i < 8; ++i) part[i] += dpp_move<float, 0x4E>(part[i]);      // quad_perm [2,3,0,1]
+#pragma unroll
+            for (int i = 0; i < 8; ++i) part[i] += dpp_move<float, 0x141>(part[i]);     // row_half_mirror
+            float dot = part[0];
+#pragma unroll
+            for (int i = 1; i < 8; ++i) dot = c8 == i ? part[i] : dot;
+            const float mval = mp ? h2f(mbits) : 0.0f;
+            score = key < KV && mval != -INFINITY ? __builtin_fmaf(dot, scale2, mval * LOG2E_F) : -INFINITY;
+            load_k(s + 1);
+            inc = wave_scan_max(score);
+            if (lane == WAVE - 1) red_m[s & 1][pw] = inc;
+            exc = dpp_fill<0x138>(inc, -INFINITY);         // wave_shr:1
+        };
+        load_v(0);
+        __builtin_amdgcn_sched_barrier(0);
+        load_k(0);
+        __builtin_amdgcn_sched_barrier(0);
+        score_phase(0);
+        __syncthreads();
+
+        float M = -INFINITY;                               // running maximum over the stages whose factors are made
+        for (int s = 1; s <= n_stages; ++s) {
+            // ---- factors of stage s - 1
+            {
+                const int f = (s - 1) & 1;
+                const float m0 = red_m[f][0], m1 = red_m[f][1], m2 = red_m[f][2];
+                float Mk = fmaxf(exc, M);                  // the maximum over every key before this one
+                if (pw > 0) Mk = fmaxf(Mk, m0);
+                if (pw > 1) Mk = fmaxf(Mk, m1);
+                const float Mend = fmaxf(fmaxf(M, m0), fmaxf(m1, m2));
+                // (-inf - -inf, a masked key before any other: NaN, which the maximum with 0 turns into 0)
+                const float e  = fmaxf(__builtin_amdgcn_exp2f(-fabsf(score - Mk)), 0.0f);
+                const float ak = fmaxf(__builtin_amdgcn_exp2f(score - Mend), 0.0f);
+                const bool raise = score > Mk;
+                const uint16_t eh = f2h_bits(e);
+                fv_lds[f][stid] = raise ? (uint16_t) 0x3c00 : eh;
+                fm_lds[f][stid] = raise ? eh : (uint16_t) 0x3c00;
+                const uint64_t rb = __ballot(raise);
+                float A = lanes_sum<16>(ak);                 // (the four rows' sums joined in a fixed order, without the LDS trip of a swizzle)
+                A = (readlane_f(A, 0) + readlane_f(A, 16)) + (readlane_f(A, 32) + readlane_f(A, 48));
+                if (lane == 0) {
+                    raise_lds[f][2 * pw] = (uint32_t) rb; raise_lds[f][2 * pw + 1] = (uint32_t)(rb >> 32);
+                    red_a[f][pw] = A;
+                    if (pw == 0) red_p[f] = fmaxf(__builtin_amdgcn_exp2f(M - Mend), 0.0f);
+                }
+                M = Mend;
+                // V rows -> [d pair][key]: dword j of the lane's eight rows is d pair 4 c + j of the keys 8 r .. 8 r + 7
+                {
+                    uint32_t * dst = v_lds[f] + (4 * c8) * PROW_PITCH;
+                    const int g = 16 * pw + 2 * r8, sw = c8 >> 2;
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        const u32x4 lo = { vrow[0][j], vrow[1][j], vrow[2][j], vrow[3][j] }, hi = { vrow[4][j], vrow[5][j], vrow[6][j], vrow[7][j] };
+                        *(u32x4 *)(dst + j * PROW_PITCH + 4 * (g ^ sw))       = lo;
+                        *(u32x4 *)(dst + j * PROW_PITCH + 4 * ((g + 1) ^ sw)) = hi;
+                    }
+                }
+                load_v(s);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            // ---- scores of stage s (there is none behind the last)
+            if (s < n_stages) score_phase(s);
+            __syncthreads();
+        }
+        return;
+    }
+
+    // ---- the walker ---------------------------------------------------------------------------------------------------
+    const int p = lane & 31;                               // d pair
+    uint32_t acc = 0;
+    constexpr int UNIT = 32;
+    struct unit { u32x4 v[UNIT / 4]; u32x4 f[UNIT / 8]; };
+    const int swz = p >> 4;
+    auto read_unit = [&](unit & u, int buf, int k0) __attribute__((always_inline)) {      // k0: a multiple of 32
+        const uint32_t * row = v_lds[buf] + p * PROW_PITCH;
+#pragma unroll
+        for (int i = 0; i < UNIT / 4; ++i) u.v[i] = *(const u32x4 *)(row + 4 * ((k0 / 4 + i) ^ swz));
+        const u32x4 * fs = (const u32x4 *)(fv_lds[buf] + k0);
+#pragma unroll
+        for (int i = 0; i < UNIT / 8; ++i) u.f[i] = fs[i];
+    };
+    // eight keys without a raise: one asm statement, so that nothing is placed between the dependent instructions
+    auto eight = [&](const u32x4 & v0, const u32x4 & v1, const u32x4 & f) __attribute__((always_inline)) {
+        asm("v_pk_fma_f16 %0, %1, %9, %0 op_sel_hi:[1,0,1]\n\t"
+            "v_pk_fma_f16 %0, %2, %9, %0 op_sel:[0,1,0] op_sel_hi:[1,1,1]\n\t"
+            "v_pk_fma_f16 %0, %3, %10, %0 op_sel_hi:[1,0,1]\n\t"
+            "v_pk_fma_f16 %0, %4, %10, %0 op_sel:[0,1,0] op_sel_hi:[1,1,1]\n\t"
+            "v_pk_fma_f16 %0, %5, %11, %0 op_sel_hi:[1,0,1]\n\t"
+            "v_pk_fma_f16 %0, %6, %11, %0 op_sel:[0,1,0] op_sel_hi:[1,1,1]\n\t"
+            "v_pk_fma_f16 %0, %7, %12, %0 op_sel_hi:[1,0,1]\n\t"
+            "v_pk_fma_f16 %0, %8, %12, %0 op_sel:[0,1,0] op_sel_hi:[1,1,1]"
+            : "+v"(acc)
+            : "v"(v0.x), "v"(v0.y), "v"(v0.z), "v"(v0.w), "v"(v1.x), "v"(v1.y), "v"(v1.z), "v"(v1.w), "v"(f.x), "v"(f.y), "v"(f.z), "v"(f.w));
+    };
+    // ... and eight keys of a unit in which some key raises the maximum: the scale by fm in front of every step.  No branch
+    // per key and no second copy of the code per raise pattern: a taken branch costs a lone wavefront as much as four keys,
+    // and code that is rarely run comes from beyond the instruction cache.
+    auto eight_scaled = [&](const u32x4 & v0, const u32x4 & v1, const u32x4 & f, const u32x4 & m) __attribute__((always_inline)) {
+        asm("v_pk_mul_f16 %0, %0, %13 op_sel_hi:[1,0]\n\t"            "v_pk_fma_f16 %0, %1, %9, %0 op_sel_hi:[1,0,1]\n\t"
+            "v_pk_mul_f16 %0, %0, %13 op_sel:[0,1] op_sel_hi:[1,1]\n\t" "v_pk_fma_f16 %0, %2, %9, %0 op_sel:[0,1,0] op_sel_hi:[1,1,1]\n\t"
+            "v_pk_mul_f16 %0, %0, %14 op_sel_hi:[1,0]\n\t"            "v_pk_fma_f16 %0, %3, %10, %0 op_sel_hi:[1,0,1]\n\t"
+            "v_pk_mul_f16 %0, %0, %14 op_sel:[0,1] op_sel_hi:[1,1]\n\t" "v_pk_fma_f16 %0, %4, %10, %0 op_sel:[0,1,0] op_sel_hi:[1,1,1]\n\t"
+            "v_pk_mul_f16 %0, %0, %15 op_sel_hi:[1,0]\n\t"            "v_pk_fma_f16 %0, %5, %11, %0 op_sel_hi:[1,0,1]\n\t"
+            "v_pk_mul_f16 %0, %0, %15 op_sel:[0,1] op_sel_hi:[1,1]\n\t" "v_pk_fma_f16 %0, %6, %11, %0 op_sel:[0,1,0] op_sel_hi:[1,1,1]\n\t"
+            "v_pk_mul_f16 %0, %0, %16 op_sel_hi:[1,0]\n\t"            "v_pk_fma_f16 %0, %7, %12, %0 op_sel_hi:[1,0,1]\n\t"
+            "v_pk_mul_f16 %0, %0, %16 op_sel:[0,1] op_sel_hi:[1,1]\n\t" "v_pk_fma_f16 %0, %8, %12, %0 op_sel:[0,1,0] op_sel_hi:[1,1,1]"
+            : "+v"(acc)
+            : "v"(v0.x), "v"(v0.y), "v"(v0.z), "v"(v0.w), "v"(v1.x), "v"(v1.y), "v"(v1.z), "v"(v1.w), "v"(f.x), "v"(f.y), "v"(f.z), "v"(f.w),
+              "v"(m.x), "v"(m.y), "v"(m.z), "v"(m.w));
+    };
+    struct scales { u32x4 m[UNIT / 8]; };
+    auto read_scales = [&](scales & t, int buf, int k0) __attribute__((always_inline)) {
+        const u32x4 * ms = (const u32x4 *)(fm_lds[buf] + k0);
+#pragma unroll
+        for (int i = 0; i < UNIT / 8; ++i) t.m[i] = ms[i];
+    };
+    auto run_unit_with = [&](const unit & u, uint32_t raised, const scales & t) __attribute__((always_inline)) {   // raised: uniform
+        if (raised == 0) {
+#pragma unroll
+            for (int g = 0; g < UNIT / 8; ++g) eight(u.v[2 * g], u.v[2 * g + 1], u.f[g]);
+        } else {                                           // rare after the first keys of a row
+#pragma unroll
+            for (int g = 0; g < UNIT / 8; ++g) eight_scaled(u.v[2 * g], u.v[2 * g + 1], u.f[g], t.m[g]);
+        }
+    };
+    auto run_unit = [&](const unit & u, uint32_t raised, int buf, int k0) __attribute__((always_inline)) {
+        scales t = {};
+        if (raised != 0) read_scales(t, buf, k0);
+        run_unit_with(u, raised, t);
+    };
+    auto raise_bits = [&](int buf, int u) __attribute__((always_inline)) { return (uint32_t) __builtin_amdgcn_readfirstlane((int) raise_lds[buf][u]); };
+
+    float S = 0.0f;
+    unit ua, ub, uc;
+    scales sc = {};                                        // of the unit held in uc, when it has a raise
+    uint32_t rc = 0;                                       // raise bits of the unit held in uc
+    bool pending = false;                                  // uc holds the sixth unit of the stage before
+    __syncthreads();                                       // stage 0 is scored
+    for (int s = 0; s < n_stages; ++s) {
+        __syncthreads();                                   // stage s has its factors and its V rows
+        const int buf = s & 1;
+        const int nk = min(ROW_STAGE, kv_pad - s * ROW_STAGE);                  // 64, 128 or 192
+        read_unit(ua, buf, 0);
+        const uint32_t r0 = raise_bits(buf, 0), r1 = raise_bits(buf, 1), r2 = raise_bits(buf, 2), r3 = raise_bits(buf, 3), r4 = raise_bits(buf, 4), r5 = raise_bits(buf, 5);
+        S = S * red_p[buf] + ((red_a[buf][0] + red_a[buf][1]) + red_a[buf][2]);
+        if (pending) run_unit_with(uc, rc, sc);           // (its scales were read before the barrier: the producers have the buffer now)
+        read_unit(ub, buf, UNIT);
+        run_unit(ua, r0, buf, 0);
+        if (nk > 2 * UNIT) read_unit(uc, buf, 2 * UNIT);
+        run_unit(ub, r1, buf, UNIT);
+        pending = false;
+        if (nk > 2 * UNIT) {
+            read_unit(ua, buf, 3 * UNIT);
+            run_unit(uc, r2, buf, 2 * UNIT);
+            if (nk > 4 * UNIT) read_unit(ub, buf, 4 * UNIT);
+            run_unit(ua, r3, buf, 3 * UNIT);
+            if (nk > 4 * UNIT) {
+                read_unit(uc, buf, 5 * UNIT);
+                if (r5 != 0) read_scales(sc, buf, 5 * UNIT);
+                run_unit(ub, r4, buf, 4 * UNIT);
+                rc = r5;
+                pending = true;
+            }
+        }
+    }
+    if (pending) run_unit_with(uc, rc, sc);
+
+    const float inv = 1.0f / S;
+    half2_t acc_h; __builtin_memcpy(&acc_h, &acc, 4);
+    const float o0 = (float) acc_h[0] * inv, o1 = (float) acc_h[1] * inv;
+    float * dp = (float *) a.d + ((i3 * a.N + n) * a.H + h) * FA_D;
+    if (lane < 32) *(float2 *)(dp + 2 * p) = make_float2(o0, o1);
+    if (a.x16) {
+        // MI355X_FA_EMIT_Q8_0 (rows [N][H * 64]: int8 quants | f32 scales | int32 block sums): 16 lanes hold a block
+        float amax = fmaxf(fabsf(o0), fabsf(o1));
+        amax = lanes_max<16>(amax);
+        const float id = amax != 0.0f ? 127.0f / amax : 0.0f;
+        const int q0 = (int) rintf(o0 * id), q1 = (int) rintf(o1 * id);
+        int qsum = q0 + q1;
+        qsum = lanes_sum<16>(qsum);
+        char * q8 = (char *) a.x16;
+        const int64_t K = a.H * FA_D, nbk = K / 32, rows = a.N * a.ne3, rowi = i3 * a.N + n;
+        if (lane < 32) {
+            *(uint16_t *)(q8 + rowi * K + h * FA_D + 2 * p) = (uint16_t)((q0 & 0xff) | ((q1 & 0xff) << 8));
+            if ((p & 15) == 0) {
+                const int64_t blk = rowi * nbk + h * 2 + (p >> 4);
+                ((float *)(q8 + rows * K))[blk] = h2f(f2h_bits(amax / 127.0f));
+                ((int32_t *)(q8 + rows * K + rows * nbk * 4))[blk] = qsum;
+            }
         }
     }
 }
@@ -1418,12 +1731,15 @@ __global__ void __launch_bounds__(256) k_fattn_mfma(fa_args a) {
 
 #define SEQ_ROW_MAX_N   8
 
-enum { FA_K_VEC = 0, FA_K_SEQ_ROW = 1, FA_K_SEQ_TILE = 2, FA_K_MFMA = 3 };
+enum { FA_K_VEC = 0, FA_K_SEQ_ROW = 1, FA_K_SEQ_TILE = 2, FA_K_MFMA = 3, FA_K_PK_ROW = 4 };
+static inline bool fa_is_row(int kernel) { return kernel == FA_K_SEQ_ROW || kernel == FA_K_PK_ROW; }
 
-static int fa_kernel(const mi355x_tensor * q, const mi355x_tensor * k, int mode) {
+// k_fattn_pk_row addresses the rows of a head's K and V with 32-bit offsets
+static bool fits_32bit_offsets(const mi355x_tensor * t) { return t->ne[1] > 0 && t->nb[1] > 0 && (uint64_t) t->ne[1] * (uint64_t) t->nb[1] < ((uint64_t) 1 << 31); }
+
+static int fa_kernel(const mi355x_tensor * q, const mi355x_tensor * k, int mode, const mi355x_tensor * v = nullptr) {
     if (mode == MI355X_FA_F32) return q->ne[1] > SEQ_ROW_MAX_N ? FA_K_MFMA : FA_K_VEC;
-    (void) k;
-    if (q->ne[1] <= SEQ_ROW_MAX_N) return FA_K_SEQ_ROW;
+    if (q->ne[1] <= SEQ_ROW_MAX_N) return mode == MI355X_FA_F16_PK && fits_32bit_offsets(k) && (!v || fits_32bit_offsets(v)) ? FA_K_PK_ROW : FA_K_SEQ_ROW;
     return FA_K_SEQ_TILE;
 }
 
@@ -1431,6 +1747,7 @@ extern "C" const char * mi355x_flash_attn_ext_kernel_name(const mi355x_tensor * 
     if (!q || !k) return "flash_attn.invalid";
     switch (fa_kernel(q, k, mode)) {
         case FA_K_SEQ_ROW:  return "flash_attn.seq_row";
+        case FA_K_PK_ROW:   return "flash_attn.seq_row_pk";
         case FA_K_SEQ_TILE: return mode == MI355X_FA_F16_PK ? "flash_attn.seq_tile_pk" : "flash_attn.seq_tile";
         case FA_K_MFMA:     return "flash_attn.mfma_f32";
         default:            return "flash_attn.vec_f32";
@@ -1451,7 +1768,7 @@ static int flash_attn_ext(const mi355x_tensor * q, const mi355x_tensor * k, cons
     if (emit && emit_q8) return MI355X_ERR_INVALID;
     if (mode != MI355X_FA_F16_SEQ && mode != MI355X_FA_F32 && mode != MI355X_FA_F16_PK) return MI355X_ERR_INVALID;
     // dst without memory: only the image is wanted (the key-by-key tile kernel with MI355X_FA_EMIT_F16)
-    if (!dst->data && !(emit && fa_kernel(q, k, mode) == FA_K_SEQ_TILE)) return MI355X_ERR_INVALID;
+    if (!dst->data && !(emit && fa_kernel(q, k, mode, v) == FA_K_SEQ_TILE)) return MI355X_ERR_INVALID;
     if (q->type != MI355X_TYPE_F32 || k->type != MI355X_TYPE_F16 || v->type != MI355X_TYPE_F16 || dst->type != MI355X_TYPE_F32) return MI355X_ERR_UNSUPPORTED;
     if (q->ne[0] != FA_D || k->ne[0] != FA_D || v->ne[0] != FA_D) return MI355X_ERR_UNSUPPORTED;
     if (q->nb[0] != 4 || k->nb[0] != 2 || v->nb[0] != 2) return MI355X_ERR_UNSUPPORTED;
@@ -1461,7 +1778,7 @@ static int flash_attn_ext(const mi355x_tensor * q, const mi355x_tensor * k, cons
     if (dst->ne[0] != FA_D || dst->ne[1] != H || dst->ne[2] != N || dst->ne[3] != q->ne[3] || !is_contiguous(dst)) return MI355X_ERR_INVALID;
     if (mask) {
         // an F32 mask is what the few-query kernel takes in place of its f16 copy (same values after its own rounding)
-        if (mask->type == MI355X_TYPE_F32) { if (fa_kernel(q, k, mode) != FA_K_SEQ_ROW) return MI355X_ERR_UNSUPPORTED; }
+        if (mask->type == MI355X_TYPE_F32) { if (!fa_is_row(fa_kernel(q, k, mode, v))) return MI355X_ERR_UNSUPPORTED; }
         else if (mask->type != MI355X_TYPE_F16) return MI355X_ERR_UNSUPPORTED;
         if (mask->ne[0] != KV || mask->ne[1] < N || mask->nb[0] != type_size(mask->type)) return MI355X_ERR_INVALID;
     }
@@ -1499,24 +1816,29 @@ static int flash_attn_ext(const mi355x_tensor * q, const mi355x_tensor * k, cons
     a.x16 = nullptr;
     if (emit) {
         // only the tile kernels write the image; say so rather than silently skip it
-        if (fa_kernel(q, k, mode) != FA_K_SEQ_TILE && fa_kernel(q, k, mode) != FA_K_MFMA) return MI355X_ERR_UNSUPPORTED;
+        if (fa_kernel(q, k, mode, v) != FA_K_SEQ_TILE && fa_kernel(q, k, mode, v) != FA_K_MFMA) return MI355X_ERR_UNSUPPORTED;
         if (!workspace || (uintptr_t) workspace % 16 != 0 || workspace_size < (size_t)(N * H * q->ne[3]) * FA_D * sizeof(half_t)) return MI355X_ERR_WORKSPACE;
         a.x16 = (half_t *) workspace;
     }
     if (emit_q8) {
         // the few-query kernel writes the Q8_0 form
-        if (fa_kernel(q, k, mode) != FA_K_SEQ_ROW) return MI355X_ERR_UNSUPPORTED;
+        if (!fa_is_row(fa_kernel(q, k, mode, v))) return MI355X_ERR_UNSUPPORTED;
         const size_t rows = (size_t)(N * q->ne[3]), K = (size_t) H * FA_D;
         if (!workspace || (uintptr_t) workspace % 16 != 0 || workspace_size < rows * K + rows * (K / 32) * 8) return MI355X_ERR_WORKSPACE;
         a.x16 = (half_t *) workspace;
     }
     hipStream_t st = (hipStream_t) stream;
 
-    switch (fa_kernel(q, k, mode)) {
+    switch (fa_kernel(q, k, mode, v)) {
         case FA_K_SEQ_ROW: {
             const int kv_pad = (int)((KV + ROW_CHUNK - 1) / ROW_CHUNK * ROW_CHUNK);
-            dim3 grid((unsigned) N, (unsigned) H, (unsigned) q->ne[3]);
+            dim3 grid((unsigned)(8 * ((H + 7) / 8) * N), 1, (unsigned) q->ne[3]);
             k_fattn_seq_row<<<grid, 256, 0, st>>>(a, kv_pad);
+        } break;
+        case FA_K_PK_ROW: {
+            const int kv_pad = (int)((KV + ROW_CHUNK - 1) / ROW_CHUNK * ROW_CHUNK);
+            dim3 grid((unsigned)(8 * ((H + 7) / 8) * N), 1, (unsigned) q->ne[3]);
+            k_fattn_pk_row<<<grid, 256, 0, st>>>(a, kv_pad);
         } break;
         case FA_K_SEQ_TILE: {
             const int64_t gx = (N + T_Q - 1) / T_Q;
