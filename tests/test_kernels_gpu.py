@@ -1049,3 +1049,17 @@ def test_measurement_probes_run_and_reject_bad_arguments(pkg, gpu):
     st = stamps.cpu()
     assert int(st[:n].min()) >= int(st[n:n + 16].min()) > 0        # every chunk finished after the first workgroup started
     assert lib.mi355x_probe_read_stamped(buf.data_ptr(), buf.numel(), out.data_ptr(), 16, None, gpu.stream) == -2
+
+
+def test_the_three_instruction_division_by_127_is_the_division(pkg, gpu):
+    # the scale of every Q8_0 block the kernels round activations to is amax / 127.0f; they compute it as a product with the
+    # reciprocal corrected once by the exact residual (div127 in csrc/kernels/common.h).  Every non-negative float, infinity
+    # included, through both on the device: no result may differ.
+    import ctypes as C
+    from pathlib import Path
+    lib = C.CDLL(str(Path(pkg.__file__).resolve().parent / "lib" / "libmi355x_probes.so"))
+    lib.mi355x_probe_div127.restype, lib.mi355x_probe_div127.argtypes = C.c_int, [C.c_void_p, C.c_void_p]
+    n = torch.ones(1, dtype=torch.int64, device=gpu.dev)
+    pkg.check(lib.mi355x_probe_div127(n.data_ptr(), gpu.stream))
+    torch.cuda.synchronize()
+    assert int(n.item()) == 0

@@ -6,6 +6,8 @@
 //   mi355x_probe_read_stamped      the read stream with a time stamp per workgroup and chunk
 //   mi355x_probe_gemv_tiles_stamped  an instance of the product's own logits kernel (k_gemv_q8_0_tiles, same source) that
 //                                  also leaves a time stamp per wavefront and tile
+//   mi355x_probe_div127            every finite non-negative float through the kernels' three-instruction a / 127.0f beside the
+//                                  division itself: the number of results that differ (the claim is none)
 // The stamped forms answer what a stream sustains between its ramp and its tail: the stamps are the device's 100 MHz
 // clock (s_memrealtime), one after each unit of work; the caller sorts the completions and divides the bytes finished
 // between the 10th and the 90th percentile by the time between them.
@@ -111,5 +113,25 @@ PROBE_API int mi355x_probe_gemv_tiles_stamped(const void * tiles, int64_t K, int
     *tiles_per_wavefront = (n_tiles + *wavefronts - 1) / *wavefronts;
     if (!stamps) return MI355X_OK;                         // (sizes only)
     k_gemv_q8_0_tiles<20, true><<<grid, 256, 0, (hipStream_t) stream>>>(a, (uint64_t *) stamps);
+    return launch_status();
+}
+
+
+// ---- div127 (kernels/common.h) against the division, over every finite non-negative float
+__global__ void __launch_bounds__(256) k_probe_div127(unsigned long long * __restrict__ differing) {
+    const uint64_t stride = (uint64_t) gridDim.x * blockDim.x;
+    unsigned long long n = 0;
+    for (uint64_t i = (uint64_t) blockIdx.x * blockDim.x + threadIdx.x; i <= 0x7f800000u; i += stride) {      // (up to and with infinity)
+        const float a = __builtin_bit_cast(float, (uint32_t) i);
+        const float want = a / 127.0f, got = div127(a);
+        n += __builtin_bit_cast(uint32_t, want) != __builtin_bit_cast(uint32_t, got);
+    }
+    if (n) atomicAdd(differing, n);
+}
+// differing: 8 bytes of device memory, zeroed by the call; the count is there when the stream has finished
+PROBE_API int mi355x_probe_div127(void * differing, void * stream) {
+    if (!differing || (uintptr_t) differing % 8 != 0) return MI355X_ERR_INVALID;
+    if (hipMemsetAsync(differing, 0, 8, (hipStream_t) stream) != hipSuccess) return MI355X_ERR_HIP;
+    k_probe_div127<<<2048, 256, 0, (hipStream_t) stream>>>((unsigned long long *) differing);
     return launch_status();
 }

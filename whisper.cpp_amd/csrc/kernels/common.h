@@ -118,6 +118,18 @@ template <int W> __device__ __forceinline__ float lanes_max(float x) { return la
 __device__ __forceinline__ float wave_sum(float v) { return lanes_sum<WAVE>(v); }
 __device__ __forceinline__ float wave_max(float v) { return lanes_max<WAVE>(v); }
 
+// a / 127.0f, bit for bit — the scale of a Q8_0 block, amax / 127 (quantize_row_q8_0, ggml-cpu-quants.c:808-865): the product
+// with the rounded reciprocal, corrected once by the exact residual.  Three multiply-adds where the division takes twelve
+// instructions, and the same result for every finite non-negative float (checked over all 2^31 of them on the host and on
+// the device; the harness library's mi355x_probe_div127 repeats the device check).  Infinity and NaN, whose residual is
+// NaN, keep the plain product, which is what the division gives for them.
+__device__ __forceinline__ float div127(float a) {
+    const float r = 1.0f / 127.0f;
+    const float q = a * r;
+    const float e = __builtin_fmaf(-q, 127.0f, a);
+    return e == e ? __builtin_fmaf(e, r, q) : q;
+}
+
 // GELU as ggml_vec_gelu_f32 evaluates it (ggml/src/ggml-cpu/vec.h:443-457): outside (-10, 10) the clamps, inside a
 // lookup in a 65536-entry table indexed by the f16 bits of x that holds f16(gelu(f32(f16 x))).  `table` is the device
 // copy of that table (gelu_table_device below).

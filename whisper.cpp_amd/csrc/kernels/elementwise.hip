@@ -367,7 +367,7 @@ __global__ void k_quantize_q8_0(const float * __restrict__ x, uint8_t * __restri
     float amax = fabsf(v);
 #pragma unroll
     for (int o = 16; o > 0; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o, 32));
-    const float d  = amax / 127.0f;
+    const float d  = div127(amax);
     const float id = amax != 0.0f ? 127.0f / amax : 0.0f;
     uint8_t * b = y + blk * 34;
     if (j == 0) *(uint16_t *) b = f2h_bits(d);

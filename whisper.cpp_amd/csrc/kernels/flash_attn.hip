@@ -633,7 +633,7 @@ __global__ void __launch_bounds__(256) k_fattn_seq_row(fa_args a, int kv_pad) {
         ((int8_t *) q8)[rowi * K + h * FA_D + lane] = (int8_t) q;
         if ((lane & 31) == 0) {
             const int64_t blk = rowi * nbk + h * 2 + (lane >> 5);
-            ((float *)(q8 + rows * K))[blk] = h2f(f2h_bits(amax / 127.0f));
+            ((float *)(q8 + rows * K))[blk] = h2f(f2h_bits(div127(amax)));
             ((int32_t *)(q8 + rows * K + rows * nbk * 4))[blk] = qsum;
         }
     }
@@ -938,7 +938,7 @@ __global__ void __launch_bounds__(256) k_fattn_pk_row(fa_args a, int kv_pad) {
             *(uint16_t *)(q8 + rowi * K + h * FA_D + 2 * p) = (uint16_t)((q0 & 0xff) | ((q1 & 0xff) << 8));
             if ((p & 15) == 0) {
                 const int64_t blk = rowi * nbk + h * 2 + (p >> 4);
-                ((float *)(q8 + rows * K))[blk] = h2f(f2h_bits(amax / 127.0f));
+                ((float *)(q8 + rows * K))[blk] = h2f(f2h_bits(div127(amax)));
                 ((int32_t *)(q8 + rows * K + rows * nbk * 4))[blk] = qsum;
             }
         }
@@ -1245,7 +1245,7 @@ __global__ void __launch_bounds__(512, 2) k_fattn_seq_tile(fa_args a) {
         amax = fmaxf(amax, __builtin_bit_cast(float, __builtin_amdgcn_ds_swizzle(__builtin_bit_cast(int, amax), 0x401F)));
         if (n < a.N) {
             const float id = amax != 0.0f ? 127.0f / amax : 0.0f;
-            const float dq = h2f(f2h_bits(amax / 127.0f));
+            const float dq = h2f(f2h_bits(div127(amax)));
             half8_t h0, h1;
 #pragma unroll
             for (int e = 0; e < 8; ++e) { h0[e] = (half_t)((rintf(o[e] * id) + 0.0f) * dq); h1[e] = (half_t)((rintf(o[8 + e] * id) + 0.0f) * dq); }
@@ -1518,7 +1518,7 @@ __global__ void __launch_bounds__(512, 2) k_fattn_pk_tile(fa_args a) {
             amax = lanes_max<8>(amax);
             if (n < a.N) {
                 const float id = amax != 0.0f ? 127.0f / amax : 0.0f;
-                const float dq = h2f(f2h_bits(amax / 127.0f));
+                const float dq = h2f(f2h_bits(div127(amax)));
                 half4_t hx;
 #pragma unroll
                 for (int e = 0; e < 4; ++e) hx[e] = (half_t)((rintf(o[e] * id) + 0.0f) * dq);
@@ -1712,7 +1712,7 @@ __global__ void __launch_bounds__(256) k_fattn_mfma(fa_args a) {
         amax = fmaxf(amax, __shfl_xor(amax, 32, WAVE));
         if (n < a.N) {
             const float id = amax != 0.0f ? 127.0f / amax : 0.0f;
-            const float dq = h2f(f2h_bits(amax / 127.0f));
+            const float dq = h2f(f2h_bits(div127(amax)));
             half_t * xp = a.x16 + row;
 #pragma unroll
             for (int q4 = 0; q4 < 4; ++q4) {

@@ -147,7 +147,7 @@ __device__ __forceinline__ void patch_epilogue(float16_t v, const epi_args & e, 
 #pragma unroll
         for (int i = 1; i < 8; ++i) mine = (lane & 7) == i ? rmax[i] : mine;
         const float id_m = mine != 0.0f ? 127.0f / mine : 0.0f;
-        const float dq_m = h2f(f2h_bits(mine / 127.0f));
+        const float dq_m = h2f(f2h_bits(div127(mine)));
         const int src = ((lane & 32) << 2);                 // byte address of lane 0 of this half-wavefront for ds_bpermute
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
@@ -274,7 +274,7 @@ __global__ void k_x_to_f16(const char * __restrict__ x, half_t * __restrict__ ou
         float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
         amax = lanes_max<8>(amax);
         const float id = amax != 0.0f ? 127.0f / amax : 0.0f;
-        const float d  = h2f(f2h_bits(amax / 127.0f));                      // the scale goes through f16, like block_q8_0.d
+        const float d  = h2f(f2h_bits(div127(amax)));                      // the scale goes through f16, like block_q8_0.d
         // (+ 0.0f: a quant that rounds to -0 is the integer 0, whose product with d is +0)
         h = (half4_t){ (half_t)((rintf(v.x * id) + 0.0f) * d), (half_t)((rintf(v.y * id) + 0.0f) * d), (half_t)((rintf(v.z * id) + 0.0f) * d), (half_t)((rintf(v.w * id) + 0.0f) * d) };
     } else {
@@ -961,7 +961,7 @@ __device__ __forceinline__ void quantize_x_to_lds(const mm_args & a, int32_t * x
                 const int idx = base + u * 256 + (int) threadIdx.x;      // lanes 8i .. 8i+7 share a block
                 float amax = fmaxf(fmaxf(fabsf(v[u].x), fabsf(v[u].y)), fmaxf(fabsf(v[u].z), fabsf(v[u].w)));
                 amax = lanes_max<8>(amax);
-                const float d  = amax / 127.0f;
+                const float d  = div127(amax);
                 const float id = amax != 0.0f ? 127.0f / amax : 0.0f;
                 const int q0 = (int) rintf(v[u].x * id), q1 = (int) rintf(v[u].y * id), q2 = (int) rintf(v[u].z * id), q3 = (int) rintf(v[u].w * id);
                 int sum = q0 + q1 + q2 + q3;
@@ -1112,7 +1112,7 @@ __global__ void __launch_bounds__(256) k_quantize_x_q8(const char * __restrict__
     const float4 v = *(const float4 *)(x + n * x_nb1 + c * 16);
     float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
     amax = lanes_max<8>(amax);
-    const float d  = amax / 127.0f;
+    const float d  = div127(amax);
     const float id = amax != 0.0f ? 127.0f / amax : 0.0f;
     const int q0 = (int) rintf(v.x * id), q1 = (int) rintf(v.y * id), q2 = (int) rintf(v.z * id), q3 = (int) rintf(v.w * id);
     int sum = q0 + q1 + q2 + q3;
@@ -1299,7 +1299,7 @@ __device__ __forceinline__ void gemv_qr_rows(const mm_args & a, PRO prologue = P
                 const int64_t bi = done_group / GPB, nb2 = a.M / QK;
                 ((int8_t *) img)[n * a.M + bi * QK + rr] = (int8_t) q;
                 if (rr == 0) {
-                    ((float *)(img + (size_t) NC * a.M))[n * nb2 + bi] = h2f(f2h_bits(amax / 127.0f));
+                    ((float *)(img + (size_t) NC * a.M))[n * nb2 + bi] = h2f(f2h_bits(div127(amax)));
                     ((int32_t *)(img + (size_t) NC * a.M + (size_t) NC * nb2 * 4))[n * nb2 + bi] = qsum;
                 }
             }
@@ -1449,7 +1449,7 @@ struct gemv_norm_prologue {
                     const int q0 = (int) rintf(r.x * id), q1 = (int) rintf(r.y * id), q2 = (int) rintf(r.z * id), q3 = (int) rintf(r.w * id);
                     const int qsum = lanes_sum<8>(q0 + q1 + q2 + q3);
                     xq[row * n4 + c] = (q0 & 0xFF) | ((q1 & 0xFF) << 8) | ((q2 & 0xFF) << 16) | ((q3 & 0xFF) << 24);
-                    if ((c & 7) == 0) { xd[row * nbk + c / 8] = h2f(f2h_bits(amax / 127.0f)); xsum[row * nbk + c / 8] = qsum; }
+                    if ((c & 7) == 0) { xd[row * nbk + c / 8] = h2f(f2h_bits(div127(amax))); xsum[row * nbk + c / 8] = qsum; }
                 }
             }
         }

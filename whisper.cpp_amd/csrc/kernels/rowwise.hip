@@ -64,7 +64,7 @@ __global__ void __launch_bounds__(ROWS_PER_BLOCK * WAVE) k_norm(tview s, tview d
                     float amax = fmaxf(fmaxf(fabsf(r.x), fabsf(r.y)), fmaxf(fabsf(r.z), fabsf(r.w)));
                     amax = lanes_max<8>(amax);
                     const float id = amax != 0.0f ? 127.0f / amax : 0.0f;
-                    const float dq = h2f(f2h_bits(amax / 127.0f));
+                    const float dq = h2f(f2h_bits(div127(amax)));
                     if (EMIT == 1) {
                         const half4_t h = { (half_t)((rintf(r.x * id) + 0.0f) * dq), (half_t)((rintf(r.y * id) + 0.0f) * dq), (half_t)((rintf(r.z * id) + 0.0f) * dq), (half_t)((rintf(r.w * id) + 0.0f) * dq) };
                         *(half4_t *)(x16 + row * ne0 + 4 * (int64_t) c) = h;
