@@ -656,8 +656,11 @@ static std::vector<float> read_filters(const std::string & path, int32_t * n_mel
     return filters;
 }
 
+// fresh_state: the call runs on a state of its own (whisper_full_with_state), made for it and freed after it.  The search's
+// first decoder keeps the generator it was given when its state was made (src/whisper.cpp:3481; the others are seeded in every
+// call, :5583), so only calls on new states draw the same candidates.
 static std::vector<whisper_token> run_full(whisper_context * ctx, const std::vector<float> & pcm, int beam, int max_tokens, int threads, int * rc, double * ms,
-                                           std::vector<int64_t> * t_dtw = nullptr, bool use_gpu_mel = false) {
+                                           std::vector<int64_t> * t_dtw = nullptr, bool use_gpu_mel = false, bool fresh_state = false) {
     whisper_full_params p = whisper_full_default_params(beam > 1 ? WHISPER_SAMPLING_BEAM_SEARCH : WHISPER_SAMPLING_GREEDY);
     p.n_threads = threads;
     p.print_progress = false; p.print_realtime = false; p.print_timestamps = false; p.print_special = false;
@@ -678,6 +681,17 @@ static std::vector<whisper_token> run_full(whisper_context * ctx, const std::vec
         g_mel_ms = now_ms() - m0;
         if (whisper_set_mel(ctx, mel.data(), (int) n_len, n_mel) != 0) { *rc = -102; *ms = 0; return {}; }
         *rc = whisper_full(ctx, p, nullptr, 0);          // no samples: transcribes from the mel it was given (src/whisper.cpp:5492)
+    } else if (fresh_state) {
+        std::vector<whisper_token> out;
+        whisper_state * st = whisper_init_state(ctx);
+        if (!st) { *rc = -103; *ms = 0; return out; }
+        *rc = whisper_full_with_state(ctx, st, p, pcm.data(), (int) pcm.size());
+        *ms = now_ms() - t0;
+        if (*rc == 0)
+            for (int i = 0; i < whisper_full_n_segments_from_state(st); ++i)
+                for (int j = 0; j < whisper_full_n_tokens_from_state(st, i); ++j) out.push_back(whisper_full_get_token_id_from_state(st, i, j));
+        whisper_free_state(st);
+        return out;
     } else
     // --processors N: whisper_full_parallel splits the audio over N states, each with its own backend instance and host thread
     *rc = g_processors > 1 ? whisper_full_parallel(ctx, p, pcm.data(), (int) pcm.size(), g_processors) : whisper_full(ctx, p, pcm.data(), (int) pcm.size());
@@ -725,8 +739,16 @@ static int cmd_full(const args & a) {
     bool repeat_identical = true;
     if (a.has("repeat")) {
         int r2 = 0; double ms2 = 0;
-        const std::vector<whisper_token> again = run_full(gpu, pcm, beam, max_tokens, threads, &r2, &ms2, nullptr, g_gpu_mel);
-        repeat_identical = r2 == 0 && again == tg;
+        if (beam > 1 && g_processors == 1 && !g_gpu_mel) {
+            // beam search: two calls on two new states (see run_full), compared with each other
+            int r1 = 0; double ms1 = 0;
+            const std::vector<whisper_token> one = run_full(gpu, pcm, beam, max_tokens, threads, &r1, &ms1, nullptr, false, true);
+            const std::vector<whisper_token> two = run_full(gpu, pcm, beam, max_tokens, threads, &r2, &ms2, nullptr, false, true);
+            repeat_identical = r1 == 0 && r2 == 0 && !one.empty() && one == two;
+        } else {
+            const std::vector<whisper_token> again = run_full(gpu, pcm, beam, max_tokens, threads, &r2, &ms2, nullptr, g_gpu_mel);
+            repeat_identical = r2 == 0 && again == tg;
+        }
     }
     const std::vector<whisper_token> tc = run_full(cpu, pcm, beam, max_tokens, threads, &rc, &ms_c, &dc);
     size_t same = 0;
