@@ -242,6 +242,23 @@ def test_whole_model_logits_and_greedy_ids(harness, models, key, steps):
         assert rows[-1]["encode_nodes"] > 1200 and rows[-1]["encode_launches"] < 300, rows[-1]
 
 
+@pytest.mark.parametrize("arch,ftype,batch", [("tiny", "q5_0", 1), ("small", "q5_0", 1), ("medium", "q8_0", 1), ("small", "q8_0", 5), ("medium", "q5_0", 5)])
+def test_whole_model_parity_on_the_other_model_sizes(harness, tmp_path, arch, ftype, batch):
+    # the widths between base and large: 384, 768 and 1024 (rows of 1.5, 3 and 4 segments of 256 for the LayerNorm, 6 / 12 / 16
+    # heads, other lanes-per-row and blocks-per-lane choices in the few-column products, other GEMM tile counts); one row per
+    # step, and five rows per step as in a beam search
+    path = tmp_path / f"{arch}-{ftype}.bin"
+    rc, rows = run_harness(harness, ["gen", "--arch", arch, "--ftype", ftype, "--out", str(path)], timeout=300)
+    assert rc == 0 and rows[-1]["ok"]
+    args = ["model", "--model", str(path), "--steps", "32"] if batch == 1 else ["model", "--model", str(path), "--batch", "5", "--kv-to", "100"]
+    rc, rows = run_harness(harness, args, timeout=1500)
+    s = rows[-1]
+    print(f"{arch} {ftype} batch {batch}: ids {s['ids_identical']}/{s['rows']}, clear {s['clear_ids_identical']}/{s['clear_steps']}, worst NMSE {s['worst_logits_nmse']:.2e}", flush=True)
+    check_model_summary(s, strict_ids=False)
+    assert rc == 0
+    path.unlink()
+
+
 @pytest.mark.parametrize("arch,ftype", [("large-v3", "q5_0"), ("large-v3-turbo", "q8_0")])
 def test_whole_model_parity_on_other_seeds(harness, tmp_path, arch, ftype):
     # the criterion above on two more random-init models and mel windows each (the parametrized test above runs seeds 1234 / 7)

@@ -13,6 +13,8 @@ static const arch k_archs[] = {
     { "micro",            51865,   1500,  128,    2,     2,     448,  128,    2,     2,      80  },
     { "tiny",             51865,   1500,  384,    6,     4,     448,  384,    6,     4,      80  },
     { "base",             51865,   1500,  512,    8,     6,     448,  512,    8,     6,      80  },
+    { "small",            51865,   1500,  768,    12,    12,    448,  768,    12,    12,     80  },
+    { "medium",           51865,   1500,  1024,   16,    24,    448,  1024,   16,    24,     80  },
     { "large-v3",         51866,   1500,  1280,   20,    32,    448,  1280,   20,    32,     128 },
     { "large-v3-turbo",   51866,   1500,  1280,   20,    32,    448,  1280,   20,    4,      128 },
 };

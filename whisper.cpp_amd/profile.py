@@ -3,7 +3,8 @@
 
     python whisper.cpp_amd/profile.py [--out gpurun_out/prof]
 
-Writes, under --out: `kernel_stats_encoder.csv`, `kernel_stats_decoder.csv` (rocprofv3 --kernel-trace --stats), `counters.json`
+Writes, under --out: `kernel_stats_encoder.csv`, `kernel_stats_decoder.csv` (rocprofv3 --kernel-trace --stats), `decode_positions.txt`
+(a decode step's launches one by one, from a kernel trace), `counters.json`
 (per-kernel averages of the --pmc passes) and `traffic.json` — HBM bytes per launch for the kernels bench.py reports, FETCH_SIZE
 and WRITE_SIZE per dispatch scaled by what the same counters read for a 256 MiB device copy.  `traffic.json` is what
 bench.py reads as `roofline.traffic` once it is copied to profiles/traffic.json; the tables under profiles/ are written from
@@ -87,6 +88,36 @@ def main() -> int:
         for f in glob.glob(str(d / "**" / "*kernel_stats.csv"), recursive=True):
             shutil.copy(f, out / f"kernel_stats_{name}.csv")
         shutil.rmtree(d, ignore_errors=True)
+
+    # ---- a decode step launch by launch: durations by position in the step (the steps begin at k_get_rows_add)
+    d = out / "trace_positions"
+    run(["rocprofv3", "--kernel-trace", "--output-format", "csv", "-d", str(d), "--", *DEC_CMD, "--reps", "1", "--warmup", "1", "--steps", "224"], out / "trace_positions.log", 170)
+    rows = []
+    for f in glob.glob(str(d / "**" / "*kernel_trace.csv"), recursive=True):
+        for r in csv.DictReader(open(f)):
+            rows.append((int(r["Start_Timestamp"]), int(r["End_Timestamp"]), r["Kernel_Name"]))
+    shutil.rmtree(d, ignore_errors=True)
+    rows.sort()
+    steps, cur = [], None
+    for st, en, name in rows:
+        if "k_get_rows_add" in name:
+            if cur: steps.append(cur)
+            cur = []
+        if cur is not None: cur.append((st, en, name))
+    if cur: steps.append(cur)
+    lengths = collections.Counter(len(x) for x in steps)
+    n_launch = lengths.most_common(1)[0][0] if lengths else 0
+    steps = [x for x in steps if len(x) == n_launch]
+    with open(out / "decode_positions.txt", "w") as f:
+        f.write(f"{len(steps)} steps of {n_launch} launches; microseconds; 'gap' is the idle time in front of the launch (under the profiler the host preparing it)\n")
+        kernel_us = gap_us = 0.0
+        for pos in range(n_launch):
+            dur = sorted((x[pos][1] - x[pos][0]) / 1e3 for x in steps)
+            gap = [(x[pos][0] - x[pos - 1][1]) / 1e3 for x in steps] if pos else [0.0]
+            name = steps[0][pos][2].split("(")[0][:46]
+            kernel_us += sum(dur) / len(dur); gap_us += sum(gap) / len(gap)
+            f.write(f"{pos:2d} {name:46s} avg {sum(dur) / len(dur):6.2f} min {dur[0]:6.2f} med {dur[len(dur) // 2]:6.2f} max {dur[-1]:6.2f}  gap avg {sum(gap) / len(gap):5.2f}\n")
+        f.write(f"kernel us per step {kernel_us:.1f}, gaps per step {gap_us:.1f}\n")
 
     # ---- HBM traffic: FETCH_SIZE and WRITE_SIZE, each a pass of its own, over encoder, decoder and a 256 MiB copy
     counters: dict = {}
