@@ -741,20 +741,23 @@ def test_flash_attn_f32_mode_emits_the_activation_image(pkg, oracle, gpu):
 
 
 def test_flash_attn_strided_views_like_whisper(pkg, oracle, gpu):
-    # Q is the permuted view of a [d, N] projection; K / V are slices of a 1-d cache with row pitch d (src/whisper.cpp:2149-2172)
-    H, N, KV, D = 4, 20, 96, 64
-    d = H * D
-    qcur, kc, vc = rnd((N, d)), rnd((KV, d)), rnd((KV, d))
-    d_q, d_k, d_v = gpu.up(qcur), gpu.up(oracle.f32_to_f16_bits(kc)), gpu.up(oracle.f32_to_f16_bits(vc))
-    d_o = torch.empty((N, H, D), dtype=torch.float32, device=gpu.dev)
-    tq = pkg.tensor(d_q, pkg.F32, ne=[D, N, H], nb=[4, d * 4, D * 4, d * 4 * N])
-    tk = pkg.tensor(d_k, pkg.F16, ne=[D, KV, H], nb=[2, d * 2, D * 2, d * 2 * KV])
-    tv = pkg.tensor(d_v, pkg.F16, ne=[D, KV, H], nb=[2, d * 2, D * 2, d * 2 * KV])
-    pkg.check(pkg.kernels().mi355x_flash_attn_ext(tq, tk, tv, None, pkg.tensor(d_o, pkg.F32), 0.125, pkg.FA_F16_SEQ, None, 0, gpu.stream))
-    q = qcur.reshape(N, H, D).transpose(1, 0, 2)
-    kb = oracle.f32_to_f16_bits(kc).reshape(KV, H, D).transpose(1, 0, 2)
-    vb = oracle.f32_to_f16_bits(vc).reshape(KV, H, D).transpose(1, 0, 2)
-    assert oracle.nmse(gpu.down(d_o), oracle.flash_attn_ext(q, kb, vb, None, 0.125)) <= 1e-6
+    # Q is the permuted view of a [d, N] projection; K / V are slices of a 1-d cache with row pitch d (src/whisper.cpp:2149-2172):
+    # many queries and a decode step's few, both forms of the step, and grouped heads (two query heads to a K / V head)
+    for N, KV, mode, bound, HKV in ((20, 96, "FA_F16_SEQ", 1e-6, 4), (20, 96, "FA_F16_PK", 1e-5, 4), (5, 500, "FA_F16_SEQ", 1e-6, 4), (5, 500, "FA_F16_PK", 1e-5, 4),
+                                    (3, 333, "FA_F16_PK", 1e-5, 2), (3, 333, "FA_F16_SEQ", 1e-6, 2)):
+        H, D = 4, 64
+        d, dkv = H * D, HKV * D
+        qcur, kc, vc = rnd((N, d)), rnd((KV, dkv)), rnd((KV, dkv))
+        d_q, d_k, d_v = gpu.up(qcur), gpu.up(oracle.f32_to_f16_bits(kc)), gpu.up(oracle.f32_to_f16_bits(vc))
+        d_o = torch.empty((N, H, D), dtype=torch.float32, device=gpu.dev)
+        tq = pkg.tensor(d_q, pkg.F32, ne=[D, N, H], nb=[4, d * 4, D * 4, d * 4 * N])
+        tk = pkg.tensor(d_k, pkg.F16, ne=[D, KV, HKV], nb=[2, dkv * 2, D * 2, dkv * 2 * KV])
+        tv = pkg.tensor(d_v, pkg.F16, ne=[D, KV, HKV], nb=[2, dkv * 2, D * 2, dkv * 2 * KV])
+        pkg.check(pkg.kernels().mi355x_flash_attn_ext(tq, tk, tv, None, pkg.tensor(d_o, pkg.F32), 0.125, getattr(pkg, mode), None, 0, gpu.stream))
+        q = qcur.reshape(N, H, D).transpose(1, 0, 2)
+        kb = np.repeat(oracle.f32_to_f16_bits(kc).reshape(KV, HKV, D).transpose(1, 0, 2), H // HKV, axis=0)
+        vb = np.repeat(oracle.f32_to_f16_bits(vc).reshape(KV, HKV, D).transpose(1, 0, 2), H // HKV, axis=0)
+        assert oracle.nmse(gpu.down(d_o), oracle.flash_attn_ext(q, np.ascontiguousarray(kb), np.ascontiguousarray(vb), None, 0.125)) <= bound, (N, KV, mode, HKV)
 
 
 # ------------------------------------------------------------------------------------------------------------------
