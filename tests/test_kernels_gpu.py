@@ -264,10 +264,12 @@ def test_mul_mat_gelu_epilogue_from_the_lds_table_slice(pkg, oracle, gpu):
     assert oracle.nmse(got[:64], oracle.gelu(plain[:64])) <= 1e-7
 
 
-@pytest.mark.parametrize("k,m,n", [(256, 320, 150), (256, 5120, 1500)])
+@pytest.mark.parametrize("k,m,n", [(256, 320, 150), (256, 5120, 1500), (128, 2080, 2950)])
 def test_mul_mat_epilogue_emits_the_next_products_activation_image(pkg, oracle, gpu, k, m, n):
     # MI355X_EPI_EMIT_F16: besides dst (here with bias and GELU, the FFN's first matrix), its rows rounded to Q8_0 as f16(q * d).
-    # The second case has the large-v3 FFN's width and rows: the 128 x 128 tiles whose operands go straight into LDS.
+    # The second case has the large-v3 FFN's width and rows: the 128 x 128 tiles whose operands go straight into LDS, and whose
+    # patches this epilogue forms transposed (a lane owns half a Q8_0 block); the third ends in tiles that dst covers in part
+    # along both axes (32 of 128 columns, 6 of 128 rows).
     lib = pkg.kernels()
     blocks = oracle.quantize(pkg.Q5_0, rnd((m, k), 0.05))
     x, bias = rnd((n, k)), rnd((m,), 0.5)
@@ -296,7 +298,18 @@ def test_mul_mat_epilogue_emits_the_next_products_activation_image(pkg, oracle, 
     assert np.array_equal(gpu.down(d_h2, np.uint16), gpu.down(d_h, np.uint16))
     epi.flags = pkg.EPI_BIAS | pkg.EPI_IMAGE_ONLY
     assert lib.mi355x_mul_mat(tw, tx, ty, C.byref(epi), ws.data_ptr(), need, gpu.stream) == -2
-    epi.flags, epi.image = pkg.EPI_BIAS | pkg.EPI_GELU | pkg.EPI_EMIT_F16, d_h.data_ptr()
+    # the epilogue's other terms in the same launch: scale and residual, no GELU (and dst as f16 is not an option with the image)
+    res = rnd((n, m))
+    d_r = gpu.up(res)
+    epi.flags, epi.scale, epi.residual, epi.image = pkg.EPI_BIAS | pkg.EPI_SCALE | pkg.EPI_RESIDUAL | pkg.EPI_EMIT_F16, 0.75, d_r.data_ptr(), d_h2.data_ptr()
+    pkg.check(lib.mi355x_mul_mat(tw, tx, ty, C.byref(epi), ws.data_ptr(), need, gpu.stream))
+    y = gpu.down(d_y)
+    assert oracle.nmse(y, (oracle.mul_mat(pkg.Q5_0, blocks, x) + bias) * np.float32(0.75) + res) <= 1e-5
+    image = oracle.dequantize(oracle.Q8_0, oracle.quantize(oracle.Q8_0, y, act=True), m).reshape(n, m)
+    assert np.array_equal(gpu.down(d_h2, np.uint16), oracle.f32_to_f16_bits(image))
+    epi.flags |= pkg.EPI_OUT_F16
+    assert lib.mi355x_mul_mat(tw, tx, ty, C.byref(epi), ws.data_ptr(), need, gpu.stream) == -2
+    epi.flags, epi.scale, epi.residual, epi.image = pkg.EPI_BIAS | pkg.EPI_GELU | pkg.EPI_EMIT_F16, 1.0, None, d_h.data_ptr()
     # the GEMV path has no such epilogue
     d_x5 = gpu.up(x[:5])
     d_y5 = torch.zeros((5, m), dtype=torch.float32, device=gpu.dev)

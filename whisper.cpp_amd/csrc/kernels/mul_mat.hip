@@ -160,6 +160,100 @@ __device__ __forceinline__ void patch_epilogue(float16_t v, const epi_args & e, 
 }
 
 
+// The same for a patch formed the other way round (the weights as the matrix instruction's A operand): the lane owns ONE dst row
+// n and 16 of the 32 consecutive m of a patch row — m = mb + 8 q + t, q = e / 4, t = e % 4, with mb = the patch's first m +
+// 4 (lane / 32) — and lane + 32 owns the other 16.  That is half a Q8_0 block per lane: the block maximum is 8 three-operand
+// maxima and one exchange with lane + 32 instead of five cross-lane steps for each of 16 registers, both divisions are the
+// lane's own (no permutes hand them round), bias, residual and stores move four consecutive values at a time.
+// M a multiple of 32 (a patch lies inside dst's columns or outside); FULL: the patch is inside and n < N.
+template <bool FULL>
+__device__ __forceinline__ void patch_epilogue_t(float16_t v, const epi_args & e, char * db, int64_t batch_off, int64_t d_nb1,
+                                                 int64_t mb, int64_t M, int64_t n, int64_t N, const uint16_t * gelu_lds) {
+    const bool    ok = FULL || (n < N && mb < M);
+    const int64_t nc = FULL || n < N ? n : N - 1;
+    const int64_t mc = FULL || mb < M ? mb : M - 32 + (mb & 31);
+    if (e.flags & MI355X_EPI_BIAS) {
+        float4 b[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) b[q] = *(const float4 *)(e.bias + mc + 8 * q);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) { v[4 * q] += b[q].x; v[4 * q + 1] += b[q].y; v[4 * q + 2] += b[q].z; v[4 * q + 3] += b[q].w; }
+    }
+    if (e.flags & MI355X_EPI_BIAS_COL) {
+        const float b = e.bias[nc];
+#pragma unroll
+        for (int i = 0; i < 16; ++i) v[i] += b;
+    }
+    if (e.flags & MI355X_EPI_GELU) {
+        if (gelu_lds) {
+            // the table slice in LDS holds |x| < 8: the f16 patterns below 0x4800 (infinity and NaN lie above); one integer
+            // maximum over the patterns decides for the wavefront, the general form is the one of patch_epilogue
+            uint32_t hb[16], top = 0;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) { hb[i] = f2h_bits(v[i]); top = max(top, hb[i] & 0x7FFFu); }
+            if (!__any(top >= GELU_LDS_HALF)) {
+#pragma unroll
+                for (int i = 0; i < 16; ++i) v[i] = h2f(gelu_lds[(hb[i] & 0x7FFFu) + (hb[i] >> 15) * GELU_LDS_HALF]);
+            } else {
+                uint16_t t[16];
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    const uint32_t a = hb[i] & 0x7FFFu;
+                    t[i] = gelu_lds[(a < GELU_LDS_HALF ? a : 0u) + (hb[i] >> 15) * GELU_LDS_HALF];
+                }
+#pragma unroll
+                for (int i = 0; i < 16; ++i) if ((hb[i] & 0x7FFFu) >= GELU_LDS_HALF) t[i] = e.gelu[hb[i]];
+#pragma unroll
+                for (int i = 0; i < 16; ++i) v[i] = v[i] <= -10.0f ? 0.0f : v[i] >= 10.0f ? v[i] : h2f(t[i]);
+            }
+        } else {
+            uint16_t t[16];
+#pragma unroll
+            for (int i = 0; i < 16; ++i) t[i] = e.gelu[f2h_bits(v[i])];
+#pragma unroll
+            for (int i = 0; i < 16; ++i) v[i] = v[i] <= -10.0f ? 0.0f : v[i] >= 10.0f ? v[i] : h2f(t[i]);
+        }
+    }
+    if (e.flags & MI355X_EPI_SCALE) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) v[i] *= e.scale;
+    }
+    if (e.flags & MI355X_EPI_RESIDUAL) {
+        float4 r[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) r[q] = *(const float4 *)(e.residual + batch_off + nc * d_nb1 + (mc + 8 * q) * 4);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) { v[4 * q] += r[q].x; v[4 * q + 1] += r[q].y; v[4 * q + 2] += r[q].z; v[4 * q + 3] += r[q].w; }
+    }
+    if (e.flags & MI355X_EPI_OUT_F16) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+            if (ok) *(half4_t *)(db + n * d_nb1 + (mb + 8 * q) * 2) = (half4_t){ (half_t) v[4 * q], (half_t) v[4 * q + 1], (half_t) v[4 * q + 2], (half_t) v[4 * q + 3] };
+    } else if (!(e.flags & MI355X_EPI_IMAGE_ONLY)) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+            if (ok) *(float4 *)(db + n * d_nb1 + (mb + 8 * q) * 4) = make_float4(v[4 * q], v[4 * q + 1], v[4 * q + 2], v[4 * q + 3]);
+    }
+    // the image: rounded to Q8_0 as the product that reads dst next rounds its rows (see patch_epilogue)
+    float amax = fmaxf(fabsf(v[0]), fabsf(v[1]));
+#pragma unroll
+    for (int i = 2; i < 16; ++i) amax = fmaxf(amax, fabsf(v[i]));
+    {   // ... and the half of the block that lane ^ 32 holds (v_permlane32_swap of the value with itself: own half, other half)
+        const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(amax), __float_as_uint(amax), false, false);
+        amax = fmaxf(__uint_as_float(sw[0]), __uint_as_float(sw[1]));
+    }
+    const float id = amax != 0.0f ? 127.0f / amax : 0.0f;
+    const float dq = h2f(f2h_bits(div127(amax)));
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        // (the addend +0 of the multiply-add turns a product -0 into the +0 that an integer quant of zero gives)
+        const half4_t h = { (half_t) __builtin_fmaf(rintf(v[4 * q] * id), dq, 0.0f), (half_t) __builtin_fmaf(rintf(v[4 * q + 1] * id), dq, 0.0f),
+                            (half_t) __builtin_fmaf(rintf(v[4 * q + 2] * id), dq, 0.0f), (half_t) __builtin_fmaf(rintf(v[4 * q + 3] * id), dq, 0.0f) };
+        if (ok) *(half4_t *)(e.image + n * M + mb + 8 * q) = h;
+    }
+}
+
+
 // ------------------------------------------------------------------------------------------------------
 // block -> 32 f16 weights
 // ------------------------------------------------------------------------------------------------------
@@ -298,8 +392,9 @@ __global__ void k_x_to_f16(const char * __restrict__ x, half_t * __restrict__ ou
 
 // What follows the K loop of a tile: GELU reads its table from LDS when the operand buffers, free now (the loop's last barrier
 // is behind every wavefront), are large enough to hold the part that matters (TABLE_FITS); then the 32x32 patches.
-// (NT: threads of the workgroup; the patches belong to the first 256)
-template <int TI, int TJ, bool EMIT, bool TABLE_FITS, int NT = 256>
+// (NT: threads of the workgroup; the patches belong to the first 256.  TR: the patches were formed with the weights as the
+// matrix instruction's A operand — lanes own dst rows, registers own columns — which the image-emitting epilogue prefers)
+template <int TI, int TJ, bool EMIT, bool TABLE_FITS, int NT = 256, bool TR = false>
 __device__ __forceinline__ void gemm_tile_epilogue(float16_t (&acc)[TI][TJ], const mm_args & a, const epi_args & epi, char * db, int64_t batch_off, int64_t d_nb1,
                                                    int64_t n0, int64_t m0, int wn, int wmo, char * smem) {
     const int tid = threadIdx.x, lane = tid & 63, l32 = lane & 31, g = lane >> 5;
@@ -315,6 +410,19 @@ __device__ __forceinline__ void gemm_tile_epilogue(float16_t (&acc)[TI][TJ], con
         }
     }
     if (NT > 256 && tid >= 256) return;
+    if constexpr (TR) {
+        static_assert(EMIT, "the transposed patches are the image-emitting kernel's");
+        // accumulator register e of a 32x32 patch: column (= n) lane%32, row (= m) 8*(e/4) + 4*g + e%4
+        auto patches_t = [&](auto full) __attribute__((always_inline)) {
+#pragma unroll
+            for (int i = 0; i < TI; ++i)
+#pragma unroll
+                for (int j = 0; j < TJ; ++j)
+                    patch_epilogue_t<decltype(full)::value>(acc[i][j], epi, db, batch_off, d_nb1, m0 + wmo + 32 * j + 4 * g, a.M, n0 + wn + 32 * i + l32, a.N, gelu_lds);
+        };
+        if (n0 + 64 * TI <= a.N && m0 + 64 * TJ <= a.M) patches_t(std::true_type{}); else patches_t(std::false_type{});
+        return;
+    }
     // accumulator register e of a 32x32 patch: row (= n) 8*(e/4) + 4*g + e%4, column (= m) lane%32
     auto patches = [&](auto full) __attribute__((always_inline)) {
 #pragma unroll
@@ -690,7 +798,9 @@ __device__ __forceinline__ void gemm_f16_tile_dl(const mm_args & a, int tiles_m,
             for (int i = 0; i < TI; ++i)
 #pragma unroll
                 for (int j = 0; j < TJ; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(av[kk][i], bv[kk][j], acc[i][j], 0, 0, 0);
+                    // (EMIT: the patch transposed — rows are m, columns n — for the epilogue that writes the Q8_0-rounded image)
+                    acc[i][j] = EMIT ? __builtin_amdgcn_mfma_f32_32x32x16_f16(bv[kk][j], av[kk][i], acc[i][j], 0, 0, 0)
+                                     : __builtin_amdgcn_mfma_f32_32x32x16_f16(av[kk][i], bv[kk][j], acc[i][j], 0, 0, 0);
         __builtin_amdgcn_sched_group_barrier(0x100, (GB_K / 16) * (TI + TJ), 0);     // the DS reads
         __builtin_amdgcn_sched_group_barrier(0x008, (GB_K / 16) * TI * TJ, 0);       // the MFMAs
     };
@@ -710,7 +820,7 @@ __device__ __forceinline__ void gemm_f16_tile_dl(const mm_args & a, int tiles_m,
     }
     wait_vmcnt<0>();                                    // the surplus loads still write LDS, which the epilogue reuses
     __syncthreads();
-    gemm_tile_epilogue<TI, TJ, EMIT, true>(acc, a, epi, db, batch_off, d_nb1, n0, m0, wn, wmo, smem);
+    gemm_tile_epilogue<TI, TJ, EMIT, true, 256, EMIT>(acc, a, epi, db, batch_off, d_nb1, n0, m0, wn, wmo, smem);
 }
 
 // Workgroups are dealt round-robin to the 8 XCDs, each with its own L2: workgroup `lin` of `total` runs on XCD lin % 8.
