@@ -1279,6 +1279,53 @@ __global__ void __launch_bounds__(512, 2) k_fattn_seq_tile(fa_args a) {
 
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
+// The factor step of a run of 16 scores, written out: s[i] becomes its factor (negated where key i raises the row's maximum),
+// M the running maximum, (P, A) the run's part of the denominator (S_after = S_before * P + A), bit i of `bits` the raise.
+// The common key raises no maximum in the whole wavefront (85 % of the keys of the encoder's launches) and takes the
+// straight path — test, difference, exponential, sum and a branch not taken; a raise anywhere in the wavefront sends it
+// through the general form at the end of the block and back.  As C++ the same loop met after every key in a join
+// for which the compiler copied three to five registers, on the straight path too: nine vector instructions and two taken
+// branches per key.  (The s_nop behind v_exp_f32 is the wait state its result needs in front of a vector instruction.)
+// The factor is 2^-|s - M|: 2^(s - M), or 2^(M - s) where s raises the maximum.  M starts at PKT_M_START, a finite number
+// below every score, so that the difference is never (-inf) - (-inf): a masked key (s = -inf) gives -inf and the factor 0
+// whatever was seen before it, the first real key of a row raises the maximum with the factor 2^-huge = 0, as with -inf.
+#define PKT_M_START (-3.0e38f)
+#define PKT_KEY(i) \
+    "v_cmp_gt_f32 vcc, %[s" #i "], %[M]\n" \
+    "v_sub_f32 %[t], %[s" #i "], %[M]\n" \
+    "s_cbranch_vccnz 1" #i "f\n" \
+    "v_exp_f32_e64 %[s" #i "], -|%[t]|\n" \
+    "s_nop 0\n" \
+    "v_add_f32 %[A], %[A], %[s" #i "]\n" \
+    "2" #i ":\n"
+#define PKT_RAISE(i) \
+    "1" #i ":\n" \
+    "v_max_f32 %[M], %[M], %[s" #i "]\n" \
+    "v_exp_f32_e64 %[ex], -|%[t]|\n" \
+    "s_nop 0\n" \
+    "v_cndmask_b32_e64 %[ms], 1.0, %[ex], vcc\n" \
+    "v_cndmask_b32_e64 %[vs], %[ex], 1.0, vcc\n" \
+    "v_mul_f32 %[P], %[P], %[ms]\n" \
+    "v_fma_f32 %[A], %[A], %[ms], %[vs]\n" \
+    "v_cndmask_b32_e64 %[s" #i "], %[ex], -%[ex], vcc\n" \
+    "v_cndmask_b32_e64 %[ms], 0, 1, vcc\n" \
+    "v_lshl_or_b32 %[bits], %[ms], " #i ", %[bits]\n" \
+    "s_branch 2" #i "b\n"
+__device__ __forceinline__ void pkt_factor_run(float (&sv)[16], float & M, float & P, float & A, uint32_t & bits) {
+    float t, ex, ms, vs;
+    asm volatile(
+        PKT_KEY(0) PKT_KEY(1) PKT_KEY(2) PKT_KEY(3) PKT_KEY(4) PKT_KEY(5) PKT_KEY(6) PKT_KEY(7)
+        PKT_KEY(8) PKT_KEY(9) PKT_KEY(10) PKT_KEY(11) PKT_KEY(12) PKT_KEY(13) PKT_KEY(14) PKT_KEY(15)
+        "s_branch 3f\n"
+        PKT_RAISE(0) PKT_RAISE(1) PKT_RAISE(2) PKT_RAISE(3) PKT_RAISE(4) PKT_RAISE(5) PKT_RAISE(6) PKT_RAISE(7)
+        PKT_RAISE(8) PKT_RAISE(9) PKT_RAISE(10) PKT_RAISE(11) PKT_RAISE(12) PKT_RAISE(13) PKT_RAISE(14) PKT_RAISE(15)
+        "3:\n"
+        : [s0] "+v"(sv[0]), [s1] "+v"(sv[1]), [s2] "+v"(sv[2]), [s3] "+v"(sv[3]), [s4] "+v"(sv[4]), [s5] "+v"(sv[5]), [s6] "+v"(sv[6]), [s7] "+v"(sv[7]),
+          [s8] "+v"(sv[8]), [s9] "+v"(sv[9]), [s10] "+v"(sv[10]), [s11] "+v"(sv[11]), [s12] "+v"(sv[12]), [s13] "+v"(sv[13]), [s14] "+v"(sv[14]), [s15] "+v"(sv[15]),
+          [M] "+v"(M), [P] "+v"(P), [A] "+v"(A), [bits] "+v"(bits), [t] "=&v"(t), [ex] "=&v"(ex), [ms] "=&v"(ms), [vs] "=&v"(vs)
+        : : "vcc");
+}
+
 __global__ void __launch_bounds__(512, 2) k_fattn_pk_tile(fa_args a) {
     extern __shared__ __attribute__((aligned(16))) char t_smem[];
     half_t *   q_s  = (half_t *) t_smem;                      // [T_Q * T_LDH]
@@ -1315,7 +1362,7 @@ __global__ void __launch_bounds__(512, 2) k_fattn_pk_tile(fa_args a) {
                 *(half4_t *)(q_s + r * T_LDH + c + 4 * i) = hq;
             }
         }
-        if (tid < T_Q) { m_run[tid] = -INFINITY; s_run[tid] = 0.0f; }
+        if (tid < T_Q) { m_run[tid] = PKT_M_START; s_run[tid] = 0.0f; }
 
         const int sq = (pw >> 1) * 32, sk = (pw & 1) * 32, l32 = lane & 31, g = lane >> 5;
         const int kr = tid >> 2, kc = (tid & 3) * 16;
@@ -1393,24 +1440,8 @@ __global__ void __launch_bounds__(512, 2) k_fattn_pk_tile(fa_args a) {
                 if (sgm > 2) M = fmaxf(M, m2);
                 float P = 1.0f, A = 0.0f;
                 uint32_t rbits = 0;                        // bit i: key i of this run raises this query's maximum
-#pragma unroll
-                for (int i = 0; i < 16; ++i) {
-                    const float s = sv[i];
-                    const bool  raised = s > M;
-                    // 2^(M - s) when raised, 2^(s - M) otherwise: the exponent is <= 0, -inf for the first key of a row (0), and
-                    // NaN for a masked key in front of every other (-inf - -inf), which the maximum with 0 turns into 0
-                    const float ex = fmaxf(__builtin_amdgcn_exp2f(-fabsf(s - M)), 0.0f);
-                    if (__any(raised)) {
-                        const float ms = raised ? ex : 1.0f, vs = raised ? 1.0f : ex;
-                        M = raised ? s : M;
-                        P *= ms; A = A * ms + vs;
-                        sv[i] = raised ? -ex : ex;             // -0.0 keeps the sign
-                        rbits |= raised ? 1u << i : 0u;
-                    } else {
-                        A = A + ex;
-                        sv[i] = ex;
-                    }
-                }
+                // sv[i] -> 2^(s - M), or -2^(M - s) where key i raises the maximum (-0.0 keeps the sign)
+                pkt_factor_run(sv, M, P, A, rbits);
                 // f16 factors, two keys to a register, into column (query ^ swizzle) of this run's eight key-pair rows
                 uint32_t * fpw = fp_s + (it & 1) * P_FP_TILE + (8 * sgm) * P_FP_ROW + (qi ^ ((sgm & 1) << 4));
 #pragma unroll
