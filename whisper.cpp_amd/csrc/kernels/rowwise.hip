@@ -15,7 +15,10 @@
 // dense [nrows][ne0] — so that the products that follow need no conversion pass of their own.
 // EMIT == 2: the row quantized to Q8_0 itself, in the layout the few-column product reads its activations from
 // (int8 q[nrows][ne0] | float d[nrows][ne0/32] | int32 sum of a block's quants).
-template <int NV, int EMIT>
+// FULL: the row fills every lane's NV float4s (ne0 = 256 NV) and both affine vectors are there — whisper's LayerNorms over 256,
+// 512, ... 1280 values: no guard around any load, reduction term or store (34 exec-mask branches less in a kernel whose time
+// is its chain of dependent instructions)
+template <int NV, int EMIT, bool FULL = false>
 __global__ void __launch_bounds__(ROWS_PER_BLOCK * WAVE) k_norm(tview s, tview d, int64_t nrows, float eps, const float * __restrict__ w, const float * __restrict__ b, half_t * __restrict__ x16) {
     const int     lane = threadIdx.x % WAVE;
     const int64_t row  = (int64_t) blockIdx.x * ROWS_PER_BLOCK + threadIdx.x / WAVE;
@@ -33,20 +36,20 @@ __global__ void __launch_bounds__(ROWS_PER_BLOCK * WAVE) k_norm(tview s, tview d
         for (int j = 0; j < NV; ++j) {
             const int c = lane + j * WAVE;
             ww[j] = make_float4(1.f, 1.f, 1.f, 1.f); bb[j] = make_float4(0.f, 0.f, 0.f, 0.f);
-            if (c < n4) { if (w) ww[j] = ((const float4 *) w)[c]; if (b) bb[j] = ((const float4 *) b)[c]; }
+            if (FULL || c < n4) { if (FULL || w) ww[j] = ((const float4 *) w)[c]; if (FULL || b) bb[j] = ((const float4 *) b)[c]; }
         }
         float sum = 0.0f;
 #pragma unroll
         for (int j = 0; j < NV; ++j) {
             const int c = lane + j * WAVE;
-            if (c < n4) { v[j] = ((const float4 *) x)[c]; sum += (v[j].x + v[j].y) + (v[j].z + v[j].w); }
+            if (FULL || c < n4) { v[j] = ((const float4 *) x)[c]; sum += (v[j].x + v[j].y) + (v[j].z + v[j].w); }
         }
         const float mean = wave_sum(sum) / (float) ne0;
         float sum2 = 0.0f;
 #pragma unroll
         for (int j = 0; j < NV; ++j) {
             const int c = lane + j * WAVE;
-            if (c < n4) {
+            if (FULL || c < n4) {
                 v[j].x -= mean; v[j].y -= mean; v[j].z -= mean; v[j].w -= mean;
                 sum2 += (v[j].x*v[j].x + v[j].y*v[j].y) + (v[j].z*v[j].z + v[j].w*v[j].w);
             }
@@ -55,10 +58,15 @@ __global__ void __launch_bounds__(ROWS_PER_BLOCK * WAVE) k_norm(tview s, tview d
 #pragma unroll
         for (int j = 0; j < NV; ++j) {
             const int c = lane + j * WAVE;
-            if (c < n4) {
+            if (FULL || c < n4) {
                 float4 r = { v[j].x * scale, v[j].y * scale, v[j].z * scale, v[j].w * scale };
-                if (w) { r.x *= ww[j].x; r.y *= ww[j].y; r.z *= ww[j].z; r.w *= ww[j].w; }
-                if (b) { r.x += bb[j].x; r.y += bb[j].y; r.z += bb[j].z; r.w += bb[j].w; }
+                // (the affine is two graph nodes, MUL then ADD: two roundings, never one fused multiply-add — without the guards
+                // around them the two would be contracted)
+                {
+#pragma clang fp contract(off)
+                    if (FULL || w) { r.x *= ww[j].x; r.y *= ww[j].y; r.z *= ww[j].z; r.w *= ww[j].w; }
+                    if (FULL || b) { r.x += bb[j].x; r.y += bb[j].y; r.z += bb[j].z; r.w += bb[j].w; }
+                }
                 if (EMIT != 1 || d.p) ((float4 *) y)[c] = r;     // (EMIT == 1 without a destination: the image is all the caller wants)
                 if (EMIT) {                                // a 32-value block = 8 consecutive lanes (ne0 % 32 == 0: they are all here)
                     float amax = fmaxf(fmaxf(fabsf(r.x), fabsf(r.y)), fmaxf(fabsf(r.z), fabsf(r.w)));
@@ -138,11 +146,18 @@ static int norm_impl(const mi355x_tensor * src, const mi355x_tensor * dst, float
     if (x16 && (!in_regs || src->ne[0] % QK != 0)) return MI355X_ERR_UNSUPPORTED;      // only that form emits, and only whole blocks
     const tview vs = make_view(src), vd = make_view(dst);
     const unsigned g = (unsigned) grid, t = ROWS_PER_BLOCK * WAVE;
+    const bool full = nv > 0 && src->ne[0] == (int64_t) 4 * WAVE * nv && w && b;
 #define NORM_LAUNCH(NV) \
     do { \
-        if (!x16)           k_norm<NV, 0><<<g, t, 0, st>>>(vs, vd, nrows, eps, w, b, nullptr); \
-        else if (emit == 2) k_norm<NV, 2><<<g, t, 0, st>>>(vs, vd, nrows, eps, w, b, (half_t *) x16); \
-        else                k_norm<NV, 1><<<g, t, 0, st>>>(vs, vd, nrows, eps, w, b, (half_t *) x16); \
+        if (full) { \
+            if (!x16)           k_norm<NV, 0, true><<<g, t, 0, st>>>(vs, vd, nrows, eps, w, b, nullptr); \
+            else if (emit == 2) k_norm<NV, 2, true><<<g, t, 0, st>>>(vs, vd, nrows, eps, w, b, (half_t *) x16); \
+            else                k_norm<NV, 1, true><<<g, t, 0, st>>>(vs, vd, nrows, eps, w, b, (half_t *) x16); \
+        } else { \
+            if (!x16)           k_norm<NV, 0><<<g, t, 0, st>>>(vs, vd, nrows, eps, w, b, nullptr); \
+            else if (emit == 2) k_norm<NV, 2><<<g, t, 0, st>>>(vs, vd, nrows, eps, w, b, (half_t *) x16); \
+            else                k_norm<NV, 1><<<g, t, 0, st>>>(vs, vd, nrows, eps, w, b, (half_t *) x16); \
+        } \
     } while (0)
     switch (nv) {
         case 0:  k_norm<0, 0><<<g, t, 0, st>>>(vs, vd, nrows, eps, w, b, nullptr); break;

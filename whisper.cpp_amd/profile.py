@@ -37,7 +37,7 @@ DEC_CMD = [str(HARNESS), "bench", "--model", DEC_MODEL, "--what", "decoder", "--
 BENCH_NAMES = [
     ("k_fattn_pk_tile", "flash_attn.seq_tile_pk", "encoder"), ("k_fattn_seq_tile", "flash_attn.seq_tile", "encoder"),
     ("void k_gemm_f16_dl_group", "mul_mat.gemm_group", "encoder"), ("void k_gemm_f16_dl<", "mul_mat.gemm_q5_0", "encoder"),
-    ("void k_gemm_f16_rs<", "mul_mat.gemm_q5_0", "encoder"), ("void k_norm<5, 1>", "norm_affine_emit", "encoder"), ("_Z6k_normILi5ELi1EE", "norm_affine_emit", "encoder"),
+    ("void k_gemm_f16_rs<", "mul_mat.gemm_q5_0", "encoder"), ("void k_norm<5, 1", "norm_affine_emit", "encoder"), ("_Z6k_normILi5ELi1E", "norm_affine_emit", "encoder"),
     ("k_fattn_pk_row", "flash_attn.seq_row_pk", "decoder"), ("k_fattn_seq_row", "flash_attn.seq_row", "decoder"), ("void k_gemv_q8_0_tiles<20", "mul_mat.gemv_q8_0.vocab", "decoder"),
 ]
 
@@ -161,7 +161,7 @@ def main() -> int:
             d = out / f"sq_{i}"
             run(["rocprofv3", "--pmc", *ctrs.split(), "--output-format", "csv", "-d", str(d), "--", *ENC_CMD, "--reps", "1", "--warmup", "0"], out / f"sq_{i}.log", 120)
             for k, v in per_kernel(d).items():
-                if k.startswith(("k_fattn", "void k_gemm_f16", "void k_norm<5, 1>", "_Z6k_normILi5ELi1EE")):
+                if k.startswith(("k_fattn", "void k_gemm_f16", "void k_norm<5, 1", "_Z6k_normILi5ELi1E")):
                     for c, (n, s) in v.items():
                         sq[k[:80]][c] = round(s / n)
             shutil.rmtree(d, ignore_errors=True)
