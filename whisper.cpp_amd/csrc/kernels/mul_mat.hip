@@ -1506,22 +1506,25 @@ struct gemv_norm_args {
     char * ws;                         // their Q8_0 form (layout of k_quantize_x_q8)
 };
 
-template <int NC>
+// NJ > 0: the rows are exactly 256 NJ values long and both affine vectors are there (whisper's LayerNorms at 512 ... 1280):
+// NJ float4s per lane instead of eight, no guard around a term, no clamped address
+template <int NC, int NJ = 0>
 struct gemv_norm_prologue {
     const gemv_norm_args & nm; int64_t K; char * lds;
     // wavefront w takes rows w and w + 4; both rows and the affine vectors are requested before anything is reduced, so
     // the prologue is one memory round trip long
     static constexpr int RW = (NC + 3) / 4;                 // rows per wavefront
-    float4 v[RW][8], ww[8], bb[8];
+    static constexpr int JN = NJ ? NJ : 8;                  // float4s per lane and row
+    float4 v[RW][JN], ww[JN], bb[JN];
 
     __device__ __forceinline__ void request() {
         const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
         const int n4 = (int)(K / 4);
         // no branch around a load: addresses are clamped into the rows, and a missing affine vector reads the source instead
-        const float4 * wp = (const float4 *)(nm.w ? (const char *) nm.w : nm.src), * bp = (const float4 *)(nm.b ? (const char *) nm.b : nm.src);
+        const float4 * wp = (const float4 *)(NJ || nm.w ? (const char *) nm.w : nm.src), * bp = (const float4 *)(NJ || nm.b ? (const char *) nm.b : nm.src);
 #pragma unroll
-        for (int jj = 0; jj < 8; ++jj) {
-            const int c = lane + jj * WAVE < n4 ? lane + jj * WAVE : n4 - 1;
+        for (int jj = 0; jj < JN; ++jj) {
+            const int c = NJ || lane + jj * WAVE < n4 ? lane + jj * WAVE : n4 - 1;
             ww[jj] = wp[c]; bb[jj] = bp[c];
 #pragma unroll
             for (int rr = 0; rr < RW; ++rr) {
@@ -1544,12 +1547,12 @@ struct gemv_norm_prologue {
             if (row >= NC) break;                           // uniform
             float sum = 0.0f;
 #pragma unroll
-            for (int jj = 0; jj < 8; ++jj) if (lane + jj * WAVE < n4) sum += (v[rr][jj].x + v[rr][jj].y) + (v[rr][jj].z + v[rr][jj].w);
+            for (int jj = 0; jj < JN; ++jj) if (NJ || lane + jj * WAVE < n4) sum += (v[rr][jj].x + v[rr][jj].y) + (v[rr][jj].z + v[rr][jj].w);
             const float mean = wave_sum(sum) / (float) K;
             float sum2 = 0.0f;
 #pragma unroll
-            for (int jj = 0; jj < 8; ++jj) {
-                if (lane + jj * WAVE < n4) {
+            for (int jj = 0; jj < JN; ++jj) {
+                if (NJ || lane + jj * WAVE < n4) {
                     float4 & t = v[rr][jj];
                     t.x -= mean; t.y -= mean; t.z -= mean; t.w -= mean;
                     sum2 += (t.x*t.x + t.y*t.y) + (t.z*t.z + t.w*t.w);
@@ -1557,12 +1560,15 @@ struct gemv_norm_prologue {
             }
             const float scale = 1.0f / sqrtf(wave_sum(sum2) / (float) K + nm.eps);
 #pragma unroll
-            for (int jj = 0; jj < 8; ++jj) {
+            for (int jj = 0; jj < JN; ++jj) {
                 const int c = lane + jj * WAVE;
-                if (c < n4) {                               // whole 8-lane groups: K is a multiple of 32
+                if (NJ || c < n4) {                         // whole 8-lane groups: K is a multiple of 32
                     float4 r = { v[rr][jj].x * scale, v[rr][jj].y * scale, v[rr][jj].z * scale, v[rr][jj].w * scale };
-                    if (nm.w) { r.x *= ww[jj].x; r.y *= ww[jj].y; r.z *= ww[jj].z; r.w *= ww[jj].w; }
-                    if (nm.b) { r.x += bb[jj].x; r.y += bb[jj].y; r.z += bb[jj].z; r.w += bb[jj].w; }
+                    {   // (MUL then ADD, two graph nodes: two roundings — without guards around them the two would be contracted)
+#pragma clang fp contract(off)
+                        if (NJ || nm.w) { r.x *= ww[jj].x; r.y *= ww[jj].y; r.z *= ww[jj].z; r.w *= ww[jj].w; }
+                        if (NJ || nm.b) { r.x += bb[jj].x; r.y += bb[jj].y; r.z += bb[jj].z; r.w += bb[jj].w; }
+                    }
                     if (writer) ((float4 *)(nm.dst + row * nm.dst_nb1))[c] = r;
                     const float amax = lanes_max<8>(fmaxf(fmaxf(fabsf(r.x), fabsf(r.y)), fmaxf(fabsf(r.z), fabsf(r.w))));
                     const float id = amax != 0.0f ? 127.0f / amax : 0.0f;
@@ -1582,13 +1588,13 @@ struct gemv_norm_prologue {
     }
 };
 
-template <int T0, int NC, int LPR, int NB>
+template <int T0, int NC, int LPR, int NB, int NJ = 0>
 __global__ void __launch_bounds__(256) k_gemv_qr_norm_group(mm_args a, gemv_group grp, gemv_norm_args nm) {
     extern __shared__ __attribute__((aligned(16))) char smem[];
     const gemv_group_entry & ge = grp.e[blockIdx.y];
     a.w = ge.w; a.d = ge.d; a.d_nb1 = ge.d_nb1;
     a.e.flags = ge.flags; a.e.scale = ge.scale; a.e.bias = ge.bias; a.e.residual = ge.residual;
-    gemv_qr_rows<T0, NC, LPR, NB>(a, gemv_norm_prologue<NC>{ nm, a.K, smem });
+    gemv_qr_rows<T0, NC, LPR, NB>(a, gemv_norm_prologue<NC, NJ>{ nm, a.K, smem });
 }
 
 // ------------------------------------------------------------------------------------------------------
@@ -1682,7 +1688,9 @@ template <int T0, int NC, int LPR, int NB>
 static int launch_gemv_r_k(const mm_args & a, unsigned grid, const gemv_group * grp, int count, const gemv_norm_args * nm, hipStream_t st) {
     if (nm) {
         const size_t lds = (size_t) NC * a.K + (size_t) NC * (a.K / QK) * 8;
-        k_gemv_qr_norm_group<T0, NC, LPR, NB><<<dim3(grid, (unsigned) count), 256, lds, st>>>(a, *grp, *nm);
+        // (the widest model's rows, 1280 values, have an instance without guards)
+        if (a.K == 1280 && nm->w && nm->b) k_gemv_qr_norm_group<T0, NC, LPR, NB, 5><<<dim3(grid, (unsigned) count), 256, lds, st>>>(a, *grp, *nm);
+        else                               k_gemv_qr_norm_group<T0, NC, LPR, NB><<<dim3(grid, (unsigned) count), 256, lds, st>>>(a, *grp, *nm);
     }
     else if (grp) k_gemv_qr_group<T0, NC, LPR, NB><<<dim3(grid, (unsigned) count), 256, 0, st>>>(a, *grp);
     else          k_gemv_qr<T0, NC, LPR, NB><<<grid, 256, 0, st>>>(a);
