@@ -1559,24 +1559,47 @@ struct gemv_norm_prologue {
                 }
             }
             const float scale = 1.0f / sqrtf(wave_sum(sum2) / (float) K + nm.eps);
+            // The JN pieces of the row go through each step together — normalize, block maximum, scale, round, block sum, store —
+            // and nothing between the steps branches: every piece is a chain of dependent instructions (three cross-lane steps
+            // for the maximum, a division, three more for the sum), and side by side the chains fill each other's waits.  (All
+            // eight lanes of a block store its scale and its sum: the same value to the same address, instead of a branch
+            // around one lane's store.)
+            float4 r[JN];
+            float amax[JN], id[JN];
+            int q[JN][4], qsum[JN];
+#pragma unroll
+            for (int jj = 0; jj < JN; ++jj) {
+                r[jj] = make_float4(v[rr][jj].x * scale, v[rr][jj].y * scale, v[rr][jj].z * scale, v[rr][jj].w * scale);
+                {   // (MUL then ADD, two graph nodes: two roundings — without guards around them the two would be contracted)
+#pragma clang fp contract(off)
+                    if (NJ || nm.w) { r[jj].x *= ww[jj].x; r[jj].y *= ww[jj].y; r[jj].z *= ww[jj].z; r[jj].w *= ww[jj].w; }
+                    if (NJ || nm.b) { r[jj].x += bb[jj].x; r[jj].y += bb[jj].y; r[jj].z += bb[jj].z; r[jj].w += bb[jj].w; }
+                }
+            }
+#pragma unroll
+            for (int jj = 0; jj < JN; ++jj)     // (lanes beyond the row hold the clamped last piece: their groups are whole, K % 32 == 0)
+                amax[jj] = lanes_max<8>(fmaxf(fmaxf(fabsf(r[jj].x), fabsf(r[jj].y)), fmaxf(fabsf(r[jj].z), fabsf(r[jj].w))));
+#pragma unroll
+            for (int jj = 0; jj < JN; ++jj) id[jj] = amax[jj] != 0.0f ? 127.0f / amax[jj] : 0.0f;
+#pragma unroll
+            for (int jj = 0; jj < JN; ++jj) {
+                q[jj][0] = (int) rintf(r[jj].x * id[jj]); q[jj][1] = (int) rintf(r[jj].y * id[jj]);
+                q[jj][2] = (int) rintf(r[jj].z * id[jj]); q[jj][3] = (int) rintf(r[jj].w * id[jj]);
+            }
+#pragma unroll
+            for (int jj = 0; jj < JN; ++jj) qsum[jj] = lanes_sum<8>((q[jj][0] + q[jj][1]) + (q[jj][2] + q[jj][3]));
 #pragma unroll
             for (int jj = 0; jj < JN; ++jj) {
                 const int c = lane + jj * WAVE;
-                if (NJ || c < n4) {                         // whole 8-lane groups: K is a multiple of 32
-                    float4 r = { v[rr][jj].x * scale, v[rr][jj].y * scale, v[rr][jj].z * scale, v[rr][jj].w * scale };
-                    {   // (MUL then ADD, two graph nodes: two roundings — without guards around them the two would be contracted)
-#pragma clang fp contract(off)
-                        if (NJ || nm.w) { r.x *= ww[jj].x; r.y *= ww[jj].y; r.z *= ww[jj].z; r.w *= ww[jj].w; }
-                        if (NJ || nm.b) { r.x += bb[jj].x; r.y += bb[jj].y; r.z += bb[jj].z; r.w += bb[jj].w; }
-                    }
-                    if (writer) ((float4 *)(nm.dst + row * nm.dst_nb1))[c] = r;
-                    const float amax = lanes_max<8>(fmaxf(fmaxf(fabsf(r.x), fabsf(r.y)), fmaxf(fabsf(r.z), fabsf(r.w))));
-                    const float id = amax != 0.0f ? 127.0f / amax : 0.0f;
-                    const int q0 = (int) rintf(r.x * id), q1 = (int) rintf(r.y * id), q2 = (int) rintf(r.z * id), q3 = (int) rintf(r.w * id);
-                    const int qsum = lanes_sum<8>(q0 + q1 + q2 + q3);
-                    xq[row * n4 + c] = (q0 & 0xFF) | ((q1 & 0xFF) << 8) | ((q2 & 0xFF) << 16) | ((q3 & 0xFF) << 24);
-                    if ((c & 7) == 0) { xd[row * nbk + c / 8] = h2f(f2h_bits(div127(amax))); xsum[row * nbk + c / 8] = qsum; }
+                if (NJ || c < n4) {
+                    xq[row * n4 + c] = (q[jj][0] & 0xFF) | ((q[jj][1] & 0xFF) << 8) | ((q[jj][2] & 0xFF) << 16) | ((q[jj][3] & 0xFF) << 24);
+                    xd[row * nbk + c / 8] = h2f(f2h_bits(div127(amax[jj])));
+                    xsum[row * nbk + c / 8] = qsum[jj];
                 }
+            }
+            if (writer) {
+#pragma unroll
+                for (int jj = 0; jj < JN; ++jj) if (NJ || lane + jj * WAVE < n4) ((float4 *)(nm.dst + row * nm.dst_nb1))[lane + jj * WAVE] = r[jj];
             }
         }
         __syncthreads();
