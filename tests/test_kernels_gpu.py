@@ -584,6 +584,8 @@ def test_flash_attn_reference_faithful(pkg, oracle, gpu, case):
 @pytest.mark.parametrize("case", [
     dict(H=2, N=70, KV=100), dict(H=3, N=200, KV=1536, flat=True, pad_from=1500), dict(H=2, N=100, KV=100, mask="causal"),
     dict(H=2, N=9, KV=63), dict(H=2, N=130, KV=448, mask="causal"), dict(H=2, N=64, KV=1500, flat=True),
+    # masked keys in front of a row's first real key (the running maximum starts at a finite number, not at -inf)
+    dict(H=2, N=70, KV=300, mask="late"), dict(H=2, N=5, KV=300, mask="late"),
     # at most 8 queries: the few-query kernel of the packed form (stages of 192 keys: one, one key into the second, many)
     dict(H=20, N=5, KV=1536, flat=True, pad_from=1500), dict(H=4, N=1, KV=1), dict(H=4, N=5, KV=37, mask="beam"), dict(H=2, N=3, KV=200, mask="causal"),
     dict(H=2, N=8, KV=448, mask="beam"), dict(H=2, N=1, KV=192), dict(H=2, N=4, KV=193, mask="beam"), dict(H=1, N=2, KV=7500), dict(H=3, N=5, KV=583, mask="beam")])
@@ -600,6 +602,9 @@ def test_flash_attn_packed_f16_chain(pkg, oracle, gpu, case):
         for r in range(N):
             if case["mask"] == "causal":
                 m[r, : KV - N + r + 1] = 0.0
+            elif case["mask"] == "late":       # a row's first keys are masked (a whole tile of 64 and more for some rows), and every seventh after
+                m[r, (r * 5) % 97 + 1:] = 0.0
+                m[r, (r * 5) % 97 + 3::7] = -np.inf
             else:
                 m[r, : (KV + 1) // 2] = 0.0
                 m[r, [c for c in range(KV) if c % N == r]] = 0.0
