@@ -103,6 +103,7 @@ def probes():
     lib.mi355x_probe_mfma.restype, lib.mi355x_probe_mfma.argtypes = C.c_int, [C.c_int, C.c_int, P, P]
     lib.mi355x_probe_gemv_tiles_stamped.restype = C.c_int
     lib.mi355x_probe_gemv_tiles_stamped.argtypes = [P, C.c_int64, C.c_int64, P, C.c_int64, P, P, C.POINTER(C.c_int64), C.POINTER(C.c_int64), P]
+    lib.mi355x_probe_load_path.restype, lib.mi355x_probe_load_path.argtypes = C.c_int, [P, C.c_size_t, C.c_int, C.c_int, C.c_int, P, P]
     return lib
 
 
@@ -310,6 +311,20 @@ def gemm_library_yardstick() -> list | None:
             tf = wgs * 4 * 4 * iters * 32768.0 / us / 1e6
             rows.append({"shape": f"matrix instruction from registers, {wgs // 256} wavefront(s) per SIMD", "us": round(us, 1),
                          "tflops": round(tf, 1), "frac_of_peak": round(tf / PEAK_MFMA_F16_TFLOPS, 4)})
+        # the path global memory -> CU that the operands of these products take (global_load_lds_dwordx4, and loads into registers):
+        # what a kernel that does nothing else moves, from L1, from L2 and from beyond L2 (mi355x_probe_load_path)
+        span17 = 1500 * 2560 + 5120 * 2560                 # the operands of the FFN-up product, which no L2 holds
+        src = torch.empty(span17 + (1 << 20), dtype=torch.uint8, device=dev).fill_(1)
+        wgs, iters = 512, 400
+        clocks = torch.zeros(2 * wgs + 2, dtype=torch.int64, device=dev)
+        for where, span in (("L1 (8 KB window)", 0), ("L2 (2 MB)", 2 << 20), ("beyond L2 (17 MB)", span17 - 8 * 32 * 2560 - 4096)):
+            for to_lds in (1, 0):
+                us = timed(lambda: pkg.check(pr.mi355x_probe_load_path(src.data_ptr(), span, to_lds, iters, wgs, clocks.data_ptr(), None)), reps=3)
+                c = clocks[: 2 * wgs].view(wgs, 2).double().mean(dim=0)
+                mhz = float(c[0] / c[1]) * 100.0
+                nbytes = wgs * 4 * iters * 8192.0
+                rows.append({"shape": f"load path, {'straight into LDS' if to_lds else 'into registers'}, from {where}", "us": round(us, 1),
+                             "tb_per_s": round(nbytes / us / 1e6, 2), "clock_mhz": round(mhz), "bytes_per_clock_and_cu": round(nbytes / 256 / (us * mhz), 1)})
         return rows
     except Exception as e:                                 # a yardstick: its absence must not fail the bench
         print(f"bench.py: gemm_library_yardstick skipped: {e}", file=sys.stderr)

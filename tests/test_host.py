@@ -97,7 +97,7 @@ def test_yardstick_kernels_live_in_a_library_of_their_own(pkg):
     probes = pkg.KERNELS_LIB.parent / "libmi355x_probes.so"
     if not pkg.KERNELS_LIB.exists() or not probes.exists():
         pytest.skip("libraries not built")
-    assert {"mi355x_probe_read", "mi355x_probe_read_stamped", "mi355x_probe_mfma", "mi355x_probe_gemv_tiles_stamped", "mi355x_probe_div127"} <= exported(probes)
+    assert {"mi355x_probe_read", "mi355x_probe_read_stamped", "mi355x_probe_mfma", "mi355x_probe_gemv_tiles_stamped", "mi355x_probe_div127", "mi355x_probe_load_path"} <= exported(probes)
     assert not any("probe" in name for name in exported(pkg.KERNELS_LIB)), [n for n in exported(pkg.KERNELS_LIB) if "probe" in n]
     assert "probe" not in (ROOT / "include" / "mi355x_kernels.h").read_text()
     for lib in (pkg.KERNELS_LIB, pkg.PLUGIN_LIB):

@@ -1070,6 +1070,20 @@ def test_measurement_probes_run_and_reject_bad_arguments(pkg, gpu):
     st = stamps.cpu()
     assert int(st[:n].min()) >= int(st[n:n + 16].min()) > 0        # every chunk finished after the first workgroup started
     assert lib.mi355x_probe_read_stamped(buf.data_ptr(), buf.numel(), out.data_ptr(), 16, None, gpu.stream) == -2
+    # the load path of the GEMM operands: clock ticks of every workgroup's loop come back, on both paths and from all three places
+    lib.mi355x_probe_load_path.restype, lib.mi355x_probe_load_path.argtypes = C.c_int, [P, C.c_size_t, C.c_int, C.c_int, C.c_int, P, P]
+    src = torch.ones((4 << 20) + (1 << 20), dtype=torch.uint8, device=gpu.dev)
+    for span in (0, 2 << 20, 4 << 20):
+        for to_lds in (1, 0):
+            clocks = torch.zeros(2 * 64 + 2, dtype=torch.int64, device=gpu.dev)
+            pkg.check(lib.mi355x_probe_load_path(src.data_ptr(), span, to_lds, 50, 64, clocks.data_ptr(), gpu.stream))
+            torch.cuda.synchronize()
+            c = clocks.cpu()[:128].view(64, 2)
+            assert int(c.min()) > 0 and 5 < float(c[:, 0].sum()) / float(c[:, 1].sum()) < 40      # 0.5 ... 4 GHz against the 100 MHz clock
+            assert int(clocks[128:].abs().sum()) == 0
+    assert lib.mi355x_probe_load_path(src.data_ptr(), 4096, 1, 50, 64, clocks.data_ptr(), gpu.stream) == -2
+    assert lib.mi355x_probe_load_path(None, 0, 1, 50, 64, clocks.data_ptr(), gpu.stream) == -2
+    assert lib.mi355x_probe_load_path(src.data_ptr(), 0, 1, 0, 64, clocks.data_ptr(), gpu.stream) == -2
 
 
 def test_the_three_instruction_division_by_127_is_the_division(pkg, gpu):

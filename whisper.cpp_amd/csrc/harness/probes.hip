@@ -135,3 +135,51 @@ PROBE_API int mi355x_probe_div127(void * differing, void * stream) {
     k_probe_div127<<<2048, 256, 0, (hipStream_t) stream>>>((unsigned long long *) differing);
     return launch_status();
 }
+
+// The path from global memory into a CU that the GEMM operands take.  Every wavefront issues rounds of eight 1 KB loads (a
+// lane's 16 bytes of a 128-byte row piece, rows 2560 bytes apart as in an f16 operand with K = 1280), either straight into LDS
+// (global_load_lds_dwordx4, one round in flight behind the one being issued) or into registers (all eight awaited).
+// span = 0: every wavefront reads the same 8 KB, which stay in the L1; span > 0: the workgroups start at scattered rows of
+// [src, src + span) and walk 20 K steps of 128 bytes, round and round — 2 MB stay in every L2, the 17 MB of an FFN-up
+// product's operands do not.  clocks[2 w], clocks[2 w + 1]: s_memtime and s_memrealtime (100 MHz) ticks of workgroup w's loop.
+// Bytes moved: workgroups * 4 wavefronts * iters * 8 KB.  `src` must hold span + 1 MB.
+template <bool TO_LDS>
+__global__ void __launch_bounds__(256, 2) k_probe_load_path(const char * __restrict__ src, size_t span, int iters, unsigned long long * __restrict__ clocks, u32x4 * __restrict__ sink) {
+    extern __shared__ __attribute__((aligned(16))) char probe_lds[];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const size_t row0 = ((size_t) blockIdx.x * 37 % 1024) * 128 + wave * 8 + (lane >> 3);
+    const char * p = span == 0 ? src + lane * 16 : src + (row0 * 2560 + (lane & 7) * 16) % span;
+    const size_t istep = span == 0 ? 1024 : (size_t) 32 * 2560, kstep = span == 0 ? 0 : 128;
+    u32x4 acc = { 0, 0, 0, 0 };
+    const unsigned long long c0 = __builtin_amdgcn_s_memtime(), r0 = __builtin_amdgcn_s_memrealtime();
+    for (int it = 0; it < iters; ++it) {
+        const size_t ko = (size_t)(it % 20) * kstep;
+        char * dst = probe_lds + ((it & 1) * 32 + wave * 8) * 1024;
+        if (TO_LDS) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+                __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(p + ko + (size_t) i * istep),
+                                                 (__attribute__((address_space(3))) void *)(dst + i * 1024), 16, 0, 0);
+            __builtin_amdgcn_s_waitcnt((8 & 15) | ((8 >> 4) << 14) | (7 << 4) | (15 << 8));      // vmcnt(8): the round before has landed
+        } else {
+            u32x4 v[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) v[i] = __builtin_nontemporal_load((const u32x4 *)(p + ko + (size_t) i * istep));
+#pragma unroll
+            for (int i = 0; i < 8; ++i) acc ^= v[i];
+        }
+    }
+    __builtin_amdgcn_s_waitcnt(0);
+    if (threadIdx.x == 0) { clocks[2 * blockIdx.x] = __builtin_amdgcn_s_memtime() - c0; clocks[2 * blockIdx.x + 1] = __builtin_amdgcn_s_memrealtime() - r0; }
+    if (!TO_LDS && acc.x == 0x12345678u) sink[0] = acc;
+}
+
+PROBE_API int mi355x_probe_load_path(const void * src, size_t span, int to_lds, int iters, int workgroups, void * clocks, void * stream) {
+    if (!src || !clocks || (uintptr_t) src % 16 != 0 || (uintptr_t) clocks % 16 != 0 || iters < 1 || iters > (1 << 20) || workgroups < 1 || workgroups > 4096) return MI355X_ERR_INVALID;
+    if (span != 0 && span < ((size_t) 1 << 20)) return MI355X_ERR_INVALID;
+    // (the last 16 bytes of `clocks`, behind the 2 * workgroups counters, take the register variant's sink)
+    u32x4 * sink = (u32x4 *)((unsigned long long *) clocks + 2 * (size_t) workgroups);
+    if (to_lds) k_probe_load_path<true ><<<(unsigned) workgroups, 256, 65536, (hipStream_t) stream>>>((const char *) src, span, iters, (unsigned long long *) clocks, sink);
+    else        k_probe_load_path<false><<<(unsigned) workgroups, 256, 65536, (hipStream_t) stream>>>((const char *) src, span, iters, (unsigned long long *) clocks, sink);
+    return launch_status();
+}
