@@ -302,6 +302,12 @@ def gemm_library_yardstick() -> list | None:
             rows.append({"shape": what, "m": m, "n": n, "k": k, "this_library_us": round(ours, 2), "vendor_blas_us": round(blas, 2),
                          "this_library_tflops": round(gflop / ours * 1e3, 1), "vendor_blas_tflops": round(gflop / blas * 1e3, 1),
                          "vendor_blas_frac_of_peak": round(gflop / blas * 1e3 / PEAK_MFMA_F16_TFLOPS, 4)})
+            if m != 3840:
+                # ... and with an f16 result like the vendor's (the epilogue's MI355X_EPI_OUT_F16): half the bytes to store
+                d16 = torch.empty(n, m, device=dev, dtype=torch.half)
+                td16, epi16 = pkg.tensor(d16, pkg.F16), pkg.Epilogue(pkg.EPI_OUT_F16, 1.0, None, None, None)
+                ours16 = timed(lambda: pkg.check(lib.mi355x_mul_mat(C.byref(tw), C.byref(tx), C.byref(td16), C.byref(epi16), None, 0, None)))
+                rows[-1]["this_library_f16_result_us"] = round(ours16, 2)
         # the matrix instruction by itself: v_mfma_f32_32x32x16_f16 from registers, one and four wavefronts per SIMD
         sink = torch.zeros(1, device=dev)
         pr = probes()
