@@ -410,7 +410,7 @@ def main() -> int:
             decode["gemv_roofline"]["plateau"] = pl
             decode["gemv_roofline"]["plateau_frac"] = pl["eight_times_the_rows"]["gemv"]["p10_to_p90_frac_of_hbm_peak"]
     for small in sorted(dk):
-        if small != gemv_name and (small.startswith("mul_mat.gemv") or small.startswith("norm_mul_mat")):
+        if small != gemv_name and (small.startswith("mul_mat.gemv") or "norm_mul_mat" in small):
             # the products over 1.7 ... 7 MB matrices: over in the launch-to-store latency of a small kernel
             decode.setdefault("gemv_small_rooflines", []).append(kernel_roofline(small, dk[small]))
     decode["kernel_breakdown"] = {n: {"launches_per_step": k["calls"] / dec["steps"], "ms_per_step": round(k["ms"] / dec["steps"], 4)}

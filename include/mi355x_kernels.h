@@ -172,6 +172,18 @@ MI355X_API int    mi355x_mul_mat_group(const mi355x_mul_mat_item * items, int co
  * mi355x_norm_emit_q8_0 and the products).  No counterpart in the reference, whose graphs hold these as separate nodes. */
 MI355X_API int    mi355x_norm_mul_mat_group(const mi355x_tensor * src, const mi355x_tensor * normed, float eps, const float * w, const float * b,
                                             const mi355x_mul_mat_item * items, int count, void * workspace, size_t workspace_size, void * stream);
+/* mi355x_norm_mul_mat_group over rows that no launch has written yet: row n of `x0` is the token embedding tok[:, tok_ids[n]]
+ * plus the positional embedding pos[:, pos_ids[n]] — what mi355x_get_rows_add would leave there (GET_ROWS, GET_ROWS and ADD of
+ * src/whisper.cpp:2526-2529) — made by every workgroup for itself from the two tables, and written to `x0` by the first for
+ * the residual connections that read it later; an index outside its table gives a NaN row, as there.  The same values bit for
+ * bit as mi355x_get_rows_add followed by mi355x_norm_mul_mat_group.  tok: Q8_0, Q5_0 or F16 [K, n_vocab]; pos: F32 [K, n_ctx],
+ * 16-byte aligned rows; tok_ids, pos_ids: dense I32 vectors of x0's row count; everything else as for
+ * mi355x_norm_mul_mat_group, and only where the products take one weight block per lane (K <= 2048 with 64 lanes per row:
+ * a layer's Q, K and V); MI355X_ERR_UNSUPPORTED otherwise (then call mi355x_get_rows_add and mi355x_norm_mul_mat_group).
+ * No counterpart in the reference, whose graphs hold these as separate nodes. */
+MI355X_API int    mi355x_embed_norm_mul_mat_group(const mi355x_tensor * tok, const mi355x_tensor * tok_ids, const mi355x_tensor * pos, const mi355x_tensor * pos_ids,
+                                                  const mi355x_tensor * x0, const mi355x_tensor * normed, float eps, const float * w, const float * b,
+                                                  const mi355x_mul_mat_item * items, int count, void * workspace, size_t workspace_size, void * stream);
 
 /* The few-column product (ggml_compute_forward_mul_mat with ggml_vec_dot_q8_0_q8_0, ggml-cpu.c:1266-1458,
  * ggml-cpu-quants.c:3597) over a Q8_0 matrix long enough to be a stream — the vocabulary projection — with the integer

@@ -297,3 +297,22 @@ def test_five_row_decode_steps_until_the_cache_is_full(harness, models, key, env
     assert s["kv_positions"] == 448 and s["batch"] == 5 and s["rows"] >= 440, s
     check_model_summary(s, strict_ids=False)
     assert rc == 0
+
+
+@pytest.mark.parametrize("key", [("large-v3-turbo", "q8_0"), ("base", "q5_0")])
+def test_the_token_embedding_of_a_decode_step_is_made_inside_the_first_layers_launch(harness, models, key):
+    # GET_ROWS, GET_ROWS and ADD of a step's few rows have no launch of their own: the launch that normalizes the rows and
+    # multiplies them by the first layer's quantized Q, K and V makes them (Q8_0 and Q5_0 token tables here; F16 tables in
+    # the kernel test); without fusion the gathers are back.  (The logits of such steps are compared in the five-row test
+    # above.)
+    args = ["bench", "--model", models[key], "--what", "decoder", "--backend", "gpu", "--reps", "1", "--warmup", "1", "--steps", "8", "--batch", "5",
+            "--kv-stride", "2", "--profile", "--threads", "4"]
+    rc, rows = run_harness(harness, args, timeout=600)
+    names = {k["kernel"] for k in rows[-1]["kernels"]}
+    assert rc == 0 and "embed_norm_mul_mat.gemv" in names and "get_rows_add" not in names and "get_rows" not in names, names
+    fused = rows[-1]["launches_per_step"]
+    if key[0] == "large-v3-turbo":
+        assert fused <= 34, fused
+    rc, rows = run_harness(harness, args, env={"GGML_MI355X_FUSE": "0"}, timeout=600)
+    names = {k["kernel"] for k in rows[-1]["kernels"]}
+    assert rc == 0 and "get_rows" in names and "embed_norm_mul_mat.gemv" not in names and rows[-1]["launches_per_step"] > fused, names

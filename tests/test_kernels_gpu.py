@@ -452,6 +452,84 @@ def test_norm_mul_mat_group(pkg, oracle, gpu, wtype, n, k, m, count):
         assert lib.mi355x_norm_mul_mat_group(tl, tl, 1e-5, None, None, (pkg.MulMatItem * 1)(), 1, None, 0, gpu.stream) in (-1, -2)
 
 
+@pytest.mark.parametrize("wtype,ttype,n,k,m,count", [("Q8_0", "Q8_0", 5, 1280, 1280, 3), ("Q5_0", "F16", 3, 512, 512, 3), ("Q8_0", "F16", 8, 384, 384, 3),
+                                                     ("Q5_0", "Q8_0", 1, 1280, 1280, 3), ("Q8_0", "Q8_0", 2, 768, 768, 1), ("Q5_0", "Q5_0", 5, 1280, 1280, 3),
+                                                     ("Q5_0", "Q5_0", 7, 512, 512, 3)])
+def test_embed_norm_mul_mat_group(pkg, oracle, gpu, wtype, ttype, n, k, m, count):
+    # the token + positional embedding of a decode step made inside the launch that normalizes it and multiplies: the same
+    # embedding rows, normalized rows, Q8_0 form and products, bit for bit, as mi355x_get_rows_add followed by
+    # mi355x_norm_mul_mat_group
+    lib = pkg.kernels()
+    t, tt = getattr(pkg, wtype), getattr(pkg, ttype)
+    n_vocab, n_ctx = 300, 48
+    table = rnd((n_vocab, k), 0.05)
+    tok = oracle.quantize(tt, table) if tt != pkg.F16 else oracle.f32_to_f16_bits(table)
+    pos = rnd((n_ctx, k), 0.05)
+    w, b = rnd((k,), 0.02, 1.0), rnd((k,), 0.02)
+    d_tok, d_pos, d_w, d_b = gpu.up(tok), gpu.up(pos), gpu.up(w), gpu.up(b)
+    t_tok, t_pos = pkg.tensor(d_tok, tt, ne=[k, n_vocab]), pkg.tensor(d_pos, pkg.F32)
+    mats = [oracle.quantize(t, rnd((m, k), 0.02)) for _ in range(count)]
+    d_m = [gpu.up(q) for q in mats]
+    tws = [pkg.tensor(q, t, ne=[k, m]) for q in d_m]
+    need = lib.mi355x_mul_mat_workspace_size(tws[0], pkg.tensor(torch.zeros((n, k), dtype=torch.float32, device=gpu.dev), pkg.F32))
+    assert need > 0
+
+    def run(fused, ids, pids):
+        d_i, d_pi = gpu.up(ids), gpu.up(pids)
+        t_i, t_pi = pkg.tensor(d_i, pkg.I32), pkg.tensor(d_pi, pkg.I32)
+        d_x = torch.full((n, k), 7.0, dtype=torch.float32, device=gpu.dev)
+        d_y = torch.zeros_like(d_x)
+        ws = torch.zeros(need, dtype=torch.uint8, device=gpu.dev)
+        outs = [torch.zeros((n, m), dtype=torch.float32, device=gpu.dev) for _ in range(count)]
+        tds = [pkg.tensor(o, pkg.F32) for o in outs]
+        items = (pkg.MulMatItem * count)()
+        for i in range(count):
+            items[i].src0, items[i].dst, items[i].epi = C.pointer(tws[i]), C.pointer(tds[i]), None
+        tx, ty = pkg.tensor(d_x, pkg.F32), pkg.tensor(d_y, pkg.F32)
+        if fused:
+            pkg.check(lib.mi355x_embed_norm_mul_mat_group(t_tok, t_i, t_pos, t_pi, tx, ty, 1e-5, d_w.data_ptr(), d_b.data_ptr(), items, count, ws.data_ptr(), need, gpu.stream))
+        else:
+            pkg.check(lib.mi355x_get_rows_add(t_tok, t_i, t_pos, t_pi, tx, gpu.stream))
+            pkg.check(lib.mi355x_norm_mul_mat_group(tx, ty, 1e-5, d_w.data_ptr(), d_b.data_ptr(), items, count, ws.data_ptr(), need, gpu.stream))
+        return gpu.down(d_x), gpu.down(d_y), gpu.down(ws)[: n * k + n * (k // 32) * 8], [gpu.down(o) for o in outs]
+
+    ids = np.array([5, 299, 0, 5, 17, 123, 1, 298], dtype=np.int32)[:n]
+    pids = np.array([7, 8, 47, 0, 7, 9, 10, 11], dtype=np.int32)[:n]
+    x1, y1, q1, o1 = run(True, ids, pids)
+    x0, y0, q0, o0 = run(False, ids, pids)
+    if tt != pkg.F16:
+        assert np.array_equal(x0, oracle.binary(0, oracle.get_rows(tt, tok, ids, k), pos[pids]))
+    else:
+        assert np.array_equal(x0, oracle.f16_bits_to_f32(tok[ids]) + pos[pids])
+    assert np.array_equal(x1, x0) and np.array_equal(y1, y0) and np.array_equal(q1, q0)
+    for a, bb in zip(o1, o0):
+        assert np.array_equal(a, bb)
+    # an index outside its table: a NaN row, as from the launch of its own, and the rows beside it untouched by that
+    if n >= 3:
+        bad, pbad = ids.copy(), pids.copy()
+        bad[1], pbad[2] = n_vocab, -1
+        x1, y1, _, o1 = run(True, bad, pbad)
+        x0, y0, _, o0 = run(False, bad, pbad)
+        assert np.isnan(x1[[1, 2]]).all() and np.isnan(y1[[1, 2]]).all()
+        keep = [r for r in range(n) if r not in (1, 2)]
+        assert np.array_equal(x1[keep], x0[keep]) and np.array_equal(y1[keep], y0[keep]) and np.array_equal(o1[0][keep], o0[0][keep])
+    # index vectors of another length, a table of another width, a token table of a type the launch does not read
+    d_i, d_pi = gpu.up(ids), gpu.up(pids)
+    d_x = torch.zeros((n, k), dtype=torch.float32, device=gpu.dev)
+    tx = pkg.tensor(d_x, pkg.F32)
+    items = (pkg.MulMatItem * 1)()
+    out = torch.zeros((n, m), dtype=torch.float32, device=gpu.dev)
+    td = pkg.tensor(out, pkg.F32)
+    items[0].src0, items[0].dst, items[0].epi = C.pointer(tws[0]), C.pointer(td), None
+    ws = torch.zeros(need, dtype=torch.uint8, device=gpu.dev)
+    args = (1e-5, d_w.data_ptr(), d_b.data_ptr(), items, 1, ws.data_ptr(), need, gpu.stream)
+    if n > 1:
+        assert lib.mi355x_embed_norm_mul_mat_group(t_tok, pkg.tensor(d_i[: n - 1], pkg.I32), t_pos, pkg.tensor(d_pi, pkg.I32), tx, tx, *args) == -1
+    assert lib.mi355x_embed_norm_mul_mat_group(t_tok, pkg.tensor(d_i, pkg.I32), pkg.tensor(d_pos[:, : k - 32], pkg.F32), pkg.tensor(d_pi, pkg.I32), tx, tx, *args) == -2
+    assert lib.mi355x_embed_norm_mul_mat_group(pkg.tensor(d_pos, pkg.F32), pkg.tensor(d_i, pkg.I32), t_pos, pkg.tensor(d_pi, pkg.I32), tx, tx, *args) == -1
+    assert lib.mi355x_embed_norm_mul_mat_group(None, pkg.tensor(d_i, pkg.I32), t_pos, pkg.tensor(d_pi, pkg.I32), tx, tx, *args) == -2
+
+
 @pytest.mark.parametrize("wtype,n,k,m", [("Q8_0", 5, 1280, 5120), ("Q5_0", 3, 512, 384), ("Q8_0", 8, 384, 1536), ("Q8_0", 1, 1280, 5120)])
 def test_few_column_product_emits_its_result_as_q8_0(pkg, oracle, gpu, wtype, n, k, m):
     # MI355X_EPI_EMIT_Q8_0: a decode step's FFN-up product (bias + GELU) leaves its rows quantized for FFN-down, in the layout

@@ -223,6 +223,7 @@ struct launch_scope {   // brackets one kernel launch with events when profiling
         if (ev.stop) (void) hipEventRecord(ev.stop, ctx->stream);
         ctx->pending.push_back(ev);
     }
+    void cancel() { ctx->counters[3] -= 1; on = false; }   // nothing was launched after all
 };
 
 double nbytes_of(const ggml_tensor * t) { return t ? (double) ggml_nbytes(t) : 0.0; }
@@ -464,7 +465,26 @@ struct graph_runner {
         bool affine = false;
     } held;
 
+    // The embedding of a decode step's tokens (GET_ROWS, GET_ROWS, ADD: a handful of rows) that only feeds a LayerNorm is
+    // held the same way: if that LayerNorm ends up inside the launch of its products, the rows are made there
+    // (mi355x_embed_norm_mul_mat_group); in every other case the embedding runs on its own first (flush_embed).
+    struct held_embed {
+        bool active = false;
+        const ggml_tensor * tok = nullptr, * tok_ids = nullptr, * pos = nullptr, * pos_ids = nullptr, * out = nullptr;
+    } emb;
+
+    int flush_embed() {
+        if (!emb.active) return MI355X_OK;
+        emb.active = false;
+        mi355x_tensor a = to_view(emb.tok), ia = to_view(emb.tok_ids), b = to_view(emb.pos), ib = to_view(emb.pos_ids), d = to_view(emb.out);
+        launch_scope ls(ctx, "get_rows_add", 3.0 * nbytes_of(emb.out), 0.0);
+        const int rc = mi355x_get_rows_add(&a, &ia, &b, &ib, &d, ctx->stream);
+        note_write(emb.out);
+        return rc;
+    }
+
     int flush_norm() {
+        if (const int rc = flush_embed()) return rc;        // (a held embedding is the held LayerNorm's source)
         if (!held.active) return MI355X_OK;
         held.active = false;
         mi355x_tensor vs = to_view(held.src), vd = to_view(held.out);
@@ -539,15 +559,33 @@ struct graph_runner {
             }
             if (!ctx->reserve_workspace(need_all)) { status = MI355X_ERR_WORKSPACE; return end - i; }
             mi355x_tensor vs = to_view(held.src), vn = to_view(held.out);
-            int rc;
-            {
-                launch_scope ls(ctx, "norm_mul_mat.gemv", bytes + nbytes_of(held.src) + nbytes_of(held.out), flops);
-                if (q8_key) { chains[0].epi.flags |= MI355X_EPI_EMIT_Q8_0; chains[0].epi.image = slot_ptr(ctx->ws_slot ^ 1); }
-                rc = mi355x_norm_mul_mat_group(&vs, &vn, held.eps, held.w, held.b, items.data(), (int) items.size(), ctx->ws, ctx->ws_size, ctx->stream);
-                if (rc == MI355X_ERR_UNSUPPORTED && q8_key) {
+            if (q8_key) { chains[0].epi.flags |= MI355X_EPI_EMIT_Q8_0; chains[0].epi.image = slot_ptr(ctx->ws_slot ^ 1); }
+            auto launch = [&](bool embed) {
+                mi355x_tensor vt, vti, vp, vpi;
+                if (embed) { vt = to_view(emb.tok); vti = to_view(emb.tok_ids); vp = to_view(emb.pos); vpi = to_view(emb.pos_ids); }
+                auto call = [&]() {
+                    return embed ? mi355x_embed_norm_mul_mat_group(&vt, &vti, &vp, &vpi, &vs, &vn, held.eps, held.w, held.b, items.data(), (int) items.size(), ctx->ws, ctx->ws_size, ctx->stream)
+                                 : mi355x_norm_mul_mat_group(&vs, &vn, held.eps, held.w, held.b, items.data(), (int) items.size(), ctx->ws, ctx->ws_size, ctx->stream);
+                };
+                int r = call();
+                if (r == MI355X_ERR_UNSUPPORTED && q8_key) {
                     chains[0].epi.flags &= ~MI355X_EPI_EMIT_Q8_0; chains[0].epi.image = nullptr; q8_key = nullptr;
-                    rc = mi355x_norm_mul_mat_group(&vs, &vn, held.eps, held.w, held.b, items.data(), (int) items.size(), ctx->ws, ctx->ws_size, ctx->stream);
+                    r = call();
                 }
+                return r;
+            };
+            int rc = MI355X_ERR_UNSUPPORTED;
+            if (emb.active) {                               // (then held.src is the embedding: nothing has written it yet)
+                launch_scope ls(ctx, "embed_norm_mul_mat.gemv", bytes + 3.0 * nbytes_of(held.src) + nbytes_of(held.out), flops);
+                rc = launch(true);
+                if (rc == MI355X_ERR_UNSUPPORTED) ls.cancel();
+                else { emb.active = false; note_write(emb.out); }
+            }
+            if (rc == MI355X_ERR_UNSUPPORTED) {
+                if ((rc = flush_embed()) != MI355X_OK) { status = rc; return end - i; }
+                launch_scope ls(ctx, "norm_mul_mat.gemv", bytes + nbytes_of(held.src) + nbytes_of(held.out), flops);
+                rc = launch(false);
+                if (rc == MI355X_ERR_UNSUPPORTED) ls.cancel();
             }
             if (rc == MI355X_ERR_UNSUPPORTED) return 0;      // the caller lets the LayerNorm run on its own and takes the usual path
             held.active = false;
@@ -699,6 +737,7 @@ struct graph_runner {
             fold_nodes(i, used, out);
             return used;
         }
+        if ((status = flush_embed()) != MI355X_OK) return used;
         const size_t image_bytes = mode == 1 ? (size_t)(out->ne[0] * out->ne[1] * 2) : (size_t)(out->ne[0] * out->ne[1] + out->ne[0] / 32 * out->ne[1] * 8);
         bool emit = key && ctx->reserve_workspace(image_bytes + 256);
         // the image and nothing else when the product that takes it is the very next launch: the f32 rows would have no reader
@@ -764,6 +803,7 @@ struct graph_runner {
         if (ggml_is_empty(n) || is_view_op(n->op)) return 1;
         const ggml_tensor * s0 = n->src[0], * s1 = n->src[1];
         if (held.active && !(n->op == GGML_OP_MUL_MAT && s1 == held.key) && (status = flush_norm()) != MI355X_OK) return 1;
+        if (emb.active && !held.active && !(n->op == GGML_OP_NORM && s0 == emb.out) && (status = flush_embed()) != MI355X_OK) return 1;
         if (n->op != GGML_OP_MUL_MAT && n->op != GGML_OP_NORM) note_write(n->op == GGML_OP_CPY ? s1 : n);
         switch (n->op) {
             case GGML_OP_MUL_MAT: return run_mul_mat(i, status);
@@ -820,6 +860,15 @@ struct graph_runner {
                         g2->src[1]->ne[0] == s1->ne[0] && g2->src[1]->ne[1] == 1 && g2->src[1]->ne[2] == 1 && g2->src[1]->ne[3] == 1) {
                         bool plain = true;                  // nothing between the three nodes may be a view of the gathered tensors
                         for (int v = i + 1; v < k; ++v) plain = plain && (v == j || (node_at(v)->src[0] != n && node_at(v)->view_src != n && node_at(v)->src[0] != g2 && node_at(v)->view_src != g2));
+                        // a handful of rows that the next launch normalizes: held, to be made inside that launch if it comes to one
+                        int nx = k + 1;
+                        while (node_at(nx) && (is_view_op(node_at(nx)->op) || ggml_is_empty(node_at(nx)))) ++nx;
+                        if (plain && add->ne[1] <= 8 && add->ne[2] == 1 && add->ne[3] == 1 && (s0->type == GGML_TYPE_Q8_0 || s0->type == GGML_TYPE_Q5_0 || s0->type == GGML_TYPE_F16) &&
+                            node_at(nx) && node_at(nx)->op == GGML_OP_NORM && node_at(nx)->src[0] == add) {
+                            emb.active = true; emb.tok = s0; emb.tok_ids = s1; emb.pos = g2->src[0]; emb.pos_ids = g2->src[1]; emb.out = add;
+                            note_write(add); fold_nodes(i, k - i + 1, add);
+                            return k - i + 1;
+                        }
                         if (plain) {
                             mi355x_tensor a = to_view(s0), ia = to_view(s1), b = to_view(g2->src[0]), ib = to_view(g2->src[1]), d = to_view(add);
                             int rc;

@@ -1253,11 +1253,14 @@ __global__ void __launch_bounds__(256) k_quantize_x_q8(const char * __restrict__
 // the activations in LDS, their reads (NC x 32 bytes per 34-byte block) are what bounds the kernel, and quantizing them
 // in every workgroup costs more than the product itself once K is large.
 struct gemv_no_prologue {
+    static constexpr bool LATE = false;
     __device__ __forceinline__ void request() {}
+    __device__ __forceinline__ void request_late() {}
     __device__ __forceinline__ const char * finish(const char * x) { return x; }
 };
 
-// `prologue` has two halves: request() issues its own loads BEFORE the first weight blocks are requested, finish() runs
+// `prologue` has two halves: request() issues its own loads BEFORE the first weight blocks are requested (request_late(),
+// if it has one, the loads that depend on those, after the first weight blocks), finish() runs
 // after them and returns where the quantized activations are (the plain product: the workspace as passed; the fused
 // LayerNorm first produces them in LDS).  Loads are waited for in the order they were issued, so in this order the
 // LayerNorm's reductions run while the weight blocks are still on their way from HBM (vmcnt(3) in front of them, where
@@ -1301,6 +1304,10 @@ __device__ __forceinline__ void gemv_qr_rows(const mm_args & a, PRO prologue = P
         for (int b = 0; b < NB; ++b) blk[b] = load_wraw<T0>(wrow, blk_ok[b] ? j + b * LPR : nbk - 1);
     };
     load_blocks();
+    if constexpr (PRO::LATE) {                          // loads whose addresses request() fetched: behind the first weight blocks
+        __builtin_amdgcn_sched_barrier(0);
+        prologue.request_late();
+    }
 
     const char * xbase = prologue.finish(a.x);
     const int32_t * xq   = (const int32_t *) xbase;
@@ -1504,11 +1511,16 @@ struct gemv_norm_args {
     const float * w; const float * b; float eps;
     char * dst; int64_t dst_nb1;       // f32 rows of the normalized activations
     char * ws;                         // their Q8_0 form (layout of k_quantize_x_q8)
+    // EMB instances: row n of the source is not read but made here, token row tok_ids[n] (Q8_0, Q5_0 or F16) plus position row
+    // pos_ids[n] (F32) as in k_get_rows_add, and the first workgroup writes it to x0
+    const char * tok; int tok_type; int64_t tok_nb1, tok_ne1; const int32_t * tok_ids;
+    const char * pos; int64_t pos_nb1, pos_ne1; const int32_t * pos_ids;
+    char * x0;
 };
 
 // NJ > 0: the rows are exactly 256 NJ values long and both affine vectors are there (whisper's LayerNorms at 512 ... 1280):
 // NJ float4s per lane instead of eight, no guard around a term, no clamped address
-template <int NC, int NJ = 0>
+template <int NC, int NJ = 0, bool EMB = false>
 struct gemv_norm_prologue {
     const gemv_norm_args & nm; int64_t K; char * lds;
     // wavefront w takes rows w and w + 4; both rows and the affine vectors are requested before anything is reduced, so
@@ -1516,20 +1528,64 @@ struct gemv_norm_prologue {
     static constexpr int RW = (NC + 3) / 4;                 // rows per wavefront
     static constexpr int JN = NJ ? NJ : 8;                  // float4s per lane and row
     float4 v[RW][JN], ww[JN], bb[JN];
+    // EMB: four values of the token row as they lie in the table (Q8_0: four quants and the block's scale; Q5_0: four bytes
+    // of nibbles, the scale and the block's fifth bits; F16: two words) next to the position row's four in v, and whether
+    // the row's two indices are inside their tables
+    uint32_t tq[EMB ? RW : 1][EMB ? JN : 1], td[EMB ? RW : 1][EMB ? JN : 1], th[EMB ? RW : 1][EMB ? JN : 1];
+    int32_t r0[RW], r1[RW];
+    bool ok[RW];
+    static constexpr bool LATE = EMB;
 
     __device__ __forceinline__ void request() {
         const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
         const int n4 = (int)(K / 4);
+        if constexpr (EMB) {                                // the rows' indices now, the rows themselves in request_late()
+#pragma unroll
+            for (int rr = 0; rr < RW; ++rr) {
+                const int row = wave + 4 * rr < NC ? wave + 4 * rr : NC - 1;
+                r0[rr] = nm.tok_ids[row]; r1[rr] = nm.pos_ids[row];
+            }
+        }
         // no branch around a load: addresses are clamped into the rows, and a missing affine vector reads the source instead
         const float4 * wp = (const float4 *)(NJ || nm.w ? (const char *) nm.w : nm.src), * bp = (const float4 *)(NJ || nm.b ? (const char *) nm.b : nm.src);
 #pragma unroll
         for (int jj = 0; jj < JN; ++jj) {
             const int c = NJ || lane + jj * WAVE < n4 ? lane + jj * WAVE : n4 - 1;
             ww[jj] = wp[c]; bb[jj] = bp[c];
+            if constexpr (!EMB) {
+#pragma unroll
+                for (int rr = 0; rr < RW; ++rr) {
+                    const int row = wave + 4 * rr < NC ? wave + 4 * rr : NC - 1;
+                    v[rr][jj] = ((const float4 *)(nm.src + row * nm.src_nb1))[c];
+                }
+            }
+        }
+    }
+
+    __device__ __forceinline__ void request_late() {
+        if constexpr (EMB) {
+            const int lane = threadIdx.x & 63;
+            const int n4 = (int)(K / 4);
 #pragma unroll
             for (int rr = 0; rr < RW; ++rr) {
-                const int row = wave + 4 * rr < NC ? wave + 4 * rr : NC - 1;
-                v[rr][jj] = ((const float4 *)(nm.src + row * nm.src_nb1))[c];
+                ok[rr] = r0[rr] >= 0 && r0[rr] < nm.tok_ne1 && r1[rr] >= 0 && r1[rr] < nm.pos_ne1;
+                const uint8_t * tp = (const uint8_t *) nm.tok + (int64_t)(ok[rr] ? r0[rr] : 0) * nm.tok_nb1;
+                const float4 *  pp = (const float4 *)(nm.pos + (int64_t)(ok[rr] ? r1[rr] : 0) * nm.pos_nb1);
+#pragma unroll
+                for (int jj = 0; jj < JN; ++jj) {
+                    const int c = NJ || lane + jj * WAVE < n4 ? lane + jj * WAVE : n4 - 1;
+                    v[rr][jj] = pp[c];
+                    if (nm.tok_type == MI355X_TYPE_Q8_0) {          // uniform
+                        const uint8_t * blk = tp + (c >> 3) * 34;
+                        td[rr][jj] = ld_u16(blk); tq[rr][jj] = *(const u32a2 *)(blk + 2 + 4 * (c & 7));
+                    } else if (nm.tok_type == MI355X_TYPE_Q5_0) {   // (weights j and j + 16 of a block share a byte)
+                        const uint8_t * blk = tp + (c >> 3) * 22;
+                        td[rr][jj] = ld_u16(blk); th[rr][jj] = *(const u32a2 *)(blk + 2); tq[rr][jj] = *(const u32a2 *)(blk + 6 + 4 * (c & 3));
+                    } else {
+                        const uint2 h = ((const uint2 *) tp)[c];
+                        tq[rr][jj] = h.x; td[rr][jj] = h.y;
+                    }
+                }
             }
         }
     }
@@ -1545,6 +1601,33 @@ struct gemv_norm_prologue {
         for (int rr = 0; rr < RW; ++rr) {
             const int row = wave + 4 * rr;
             if (row >= NC) break;                           // uniform
+            if constexpr (EMB) {                            // the source row: dequantized token values plus position values
+#pragma unroll
+                for (int jj = 0; jj < JN; ++jj) {
+                    float4 e;
+                    const uint32_t q = tq[rr][jj], d = td[rr][jj];
+                    if (nm.tok_type == MI355X_TYPE_Q8_0) {
+                        const float sc = h2f((uint16_t) d);
+                        e.x = (float)(int8_t) q * sc;         e.y = (float)(int8_t)(q >> 8) * sc;
+                        e.z = (float)(int8_t)(q >> 16) * sc;  e.w = (float)(int8_t)(q >> 24) * sc;
+                    } else if (nm.tok_type == MI355X_TYPE_Q5_0) {
+                        const float sc = h2f((uint16_t) d);
+                        const int c = NJ || lane + jj * WAVE < n4 ? lane + jj * WAVE : n4 - 1;
+                        const int j0 = 4 * (c & 7);                                     // first of the lane's four weights in the block
+                        const uint32_t nib = (j0 < 16 ? q : q >> 4) & 0x0F0F0F0Fu, hb = th[rr][jj] >> j0;
+                        e.x = (float)((int)((nib & 15)         | ((hb & 1) << 4))        - 16) * sc;
+                        e.y = (float)((int)(((nib >> 8) & 15)  | (((hb >> 1) & 1) << 4)) - 16) * sc;
+                        e.z = (float)((int)(((nib >> 16) & 15) | (((hb >> 2) & 1) << 4)) - 16) * sc;
+                        e.w = (float)((int)(((nib >> 24) & 15) | (((hb >> 3) & 1) << 4)) - 16) * sc;
+                    } else {
+                        e.x = h2f((uint16_t) q); e.y = h2f((uint16_t)(q >> 16)); e.z = h2f((uint16_t) d); e.w = h2f((uint16_t)(d >> 16));
+                    }
+                    float4 & t = v[rr][jj];
+                    const float nan = __builtin_nanf("");
+                    t.x = ok[rr] ? e.x + t.x : nan; t.y = ok[rr] ? e.y + t.y : nan; t.z = ok[rr] ? e.z + t.z : nan; t.w = ok[rr] ? e.w + t.w : nan;
+                    if (writer && (NJ || lane + jj * WAVE < n4)) ((float4 *)(nm.x0 + row * nm.src_nb1))[lane + jj * WAVE] = t;
+                }
+            }
             float sum = 0.0f;
 #pragma unroll
             for (int jj = 0; jj < JN; ++jj) if (NJ || lane + jj * WAVE < n4) sum += (v[rr][jj].x + v[rr][jj].y) + (v[rr][jj].z + v[rr][jj].w);
@@ -1611,13 +1694,13 @@ struct gemv_norm_prologue {
     }
 };
 
-template <int T0, int NC, int LPR, int NB, int NJ = 0>
+template <int T0, int NC, int LPR, int NB, int NJ = 0, bool EMB = false>
 __global__ void __launch_bounds__(256) k_gemv_qr_norm_group(mm_args a, gemv_group grp, gemv_norm_args nm) {
     extern __shared__ __attribute__((aligned(16))) char smem[];
     const gemv_group_entry & ge = grp.e[blockIdx.y];
     a.w = ge.w; a.d = ge.d; a.d_nb1 = ge.d_nb1;
     a.e.flags = ge.flags; a.e.scale = ge.scale; a.e.bias = ge.bias; a.e.residual = ge.residual;
-    gemv_qr_rows<T0, NC, LPR, NB>(a, gemv_norm_prologue<NC, NJ>{ nm, a.K, smem });
+    gemv_qr_rows<T0, NC, LPR, NB>(a, gemv_norm_prologue<NC, NJ, EMB>{ nm, a.K, smem });
 }
 
 // ------------------------------------------------------------------------------------------------------
@@ -1712,8 +1795,16 @@ static int launch_gemv_r_k(const mm_args & a, unsigned grid, const gemv_group * 
     if (nm) {
         const size_t lds = (size_t) NC * a.K + (size_t) NC * (a.K / QK) * 8;
         // (the widest model's rows, 1280 values, have an instance without guards)
-        if (a.K == 1280 && nm->w && nm->b) k_gemv_qr_norm_group<T0, NC, LPR, NB, 5><<<dim3(grid, (unsigned) count), 256, lds, st>>>(a, *grp, *nm);
-        else                               k_gemv_qr_norm_group<T0, NC, LPR, NB><<<dim3(grid, (unsigned) count), 256, lds, st>>>(a, *grp, *nm);
+        const bool full = a.K == 1280 && nm->w && nm->b;
+        if (nm->tok) {                                      // (made for one block per lane, the shape of a layer's Q, K and V)
+            if constexpr (NB == 1) {
+                if (full) k_gemv_qr_norm_group<T0, NC, LPR, NB, 5, true><<<dim3(grid, (unsigned) count), 256, lds, st>>>(a, *grp, *nm);
+                else      k_gemv_qr_norm_group<T0, NC, LPR, NB, 0, true><<<dim3(grid, (unsigned) count), 256, lds, st>>>(a, *grp, *nm);
+            }
+            else return MI355X_ERR_UNSUPPORTED;
+        }
+        else if (full) k_gemv_qr_norm_group<T0, NC, LPR, NB, 5><<<dim3(grid, (unsigned) count), 256, lds, st>>>(a, *grp, *nm);
+        else           k_gemv_qr_norm_group<T0, NC, LPR, NB><<<dim3(grid, (unsigned) count), 256, lds, st>>>(a, *grp, *nm);
     }
     else if (grp) k_gemv_qr_group<T0, NC, LPR, NB><<<dim3(grid, (unsigned) count), 256, 0, st>>>(a, *grp);
     else          k_gemv_qr<T0, NC, LPR, NB><<<grid, 256, 0, st>>>(a);
@@ -1910,8 +2001,9 @@ static int mul_mat_group_gemv(const mi355x_mul_mat_item * items, int count, cons
     return w0->type == MI355X_TYPE_Q8_0 ? launch_gemv_r_n<MI355X_TYPE_Q8_0>(a, st, &grp, count) : launch_gemv_r_n<MI355X_TYPE_Q5_0>(a, st, &grp, count);
 }
 
-extern "C" int mi355x_norm_mul_mat_group(const mi355x_tensor * src, const mi355x_tensor * normed, float eps, const float * w, const float * b,
-                                         const mi355x_mul_mat_item * items, int count, void * workspace, size_t workspace_size, void * stream) {
+// the checks common to the LayerNorm-and-products entries; `nm` arrives with the gather fields set or zero
+static int norm_mul_mat_group(const mi355x_tensor * src, const mi355x_tensor * normed, float eps, const float * w, const float * b,
+                              const mi355x_mul_mat_item * items, int count, void * workspace, size_t workspace_size, void * stream, gemv_norm_args nm) {
     if (!src || !normed || !items || count < 1 || !(eps >= 0.0f)) return MI355X_ERR_INVALID;
     if (!items[0].src0 || !items[0].dst) return MI355X_ERR_INVALID;
     if (src->type != MI355X_TYPE_F32 || normed->type != MI355X_TYPE_F32 || src->nb[0] != 4 || normed->nb[0] != 4) return MI355X_ERR_UNSUPPORTED;
@@ -1920,8 +2012,36 @@ extern "C" int mi355x_norm_mul_mat_group(const mi355x_tensor * src, const mi355x
     if (src->ne[2] != 1 || src->ne[3] != 1 || N < 1 || N > MI355X_GEMV_MAX_COLS || K % QK != 0 || K > 2048) return MI355X_ERR_UNSUPPORTED;
     if (!aligned16(src) || !aligned16(normed) || (uintptr_t) w % 16 != 0 || (uintptr_t) b % 16 != 0) return MI355X_ERR_UNSUPPORTED;
     if (blck_size(items[0].src0->type) <= 1) return MI355X_ERR_UNSUPPORTED;
-    gemv_norm_args nm = { (const char *) src->data, (int64_t) src->nb[1], w, b, eps, (char *) normed->data, (int64_t) normed->nb[1], nullptr };
+    nm.src = (const char *) src->data; nm.src_nb1 = (int64_t) src->nb[1]; nm.w = w; nm.b = b; nm.eps = eps;
+    nm.dst = (char *) normed->data; nm.dst_nb1 = (int64_t) normed->nb[1]; nm.ws = nullptr;
     return mul_mat_group_gemv(items, count, normed, 0, workspace, workspace_size, stream, &nm);
+}
+
+extern "C" int mi355x_norm_mul_mat_group(const mi355x_tensor * src, const mi355x_tensor * normed, float eps, const float * w, const float * b,
+                                         const mi355x_mul_mat_item * items, int count, void * workspace, size_t workspace_size, void * stream) {
+    return norm_mul_mat_group(src, normed, eps, w, b, items, count, workspace, workspace_size, stream, gemv_norm_args{});
+}
+
+extern "C" int mi355x_embed_norm_mul_mat_group(const mi355x_tensor * tok, const mi355x_tensor * tok_ids, const mi355x_tensor * pos, const mi355x_tensor * pos_ids,
+                                               const mi355x_tensor * x0, const mi355x_tensor * normed, float eps, const float * w, const float * b,
+                                               const mi355x_mul_mat_item * items, int count, void * workspace, size_t workspace_size, void * stream) {
+    if (!tok || !tok_ids || !pos || !pos_ids || !x0) return MI355X_ERR_INVALID;
+    if (tok_ids->type != MI355X_TYPE_I32 || pos_ids->type != MI355X_TYPE_I32 || pos->type != MI355X_TYPE_F32) return MI355X_ERR_UNSUPPORTED;
+    if (tok->type != MI355X_TYPE_Q8_0 && tok->type != MI355X_TYPE_Q5_0 && tok->type != MI355X_TYPE_F16) return MI355X_ERR_UNSUPPORTED;
+    const int64_t K = x0->ne[0], N = x0->ne[1];
+    for (int i = 1; i < 4; ++i) if (tok_ids->ne[i] != 1 || pos_ids->ne[i] != 1) return MI355X_ERR_UNSUPPORTED;
+    if (tok_ids->ne[0] != N || pos_ids->ne[0] != N || tok_ids->nb[0] != 4 || pos_ids->nb[0] != 4) return MI355X_ERR_UNSUPPORTED;
+    if (tok->ne[2] != 1 || tok->ne[3] != 1 || pos->ne[2] != 1 || pos->ne[3] != 1) return MI355X_ERR_UNSUPPORTED;
+    if (tok->ne[0] != K || pos->ne[0] != K || pos->nb[0] != 4 || tok->nb[0] != type_size(tok->type)) return MI355X_ERR_INVALID;
+    // (a lane reads four values of a row at a time: 8 bytes of an F16 row, 16 of a position row; quantized blocks sit at even addresses)
+    const uintptr_t ta = tok->type == MI355X_TYPE_F16 ? 8 : 2;
+    if ((uintptr_t) tok->data % ta != 0 || tok->nb[1] % ta != 0 || (uintptr_t) pos->data % 16 != 0 || pos->nb[1] % 16 != 0 ||
+        (uintptr_t) tok_ids->data % 4 != 0 || (uintptr_t) pos_ids->data % 4 != 0) return MI355X_ERR_UNSUPPORTED;
+    gemv_norm_args nm{};
+    nm.tok = (const char *) tok->data; nm.tok_type = tok->type; nm.tok_nb1 = (int64_t) tok->nb[1]; nm.tok_ne1 = tok->ne[1]; nm.tok_ids = (const int32_t *) tok_ids->data;
+    nm.pos = (const char *) pos->data; nm.pos_nb1 = (int64_t) pos->nb[1]; nm.pos_ne1 = pos->ne[1]; nm.pos_ids = (const int32_t *) pos_ids->data;
+    nm.x0 = (char *) x0->data;
+    return norm_mul_mat_group(x0, normed, eps, w, b, items, count, workspace, workspace_size, stream, nm);
 }
 
 extern "C" int mi355x_mul_mat_group(const mi355x_mul_mat_item * items, int count, const mi355x_tensor * src1, int flags,

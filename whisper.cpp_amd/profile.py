@@ -89,7 +89,8 @@ def main() -> int:
             shutil.copy(f, out / f"kernel_stats_{name}.csv")
         shutil.rmtree(d, ignore_errors=True)
 
-    # ---- a decode step launch by launch: durations by position in the step (the steps begin at k_get_rows_add)
+    # ---- a decode step launch by launch: durations by position in the step (the steps begin where the token rows are
+    # gathered: the instance of k_gemv_qr_norm_group whose last template argument is true, else k_get_rows_add)
     d = out / "trace_positions"
     run(["rocprofv3", "--kernel-trace", "--output-format", "csv", "-d", str(d), "--", *DEC_CMD, "--reps", "1", "--warmup", "1", "--steps", "224"], out / "trace_positions.log", 170)
     rows = []
@@ -100,7 +101,7 @@ def main() -> int:
     rows.sort()
     steps, cur = [], None
     for st, en, name in rows:
-        if "k_get_rows_add" in name:
+        if "k_get_rows_add" in name or ("k_gemv_qr_norm_group" in name and (", true>" in name or "ELb1EE" in name)):
             if cur: steps.append(cur)
             cur = []
         if cur is not None: cur.append((st, en, name))
