@@ -393,7 +393,8 @@ def main() -> int:
     dec_x86 = run_harness(dec_args + ["--backend", "gpu", "--threads", str(a.threads)], env={"GGML_MI355X_FA_CHAIN": "0"})
     dk = {k["kernel"]: k for k in dec["kernels"]}
     # the logits product, 70.5 MB of Q8_0 blocks: the one GEMV that bandwidth bounds
-    gemv_name = "mul_mat.gemv_q8_0.vocab"
+    # (launched with the decoder's last LayerNorm of the step's rows in front, inside the same launch, under the arrival of the first tile rows)
+    gemv_name = "norm_mul_mat.gemv_q8_0.vocab" if "norm_mul_mat.gemv_q8_0.vocab" in dk else "mul_mat.gemv_q8_0.vocab"
     gemv = dk.get(gemv_name)
     decode = {"model": "large-v3-turbo Q8_0", "steps": dec["steps"], "beams": dec["batch"], "max_kv_positions": dec["max_kv_positions"],
               "ms_per_step": round(dec["ms_per_step"], 4), "steps_per_s": round(dec["steps_per_s"], 1), "beam_tokens_per_s": round(dec["batch_tokens_per_s"], 1),

@@ -203,6 +203,15 @@ MI355X_API size_t mi355x_q8_0_tiles_size(int64_t K, int64_t M);
 MI355X_API int    mi355x_q8_0_tiles_pack(const mi355x_tensor * src0, void * tiles, void * stream);
 MI355X_API int    mi355x_mul_mat_q8_0_tiles(const void * tiles, int64_t K, int64_t M, const mi355x_tensor * src1, const mi355x_tensor * dst,
                                             int flags, void * workspace, size_t workspace_size, void * stream);
+/* mi355x_mul_mat_q8_0_tiles over LayerNorm(src) (mi355x_norm: eps, optional affine w / b) in one launch — the decoder's last
+ * LayerNorm and the logits of a decode step: every workgroup normalizes the step's rows while its first tile row is on the
+ * way; the first also writes the rows to `normed` and their Q8_0 form to `workspace`, as mi355x_norm_emit_q8_0 would.  The
+ * same values bit for bit as that call followed by mi355x_mul_mat_q8_0_tiles with MI355X_MM_WS_READY.  src / normed: F32
+ * [K, N <= 8], 16-byte aligned rows; `flags`: MI355X_EPI_OUT_F16 or 0; K as for mi355x_mul_mat_q8_0_tiles.  No counterpart in
+ * the reference, whose graphs hold these as separate nodes. */
+MI355X_API int    mi355x_norm_mul_mat_q8_0_tiles(const void * tiles, int64_t K, int64_t M, const mi355x_tensor * src, const mi355x_tensor * normed,
+                                                 float eps, const float * w, const float * b, const mi355x_tensor * dst, int flags,
+                                                 void * workspace, size_t workspace_size, void * stream);
 
 /* FLASH_ATTN_EXT --------------------------------------------------------------------------------------
  * ggml_compute_forward_flash_attn_ext_f16 (ggml/src/ggml-cpu/ops.cpp:6638-6851), max_bias = 0 and

@@ -312,7 +312,8 @@ def test_the_token_embedding_of_a_decode_step_is_made_inside_the_first_layers_la
     assert rc == 0 and "embed_norm_mul_mat.gemv" in names and "get_rows_add" not in names and "get_rows" not in names, names
     fused = rows[-1]["launches_per_step"]
     if key[0] == "large-v3-turbo":
-        assert fused <= 34, fused
+        # ... and the decoder's last LayerNorm has none either: it runs inside the launch of the logits product
+        assert fused <= 33 and "norm_mul_mat.gemv_q8_0.vocab" in names and "norm_affine_emit" not in names, (fused, names)
     rc, rows = run_harness(harness, args, env={"GGML_MI355X_FUSE": "0"}, timeout=600)
     names = {k["kernel"] for k in rows[-1]["kernels"]}
     assert rc == 0 and "get_rows" in names and "embed_norm_mul_mat.gemv" not in names and rows[-1]["launches_per_step"] > fused, names

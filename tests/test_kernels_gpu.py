@@ -123,6 +123,56 @@ def test_mul_mat_quantized(pkg, oracle, gpu, wtype, shape):
         assert oracle.nmse(alone if n * m * k <= 2e9 else alone[:, sel], want) <= 1e-10
 
 
+@pytest.mark.parametrize("shape", [(1280, 51866, 5), (1280, 2000, 8), (384, 1000, 1), (512, 51865, 3), (768, 16, 2), (1024, 333, 7), (1280, 4000, 1)])
+def test_norm_mul_mat_q8_0_tiles(pkg, oracle, gpu, shape):
+    # the decoder's last LayerNorm inside the launch of the logits product: the same normalized rows, Q8_0 form and logits, bit
+    # for bit, as mi355x_norm_emit_q8_0 followed by mi355x_mul_mat_q8_0_tiles over the workspace
+    lib = pkg.kernels()
+    k, m, n = shape
+    blocks = oracle.quantize(pkg.Q8_0, rnd((m, k), 0.02))
+    x = rnd((n, k), 2.0, 0.3)
+    w, b = rnd((k,), 0.02, 1.0), rnd((k,), 0.02)
+    d_blk, d_x, d_w, d_b = gpu.up(blocks), gpu.up(x), gpu.up(w), gpu.up(b)
+    size = lib.mi355x_q8_0_tiles_size(k, m)
+    tiles = torch.zeros((size,), dtype=torch.uint8, device=gpu.dev)
+    pkg.check(lib.mi355x_q8_0_tiles_pack(pkg.tensor(d_blk, pkg.Q8_0, ne=[k, m]), tiles.data_ptr(), gpu.stream))
+    need = (n * k + n * (k // 32) * 8 + 255) // 256 * 256
+    tx = pkg.tensor(d_x, pkg.F32)
+
+    def run(fused, affine, f16):
+        d_n = torch.zeros_like(d_x)
+        ws = torch.zeros(need, dtype=torch.uint8, device=gpu.dev)
+        d_y = torch.full((n, m), 7.0, dtype=torch.float16 if f16 else torch.float32, device=gpu.dev)
+        tn, ty = pkg.tensor(d_n, pkg.F32), pkg.tensor(d_y, pkg.F16 if f16 else pkg.F32)
+        pw, pb = (d_w.data_ptr(), d_b.data_ptr()) if affine else (None, None)
+        fl = pkg.EPI_OUT_F16 if f16 else 0
+        if fused:
+            pkg.check(lib.mi355x_norm_mul_mat_q8_0_tiles(tiles.data_ptr(), k, m, tx, tn, 1e-5, pw, pb, ty, fl, ws.data_ptr(), need, gpu.stream))
+        else:
+            pkg.check(lib.mi355x_norm_emit_q8_0(tx, tn, 1e-5, pw, pb, ws.data_ptr(), gpu.stream))
+            pkg.check(lib.mi355x_mul_mat_q8_0_tiles(tiles.data_ptr(), k, m, tn, ty, fl | pkg.MM_WS_READY, ws.data_ptr(), need, gpu.stream))
+        y = gpu.down(d_y)
+        return gpu.down(d_n), gpu.down(ws)[: n * k + n * (k // 32) * 8], y.view(np.uint16) if f16 else y
+
+    for affine, f16 in ((True, False), (False, False), (True, True)):
+        n1, q1, y1 = run(True, affine, f16)
+        n0, q0, y0 = run(False, affine, f16)
+        assert np.array_equal(n1, n0) and np.array_equal(q1, q0) and np.array_equal(y1, y0), (affine, f16)
+        if affine and not f16:
+            assert oracle.nmse(n1, oracle.norm(x, 1e-5) * w + b) <= 1e-10
+            sel = np.r_[0:min(64, m), max(m - 64, 0):m]
+            assert oracle.nmse(y1[:, sel], oracle.mul_mat(pkg.Q8_0, blocks.reshape(m, -1)[sel], n1)) <= 1e-10
+    # what it does not take: another K, no workspace, rows of another length, flags of the plain product
+    d_n = torch.zeros_like(d_x)
+    d_y = torch.zeros((n, m), dtype=torch.float32, device=gpu.dev)
+    ws = torch.zeros(need, dtype=torch.uint8, device=gpu.dev)
+    tn, ty = pkg.tensor(d_n, pkg.F32), pkg.tensor(d_y, pkg.F32)
+    assert lib.mi355x_norm_mul_mat_q8_0_tiles(tiles.data_ptr(), 640, m, tx, tn, 1e-5, None, None, ty, 0, ws.data_ptr(), need, gpu.stream) == -1
+    assert lib.mi355x_norm_mul_mat_q8_0_tiles(tiles.data_ptr(), k, m, tx, tn, 1e-5, None, None, ty, 0, None, 0, gpu.stream) == -3
+    assert lib.mi355x_norm_mul_mat_q8_0_tiles(tiles.data_ptr(), k, m, tx, tn, 1e-5, None, None, ty, pkg.MM_WS_READY, ws.data_ptr(), need, gpu.stream) == -1
+    assert lib.mi355x_norm_mul_mat_q8_0_tiles(tiles.data_ptr(), k, m + 16, tx, tn, 1e-5, None, None, ty, 0, ws.data_ptr(), need, gpu.stream) == -2
+
+
 @pytest.mark.parametrize("shape", [(1280, 51866, 5), (1280, 2000, 8), (384, 1000, 1), (512, 47, 3), (768, 16, 2), (1024, 333, 7)])
 def test_mul_mat_q8_0_tiles(pkg, oracle, gpu, shape):
     # the matrix-core form of the few-column product: the block rows repacked 16 rows x 2 blocks at a time

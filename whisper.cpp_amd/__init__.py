@@ -75,6 +75,7 @@ def kernels() -> C.CDLL:
             "mi355x_q8_0_tiles_size": (C.c_size_t, [C.c_int64, C.c_int64]),
             "mi355x_q8_0_tiles_pack": (C.c_int, [T, P, P]),
             "mi355x_mul_mat_q8_0_tiles": (C.c_int, [P, C.c_int64, C.c_int64, T, T, C.c_int, P, C.c_size_t, P]),
+            "mi355x_norm_mul_mat_q8_0_tiles": (C.c_int, [P, C.c_int64, C.c_int64, T, T, C.c_float, P, P, T, C.c_int, P, C.c_size_t, P]),
             "mi355x_norm_mul_mat_group": (C.c_int, [T, T, C.c_float, P, P, C.POINTER(MulMatItem), C.c_int, P, C.c_size_t, P]),
             "mi355x_embed_norm_mul_mat_group": (C.c_int, [T, T, T, T, T, T, C.c_float, P, P, C.POINTER(MulMatItem), C.c_int, P, C.c_size_t, P]),
             "mi355x_flash_attn_ext_kernel_name": (C.c_char_p, [T, T, C.c_int]),

@@ -615,6 +615,28 @@ struct graph_runner {
         const mm_chain c = plan_chain(i);
         mm_operands o = describe(c);
         if (const int grouped = run_mul_mat_group(i, c, o, status)) return grouped;
+        // the decoder's last LayerNorm, held, in front of the logits over the tile-ordered vocabulary matrix: one launch, the
+        // LayerNorm under the 7 us the first tile rows take to arrive
+        if (held.active && held.key == c.x && o.tiles && !emb.active &&
+            ctx->reserve_workspace((size_t)(c.x->ne[0] * c.x->ne[1] + c.x->ne[0] / 32 * c.x->ne[1] * 8) + 256)) {
+            mi355x_tensor vs = to_view(held.src), vn = to_view(held.out);
+            int rc;
+            {
+                launch_scope ls(ctx, "norm_mul_mat.gemv_q8_0.vocab", chain_bytes(c) + nbytes_of(held.src) + nbytes_of(held.out), chain_flops(c));
+                rc = mi355x_norm_mul_mat_q8_0_tiles(o.tiles, c.w->ne[0], c.w->ne[1], &vs, &vn, held.eps, held.w, held.b, &o.vd,
+                                                    c.epi.flags & MI355X_EPI_OUT_F16, ctx->ws, ctx->ws_size, ctx->stream);
+                if (rc == MI355X_ERR_UNSUPPORTED) ls.cancel();
+            }
+            if (rc != MI355X_ERR_UNSUPPORTED) {
+                held.active = false;
+                status = rc;
+                note_write(held.out);
+                if (rc == MI355X_OK) workspace_holds(held.key, ctx->ws_slot, 2);
+                note_write(c.out);
+                fold_nodes(i, c.used, c.out);
+                return c.used;
+            }
+        }
         if (held.active && (status = flush_norm()) != MI355X_OK) return c.used;
 
         mi355x_epilogue epi = c.epi;

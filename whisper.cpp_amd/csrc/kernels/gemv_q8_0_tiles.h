@@ -9,12 +9,21 @@
 
 #define Q8T_STEP 1088      // bytes of 16 rows x one pair of blocks
 
+// the activations as they come: quantized ahead, in global memory
+struct q8t_no_prologue {
+    __device__ __forceinline__ void request() {}
+    __device__ __forceinline__ const char * finish(const char * x) { return x; }
+};
+
 // a.w: the tiles; a.x: the activations quantized ahead (layout of k_quantize_x_q8); K = 64 KSTEPS
 // STAMPS (measurement instances only, never the product's): every wavefront leaves the device's 100 MHz clock at its start and
 // after each of its tiles in `stamps` ([wavefront][1 + tiles per wavefront]; 0 = no such tile), from which the rate of the
 // stream between its ramp and its tail can be read.
-template <int KSTEPS, bool STAMPS>
-__global__ void __launch_bounds__(256, 2) k_gemv_q8_0_tiles(mm_args a, uint64_t * stamps) {
+// `pro`: where the quantized activations come from.  request() issues its loads in front of the first tile's, finish() runs
+// behind them and returns the activations' address (the plain product: a.x as passed; with a LayerNorm in front, the rows
+// it has just normalized and rounded, in LDS) — the first tile takes 7 us to arrive, which is the time such a prologue has.
+template <int KSTEPS, bool STAMPS, typename PRO>
+__device__ __forceinline__ void gemv_q8_0_tiles_body(const mm_args & a, uint64_t * stamps, PRO pro) {
     __shared__ __attribute__((aligned(16))) float xs_lds[KSTEPS * 2 * 8];       // activation scales, [block][column 0 .. 7]
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int r = lane & 15, g = lane >> 4;
@@ -40,14 +49,18 @@ __global__ void __launch_bounds__(256, 2) k_gemv_q8_0_tiles(mm_args a, uint64_t 
         if (lane == 0) my_stamps[0] = __builtin_amdgcn_s_memrealtime();
     }
     const bool live = tile < n_tiles;                   // (a matrix of fewer than 64 rows)
+    if constexpr (!std::is_same<PRO, q8t_no_prologue>::value) {
+        pro.request();
+        __builtin_amdgcn_sched_barrier(0);
+    }
     request(0, live ? tile : n_tiles - 1);
     __builtin_amdgcn_sched_barrier(0);
     request(1, live ? tile : n_tiles - 1);
     __builtin_amdgcn_sched_barrier(0);
 
     // activations: quants as the A operand (lane = A row r, 16 k of group g), scales through LDS
-    const char *  xq = a.x;
-    const float * xd = (const float *)(a.x + (size_t) a.N * a.K);
+    const char *  xq = pro.finish(a.x);
+    const float * xd = (const float *)(xq + (size_t) a.N * a.K);
     const int col = r & 7;
     const bool mine = ((r < 8) == (g < 2)) && col < a.N;
     v4i_t xa[KSTEPS];
@@ -98,5 +111,10 @@ __global__ void __launch_bounds__(256, 2) k_gemv_q8_0_tiles(mm_args a, uint64_t 
     // every tile but the wavefront's last requests the next one's halves as its own are used up
     for (; tile + stride < n_tiles; tile += stride) do_tile(std::true_type{});
     do_tile(std::false_type{});
+}
+
+template <int KSTEPS, bool STAMPS>
+__global__ void __launch_bounds__(256, 2) k_gemv_q8_0_tiles(mm_args a, uint64_t * stamps) {
+    gemv_q8_0_tiles_body<KSTEPS, STAMPS>(a, stamps, q8t_no_prologue{});
 }
 

@@ -1703,6 +1703,41 @@ __global__ void __launch_bounds__(256) k_gemv_qr_norm_group(mm_args a, gemv_grou
     gemv_qr_rows<T0, NC, LPR, NB>(a, gemv_norm_prologue<NC, NJ, EMB>{ nm, a.K, smem });
 }
 
+// the product over the tile-ordered vocabulary matrix with the decoder's last LayerNorm in front, the same way: the
+// LayerNorm of the step's rows runs in every workgroup while its first tile row is on the way
+template <int KSTEPS, int NC, int NJ>
+__global__ void __launch_bounds__(256, 2) k_gemv_q8_0_tiles_norm(mm_args a, gemv_norm_args nm) {
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    gemv_q8_0_tiles_body<KSTEPS, false>(a, nullptr, gemv_norm_prologue<NC, NJ>{ nm, a.K, smem });
+}
+
+template <int KSTEPS, int NC>
+static int launch_gemv_q8_0_tiles_norm_kn(const mm_args & a, const gemv_norm_args & nm, hipStream_t st) {
+    const int64_t n_tiles = (a.M + 15) / 16;
+    const int64_t resident = 256 * 2 * 4;                 // wavefronts: two workgroups of four per CU
+    const int64_t rounds = (n_tiles + resident - 1) / resident;
+    const int64_t waves = (n_tiles + rounds - 1) / rounds;
+    const unsigned grid = (unsigned)(waves / 4 > 0 ? waves / 4 : 1);
+    const size_t lds = (size_t) NC * a.K + (size_t) NC * (a.K / QK) * 8;
+    if (KSTEPS == 20 && nm.w && nm.b) k_gemv_q8_0_tiles_norm<KSTEPS, NC, KSTEPS == 20 ? 5 : 0><<<grid, 256, lds, st>>>(a, nm);
+    else                              k_gemv_q8_0_tiles_norm<KSTEPS, NC, 0><<<grid, 256, lds, st>>>(a, nm);
+    return launch_status();
+}
+template <int KSTEPS>
+static int launch_gemv_q8_0_tiles_norm_k(const mm_args & a, const gemv_norm_args & nm, hipStream_t st) {
+    switch (a.N) {
+        case 1: return launch_gemv_q8_0_tiles_norm_kn<KSTEPS, 1>(a, nm, st);
+        case 2: return launch_gemv_q8_0_tiles_norm_kn<KSTEPS, 2>(a, nm, st);
+        case 3: return launch_gemv_q8_0_tiles_norm_kn<KSTEPS, 3>(a, nm, st);
+        case 4: return launch_gemv_q8_0_tiles_norm_kn<KSTEPS, 4>(a, nm, st);
+        case 5: return launch_gemv_q8_0_tiles_norm_kn<KSTEPS, 5>(a, nm, st);
+        case 6: return launch_gemv_q8_0_tiles_norm_kn<KSTEPS, 6>(a, nm, st);
+        case 7: return launch_gemv_q8_0_tiles_norm_kn<KSTEPS, 7>(a, nm, st);
+        case 8: return launch_gemv_q8_0_tiles_norm_kn<KSTEPS, 8>(a, nm, st);
+    }
+    return MI355X_ERR_INVALID;
+}
+
 // ------------------------------------------------------------------------------------------------------
 // generic fallback: one wavefront per (m, group of up to 8 columns, batch); element-wise dequant, f32 FMA
 // ------------------------------------------------------------------------------------------------------
@@ -2148,6 +2183,41 @@ extern "C" int mi355x_mul_mat_q8_0_tiles(const void * tiles, int64_t K, int64_t 
         case 768:  return launch_gemv_q8_0_tiles_k<12>(a, st);
         case 1024: return launch_gemv_q8_0_tiles_k<16>(a, st);
         default:   return launch_gemv_q8_0_tiles_k<20>(a, st);
+    }
+}
+
+extern "C" int mi355x_norm_mul_mat_q8_0_tiles(const void * tiles, int64_t K, int64_t M, const mi355x_tensor * src, const mi355x_tensor * normed,
+                                              float eps, const float * w, const float * b, const mi355x_tensor * dst, int flags,
+                                              void * workspace, size_t workspace_size, void * stream) {
+    if (!tiles || !src || !normed || !dst || !(eps >= 0.0f)) return MI355X_ERR_INVALID;
+    if (!q8_0_tiles_k_ok(K) || M <= 0 || (uintptr_t) tiles % 16 != 0) return MI355X_ERR_UNSUPPORTED;
+    if (flags & ~MI355X_EPI_OUT_F16) return MI355X_ERR_UNSUPPORTED;
+    const int td = (flags & MI355X_EPI_OUT_F16) ? MI355X_TYPE_F16 : MI355X_TYPE_F32;
+    const int64_t N = src->ne[1];
+    if (src->type != MI355X_TYPE_F32 || normed->type != MI355X_TYPE_F32 || dst->type != td || src->nb[0] != 4 || normed->nb[0] != 4 || dst->nb[0] != type_size(td)) return MI355X_ERR_UNSUPPORTED;
+    for (int i = 0; i < 4; ++i) if (src->ne[i] != normed->ne[i]) return MI355X_ERR_INVALID;
+    if (src->ne[0] != K || dst->ne[0] != M || dst->ne[1] != N) return MI355X_ERR_INVALID;
+    if (N < 1 || N > MI355X_GEMV_MAX_COLS || src->ne[2] != 1 || src->ne[3] != 1 || dst->ne[2] != 1 || dst->ne[3] != 1) return MI355X_ERR_UNSUPPORTED;
+    if (!aligned16(src) || !aligned16(normed) || (uintptr_t) w % 16 != 0 || (uintptr_t) b % 16 != 0) return MI355X_ERR_UNSUPPORTED;
+    const size_t need = round256((size_t)(N * K + N * (K / QK) * 8));
+    if (!workspace || workspace_size < need || (uintptr_t) workspace % 16 != 0) return MI355X_ERR_WORKSPACE;
+    gemv_norm_args nm{};
+    nm.src = (const char *) src->data; nm.src_nb1 = (int64_t) src->nb[1]; nm.w = w; nm.b = b; nm.eps = eps;
+    nm.dst = (char *) normed->data; nm.dst_nb1 = (int64_t) normed->nb[1]; nm.ws = (char *) workspace;
+    mm_args a;
+    a.K = K; a.M = M; a.N = N;
+    a.w = (const char *) tiles; a.x = (const char *) workspace; a.d = (char *) dst->data;
+    a.w_nb1 = a.w_nb2 = a.w_nb3 = 0; a.x_nb1 = a.x_nb2 = a.x_nb3 = 0;
+    a.d_nb1 = dst->nb[1]; a.d_nb2 = a.d_nb3 = 0;
+    a.ne12 = a.ne13 = a.r2 = a.r3 = 1;
+    a.e.flags = flags & MI355X_EPI_OUT_F16; a.e.scale = 1.0f; a.e.bias = nullptr; a.e.residual = nullptr; a.e.gelu = nullptr; a.e.image = nullptr;
+    hipStream_t st = (hipStream_t) stream;
+    switch (K) {
+        case 384:  return launch_gemv_q8_0_tiles_norm_k<6>(a, nm, st);
+        case 512:  return launch_gemv_q8_0_tiles_norm_k<8>(a, nm, st);
+        case 768:  return launch_gemv_q8_0_tiles_norm_k<12>(a, nm, st);
+        case 1024: return launch_gemv_q8_0_tiles_norm_k<16>(a, nm, st);
+        default:   return launch_gemv_q8_0_tiles_norm_k<20>(a, nm, st);
     }
 }
 

@@ -39,6 +39,7 @@ BENCH_NAMES = [
     ("void k_gemm_f16_dl_group", "mul_mat.gemm_group", "encoder"), ("void k_gemm_f16_dl<", "mul_mat.gemm_q5_0", "encoder"),
     ("void k_gemm_f16_rs<", "mul_mat.gemm_q5_0", "encoder"), ("void k_norm<5, 1", "norm_affine_emit", "encoder"), ("_Z6k_normILi5ELi1E", "norm_affine_emit", "encoder"),
     ("k_fattn_pk_row", "flash_attn.seq_row_pk", "decoder"), ("k_fattn_seq_row", "flash_attn.seq_row", "decoder"), ("void k_gemv_q8_0_tiles<20", "mul_mat.gemv_q8_0.vocab", "decoder"),
+    ("void k_gemv_q8_0_tiles_norm<20", "norm_mul_mat.gemv_q8_0.vocab", "decoder"),
 ]
 
 SQ_PASSES = [
