@@ -402,6 +402,8 @@ def main() -> int:
               "ms_per_step_with_the_x86_form_of_the_attention_step": round(dec_x86["ms_per_step"], 4)}
     if gemv:
         decode["gemv_roofline"] = kernel_roofline(gemv_name, gemv)
+        if gemv_name.startswith("norm_"):
+            decode["gemv_roofline"]["launch_includes"] = "the decoder's last LayerNorm over the step's rows, in every workgroup, while its first tile row is on the way"
         # what a bare stream of the same bytes takes here, measured the same way: the ceiling that applies to a single launch
         y = read_yardstick(int(gemv["bytes"] / gemv["calls"]))
         decode["gemv_roofline"]["read_yardstick"] = y
