@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """rocprofv3 passes over the harness commands that bench.py times; run on a box with an MI355X:
 
-    python whisper.cpp_amd/profile.py [--out gpurun_out/prof]
+    python whisper.cpp_amd/profile.py [--out DIR]
 
 Writes, under --out: `kernel_stats_encoder.csv`, `kernel_stats_decoder.csv` (rocprofv3 --kernel-trace --stats), `decode_positions.txt`
 (a decode step's launches one by one, from a kernel trace), `counters.json`
